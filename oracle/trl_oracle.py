@@ -1,0 +1,575 @@
+"""CPU restatement (PyTorch, host only) of the reference's log-probability / entropy /
+policy-loss path.  TEST INFRASTRUCTURE: this module is the *checker* for the HIP
+kernels and the CPU baseline of the benchmark.  The shipped package never imports it.
+
+Every function cites the reference lines (paths relative to the reference tree) whose
+arithmetic it follows.  The functions keep the reference's *order of operations and
+dtypes* (row loops, 128-row chunks, in-dtype temperature division) because those are
+what a user of the reference observes; `*_f32` variants are the same mathematics with
+fp32 op-math on the same (possibly bf16-valued) inputs and are what low-precision
+kernel outputs are compared against.
+
+Pinning status (what checks each function against something other than itself):
+  selective_log_softmax / entropy_from_logits : torch library routines
+      (`log_softmax().gather()`, `-(p*log p).sum()`), closed forms (uniform row,
+      shift invariance), reference unit-test shapes  -> tests/test_oracle.py
+  nanstd / nanmin / nanmax  : reference unit-test vectors (tests/test_utils.py:316-331)
+  group_advantages          : torch.std(unbiased) on NaN-free groups, zero-variance
+                              closed form, golden vectors from the reference's formula
+  grpo_loss                 : golden vectors written by the reference's
+                              `GRPOTrainer._compute_loss` on a mocked trainer
+                              (tests/golden/), closed forms (on-policy, ref == logps)
+  dpo_*                     : golden vectors from the reference's
+                              `DPOTrainer._compute_loss` (mocked), closed form ln 2
+  rloo_loss                 : golden vectors from `RLOOTrainer._compute_loss` (mocked)
+  chunked_logprob           : naive `(h @ W.T).float()/T -> log_softmax` routine and
+                              autograd of it (reference test tests/test_utils.py:1161-1232)
+  get_off_policy_mask       : reference unit-test vectors (tests/test_grpo_trainer.py:1456-1520)
+  get_high_entropy_mask     : reference unit-test vectors (tests/test_grpo_trainer.py:110-160)
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+__all__ = [
+    "selective_log_softmax",
+    "selective_log_softmax_f32",
+    "entropy_from_logits",
+    "entropy_from_logits_f32",
+    "nanstd",
+    "nanmin",
+    "nanmax",
+    "group_advantages",
+    "rloo_advantages",
+    "get_off_policy_mask",
+    "get_high_entropy_mask",
+    "logps_and_entropies_from_logits",
+    "grpo_loss",
+    "dpo_sequence_logps",
+    "dpo_sigmoid_loss",
+    "rloo_loss",
+    "chunked_logprob_naive",
+    "chunked_logprob_online",
+    "chunked_logprob_backward",
+    "ChunkedLogProbOracle",
+    "patch_chunked_rows",
+]
+
+
+# --------------------------------------------------------------------------------------
+# A1  selective_log_softmax               trl/trainer/utils.py:479-523
+# --------------------------------------------------------------------------------------
+def selective_log_softmax(logits: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+    """`log_softmax(logits)[..., index]` with the reference's two dtype branches.
+
+    fp32/fp64 (utils.py:506-510): gather the selected logits, subtract a per-leading-row
+    `logsumexp`.  Other dtypes (utils.py:511-518): per-leading-row `log_softmax` in the
+    input dtype followed by `gather` (output stays in the low-precision dtype).
+    `index` has either the leading shape of `logits` or one extra trailing axis K
+    (utils.py:502-504, 520-521).
+    """
+    drop_last = index.ndim == logits.ndim - 1
+    idx = index.unsqueeze(-1) if drop_last else index
+    if logits.dtype in (torch.float32, torch.float64):
+        picked = logits.gather(-1, idx)
+        lse = torch.stack([torch.logsumexp(block, dim=-1) for block in logits])
+        out = picked - lse.unsqueeze(-1)
+    else:
+        rows = []
+        for block, block_idx in zip(logits, idx, strict=True):
+            rows.append(F.log_softmax(block, dim=-1).gather(-1, block_idx))
+        out = torch.stack(rows)
+    return out.squeeze(-1) if drop_last else out
+
+
+def selective_log_softmax_f32(logits: torch.Tensor, index: torch.Tensor, temperature: float = 1.0) -> torch.Tensor:
+    """Same quantity with fp32 op-math on the stored values: the reference function
+    applied to `logits.float() / temperature` (grpo_trainer.py:1519 + utils.py:506-510).
+    Processed block-wise so that a bf16 input is never widened all at once."""
+    drop_last = index.ndim == logits.ndim - 1
+    idx = index.unsqueeze(-1) if drop_last else index
+    flat = logits.reshape(-1, logits.shape[-1]) if logits.ndim > 1 else logits.unsqueeze(0)
+    flat_idx = idx.reshape(-1, idx.shape[-1])
+    out = torch.empty(flat_idx.shape, dtype=torch.float32)
+    for r0 in range(0, flat.shape[0], 256):
+        z = flat[r0 : r0 + 256].float() / temperature
+        out[r0 : r0 + 256] = z.gather(-1, flat_idx[r0 : r0 + 256]) - torch.logsumexp(z, -1, keepdim=True)
+    out = out.reshape(idx.shape)
+    return out.squeeze(-1) if drop_last else out
+
+
+# --------------------------------------------------------------------------------------
+# A2  entropy_from_logits                 trl/trainer/utils.py:526-560
+# --------------------------------------------------------------------------------------
+def entropy_from_logits(logits: torch.Tensor, chunk_size: int = 128) -> torch.Tensor:
+    """Shannon entropy (nats) of softmax(logits) per row.  Rows are flattened
+    (utils.py:551) and handled `chunk_size` at a time (utils.py:554-557) with all
+    intermediates in the input dtype: H = -sum(exp(lp) * lp), lp = log_softmax(row)."""
+    lead = logits.shape[:-1]
+    rows = logits.reshape(-1, logits.shape[-1])
+    pieces = []
+    for piece in rows.split(chunk_size, dim=0):
+        lp = F.log_softmax(piece, dim=-1)
+        pieces.append(-(lp.exp() * lp).sum(-1))
+    return torch.cat(pieces, 0).reshape(lead)
+
+
+def entropy_from_logits_f32(logits: torch.Tensor, temperature: float = 1.0) -> torch.Tensor:
+    """fp32 op-math entropy of `softmax(logits.float() / temperature)`."""
+    lead = logits.shape[:-1]
+    rows = logits.reshape(-1, logits.shape[-1])
+    out = torch.empty(rows.shape[0], dtype=torch.float32)
+    for r0 in range(0, rows.shape[0], 256):
+        lp = F.log_softmax(rows[r0 : r0 + 256].float() / temperature, dim=-1)
+        out[r0 : r0 + 256] = -(lp.exp() * lp).sum(-1)
+    return out.reshape(lead)
+
+
+# --------------------------------------------------------------------------------------
+# nanstd / nanmin / nanmax                trl/trainer/utils.py:857-890, 960-987
+# --------------------------------------------------------------------------------------
+def nanstd(x: torch.Tensor, dim=None, keepdim: bool = False) -> torch.Tensor:
+    """Bessel-corrected standard deviation over the non-NaN entries (utils.py:874-880):
+    sqrt(nanmean((x - nanmean(x))^2) * n/(n-1)), NaN when n <= 1."""
+    mu = torch.nanmean(x, dim=dim, keepdim=True)
+    var = torch.nanmean((x - mu) ** 2, dim=dim, keepdim=True)
+    n = (~x.isnan()).sum(dim=dim, keepdim=True)
+    bessel = torch.where(n > 1, n / (n - 1), torch.full_like(var, float("nan")))
+    sd = (var * bessel).sqrt()
+    if keepdim:
+        return sd
+    if dim is None:
+        return sd.squeeze()
+    if isinstance(dim, int):
+        return sd.squeeze(dim)
+    for d in sorted((d % sd.ndim for d in dim), reverse=True):
+        sd = sd.squeeze(d)
+    return sd
+
+
+def nanmin(x: torch.Tensor) -> torch.Tensor:
+    """Minimum over non-NaN entries of a 1-D tensor; NaN if there are none (utils.py:960-972)."""
+    keep = ~x.isnan()
+    return x[keep].min() if keep.any() else x.new_tensor(float("nan"))
+
+
+def nanmax(x: torch.Tensor) -> torch.Tensor:
+    """Maximum over non-NaN entries of a 1-D tensor; NaN if there are none (utils.py:975-987)."""
+    keep = ~x.isnan()
+    return x[keep].max() if keep.any() else x.new_tensor(float("nan"))
+
+
+# --------------------------------------------------------------------------------------
+# A5  group-relative advantages           trl/trainer/grpo_trainer.py:2685-2707, 2730
+# --------------------------------------------------------------------------------------
+def group_advantages(rewards: torch.Tensor, num_generations: int, scale_rewards: str = "group") -> torch.Tensor:
+    """`rewards` [B] (NaN = unscorable), groups are `num_generations` consecutive rows
+    (`view(-1, G)`, grpo_trainer.py:2685).  A = r - nanmean_g; divided by
+    (nanstd_g + 1e-4) for "group", by (nanstd_all + 1e-4) for "batch", not at all for
+    "none" (grpo_trainer.py:2687-2707); NaN -> 0 (grpo_trainer.py:2730)."""
+    G = num_generations
+    grouped = rewards.view(-1, G)
+    mean_g = torch.nanmean(grouped, dim=1).repeat_interleave(G)
+    if scale_rewards in ("group", "none"):
+        std = nanstd(grouped, dim=1).repeat_interleave(G) if G > 1 else torch.zeros_like(rewards)
+    elif scale_rewards == "batch":
+        std = nanstd(rewards).expand_as(rewards) if rewards.numel() > 1 else torch.zeros_like(rewards)
+    else:
+        raise ValueError(f"Invalid value for scale_rewards: {scale_rewards}")
+    adv = rewards - mean_g
+    if scale_rewards != "none":
+        adv = adv / (std + 1e-4)
+    return torch.nan_to_num(adv, nan=0.0)
+
+
+def rloo_advantages(rewards: torch.Tensor, num_generations: int, normalize_advantages: bool = False) -> torch.Tensor:
+    """Leave-one-out baseline over scorable siblings (rloo_trainer.py:1537-1561):
+    b_i = (nansum_g - r_i) / (n_scorable - 1), A = r - b, optional global
+    (A - nanmean)/(nanstd + 1e-4), NaN -> 0."""
+    G = num_generations
+    grouped = rewards.view(-1, G)
+    if G > 1:
+        n = (~grouped.isnan()).sum(1, keepdim=True)
+        total = torch.nansum(grouped, dim=1, keepdim=True)
+        adv = rewards - ((total - grouped) / (n - 1)).view(-1)
+    else:
+        adv = torch.zeros_like(rewards)
+    if normalize_advantages:
+        adv = (adv - torch.nanmean(adv)) / (nanstd(adv) + 1e-4)
+    return torch.nan_to_num(adv, nan=0.0)
+
+
+# --------------------------------------------------------------------------------------
+# sequence masks                          trl/trainer/grpo_trainer.py:2920-2939, 1396-1432
+# --------------------------------------------------------------------------------------
+def get_off_policy_mask(advantages, per_token_logps, sampling_per_token_logps, mask, off_policy_threshold):
+    """(B,1) keep-mask: keep if A >= 0 or masked-mean(sampling_logp - logp) <= threshold
+    (grpo_trainer.py:2934-2939)."""
+    gap = sampling_per_token_logps - per_token_logps.detach()
+    mean_gap = (gap * mask).sum(1, keepdim=True) / mask.sum(1, keepdim=True).clamp(min=1.0)
+    return ((advantages >= 0) | (mean_gap <= off_policy_threshold)).to(mask.dtype)
+
+
+def get_high_entropy_mask(entropies, mask, threshold):
+    """Boolean mask of active tokens whose entropy is >= the `threshold` quantile of all
+    active-token entropies (single process: the cross-rank gather is the identity)
+    (grpo_trainer.py:1413-1432)."""
+    active = entropies[mask.bool()].float()
+    if active.numel() == 0:
+        return torch.zeros_like(entropies, dtype=torch.bool)
+    cut = torch.quantile(active, threshold)
+    return ((entropies * mask.float()) >= cut) & mask.bool()
+
+
+# --------------------------------------------------------------------------------------
+# A3 + A4  logits -> per-token logps / entropies   trl/trainer/grpo_trainer.py:1511-1533
+# --------------------------------------------------------------------------------------
+def logps_and_entropies_from_logits(
+    logits: torch.Tensor,
+    input_ids: torch.Tensor,
+    logits_to_keep: int,
+    temperature: float = 1.0,
+    compute_entropy: bool = True,
+    entropy_requires_grad: bool = False,
+):
+    """The part of `_get_per_token_logps_and_entropies` after the model call: drop the
+    last position (grpo_trainer.py:1514), keep the last `logits_to_keep` (:1516),
+    divide by the temperature *in the logits dtype* (:1519, here out of place so the
+    caller's tensor survives), select log-probs of `input_ids[:, -K:]` (:1520-1521),
+    entropy with or without grad (:1528-1532)."""
+    z = logits[:, :-1, :][:, -logits_to_keep:, :]
+    z = z / temperature
+    ids = input_ids[:, -logits_to_keep:]
+    logps = selective_log_softmax(z, ids)
+    ent = None
+    if compute_entropy:
+        if entropy_requires_grad:
+            ent = entropy_from_logits(z)
+        else:
+            with torch.no_grad():
+                ent = entropy_from_logits(z)
+    return logps, ent
+
+
+# --------------------------------------------------------------------------------------
+# A6-A9  GRPO loss                        trl/trainer/grpo_trainer.py:3026-3258
+# --------------------------------------------------------------------------------------
+def grpo_loss(
+    per_token_logps: torch.Tensor,
+    advantages: torch.Tensor,
+    mask: torch.Tensor,
+    *,
+    entropies: torch.Tensor | None = None,
+    old_per_token_logps: torch.Tensor | None = None,
+    ref_per_token_logps: torch.Tensor | None = None,
+    loss_type: str = "dapo",
+    epsilon_low: float = 0.2,
+    epsilon_high: float = 0.2,
+    beta: float = 0.0,
+    delta: float | None = None,
+    max_completion_length: int | None = None,
+    num_items_in_batch: torch.Tensor | float | None = None,
+    num_processes: int = 1,
+    grad_accum_steps: float = 1.0,
+    importance_sampling_level: str = "token",
+    use_bias_correction_kl: bool = False,
+    off_policy_mask_threshold: float | None = None,
+    sampling_per_token_logps: torch.Tensor | None = None,
+    top_entropy_quantile: float = 1.0,
+    importance_sampling_ratio: torch.Tensor | None = None,
+    entropy_coef: float = 0.0,
+):
+    """Clipped-surrogate GRPO family loss on `[B, T]` log-probs.  Returns
+    `(loss, metrics)` where `metrics` holds python floats named as the reference logs
+    them (grpo_trainer.py:3237-3253).  Covers loss types grpo / bnpo / dr_grpo / dapo
+    (grpo_trainer.py:3083-3091, 3124-3142), token- and sequence-level importance
+    weights (:3054-3059), k3 KL (:3069-3076), delta clamp (:3086-3087), off-policy and
+    entropy-quantile masks (:3039-3052, 3020-3021, 3111-3115), a given importance
+    sampling ratio (:3117-3118) and the static entropy bonus (:3155-3181)."""
+    adv = advantages.unsqueeze(1) if advantages.dim() == 1 else advantages
+    old = per_token_logps.detach() if old_per_token_logps is None else old_per_token_logps
+
+    entropy_mask = None
+    if top_entropy_quantile < 1.0:
+        entropy_mask = get_high_entropy_mask(entropies, mask, 1 - top_entropy_quantile)
+
+    off_mask = None
+    if off_policy_mask_threshold is not None:
+        sampling = old if sampling_per_token_logps is None else sampling_per_token_logps
+        off_mask = get_off_policy_mask(adv, per_token_logps, sampling, mask, off_policy_mask_threshold)
+
+    log_ratio = per_token_logps - old
+    if importance_sampling_level == "token":
+        log_w = log_ratio
+    elif importance_sampling_level == "sequence":
+        log_w = ((log_ratio * mask).sum(-1) / mask.sum(-1).clamp(min=1.0)).unsqueeze(-1)
+    else:
+        raise ValueError(f"Unknown importance sampling level: {importance_sampling_level}")
+    coef_1 = log_w.exp()
+
+    per_token_kl = None
+    if beta != 0.0:
+        # the difference is formed twice, as in the reference: with low-precision log-probs each
+        # use is a separate cast in autograd and the gradient contributions are rounded separately
+        per_token_kl = (
+            torch.exp(ref_per_token_logps - per_token_logps) - (ref_per_token_logps - per_token_logps) - 1
+        )
+        if use_bias_correction_kl:
+            per_token_kl = per_token_kl * coef_1
+
+    if loss_type not in ("grpo", "bnpo", "dr_grpo", "dapo"):
+        raise ValueError(f"loss type not restated in the oracle: {loss_type}")
+    coef_2 = coef_1.clamp(1 - epsilon_low, 1 + epsilon_high)
+    if delta is not None:
+        coef_1 = coef_1.clamp(max=delta)
+    per_token_loss = -torch.min(coef_1 * adv, coef_2 * adv)
+
+    if off_mask is not None:
+        per_token_loss = per_token_loss * off_mask
+    if entropy_mask is not None:
+        per_token_loss = per_token_loss * entropy_mask
+    if importance_sampling_ratio is not None:
+        per_token_loss = per_token_loss * importance_sampling_ratio
+    if beta != 0.0:
+        per_token_loss = per_token_loss + beta * per_token_kl
+
+    if loss_type == "grpo":
+        loss = ((per_token_loss * mask).sum(-1) / mask.sum(-1).clamp(min=1.0)).mean()
+        normalizer = grad_accum_steps
+        loss = loss / normalizer
+    elif loss_type == "bnpo":
+        loss = (per_token_loss * mask).sum() / mask.sum().clamp(min=1.0)
+        normalizer = grad_accum_steps
+        loss = loss / normalizer
+    elif loss_type == "dr_grpo":
+        loss = (per_token_loss * mask).sum() / (per_token_loss.size(0) * max_completion_length)
+        normalizer = grad_accum_steps
+        loss = loss / normalizer
+    else:  # dapo
+        n_items = num_items_in_batch
+        if not torch.is_tensor(n_items):
+            n_items = torch.tensor(float(n_items))
+        normalizer = n_items.clamp(min=1.0) / num_processes
+        loss = (per_token_loss * mask).sum() / normalizer
+    policy_loss = loss.detach()
+
+    metrics: dict[str, float] = {}
+    if entropy_coef != 0.0:
+        eff = mask if entropy_mask is None else mask * entropy_mask
+        if loss_type == "dapo":
+            ent_term = (entropies * eff).sum() / normalizer
+        else:
+            ent_term = (entropies * eff).sum() / eff.sum().clamp(min=1.0) / normalizer
+        loss = loss - entropy_coef * ent_term
+        metrics["policy_loss"] = float(policy_loss)
+        metrics["entropy_coef"] = float(entropy_coef)  # logged at optimizer-step boundaries (:3214-3215)
+
+    def seq_mean(x):
+        if x.shape[1] == 1:
+            return x.squeeze(1)
+        return (x * mask).sum(-1) / mask.sum(-1)  # unclamped: NaN for empty rows (:3227)
+
+    def global_mean(x):
+        if x.shape[1] == 1:
+            s, c = x.sum(), torch.tensor(float(x.shape[0]))
+        else:
+            s, c = (x * mask).sum(), mask.sum().float()
+        return float(s / c.clamp(min=1.0))
+
+    if beta != 0.0:
+        metrics["kl"] = global_mean(per_token_kl.detach())
+    if entropies is not None:
+        metrics["entropy"] = global_mean(entropies.detach())
+    low = ((coef_1 < 1 - epsilon_low) & (adv < 0)).float()
+    high = ((coef_1 > 1 + epsilon_high) & (adv > 0)).float()
+    region = ((low + high) > 0).float()
+    metrics["clip_ratio/low_mean"] = global_mean(low)
+    metrics["clip_ratio/high_mean"] = global_mean(high)
+    metrics["clip_ratio/region_mean"] = global_mean(region)
+    metrics["clip_ratio/low_min"] = float(nanmin(seq_mean(low)))
+    metrics["clip_ratio/high_max"] = float(nanmax(seq_mean(high)))
+    return loss, metrics
+
+
+# --------------------------------------------------------------------------------------
+# A10-A11  DPO                             trl/trainer/dpo_trainer.py:1342-1362, 1396-1435, 1578
+# --------------------------------------------------------------------------------------
+def dpo_sequence_logps(logits: torch.Tensor, input_ids: torch.Tensor, completion_mask: torch.Tensor):
+    """Shift by one (dpo_trainer.py:1344-1346), per-token log-probs (:1347), zero the
+    non-completion positions (:1348), sum over the sequence (:1350).  Returns
+    `(sequence_logps [B], per_token_logps [B, L-1])`."""
+    shift_logits = logits[..., :-1, :]
+    shift_labels = input_ids[..., 1:]
+    shift_mask = completion_mask[..., 1:]
+    tok = selective_log_softmax(shift_logits, shift_labels)
+    tok = torch.where(shift_mask == 0, torch.zeros_like(tok), tok)
+    return tok.sum(dim=1), tok
+
+
+def dpo_sigmoid_loss(seq_logps: torch.Tensor, ref_chosen_logps: torch.Tensor, ref_rejected_logps: torch.Tensor, beta: float):
+    """Batch layout [chosen; rejected] (dpo_trainer.py:1362).  delta = (pi_c - ref_c) -
+    (pi_r - ref_r) (:1397-1402, 1430); loss = mean(-logsigmoid(beta * delta))
+    (:1435, 1578).  Metrics as logged at dpo_trainer.py:1634-1653."""
+    chosen, rejected = seq_logps.chunk(2, dim=0)
+    chosen_lr = chosen - ref_chosen_logps
+    rejected_lr = rejected - ref_rejected_logps
+    loss = (-F.logsigmoid(beta * (chosen_lr - rejected_lr))).mean()
+    c_rew = beta * chosen_lr.detach()
+    r_rew = beta * rejected_lr.detach()
+    metrics = {
+        "rewards/chosen": float(c_rew.mean()),
+        "rewards/rejected": float(r_rew.mean()),
+        "rewards/accuracies": float((c_rew > r_rew).float().mean()),
+        "rewards/margins": float((c_rew - r_rew).mean()),
+        "logps/chosen": float(chosen.detach().mean()),
+        "logps/rejected": float(rejected.detach().mean()),
+    }
+    return loss, metrics
+
+
+# --------------------------------------------------------------------------------------
+# A12  RLOO sequence-level loss            trl/trainer/rloo_trainer.py:1683-1694, 1711-1721
+# --------------------------------------------------------------------------------------
+def rloo_loss(per_token_logps, completion_mask, old_logps, advantages, epsilon_low: float, epsilon_high: float):
+    """Sequence log-prob = sum(logp * mask) (rloo_trainer.py:1683); ratio, clamp, min and
+    mean over sequences (:1685-1694); clip metrics (:1711-1721)."""
+    seq = (per_token_logps * completion_mask).sum(1)
+    coef_1 = (seq - old_logps).exp()
+    coef_2 = coef_1.clamp(1 - epsilon_low, 1 + epsilon_high)
+    loss = (-torch.min(coef_1 * advantages, coef_2 * advantages)).mean()
+    low = ((coef_1 < 1 - epsilon_low) & (advantages < 0)).float()
+    high = ((coef_1 > 1 + epsilon_high) & (advantages > 0)).float()
+    region = ((low + high) > 0).float()
+    metrics = {
+        "clip_ratio/low_mean": float(low.mean()),
+        "clip_ratio/low_min": float(nanmin(low)),
+        "clip_ratio/high_mean": float(high.mean()),
+        "clip_ratio/high_max": float(nanmax(high)),
+        "clip_ratio/region_mean": float(region.mean()),
+    }
+    return loss, metrics
+
+
+# --------------------------------------------------------------------------------------
+# A13-A14  fused lm_head + log-prob        trl/trainer/utils.py:1291-1424
+# --------------------------------------------------------------------------------------
+def _head_logits(hidden, w_rows, temperature, softcap, logit_scale):
+    """fp32 logits of one vocab slab: matmul in the hidden dtype, widen, scale, optional
+    soft-cap, inverse temperature (utils.py:1328-1337)."""
+    z = (hidden @ w_rows.to(hidden.dtype).t()).float() * logit_scale
+    if softcap is not None:
+        z = torch.tanh(z / softcap) * softcap
+    return z * (1 / temperature)
+
+
+def chunked_logprob_naive(hidden, weight, targets, temperature=1.0, softcap=None, logit_scale=1.0):
+    """Library-routine form: full `[N, V]` fp32 logits then log_softmax / gather /
+    entropy (the expression the reference's own test uses, tests/test_utils.py:1165-1171)."""
+    z = _head_logits(hidden, weight, temperature, softcap, logit_scale)
+    lp = F.log_softmax(z, dim=-1)
+    return lp.gather(-1, targets.unsqueeze(-1)).squeeze(-1), -(lp.exp() * lp).sum(-1)
+
+
+def chunked_logprob_online(hidden, weight, targets, temperature=1.0, chunk_size=8192, softcap=None, logit_scale=1.0):
+    """Vocabulary-slab sweep with running (max, sum e, sum e*z) per row and target pick
+    (utils.py:1323-1357).  Returns (logprobs, entropy, log_z), all fp32 [N]."""
+    n = hidden.shape[0]
+    v = weight.shape[0]
+    run_max = torch.full((n,), -math.inf)
+    run_s = torch.zeros(n)
+    run_u = torch.zeros(n)
+    tgt = torch.zeros(n)
+    rows = torch.arange(n)
+    for lo in range(0, v, chunk_size):
+        hi = min(lo + chunk_size, v)
+        z = _head_logits(hidden, weight[lo:hi], temperature, softcap, logit_scale)
+        new_max = torch.maximum(run_max, z.amax(-1))
+        keep = (run_max - new_max).exp()
+        e = (z - new_max[:, None]).exp()
+        run_s = run_s * keep + e.sum(-1)
+        run_u = run_u * keep + (e * z).sum(-1)
+        run_max = new_max
+        inside = (targets >= lo) & (targets < hi)
+        tgt = tgt + z[rows, (targets - lo).clamp(0, hi - lo - 1)] * inside
+    log_z = run_max + run_s.log()
+    return tgt - log_z, log_z - run_u / run_s, log_z
+
+
+def chunked_logprob_backward(hidden, weight, targets, log_z, grad_logprobs, temperature=1.0, chunk_size=8192,
+                             softcap=None, logit_scale=1.0):
+    """Recompute each slab, dz = g * (onehot - p) with p = exp(z - log_z), chain through
+    1/T, soft-cap and logit_scale, accumulate dHidden / dW in fp32 and round once to the
+    input dtypes (utils.py:1380-1424).  The entropy output carries no gradient (:1368)."""
+    n = hidden.shape[0]
+    v = weight.shape[0]
+    g = grad_logprobs.float()
+    d_hidden = torch.zeros(hidden.shape, dtype=torch.float32)
+    d_weight = torch.zeros(weight.shape, dtype=torch.float32)
+    rows = torch.arange(n)
+    for lo in range(0, v, chunk_size):
+        hi = min(lo + chunk_size, v)
+        w_rows = weight[lo:hi]
+        y = (hidden @ w_rows.to(hidden.dtype).t()).float() * logit_scale
+        if softcap is not None:
+            th = torch.tanh(y / softcap)
+            y = th * softcap
+        z = y * (1 / temperature)
+        dz = -g[:, None] * (z - log_z[:, None]).exp()
+        inside = (targets >= lo) & (targets < hi)
+        dz[rows, (targets - lo).clamp(0, hi - lo - 1)] += g * inside
+        dz = dz * (1 / temperature)
+        if softcap is not None:
+            dz = dz * (1 - th.pow(2))
+        dz = dz * logit_scale
+        d_hidden += dz @ w_rows.float()
+        d_weight[lo:hi] += dz.t() @ hidden.float()
+    return d_hidden.to(hidden.dtype), d_weight.to(weight.dtype)
+
+
+class ChunkedLogProbOracle(torch.autograd.Function):
+    """autograd wrapper with the reference operator's argument order (utils.py:1298-1307)."""
+
+    @staticmethod
+    def forward(ctx, last_hidden, weight, targets, temperature, chunk_size, final_logit_softcapping=None, logit_scale=1.0):
+        logp, ent, log_z = chunked_logprob_online(
+            last_hidden, weight, targets, temperature, chunk_size, final_logit_softcapping, logit_scale
+        )
+        ctx.save_for_backward(last_hidden, weight, targets, log_z)
+        ctx.cfg = (temperature, chunk_size, final_logit_softcapping, logit_scale)
+        return logp, ent
+
+    @staticmethod
+    def backward(ctx, grad_logprobs, grad_entropy):
+        hidden, weight, targets, log_z = ctx.saved_tensors
+        t, c, cap, scale = ctx.cfg
+        dh, dw = chunked_logprob_backward(hidden, weight, targets, log_z, grad_logprobs, t, c, cap, scale)
+        return dh, dw, None, None, None, None, None
+
+
+# --------------------------------------------------------------------------------------
+# A15  row compaction / scatter around the fused head   trl/trainer/utils.py:1452-1481
+# --------------------------------------------------------------------------------------
+def patch_chunked_rows(hidden_states, labels, completion_mask, weight, temperature, chunk_size,
+                       softcap=None, logit_scale=1.0):
+    """Shift (utils.py:1452-1453), keep completion rows only (:1461-1465), run the fused
+    head on them, scatter into zero-filled `[B, S-1]` outputs (:1477-1481)."""
+    hs = hidden_states[:, :-1, :]
+    lab = labels[:, 1:]
+    b, s, h = hs.shape
+    flat_h = hs.reshape(b * s, h)
+    flat_t = lab.reshape(b * s)
+    keep = None
+    if completion_mask is not None:
+        keep = completion_mask[:, 1:].bool().reshape(b * s)
+        flat_h, flat_t = flat_h[keep], flat_t[keep]
+    lp_v, ent_v = ChunkedLogProbOracle.apply(flat_h, weight, flat_t, temperature, chunk_size, softcap, logit_scale)
+    if keep is None:
+        return lp_v.reshape(b, s), ent_v.reshape(b, s)
+    lp = torch.zeros(b * s, dtype=lp_v.dtype)
+    ent = torch.zeros(b * s, dtype=ent_v.dtype)
+    lp[keep] = lp_v
+    ent[keep] = ent_v
+    return lp.reshape(b, s), ent.reshape(b, s)

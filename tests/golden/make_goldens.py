@@ -1,0 +1,419 @@
+"""Writes the golden fixtures in this directory by running the *reference* implementation.
+
+Run only in the development container (needs the reference tree, default
+/root/reference; nothing here runs on the GPU box):
+
+    python tests/golden/make_goldens.py [--reference /root/reference]
+
+The reference's trainer methods are called unbound on a `Mock` trainer -- the pattern
+its own tests use (tests/test_grpo_trainer.py:95-108) -- whose `accelerator.gather /
+reduce / gather_for_metrics` are the identity and whose "model" is a callable that
+returns fixed synthetic logits.  Outputs: loss, logged metrics, per-token log-probs,
+entropies and the gradient w.r.t. the logits.  Fixtures are small `.npz` files (plain
+arrays, loadable with `allow_pickle=False`) plus a JSON index of the case settings.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+from collections import defaultdict
+from types import SimpleNamespace
+from unittest.mock import Mock
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _np(t):
+    t = t.detach()
+    if t.dtype == torch.bfloat16:
+        t = t.float()
+    return t.cpu().numpy()
+
+
+def _identity(x, *a, **k):
+    return x
+
+
+def _fake_accelerator():
+    acc = Mock()
+    acc.gather = _identity
+    acc.gather_for_metrics = _identity
+    acc.reduce = _identity
+    acc.pad_across_processes = _identity
+    acc.num_processes = 1
+    acc.device = torch.device("cpu")
+    acc.sync_gradients = True
+    return acc
+
+
+class _FixedLogitsModel:
+    """Stands in for the policy: returns clones of fixed logits, sliced like the batch."""
+
+    def __init__(self, logits):
+        self.logits = logits
+        self.training = True
+
+    def __call__(self, input_ids=None, **kw):
+        return SimpleNamespace(logits=self.logits[: input_ids.shape[0]].clone(), aux_loss=None)
+
+
+def _lengths_mask(lengths, t):
+    return (torch.arange(t)[None, :] < torch.tensor(lengths)[:, None]).long()
+
+
+# ------------------------------------------------------------------------------------ GRPO
+GRPO_CASES = [
+    dict(name="dapo_beta0", loss_type="dapo", beta=0.0, eps_low=0.2, eps_high=0.2),
+    dict(name="dapo_beta", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.28),
+    dict(name="grpo_beta", loss_type="grpo", beta=0.04, eps_low=0.2, eps_high=0.2, grad_accum=2),
+    dict(name="dr_grpo_beta", loss_type="dr_grpo", beta=0.04, eps_low=0.1, eps_high=0.3, grad_accum=4),
+    dict(name="bnpo_beta", loss_type="bnpo", beta=0.1, eps_low=0.2, eps_high=0.2),
+    dict(name="grpo_onpolicy", loss_type="grpo", beta=0.0, eps_low=0.2, eps_high=0.2, on_policy=True),
+    dict(name="dapo_delta", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, delta=1.05),
+    dict(name="grpo_seq_is", loss_type="grpo", beta=0.04, eps_low=0.05, eps_high=0.05, is_level="sequence"),
+    dict(name="dapo_bf16", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, dtype="bfloat16", temperature=0.9),
+    dict(name="grpo_temp", loss_type="grpo", beta=0.04, eps_low=0.2, eps_high=0.2, temperature=0.7),
+    dict(name="dapo_biaskl", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, bias_kl=True),
+    dict(name="grpo_offpolicy", loss_type="grpo", beta=0.0, eps_low=0.2, eps_high=0.2, off_policy=0.02),
+    dict(name="dapo_entq", loss_type="dapo", beta=0.0, eps_low=0.2, eps_high=0.2, top_entropy_quantile=0.5),
+    dict(name="grpo_entbonus", loss_type="grpo", beta=0.04, eps_low=0.2, eps_high=0.2, entropy_coef=0.01),
+    dict(name="dapo_entbonus", loss_type="dapo", beta=0.0, eps_low=0.2, eps_high=0.2, entropy_coef=0.02),
+    dict(name="dapo_emptyrow", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, empty_row=True),
+]
+
+
+def make_grpo(GRPOTrainer, out_dir):
+    index = []
+    arrays = {}
+    for ci, case in enumerate(GRPO_CASES):
+        g = torch.Generator().manual_seed(1000 + ci)
+        B, P, T, V = 6, 3, 7, 41
+        dtype = getattr(torch, case.get("dtype", "float32"))
+        temperature = case.get("temperature", 1.0)
+        logits = (2.0 * torch.randn(B, P + T, V, generator=g)).to(dtype)
+        prompt_ids = torch.randint(0, V, (B, P), generator=g)
+        completion_ids = torch.randint(0, V, (B, T), generator=g)
+        lengths = [7, 3, 5, 1, 6, 4]
+        if case.get("empty_row"):
+            lengths[3] = 0
+        completion_mask = _lengths_mask(lengths, T)
+        prompt_mask = torch.ones(B, P, dtype=torch.long)
+        advantages = torch.randn(B, generator=g)
+        advantages[1] = 0.0
+
+        trainer = Mock(spec=GRPOTrainer)
+        trainer.accelerator = _fake_accelerator()
+        trainer.temperature = temperature
+        trainer.model_kwarg_keys = set()
+        trainer._entropy_bonus_enabled = case.get("entropy_coef", 0.0) != 0.0
+        trainer.entropy_coef = case.get("entropy_coef", 0.0)
+        trainer.use_adaptive_entropy = False
+        trainer.aux_loss_enabled = False
+        trainer.top_entropy_quantile = case.get("top_entropy_quantile", 1.0)
+        trainer.off_policy_mask_threshold = case.get("off_policy")
+        trainer.importance_sampling_level = case.get("is_level", "token")
+        trainer.beta = case["beta"]
+        trainer.loss_type = case["loss_type"]
+        trainer.epsilon_low = case["eps_low"]
+        trainer.epsilon_high = case["eps_high"]
+        trainer.use_vllm = False
+        trainer.vllm_importance_sampling_correction = False
+        trainer.max_completion_length = T
+        trainer.current_gradient_accumulation_steps = case.get("grad_accum", 1)
+        trainer.args = SimpleNamespace(delta=case.get("delta"), use_bias_correction_kl=case.get("bias_kl", False))
+        trainer._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
+        trainer.model = SimpleNamespace(training=True)
+        trainer._get_per_token_logps_and_entropies = (
+            lambda *a, **k: GRPOTrainer._get_per_token_logps_and_entropies(trainer, *a, **k)
+        )
+        trainer.get_high_entropy_mask = lambda *a, **k: GRPOTrainer.get_high_entropy_mask(trainer, *a, **k)
+        trainer.get_off_policy_mask = GRPOTrainer.get_off_policy_mask
+
+        # old / ref log-probs: perturbations of the no-grad policy log-probs
+        input_ids = torch.cat([prompt_ids, completion_ids], 1)
+        attn = torch.cat([prompt_mask, completion_mask], 1)
+        with torch.no_grad():
+            base_logps, _, _ = GRPOTrainer._get_per_token_logps_and_entropies(
+                trainer, _FixedLogitsModel(logits), input_ids, attn, T, compute_entropy=False
+            )
+        base_logps = base_logps.float()
+        inputs = dict(
+            prompt_ids=prompt_ids,
+            prompt_mask=prompt_mask,
+            completion_ids=completion_ids,
+            completion_mask=completion_mask,
+            advantages=advantages,
+            num_items_in_batch=completion_mask.sum().float() * 2.0,  # as if a second, equal micro-batch existed
+        )
+        if not case.get("on_policy"):
+            inputs["old_per_token_logps"] = base_logps + 0.15 * torch.randn(B, T, generator=g)
+        if case["beta"] != 0.0:
+            inputs["ref_per_token_logps"] = base_logps + 0.3 * torch.randn(B, T, generator=g)
+
+        leaf = logits.clone().requires_grad_(True)
+
+        class _Model(_FixedLogitsModel):
+            def __call__(self, input_ids=None, **kw):
+                return SimpleNamespace(logits=leaf[: input_ids.shape[0]] * 1.0, aux_loss=None)
+
+        captured = {}
+        real = GRPOTrainer._get_per_token_logps_and_entropies
+
+        def spy(*a, **k):
+            out = real(trainer, *a, **k)
+            captured["logps"], captured["entropies"] = out[0], out[1]
+            return out
+
+        trainer._get_per_token_logps_and_entropies = spy
+        loss = GRPOTrainer._compute_loss(trainer, _Model(logits), inputs)
+        loss.backward()
+
+        pre = f"c{ci}_"
+        arrays[pre + "logits"] = _np(logits)
+        arrays[pre + "prompt_ids"] = _np(prompt_ids)
+        arrays[pre + "completion_ids"] = _np(completion_ids)
+        arrays[pre + "completion_mask"] = _np(completion_mask)
+        arrays[pre + "advantages"] = _np(advantages)
+        arrays[pre + "num_items_in_batch"] = _np(inputs["num_items_in_batch"])
+        if "old_per_token_logps" in inputs:
+            arrays[pre + "old_per_token_logps"] = _np(inputs["old_per_token_logps"])
+        if "ref_per_token_logps" in inputs:
+            arrays[pre + "ref_per_token_logps"] = _np(inputs["ref_per_token_logps"])
+        arrays[pre + "out_logps"] = _np(captured["logps"])
+        arrays[pre + "out_entropies"] = _np(captured["entropies"])
+        arrays[pre + "out_loss"] = _np(loss)
+        arrays[pre + "out_dlogits"] = _np(leaf.grad)
+        metrics = {k: float(v[-1]) for k, v in trainer._metrics["train"].items()}
+        index.append(dict(case, id=ci, shape=[B, P, T, V], metrics=metrics))
+    np.savez_compressed(os.path.join(out_dir, "grpo_compute_loss.npz"), **arrays)
+    with open(os.path.join(out_dir, "grpo_compute_loss.json"), "w") as f:
+        json.dump(index, f, indent=1)
+
+
+# ------------------------------------------------------------------------------------ DPO
+DPO_CASES = [
+    dict(name="sigmoid_f32", beta=0.1, dtype="float32"),
+    dict(name="sigmoid_beta05", beta=0.5, dtype="float32"),
+    dict(name="sigmoid_bf16", beta=0.1, dtype="bfloat16"),
+    dict(name="sigmoid_ref_equal", beta=0.1, dtype="float32", ref_equal=True),
+]
+
+
+def make_dpo(DPOTrainer, out_dir):
+    index, arrays = [], {}
+    for ci, case in enumerate(DPO_CASES):
+        g = torch.Generator().manual_seed(2000 + ci)
+        Pn, L, V = 3, 10, 37
+        B = 2 * Pn
+        dtype = getattr(torch, case["dtype"])
+        logits = (2.0 * torch.randn(B, L, V, generator=g)).to(dtype)
+        input_ids = torch.randint(0, V, (B, L), generator=g)
+        prompt_len = [2, 3, 4]
+        comp_len = [5, 4, 6, 8, 3, 2]
+        completion_mask = torch.zeros(B, L, dtype=torch.long)
+        attention_mask = torch.zeros(B, L, dtype=torch.long)
+        for i in range(B):
+            lp = prompt_len[i % Pn]
+            completion_mask[i, lp : lp + comp_len[i]] = 1
+            attention_mask[i, : lp + comp_len[i]] = 1
+
+        trainer = Mock(spec=DPOTrainer)
+        trainer.accelerator = _fake_accelerator()
+        trainer.aux_loss_enabled = False
+        trainer.ld_alpha = None
+        trainer.precompute_ref_logps = True
+        trainer.f_divergence_type = "reverse_kl"
+        trainer.loss_types = ["sigmoid"]
+        trainer.loss_weights = [1.0]
+        trainer.beta = case["beta"]
+        trainer.label_smoothing = 0.0
+        trainer.use_weighting = False
+        trainer._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
+        trainer._total_train_tokens = 0
+        trainer.model = SimpleNamespace(training=True)
+
+        leaf = logits.clone().requires_grad_(True)
+
+        def model(**kw):
+            return SimpleNamespace(logits=leaf * 1.0, aux_loss=None)
+
+        # reference log-probs: the policy's own sequence log-probs, perturbed
+        from trl.trainer.utils import selective_log_softmax as ref_sls
+
+        with torch.no_grad():
+            tok = ref_sls(logits[..., :-1, :], input_ids[..., 1:]).float()
+            tok = tok * completion_mask[..., 1:]
+            seq = tok.sum(1)
+        noise = torch.zeros(B) if case.get("ref_equal") else 0.5 * torch.randn(B, generator=g)
+        ref = seq + noise
+        if case.get("ref_equal"):
+            ref = ref.to(dtype)
+        inputs = dict(
+            input_ids=input_ids,
+            attention_mask=attention_mask,
+            completion_mask=completion_mask,
+            ref_chosen_logps=ref[:Pn],
+            ref_rejected_logps=ref[Pn:],
+        )
+        loss = DPOTrainer._compute_loss(trainer, model, inputs, False)
+        loss.backward()
+        pre = f"c{ci}_"
+        arrays[pre + "logits"] = _np(logits)
+        arrays[pre + "input_ids"] = _np(input_ids)
+        arrays[pre + "completion_mask"] = _np(completion_mask)
+        arrays[pre + "attention_mask"] = _np(attention_mask)
+        arrays[pre + "ref_chosen_logps"] = _np(ref[:Pn])
+        arrays[pre + "ref_rejected_logps"] = _np(ref[Pn:])
+        arrays[pre + "out_loss"] = _np(loss)
+        arrays[pre + "out_dlogits"] = _np(leaf.grad)
+        metrics = {k: float(v[-1]) for k, v in trainer._metrics["train"].items()}
+        index.append(dict(case, id=ci, shape=[B, L, V], metrics=metrics))
+    np.savez_compressed(os.path.join(out_dir, "dpo_compute_loss.npz"), **arrays)
+    with open(os.path.join(out_dir, "dpo_compute_loss.json"), "w") as f:
+        json.dump(index, f, indent=1)
+
+
+# ------------------------------------------------------------------------------------ RLOO
+RLOO_CASES = [
+    dict(name="rloo_sym", eps_low=0.2, eps_high=0.2, temperature=1.0),
+    dict(name="rloo_asym_temp", eps_low=0.1, eps_high=0.3, temperature=0.8),
+]
+
+
+def make_rloo(RLOOTrainer, out_dir):
+    index, arrays = [], {}
+    for ci, case in enumerate(RLOO_CASES):
+        g = torch.Generator().manual_seed(3000 + ci)
+        B, P, T, V = 6, 2, 5, 29
+        logits = 2.0 * torch.randn(B, P + T, V, generator=g)
+        prompt_ids = torch.randint(0, V, (B, P), generator=g)
+        completion_ids = torch.randint(0, V, (B, T), generator=g)
+        completion_mask = _lengths_mask([5, 2, 4, 1, 3, 5], T)
+        prompt_mask = torch.ones(B, P, dtype=torch.long)
+        advantages = torch.randn(B, generator=g)
+
+        trainer = Mock(spec=RLOOTrainer)
+        trainer.accelerator = _fake_accelerator()
+        trainer.temperature = case["temperature"]
+        trainer.model_kwarg_keys = set()
+        trainer.aux_loss_enabled = False
+        trainer.epsilon_low = case["eps_low"]
+        trainer.epsilon_high = case["eps_high"]
+        trainer._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
+        trainer.model = SimpleNamespace(training=True)
+        trainer._get_per_token_logps_and_entropies = (
+            lambda *a, **k: RLOOTrainer._get_per_token_logps_and_entropies(trainer, *a, **k)
+        )
+        input_ids = torch.cat([prompt_ids, completion_ids], 1)
+        attn = torch.cat([prompt_mask, completion_mask], 1)
+        with torch.no_grad():
+            base, _, _ = RLOOTrainer._get_per_token_logps_and_entropies(
+                trainer, _FixedLogitsModel(logits), input_ids, attn, T
+            )
+        old_logps = (base * completion_mask).sum(1) + 0.2 * torch.randn(B, generator=g)
+        leaf = logits.clone().requires_grad_(True)
+
+        def model(input_ids=None, **kw):
+            return SimpleNamespace(logits=leaf[: input_ids.shape[0]] * 1.0, aux_loss=None)
+
+        inputs = dict(
+            prompt_ids=prompt_ids,
+            prompt_mask=prompt_mask,
+            completion_ids=completion_ids,
+            completion_mask=completion_mask,
+            advantages=advantages,
+            old_logps=old_logps,
+        )
+        loss = RLOOTrainer._compute_loss(trainer, model, inputs)
+        loss.backward()
+        pre = f"c{ci}_"
+        for k, v in dict(
+            logits=logits, prompt_ids=prompt_ids, completion_ids=completion_ids, completion_mask=completion_mask,
+            advantages=advantages, old_logps=old_logps, out_loss=loss, out_dlogits=leaf.grad,
+        ).items():
+            arrays[pre + k] = _np(v)
+        metrics = {k: float(v[-1]) for k, v in trainer._metrics["train"].items()}
+        index.append(dict(case, id=ci, shape=[B, P, T, V], metrics=metrics))
+    np.savez_compressed(os.path.join(out_dir, "rloo_compute_loss.npz"), **arrays)
+    with open(os.path.join(out_dir, "rloo_compute_loss.json"), "w") as f:
+        json.dump(index, f, indent=1)
+
+
+# ------------------------------------------------------------------------------------ fused head
+HEAD_CASES = [
+    dict(name="plain", temperature=1.0, softcap=None, logit_scale=1.0, dtype="float32", chunk=32),
+    dict(name="temp", temperature=0.7, softcap=None, logit_scale=1.0, dtype="float32", chunk=48),
+    dict(name="softcap_scale", temperature=0.9, softcap=5.0, logit_scale=0.5, dtype="float32", chunk=32),
+    dict(name="bf16", temperature=0.7, softcap=None, logit_scale=1.0, dtype="bfloat16", chunk=32),
+]
+
+
+def make_head(ChunkedFn, out_dir):
+    index, arrays = [], {}
+    for ci, case in enumerate(HEAD_CASES):
+        torch.manual_seed(42)  # the seed the reference's own test uses (tests/test_utils.py:1175)
+        N, H, V = 64, 32, 128
+        dtype = getattr(torch, case["dtype"])
+        hidden = torch.randn(N, H, dtype=dtype, requires_grad=True)
+        weight = torch.randn(V, H, dtype=dtype, requires_grad=True)
+        labels = torch.randint(0, V, (N,))
+        gout = torch.randn(N)
+        lp, ent = ChunkedFn.apply(hidden, weight, labels, case["temperature"], case["chunk"], case["softcap"], case["logit_scale"])
+        (lp * gout).sum().backward()
+        pre = f"c{ci}_"
+        for k, v in dict(hidden=hidden, weight=weight, labels=labels, grad_out=gout, out_logprobs=lp, out_entropy=ent,
+                         out_dhidden=hidden.grad, out_dweight=weight.grad).items():
+            arrays[pre + k] = _np(v)
+        index.append(dict(case, id=ci, shape=[N, H, V]))
+    np.savez_compressed(os.path.join(out_dir, "chunked_logprob.npz"), **arrays)
+    with open(os.path.join(out_dir, "chunked_logprob.json"), "w") as f:
+        json.dump(index, f, indent=1)
+
+
+# ------------------------------------------------------------------------------------ utils
+def make_utils(utils, out_dir):
+    """selective_log_softmax / entropy_from_logits on bf16 and fp32 rows, incl. strided views and K > 1."""
+    g = torch.Generator().manual_seed(4000)
+    arrays = {}
+    for tag, dtype in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+        logits = (3.0 * torch.randn(3, 9, 257, generator=g)).to(dtype)
+        idx = torch.randint(0, 257, (3, 9), generator=g)
+        idxk = torch.randint(0, 257, (3, 9, 4), generator=g)
+        arrays[f"{tag}_logits"] = _np(logits)
+        arrays[f"{tag}_index"] = _np(idx)
+        arrays[f"{tag}_index_k"] = _np(idxk)
+        arrays[f"{tag}_out_logps"] = _np(utils.selective_log_softmax(logits, idx))
+        arrays[f"{tag}_out_logps_k"] = _np(utils.selective_log_softmax(logits, idxk))
+        arrays[f"{tag}_out_entropy"] = _np(utils.entropy_from_logits(logits))
+        view = logits[:, :-1, :][:, -5:, :]
+        arrays[f"{tag}_out_logps_view"] = _np(utils.selective_log_softmax(view, idx[:, -5:]))
+        arrays[f"{tag}_out_entropy_view"] = _np(utils.entropy_from_logits(view))
+    np.savez_compressed(os.path.join(out_dir, "utils_logps_entropy.npz"), **arrays)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--reference", default="/root/reference")
+    ap.add_argument("--out", default=HERE)
+    args = ap.parse_args()
+    sys.path.insert(0, args.reference)
+    import trl.trainer.utils as ref_utils
+    from trl.trainer.dpo_trainer import DPOTrainer
+    from trl.trainer.grpo_trainer import GRPOTrainer
+    from trl.trainer.rloo_trainer import RLOOTrainer
+
+    make_utils(ref_utils, args.out)
+    make_head(ref_utils._ChunkedLogProbFunction, args.out)
+    make_grpo(GRPOTrainer, args.out)
+    make_dpo(DPOTrainer, args.out)
+    make_rloo(RLOOTrainer, args.out)
+    print("golden fixtures written to", args.out)
+
+
+if __name__ == "__main__":
+    main()
