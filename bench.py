@@ -1,0 +1,241 @@
+#!/usr/bin/env python3
+"""Benchmark of the GRPO log-prob + loss forward/backward path on one MI355X.
+
+One "step" = one pass of the hot path over one synthetic batch that is already resident in HBM:
+  K1  log-prob + entropy forward over bf16 logits [64, 1024, 151936] (temperature 0.9)
+  K2  GRPO loss + metrics + d loss/d logp on [64, 1024]
+  K3  recompute backward writing dlogits [64, 1024, 151936] bf16
+(BASELINE.json config "GRPO loss fwd+bwd").  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--loss-type dapo] [--no-cpu-baseline]
+
+`value` is token positions per second over the K timed steps (events on torch's current stream,
+which is the stream the kernels are enqueued on, bracketed by device synchronisation).
+`roofline` is for the dominant kernel (K3): algorithmic bytes per launch / average launch time,
+measured live with events around K launches of that kernel alone.
+`cpu_baseline` times the CPU oracle (a port of the reference path, oracle/) on a bounded row
+sample of the same workload on this host's cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+WORKLOADS = {
+    # name: (n_seq, completion_len, vocab, temperature, group_size, min_len)
+    "grpo_c3": dict(B=64, T=1024, V=151936, temperature=0.9, G=8, min_len=64, beta=0.04, eps_low=0.2, eps_high=0.2,
+                    rewards="normal", desc="GRPO fwd+bwd, bf16 logits [64,1024,151936], T=0.9, G=8, lens~U[64,1024]"),
+    "grpo_c4": dict(B=32, T=4096, V=151936, temperature=1.0, G=16, min_len=512, beta=0.0, eps_low=0.2, eps_high=0.28,
+                    rewards="bernoulli", desc="long-context GRPO fwd+bwd, bf16 logits [32,4096,151936], G=16"),
+    "tiny": dict(B=8, T=64, V=151936, temperature=0.9, G=8, min_len=8, beta=0.04, eps_low=0.2, eps_high=0.2,
+                 rewards="normal", desc="reduced-size functional check (not a benchmark configuration)"),
+}
+
+
+def make_inputs(w, device, seed=0):
+    """Synthetic batch of the workload's shape, generated on the device one sequence at a time."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    B, T, V = w["B"], w["T"], w["V"]
+    logits = torch.empty((B, T, V), dtype=torch.bfloat16, device=device)
+    for b in range(B):
+        logits[b] = (2.0 * torch.randn((T, V), generator=g, device=device)).bfloat16()
+    ids = torch.randint(0, V, (B, T), generator=g, device=device)
+    lengths = torch.randint(w["min_len"], T + 1, (B,), generator=g, device=device)
+    mask = (torch.arange(T, device=device)[None] < lengths[:, None]).long()
+    if w["rewards"] == "normal":
+        rewards = torch.randn((B,), generator=g, device=device)
+    else:
+        rewards = (torch.rand((B,), generator=g, device=device) < 0.3).float()
+    return logits, ids, mask, rewards, g
+
+
+def cpu_baseline(w, loss_type, rows_per_seq=32, n_seq=8, repeats=2):
+    """The oracle (CPU port of the reference path: row-looped log_softmax / 128-row entropy chunks /
+    autograd backward) on a [n_seq, rows_per_seq, V] bf16 sample of the workload."""
+    import oracle
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    g = torch.Generator().manual_seed(0)
+    V, G = w["V"], min(w["G"], n_seq)
+    logits = (2.0 * torch.randn(n_seq, rows_per_seq + 1, V, generator=g)).bfloat16()
+    ids = torch.randint(0, V, (n_seq, rows_per_seq + 1), generator=g)
+    lengths = torch.randint(max(1, rows_per_seq // 16), rows_per_seq + 1, (n_seq,), generator=g)
+    mask = (torch.arange(rows_per_seq)[None] < lengths[:, None]).long()
+    adv = oracle.group_advantages(torch.randn(n_seq, generator=g), G)
+    with torch.no_grad():
+        base, _ = oracle.logps_and_entropies_from_logits(logits, ids, rows_per_seq, w["temperature"], False)
+    base = base.float()
+    old = base + 0.05 * torch.randn(base.shape, generator=g)
+    ref = base + 0.1 * torch.randn(base.shape, generator=g)
+    best = float("inf")
+    for _ in range(repeats):
+        leaf = logits.clone().requires_grad_(True)
+        t0 = time.perf_counter()
+        lp, ent = oracle.logps_and_entropies_from_logits(leaf, ids, rows_per_seq, w["temperature"], True)
+        loss, _ = oracle.grpo_loss(
+            lp, adv, mask, entropies=ent, old_per_token_logps=old, ref_per_token_logps=ref if w["beta"] else None,
+            loss_type=loss_type, epsilon_low=w["eps_low"], epsilon_high=w["eps_high"], beta=w["beta"],
+            max_completion_length=rows_per_seq, num_items_in_batch=mask.sum().float())
+        loss.backward()
+        best = min(best, time.perf_counter() - t0)
+    rows = n_seq * rows_per_seq
+    return {
+        "value": rows / best,
+        "unit": "tokens/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"oracle fwd+bwd on bf16 logits [{n_seq},{rows_per_seq}+1,{V}] ({rows} of the workload's rows), "
+                  f"best of {repeats}, {best:.2f} s; torch {torch.__version__} CPU",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="grpo_c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--loss-type", default="dapo", choices=["grpo", "dapo", "dr_grpo", "bnpo"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; rows are independent, so N GPUs would each run this same "
+                 "kernel on B/N sequences (see DESIGN.md). Run with --gpus 1.")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the hot path has no CPU fallback.")
+
+    import trl_amd
+    from trl_amd import ops
+
+    w = WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, T, V = w["B"], w["T"], w["V"]
+    R = B * T
+    logits, ids, mask, rewards, g = make_inputs(w, dev)
+    adv = trl_amd.group_advantages(rewards, w["G"])
+    with torch.no_grad():
+        base, _ = trl_amd.logps_and_entropies(logits, ids, w["temperature"])
+    old = base + 0.05 * torch.randn(base.shape, generator=g, device=dev)
+    ref = base + 0.1 * torch.randn(base.shape, generator=g, device=dev) if w["beta"] else None
+    n_items = mask.sum().float()
+    leaf = logits.requires_grad_(True)
+
+    def step():
+        leaf.grad = None
+        lp, ent = trl_amd.logps_and_entropies(leaf, ids, w["temperature"])
+        loss, metrics = trl_amd.grpo_loss(
+            lp, adv, mask, entropies=ent.detach(), old_per_token_logps=old, ref_per_token_logps=ref,
+            loss_type=args.loss_type, epsilon_low=w["eps_low"], epsilon_high=w["eps_high"], beta=w["beta"],
+            max_completion_length=T, num_items_in_batch=n_items)
+        loss.backward()
+        return loss, metrics
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        loss, metrics = step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ev_ms = e0.elapsed_time(e1)
+    ms_per_step = max(wall_ms, ev_ms) / args.steps
+    tokens_per_s = R / (ms_per_step * 1e-3)
+    loss_value = float(loss)
+    assert loss_value == loss_value, "loss is NaN"
+
+    # ---- per-kernel timing: each kernel alone, events around `reps` back-to-back launches -----------
+    idx = ids.reshape(R, 1)
+    with torch.no_grad():
+        lp_flat, ent_flat, lse = ops.logp_entropy_fwd(logits.detach(), idx, w["temperature"], 0, T, None)
+    g_logp = (leaf.grad is not None) and None
+    loss2, _, dlogp, _ = ops.grpo_loss_op(
+        lp_flat.view(B, T), old, ref, ent_flat.view(B, T), adv, mask, None, None, n_items,
+        ops.LOSS_TYPES[args.loss_type], w["eps_low"], w["eps_high"], float("nan"), w["beta"], False, 1.0,
+        float(B * T), 1.0, 0.0)
+    g_logp = dlogp.reshape(R, 1).contiguous()
+    leaf.grad = None
+    reps = max(3, min(args.steps, 10))
+
+    def time_kernel(fn):
+        fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            out = fn()
+            del out
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps
+
+    with torch.no_grad():
+        fwd_ms = time_kernel(lambda: ops.logp_entropy_fwd(logits.detach(), idx, w["temperature"], 0, T, None))
+        bwd_ms = time_kernel(lambda: ops.logp_entropy_bwd(logits.detach(), idx, w["temperature"], 0, T, lse, None,
+                                                          g_logp, None))
+    row_bytes = V * 2
+    active_rows = int((g_logp != 0).sum())
+    fwd_bytes = R * row_bytes
+    bwd_bytes = active_rows * 2 * row_bytes + (R - active_rows) * row_bytes  # masked rows: zero-fill write only
+    fwd_gbps = fwd_bytes / (fwd_ms * 1e-3) / 1e9
+    bwd_gbps = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "tokens/sec + achieved HBM TB/s (% of peak) for GRPO logprob+loss fwd+bwd",
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "description": w["desc"], "rows": R, "vocab": V,
+                   "loss_type": args.loss_type, "active_rows": active_rows, "loss": loss_value},
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "logp_entropy_bwd_kernel (K3)",
+            "achieved": bwd_gbps,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": bwd_gbps / HBM_PEAK_GBPS,
+            "traffic": None,
+            "algorithmic_bytes": bwd_bytes,
+            "avg_launch_ms": bwd_ms,
+        },
+        "kernels": {
+            "logp_entropy_fwd_kernel (K1)": {"avg_launch_ms": fwd_ms, "algorithmic_bytes": fwd_bytes,
+                                             "achieved_GBps": fwd_gbps, "frac": fwd_gbps / HBM_PEAK_GBPS},
+            "logp_entropy_bwd_kernel (K3)": {"avg_launch_ms": bwd_ms, "algorithmic_bytes": bwd_bytes,
+                                             "achieved_GBps": bwd_gbps, "frac": bwd_gbps / HBM_PEAK_GBPS},
+            "step_hbm_GBps": (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9,
+        },
+    }
+    if not args.no_cpu_baseline:
+        del leaf, logits
+        torch.cuda.empty_cache()
+        result["cpu_baseline"] = cpu_baseline(w, args.loss_type)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

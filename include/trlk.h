@@ -1,0 +1,195 @@
+/*
+ * trlk -- C ABI of the MI355X (gfx950) kernels for TRL's per-token log-probability,
+ * entropy and policy-loss path.
+ *
+ * Conventions (all entry points):
+ *   - every pointer named `d_*` is DEVICE memory owned by the caller; the library never
+ *     allocates, frees or keeps a pointer after the call returns;
+ *   - calls only enqueue work on `stream` (a hipStream_t passed as void*; NULL = the
+ *     default stream) and never synchronise the host;
+ *   - return value: 0 = enqueued; negative = argument error found on the host before
+ *     anything was launched (see trlk_status, text in trlk_last_error()); positive =
+ *     the hipError_t of a failed launch;
+ *   - "rows" are token positions.  A logits operand is a strided 3-D view
+ *     [n_seq, rows_per_seq, vocab] whose last axis is contiguous: element (b, t, v) is at
+ *     `base + b*seq_stride + t*row_stride + v` (strides in ELEMENTS).  Per-row operands
+ *     (indices, log-probs, masks, gradients) are dense row-major [n_seq*rows_per_seq(, K)].
+ *
+ * The reference has no native code; each entry point names the Python lines whose
+ * arithmetic it replaces (paths relative to the reference tree).
+ */
+#ifndef TRLK_H
+#define TRLK_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TRLK_VERSION 1
+
+typedef void* trlk_stream_t; /* hipStream_t */
+
+enum trlk_dtype { TRLK_F32 = 0, TRLK_BF16 = 1, TRLK_F16 = 2 };
+
+enum trlk_status {
+    TRLK_OK = 0,
+    TRLK_ERR_NULL_POINTER = -1,
+    TRLK_ERR_BAD_SHAPE = -2,
+    TRLK_ERR_BAD_DTYPE = -3,
+    TRLK_ERR_BAD_STRIDE = -4,
+    TRLK_ERR_BAD_VALUE = -5,
+    TRLK_ERR_WORKSPACE = -6,
+    TRLK_ERR_UNSUPPORTED = -7
+};
+
+/* loss normalisations of GRPOTrainer._compute_loss (trl/trainer/grpo_trainer.py:3124-3142) */
+enum trlk_grpo_loss_type { TRLK_GRPO = 0, TRLK_BNPO = 1, TRLK_DR_GRPO = 2, TRLK_DAPO = 3 };
+
+/* scale_rewards modes (trl/trainer/grpo_trainer.py:2687-2707) */
+enum trlk_scale_rewards { TRLK_SCALE_GROUP = 0, TRLK_SCALE_BATCH = 1, TRLK_SCALE_NONE = 2 };
+
+/* bits of the int32 word the kernels OR into `d_error_flag` */
+#define TRLK_FLAG_INDEX_OUT_OF_RANGE 1
+
+int trlk_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char* trlk_last_error(void);
+
+/* ---------------------------------------------------------------------------------------
+ * K1  log-prob + entropy forward, one streaming pass over the logits.
+ * Replaces selective_log_softmax (trl/trainer/utils.py:479-523), entropy_from_logits
+ * (utils.py:526-560) and the temperature division in front of them
+ * (trl/trainer/grpo_trainer.py:1519): with z = logits / temperature,
+ *   out_logp[r, k] = z[r, index[r, k]] - logsumexp(z[r, :])
+ *   out_entropy[r] = logsumexp(z[r, :]) - sum_v softmax(z[r])_v * z[r, v]
+ *   out_lse[r]     = logsumexp(z[r, :])            (the only state the backward needs)
+ * All arithmetic is fp32 whatever `dtype` is; outputs are fp32.
+ * d_index: int64 [rows, n_index].  d_row_mask (optional, uint8 [rows]): rows whose mask is 0
+ * are not read and get 0 in every output.  d_out_entropy / d_out_lse / d_error_flag may be
+ * NULL.  An index outside [0, vocab) yields NaN for that entry and sets
+ * TRLK_FLAG_INDEX_OUT_OF_RANGE in *d_error_flag.
+ */
+int trlk_logp_entropy_fwd(const void* d_logits, int dtype, int64_t n_seq, int64_t rows_per_seq, int64_t vocab,
+                          int64_t seq_stride, int64_t row_stride, const int64_t* d_index, int32_t n_index,
+                          float temperature, const uint8_t* d_row_mask, float* d_out_logp, float* d_out_entropy,
+                          float* d_out_lse, int32_t* d_error_flag, trlk_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * K3  backward of K1 by recomputation from the saved lse: one read and one write of the
+ * logits-sized data.  Replaces autograd's log_softmax / gather / div / slice backward chain
+ * behind utils.py:506-518 and grpo_trainer.py:1514-1519:
+ *   dlogits[r, v] = ( sum_k g_logp[r,k] * (1[v == index[r,k]] - p_v)
+ *                     - g_entropy[r] * p_v * ((z_v - lse_r) + H_r) ) / temperature,  p_v = exp(z_v - lse_r)
+ * The output is a strided [n_seq, out_rows_per_seq, vocab] tensor of the same dtype as the
+ * logits; the rows_per_seq input rows of a sequence land at output rows
+ * [out_row_offset, out_row_offset + rows_per_seq) and every other output row is zero-filled
+ * (the zero padding of the slice backward).  Rows whose upstream gradients are all exactly
+ * zero are zero-filled without reading the logits.
+ * d_g_entropy and d_entropy may be NULL together (no entropy gradient).
+ */
+int trlk_logp_entropy_bwd(const void* d_logits, int dtype, int64_t n_seq, int64_t rows_per_seq, int64_t vocab,
+                          int64_t seq_stride, int64_t row_stride, const int64_t* d_index, int32_t n_index,
+                          float temperature, const float* d_lse, const float* d_entropy, const float* d_g_logp,
+                          const float* d_g_entropy, void* d_dlogits, int64_t out_rows_per_seq, int64_t out_row_offset,
+                          int64_t out_seq_stride, int64_t out_row_stride, trlk_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * K2a  group-relative advantages (trl/trainer/grpo_trainer.py:2685-2707, 2730 with nanstd,
+ * trl/trainer/utils.py:874-880).  d_rewards fp32 [n] (NaN = unscorable), groups are
+ * `group_size` consecutive entries, n % group_size == 0.
+ *   adv = (r - nanmean_group) / (nanstd + 1e-4), NaN -> 0; nanstd per group, over the batch,
+ *   or no division, per `scale_mode` (trlk_scale_rewards).
+ */
+int trlk_group_advantages(const float* d_rewards, int64_t n, int32_t group_size, int32_t scale_mode,
+                          float* d_out_advantages, trlk_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * K2  GRPO clipped-surrogate loss, its metrics and d(loss)/d(logp) in one call
+ * (trl/trainer/grpo_trainer.py:3054-3150 token-level importance weights, :3155-3181 entropy
+ * bonus, :3224-3253 metrics).  All [B, T] operands are dense fp32.
+ *   d_old_logp  NULL  -> old = logp (on-policy, :3037)
+ *   d_ref_logp  NULL  -> requires beta == 0
+ *   d_entropy   NULL  -> no entropy metric / bonus
+ *   d_token_weight NULL -> 1; otherwise multiplies the policy term before the KL is added
+ *                  (product of the off-policy, entropy-quantile and importance-sampling
+ *                  factors of :3111-3118)
+ *   d_entropy_mask NULL -> 1; extra factor on the mask of the entropy bonus (:3158)
+ *   advantages: element (b, t) at d_advantages[b*adv_stride_b + t*adv_stride_t]
+ *   delta: NaN = no upper clamp of the ratio (:3086-3087)
+ *   d_dapo_normalizer: device scalar holding num_items_in_batch (DAPO only, :3140)
+ *   dr_grpo_denominator: B * max_completion_length (:3135)
+ * Outputs: d_out_loss [1]; d_out_metrics [TRLK_GRPO_NUM_METRICS]; d_out_dlogp [B, T] =
+ * d loss / d logp; d_out_dentropy [B, T] (may be NULL unless entropy_coef != 0).
+ * Reductions run in a fixed order: results are bit-reproducible.
+ * d_workspace: trlk_grpo_workspace_bytes(B) bytes.
+ */
+enum trlk_grpo_metric {
+    TRLK_M_KL_MEAN = 0,          /* masked mean of the k3 KL (NaN if beta == 0) */
+    TRLK_M_ENTROPY_MEAN = 1,     /* masked mean entropy (NaN if no entropy given) */
+    TRLK_M_CLIP_LOW_MEAN = 2,
+    TRLK_M_CLIP_HIGH_MEAN = 3,
+    TRLK_M_CLIP_REGION_MEAN = 4,
+    TRLK_M_CLIP_LOW_MIN = 5,     /* min over sequences of the per-sequence mean, NaN rows skipped */
+    TRLK_M_CLIP_HIGH_MAX = 6,
+    TRLK_M_POLICY_LOSS = 7,      /* loss before the entropy bonus and before /grad_accum (:3127) */
+    TRLK_M_MASK_SUM = 8,
+    TRLK_M_KL_SUM = 9,
+    TRLK_M_ENTROPY_SUM = 10,
+    TRLK_GRPO_NUM_METRICS = 16
+};
+
+size_t trlk_grpo_workspace_bytes(int64_t n_seq);
+
+int trlk_grpo_loss(const float* d_logp, const float* d_old_logp, const float* d_ref_logp, const float* d_entropy,
+                   const float* d_advantages, int64_t adv_stride_b, int64_t adv_stride_t, const float* d_mask,
+                   const float* d_token_weight, const float* d_entropy_mask, int64_t n_seq, int64_t seq_len,
+                   int32_t loss_type, float epsilon_low, float epsilon_high, float delta, float beta,
+                   int32_t use_bias_correction_kl, float grad_accum_steps, float dr_grpo_denominator,
+                   const float* d_dapo_normalizer, float num_processes, float entropy_coef, float* d_out_loss,
+                   float* d_out_metrics, float* d_out_dlogp, float* d_out_dentropy, void* d_workspace,
+                   size_t workspace_bytes, trlk_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * K4  sequence-level losses on top of per-token log-probs.
+ *
+ * trlk_dpo_loss: DPO sequence log-probs and sigmoid loss (trl/trainer/dpo_trainer.py:1348-1350,
+ * 1362, 1396-1402, 1430-1435, 1578).  d_token_logp, d_mask: dense fp32 [n_seq, seq_len]
+ * (already shifted); n_seq is even, first half chosen, second half rejected.
+ *   seq[b]  = sum_t logp[b,t] * 1[mask[b,t] != 0]
+ *   delta_p = (seq_c - ref_c) - (seq_r - ref_r);  loss = mean_p -logsigmoid(beta * delta_p)
+ * Outputs: d_out_seq_logps [n_seq], d_out_loss [1], d_out_metrics [TRLK_DPO_NUM_METRICS],
+ * d_out_dlogp [n_seq, seq_len] = d loss / d token_logp.
+ */
+enum trlk_dpo_metric {
+    TRLK_D_REWARD_CHOSEN = 0,    /* mean beta*(seq_c - ref_c)   (dpo_trainer.py:1634-1639) */
+    TRLK_D_REWARD_REJECTED = 1,
+    TRLK_D_REWARD_ACCURACY = 2,
+    TRLK_D_REWARD_MARGIN = 3,
+    TRLK_D_LOGPS_CHOSEN = 4,
+    TRLK_D_LOGPS_REJECTED = 5,
+    TRLK_DPO_NUM_METRICS = 8
+};
+
+int trlk_dpo_loss(const float* d_token_logp, const float* d_mask, const float* d_ref_chosen,
+                  const float* d_ref_rejected, int64_t n_seq, int64_t seq_len, float beta, float* d_out_seq_logps,
+                  float* d_out_loss, float* d_out_metrics, float* d_out_dlogp, trlk_stream_t stream);
+
+/* trlk_rloo_loss: RLOO sequence-level clipped loss (trl/trainer/rloo_trainer.py:1683-1694,
+ * 1711-1721).  seq[b] = sum_t logp*mask; ratio = exp(seq - old_seq); loss = mean_b
+ * -min(ratio*A, clamp(ratio, 1-eps_low, 1+eps_high)*A).
+ * Metrics: [0] low_mean [1] low_min [2] high_mean [3] high_max [4] region_mean.
+ */
+#define TRLK_RLOO_NUM_METRICS 8
+int trlk_rloo_loss(const float* d_token_logp, const float* d_mask, const float* d_old_seq_logps,
+                   const float* d_advantages, int64_t n_seq, int64_t seq_len, float epsilon_low, float epsilon_high,
+                   float* d_out_seq_logps, float* d_out_loss, float* d_out_metrics, float* d_out_dlogp,
+                   trlk_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRLK_H */

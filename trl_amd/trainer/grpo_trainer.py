@@ -1,0 +1,277 @@
+"""The log-prob / loss part of the reference's `GRPOTrainer`, as mix-in methods with the
+reference's signatures plus the functional forms they are built from.
+
+`GRPOLossMixin._get_per_token_logps_and_entropies` and `GRPOLossMixin._compute_loss` read the
+same trainer attributes and `inputs` keys as the reference methods
+(trl/trainer/grpo_trainer.py:1435-1541, 2991-3260) and can be bound onto a `GRPOTrainer`
+(see `trl_amd.integration.patch_trl`).  Differences, all deliberate:
+  * the logits are never divided in place; the temperature is applied inside the kernel;
+  * log-probs and entropies come back in fp32 whatever the logits dtype;
+  * one kernel call returns every metric; they reach the host in a single copy.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+from torch import Tensor
+
+from .. import _lib, ops
+from .utils import logps_and_entropies, nanmax, nanmin  # noqa: F401  (re-exported for callers that patch)
+
+__all__ = [
+    "per_token_logps_and_entropies",
+    "grpo_loss",
+    "group_advantages",
+    "get_off_policy_mask",
+    "get_high_entropy_mask",
+    "GRPOLossMixin",
+]
+
+group_advantages = ops.group_advantages
+
+
+def per_token_logps_and_entropies(
+    logits: Tensor, input_ids: Tensor, logits_to_keep: int, temperature: float = 1.0, compute_entropy: bool = True,
+    entropy_requires_grad: bool = False,
+) -> tuple[Tensor, Tensor | None]:
+    """`[B, L, V]` model logits -> fp32 `(logps [B, K], entropies [B, K] | None)` for the last
+    `K = logits_to_keep` tokens of `input_ids`: drops the last position, keeps the last K, divides by
+    the temperature (trl/trainer/grpo_trainer.py:1514-1521) -- as index arithmetic on the full tensor,
+    so the backward writes the `[B, L, V]` gradient directly (rows outside the window zero)."""
+    if logits.dim() != 3:
+        raise ValueError("expected [B, L, V] logits")
+    length = logits.shape[1]
+    keep_len = min(logits_to_keep, length - 1)
+    keep_start = length - 1 - keep_len
+    ids = input_ids[:, -keep_len:] if keep_len > 0 else input_ids[:, :0]
+    if logits.shape[-1] > 1 and logits.stride(-1) != 1:
+        logits = logits.contiguous()
+    logp, ent = logps_and_entropies(logits, ids, temperature, keep_start, keep_len)
+    if not compute_entropy:
+        return logp, None
+    return logp, (ent if entropy_requires_grad else ent.detach())
+
+
+def get_off_policy_mask(advantages, per_token_logps, sampling_per_token_logps, mask, off_policy_threshold):
+    """(B, 1) keep-mask of trl/trainer/grpo_trainer.py:2920-2939 ([B, T]-sized torch ops)."""
+    gap = sampling_per_token_logps - per_token_logps.detach()
+    mean_gap = (gap * mask).sum(dim=1, keepdim=True) / mask.sum(dim=1, keepdim=True).clamp(min=1.0)
+    return ((advantages >= 0) | (mean_gap <= off_policy_threshold)).to(dtype=mask.dtype)
+
+
+def get_high_entropy_mask(entropies, mask, threshold, accelerator=None):
+    """Boolean mask of the tokens at or above the `threshold` entropy quantile
+    (trl/trainer/grpo_trainer.py:1396-1432); with an `accelerator` the active entropies are padded
+    and gathered across processes first, as the reference does."""
+    local = entropies[mask.bool()].float()
+    if accelerator is not None:
+        pad_value = -1e9
+        gathered = accelerator.gather(accelerator.pad_across_processes(local, dim=0, pad_index=pad_value))
+        gathered = gathered[gathered != pad_value]
+    else:
+        gathered = local
+    if gathered.numel() == 0:
+        return torch.zeros_like(entropies, dtype=torch.bool)
+    cut = torch.quantile(gathered, threshold)
+    return ((entropies * mask.float()) >= cut) & mask.bool()
+
+
+def grpo_loss(
+    per_token_logps: Tensor,
+    advantages: Tensor,
+    mask: Tensor,
+    *,
+    entropies: Tensor | None = None,
+    old_per_token_logps: Tensor | None = None,
+    ref_per_token_logps: Tensor | None = None,
+    loss_type: str = "dapo",
+    epsilon_low: float = 0.2,
+    epsilon_high: float = 0.2,
+    beta: float = 0.0,
+    delta: float | None = None,
+    max_completion_length: int | None = None,
+    num_items_in_batch: Tensor | float | None = None,
+    num_processes: int = 1,
+    grad_accum_steps: float = 1.0,
+    use_bias_correction_kl: bool = False,
+    token_weight: Tensor | None = None,
+    entropy_mask: Tensor | None = None,
+    entropy_coef: float = 0.0,
+) -> tuple[Tensor, Tensor]:
+    """Fused GRPO-family loss (token-level importance weights) on `[B, T]` log-probs.
+
+    Returns `(loss, metrics)`; `metrics` is the fp32 device vector indexed by
+    `trl_amd._lib`'s `trlk_grpo_metric` order (see include/trlk.h).  Differentiable w.r.t.
+    `per_token_logps` (and `entropies` when `entropy_coef != 0`)."""
+    if loss_type not in ops.LOSS_TYPES:
+        raise ValueError(f"Unknown loss type: {loss_type}")
+    if beta != 0.0 and ref_per_token_logps is None:
+        raise KeyError("ref_per_token_logps")
+    dev = per_token_logps.device
+    dapo_norm = None
+    dr_denominator = 1.0
+    if loss_type == "dapo":
+        if num_items_in_batch is None:
+            raise KeyError("num_items_in_batch")
+        dapo_norm = (
+            num_items_in_batch.to(device=dev, dtype=torch.float32)
+            if torch.is_tensor(num_items_in_batch)
+            else torch.tensor(float(num_items_in_batch), dtype=torch.float32, device=dev)
+        )
+    if loss_type == "dr_grpo":
+        if max_completion_length is None:
+            raise ValueError("dr_grpo needs max_completion_length")
+        dr_denominator = float(per_token_logps.shape[0] * max_completion_length)
+    loss, metrics, _, _ = ops.grpo_loss_op(
+        per_token_logps, old_per_token_logps, ref_per_token_logps if beta != 0.0 else None, entropies, advantages,
+        mask, token_weight, entropy_mask, dapo_norm, ops.LOSS_TYPES[loss_type], float(epsilon_low),
+        float(epsilon_high), math.nan if delta is None else float(delta), float(beta), bool(use_bias_correction_kl),
+        float(grad_accum_steps), dr_denominator, float(num_processes), float(entropy_coef),
+    )
+    return loss, metrics
+
+
+class GRPOLossMixin:
+    """Methods with the reference's names and signatures; bind them onto a `GRPOTrainer`."""
+
+    def _get_per_token_logps_and_entropies(
+        self, model, input_ids, attention_mask, logits_to_keep, batch_size=None, compute_entropy=False,
+        compute_aux_loss=False, **model_extra_inputs,
+    ):
+        """Reference: trl/trainer/grpo_trainer.py:1435-1541.  Multimodal extras are forwarded to the
+        model only when the whole batch goes through in one piece (no per-sample splitting here)."""
+        batch_size = batch_size or input_ids.size(0)
+        extras = {k: v for k, v in model_extra_inputs.items() if v is not None}
+        if extras and batch_size < input_ids.size(0):
+            raise NotImplementedError("sub-batching of multimodal inputs is not supported by trl_amd")
+        all_logps, all_entropies, all_aux = [], [], []
+        entropy_grad = bool(getattr(self, "_entropy_bonus_enabled", False))
+        for start in range(0, input_ids.size(0), batch_size):
+            ids = input_ids[start : start + batch_size]
+            model_inputs = {"input_ids": ids, "attention_mask": attention_mask[start : start + batch_size], **extras}
+            if "logits_to_keep" in getattr(self, "model_kwarg_keys", ()):
+                model_inputs["logits_to_keep"] = logits_to_keep + 1
+            model_inputs["use_cache"] = False
+            if compute_aux_loss:
+                model_inputs["output_router_logits"] = True
+            outputs = model(**model_inputs)
+            logps, ent = per_token_logps_and_entropies(
+                outputs.logits, ids, logits_to_keep, self.temperature, compute_entropy, entropy_grad
+            )
+            all_logps.append(logps)
+            if compute_entropy:
+                all_entropies.append(ent)
+            if compute_aux_loss:
+                all_aux.append(outputs.aux_loss)
+        logps = torch.cat(all_logps, dim=0) if len(all_logps) > 1 else all_logps[0]
+        entropies = (torch.cat(all_entropies, dim=0) if len(all_entropies) > 1 else all_entropies[0]) if compute_entropy else None
+        aux_loss = torch.stack(all_aux).mean() if compute_aux_loss else None
+        return logps, entropies, aux_loss
+
+    def _compute_loss(self, model, inputs):
+        """Reference: trl/trainer/grpo_trainer.py:2991-3260 for loss types grpo / bnpo / dr_grpo / dapo
+        with token-level importance weights."""
+        if self.loss_type not in ops.LOSS_TYPES:
+            raise NotImplementedError(f"loss_type={self.loss_type!r} is not implemented by trl_amd")
+        if self.importance_sampling_level != "token":
+            raise NotImplementedError("importance_sampling_level='sequence' is not implemented by trl_amd")
+        if getattr(self, "use_adaptive_entropy", False):
+            raise NotImplementedError("adaptive entropy control is not implemented by trl_amd")
+        prompt_ids, prompt_mask = inputs["prompt_ids"], inputs["prompt_mask"]
+        completion_ids, completion_mask = inputs["completion_ids"], inputs["completion_mask"]
+        input_ids = torch.cat([prompt_ids, completion_ids], dim=1)
+        attention_mask = torch.cat([prompt_mask, completion_mask], dim=1)
+        logits_to_keep = completion_ids.size(1)
+        mask = completion_mask if "tool_mask" not in inputs else completion_mask * inputs["tool_mask"]
+        aux_enabled = bool(getattr(self, "aux_loss_enabled", False))
+        extra_keys = ("pixel_values", "image_grid_thw", "num_images", "pixel_attention_mask", "spatial_shapes",
+                      "num_tiles", "image_sizes", "token_type_ids", "mm_token_type_ids", "image_position_ids")
+        per_token_logps, entropies, aux_loss = self._get_per_token_logps_and_entropies(
+            model, input_ids, attention_mask, logits_to_keep, compute_entropy=True, compute_aux_loss=aux_enabled,
+            **{k: inputs.get(k) for k in extra_keys},
+        )
+        advantages = inputs["advantages"]
+        entropy_mask = None
+        if self.top_entropy_quantile < 1.0:
+            entropy_mask = get_high_entropy_mask(entropies.detach(), mask, 1 - self.top_entropy_quantile, self.accelerator)
+        token_weight = None
+        old = inputs.get("old_per_token_logps")
+        if self.off_policy_mask_threshold is not None:
+            adv2 = advantages.unsqueeze(1) if advantages.dim() == 1 else advantages
+            sampling = inputs.get("sampling_per_token_logps", per_token_logps.detach() if old is None else old)
+            token_weight = get_off_policy_mask(adv2, per_token_logps, sampling, mask, self.off_policy_mask_threshold)
+            token_weight = token_weight.float().expand_as(per_token_logps)
+        if entropy_mask is not None:
+            em = entropy_mask.float()
+            token_weight = em if token_weight is None else token_weight * em
+        if self.use_vllm and self.vllm_importance_sampling_correction:
+            isr = inputs["importance_sampling_ratio"].float().expand_as(per_token_logps)
+            token_weight = isr if token_weight is None else token_weight * isr
+
+        mode = "train" if self.model.training else "eval"
+        grad_accum = self.current_gradient_accumulation_steps if mode == "train" else 1.0
+        bonus = bool(getattr(self, "_entropy_bonus_enabled", False))
+        loss, metrics = grpo_loss(
+            per_token_logps, advantages, mask, entropies=entropies, old_per_token_logps=old,
+            ref_per_token_logps=inputs["ref_per_token_logps"] if self.beta != 0.0 else None,
+            loss_type=self.loss_type, epsilon_low=self.epsilon_low, epsilon_high=self.epsilon_high, beta=self.beta,
+            delta=self.args.delta, max_completion_length=self.max_completion_length,
+            num_items_in_batch=inputs.get("num_items_in_batch"), num_processes=self.accelerator.num_processes,
+            grad_accum_steps=grad_accum, use_bias_correction_kl=self.args.use_bias_correction_kl,
+            token_weight=token_weight, entropy_mask=None if entropy_mask is None else entropy_mask.float(),
+            entropy_coef=self.entropy_coef if bonus else 0.0,
+        )
+        if aux_enabled:
+            loss = loss + self.router_aux_loss_coef * aux_loss / grad_accum
+            self._metrics[mode]["aux_loss"].append(self.accelerator.gather_for_metrics(aux_loss).mean().item())
+
+        # metrics: cross-process sums of (sum, count) pairs, then one host copy
+        m = metrics.detach()
+        sums = torch.stack([m[_lib_metric("KL_SUM")], m[_lib_metric("ENTROPY_SUM")], m[_lib_metric("MASK_SUM")]])
+        clip = m[2:5] * m[_lib_metric("MASK_SUM")].clamp(min=1.0)
+        totals = self.accelerator.reduce(torch.cat([sums, clip]), reduction="sum")
+        low_min = nanmin(self.accelerator.gather(m[5:6]))
+        high_max = nanmax(self.accelerator.gather(m[6:7]))
+        host = torch.cat([totals, low_min.reshape(1), high_max.reshape(1), m[7:8]]).tolist()
+        kl_sum, ent_sum, cnt, low, high, region, lmin, hmax, policy_loss = host
+        cnt = max(cnt, 1.0)
+        log = self._metrics[mode]
+        if bonus:
+            log["policy_loss"].append(policy_loss)
+            if mode == "train" and self.accelerator.sync_gradients:
+                log["entropy_coef"].append(self.entropy_coef)
+        if self.beta != 0.0:
+            log["kl"].append(kl_sum / cnt)
+        log["entropy"].append(ent_sum / cnt)
+        log["clip_ratio/low_mean"].append(low / cnt)
+        log["clip_ratio/high_mean"].append(high / cnt)
+        log["clip_ratio/region_mean"].append(region / cnt)
+        log["clip_ratio/low_min"].append(lmin)
+        log["clip_ratio/high_max"].append(hmax)
+        return loss
+
+
+_METRIC_INDEX = {"KL_MEAN": 0, "ENTROPY_MEAN": 1, "CLIP_LOW_MEAN": 2, "CLIP_HIGH_MEAN": 3, "CLIP_REGION_MEAN": 4,
+                 "CLIP_LOW_MIN": 5, "CLIP_HIGH_MAX": 6, "POLICY_LOSS": 7, "MASK_SUM": 8, "KL_SUM": 9, "ENTROPY_SUM": 10}
+
+
+def _lib_metric(name: str) -> int:
+    return _METRIC_INDEX[name]
+
+
+def metrics_to_dict(metrics: Tensor, beta: float, has_entropy: bool = True) -> dict[str, float]:
+    """Host dictionary with the reference's metric names (single device->host copy)."""
+    m = metrics.detach().tolist()
+    out = {}
+    if beta != 0.0:
+        out["kl"] = m[0]
+    if has_entropy:
+        out["entropy"] = m[1]
+    out["clip_ratio/low_mean"] = m[2]
+    out["clip_ratio/high_mean"] = m[3]
+    out["clip_ratio/region_mean"] = m[4]
+    out["clip_ratio/low_min"] = m[5]
+    out["clip_ratio/high_max"] = m[6]
+    out["policy_loss"] = m[7]
+    return out

@@ -1,0 +1,136 @@
+"""Drop-in counterparts of the hot-path helpers in the reference's `trl/trainer/utils.py`.
+
+Same names, argument meaning and error behaviour as the reference functions; the arithmetic
+runs in the HIP kernels behind `trl_amd.ops` (device tensors only).
+"""
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+
+from .. import ops
+
+__all__ = ["selective_log_softmax", "entropy_from_logits", "logps_and_entropies", "nanstd", "nanmin", "nanmax"]
+
+
+def _as_3d(logits: Tensor) -> Tensor:
+    """View `[..., V]` logits as `[n_seq, rows, V]` without copying when the strides allow it."""
+    if logits.dim() == 0:
+        raise ValueError("logits must have at least one dimension")
+    v = logits.shape[-1]
+    if v > 1 and logits.stride(-1) != 1:
+        logits = logits.contiguous()
+    if logits.dim() == 1:
+        return logits.view(1, 1, v)
+    if logits.dim() == 2:
+        out = logits.unsqueeze(0)
+    elif logits.dim() == 3:
+        out = logits
+    else:
+        try:
+            out = logits.view(-1, logits.shape[-2], v)
+        except RuntimeError:
+            out = logits.reshape(-1, logits.shape[-2], v)
+    if out.shape[1] > 1 and out.stride(1) < v:  # expanded / overlapping rows
+        out = out.contiguous()
+    return out
+
+
+def logps_and_entropies(
+    logits: Tensor, index: Tensor, temperature: float = 1.0, keep_start: int = 0, keep_len: int | None = None,
+    row_mask: Tensor | None = None,
+) -> tuple[Tensor, Tensor]:
+    """One streaming pass over `[n_seq, L, V]` logits: fp32 log-probs of `index` and fp32 entropies
+    of rows `keep_start .. keep_start + keep_len` of every sequence, of `softmax(logits / temperature)`.
+    `index` is `[n_seq, keep_len]` or `[n_seq, keep_len, K]`.  Differentiable w.r.t. `logits` (both
+    outputs); the gradient covers all `L` rows (zero outside the window).  With `row_mask`
+    (`[n_seq, keep_len]`, zero = skip) masked rows are not read and yield 0."""
+    if logits.dim() != 3:
+        raise ValueError("logps_and_entropies expects [n_seq, L, V] logits")
+    n_seq, length, _ = logits.shape
+    keep_len = length - keep_start if keep_len is None else keep_len
+    if keep_start < 0 or keep_len < 0 or keep_start + keep_len > length:
+        raise ValueError(f"rows [{keep_start}, {keep_start + keep_len}) are outside the {length} rows of the logits")
+    squeeze = index.dim() == 2
+    idx = index.reshape(n_seq * keep_len, -1)
+    if idx.dtype != torch.int64:
+        idx = idx.long()
+    rm = None
+    if row_mask is not None:
+        rm = (row_mask.reshape(-1) != 0).to(torch.uint8).contiguous()
+    logp, ent, _ = ops.logp_entropy_fwd(logits, idx, float(temperature), keep_start, keep_len, rm)
+    logp = logp.view(n_seq, keep_len) if squeeze else logp.view(n_seq, keep_len, -1)
+    return logp, ent.view(n_seq, keep_len)
+
+
+def selective_log_softmax(logits: Tensor, index: Tensor, out_dtype: torch.dtype | None = None) -> Tensor:
+    """`torch.gather(logits.log_softmax(-1), -1, index)` without materialising the log-softmax
+    (reference: trl/trainer/utils.py:479-523).  `index` has shape `(...)` or `(..., K)`.
+
+    The kernel always computes in fp32.  `out_dtype=None` returns the logits dtype as the
+    reference does (for bf16/fp16 logits the fp32 result is rounded once to that dtype);
+    `out_dtype=torch.float32` keeps the unrounded values."""
+    squeeze = index.dim() == logits.dim() - 1
+    if not squeeze and index.dim() != logits.dim():
+        raise ValueError(f"index of shape {tuple(index.shape)} does not match logits of shape {tuple(logits.shape)}")
+    if tuple(index.shape[: logits.dim() - 1]) != tuple(logits.shape[:-1]):
+        raise RuntimeError(
+            f"Size does not match at the leading dimensions: index {tuple(index.shape)}, logits {tuple(logits.shape)}"
+        )
+    x = _as_3d(logits)
+    k = 1 if squeeze else index.shape[-1]
+    idx = index.reshape(x.shape[0] * x.shape[1], k)
+    if idx.dtype != torch.int64:
+        raise RuntimeError(f"gather(): Expected dtype int64 for index, got {idx.dtype}")
+    logp, _, _ = ops.logp_entropy_fwd(x, idx, 1.0, 0, x.shape[1], None)
+    logp = logp.view(index.shape)
+    out_dtype = logits.dtype if out_dtype is None else out_dtype
+    return logp if out_dtype == torch.float32 else logp.to(out_dtype)
+
+
+def entropy_from_logits(logits: Tensor, chunk_size: int = 128, out_dtype: torch.dtype | None = None) -> Tensor:
+    """Shannon entropy (nats) of `softmax(logits)` over the last axis, shape `logits.shape[:-1]`
+    (reference: trl/trainer/utils.py:526-560).  `chunk_size` is accepted for signature
+    compatibility; the kernel streams each row once and needs no chunking."""
+    x = _as_3d(logits)
+    idx = torch.empty((x.shape[0] * x.shape[1], 0), dtype=torch.int64, device=logits.device)
+    _, ent, _ = ops.logp_entropy_fwd(x, idx, 1.0, 0, x.shape[1], None)
+    ent = ent.view(logits.shape[:-1])
+    out_dtype = logits.dtype if out_dtype is None else out_dtype
+    return ent if out_dtype == torch.float32 else ent.to(out_dtype)
+
+
+# ----------------------------------------------------------------------------------------------
+# O(B) helpers on tiny tensors: plain torch, as in the reference (trl/trainer/utils.py:857-890, 960-987)
+# ----------------------------------------------------------------------------------------------
+def nanstd(tensor: Tensor, dim=None, keepdim: bool = False) -> Tensor:
+    """Bessel-corrected standard deviation ignoring NaNs; NaN where fewer than two values remain."""
+    mean = torch.nanmean(tensor, dim=dim, keepdim=True)
+    var = torch.nanmean((tensor - mean) ** 2, dim=dim, keepdim=True)
+    count = torch.sum(~torch.isnan(tensor), dim=dim, keepdim=True)
+    var = var * torch.where(count > 1, count / (count - 1), torch.full_like(var, float("nan")))
+    std = var.sqrt()
+    if keepdim:
+        return std
+    if dim is None:
+        return std.squeeze()
+    dims = (dim,) if isinstance(dim, int) else dim
+    for d in sorted((d % std.dim() for d in dims), reverse=True):
+        std = std.squeeze(d)
+    return std
+
+
+def nanmin(tensor: Tensor) -> Tensor:
+    """Minimum of a 1-D tensor ignoring NaNs; NaN if every entry is NaN."""
+    keep = ~torch.isnan(tensor)
+    if not keep.any():
+        return torch.tensor(float("nan"), dtype=tensor.dtype, device=tensor.device)
+    return tensor[keep].min()
+
+
+def nanmax(tensor: Tensor) -> Tensor:
+    """Maximum of a 1-D tensor ignoring NaNs; NaN if every entry is NaN."""
+    keep = ~torch.isnan(tensor)
+    if not keep.any():
+        return torch.tensor(float("nan"), dtype=tensor.dtype, device=tensor.device)
+    return tensor[keep].max()
