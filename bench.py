@@ -59,7 +59,7 @@ def make_inputs(w, device, seed=0):
     return logits, ids, mask, rewards, g
 
 
-def cpu_baseline(w, loss_type, rows_per_seq=32, n_seq=8, repeats=2):
+def cpu_baseline(w, loss_type, rows_per_seq=512, n_seq=32, repeats=2):
     """The oracle (CPU port of the reference path: row-looped log_softmax / 128-row entropy chunks /
     autograd backward) on a [n_seq, rows_per_seq, V] bf16 sample of the workload."""
     import oracle
@@ -107,6 +107,8 @@ def main():
     ap.add_argument("--workload", default="grpo_c3", choices=sorted(WORKLOADS))
     ap.add_argument("--loss-type", default="dapo", choices=["grpo", "dapo", "dr_grpo", "bnpo"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain device copy of the logits (known bytes) to scale profiler counters by")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs on ONE GPU; rows are independent, so N GPUs would each run this same "
@@ -155,7 +157,7 @@ def main():
     ev_ms = e0.elapsed_time(e1)
     ms_per_step = max(wall_ms, ev_ms) / args.steps
     tokens_per_s = R / (ms_per_step * 1e-3)
-    loss_value = float(loss)
+    loss_value = float(loss.detach())
     assert loss_value == loss_value, "loss is NaN"
 
     # ---- per-kernel timing: each kernel alone, events around `reps` back-to-back launches -----------
@@ -228,6 +230,13 @@ def main():
             "step_hbm_GBps": (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9,
         },
     }
+    if args.calibrate_copy:
+        dst = torch.empty_like(logits)
+        for _ in range(3):
+            dst.copy_(logits.detach())  # reads and writes R*V*2 bytes each
+        torch.cuda.synchronize()
+        result["calibration_copy_bytes_each_way"] = fwd_bytes
+        del dst
     if not args.no_cpu_baseline:
         del leaf, logits
         torch.cuda.empty_cache()

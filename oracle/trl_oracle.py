@@ -336,17 +336,21 @@ def grpo_loss(
     if beta != 0.0:
         per_token_loss = per_token_loss + beta * per_token_kl
 
+    # policy_loss is taken before the division by the gradient-accumulation steps (:3127, 3132, 3137, 3142)
     if loss_type == "grpo":
         loss = ((per_token_loss * mask).sum(-1) / mask.sum(-1).clamp(min=1.0)).mean()
         normalizer = grad_accum_steps
+        policy_loss = loss.detach()
         loss = loss / normalizer
     elif loss_type == "bnpo":
         loss = (per_token_loss * mask).sum() / mask.sum().clamp(min=1.0)
         normalizer = grad_accum_steps
+        policy_loss = loss.detach()
         loss = loss / normalizer
     elif loss_type == "dr_grpo":
         loss = (per_token_loss * mask).sum() / (per_token_loss.size(0) * max_completion_length)
         normalizer = grad_accum_steps
+        policy_loss = loss.detach()
         loss = loss / normalizer
     else:  # dapo
         n_items = num_items_in_batch
@@ -354,7 +358,7 @@ def grpo_loss(
             n_items = torch.tensor(float(n_items))
         normalizer = n_items.clamp(min=1.0) / num_processes
         loss = (per_token_loss * mask).sum() / normalizer
-    policy_loss = loss.detach()
+        policy_loss = loss.detach()
 
     metrics: dict[str, float] = {}
     if entropy_coef != 0.0:

@@ -84,6 +84,10 @@ GRPO_CASES = [
     dict(name="grpo_entbonus", loss_type="grpo", beta=0.04, eps_low=0.2, eps_high=0.2, entropy_coef=0.01),
     dict(name="dapo_entbonus", loss_type="dapo", beta=0.0, eps_low=0.2, eps_high=0.2, entropy_coef=0.02),
     dict(name="dapo_emptyrow", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, empty_row=True),
+    dict(name="grpo_entbonus_ga", loss_type="grpo", beta=0.04, eps_low=0.2, eps_high=0.2, entropy_coef=0.01, grad_accum=4),
+    dict(name="bnpo_entbonus_ga", loss_type="bnpo", beta=0.0, eps_low=0.2, eps_high=0.2, entropy_coef=0.02, grad_accum=2),
+    dict(name="dr_grpo_entq_bonus", loss_type="dr_grpo", beta=0.04, eps_low=0.2, eps_high=0.2, entropy_coef=0.02,
+         top_entropy_quantile=0.6, grad_accum=2),
 ]
 
 

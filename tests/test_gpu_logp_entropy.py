@@ -107,8 +107,17 @@ def test_config1_full_size_fp32(amd):
     dl = logits.to(DEV)
     got_lp = amd.selective_log_softmax(dl, idx.to(DEV)).cpu()
     got_h = amd.entropy_from_logits(dl).cpu()
-    torch.testing.assert_close(got_lp, oracle.selective_log_softmax(logits, idx), atol=1e-5, rtol=0)
-    torch.testing.assert_close(got_h, oracle.entropy_from_logits(logits), atol=1e-5, rtol=0)
+    want_lp, want_h = oracle.selective_log_softmax(logits, idx), oracle.entropy_from_logits(logits)
+    torch.testing.assert_close(got_lp, want_lp, atol=1e-5, rtol=0)
+    # The fp32 entropy of the reference formulation (sum of exp(lp) * lp over 32000 terms) is itself up to
+    # ~1.3e-5 away from the exact value on this input, so the 1e-5 bar is applied against the fp64
+    # evaluation of the same formula, and the fp32 oracle is allowed its own rounding error on top.
+    exact_h = oracle.entropy_from_logits(logits.double())
+    exact_lp = oracle.selective_log_softmax(logits.double(), idx)
+    assert (got_h.double() - exact_h).abs().max() <= 1e-5
+    assert (got_lp.double() - exact_lp).abs().max() <= 1e-5
+    slack = (want_h.double() - exact_h).abs()
+    assert ((got_h - want_h).abs().double() <= 1e-5 + slack).all()
 
 
 # ------------------------------------------------------------------ real vocabulary sizes, bf16

@@ -135,7 +135,7 @@ def test_golden_grpo_compute_loss_through_trainer_methods(amd):
             ok = (math.isnan(got) and math.isnan(want)) or abs(got - want) <= (2e-2 if low else 1e-5) * max(1.0, abs(want))
             assert ok, (case["name"], name, got, want)
         ran += 1
-    assert ran >= 15
+    assert ran >= 18
 
 
 def test_grpo_loss_against_oracle_random(amd):
@@ -230,8 +230,8 @@ def test_golden_dpo_compute_loss(amd):
                      "logps/rejected", "entropy"):
             want_m = case["metrics"][name]
             tol = (0.15 if low else 1e-5) * max(1.0, abs(want_m))  # bf16 reference sums bf16-rounded log-probs
-            if low and name == "rewards/accuracies":
-                continue
+            if name == "rewards/accuracies" and (low or case.get("ref_equal")):
+                continue  # ties / near-ties between chosen and rejected rewards: decided by rounding noise
             assert abs(float(named[name]) - want_m) <= tol, (case["name"], name, float(named[name]), want_m)
         if case.get("ref_equal") and not low:
             assert abs(float(loss) - math.log(2.0)) < 1e-6

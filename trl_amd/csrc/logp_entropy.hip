@@ -2,9 +2,9 @@
 //
 // One workgroup owns one row (token position).  The row is streamed once with 16-byte
 // non-temporal loads, `UNR` loads in flight per lane; every lane keeps an online
-// (max, sum e^(z-max), sum e^(z-max)*x) triple in fp32 and the triples are merged across the
-// workgroup through wave shuffles and LDS.  The temperature is folded into the exponent
-// multiplier (exp2(x*c - m*c), c = log2(e)/T), so no scaled copy of the row ever exists.
+// (reference exponent r, sum 2^(x*c-r), sum 2^(x*c-r)*x) triple in fp32 and the triples are merged
+// across the workgroup through wave shuffles and LDS.  The temperature is folded into the
+// exponent multiplier (c = log2(e)/T), so no scaled copy of the row ever exists.
 // The backward re-streams the row and the saved lse and writes dlogits in the same pass.
 #include "common.hpp"
 
@@ -28,22 +28,27 @@ struct FwdArgs {
     int32_t* error_flag;
 };
 
+// Per-lane online log-sum-exp state in base 2.  The reference point `r` is an INTEGER (held in a
+// float): ceil(max * c) of the values seen so far.  exp2(x*c - r) then has no rounding in the
+// reference itself (the fma rounds once, relative to the small difference near the maximum), and
+// moving to a larger reference is an exact power-of-two rescale.
 struct OnlineLse {
-    float m = -INFINITY;  // running max of the raw (unscaled) logits
-    float mc = 0.f;       // m * c, with 0 standing in while m is still -inf
-    float s = 0.f;        // sum exp2(x*c - mc)
-    float u = 0.f;        // sum exp2(x*c - mc) * x
+    float r = -INFINITY;  // integer reference exponent (-inf until a finite value was seen)
+    float rr = 0.f;       // r, with 0 standing in while r is still -inf
+    float s = 0.f;        // sum exp2(x*c - r)
+    float u = 0.f;        // sum exp2(x*c - r) * x
     __device__ __forceinline__ void raise(float bm, float c) {
-        if (bm > m) {
-            const float sc = fast_exp2((m - bm) * c);  // m = -inf gives 0, and s = u = 0 then
+        const float need = ceilf(bm * c);
+        if (need > r) {
+            const float sc = fast_exp2(r - need);  // r = -inf gives 0, and s = u = 0 then
             s *= sc;
             u *= sc;
-            m = bm;
-            mc = bm * c;
+            r = need;
+            rr = need;
         }
     }
     __device__ __forceinline__ void add(float x, float c) {
-        const float e = fast_exp2(fmaf(x, c, -mc));
+        const float e = fast_exp2(fmaf(x, c, -rr));
         s += e;
         u = fmaf(e, x, u);
     }
@@ -114,16 +119,16 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
         }
     }
 
-    // ---- merge the per-lane triples: global max first, then two sums --------------------
+    // ---- merge the per-lane triples: common reference first (exact rescale), then two sums -----
     const int lane = tid & (kWave - 1), wave = tid / kWave;
-    float wm = wave_max(acc.m);
-    if (lane == 0) red[0][wave] = wm;
+    float wr = wave_max(acc.r);
+    if (lane == 0) red[0][wave] = wr;
     __syncthreads();
-    float M = red[0][0];
+    float R = red[0][0];
 #pragma unroll
-    for (int w = 1; w < NW; ++w) M = fmaxf(M, red[0][w]);
-    // lanes that saw nothing finite have m = -inf and s = 0; exp2(-inf) = 0 keeps them out
-    const float sc = (acc.m == -INFINITY) ? 0.f : fast_exp2((acc.m - M) * c);
+    for (int w = 1; w < NW; ++w) R = fmaxf(R, red[0][w]);
+    // lanes that saw nothing finite have r = -inf and s = 0; a zero factor keeps them out
+    const float sc = (acc.r == -INFINITY) ? 0.f : fast_exp2(acc.r - R);
     float s = wave_sum(acc.s * sc);
     float u = wave_sum(acc.u * sc);
     if (lane == 0) {
@@ -138,7 +143,9 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
             S += red[1][w];
             U += red[2][w];
         }
-        const float lse = M / a.temperature + logf(S);
+        // lse = R*ln2 + ln S with ln2 split in two so that the product carries no rounding of ln2
+        constexpr float kLn2Hi = 0.693145751953125f, kLn2Lo = 1.42860677e-06f;
+        const float lse = fmaf(R, kLn2Hi, fmaf(R, kLn2Lo, logf(S)));
         const float ent = lse - (U / S) / a.temperature;
         bcast[0] = lse;
         if (a.out_entropy) a.out_entropy[row] = ent;
