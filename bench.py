@@ -133,9 +133,9 @@ def main():
     n_items = mask.sum().float()
     leaf = logits.requires_grad_(True)
 
-    def step():
+    def step(row_mask=None):
         leaf.grad = None
-        lp, ent = trl_amd.logps_and_entropies(leaf, ids, w["temperature"])
+        lp, ent = trl_amd.logps_and_entropies(leaf, ids, w["temperature"], row_mask=row_mask)
         loss, metrics = trl_amd.grpo_loss(
             lp, adv, mask, entropies=ent.detach(), old_per_token_logps=old, ref_per_token_logps=ref,
             loss_type=args.loss_type, epsilon_low=w["eps_low"], epsilon_high=w["eps_high"], beta=w["beta"],
@@ -143,22 +143,27 @@ def main():
         loss.backward()
         return loss, metrics
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(args.steps):
-        loss, metrics = step()
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    ev_ms = e0.elapsed_time(e1)
-    ms_per_step = max(wall_ms, ev_ms) / args.steps
+    def timed(row_mask):
+        for _ in range(args.warmup):
+            step(row_mask)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            loss, _ = step(row_mask)
+        e1.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        return max(wall_ms, e0.elapsed_time(e1)) / args.steps, float(loss.detach())
+
+    # headline: every row's log-prob and entropy is produced (the configuration's stated outputs)
+    ms_per_step, loss_value = timed(None)
     tokens_per_s = R / (ms_per_step * 1e-3)
-    loss_value = float(loss.detach())
     assert loss_value == loss_value, "loss is NaN"
+    # secondary: the forward also skips the rows the completion mask zeroes (what `_compute_loss` does by default)
+    ms_mask_aware, loss_mask_aware = timed(mask)
+    assert abs(loss_mask_aware - loss_value) <= 1e-6 * max(1.0, abs(loss_value)), "mask-aware loss differs"
 
     # ---- per-kernel timing: each kernel alone, events around `reps` back-to-back launches -----------
     idx = ids.reshape(R, 1)
@@ -229,6 +234,9 @@ def main():
                                              "achieved_GBps": bwd_gbps, "frac": bwd_gbps / HBM_PEAK_GBPS},
             "step_hbm_GBps": (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9,
         },
+        "mask_aware": {"ms_per_step": ms_mask_aware, "tokens_per_s": R / (ms_mask_aware * 1e-3),
+                       "note": "forward also skips rows with completion_mask == 0 (their outputs are 0); "
+                               "loss, metrics and dlogits identical"},
     }
     if args.calibrate_copy:
         dst = torch.empty_like(logits)

@@ -95,6 +95,10 @@ __global__ __launch_bounds__(kThreads) void grpo_rows_kernel(GrpoArgs a) {
     float s_mask = 0, s_loss = 0, s_kl = 0, s_ent = 0, s_low = 0, s_high = 0, s_reg = 0, s_ent_eff = 0, s_eff = 0;
     for (int64_t t = tid; t < a.T; t += kThreads) {
         const float m = a.mask[off + t];
+        if (m == 0.f) {  // a masked token contributes exactly nothing, whatever its (possibly skipped) inputs hold
+            a.out_dlogp[off + t] = 0.f;
+            continue;
+        }
         const float lp = a.logp[off + t];
         const float A = a.adv[b * a.adv_stride_b + t * a.adv_stride_t];
         const float c1_raw = a.old_logp ? expf(lp - a.old_logp[off + t]) : 1.f;

@@ -33,12 +33,13 @@ group_advantages = ops.group_advantages
 
 def per_token_logps_and_entropies(
     logits: Tensor, input_ids: Tensor, logits_to_keep: int, temperature: float = 1.0, compute_entropy: bool = True,
-    entropy_requires_grad: bool = False,
+    entropy_requires_grad: bool = False, row_mask: Tensor | None = None,
 ) -> tuple[Tensor, Tensor | None]:
     """`[B, L, V]` model logits -> fp32 `(logps [B, K], entropies [B, K] | None)` for the last
     `K = logits_to_keep` tokens of `input_ids`: drops the last position, keeps the last K, divides by
     the temperature (trl/trainer/grpo_trainer.py:1514-1521) -- as index arithmetic on the full tensor,
-    so the backward writes the `[B, L, V]` gradient directly (rows outside the window zero)."""
+    so the backward writes the `[B, L, V]` gradient directly (rows outside the window zero).
+    `row_mask` (`[B, K]`, zero = skip) makes the kernel skip those rows: they are not read and yield 0."""
     if logits.dim() != 3:
         raise ValueError("expected [B, L, V] logits")
     length = logits.shape[1]
@@ -47,7 +48,7 @@ def per_token_logps_and_entropies(
     ids = input_ids[:, -keep_len:] if keep_len > 0 else input_ids[:, :0]
     if logits.shape[-1] > 1 and logits.stride(-1) != 1:
         logits = logits.contiguous()
-    logp, ent = logps_and_entropies(logits, ids, temperature, keep_start, keep_len)
+    logp, ent = logps_and_entropies(logits, ids, temperature, keep_start, keep_len, row_mask)
     if not compute_entropy:
         return logp, None
     return logp, (ent if entropy_requires_grad else ent.detach())
@@ -137,10 +138,12 @@ class GRPOLossMixin:
 
     def _get_per_token_logps_and_entropies(
         self, model, input_ids, attention_mask, logits_to_keep, batch_size=None, compute_entropy=False,
-        compute_aux_loss=False, **model_extra_inputs,
+        compute_aux_loss=False, skip_rows_mask=None, **model_extra_inputs,
     ):
         """Reference: trl/trainer/grpo_trainer.py:1435-1541.  Multimodal extras are forwarded to the
-        model only when the whole batch goes through in one piece (no per-sample splitting here)."""
+        model only when the whole batch goes through in one piece (no per-sample splitting here).
+        `skip_rows_mask` (`[B, logits_to_keep]`, not in the reference) names rows whose log-prob and
+        entropy the caller will discard: they are not read and come back as 0."""
         batch_size = batch_size or input_ids.size(0)
         extras = {k: v for k, v in model_extra_inputs.items() if v is not None}
         if extras and batch_size < input_ids.size(0):
@@ -156,8 +159,9 @@ class GRPOLossMixin:
             if compute_aux_loss:
                 model_inputs["output_router_logits"] = True
             outputs = model(**model_inputs)
+            rows = None if skip_rows_mask is None else skip_rows_mask[start : start + batch_size]
             logps, ent = per_token_logps_and_entropies(
-                outputs.logits, ids, logits_to_keep, self.temperature, compute_entropy, entropy_grad
+                outputs.logits, ids, logits_to_keep, self.temperature, compute_entropy, entropy_grad, rows
             )
             all_logps.append(logps)
             if compute_entropy:
@@ -187,9 +191,12 @@ class GRPOLossMixin:
         aux_enabled = bool(getattr(self, "aux_loss_enabled", False))
         extra_keys = ("pixel_values", "image_grid_thw", "num_images", "pixel_attention_mask", "spatial_shapes",
                       "num_tiles", "image_sizes", "token_type_ids", "mm_token_type_ids", "image_position_ids")
+        # Every use of the log-probs and entropies below is multiplied by `mask`, so rows with mask == 0
+        # need not be computed at all (set `trl_amd_skip_masked_rows = False` on the trainer to compute them).
+        skip = mask if getattr(self, "trl_amd_skip_masked_rows", True) else None
         per_token_logps, entropies, aux_loss = self._get_per_token_logps_and_entropies(
             model, input_ids, attention_mask, logits_to_keep, compute_entropy=True, compute_aux_loss=aux_enabled,
-            **{k: inputs.get(k) for k in extra_keys},
+            skip_rows_mask=skip, **{k: inputs.get(k) for k in extra_keys},
         )
         advantages = inputs["advantages"]
         entropy_mask = None
