@@ -189,6 +189,42 @@ int trlk_rloo_loss(const float* d_token_logp, const float* d_mask, const float* 
                    float* d_out_seq_logps, float* d_out_loss, float* d_out_metrics, float* d_out_dlogp,
                    trlk_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------
+ * K5 / K6  lm_head fused with the log-prob / entropy reduction; the [N, V] logits are never
+ * written to memory.  Replaces _ChunkedLogProbFunction (trl/trainer/utils.py:1291-1424):
+ *   y = hidden @ weight^T   (bf16/fp16 operands on the matrix cores, fp32 accumulation)
+ *   z = softcap(y * logit_scale) / temperature,  softcap(x) = cap * tanh(x / cap) if cap > 0
+ *   out_logp[n] = z[n, targets[n]] - logsumexp(z[n, :]);  out_entropy[n] = logsumexp - E_p[z];
+ *   out_log_z[n] = logsumexp(z[n, :])   (saved for the backward)
+ * d_hidden [n_tokens, hidden_size] and d_weight [vocab, hidden_size] are row-major with row
+ * strides (elements) that are multiples of 8, 16-byte aligned; dtype TRLK_BF16 or TRLK_F16.
+ * Unlike the reference, the logits are not rounded to the operand dtype before the reduction.
+ * A target outside [0, vocab) yields NaN and sets TRLK_FLAG_INDEX_OUT_OF_RANGE.
+ */
+size_t trlk_fused_head_fwd_workspace_bytes(int64_t n_tokens);
+
+int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, const int64_t* d_targets, int dtype,
+                        int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
+                        int64_t weight_stride, float temperature, float final_logit_softcapping, float logit_scale,
+                        float* d_out_logp, float* d_out_entropy, float* d_out_log_z, int32_t* d_error_flag,
+                        void* d_workspace, size_t workspace_bytes, trlk_stream_t stream);
+
+/* Backward of the above w.r.t. hidden and weight for an upstream gradient on the log-probs
+ * (the entropy output carries no gradient, as in the reference, utils.py:1368):
+ *   dz[n, v] = g[n] * (1[v == targets[n]] - exp(z[n, v] - log_z[n])) * d z / d y
+ *   out_dhidden = dz @ weight,  out_dweight = dz^T @ hidden   (fp32 accumulation, outputs in `dtype`,
+ *   dense [n_tokens, hidden_size] and [vocab, hidden_size]).
+ * The vocabulary is processed in chunks of `chunk_size` rows (rounded up to 256); dz exists only
+ * for one chunk at a time, in bf16/fp16, inside the workspace.
+ */
+size_t trlk_fused_head_bwd_workspace_bytes(int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t chunk_size);
+
+int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, const int64_t* d_targets, int dtype,
+                        int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
+                        int64_t weight_stride, float temperature, float final_logit_softcapping, float logit_scale,
+                        const float* d_log_z, const float* d_g_logp, int64_t chunk_size, void* d_out_dhidden,
+                        void* d_out_dweight, void* d_workspace, size_t workspace_bytes, trlk_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,163 @@
+"""GPU parity of the fused lm_head + log-prob kernels (K5 forward, K6 backward) against the golden
+vectors written by the reference's `_ChunkedLogProbFunction`, and against the CPU oracle / plain
+fp32 autograd on the same bf16-valued operands.
+
+Tolerances: the reference's own bf16 test uses 1e-2 (tests/test_utils.py:1212-1232).  Against
+fp32 op-math on the same stored values: log-probs / entropies 2e-3 abs; gradients (bf16 outputs,
+bf16 dz workspace) 1e-2 relative L2."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from conftest import load_golden
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _t(a, dtype=None):
+    t = torch.from_numpy(np.asarray(a))
+    return t.to(dtype) if dtype is not None else t
+
+
+def _rel_l2(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    return float((got - want).norm() / want.norm().clamp(min=1e-30))
+
+
+@pytest.fixture(scope="module")
+def amd():
+    import trl_amd
+
+    return trl_amd
+
+
+def _fp32_reference(hidden, weight, labels, temperature, softcap, scale, gout):
+    """fp32 op-math on the stored (bf16-valued) operands, autograd for the gradients."""
+    h = hidden.float().requires_grad_(True)
+    w = weight.float().requires_grad_(True)
+    y = (h @ w.t()) * scale
+    if softcap:
+        y = torch.tanh(y / softcap) * softcap
+    z = y / temperature
+    lp_all = F.log_softmax(z, -1)
+    lp = lp_all.gather(-1, labels[:, None]).squeeze(-1)
+    ent = -(lp_all.exp() * lp_all).sum(-1)
+    (lp * gout).sum().backward()
+    return lp.detach(), ent.detach(), h.grad, w.grad
+
+
+def _run_device(amd, hidden, weight, labels, temperature, chunk, softcap, scale, gout):
+    h = hidden.to(DEV).requires_grad_(True)
+    w = weight.to(DEV).requires_grad_(True)
+    lp, ent = amd._ChunkedLogProbFunction.apply(h, w, labels.to(DEV), temperature, chunk, softcap, scale)
+    (lp * gout.to(DEV)).sum().backward()
+    assert lp.dtype == torch.float32 and ent.dtype == torch.float32 and not ent.requires_grad
+    return lp.detach().cpu(), ent.detach().cpu(), h.grad.cpu(), w.grad.cpu()
+
+
+def test_golden_chunked_logprob_bf16(amd):
+    cases, g = load_golden("chunked_logprob")
+    ran = 0
+    for case in cases:
+        if case["dtype"] != "bfloat16":
+            continue
+        c = f"c{case['id']}_"
+        hidden, weight = _t(g[c + "hidden"], torch.bfloat16), _t(g[c + "weight"], torch.bfloat16)
+        labels, gout = _t(g[c + "labels"]), _t(g[c + "grad_out"])
+        lp, ent, dh, dw = _run_device(amd, hidden, weight, labels, case["temperature"], case["chunk"], case["softcap"],
+                                      case["logit_scale"], gout)
+        tol = dict(atol=1e-2, rtol=1e-2)  # the reference's bf16 tolerance; its logits are rounded to bf16, ours are not
+        torch.testing.assert_close(lp, _t(g[c + "out_logprobs"]), atol=6e-2, rtol=1e-2)
+        torch.testing.assert_close(ent, _t(g[c + "out_entropy"]), atol=6e-2, rtol=1e-2)
+        assert _rel_l2(dh.float(), _t(g[c + "out_dhidden"])) < 2e-2
+        assert _rel_l2(dw.float(), _t(g[c + "out_dweight"])) < 2e-2
+        # and tightly against fp32 op-math on the same stored operands
+        rlp, rent, rdh, rdw = _fp32_reference(hidden, weight, labels, case["temperature"], case["softcap"],
+                                              case["logit_scale"], gout)
+        torch.testing.assert_close(lp, rlp, atol=2e-3, rtol=0)
+        torch.testing.assert_close(ent, rent, atol=2e-3, rtol=0)
+        assert _rel_l2(dh.float(), rdh) < 1e-2 and _rel_l2(dw.float(), rdw) < 1e-2
+        del tol
+        ran += 1
+    assert ran >= 1
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,h,v,chunk,temperature,softcap,scale", [
+    (64, 32, 128, 32, 0.7, None, 1.0),       # the reference test's shape (tests/test_utils.py:1161-1163)
+    (300, 256, 1000, 256, 0.9, None, 1.0),   # ragged in every dimension, four vocabulary chunks
+    (257, 136, 777, 512, 1.0, 5.0, 0.5),     # soft-capping + logit_scale, K tail, odd vocabulary
+    (1, 8, 3, 8192, 1.3, None, 1.0),         # minimal sizes
+    (600, 512, 2304, 1024, 0.8, None, 1.0),  # several token blocks x several vocabulary tiles
+])
+def test_fused_head_against_fp32_reference(amd, dtype, n, h, v, chunk, temperature, softcap, scale):
+    g = torch.Generator().manual_seed(n * 7 + v)
+    hidden = torch.randn(n, h, generator=g).to(dtype)
+    weight = (torch.randn(v, h, generator=g) * (2.0 / h**0.5)).to(dtype)
+    labels = torch.randint(0, v, (n,), generator=g)
+    gout = torch.randn(n, generator=g)
+    lp, ent, dh, dw = _run_device(amd, hidden, weight, labels, temperature, chunk, softcap, scale, gout)
+    rlp, rent, rdh, rdw = _fp32_reference(hidden, weight, labels, temperature, softcap, scale, gout)
+    torch.testing.assert_close(lp, rlp, atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent, rent, atol=2e-3, rtol=0)
+    assert dh.dtype == dtype and dw.dtype == dtype and dh.shape == hidden.shape and dw.shape == weight.shape
+    assert _rel_l2(dh.float(), rdh) < 1e-2, _rel_l2(dh.float(), rdh)
+    assert _rel_l2(dw.float(), rdw) < 1e-2, _rel_l2(dw.float(), rdw)
+    # the oracle's online sweep (chunked like the reference) agrees as well
+    olp, oent, _ = oracle.chunked_logprob_online(hidden.float(), weight.float(), labels, temperature, max(chunk, 8),
+                                                 softcap, scale)
+    torch.testing.assert_close(lp, olp, atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent, oent, atol=2e-3, rtol=0)
+
+
+def test_masked_rows_and_scatter(amd):
+    # reference tests/test_utils.py:1338-1398: masked == unmasked on completion rows, exact zeros elsewhere,
+    # and the lm_head gradient only sees completion rows
+    g = torch.Generator().manual_seed(5)
+    B, S, H, V = 3, 17, 64, 500
+    hs = torch.randn(B, S, H, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(V, H, generator=g) * 0.3).bfloat16().to(DEV).requires_grad_(True)
+    labels = torch.randint(0, V, (B, S), generator=g).to(DEV)
+    cm = torch.zeros(B, S, dtype=torch.long)
+    cm[0, 3:9] = 1
+    cm[1, 10:] = 1
+    cm = cm.to(DEV)
+    lp_m, ent_m = amd.chunked_logprobs_from_hidden(hs, w, labels, cm, 0.8, 256)
+    lp_u, ent_u = amd.chunked_logprobs_from_hidden(hs, w, labels, None, 0.8, 256)
+    keep = cm[:, 1:].bool()
+    torch.testing.assert_close(lp_m[keep], lp_u[keep], atol=1e-5, rtol=0)
+    torch.testing.assert_close(ent_m[keep], ent_u[keep], atol=1e-5, rtol=0)
+    assert torch.count_nonzero(lp_m[~keep]) == 0 and torch.count_nonzero(ent_m[~keep]) == 0
+    lp_m.sum().backward()
+    gm = w.grad.clone()
+    w.grad = None
+    (lp_u * keep).sum().backward()
+    assert _rel_l2(gm.float(), w.grad.float()) < 1e-2
+    # an empty selection is a valid call
+    lp_e, _ = amd.chunked_logprobs_from_hidden(hs, w, labels, torch.zeros_like(cm), 0.8, 256)
+    assert torch.count_nonzero(lp_e) == 0
+
+
+def test_fp32_operands_are_rejected_loudly(amd):
+    with pytest.raises(TypeError):
+        amd._ChunkedLogProbFunction.apply(torch.randn(4, 8, device=DEV), torch.randn(16, 8, device=DEV),
+                                          torch.zeros(4, dtype=torch.long, device=DEV), 1.0, 8)
+
+
+def test_real_head_shape_row_subsample(amd):
+    """Qwen2.5-7B head shape of BASELINE config 5 (H = 3584, V = 151936) on 256 tokens."""
+    g = torch.Generator().manual_seed(55)
+    n, h, v = 256, 3584, 151936
+    hidden = torch.randn(n, h, generator=g).bfloat16()
+    weight = (0.02 * torch.randn(v, h, generator=g)).bfloat16()
+    labels = torch.randint(0, v, (n,), generator=g)
+    gout = torch.randn(n, generator=g)
+    lp, ent, dh, dw = _run_device(amd, hidden, weight, labels, 1.0, 8192, None, 1.0, gout)
+    rlp, rent, rdh, rdw = _fp32_reference(hidden, weight, labels, 1.0, None, 1.0, gout)
+    torch.testing.assert_close(lp, rlp, atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent, rent, atol=2e-3, rtol=0)
+    assert _rel_l2(dh.float(), rdh) < 1e-2
+    assert _rel_l2(dw.float(), rdw) < 1e-2

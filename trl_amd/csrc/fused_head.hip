@@ -1,0 +1,690 @@
+// K5 / K6: lm_head fused with the log-prob / entropy reduction (forward) and its backward.
+//
+// All contractions run on the matrix cores (v_mfma_f32_32x32x16_{bf16,f16}, fp32 accumulate)
+// through ONE "NT" tile loop: C[256 x 256] += A[256 x K] * B[256 x K]^T with both operands
+// row-major and K contiguous, which is the layout the MFMA A/B fragments want (a lane holds 8
+// consecutive k of one row), so fragments come straight out of LDS with 16-byte reads and nothing
+// is ever transposed on the fly.  512 threads = 8 waves as 2 (M) x 4 (N); a wave owns 128 x 64 of
+// the tile = 4 x 2 MFMA blocks = 128 accumulator registers per lane.  Global -> registers -> LDS
+// staging with two LDS buffers (one barrier per 64-wide k step).
+//
+// Forward (K5): the tile is computed TRANSPOSED -- M = vocabulary rows of W, N = tokens -- so that
+// a lane of the accumulator layout holds 16 vocabulary entries of ONE token per block.  The online
+// log-sum-exp state of a token therefore lives in the lane's own registers and the per-tile
+// epilogue needs no cross-lane traffic; a workgroup keeps 256 tokens and walks over its share of
+// the vocabulary tiles, the logits exist only as accumulators.
+//
+// Backward (K6), per vocabulary chunk: (1) recompute the chunk's logits the same way and turn
+// them into dz = dL/dlogits (bf16), written both as [tokens, chunk] and as [chunk, tokens];
+// (2) dHidden += dz * W_chunk as an NT product against W^T; (3) dW_chunk = dz^T * hidden as an NT
+// product against hidden^T.  The contraction of (2)/(3) is over a different axis than the
+// recompute, and with H in the thousands the output tile of a fused kernel cannot stay in
+// registers, so dz goes through a chunk-sized workspace (never the whole [N, V] matrix).
+#include "common.hpp"
+
+namespace trlk {
+namespace {
+
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int kHeadThreads = 512;
+constexpr int kLdsRow = BK + 8;  // bf16 elements per LDS row: 144 bytes, conflict-free 16-byte reads
+constexpr int WM = 128, WN = 64;  // per-wave tile
+constexpr int WGN = BN / WN;      // 4 waves along N, 2 along M
+constexpr int MB = WM / 32, NB = WN / 32;
+constexpr int kTileLdsBytes = BM * kLdsRow * 2;          // one operand tile
+constexpr int kHeadLdsBytes = 4 * kTileLdsBytes;         // A and B, two stages = 147456 bytes
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <int DT>
+__device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+    if constexpr (DT == TRLK_BF16)
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                       0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                      0, 0);
+}
+
+// One operand of the NT product: `rows` x K, row-major with leading dimension ld (elements).
+struct Operand {
+    const uint16_t* p;
+    int64_t ld;
+    int rows;
+};
+
+// acc[mb][nb] = sum_k A[m0 + .., k] * B[n0 + .., k].  Rows beyond the operand's end are clamped to
+// its last row (callers ignore those outputs); k beyond K reads as zero (K % 8 == 0).
+template <int DT>
+__device__ __forceinline__ void gemm_tile_nt(const Operand A, int m0, const Operand B, int n0, int K,
+                                             f32x16 (&acc)[MB][NB], char* smem) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int kc = tid & 7, r0 = tid >> 3;  // this thread stages rows r0 + 64*j, 16-byte column chunk kc
+
+    const uint16_t* ga[4];
+    const uint16_t* gb[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        int ra = m0 + r0 + 64 * j, rb = n0 + r0 + 64 * j;
+        ra = ra < A.rows ? ra : A.rows - 1;
+        rb = rb < B.rows ? rb : B.rows - 1;
+        ga[j] = A.p + int64_t(ra) * A.ld + kc * 8;
+        gb[j] = B.p + int64_t(rb) * B.ld + kc * 8;
+    }
+    const int st_off = (r0 * kLdsRow + kc * 8) * 2;        // + j * 64 rows
+    const int fa_off = ((wm * WM + (lane & 31)) * kLdsRow + (lane >> 5) * 8) * 2;  // + mb*32 rows, + ks*16
+    const int fb_off = ((wn * WN + (lane & 31)) * kLdsRow + (lane >> 5) * 8) * 2;
+
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0.f;
+
+    u32x4 ra[4], rb[4];
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    auto load_stage = [&](int k0) {
+        const bool in = k0 + kc * 8 < K;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            ra[j] = in ? *reinterpret_cast<const u32x4*>(ga[j] + k0) : zero;
+            rb[j] = in ? *reinterpret_cast<const u32x4*>(gb[j] + k0) : zero;
+        }
+    };
+    auto store_stage = [&](int buf) {
+        char* sa = smem + buf * 2 * kTileLdsBytes;
+        char* sb = sa + kTileLdsBytes;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            *reinterpret_cast<u32x4*>(sa + st_off + j * 64 * kLdsRow * 2) = ra[j];
+            *reinterpret_cast<u32x4*>(sb + st_off + j * 64 * kLdsRow * 2) = rb[j];
+        }
+    };
+
+    const int nk = (K + BK - 1) / BK;
+    load_stage(0);
+    store_stage(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const bool more = kt + 1 < nk;
+        if (more) load_stage((kt + 1) * BK);
+        const char* sa = smem + (kt & 1) * 2 * kTileLdsBytes;
+        const char* sb = sa + kTileLdsBytes;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            u32x4 fa[MB], fb[NB];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                fa[mb] = *reinterpret_cast<const u32x4*>(sa + fa_off + (mb * 32 * kLdsRow + ks * 16) * 2);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+                fb[nb] = *reinterpret_cast<const u32x4*>(sb + fb_off + (nb * 32 * kLdsRow + ks * 16) * 2);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = mfma<DT>(fa[mb], fb[nb], acc[mb][nb]);
+        }
+        if (more) store_stage((kt + 1) & 1);
+        __syncthreads();
+    }
+}
+
+// Row (M index) inside the workgroup tile of accumulator element r of block mb, for this lane.
+__device__ __forceinline__ int acc_row(int wm, int mb, int r, int lane) {
+    return wm * WM + mb * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+}
+// Column (N index) inside the workgroup tile of block nb, for this lane.
+__device__ __forceinline__ int acc_col(int wn, int nb, int lane) { return wn * WN + nb * 32 + (lane & 31); }
+
+// Workgroup id -> (tile along N-like axis `a`, tile along the other axis `b`) such that the
+// workgroups that run together on one XCD (ids congruent mod 8, dispatched round-robin) form
+// 4 x 8 patches: they share operand slabs through that XCD's L2.
+__device__ __forceinline__ void xcd_patch(int w, int n_b, int& ta, int& tb) {
+    const int xcd = w & 7, q = w >> 3;
+    const int nb4 = (n_b + 7) / 8 * 8;  // b tiles padded to a multiple of 8 (callers skip the excess)
+    tb = (q >> 2) % nb4;
+    ta = ((q & 3) + 4 * (q / (4 * nb4))) * 8 + xcd;
+}
+inline int xcd_patch_grid(int n_a, int n_b) {
+    const int na32 = (n_a + 31) / 32 * 32, nb8 = (n_b + 7) / 8 * 8;
+    return na32 * nb8;
+}
+
+struct HeadArgs {
+    const uint16_t* hidden;  // [N, H]
+    const uint16_t* weight;  // [V, H]
+    const int64_t* targets;  // [N]
+    int N, V, H;
+    int64_t ldh, ldw;
+    float logit_scale, inv_t, softcap;  // softcap <= 0: none
+    // forward
+    int v_splits, tiles_per_split;
+    float* partial;  // [N, v_splits, 4]: (reference exponent, S, U, unused)
+    float* tgt;      // [N] logit of the target token (NaN until found)
+    // backward (dz pass)
+    const float* log_z;  // [N]
+    const float* g;      // [N] upstream d loss / d logp
+    int c0, c1;          // vocabulary rows of this chunk
+    uint16_t* dz;        // [N, ldz]   (columns = chunk-local vocabulary index)
+    uint16_t* dzT;       // [chunk rows padded, ldzt]
+    int64_t ldz, ldzt;
+};
+
+// z = logit in natural units after logit_scale, optional soft-capping and temperature.
+__device__ __forceinline__ float head_z(float y, const HeadArgs& a) {
+    y *= a.logit_scale;
+    if (a.softcap > 0.f) y = tanhf(y / a.softcap) * a.softcap;
+    return y * a.inv_t;
+}
+
+template <int DT>
+__global__ __launch_bounds__(kHeadThreads) void fused_head_fwd_kernel(HeadArgs a) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int n_tb = (a.N + BN - 1) / BN;
+    int tb, vs;
+    xcd_patch(blockIdx.x, a.v_splits, tb, vs);
+    if (tb >= n_tb || vs >= a.v_splits) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int n0 = tb * BN;
+    const int n_vt = (a.V + BM - 1) / BM;
+    const int vt0 = vs * a.tiles_per_split;
+    const int vt1 = vt0 + a.tiles_per_split < n_vt ? vt0 + a.tiles_per_split : n_vt;
+
+    // per-lane online state of the NB tokens this lane owns (base-2, integer reference exponent)
+    float ref[NB], rr[NB], S[NB], U[NB];
+    int64_t tg[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        ref[nb] = -INFINITY;
+        rr[nb] = 0.f;
+        S[nb] = 0.f;
+        U[nb] = 0.f;
+        const int tok = n0 + acc_col(wn, nb, lane);
+        tg[nb] = tok < a.N ? a.targets[tok] : -1;
+    }
+    const Operand W{a.weight, a.ldw, a.V}, Hd{a.hidden, a.ldh, a.N};
+
+    for (int vt = vt0; vt < vt1; ++vt) {
+        const int m0 = vt * BM;
+        f32x16 acc[MB][NB];
+        gemm_tile_nt<DT>(W, m0, Hd, n0, a.H, acc, smem);
+        const bool partial_tile = m0 + BM > a.V;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            float bm = -INFINITY;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float z = head_z(acc[mb][nb][r], a);
+                    if (partial_tile && m0 + acc_row(wm, mb, r, lane) >= a.V) z = -INFINITY;
+                    acc[mb][nb][r] = z;
+                    bm = fmaxf(bm, z);
+                }
+            const float need = ceilf(bm * kLog2e);
+            if (need > ref[nb]) {
+                const float sc = fast_exp2(ref[nb] - need);
+                S[nb] *= sc;
+                U[nb] *= sc;
+                ref[nb] = need;
+                rr[nb] = need;
+            }
+            float s = 0.f, u = 0.f;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float z = acc[mb][nb][r];
+                    const float e = fast_exp2(fmaf(z, kLog2e, -rr[nb]));
+                    s += e;
+                    u = (z == -INFINITY) ? u : fmaf(e, z, u);
+                }
+            S[nb] += s;
+            U[nb] += u;
+            // target logit: rarely inside this wave's 128 vocabulary rows
+            const int64_t rel = tg[nb] - (m0 + wm * WM);
+            if (rel >= 0 && rel < WM) {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (acc_row(0, mb, r, lane) == int(rel)) a.tgt[n0 + acc_col(wn, nb, lane)] = acc[mb][nb][r];
+            }
+        }
+    }
+
+    // merge the 4 partial states of every token (2 lane halves x 2 M-waves) through LDS
+    float* sm = reinterpret_cast<float*>(smem);  // [4 parts][256 tokens][3]
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int col = acc_col(wn, nb, lane);
+        const int part = wm * 2 + (lane >> 5);
+        float* dst = sm + (part * BN + col) * 3;
+        dst[0] = ref[nb];
+        dst[1] = S[nb];
+        dst[2] = U[nb];
+    }
+    __syncthreads();
+    if (tid < BN && n0 + tid < a.N) {
+        float R = -INFINITY;
+        for (int p = 0; p < 4; ++p) R = fmaxf(R, sm[(p * BN + tid) * 3]);
+        float s = 0.f, u = 0.f;
+        for (int p = 0; p < 4; ++p) {
+            const float* src = sm + (p * BN + tid) * 3;
+            const float sc = (src[0] == -INFINITY) ? 0.f : fast_exp2(src[0] - R);
+            s += src[1] * sc;
+            u += src[2] * sc;
+        }
+        float* out = a.partial + (int64_t(n0 + tid) * a.v_splits + vs) * 4;
+        out[0] = R;
+        out[1] = s;
+        out[2] = u;
+        out[3] = 0.f;
+    }
+}
+
+__global__ void head_fill_kernel(float* p, int64_t n, float v) {
+    const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// merges the vocabulary splits of every token: logp, entropy, log_z
+__global__ void head_merge_kernel(const float* partial, const float* tgt, const int64_t* targets, int N, int V,
+                                  int v_splits, float* logp, float* entropy, float* log_z, int32_t* error_flag) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= N) return;
+    const float* p = partial + int64_t(n) * v_splits * 4;
+    float R = -INFINITY;
+    for (int s = 0; s < v_splits; ++s) R = fmaxf(R, p[s * 4]);
+    float S = 0.f, U = 0.f;
+    for (int s = 0; s < v_splits; ++s) {
+        const float sc = (p[s * 4] == -INFINITY) ? 0.f : fast_exp2(p[s * 4] - R);
+        S += p[s * 4 + 1] * sc;
+        U += p[s * 4 + 2] * sc;
+    }
+    constexpr float kLn2Hi = 0.693145751953125f, kLn2Lo = 1.42860677e-06f;
+    const float lz = fmaf(R, kLn2Hi, fmaf(R, kLn2Lo, logf(S)));
+    const int64_t t = targets[n];
+    float lp;
+    if (t < 0 || t >= V) {
+        lp = NAN;
+        if (error_flag) atomicOr(error_flag, TRLK_FLAG_INDEX_OUT_OF_RANGE);
+    } else {
+        lp = tgt[n] - lz;
+    }
+    logp[n] = lp;
+    entropy[n] = lz - U / S;
+    log_z[n] = lz;
+}
+
+// dz pass of the backward: one 256 (vocabulary) x 256 (tokens) tile per workgroup.
+template <int DT>
+__global__ __launch_bounds__(kHeadThreads) void fused_head_dz_kernel(HeadArgs a) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    typedef Elem<DT> E;
+    const int n_tb = (a.N + BN - 1) / BN;
+    const int n_vt = (a.c1 - a.c0 + BM - 1) / BM;
+    int tb, vt;
+    xcd_patch(blockIdx.x, n_vt, tb, vt);
+    if (tb >= n_tb || vt >= n_vt) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int n0 = tb * BN, m0 = a.c0 + vt * BM;
+    const Operand W{a.weight, a.ldw, a.V}, Hd{a.hidden, a.ldh, a.N};
+    f32x16 acc[MB][NB];
+    gemm_tile_nt<DT>(W, m0, Hd, n0, a.H, acc, smem);
+
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int tok = n0 + acc_col(wn, nb, lane);
+        const bool tok_ok = tok < a.N;
+        const float g = tok_ok ? a.g[tok] : 0.f;
+        const float lzc = tok_ok ? a.log_z[tok] * kLog2e : 0.f;
+        const int64_t tg = tok_ok ? a.targets[tok] : -1;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            float d[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int v = m0 + acc_row(wm, mb, r, lane);
+                float y = acc[mb][nb][r] * a.logit_scale;
+                float chain = a.inv_t * a.logit_scale;
+                if (a.softcap > 0.f) {
+                    const float th = tanhf(y / a.softcap);
+                    y = th * a.softcap;
+                    chain *= 1.f - th * th;
+                }
+                const float z = y * a.inv_t;
+                const float p = fast_exp2(fmaf(z, kLog2e, -lzc));
+                float dzv = -g * p;
+                if (v == tg) dzv += g;
+                d[r] = (v < a.c1 && tok_ok) ? dzv * chain : 0.f;
+            }
+            // dz^T [chunk row][token]: lanes = consecutive tokens -> 64-byte runs per vocabulary row
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int vrow = vt * BM + acc_row(wm, mb, r, lane);  // chunk-local (padding rows are written as 0)
+                E::store1(a.dzT + int64_t(vrow) * a.ldzt + (n0 + acc_col(wn, nb, lane)), d[r]);
+            }
+            // dz [token][chunk column]: 4 consecutive vocabulary entries per register group
+            if (tok_ok) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int vcol = vt * BM + acc_row(wm, mb, q * 4, lane);
+                    uint2 w;
+                    w.x = E::pack2(d[q * 4 + 0], d[q * 4 + 1]);
+                    w.y = E::pack2(d[q * 4 + 2], d[q * 4 + 3]);
+                    *reinterpret_cast<uint2*>(a.dz + int64_t(tok) * a.ldz + vcol) = w;
+                }
+            }
+        }
+    }
+}
+
+// Plain NT product with an output epilogue: C[M, N] (+)= A[M, K] * B[N, K]^T.
+//   MODE 0: store to `out_lp` in the storage dtype.
+//   MODE 1: fp32 accumulate into `out_f32` (first = overwrite).
+//   MODE 2: like 1 but the sum is rounded into `out_lp` instead of being written back (last chunk).
+struct GemmArgs {
+    Operand A, B;
+    int M, N, K;
+    float* out_f32;
+    int64_t ld_f32;
+    uint16_t* out_lp;
+    int64_t ld_lp;
+    int first;
+};
+
+template <int DT, int MODE>
+__global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmArgs a) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    typedef Elem<DT> E;
+    const int n_mt = (a.M + BM - 1) / BM, n_nt = (a.N + BN - 1) / BN;
+    int tm, tn;
+    xcd_patch(blockIdx.x, n_nt, tm, tn);
+    if (tm >= n_mt || tn >= n_nt) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int m0 = tm * BM, n0 = tn * BN;
+    f32x16 acc[MB][NB];
+    gemm_tile_nt<DT>(a.A, m0, a.B, n0, a.K, acc, smem);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int col = n0 + acc_col(wn, nb, lane);
+            if (col >= a.N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + acc_row(wm, mb, r, lane);
+                if (row >= a.M) continue;
+                float v = acc[mb][nb][r];
+                if (MODE != 0 && !a.first) v += a.out_f32[int64_t(row) * a.ld_f32 + col];
+                if (MODE == 1)
+                    a.out_f32[int64_t(row) * a.ld_f32 + col] = v;
+                else
+                    E::store1(a.out_lp + int64_t(row) * a.ld_lp + col, v);
+            }
+        }
+}
+
+// [R, C] (ld) -> [C, ldo] with columns >= R zero-filled up to ldo: 64 x 64 tiles through LDS.
+__global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* in, int64_t ld, int R, int C, uint16_t* out,
+                                                          int64_t ldo) {
+    __shared__ uint16_t tile[64][66];
+    const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int i = ty; i < 64; i += 4) {
+        const int r = r0 + i, c = c0 + tx;
+        tile[i][tx] = (r < R && c < C) ? in[int64_t(r) * ld + c] : uint16_t(0);
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+        const int c = c0 + i, r = r0 + tx;
+        if (c < C && r < ldo) out[int64_t(c) * ldo + r] = tile[tx][i];
+    }
+}
+
+int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+struct BwdLayout {
+    int64_t vpad, npad, cpad;
+    size_t off_wt, off_ht, off_dz, off_dzt, off_dh, total;
+};
+BwdLayout bwd_layout(int64_t N, int64_t V, int64_t H, int64_t chunk) {
+    BwdLayout l;
+    l.vpad = round_up(V, BK);
+    l.npad = round_up(N, BN);
+    l.cpad = round_up(chunk < V ? chunk : V, BM);
+    size_t o = 0;
+    auto take = [&](size_t bytes) {
+        const size_t at = o;
+        o += (bytes + 255) / 256 * 256;
+        return at;
+    };
+    l.off_wt = take(size_t(H) * l.vpad * 2);
+    l.off_ht = take(size_t(H) * l.npad * 2);
+    l.off_dz = take(size_t(N) * l.cpad * 2);
+    l.off_dzt = take(size_t(l.cpad) * l.npad * 2);
+    l.off_dh = take(size_t(N) * H * 4);
+    l.total = o;
+    return l;
+}
+
+constexpr int kFwdSplits = 8;
+
+int check_head(const char* what, const void* hidden, const void* weight, const int64_t* targets, int dtype, int64_t N,
+               int64_t V, int64_t H, int64_t ldh, int64_t ldw, float temperature) {
+    TRLK_REQUIRE(dtype == TRLK_BF16 || dtype == TRLK_F16, TRLK_ERR_BAD_DTYPE,
+                 "%s: the fused head takes bf16 or fp16 operands (dtype code %d)", what, dtype);
+    TRLK_REQUIRE(N >= 0 && V >= 1 && H >= 1, TRLK_ERR_BAD_SHAPE, "%s: bad sizes N=%lld V=%lld H=%lld", what, (long long)N,
+                 (long long)V, (long long)H);
+    TRLK_REQUIRE(N < (int64_t(1) << 31) - BN && V < (int64_t(1) << 31) - BM, TRLK_ERR_BAD_SHAPE, "%s: N or V too large",
+                 what);
+    TRLK_REQUIRE(H % 8 == 0 && ldh % 8 == 0 && ldw % 8 == 0 && ldh >= H && ldw >= H, TRLK_ERR_BAD_STRIDE,
+                 "%s: H and the row strides must be multiples of 8 elements (H=%lld ldh=%lld ldw=%lld)", what,
+                 (long long)H, (long long)ldh, (long long)ldw);
+    TRLK_REQUIRE(temperature > 0.f && temperature < INFINITY, TRLK_ERR_BAD_VALUE, "%s: temperature must be positive", what);
+    if (N > 0) {
+        TRLK_REQUIRE(hidden && weight && targets, TRLK_ERR_NULL_POINTER, "%s: null operand pointer", what);
+        TRLK_REQUIRE(reinterpret_cast<uintptr_t>(hidden) % 16 == 0 && reinterpret_cast<uintptr_t>(weight) % 16 == 0,
+                     TRLK_ERR_BAD_STRIDE, "%s: operands must be 16-byte aligned", what);
+    }
+    return TRLK_OK;
+}
+
+template <typename Kern, typename Args>
+int launch_head(Kern kern, int grid, const Args& a, hipStream_t s, const char* what) {
+    static thread_local const void* configured[16] = {};
+    // dynamic LDS above 64 KiB has to be allowed per kernel once
+    bool done = false;
+    for (const void* c : configured) done |= (c == reinterpret_cast<const void*>(kern));
+    if (!done) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kHeadLdsBytes);
+        if (e != hipSuccess) return fail(int(e), "%s: cannot reserve %d bytes of LDS: %s", what, kHeadLdsBytes, hipGetErrorString(e));
+        for (const void*& c : configured)
+            if (c == nullptr) {
+                c = reinterpret_cast<const void*>(kern);
+                break;
+            }
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kHeadThreads), kHeadLdsBytes, s, a);
+    return launch_status(what);
+}
+
+}  // namespace
+}  // namespace trlk
+
+using namespace trlk;
+
+extern "C" size_t trlk_fused_head_fwd_workspace_bytes(int64_t n_tokens) {
+    return n_tokens > 0 ? size_t(n_tokens) * (kFwdSplits * 4 + 1) * sizeof(float) : 0;
+}
+
+extern "C" size_t trlk_fused_head_bwd_workspace_bytes(int64_t n_tokens, int64_t vocab, int64_t hidden_size,
+                                                      int64_t chunk_size) {
+    if (n_tokens <= 0 || vocab <= 0 || hidden_size <= 0 || chunk_size <= 0) return 0;
+    return bwd_layout(n_tokens, vocab, hidden_size, chunk_size).total;
+}
+
+extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, const int64_t* d_targets, int dtype,
+                                   int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
+                                   int64_t weight_stride, float temperature, float final_logit_softcapping,
+                                   float logit_scale, float* d_out_logp, float* d_out_entropy, float* d_out_log_z,
+                                   int32_t* d_error_flag, void* d_workspace, size_t workspace_bytes,
+                                   trlk_stream_t stream) {
+    clear_error();
+    if (int rc = check_head("fused_head_fwd", d_hidden, d_weight, d_targets, dtype, n_tokens, vocab, hidden_size,
+                            hidden_stride, weight_stride, temperature))
+        return rc;
+    if (n_tokens == 0) return TRLK_OK;
+    TRLK_REQUIRE(d_out_logp && d_out_entropy && d_out_log_z, TRLK_ERR_NULL_POINTER, "fused_head_fwd: null output pointer");
+    TRLK_REQUIRE(d_workspace && workspace_bytes >= trlk_fused_head_fwd_workspace_bytes(n_tokens), TRLK_ERR_WORKSPACE,
+                 "fused_head_fwd: workspace of %zu bytes needed, %zu given", trlk_fused_head_fwd_workspace_bytes(n_tokens),
+                 workspace_bytes);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    HeadArgs a{};
+    a.hidden = static_cast<const uint16_t*>(d_hidden);
+    a.weight = static_cast<const uint16_t*>(d_weight);
+    a.targets = d_targets;
+    a.N = int(n_tokens);
+    a.V = int(vocab);
+    a.H = int(hidden_size);
+    a.ldh = hidden_stride;
+    a.ldw = weight_stride;
+    a.logit_scale = logit_scale;
+    a.inv_t = 1.f / temperature;
+    a.softcap = final_logit_softcapping > 0.f ? final_logit_softcapping : 0.f;
+    const int n_vt = int((vocab + BM - 1) / BM);
+    a.v_splits = kFwdSplits;
+    a.tiles_per_split = (n_vt + kFwdSplits - 1) / kFwdSplits;
+    a.partial = static_cast<float*>(d_workspace);
+    a.tgt = a.partial + size_t(n_tokens) * kFwdSplits * 4;
+    hipLaunchKernelGGL(head_fill_kernel, dim3(unsigned((n_tokens + 255) / 256)), dim3(256), 0, s, a.tgt, n_tokens, NAN);
+    if (int rc = launch_status("fused_head_fwd (fill)")) return rc;
+    const int n_tb = int((n_tokens + BN - 1) / BN);
+    const int grid = xcd_patch_grid(n_tb, kFwdSplits);
+    int rc = dtype == TRLK_BF16 ? launch_head(fused_head_fwd_kernel<TRLK_BF16>, grid, a, s, "fused_head_fwd")
+                                : launch_head(fused_head_fwd_kernel<TRLK_F16>, grid, a, s, "fused_head_fwd");
+    if (rc) return rc;
+    hipLaunchKernelGGL(head_merge_kernel, dim3(unsigned((n_tokens + 255) / 256)), dim3(256), 0, s, a.partial, a.tgt,
+                       d_targets, int(n_tokens), int(vocab), kFwdSplits, d_out_logp, d_out_entropy, d_out_log_z,
+                       d_error_flag);
+    return launch_status("fused_head_fwd (merge)");
+}
+
+extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, const int64_t* d_targets, int dtype,
+                                   int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
+                                   int64_t weight_stride, float temperature, float final_logit_softcapping,
+                                   float logit_scale, const float* d_log_z, const float* d_g_logp, int64_t chunk_size,
+                                   void* d_out_dhidden, void* d_out_dweight, void* d_workspace, size_t workspace_bytes,
+                                   trlk_stream_t stream) {
+    clear_error();
+    if (int rc = check_head("fused_head_bwd", d_hidden, d_weight, d_targets, dtype, n_tokens, vocab, hidden_size,
+                            hidden_stride, weight_stride, temperature))
+        return rc;
+    TRLK_REQUIRE(chunk_size >= 1, TRLK_ERR_BAD_VALUE, "fused_head_bwd: chunk_size must be >= 1");
+    TRLK_REQUIRE(d_out_dhidden && d_out_dweight, TRLK_ERR_NULL_POINTER, "fused_head_bwd: null output pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t es = 2;
+    if (n_tokens == 0) {  // no tokens: both gradients are zero
+        hipLaunchKernelGGL(head_fill_kernel, dim3(unsigned((vocab * hidden_size / 2 + 255) / 256)), dim3(256), 0, s,
+                           static_cast<float*>(d_out_dweight), vocab * hidden_size / 2, 0.f);
+        return launch_status("fused_head_bwd (zero dW)");
+    }
+    TRLK_REQUIRE(d_log_z && d_g_logp, TRLK_ERR_NULL_POINTER, "fused_head_bwd: log_z / g_logp pointer is null");
+    const int64_t chunk = round_up(chunk_size < vocab ? chunk_size : vocab, BM);
+    const BwdLayout l = bwd_layout(n_tokens, vocab, hidden_size, chunk);
+    TRLK_REQUIRE(d_workspace && workspace_bytes >= l.total, TRLK_ERR_WORKSPACE,
+                 "fused_head_bwd: workspace of %zu bytes needed, %zu given", l.total, workspace_bytes);
+    char* ws = static_cast<char*>(d_workspace);
+    uint16_t* wt = reinterpret_cast<uint16_t*>(ws + l.off_wt);    // [H, vpad]
+    uint16_t* ht = reinterpret_cast<uint16_t*>(ws + l.off_ht);    // [H, npad]
+    uint16_t* dz = reinterpret_cast<uint16_t*>(ws + l.off_dz);    // [N, cpad]
+    uint16_t* dzt = reinterpret_cast<uint16_t*>(ws + l.off_dzt);  // [cpad, npad]
+    float* dh = reinterpret_cast<float*>(ws + l.off_dh);          // [N, H]
+    (void)es;
+    const int H = int(hidden_size), N = int(n_tokens), V = int(vocab);
+    hipLaunchKernelGGL(transpose16_kernel, dim3((H + 63) / 64, unsigned((l.vpad + 63) / 64)), dim3(256), 0, s,
+                       static_cast<const uint16_t*>(d_weight), weight_stride, V, H, wt, l.vpad);
+    if (int rc = launch_status("fused_head_bwd (W^T)")) return rc;
+    hipLaunchKernelGGL(transpose16_kernel, dim3((H + 63) / 64, unsigned((l.npad + 63) / 64)), dim3(256), 0, s,
+                       static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.npad);
+    if (int rc = launch_status("fused_head_bwd (hidden^T)")) return rc;
+
+    HeadArgs a{};
+    a.hidden = static_cast<const uint16_t*>(d_hidden);
+    a.weight = static_cast<const uint16_t*>(d_weight);
+    a.targets = d_targets;
+    a.N = N;
+    a.V = V;
+    a.H = H;
+    a.ldh = hidden_stride;
+    a.ldw = weight_stride;
+    a.logit_scale = logit_scale;
+    a.inv_t = 1.f / temperature;
+    a.softcap = final_logit_softcapping > 0.f ? final_logit_softcapping : 0.f;
+    a.log_z = d_log_z;
+    a.g = d_g_logp;
+    a.dz = dz;
+    a.dzT = dzt;
+    a.ldz = l.cpad;
+    a.ldzt = l.npad;
+    const int n_tb = int((n_tokens + BN - 1) / BN);
+    const int n_ht = (H + BN - 1) / BN;
+    for (int64_t c0 = 0; c0 < vocab; c0 += chunk) {
+        const int64_t c1 = c0 + chunk < vocab ? c0 + chunk : vocab;
+        const int rows = int(c1 - c0);
+        const int kpad = int(round_up(rows, BM));  // dz / dz^T are zero beyond the chunk's rows
+        a.c0 = int(c0);
+        a.c1 = int(c1);
+        const int n_vt = (rows + BM - 1) / BM;
+        int rc = dtype == TRLK_BF16
+                     ? launch_head(fused_head_dz_kernel<TRLK_BF16>, xcd_patch_grid(n_tb, n_vt), a, s, "fused_head_bwd (dz)")
+                     : launch_head(fused_head_dz_kernel<TRLK_F16>, xcd_patch_grid(n_tb, n_vt), a, s, "fused_head_bwd (dz)");
+        if (rc) return rc;
+        const bool first = c0 == 0, last = c1 == vocab;
+        // dHidden[N, H] += dz[N, chunk] * (W^T[H, chunk])^T ; W^T columns beyond V are zero and so is dz there
+        GemmArgs gh{};
+        gh.A = Operand{dz, l.cpad, N};
+        gh.B = Operand{wt + c0, l.vpad, H};
+        gh.M = N;
+        gh.N = H;
+        gh.K = int(c0 + kpad <= l.vpad ? kpad : l.vpad - c0);
+        gh.out_f32 = dh;
+        gh.ld_f32 = H;
+        gh.out_lp = static_cast<uint16_t*>(d_out_dhidden);
+        gh.ld_lp = H;
+        gh.first = first;
+        const int ghgrid = xcd_patch_grid(n_tb, n_ht);
+        if (last)
+            rc = dtype == TRLK_BF16 ? launch_head(gemm_nt_kernel<TRLK_BF16, 2>, ghgrid, gh, s, "fused_head_bwd (dHidden)")
+                                    : launch_head(gemm_nt_kernel<TRLK_F16, 2>, ghgrid, gh, s, "fused_head_bwd (dHidden)");
+        else
+            rc = dtype == TRLK_BF16 ? launch_head(gemm_nt_kernel<TRLK_BF16, 1>, ghgrid, gh, s, "fused_head_bwd (dHidden)")
+                                    : launch_head(gemm_nt_kernel<TRLK_F16, 1>, ghgrid, gh, s, "fused_head_bwd (dHidden)");
+        if (rc) return rc;
+        // dW[chunk, H] = dz^T[chunk, N] * (hidden^T[H, N])^T
+        GemmArgs gw{};
+        gw.A = Operand{dzt, l.npad, kpad};
+        gw.B = Operand{ht, l.npad, H};
+        gw.M = rows;
+        gw.N = H;
+        gw.K = int(l.npad);
+        gw.out_lp = static_cast<uint16_t*>(d_out_dweight) + c0 * hidden_size;
+        gw.ld_lp = hidden_size;
+        gw.first = 1;
+        rc = dtype == TRLK_BF16
+                 ? launch_head(gemm_nt_kernel<TRLK_BF16, 0>, xcd_patch_grid(n_vt, n_ht), gw, s, "fused_head_bwd (dW)")
+                 : launch_head(gemm_nt_kernel<TRLK_F16, 0>, xcd_patch_grid(n_vt, n_ht), gw, s, "fused_head_bwd (dW)");
+        if (rc) return rc;
+    }
+    return TRLK_OK;
+}

@@ -370,4 +370,94 @@ def _rloo_setup(ctx, inputs, output):
 
 rloo_loss_op.register_autograd(_seq_backward, setup_context=_rloo_setup)
 
+
+
+# --------------------------------------------------------------------------------------------
+# fused lm_head + log-prob (K5 / K6)
+# --------------------------------------------------------------------------------------------
+def _head_operands(hidden: Tensor, weight: Tensor, targets: Tensor):
+    if hidden.dim() != 2 or weight.dim() != 2 or targets.dim() != 1:
+        raise ValueError("fused head: expected hidden [N, H], weight [V, H], targets [N]")
+    if hidden.shape[1] != weight.shape[1] or hidden.shape[0] != targets.shape[0]:
+        raise ValueError(f"fused head: shapes do not match: hidden {tuple(hidden.shape)}, weight {tuple(weight.shape)}, "
+                         f"targets {tuple(targets.shape)}")
+    if hidden.dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError(f"fused head: hidden must be bfloat16 or float16 (got {hidden.dtype}); the matrix-core kernels "
+                        "have no fp32/fp64 operand path")
+    if weight.dtype != hidden.dtype:
+        weight = weight.to(hidden.dtype)  # the reference casts the weight slab to the hidden dtype (utils.py:1328)
+    if hidden.shape[1] % 8 != 0:
+        raise ValueError("fused head: hidden_size must be a multiple of 8")
+
+    def rows_ok(t):
+        return t.stride(1) == 1 and t.stride(0) % 8 == 0 and t.stride(0) >= t.shape[1] and t.data_ptr() % 16 == 0
+
+    if not rows_ok(hidden):
+        hidden = hidden.contiguous()
+    if not rows_ok(weight):
+        weight = weight.contiguous()
+    if targets.dtype != torch.int64:
+        targets = targets.long()
+    return hidden, weight, targets.contiguous()
+
+
+@torch.library.custom_op("trl_amd::fused_head_fwd", mutates_args=(), device_types="cuda")
+def fused_head_fwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature: float, softcap: float,
+                   logit_scale: float) -> tuple[Tensor, Tensor, Tensor]:
+    """hidden [N, H], weight [V, H] (bf16/fp16), targets int64 [N] -> fp32 (logp, entropy, log_z), each [N].
+    `softcap <= 0` means no soft-capping."""
+    hidden, weight, targets = _head_operands(hidden, weight, targets)
+    n, h = hidden.shape
+    v = weight.shape[0]
+    dev = hidden.device
+    logp = torch.empty((n,), dtype=torch.float32, device=dev)
+    ent = torch.empty((n,), dtype=torch.float32, device=dev)
+    log_z = torch.empty((n,), dtype=torch.float32, device=dev)
+    if n == 0:
+        return logp, ent, log_z
+    ws_bytes = lib.trlk_fused_head_fwd_workspace_bytes(n)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        check(lib.trlk_fused_head_fwd(ptr(hidden), ptr(weight), ptr(targets), dtype_code(hidden.dtype), n, v, h,
+                                      hidden.stride(0), weight.stride(0), temperature, softcap, logit_scale, ptr(logp),
+                                      ptr(ent), ptr(log_z), ptr(_error_flag(dev)), ptr(ws), ws_bytes,
+                                      current_stream(dev)))
+    if _SYNC_CHECKS:
+        check_device_errors()
+    return logp, ent, log_z
+
+
+@fused_head_fwd.register_fake
+def _(hidden, weight, targets, temperature, softcap, logit_scale):
+    f = lambda: torch.empty((hidden.shape[0],), dtype=torch.float32, device=hidden.device)  # noqa: E731
+    return f(), f(), f()
+
+
+@torch.library.custom_op("trl_amd::fused_head_bwd", mutates_args=(), device_types="cuda")
+def fused_head_bwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature: float, softcap: float,
+                   logit_scale: float, log_z: Tensor, g_logp: Tensor, chunk_size: int) -> tuple[Tensor, Tensor]:
+    """Returns (d hidden [N, H], d weight [V, H]) in the operand dtype."""
+    w_dtype = weight.dtype
+    hidden, weight, targets = _head_operands(hidden, weight, targets)
+    n, h = hidden.shape
+    v = weight.shape[0]
+    dev = hidden.device
+    d_hidden = torch.empty((n, h), dtype=hidden.dtype, device=dev)
+    d_weight = torch.empty((v, h), dtype=hidden.dtype, device=dev)
+    g = g_logp.contiguous().float()
+    ws_bytes = lib.trlk_fused_head_bwd_workspace_bytes(max(n, 1), v, h, chunk_size)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        check(lib.trlk_fused_head_bwd(ptr(hidden), ptr(weight), ptr(targets), dtype_code(hidden.dtype), n, v, h,
+                                      hidden.stride(0), weight.stride(0), temperature, softcap, logit_scale, ptr(log_z),
+                                      ptr(g), chunk_size, ptr(d_hidden), ptr(d_weight), ptr(ws), ws_bytes,
+                                      current_stream(dev)))
+    return d_hidden, (d_weight if w_dtype == d_weight.dtype else d_weight.to(w_dtype))
+
+
+@fused_head_bwd.register_fake
+def _(hidden, weight, targets, temperature, softcap, logit_scale, log_z, g_logp, chunk_size):
+    return torch.empty_like(hidden), torch.empty_like(weight)
+
+
 NAN = math.nan

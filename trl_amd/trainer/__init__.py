@@ -2,4 +2,5 @@ from .dpo_trainer import dpo_loss_from_logits, dpo_per_token_logps, dpo_sigmoid_
 from .grpo_trainer import (GRPOLossMixin, get_high_entropy_mask, get_off_policy_mask, group_advantages, grpo_loss,
                            metrics_to_dict, per_token_logps_and_entropies)
 from .rloo_trainer import rloo_advantages, rloo_loss
-from .utils import entropy_from_logits, logps_and_entropies, nanmax, nanmin, nanstd, selective_log_softmax
+from .utils import (_ChunkedLogProbFunction, chunked_logprobs_from_hidden, entropy_from_logits, logps_and_entropies,
+                    nanmax, nanmin, nanstd, patch_chunked_lm_head, selective_log_softmax)

@@ -10,7 +10,8 @@ from torch import Tensor
 
 from .. import ops
 
-__all__ = ["selective_log_softmax", "entropy_from_logits", "logps_and_entropies", "nanstd", "nanmin", "nanmax"]
+__all__ = ["selective_log_softmax", "entropy_from_logits", "logps_and_entropies", "nanstd", "nanmin", "nanmax",
+           "_ChunkedLogProbFunction", "chunked_logprobs_from_hidden", "patch_chunked_lm_head"]
 
 
 def _as_3d(logits: Tensor) -> Tensor:
@@ -134,3 +135,85 @@ def nanmax(tensor: Tensor) -> Tensor:
     if not keep.any():
         return torch.tensor(float("nan"), dtype=tensor.dtype, device=tensor.device)
     return tensor[keep].max()
+
+
+# ----------------------------------------------------------------------------------------------
+# fused lm_head + log-prob (reference: trl/trainer/utils.py:1291-1517)
+# ----------------------------------------------------------------------------------------------
+class _ChunkedLogProbFunction(torch.autograd.Function):
+    """Per-token log-probs and entropy of `softmax((hidden @ weight.T) / temperature)` without ever
+    materialising the `[N, V]` logits.  Same call signature as the reference operator
+    (utils.py:1298-1307): `apply(last_hidden [N, H], weight [V, H], targets [N], temperature,
+    chunk_size, final_logit_softcapping=None, logit_scale=1.0) -> (logprobs fp32 [N], entropy fp32 [N])`.
+
+    The forward is one matrix-core kernel sweep (no vocabulary chunking is needed, `chunk_size` only
+    sizes the backward's dz workspace).  The entropy output is not differentiable, as in the reference."""
+
+    @staticmethod
+    def forward(ctx, last_hidden, weight, targets, temperature, chunk_size, final_logit_softcapping=None,
+                logit_scale=1.0):
+        cap = 0.0 if final_logit_softcapping is None else float(final_logit_softcapping)
+        logp, ent, log_z = ops.fused_head_fwd(last_hidden, weight, targets, float(temperature), cap, float(logit_scale))
+        ctx.save_for_backward(last_hidden, weight, targets, log_z)
+        ctx.cfg = (float(temperature), int(chunk_size), cap, float(logit_scale))
+        ctx.mark_non_differentiable(ent)
+        return logp, ent
+
+    @staticmethod
+    def backward(ctx, grad_logprobs, grad_entropy):
+        hidden, weight, targets, log_z = ctx.saved_tensors
+        temperature, chunk_size, cap, logit_scale = ctx.cfg
+        d_hidden, d_weight = ops.fused_head_bwd(hidden, weight, targets, temperature, cap, logit_scale, log_z,
+                                                grad_logprobs, chunk_size)
+        return d_hidden, d_weight, None, None, None, None, None
+
+
+def chunked_logprobs_from_hidden(hidden_states: Tensor, lm_head_weight: Tensor, labels: Tensor,
+                                 completion_mask: Tensor | None, temperature: float, chunk_size: int = 8192,
+                                 final_logit_softcapping: float | None = None, logit_scale: float = 1.0):
+    """The tensor part of the reference's patched forward (utils.py:1449-1484): shift by one, keep only
+    completion rows, run the fused head on them, scatter into zero-filled `[B, S-1]` outputs.
+    Returns `(log_probs, entropy)`."""
+    hs = hidden_states[:, :-1, :]
+    lab = labels[:, 1:]
+    b, s, h = hs.shape
+    flat_h = hs.reshape(b * s, h)
+    flat_t = lab.reshape(b * s)
+    keep = None
+    if completion_mask is not None:
+        keep = completion_mask[:, 1:].bool().reshape(b * s)
+        flat_h = flat_h[keep]
+        flat_t = flat_t[keep]
+    lp_v, ent_v = _ChunkedLogProbFunction.apply(flat_h, lm_head_weight, flat_t, temperature, chunk_size,
+                                                final_logit_softcapping, logit_scale)
+    if keep is None:
+        return lp_v.reshape(b, s), ent_v.reshape(b, s)
+    lp = torch.zeros(b * s, device=lp_v.device, dtype=lp_v.dtype)
+    ent = torch.zeros(b * s, device=ent_v.device, dtype=ent_v.dtype)
+    lp[keep] = lp_v
+    ent[keep] = ent_v
+    return lp.reshape(b, s), ent.reshape(b, s)
+
+
+def patch_chunked_lm_head(model: torch.nn.Module, chunk_size: int, temperature: float,
+                          output_router_logits: bool = False) -> None:
+    """Replaces `model.forward` by one that runs the backbone, then the fused head, and returns
+    `{"log_probs" [B, S-1], "entropy" [B, S-1], "aux_loss"}` (reference: utils.py:1427-1517).
+    The MoE load-balancing auxiliary loss of the reference is not reproduced here."""
+    import types
+
+    if output_router_logits:
+        raise NotImplementedError("patch_chunked_lm_head(output_router_logits=True) is not implemented by trl_amd")
+    final_logit_softcapping = getattr(model.config, "final_logit_softcapping", None)
+
+    def _chunked_forward(self, input_ids=None, attention_mask=None, labels=None, completion_mask=None,
+                         use_cache=False, **kwargs):
+        assert labels is not None, "requires labels to not be None for logprob computation"
+        outputs = self.model(input_ids=input_ids, attention_mask=attention_mask, use_cache=use_cache, **kwargs)
+        logit_scale = getattr(self.config, "logit_scale", 1.0)
+        log_probs, entropy = chunked_logprobs_from_hidden(
+            outputs.last_hidden_state, self.lm_head.weight, labels, completion_mask, temperature, chunk_size,
+            final_logit_softcapping, logit_scale)
+        return {"log_probs": log_probs, "entropy": entropy, "aux_loss": None}
+
+    model.forward = types.MethodType(_chunked_forward, model)
