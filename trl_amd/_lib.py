@@ -13,7 +13,8 @@ from ctypes import c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p
 
 import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libtrlk.so")
+# TRLK_LIBRARY_PATH points at another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("TRLK_LIBRARY_PATH") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libtrlk.so")
 
 F32, BF16, F16 = 0, 1, 2
 GRPO, BNPO, DR_GRPO, DAPO = 0, 1, 2, 3

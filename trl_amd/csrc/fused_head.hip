@@ -25,14 +25,40 @@
 namespace trlk {
 namespace {
 
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kHeadThreads = 512;
-constexpr int kLdsRow = BK + 8;  // bf16 elements per LDS row: 144 bytes, conflict-free 16-byte reads
-constexpr int WM = 128, WN = 64;  // per-wave tile
-constexpr int WGN = BN / WN;      // 4 waves along N, 2 along M
+// Tile configuration (overridable with -D for experiments).
+#ifndef TRLK_HEAD_BM
+#define TRLK_HEAD_BM 256
+#endif
+#ifndef TRLK_HEAD_BN
+#define TRLK_HEAD_BN 256
+#endif
+#ifndef TRLK_HEAD_BK
+#define TRLK_HEAD_BK 64
+#endif
+#ifndef TRLK_HEAD_WGM
+#define TRLK_HEAD_WGM 2
+#endif
+#ifndef TRLK_HEAD_WGN
+#define TRLK_HEAD_WGN 4
+#endif
+constexpr int BM = TRLK_HEAD_BM, BN = TRLK_HEAD_BN, BK = TRLK_HEAD_BK;
+constexpr int WGM = TRLK_HEAD_WGM, WGN = TRLK_HEAD_WGN;  // waves along M and N
+constexpr int kHeadThreads = WGM * WGN * 64;
+#ifndef TRLK_HEAD_WAVES_PER_EU
+#define TRLK_HEAD_WAVES_PER_EU 2
+#endif
+#define TRLK_HEAD_KERNEL __global__ __launch_bounds__(kHeadThreads) __attribute__((amdgpu_waves_per_eu(TRLK_HEAD_WAVES_PER_EU, TRLK_HEAD_WAVES_PER_EU)))
+constexpr int kLdsRow = BK + 8;  // elements per LDS row: 16 bytes of padding keep 16-byte reads conflict-free
+constexpr int WM = BM / WGM, WN = BN / WGN;  // per-wave tile
 constexpr int MB = WM / 32, NB = WN / 32;
-constexpr int kTileLdsBytes = BM * kLdsRow * 2;          // one operand tile
-constexpr int kHeadLdsBytes = 4 * kTileLdsBytes;         // A and B, two stages = 147456 bytes
+constexpr int kCpr = BK / 8;                        // 16-byte chunks per tile row
+constexpr int kRowStep = kHeadThreads / kCpr;       // rows staged per pass of the workgroup
+constexpr int kLoadsA = BM / kRowStep, kLoadsB = BN / kRowStep;
+constexpr int kTileABytes = BM * kLdsRow * 2, kTileBBytes = BN * kLdsRow * 2;
+constexpr int kStageBytes = kTileABytes + kTileBBytes;
+constexpr int kHeadLdsBytes = 2 * kStageBytes;  // two stages
+static_assert(2 * WGM * BN * 3 * 4 <= kHeadLdsBytes && BN <= kHeadThreads, "merge scratch");
+static_assert(BM % kRowStep == 0 && BN % kRowStep == 0 && WM % 32 == 0 && WN % 32 == 0 && BK % 16 == 0, "tile shape");
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -63,19 +89,29 @@ __device__ __forceinline__ void gemm_tile_nt(const Operand A, int m0, const Oper
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
-    const int kc = tid & 7, r0 = tid >> 3;  // this thread stages rows r0 + 64*j, 16-byte column chunk kc
+    const int kc = tid % kCpr, r0 = tid / kCpr;  // this thread stages rows r0 + kRowStep*j, 16-byte chunk kc
 
-    const uint16_t* ga[4];
-    const uint16_t* gb[4];
+    // uniform tile base + 32-bit per-lane byte offsets (a tile spans < 4 GiB)
+#if defined(TRLK_EXP_SAMETILE)
+    m0 = 0;  // experiment: every workgroup reads the same tile (all loads hit L2; results are wrong)
+    n0 = 0;
+#endif
+    const char* abase = reinterpret_cast<const char*>(A.p + int64_t(m0) * A.ld);
+    const char* bbase = reinterpret_cast<const char*>(B.p + int64_t(n0) * B.ld);
+    uint32_t ao[kLoadsA], bo[kLoadsB];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        int ra = m0 + r0 + 64 * j, rb = n0 + r0 + 64 * j;
-        ra = ra < A.rows ? ra : A.rows - 1;
-        rb = rb < B.rows ? rb : B.rows - 1;
-        ga[j] = A.p + int64_t(ra) * A.ld + kc * 8;
-        gb[j] = B.p + int64_t(rb) * B.ld + kc * 8;
+    for (int j = 0; j < kLoadsA; ++j) {
+        int ra = r0 + kRowStep * j;
+        ra = m0 + ra < A.rows ? ra : A.rows - 1 - m0;  // clamp to the operand's last row
+        ao[j] = uint32_t((int64_t(ra) * A.ld + kc * 8) * 2);
     }
-    const int st_off = (r0 * kLdsRow + kc * 8) * 2;        // + j * 64 rows
+#pragma unroll
+    for (int j = 0; j < kLoadsB; ++j) {
+        int rb = r0 + kRowStep * j;
+        rb = n0 + rb < B.rows ? rb : B.rows - 1 - n0;
+        bo[j] = uint32_t((int64_t(rb) * B.ld + kc * 8) * 2);
+    }
+    const int st_off = (r0 * kLdsRow + kc * 8) * 2;        // + j * kRowStep rows
     const int fa_off = ((wm * WM + (lane & 31)) * kLdsRow + (lane >> 5) * 8) * 2;  // + mb*32 rows, + ks*16
     const int fb_off = ((wn * WN + (lane & 31)) * kLdsRow + (lane >> 5) * 8) * 2;
 
@@ -86,35 +122,35 @@ __device__ __forceinline__ void gemm_tile_nt(const Operand A, int m0, const Oper
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0.f;
 
-    u32x4 ra[4], rb[4];
     const u32x4 zero = {0u, 0u, 0u, 0u};
-    auto load_stage = [&](int k0) {
-        const bool in = k0 + kc * 8 < K;
+    // full k steps load unconditionally; only the last, partial step (K % BK != 0) masks its chunks
+    auto load_stage = [&](u32x4(&ra)[kLoadsA], u32x4(&rb)[kLoadsB], int k0) {
+        const char* ap = abase + int64_t(k0) * 2;
+        const char* bp = bbase + int64_t(k0) * 2;
+        if (k0 + BK <= K) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            ra[j] = in ? *reinterpret_cast<const u32x4*>(ga[j] + k0) : zero;
-            rb[j] = in ? *reinterpret_cast<const u32x4*>(gb[j] + k0) : zero;
+            for (int j = 0; j < kLoadsA; ++j) ra[j] = *reinterpret_cast<const u32x4*>(ap + ao[j]);
+#pragma unroll
+            for (int j = 0; j < kLoadsB; ++j) rb[j] = *reinterpret_cast<const u32x4*>(bp + bo[j]);
+        } else {
+            const bool in = k0 + kc * 8 < K;
+#pragma unroll
+            for (int j = 0; j < kLoadsA; ++j) ra[j] = in ? *reinterpret_cast<const u32x4*>(ap + ao[j]) : zero;
+#pragma unroll
+            for (int j = 0; j < kLoadsB; ++j) rb[j] = in ? *reinterpret_cast<const u32x4*>(bp + bo[j]) : zero;
         }
     };
-    auto store_stage = [&](int buf) {
-        char* sa = smem + buf * 2 * kTileLdsBytes;
-        char* sb = sa + kTileLdsBytes;
+    auto store_stage = [&](const u32x4(&ra)[kLoadsA], const u32x4(&rb)[kLoadsB], int buf) {
+        char* sa = smem + buf * kStageBytes;
+        char* sb = sa + kTileABytes;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            *reinterpret_cast<u32x4*>(sa + st_off + j * 64 * kLdsRow * 2) = ra[j];
-            *reinterpret_cast<u32x4*>(sb + st_off + j * 64 * kLdsRow * 2) = rb[j];
-        }
+        for (int j = 0; j < kLoadsA; ++j) *reinterpret_cast<u32x4*>(sa + st_off + j * kRowStep * kLdsRow * 2) = ra[j];
+#pragma unroll
+        for (int j = 0; j < kLoadsB; ++j) *reinterpret_cast<u32x4*>(sb + st_off + j * kRowStep * kLdsRow * 2) = rb[j];
     };
-
-    const int nk = (K + BK - 1) / BK;
-    load_stage(0);
-    store_stage(0);
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const bool more = kt + 1 < nk;
-        if (more) load_stage((kt + 1) * BK);
-        const char* sa = smem + (kt & 1) * 2 * kTileLdsBytes;
-        const char* sb = sa + kTileLdsBytes;
+    auto compute = [&](int buf) {
+        const char* sa = smem + buf * kStageBytes;
+        const char* sb = sa + kTileABytes;
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
             u32x4 fa[MB], fb[NB];
@@ -129,8 +165,31 @@ __device__ __forceinline__ void gemm_tile_nt(const Operand A, int m0, const Oper
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = mfma<DT>(fa[mb], fb[nb], acc[mb][nb]);
         }
-        if (more) store_stage((kt + 1) & 1);
+    };
+
+    // Registers hold the tile of step kt+1 while step kt computes out of LDS; it is written to the
+    // other LDS buffer at the end of the step (one barrier per step).
+    const int nk = (K + BK - 1) / BK;
+    u32x4 ra[kLoadsA], rb[kLoadsB];
+    load_stage(ra, rb, 0);
+    store_stage(ra, rb, 0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+#if defined(TRLK_EXP_NOGLOBAL)
+        const bool more = false;  // experiment: measures the LDS + MFMA loop alone (results are wrong)
+#else
+        const bool more = kt + 1 < nk;
+#endif
+        if (more) load_stage(ra, rb, (kt + 1) * BK);
+#if defined(TRLK_EXP_NOGLOBAL)
+        compute(0);
+#else
+        compute(kt & 1);
+#endif
+        if (more) store_stage(ra, rb, (kt + 1) & 1);
+#if !defined(TRLK_EXP_NOBARRIER)
         __syncthreads();
+#endif
     }
 }
 
@@ -183,7 +242,7 @@ __device__ __forceinline__ float head_z(float y, const HeadArgs& a) {
 }
 
 template <int DT>
-__global__ __launch_bounds__(kHeadThreads) void fused_head_fwd_kernel(HeadArgs a) {
+TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int n_tb = (a.N + BN - 1) / BN;
     int tb, vs;
@@ -259,8 +318,9 @@ __global__ __launch_bounds__(kHeadThreads) void fused_head_fwd_kernel(HeadArgs a
         }
     }
 
-    // merge the 4 partial states of every token (2 lane halves x 2 M-waves) through LDS
-    float* sm = reinterpret_cast<float*>(smem);  // [4 parts][256 tokens][3]
+    // merge the partial states of every token (2 lane halves x WGM M-waves) through LDS
+    constexpr int kParts = 2 * WGM;
+    float* sm = reinterpret_cast<float*>(smem);  // [kParts][BN tokens][3]
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         const int col = acc_col(wn, nb, lane);
@@ -273,9 +333,9 @@ __global__ __launch_bounds__(kHeadThreads) void fused_head_fwd_kernel(HeadArgs a
     __syncthreads();
     if (tid < BN && n0 + tid < a.N) {
         float R = -INFINITY;
-        for (int p = 0; p < 4; ++p) R = fmaxf(R, sm[(p * BN + tid) * 3]);
+        for (int p = 0; p < kParts; ++p) R = fmaxf(R, sm[(p * BN + tid) * 3]);
         float s = 0.f, u = 0.f;
-        for (int p = 0; p < 4; ++p) {
+        for (int p = 0; p < kParts; ++p) {
             const float* src = sm + (p * BN + tid) * 3;
             const float sc = (src[0] == -INFINITY) ? 0.f : fast_exp2(src[0] - R);
             s += src[1] * sc;
@@ -325,7 +385,7 @@ __global__ void head_merge_kernel(const float* partial, const float* tgt, const 
 
 // dz pass of the backward: one 256 (vocabulary) x 256 (tokens) tile per workgroup.
 template <int DT>
-__global__ __launch_bounds__(kHeadThreads) void fused_head_dz_kernel(HeadArgs a) {
+TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     typedef Elem<DT> E;
     const int n_tb = (a.N + BN - 1) / BN;
@@ -402,7 +462,7 @@ struct GemmArgs {
 };
 
 template <int DT, int MODE>
-__global__ __launch_bounds__(kHeadThreads) void gemm_nt_kernel(GemmArgs a) {
+TRLK_HEAD_KERNEL void gemm_nt_kernel(GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     typedef Elem<DT> E;
     const int n_mt = (a.M + BM - 1) / BM, n_nt = (a.N + BN - 1) / BN;

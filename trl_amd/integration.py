@@ -1,0 +1,50 @@
+"""Binds the kernels into an installed `trl` (the reference) at run time.
+
+TRL has no plugin registry: its hot-path helpers are module-level functions imported *by name* into
+every trainer module, and the loss is a trainer method.  `patch_trl()` therefore rebinds
+  * `selective_log_softmax`, `entropy_from_logits`, `_ChunkedLogProbFunction`, `patch_chunked_lm_head`
+    in `trl.trainer.utils` **and** in every already-imported `trl.*` module that holds its own reference;
+  * `GRPOTrainer._get_per_token_logps_and_entropies` / `_compute_loss` (optional, `grpo=True`).
+`unpatch_trl()` restores the originals.
+"""
+from __future__ import annotations
+
+import sys
+
+from .trainer import grpo_trainer as _grpo
+from .trainer import utils as _utils
+
+_FUNCTIONS = ("selective_log_softmax", "entropy_from_logits", "_ChunkedLogProbFunction", "patch_chunked_lm_head")
+_saved: list[tuple[object, str, object]] = []
+
+
+def patch_trl(grpo: bool = True) -> int:
+    """Returns the number of names rebound.  Needs `trl` to be importable."""
+    import trl.trainer.utils as ref_utils
+
+    if _saved:
+        return 0
+    originals = {name: getattr(ref_utils, name) for name in _FUNCTIONS if hasattr(ref_utils, name)}
+    count = 0
+    for mod_name, mod in list(sys.modules.items()):
+        if mod is None or not (mod_name == "trl" or mod_name.startswith("trl.")):
+            continue
+        for name, orig in originals.items():
+            if getattr(mod, name, None) is orig:
+                _saved.append((mod, name, orig))
+                setattr(mod, name, getattr(_utils, name))
+                count += 1
+    if grpo:
+        from trl.trainer.grpo_trainer import GRPOTrainer
+
+        for name in ("_get_per_token_logps_and_entropies", "_compute_loss"):
+            _saved.append((GRPOTrainer, name, GRPOTrainer.__dict__[name]))
+            setattr(GRPOTrainer, name, getattr(_grpo.GRPOLossMixin, name))
+            count += 1
+    return count
+
+
+def unpatch_trl() -> None:
+    while _saved:
+        obj, name, orig = _saved.pop()
+        setattr(obj, name, orig)
