@@ -81,10 +81,131 @@ struct Operand {
     int rows;
 };
 
+#ifndef TRLK_HEAD_DIRECT_LDS
+#define TRLK_HEAD_DIRECT_LDS 1
+#endif
+
+// Direct-to-LDS variant of the tile loop (K % 64 == 0): `global_load_lds_dwordx4` moves 16 bytes per
+// lane from memory straight into LDS, 1 KiB contiguous per wave instruction = 8 tile rows of 128
+// bytes, with no register staging and no ds_write.  Rows are dense (no padding is possible inside a
+// wave's 1 KiB), so bank conflicts are avoided by an XOR swizzle of the 16-byte chunk index: the
+// chunk at physical position pc of row r holds logical chunk pc ^ (r & 7) ^ ((r >> 3) & 1).  The
+// lane fetches that logical chunk from memory (a permutation inside one 128-byte line, still
+// coalesced) and the fragment reads apply the same XOR.
+template <int DT>
+__device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, const Operand B, int n0, int K,
+                                                    f32x16 (&acc)[MB][NB], char* smem) {
+    static_assert(BK == 64, "the direct-to-LDS layout assumes 128-byte tile rows");
+    constexpr int kWaves = kHeadThreads / 64;
+    constexpr int kBlkA = BM / 8 / kWaves, kBlkB = BN / 8 / kWaves;  // 8-row blocks per wave and stage
+    constexpr int kDenseA = BM * BK * 2, kDenseStage = (BM + BN) * BK * 2;
+    static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0, "blocks per wave");
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+
+    // --- loader side: this lane's row inside a block and the logical chunk it fetches
+    const int rr = lane >> 3, pc = lane & 7;
+    const int kc = pc ^ rr ^ (wave & 1);  // blocks of a wave all have the parity of the wave index
+#if defined(TRLK_EXP_SAMETILE)
+    m0 = 0;  // experiment: every workgroup reads the same tile (all loads hit L2; results are wrong)
+    n0 = 0;
+#endif
+    const char* abase = reinterpret_cast<const char*>(A.p + int64_t(m0) * A.ld);
+    const char* bbase = reinterpret_cast<const char*>(B.p + int64_t(n0) * B.ld);
+    uint32_t ao[kBlkA], bo[kBlkB];
+#pragma unroll
+    for (int j = 0; j < kBlkA; ++j) {
+        int r = (wave + kWaves * j) * 8 + rr;
+        r = m0 + r < A.rows ? r : A.rows - 1 - m0;
+        ao[j] = uint32_t((int64_t(r) * A.ld + kc * 8) * 2);
+    }
+#pragma unroll
+    for (int j = 0; j < kBlkB; ++j) {
+        int r = (wave + kWaves * j) * 8 + rr;
+        r = n0 + r < B.rows ? r : B.rows - 1 - n0;
+        bo[j] = uint32_t((int64_t(r) * B.ld + kc * 8) * 2);
+    }
+    typedef __attribute__((address_space(1))) const void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    auto issue_stage = [&](int buf, int k0) {
+        const char* ap = abase + int64_t(k0) * 2;
+        const char* bp = bbase + int64_t(k0) * 2;
+        char* sa = smem + buf * kDenseStage;
+        char* sb = sa + kDenseA;
+#pragma unroll
+        for (int j = 0; j < kBlkA; ++j)
+            __builtin_amdgcn_global_load_lds((gptr_t)(ap + ao[j]), (lptr_t)(sa + (wave + kWaves * j) * 1024), 16, 0, 0);
+#if !defined(TRLK_EXP_HALFLOADS)
+#pragma unroll
+        for (int j = 0; j < kBlkB; ++j)
+            __builtin_amdgcn_global_load_lds((gptr_t)(bp + bo[j]), (lptr_t)(sb + (wave + kWaves * j) * 1024), 16, 0, 0);
+#endif
+    };
+
+    // --- fragment side
+    const int swz = (lane & 7) ^ ((lane >> 3) & 1);
+    const int hl = lane >> 5;
+    const int fa_row = (wm * WM + (lane & 31)) * 128, fb_row = (wn * WN + (lane & 31)) * 128;
+    int koff[BK / 16];
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) koff[ks] = ((ks * 2 + hl) ^ swz) * 16;
+
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0.f;
+
+    // Fragment loads run one 16-wide k slice ahead of the MFMAs that consume them, so the LDS
+    // latency of slice ks+1 hides behind the 8 MFMAs of slice ks.
+    auto load_frags = [&](const char* sa, const char* sb, int ks, u32x4(&fa)[MB], u32x4(&fb)[NB]) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+            fa[mb] = *reinterpret_cast<const u32x4*>(sa + fa_row + mb * 32 * 128 + koff[ks]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+            fb[nb] = *reinterpret_cast<const u32x4*>(sb + fb_row + nb * 32 * 128 + koff[ks]);
+    };
+    auto compute = [&](int buf) {
+        const char* sa = smem + buf * kDenseStage;
+        const char* sb = sa + kDenseA;
+        u32x4 fa[2][MB], fb[2][NB];
+        load_frags(sa, sb, 0, fa[0], fb[0]);
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            if (ks + 1 < BK / 16) load_frags(sa, sb, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = mfma<DT>(fa[ks & 1][mb], fb[ks & 1][nb], acc[mb][nb]);
+        }
+    };
+
+    const int nk = K / BK;
+    issue_stage(0, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        // the other buffer was last read before the previous barrier: refill it asynchronously now
+#if defined(TRLK_EXP_NOGLOBAL)
+        compute(0);  // experiment: LDS + MFMA loop alone (results are wrong)
+#else
+        if (kt + 1 < nk) issue_stage((kt + 1) & 1, (kt + 1) * BK);
+        compute(kt & 1);
+#endif
+#if !defined(TRLK_EXP_NOWAIT)
+        __builtin_amdgcn_s_waitcnt(0);  // this wave's transfers have landed in LDS
+#endif
+        __syncthreads();                // ... and so have everyone else's; all reads of this buffer are done
+    }
+}
+
 // acc[mb][nb] = sum_k A[m0 + .., k] * B[n0 + .., k].  Rows beyond the operand's end are clamped to
 // its last row (callers ignore those outputs); k beyond K reads as zero (K % 8 == 0).
 template <int DT>
-__device__ __forceinline__ void gemm_tile_nt(const Operand A, int m0, const Operand B, int n0, int K,
+__device__ __forceinline__ void gemm_tile_nt_staged(const Operand A, int m0, const Operand B, int n0, int K,
                                              f32x16 (&acc)[MB][NB], char* smem) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -191,6 +312,17 @@ __device__ __forceinline__ void gemm_tile_nt(const Operand A, int m0, const Oper
         __syncthreads();
 #endif
     }
+}
+
+template <int DT>
+__device__ __forceinline__ void gemm_tile_nt(const Operand A, int m0, const Operand B, int n0, int K,
+                                             f32x16 (&acc)[MB][NB], char* smem) {
+#if TRLK_HEAD_DIRECT_LDS
+    if ((K & (BK - 1)) == 0)
+        gemm_tile_nt_direct<DT>(A, m0, B, n0, K, acc, smem);
+    else
+#endif
+        gemm_tile_nt_staged<DT>(A, m0, B, n0, K, acc, smem);
 }
 
 // Row (M index) inside the workgroup tile of accumulator element r of block mb, for this lane.
