@@ -37,6 +37,9 @@ WORKLOADS = {
                     rewards="normal", desc="GRPO fwd+bwd, bf16 logits [64,1024,151936], T=0.9, G=8, lens~U[64,1024]"),
     "grpo_c4": dict(B=32, T=4096, V=151936, temperature=1.0, G=16, min_len=512, beta=0.0, eps_low=0.2, eps_high=0.28,
                     rewards="bernoulli", desc="long-context GRPO fwd+bwd, bf16 logits [32,4096,151936], G=16"),
+    "head_c5": dict(B=16, T=2048, V=151936, H=3584, temperature=1.0, G=8, min_len=64, beta=0.04, eps_low=0.2,
+                    eps_high=0.2, rewards="normal", head=True,
+                    desc="fused lm_head + log-prob + GRPO loss fwd+bwd, hidden bf16 [16x2048,3584], W bf16 [151936,3584]"),
     "tiny": dict(B=8, T=64, V=151936, temperature=0.9, G=8, min_len=8, beta=0.04, eps_low=0.2, eps_high=0.2,
                  rewards="normal", desc="reduced-size functional check (not a benchmark configuration)"),
 }
@@ -99,6 +102,91 @@ def cpu_baseline(w, loss_type, rows_per_seq=512, n_seq=32, repeats=2):
     }
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
+
+
+def bench_head(args, w):
+    """BASELINE.json config 5: the logits are never materialised.  Step = fused head forward, GRPO loss,
+    fused head backward (dHidden and dW)."""
+    import trl_amd
+    from trl_amd import ops
+
+    dev = torch.device("cuda:0")
+    B, T, V, H = w["B"], w["T"], w["V"], w["H"]
+    N = B * T
+    g = torch.Generator(device=dev).manual_seed(0)
+    hidden = torch.randn((N, H), generator=g, device=dev).bfloat16().requires_grad_(True)
+    weight = (0.02 * torch.randn((V, H), generator=g, device=dev)).bfloat16().requires_grad_(True)
+    targets = torch.randint(0, V, (N,), generator=g, device=dev)
+    lengths = torch.randint(w["min_len"], T + 1, (B,), generator=g, device=dev)
+    mask = (torch.arange(T, device=dev)[None] < lengths[:, None]).long()
+    adv = trl_amd.group_advantages(torch.randn((B,), generator=g, device=dev), w["G"])
+    with torch.no_grad():
+        base, _, _ = ops.fused_head_fwd(hidden, weight, targets, w["temperature"], 0.0, 1.0)
+    base = base.view(B, T)
+    old = base + 0.05 * torch.randn(base.shape, generator=g, device=dev)
+    ref = base + 0.1 * torch.randn(base.shape, generator=g, device=dev)
+    n_items = mask.sum().float()
+
+    def step():
+        hidden.grad = weight.grad = None
+        lp, ent = trl_amd._ChunkedLogProbFunction.apply(hidden, weight, targets, w["temperature"], 8192)
+        loss, _ = trl_amd.grpo_loss(lp.view(B, T), adv, mask, entropies=ent.view(B, T), old_per_token_logps=old,
+                                    ref_per_token_logps=ref, loss_type=args.loss_type, epsilon_low=w["eps_low"],
+                                    epsilon_high=w["eps_high"], beta=w["beta"], max_completion_length=T,
+                                    num_items_in_batch=n_items)
+        loss.backward()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        loss = step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms_per_step = max((time.perf_counter() - t0) * 1e3, e0.elapsed_time(e1)) / args.steps
+
+    def time_op(fn, reps=3):
+        fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps
+
+    with torch.no_grad():
+        _, _, log_z = ops.fused_head_fwd(hidden, weight, targets, w["temperature"], 0.0, 1.0)
+        gl = torch.randn((N,), generator=g, device=dev)
+        fwd_ms = time_op(lambda: ops.fused_head_fwd(hidden, weight, targets, w["temperature"], 0.0, 1.0))
+        bwd_ms = time_op(lambda: ops.fused_head_bwd(hidden, weight, targets, w["temperature"], 0.0, 1.0, log_z, gl, 8192))
+    flop = 2.0 * N * H * V
+    fwd_tf, bwd_tf = flop / (fwd_ms * 1e-3) / 1e12, 3 * flop / (bwd_ms * 1e-3) / 1e12
+    total_tf = 4 * flop / ((fwd_ms + bwd_ms) * 1e-3) / 1e12
+    result = {
+        "metric": "tokens/sec + MFMA bf16 utilisation for fused lm_head+logprob+GRPO loss fwd+bwd",
+        "value": N / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "description": w["desc"], "tokens": N, "hidden": H, "vocab": V,
+                   "loss_type": args.loss_type, "loss": float(loss.detach())},
+        "roofline": {"bound": "mfma", "kernel": "fused head forward + backward (all MFMA kernels)",
+                     "achieved": total_tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": total_tf / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "algorithmic_flop": 4 * flop, "avg_launch_ms": fwd_ms + bwd_ms},
+        "kernels": {"fused_head_fwd": {"avg_ms": fwd_ms, "TFLOPs": fwd_tf, "frac": fwd_tf / MFMA_BF16_PEAK_TFLOPS},
+                    "fused_head_bwd": {"avg_ms": bwd_ms, "TFLOPs": bwd_tf, "frac": bwd_tf / MFMA_BF16_PEAK_TFLOPS}},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -120,6 +208,9 @@ def main():
     from trl_amd import ops
 
     w = WORKLOADS[args.workload]
+    if w.get("head"):
+        torch.cuda.set_device(0)
+        return bench_head(args, w)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     B, T, V = w["B"], w["T"], w["V"]
