@@ -30,6 +30,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+# HBM bytes per K3 launch from rocprofv3 FETCH_SIZE / WRITE_SIZE (two --pmc runs of this file, scaled by a plain
+# device copy of known size: FETCH x 2.000, WRITE x 1.000 KiB); the inputs are seeded, so the figure is stable.
+MEASURED_K3_TRAFFIC_BYTES = {("grpo_c3", "dapo"): (10116130 + 19461194) * 1024}
 
 WORKLOADS = {
     # name: (n_seq, completion_len, vocab, temperature, group_size, min_len)
@@ -314,7 +317,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": bwd_gbps / HBM_PEAK_GBPS,
-            "traffic": None,
+            "traffic": MEASURED_K3_TRAFFIC_BYTES.get((args.workload, args.loss_type)),
             "algorithmic_bytes": bwd_bytes,
             "avg_launch_ms": bwd_ms,
         },

@@ -5,8 +5,9 @@
 // row-major and K contiguous, which is the layout the MFMA A/B fragments want (a lane holds 8
 // consecutive k of one row), so fragments come straight out of LDS with 16-byte reads and nothing
 // is ever transposed on the fly.  512 threads = 8 waves as 2 (M) x 4 (N); a wave owns 128 x 64 of
-// the tile = 4 x 2 MFMA blocks = 128 accumulator registers per lane.  Global -> registers -> LDS
-// staging with two LDS buffers (one barrier per 64-wide k step).
+// the tile = 4 x 2 MFMA blocks = 128 accumulator registers per lane.  Two LDS stages, one barrier
+// per 64-wide k step; tiles go from memory straight into LDS (global_load_lds_dwordx4) when K is a
+// multiple of 64, through registers otherwise.
 //
 // Forward (K5): the tile is computed TRANSPOSED -- M = vocabulary rows of W, N = tokens -- so that
 // a lane of the accumulator layout holds 16 vocabulary entries of ONE token per block.  The online
@@ -57,6 +58,8 @@ constexpr int kLoadsA = BM / kRowStep, kLoadsB = BN / kRowStep;
 constexpr int kTileABytes = BM * kLdsRow * 2, kTileBBytes = BN * kLdsRow * 2;
 constexpr int kStageBytes = kTileABytes + kTileBBytes;
 constexpr int kHeadLdsBytes = 2 * kStageBytes;  // two stages
+constexpr int kDzLdsRow = BM * 2 + 16;     // bytes per token row of the dz tile staged in LDS by the backward
+static_assert(BN * kDzLdsRow <= kHeadLdsBytes, "dz staging tile");
 static_assert(2 * WGM * BN * 3 * 4 <= kHeadLdsBytes && BN <= kHeadThreads, "merge scratch");
 static_assert(BM % kRowStep == 0 && BN % kRowStep == 0 && WM % 32 == 0 && WN % 32 == 0 && BK % 16 == 0, "tile shape");
 
@@ -107,10 +110,6 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
     // --- loader side: this lane's row inside a block and the logical chunk it fetches
     const int rr = lane >> 3, pc = lane & 7;
     const int kc = pc ^ rr ^ (wave & 1);  // blocks of a wave all have the parity of the wave index
-#if defined(TRLK_EXP_SAMETILE)
-    m0 = 0;  // experiment: every workgroup reads the same tile (all loads hit L2; results are wrong)
-    n0 = 0;
-#endif
     const char* abase = reinterpret_cast<const char*>(A.p + int64_t(m0) * A.ld);
     const char* bbase = reinterpret_cast<const char*>(B.p + int64_t(n0) * B.ld);
     uint32_t ao[kBlkA], bo[kBlkB];
@@ -136,11 +135,9 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
 #pragma unroll
         for (int j = 0; j < kBlkA; ++j)
             __builtin_amdgcn_global_load_lds((gptr_t)(ap + ao[j]), (lptr_t)(sa + (wave + kWaves * j) * 1024), 16, 0, 0);
-#if !defined(TRLK_EXP_HALFLOADS)
 #pragma unroll
         for (int j = 0; j < kBlkB; ++j)
             __builtin_amdgcn_global_load_lds((gptr_t)(bp + bo[j]), (lptr_t)(sb + (wave + kWaves * j) * 1024), 16, 0, 0);
-#endif
     };
 
     // --- fragment side
@@ -189,15 +186,9 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
     __syncthreads();
     for (int kt = 0; kt < nk; ++kt) {
         // the other buffer was last read before the previous barrier: refill it asynchronously now
-#if defined(TRLK_EXP_NOGLOBAL)
-        compute(0);  // experiment: LDS + MFMA loop alone (results are wrong)
-#else
         if (kt + 1 < nk) issue_stage((kt + 1) & 1, (kt + 1) * BK);
         compute(kt & 1);
-#endif
-#if !defined(TRLK_EXP_NOWAIT)
         __builtin_amdgcn_s_waitcnt(0);  // this wave's transfers have landed in LDS
-#endif
         __syncthreads();                // ... and so have everyone else's; all reads of this buffer are done
     }
 }
@@ -213,10 +204,6 @@ __device__ __forceinline__ void gemm_tile_nt_staged(const Operand A, int m0, con
     const int kc = tid % kCpr, r0 = tid / kCpr;  // this thread stages rows r0 + kRowStep*j, 16-byte chunk kc
 
     // uniform tile base + 32-bit per-lane byte offsets (a tile spans < 4 GiB)
-#if defined(TRLK_EXP_SAMETILE)
-    m0 = 0;  // experiment: every workgroup reads the same tile (all loads hit L2; results are wrong)
-    n0 = 0;
-#endif
     const char* abase = reinterpret_cast<const char*>(A.p + int64_t(m0) * A.ld);
     const char* bbase = reinterpret_cast<const char*>(B.p + int64_t(n0) * B.ld);
     uint32_t ao[kLoadsA], bo[kLoadsB];
@@ -296,21 +283,11 @@ __device__ __forceinline__ void gemm_tile_nt_staged(const Operand A, int m0, con
     store_stage(ra, rb, 0);
     __syncthreads();
     for (int kt = 0; kt < nk; ++kt) {
-#if defined(TRLK_EXP_NOGLOBAL)
-        const bool more = false;  // experiment: measures the LDS + MFMA loop alone (results are wrong)
-#else
         const bool more = kt + 1 < nk;
-#endif
         if (more) load_stage(ra, rb, (kt + 1) * BK);
-#if defined(TRLK_EXP_NOGLOBAL)
-        compute(0);
-#else
         compute(kt & 1);
-#endif
         if (more) store_stage(ra, rb, (kt + 1) & 1);
-#if !defined(TRLK_EXP_NOBARRIER)
         __syncthreads();
-#endif
     }
 }
 
@@ -564,18 +541,26 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
                 const int vrow = vt * BM + acc_row(wm, mb, r, lane);  // chunk-local (padding rows are written as 0)
                 E::store1(a.dzT + int64_t(vrow) * a.ldzt + (n0 + acc_col(wn, nb, lane)), d[r]);
             }
-            // dz [token][chunk column]: 4 consecutive vocabulary entries per register group
-            if (tok_ok) {
+            // dz [token][chunk column] goes through LDS: a lane owns scattered 8-byte pieces of 32
+            // different token rows, which would reach memory as partial sectors; staged as a
+            // [token][vocabulary] tile they leave as 512-byte runs (below)
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int vcol = vt * BM + acc_row(wm, mb, q * 4, lane);
-                    uint2 w;
-                    w.x = E::pack2(d[q * 4 + 0], d[q * 4 + 1]);
-                    w.y = E::pack2(d[q * 4 + 2], d[q * 4 + 3]);
-                    *reinterpret_cast<uint2*>(a.dz + int64_t(tok) * a.ldz + vcol) = w;
-                }
+            for (int q = 0; q < 4; ++q) {
+                uint2 w;
+                w.x = E::pack2(d[q * 4 + 0], d[q * 4 + 1]);
+                w.y = E::pack2(d[q * 4 + 2], d[q * 4 + 3]);
+                *reinterpret_cast<uint2*>(smem + acc_col(wn, nb, lane) * kDzLdsRow + acc_row(wm, mb, q * 4, lane) * 2) = w;
             }
         }
+    }
+    __syncthreads();
+    constexpr int kChunksPerRow = BM / 8;  // 16-byte pieces per token row of the tile
+#pragma unroll 4
+    for (int c = tid; c < BN * kChunksPerRow; c += kHeadThreads) {
+        const int tok_local = c / kChunksPerRow, vc = c % kChunksPerRow;
+        if (n0 + tok_local < a.N)
+            *reinterpret_cast<u32x4*>(a.dz + int64_t(n0 + tok_local) * a.ldz + vt * BM + vc * 8) =
+                *reinterpret_cast<const u32x4*>(smem + tok_local * kDzLdsRow + vc * 16);
     }
 }
 
