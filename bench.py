@@ -125,7 +125,7 @@ def bench_head(args, w):
     mask = (torch.arange(T, device=dev)[None] < lengths[:, None]).long()
     adv = trl_amd.group_advantages(torch.randn((B,), generator=g, device=dev), w["G"])
     with torch.no_grad():
-        base, _, _ = ops.fused_head_fwd(hidden, weight, targets, w["temperature"], 0.0, 1.0)
+        base, _, _, _ = ops.fused_head_fwd(hidden, weight, targets, w["temperature"], 0.0, 1.0)
     base = base.view(B, T)
     old = base + 0.05 * torch.randn(base.shape, generator=g, device=dev)
     ref = base + 0.1 * torch.randn(base.shape, generator=g, device=dev)
@@ -165,7 +165,7 @@ def bench_head(args, w):
         return a.elapsed_time(b) / reps
 
     with torch.no_grad():
-        _, _, log_z = ops.fused_head_fwd(hidden, weight, targets, w["temperature"], 0.0, 1.0)
+        _, _, log_z, _ = ops.fused_head_fwd(hidden, weight, targets, w["temperature"], 0.0, 1.0)
         gl = torch.randn((N,), generator=g, device=dev)
         fwd_ms = time_op(lambda: ops.fused_head_fwd(hidden, weight, targets, w["temperature"], 0.0, 1.0))
         bwd_ms = time_op(lambda: ops.fused_head_bwd(hidden, weight, targets, w["temperature"], 0.0, 1.0, log_z, gl, 8192))

@@ -200,14 +200,17 @@ int trlk_rloo_loss(const float* d_token_logp, const float* d_mask, const float* 
  * strides (elements) that are multiples of 8, 16-byte aligned; dtype TRLK_BF16 or TRLK_F16.
  * Unlike the reference, the logits are not rounded to the operand dtype before the reduction.
  * A target outside [0, vocab) yields NaN and sets TRLK_FLAG_INDEX_OUT_OF_RANGE.
+ * d_out_target_is_max (optional, fp32 [n_tokens]): 1 where the target's logit is the row maximum, i.e.
+ * argmax(logits) == target up to ties -- the token-accuracy count of the chunked cross-entropy
+ * (trl/trainer/sft_trainer.py:99-114) comes out of the same pass.
  */
 size_t trlk_fused_head_fwd_workspace_bytes(int64_t n_tokens);
 
 int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, const int64_t* d_targets, int dtype,
                         int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                         int64_t weight_stride, float temperature, float final_logit_softcapping, float logit_scale,
-                        float* d_out_logp, float* d_out_entropy, float* d_out_log_z, int32_t* d_error_flag,
-                        void* d_workspace, size_t workspace_bytes, trlk_stream_t stream);
+                        float* d_out_logp, float* d_out_entropy, float* d_out_log_z, float* d_out_target_is_max,
+                        int32_t* d_error_flag, void* d_workspace, size_t workspace_bytes, trlk_stream_t stream);
 
 /* Backward of the above w.r.t. hidden and weight for an upstream gradient on the log-probs
  * (the entropy output carries no gradient, as in the reference, utils.py:1368):

@@ -24,6 +24,8 @@ Pinning status (what checks each function against something other than itself):
   rloo_loss                 : golden vectors from `RLOOTrainer._compute_loss` (mocked)
   chunked_logprob           : naive `(h @ W.T).float()/T -> log_softmax` routine and
                               autograd of it (reference test tests/test_utils.py:1161-1232)
+  chunked_cross_entropy_loss: golden vectors from the reference's `_chunked_cross_entropy_loss`,
+                              `F.cross_entropy` library routine
   get_off_policy_mask       : reference unit-test vectors (tests/test_grpo_trainer.py:1456-1520)
   get_high_entropy_mask     : reference unit-test vectors (tests/test_grpo_trainer.py:110-160)
 """
@@ -56,6 +58,7 @@ __all__ = [
     "chunked_logprob_backward",
     "ChunkedLogProbOracle",
     "patch_chunked_rows",
+    "chunked_cross_entropy_loss",
 ]
 
 
@@ -577,3 +580,41 @@ def patch_chunked_rows(hidden_states, labels, completion_mask, weight, temperatu
     lp[keep] = lp_v
     ent[keep] = ent_v
     return lp.reshape(b, s), ent.reshape(b, s)
+
+
+# --------------------------------------------------------------------------------------
+# SFT chunked cross-entropy              trl/trainer/sft_trainer.py:99-234
+# --------------------------------------------------------------------------------------
+def chunked_cross_entropy_loss(hidden_states, lm_head_weight, chunk_size, labels=None, shift_labels=None,
+                               num_items_in_batch=None, logit_scale=1.0, final_logit_softcapping=None):
+    """Shift (or take pre-shifted labels) (sft_trainer.py:175-180), drop `-100` rows, and over token
+    chunks of `chunk_size` accumulate fp32 NLL sum, argmax hits and entropy sum (`_chunk`, :99-114);
+    loss = sum / num_items_in_batch, or / n_valid (:228-233).  Returns (loss, correct, entropy_sum, n_valid)."""
+    if shift_labels is not None:
+        hidden = hidden_states.reshape(-1, hidden_states.size(-1))
+        lab = shift_labels.reshape(-1)
+    else:
+        hidden = hidden_states[..., :-1, :].reshape(-1, hidden_states.size(-1))
+        lab = labels[..., 1:].reshape(-1)
+    keep = lab != -100
+    n_valid = keep.sum()
+    if int(n_valid) == 0:
+        zero = torch.zeros((), dtype=torch.float32)
+        return (hidden_states.float().sum() + lm_head_weight.float().sum()) * 0.0, zero, zero.clone(), n_valid
+    hidden, lab = hidden[keep], lab[keep]
+    loss = torch.zeros((), dtype=torch.float32)
+    correct = torch.zeros((), dtype=torch.float32)
+    entropy_sum = torch.zeros((), dtype=torch.float32)
+    for lo in range(0, hidden.shape[0], chunk_size):
+        z = hidden[lo : lo + chunk_size].float() @ lm_head_weight.float().t()
+        if logit_scale != 1.0:
+            z = z * logit_scale
+        if final_logit_softcapping is not None:
+            z = final_logit_softcapping * torch.tanh(z / final_logit_softcapping)
+        lp = F.log_softmax(z, dim=-1)
+        tgt = lab[lo : lo + chunk_size]
+        loss = loss + F.nll_loss(lp, tgt, reduction="sum")
+        correct = correct + (z.argmax(-1) == tgt).sum().float()
+        entropy_sum = entropy_sum + (-(lp.exp() * lp).sum(-1)).sum()
+    denom = n_valid if num_items_in_batch is None else num_items_in_batch
+    return loss / denom, correct, entropy_sum, n_valid

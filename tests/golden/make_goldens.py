@@ -379,6 +379,41 @@ def make_head(ChunkedFn, out_dir):
         json.dump(index, f, indent=1)
 
 
+# ------------------------------------------------------------------------------------ SFT chunked NLL
+SFT_CASES = [
+    dict(name="labels_mean", dtype="float32", chunk=16, shift=False, nitems=None, softcap=None, scale=1.0),
+    dict(name="shift_labels_nitems", dtype="float32", chunk=7, shift=True, nitems=50.0, softcap=None, scale=1.0),
+    dict(name="softcap_scale", dtype="float32", chunk=32, shift=False, nitems=None, softcap=4.0, scale=0.5),
+    dict(name="bf16", dtype="bfloat16", chunk=16, shift=False, nitems=None, softcap=None, scale=1.0),
+]
+
+
+def make_sft(chunked_ce, out_dir):
+    index, arrays = [], {}
+    for ci, case in enumerate(SFT_CASES):
+        g = torch.Generator().manual_seed(5000 + ci)
+        B, S, H, V = 3, 12, 32, 96
+        dtype = getattr(torch, case["dtype"])
+        hs = torch.randn(B, S, H, generator=g).to(dtype).requires_grad_(True)
+        w = (torch.randn(V, H, generator=g) * 0.4).to(dtype).requires_grad_(True)
+        labels = torch.randint(0, V, (B, S), generator=g)
+        labels[0, :4] = -100
+        labels[1, 7:] = -100
+        labels[2, 5] = -100
+        kw = dict(shift_labels=labels) if case["shift"] else dict(labels=labels)
+        loss, correct, ent, nv = chunked_ce(hs, w, case["chunk"], num_items_in_batch=case["nitems"],
+                                            logit_scale=case["scale"], final_logit_softcapping=case["softcap"], **kw)
+        loss.backward()
+        pre = f"c{ci}_"
+        for k, v in dict(hidden=hs, weight=w, labels=labels, out_loss=loss, out_correct=correct, out_entropy_sum=ent,
+                         out_n_valid=nv, out_dhidden=hs.grad, out_dweight=w.grad).items():
+            arrays[pre + k] = _np(v)
+        index.append(dict(case, id=ci, shape=[B, S, H, V]))
+    np.savez_compressed(os.path.join(out_dir, "sft_chunked_nll.npz"), **arrays)
+    with open(os.path.join(out_dir, "sft_chunked_nll.json"), "w") as f:
+        json.dump(index, f, indent=1)
+
+
 # ------------------------------------------------------------------------------------ utils
 def make_utils(utils, out_dir):
     """selective_log_softmax / entropy_from_logits on bf16 and fp32 rows, incl. strided views and K > 1."""
@@ -411,6 +446,9 @@ def main():
     from trl.trainer.grpo_trainer import GRPOTrainer
     from trl.trainer.rloo_trainer import RLOOTrainer
 
+    from trl.trainer.sft_trainer import _chunked_cross_entropy_loss
+
+    make_sft(_chunked_cross_entropy_loss, args.out)
     make_utils(ref_utils, args.out)
     make_head(ref_utils._ChunkedLogProbFunction, args.out)
     make_grpo(GRPOTrainer, args.out)

@@ -161,3 +161,38 @@ def test_real_head_shape_row_subsample(amd):
     torch.testing.assert_close(ent, rent, atol=2e-3, rtol=0)
     assert _rel_l2(dh.float(), rdh) < 1e-2
     assert _rel_l2(dw.float(), rdw) < 1e-2
+
+
+def test_golden_sft_chunked_nll(amd):
+    """The reference's `_chunked_cross_entropy_loss` wrote these; fp32 cases are run in bf16 on the device
+    (the matrix-core kernels take bf16/fp16) and compared with the oracle on the bf16-rounded operands."""
+    from trl_amd.trainer.sft_trainer import _chunked_cross_entropy_loss
+
+    cases, g = load_golden("sft_chunked_nll")
+    for case in cases:
+        c = f"c{case['id']}_"
+        hs = _t(g[c + "hidden"]).bfloat16()
+        w = _t(g[c + "weight"]).bfloat16()
+        labels = _t(g[c + "labels"])
+        kw = dict(shift_labels=labels) if case["shift"] else dict(labels=labels)
+        common = dict(num_items_in_batch=case["nitems"], logit_scale=case["scale"], final_logit_softcapping=case["softcap"])
+        ohs, ow = hs.float().requires_grad_(True), w.float().requires_grad_(True)
+        oloss, ocorrect, oent, onv = oracle.chunked_cross_entropy_loss(ohs, ow, case["chunk"], **common, **kw)
+        oloss.backward()
+        dhs, dw = hs.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+        dkw = {k: v.to(DEV) for k, v in kw.items()}
+        loss, correct, ent, nv = _chunked_cross_entropy_loss(dhs, dw, 256, **common, **dkw)
+        loss.backward()
+        assert int(nv) == int(onv) == int(g[c + "out_n_valid"])
+        assert abs(float(loss) - float(oloss)) <= 1e-3 * abs(float(oloss))
+        assert abs(float(correct) - float(ocorrect)) <= 1.0  # a near-tie between the two largest logits may flip
+        assert abs(float(ent) - float(oent)) <= 2e-3 * int(nv)
+        assert _rel_l2(dhs.grad.float(), ohs.grad) < 1e-2 and _rel_l2(dw.grad.float(), ow.grad) < 1e-2
+        if case["dtype"] == "float32":  # and loosely against the reference's own fp32 numbers (bf16 operand rounding)
+            assert abs(float(loss) - float(g[c + "out_loss"])) <= 2e-2 * abs(float(g[c + "out_loss"]))
+    # all positions masked: zero loss that still backpropagates
+    dhs = torch.randn(2, 5, 32, device=DEV).bfloat16().requires_grad_(True)
+    dw = torch.randn(64, 32, device=DEV).bfloat16().requires_grad_(True)
+    loss, correct, ent, nv = _chunked_cross_entropy_loss(dhs, dw, 256, labels=torch.full((2, 5), -100, device=DEV))
+    loss.backward()
+    assert float(loss) == 0.0 and int(nv) == 0 and torch.count_nonzero(dw.grad) == 0

@@ -345,3 +345,38 @@ def test_patch_chunked_rows_masking():
     torch.testing.assert_close(lp_m[keep], lp_u[keep])
     torch.testing.assert_close(ent_m[keep], ent_u[keep])
     assert torch.equal(lp_m[~keep], torch.zeros_like(lp_m[~keep])) and torch.equal(ent_m[~keep], torch.zeros_like(ent_m[~keep]))
+
+
+# ----------------------------------------------------------------------------- SFT chunked NLL
+def test_golden_sft_chunked_nll():
+    cases, g = load_golden("sft_chunked_nll")
+    for case in cases:
+        c = f"c{case['id']}_"
+        dtype = getattr(torch, case["dtype"])
+        hs = _t(g[c + "hidden"], dtype).requires_grad_(True)
+        w = _t(g[c + "weight"], dtype).requires_grad_(True)
+        labels = _t(g[c + "labels"])
+        kw = dict(shift_labels=labels) if case["shift"] else dict(labels=labels)
+        loss, correct, ent, nv = oracle.chunked_cross_entropy_loss(
+            hs, w, case["chunk"], num_items_in_batch=case["nitems"], logit_scale=case["scale"],
+            final_logit_softcapping=case["softcap"], **kw)
+        loss.backward()
+        tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+        torch.testing.assert_close(loss.detach().float(), _t(g[c + "out_loss"]).float(), **tol)
+        assert float(correct) == float(g[c + "out_correct"]) and int(nv) == int(g[c + "out_n_valid"])
+        torch.testing.assert_close(ent.detach(), _t(g[c + "out_entropy_sum"]), rtol=1e-5, atol=1e-4)
+        torch.testing.assert_close(hs.grad.float(), _t(g[c + "out_dhidden"]), **tol)
+        torch.testing.assert_close(w.grad.float(), _t(g[c + "out_dweight"]), **tol)
+    # library routine: mean cross-entropy over the valid positions
+    torch.manual_seed(9)
+    hs, w = torch.randn(2, 7, 16), torch.randn(40, 16)
+    labels = torch.randint(0, 40, (2, 7))
+    labels[0, 2] = -100
+    loss, _, _, nv = oracle.chunked_cross_entropy_loss(hs, w, 4, labels=labels)
+    want = F.cross_entropy((hs[:, :-1] @ w.t()).reshape(-1, 40), labels[:, 1:].reshape(-1), ignore_index=-100)
+    torch.testing.assert_close(loss, want)
+    # an all-masked batch still yields a differentiable zero
+    hs.requires_grad_(True)
+    loss, correct, ent, nv = oracle.chunked_cross_entropy_loss(hs, w, 4, labels=torch.full((2, 7), -100))
+    loss.backward()
+    assert float(loss) == 0.0 and int(nv) == 0 and torch.count_nonzero(hs.grad) == 0

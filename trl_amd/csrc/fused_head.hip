@@ -60,7 +60,7 @@ constexpr int kStageBytes = kTileABytes + kTileBBytes;
 constexpr int kHeadLdsBytes = 2 * kStageBytes;  // two stages
 constexpr int kDzLdsRow = BM * 2 + 16;     // bytes per token row of the dz tile staged in LDS by the backward
 static_assert(BN * kDzLdsRow <= kHeadLdsBytes, "dz staging tile");
-static_assert(2 * WGM * BN * 3 * 4 <= kHeadLdsBytes && BN <= kHeadThreads, "merge scratch");
+static_assert(2 * WGM * BN * 4 * 4 <= kHeadLdsBytes && BN <= kHeadThreads, "merge scratch");
 static_assert(BM % kRowStep == 0 && BN % kRowStep == 0 && WM % 32 == 0 && WN % 32 == 0 && BK % 16 == 0, "tile shape");
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -332,7 +332,7 @@ struct HeadArgs {
     float logit_scale, inv_t, softcap;  // softcap <= 0: none
     // forward
     int v_splits, tiles_per_split;
-    float* partial;  // [N, v_splits, 4]: (reference exponent, S, U, unused)
+    float* partial;  // [N, v_splits, 4]: (reference exponent, S, U, exact max of z)
     float* tgt;      // [N] logit of the target token (NaN until found)
     // backward (dz pass)
     const float* log_z;  // [N]
@@ -365,11 +365,12 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
     const int vt1 = vt0 + a.tiles_per_split < n_vt ? vt0 + a.tiles_per_split : n_vt;
 
     // per-lane online state of the NB tokens this lane owns (base-2, integer reference exponent)
-    float ref[NB], rr[NB], S[NB], U[NB];
+    float ref[NB], rr[NB], S[NB], U[NB], zmax[NB];
     int64_t tg[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         ref[nb] = -INFINITY;
+        zmax[nb] = -INFINITY;
         rr[nb] = 0.f;
         S[nb] = 0.f;
         U[nb] = 0.f;
@@ -395,6 +396,7 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
                     acc[mb][nb][r] = z;
                     bm = fmaxf(bm, z);
                 }
+            zmax[nb] = fmaxf(zmax[nb], bm);
             const float need = ceilf(bm * kLog2e);
             if (need > ref[nb]) {
                 const float sc = fast_exp2(ref[nb] - need);
@@ -429,23 +431,28 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
 
     // merge the partial states of every token (2 lane halves x WGM M-waves) through LDS
     constexpr int kParts = 2 * WGM;
-    float* sm = reinterpret_cast<float*>(smem);  // [kParts][BN tokens][3]
+    float* sm = reinterpret_cast<float*>(smem);  // [kParts][BN tokens][4]
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         const int col = acc_col(wn, nb, lane);
         const int part = wm * 2 + (lane >> 5);
-        float* dst = sm + (part * BN + col) * 3;
+        float* dst = sm + (part * BN + col) * 4;
         dst[0] = ref[nb];
         dst[1] = S[nb];
         dst[2] = U[nb];
+        dst[3] = zmax[nb];
     }
     __syncthreads();
     if (tid < BN && n0 + tid < a.N) {
         float R = -INFINITY;
-        for (int p = 0; p < kParts; ++p) R = fmaxf(R, sm[(p * BN + tid) * 3]);
+        float zm = -INFINITY;
+        for (int p = 0; p < kParts; ++p) {
+            R = fmaxf(R, sm[(p * BN + tid) * 4]);
+            zm = fmaxf(zm, sm[(p * BN + tid) * 4 + 3]);
+        }
         float s = 0.f, u = 0.f;
         for (int p = 0; p < kParts; ++p) {
-            const float* src = sm + (p * BN + tid) * 3;
+            const float* src = sm + (p * BN + tid) * 4;
             const float sc = (src[0] == -INFINITY) ? 0.f : fast_exp2(src[0] - R);
             s += src[1] * sc;
             u += src[2] * sc;
@@ -454,7 +461,7 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
         out[0] = R;
         out[1] = s;
         out[2] = u;
-        out[3] = 0.f;
+        out[3] = zm;
     }
 }
 
@@ -465,14 +472,16 @@ __global__ void head_fill_kernel(float* p, int64_t n, float v) {
 
 // merges the vocabulary splits of every token: logp, entropy, log_z
 __global__ void head_merge_kernel(const float* partial, const float* tgt, const int64_t* targets, int N, int V,
-                                  int v_splits, float* logp, float* entropy, float* log_z, int32_t* error_flag) {
+                                  int v_splits, float* logp, float* entropy, float* log_z, float* target_is_max,
+                                  int32_t* error_flag) {
     const int n = blockIdx.x * blockDim.x + threadIdx.x;
     if (n >= N) return;
     const float* p = partial + int64_t(n) * v_splits * 4;
     float R = -INFINITY;
     for (int s = 0; s < v_splits; ++s) R = fmaxf(R, p[s * 4]);
-    float S = 0.f, U = 0.f;
+    float S = 0.f, U = 0.f, zm = -INFINITY;
     for (int s = 0; s < v_splits; ++s) {
+        zm = fmaxf(zm, p[s * 4 + 3]);
         const float sc = (p[s * 4] == -INFINITY) ? 0.f : fast_exp2(p[s * 4] - R);
         S += p[s * 4 + 1] * sc;
         U += p[s * 4 + 2] * sc;
@@ -490,6 +499,8 @@ __global__ void head_merge_kernel(const float* partial, const float* tgt, const 
     logp[n] = lp;
     entropy[n] = lz - U / S;
     log_z[n] = lz;
+    // 1 if the target holds the row maximum, i.e. argmax(logits) == target up to ties
+    if (target_is_max) target_is_max[n] = (t >= 0 && t < V && tgt[n] >= zm) ? 1.f : 0.f;
 }
 
 // dz pass of the backward: one 256 (vocabulary) x 256 (tokens) tile per workgroup.
@@ -715,8 +726,8 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
                                    int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                                    int64_t weight_stride, float temperature, float final_logit_softcapping,
                                    float logit_scale, float* d_out_logp, float* d_out_entropy, float* d_out_log_z,
-                                   int32_t* d_error_flag, void* d_workspace, size_t workspace_bytes,
-                                   trlk_stream_t stream) {
+                                   float* d_out_target_is_max, int32_t* d_error_flag, void* d_workspace,
+                                   size_t workspace_bytes, trlk_stream_t stream) {
     clear_error();
     if (int rc = check_head("fused_head_fwd", d_hidden, d_weight, d_targets, dtype, n_tokens, vocab, hidden_size,
                             hidden_stride, weight_stride, temperature))
@@ -753,7 +764,7 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
     if (rc) return rc;
     hipLaunchKernelGGL(head_merge_kernel, dim3(unsigned((n_tokens + 255) / 256)), dim3(256), 0, s, a.partial, a.tgt,
                        d_targets, int(n_tokens), int(vocab), kFwdSplits, d_out_logp, d_out_entropy, d_out_log_z,
-                       d_error_flag);
+                       d_out_target_is_max, d_error_flag);
     return launch_status("fused_head_fwd (merge)");
 }
 

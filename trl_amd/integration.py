@@ -4,6 +4,7 @@ TRL has no plugin registry: its hot-path helpers are module-level functions impo
 every trainer module, and the loss is a trainer method.  `patch_trl()` therefore rebinds
   * `selective_log_softmax`, `entropy_from_logits`, `_ChunkedLogProbFunction`, `patch_chunked_lm_head`
     in `trl.trainer.utils` **and** in every already-imported `trl.*` module that holds its own reference;
+  * `trl.trainer.sft_trainer._chunked_cross_entropy_loss` (the default SFT loss);
   * `GRPOTrainer._get_per_token_logps_and_entropies` / `_compute_loss` (optional, `grpo=True`).
 `unpatch_trl()` restores the originals.
 """
@@ -34,6 +35,17 @@ def patch_trl(grpo: bool = True) -> int:
                 _saved.append((mod, name, orig))
                 setattr(mod, name, getattr(_utils, name))
                 count += 1
+    try:  # SFT's default `chunked_nll` loss (trl/trainer/sft_trainer.py:117-234)
+        import trl.trainer.sft_trainer as ref_sft
+
+        from .trainer.sft_trainer import _chunked_cross_entropy_loss
+
+        if hasattr(ref_sft, "_chunked_cross_entropy_loss"):
+            _saved.append((ref_sft, "_chunked_cross_entropy_loss", ref_sft._chunked_cross_entropy_loss))
+            ref_sft._chunked_cross_entropy_loss = _chunked_cross_entropy_loss
+            count += 1
+    except ImportError:
+        pass
     if grpo:
         from trl.trainer.grpo_trainer import GRPOTrainer
 

@@ -403,9 +403,9 @@ def _head_operands(hidden: Tensor, weight: Tensor, targets: Tensor):
 
 @torch.library.custom_op("trl_amd::fused_head_fwd", mutates_args=(), device_types="cuda")
 def fused_head_fwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature: float, softcap: float,
-                   logit_scale: float) -> tuple[Tensor, Tensor, Tensor]:
-    """hidden [N, H], weight [V, H] (bf16/fp16), targets int64 [N] -> fp32 (logp, entropy, log_z), each [N].
-    `softcap <= 0` means no soft-capping."""
+                   logit_scale: float) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    """hidden [N, H], weight [V, H] (bf16/fp16), targets int64 [N] -> fp32 (logp, entropy, log_z, target_is_max),
+    each [N]; target_is_max is 1 where argmax(logits) == target.  `softcap <= 0` means no soft-capping."""
     hidden, weight, targets = _head_operands(hidden, weight, targets)
     n, h = hidden.shape
     v = weight.shape[0]
@@ -413,24 +413,25 @@ def fused_head_fwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
     logp = torch.empty((n,), dtype=torch.float32, device=dev)
     ent = torch.empty((n,), dtype=torch.float32, device=dev)
     log_z = torch.empty((n,), dtype=torch.float32, device=dev)
+    hit = torch.empty((n,), dtype=torch.float32, device=dev)
     if n == 0:
-        return logp, ent, log_z
+        return logp, ent, log_z, hit
     ws_bytes = lib.trlk_fused_head_fwd_workspace_bytes(n)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         check(lib.trlk_fused_head_fwd(ptr(hidden), ptr(weight), ptr(targets), dtype_code(hidden.dtype), n, v, h,
                                       hidden.stride(0), weight.stride(0), temperature, softcap, logit_scale, ptr(logp),
-                                      ptr(ent), ptr(log_z), ptr(_error_flag(dev)), ptr(ws), ws_bytes,
+                                      ptr(ent), ptr(log_z), ptr(hit), ptr(_error_flag(dev)), ptr(ws), ws_bytes,
                                       current_stream(dev)))
     if _SYNC_CHECKS:
         check_device_errors()
-    return logp, ent, log_z
+    return logp, ent, log_z, hit
 
 
 @fused_head_fwd.register_fake
 def _(hidden, weight, targets, temperature, softcap, logit_scale):
     f = lambda: torch.empty((hidden.shape[0],), dtype=torch.float32, device=hidden.device)  # noqa: E731
-    return f(), f(), f()
+    return f(), f(), f(), f()
 
 
 @torch.library.custom_op("trl_amd::fused_head_bwd", mutates_args=(), device_types="cuda")

@@ -4,3 +4,4 @@ from .grpo_trainer import (GRPOLossMixin, get_high_entropy_mask, get_off_policy_
 from .rloo_trainer import rloo_advantages, rloo_loss
 from .utils import (_ChunkedLogProbFunction, chunked_logprobs_from_hidden, entropy_from_logits, logps_and_entropies,
                     nanmax, nanmin, nanstd, patch_chunked_lm_head, selective_log_softmax)
+from .sft_trainer import _chunked_cross_entropy_loss

@@ -153,7 +153,8 @@ class _ChunkedLogProbFunction(torch.autograd.Function):
     def forward(ctx, last_hidden, weight, targets, temperature, chunk_size, final_logit_softcapping=None,
                 logit_scale=1.0):
         cap = 0.0 if final_logit_softcapping is None else float(final_logit_softcapping)
-        logp, ent, log_z = ops.fused_head_fwd(last_hidden, weight, targets, float(temperature), cap, float(logit_scale))
+        logp, ent, log_z, _ = ops.fused_head_fwd(last_hidden, weight, targets, float(temperature), cap,
+                                                 float(logit_scale))
         ctx.save_for_backward(last_hidden, weight, targets, log_z)
         ctx.cfg = (float(temperature), int(chunk_size), cap, float(logit_scale))
         ctx.mark_non_differentiable(ent)
