@@ -266,8 +266,8 @@ def main():
     g_logp = (leaf.grad is not None) and None
     loss2, _, dlogp, _ = ops.grpo_loss_op(
         lp_flat.view(B, T), old, ref, ent_flat.view(B, T), adv, mask, None, None, n_items,
-        ops.LOSS_TYPES[args.loss_type], w["eps_low"], w["eps_high"], float("nan"), w["beta"], False, 1.0,
-        float(B * T), 1.0, 0.0)
+        ops.LOSS_TYPES[args.loss_type][0], w["eps_low"], w["eps_high"], float("nan"), w["beta"], False, 1.0,
+        float(B * T), 1.0, 0.0, ops.LOSS_TYPES[args.loss_type][1])
     g_logp = dlogp.reshape(R, 1).contiguous()
     leaf.grad = None
     reps = max(3, min(args.steps, 10))

@@ -46,7 +46,14 @@ enum trlk_status {
 };
 
 /* loss normalisations of GRPOTrainer._compute_loss (trl/trainer/grpo_trainer.py:3124-3142) */
-enum trlk_grpo_loss_type { TRLK_GRPO = 0, TRLK_BNPO = 1, TRLK_DR_GRPO = 2, TRLK_DAPO = 3 };
+enum trlk_grpo_loss_type { TRLK_GRPO = 0, TRLK_BNPO = 1, TRLK_DR_GRPO = 2, TRLK_DAPO = 3, TRLK_LUSPO = 4 };
+
+/* per-token policy term of the GRPO family (trl/trainer/grpo_trainer.py:3080-3107); c = importance ratio, A = advantage
+ *   CLIP:          -min(min(c, delta) * A, clamp(c, 1-eps_low, 1+eps_high) * A)     grpo, bnpo, dr_grpo, dapo, luspo
+ *   CISPO:         -min(c, eps_high).detach() * A * logp                            cispo
+ *   SAPO:          -sigmoid(tau * (c - 1)) * 4 / tau * A, tau = A > 0 ? pos : neg    sapo
+ *   WEIGHTED_LOGP: -coef[b] * A * logp with a given, detached per-sequence coef      vespo (coef = gamma weights) */
+enum trlk_grpo_policy_term { TRLK_TERM_CLIP = 0, TRLK_TERM_CISPO = 1, TRLK_TERM_SAPO = 2, TRLK_TERM_WEIGHTED_LOGP = 3 };
 
 /* scale_rewards modes (trl/trainer/grpo_trainer.py:2687-2707) */
 enum trlk_scale_rewards { TRLK_SCALE_GROUP = 0, TRLK_SCALE_BATCH = 1, TRLK_SCALE_NONE = 2 };
@@ -109,8 +116,10 @@ int trlk_group_advantages(const float* d_rewards, int64_t n, int32_t group_size,
 
 /* ---------------------------------------------------------------------------------------
  * K2  GRPO clipped-surrogate loss, its metrics and d(loss)/d(logp) in one call
- * (trl/trainer/grpo_trainer.py:3054-3150 token-level importance weights, :3155-3181 entropy
- * bonus, :3224-3253 metrics).  All [B, T] operands are dense fp32.
+ * (trl/trainer/grpo_trainer.py:3054-3150, :3155-3181 entropy bonus, :3224-3258 metrics).
+ * All [B, T] operands are dense fp32.  `loss_type` picks the normalisation (cispo and vespo use
+ * TRLK_DAPO, sapo uses TRLK_GRPO), `policy_term` the per-token term, `sequence_level` != 0 the
+ * sequence-level importance weight exp(masked mean of logp - old_logp) (:3057-3059).
  *   d_old_logp  NULL  -> old = logp (on-policy, :3037)
  *   d_ref_logp  NULL  -> requires beta == 0
  *   d_entropy   NULL  -> no entropy metric / bonus
@@ -118,6 +127,7 @@ int trlk_group_advantages(const float* d_rewards, int64_t n, int32_t group_size,
  *                  (product of the off-policy, entropy-quantile and importance-sampling
  *                  factors of :3111-3118)
  *   d_entropy_mask NULL -> 1; extra factor on the mask of the entropy bonus (:3158)
+ *   d_seq_coef  fp32 [B], only for TRLK_TERM_WEIGHTED_LOGP
  *   advantages: element (b, t) at d_advantages[b*adv_stride_b + t*adv_stride_t]
  *   delta: NaN = no upper clamp of the ratio (:3086-3087)
  *   d_dapo_normalizer: device scalar holding num_items_in_batch (DAPO only, :3140)
@@ -139,6 +149,10 @@ enum trlk_grpo_metric {
     TRLK_M_MASK_SUM = 8,
     TRLK_M_KL_SUM = 9,
     TRLK_M_ENTROPY_SUM = 10,
+    TRLK_M_AUX_MEAN = 11,        /* cispo: clip ratio (:3255-3256); weighted-logp: mean coefficient (:3258) */
+    TRLK_M_CLIP_COUNT = 12,      /* denominator of the clip means: mask sum, or B with sequence-level weights */
+    TRLK_M_AUX_SUM = 13,
+    TRLK_M_AUX_COUNT = 14,
     TRLK_GRPO_NUM_METRICS = 16
 };
 
@@ -146,12 +160,13 @@ size_t trlk_grpo_workspace_bytes(int64_t n_seq);
 
 int trlk_grpo_loss(const float* d_logp, const float* d_old_logp, const float* d_ref_logp, const float* d_entropy,
                    const float* d_advantages, int64_t adv_stride_b, int64_t adv_stride_t, const float* d_mask,
-                   const float* d_token_weight, const float* d_entropy_mask, int64_t n_seq, int64_t seq_len,
-                   int32_t loss_type, float epsilon_low, float epsilon_high, float delta, float beta,
-                   int32_t use_bias_correction_kl, float grad_accum_steps, float dr_grpo_denominator,
-                   const float* d_dapo_normalizer, float num_processes, float entropy_coef, float* d_out_loss,
-                   float* d_out_metrics, float* d_out_dlogp, float* d_out_dentropy, void* d_workspace,
-                   size_t workspace_bytes, trlk_stream_t stream);
+                   const float* d_token_weight, const float* d_entropy_mask, const float* d_seq_coef, int64_t n_seq,
+                   int64_t seq_len, int32_t loss_type, int32_t policy_term, int32_t sequence_level, float epsilon_low,
+                   float epsilon_high, float delta, float beta, int32_t use_bias_correction_kl, float grad_accum_steps,
+                   float dr_grpo_denominator, const float* d_dapo_normalizer, float num_processes, float entropy_coef,
+                   float sapo_temperature_pos, float sapo_temperature_neg, float* d_out_loss, float* d_out_metrics,
+                   float* d_out_dlogp, float* d_out_dentropy, void* d_workspace, size_t workspace_bytes,
+                   trlk_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------
  * K4  sequence-level losses on top of per-token log-probs.

@@ -48,6 +48,7 @@ __all__ = [
     "rloo_advantages",
     "get_off_policy_mask",
     "get_high_entropy_mask",
+    "get_gamma_weights",
     "logps_and_entropies_from_logits",
     "grpo_loss",
     "dpo_sequence_logps",
@@ -227,6 +228,23 @@ def get_high_entropy_mask(entropies, mask, threshold):
     return ((entropies * mask.float()) >= cut) & mask.bool()
 
 
+@torch.no_grad()
+def get_gamma_weights(advantages, log_ratio_per_token, mask, importance_sampling_ratio=None, k_pos=2.0, lambda_pos=3.0,
+                      k_neg=3.0, lambda_neg=2.0):
+    """VESPO sequence weights phi(w) = e^lambda * w^k * e^(-lambda w) in log space, w = exp(sum of the clamped
+    per-token log-ratios) (grpo_trainer.py:2941-2989); (B, 1), no gradient."""
+    floor = math.log(1e-8)
+    seq = (log_ratio_per_token.clamp(-20.0, 20.0) * mask).sum(-1, keepdim=True)
+    if importance_sampling_ratio is not None:
+        seq = seq + importance_sampling_ratio.log().clamp(floor, 20.0).sum(-1, keepdim=True)
+    log_w = seq.clamp(floor, 20.0)
+    w = log_w.exp()
+    pos = advantages >= 0
+    k = torch.where(pos, k_pos, k_neg)
+    lam = torch.where(pos, lambda_pos, lambda_neg).clamp(min=1e-4)
+    return (lam + k * log_w - lam * w).exp().nan_to_num(nan=0.0, posinf=0.0, neginf=0.0)
+
+
 # --------------------------------------------------------------------------------------
 # A3 + A4  logits -> per-token logps / entropies   trl/trainer/grpo_trainer.py:1511-1533
 # --------------------------------------------------------------------------------------
@@ -284,11 +302,14 @@ def grpo_loss(
     top_entropy_quantile: float = 1.0,
     importance_sampling_ratio: torch.Tensor | None = None,
     entropy_coef: float = 0.0,
+    sapo_temperature_pos: float = 1.0,
+    sapo_temperature_neg: float = 1.05,
+    vespo_params: tuple[float, float, float, float] = (2.0, 3.0, 3.0, 2.0),
 ):
     """Clipped-surrogate GRPO family loss on `[B, T]` log-probs.  Returns
     `(loss, metrics)` where `metrics` holds python floats named as the reference logs
-    them (grpo_trainer.py:3237-3253).  Covers loss types grpo / bnpo / dr_grpo / dapo
-    (grpo_trainer.py:3083-3091, 3124-3142), token- and sequence-level importance
+    them (grpo_trainer.py:3237-3258).  Covers loss types grpo / bnpo / dr_grpo / dapo / luspo / cispo /
+    sapo / vespo (grpo_trainer.py:3080-3107, 3124-3148), token- and sequence-level importance
     weights (:3054-3059), k3 KL (:3069-3076), delta clamp (:3086-3087), off-policy and
     entropy-quantile masks (:3039-3052, 3020-3021, 3111-3115), a given importance
     sampling ratio (:3117-3118) and the static entropy bonus (:3155-3181)."""
@@ -323,12 +344,22 @@ def grpo_loss(
         if use_bias_correction_kl:
             per_token_kl = per_token_kl * coef_1
 
-    if loss_type not in ("grpo", "bnpo", "dr_grpo", "dapo"):
-        raise ValueError(f"loss type not restated in the oracle: {loss_type}")
-    coef_2 = coef_1.clamp(1 - epsilon_low, 1 + epsilon_high)
-    if delta is not None:
-        coef_1 = coef_1.clamp(max=delta)
-    per_token_loss = -torch.min(coef_1 * adv, coef_2 * adv)
+    phi_seq = None
+    if loss_type == "cispo":  # (:3080-3082)
+        per_token_loss = -coef_1.clamp(max=epsilon_high).detach() * adv * per_token_logps
+    elif loss_type in ("grpo", "bnpo", "dr_grpo", "dapo", "luspo"):  # (:3083-3091)
+        coef_2 = coef_1.clamp(1 - epsilon_low, 1 + epsilon_high)
+        if delta is not None:
+            coef_1 = coef_1.clamp(max=delta)
+        per_token_loss = -torch.min(coef_1 * adv, coef_2 * adv)
+    elif loss_type == "sapo":  # (:3092-3095)
+        temps = torch.where(adv > 0, sapo_temperature_pos, sapo_temperature_neg)
+        per_token_loss = -(torch.sigmoid(temps * (coef_1 - 1)) * 4 / temps) * adv
+    elif loss_type == "vespo":  # (:3096-3107)
+        phi_seq = get_gamma_weights(adv, log_ratio, mask, None, *vespo_params)
+        per_token_loss = -phi_seq * adv * per_token_logps
+    else:
+        raise ValueError(f"Unknown loss type: {loss_type}")
 
     if off_mask is not None:
         per_token_loss = per_token_loss * off_mask
@@ -340,8 +371,13 @@ def grpo_loss(
         per_token_loss = per_token_loss + beta * per_token_kl
 
     # policy_loss is taken before the division by the gradient-accumulation steps (:3127, 3132, 3137, 3142)
-    if loss_type == "grpo":
+    if loss_type in ("grpo", "sapo"):
         loss = ((per_token_loss * mask).sum(-1) / mask.sum(-1).clamp(min=1.0)).mean()
+        normalizer = grad_accum_steps
+        policy_loss = loss.detach()
+        loss = loss / normalizer
+    elif loss_type == "luspo":  # (:3143-3148): no mask on the per-token term
+        loss = (per_token_loss * mask.sum(1, keepdim=True)).mean()
         normalizer = grad_accum_steps
         policy_loss = loss.detach()
         loss = loss / normalizer
@@ -355,7 +391,7 @@ def grpo_loss(
         normalizer = grad_accum_steps
         policy_loss = loss.detach()
         loss = loss / normalizer
-    else:  # dapo
+    else:  # dapo, cispo, vespo
         n_items = num_items_in_batch
         if not torch.is_tensor(n_items):
             n_items = torch.tensor(float(n_items))
@@ -366,7 +402,7 @@ def grpo_loss(
     metrics: dict[str, float] = {}
     if entropy_coef != 0.0:
         eff = mask if entropy_mask is None else mask * entropy_mask
-        if loss_type == "dapo":
+        if loss_type in ("dapo", "cispo", "vespo"):
             ent_term = (entropies * eff).sum() / normalizer
         else:
             ent_term = (entropies * eff).sum() / eff.sum().clamp(min=1.0) / normalizer
@@ -390,14 +426,19 @@ def grpo_loss(
         metrics["kl"] = global_mean(per_token_kl.detach())
     if entropies is not None:
         metrics["entropy"] = global_mean(entropies.detach())
-    low = ((coef_1 < 1 - epsilon_low) & (adv < 0)).float()
-    high = ((coef_1 > 1 + epsilon_high) & (adv > 0)).float()
-    region = ((low + high) > 0).float()
-    metrics["clip_ratio/low_mean"] = global_mean(low)
-    metrics["clip_ratio/high_mean"] = global_mean(high)
-    metrics["clip_ratio/region_mean"] = global_mean(region)
-    metrics["clip_ratio/low_min"] = float(nanmin(seq_mean(low)))
-    metrics["clip_ratio/high_max"] = float(nanmax(seq_mean(high)))
+    if loss_type in ("grpo", "bnpo", "dr_grpo", "dapo", "luspo"):
+        low = ((coef_1 < 1 - epsilon_low) & (adv < 0)).float()
+        high = ((coef_1 > 1 + epsilon_high) & (adv > 0)).float()
+        region = ((low + high) > 0).float()
+        metrics["clip_ratio/low_mean"] = global_mean(low)
+        metrics["clip_ratio/high_mean"] = global_mean(high)
+        metrics["clip_ratio/region_mean"] = global_mean(region)
+        metrics["clip_ratio/low_min"] = float(nanmin(seq_mean(low)))
+        metrics["clip_ratio/high_max"] = float(nanmax(seq_mean(high)))
+    elif loss_type == "cispo":
+        metrics["cispo_clip_ratio"] = global_mean(((coef_1 > epsilon_high) & (adv > 0)).float())
+    elif loss_type == "vespo":
+        metrics["vespo/phi_seq_mean"] = global_mean(phi_seq)
     return loss, metrics
 
 

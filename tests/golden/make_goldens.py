@@ -88,6 +88,15 @@ GRPO_CASES = [
     dict(name="bnpo_entbonus_ga", loss_type="bnpo", beta=0.0, eps_low=0.2, eps_high=0.2, entropy_coef=0.02, grad_accum=2),
     dict(name="dr_grpo_entq_bonus", loss_type="dr_grpo", beta=0.04, eps_low=0.2, eps_high=0.2, entropy_coef=0.02,
          top_entropy_quantile=0.6, grad_accum=2),
+    dict(name="cispo", loss_type="cispo", beta=0.04, eps_low=0.2, eps_high=1.1),
+    dict(name="sapo", loss_type="sapo", beta=0.0, eps_low=0.2, eps_high=0.2, grad_accum=2),
+    dict(name="sapo_beta_seq", loss_type="sapo", beta=0.04, eps_low=0.2, eps_high=0.2, is_level="sequence"),
+    dict(name="vespo", loss_type="vespo", beta=0.04, eps_low=0.2, eps_high=0.2),
+    dict(name="luspo_seq", loss_type="luspo", beta=0.0, eps_low=0.05, eps_high=0.05, is_level="sequence", grad_accum=2),
+    dict(name="dapo_seq_is", loss_type="dapo", beta=0.04, eps_low=0.03, eps_high=0.04, is_level="sequence", bias_kl=True),
+    dict(name="bnpo_seq_delta", loss_type="bnpo", beta=0.0, eps_low=0.03, eps_high=0.04, is_level="sequence", delta=1.02),
+    dict(name="grpo_seq_offpolicy_entq", loss_type="grpo", beta=0.04, eps_low=0.05, eps_high=0.05, is_level="sequence",
+         off_policy=0.02, top_entropy_quantile=0.5),
 ]
 
 
@@ -129,7 +138,10 @@ def make_grpo(GRPOTrainer, out_dir):
         trainer.vllm_importance_sampling_correction = False
         trainer.max_completion_length = T
         trainer.current_gradient_accumulation_steps = case.get("grad_accum", 1)
-        trainer.args = SimpleNamespace(delta=case.get("delta"), use_bias_correction_kl=case.get("bias_kl", False))
+        trainer.args = SimpleNamespace(delta=case.get("delta"), use_bias_correction_kl=case.get("bias_kl", False),
+                                       sapo_temperature_pos=1.0, sapo_temperature_neg=1.05, vespo_k_pos=2.0,
+                                       vespo_lambda_pos=3.0, vespo_k_neg=3.0, vespo_lambda_neg=2.0)
+        trainer.get_gamma_weights = GRPOTrainer.get_gamma_weights
         trainer._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
         trainer.model = SimpleNamespace(training=True)
         trainer._get_per_token_logps_and_entropies = (

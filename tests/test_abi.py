@@ -61,18 +61,25 @@ def test_host_side_argument_validation():
     assert lib.trlk_group_advantages(fake, 7, 2, 0, fake, None) == -2
     assert lib.trlk_group_advantages(fake, 8, 2, 5, fake, None) == -5
     # grpo: beta != 0 without reference log-probs; missing workspace; bad loss type
-    args = dict(ref=None, beta=0.04, ws=fake, ws_bytes=1 << 20, loss_type=_lib.GRPO)
+    args = dict(ref=None, beta=0.04, ws=fake, ws_bytes=1 << 20, loss_type=_lib.GRPO, term=_lib.TERM_CLIP, seq=0,
+                adv_stride_t=0, tau=1.0)
 
     def grpo(**kw):
         a = dict(args, **kw)
-        return lib.trlk_grpo_loss(fake, None, a["ref"], None, fake, 1, 0, fake, None, None, 4, 16, a["loss_type"], 0.2,
-                                  0.2, float("nan"), a["beta"], 0, 1.0, 1.0, None, 1.0, 0.0, fake, fake, fake, None,
-                                  a["ws"], a["ws_bytes"], None)
+        return lib.trlk_grpo_loss(fake, None, a["ref"], None, fake, 1, a["adv_stride_t"], fake, None, None, None, 4,
+                                  16, a["loss_type"], a["term"], a["seq"], 0.2, 0.2, float("nan"), a["beta"], 0, 1.0,
+                                  1.0, None, 1.0, 0.0, a["tau"], 1.05, fake, fake, fake, None, a["ws"], a["ws_bytes"],
+                                  None)
 
     assert grpo() == -1 and "reference log-probs" in _lib.last_error()
     assert grpo(beta=0.0, ws_bytes=8) == -6
     assert grpo(beta=0.0, loss_type=9) == -5
     assert grpo(beta=0.0, loss_type=_lib.DAPO) == -1  # DAPO needs the normaliser scalar
+    assert grpo(beta=0.0, term=7) == -5
+    assert grpo(beta=0.0, term=_lib.TERM_WEIGHTED_LOGP) == -1  # needs the per-sequence coefficients
+    assert grpo(beta=0.0, term=_lib.TERM_SAPO, tau=0.0) == -5
+    assert grpo(beta=0.0, seq=1, adv_stride_t=1) == -7  # sequence-level weights with per-token advantages
+    assert grpo(beta=0.0, loss_type=_lib.LUSPO) == -7  # LUSPO only with sequence-level weights
     assert lib.trlk_grpo_workspace_bytes(64) >= 64 * 10 * 4
     # dpo: odd batch
     assert lib.trlk_dpo_loss(fake, fake, fake, fake, 3, 8, 0.1, fake, fake, fake, fake, None) == -2

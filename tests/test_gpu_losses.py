@@ -100,10 +100,6 @@ def test_golden_grpo_compute_loss_through_trainer_methods(amd, skip_masked):
             if c + key in g:
                 inputs[key] = _t(g[c + key]).to(DEV)
         model = lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None)  # noqa: E731
-        if case.get("is_level") == "sequence":
-            with pytest.raises(NotImplementedError):
-                tr._compute_loss(model, inputs)
-            continue
         captured = {}
         inner = tr._get_per_token_logps_and_entropies
 
@@ -139,7 +135,7 @@ def test_golden_grpo_compute_loss_through_trainer_methods(amd, skip_masked):
             ok = (math.isnan(got) and math.isnan(want)) or abs(got - want) <= (2e-2 if low else 1e-5) * max(1.0, abs(want))
             assert ok, (case["name"], name, got, want)
         ran += 1
-    assert ran >= 18
+    assert ran >= 27
 
 
 def test_grpo_loss_against_oracle_random(amd):
@@ -178,6 +174,36 @@ def test_grpo_loss_against_oracle_random(amd):
                 if name == "entropy_coef":
                     continue
                 assert abs(md[name] - want) <= 1e-5 * max(1.0, abs(want)), (lt, name, md[name], want)
+    # the remaining policy terms and sequence-level importance weights
+    variants = [("cispo", "token", 0.04), ("cispo", "sequence", 0.0), ("sapo", "token", 0.04), ("sapo", "sequence", 0.04),
+                ("vespo", "token", 0.04), ("vespo", "sequence", 0.04), ("luspo", "sequence", 0.0),
+                ("grpo", "sequence", 0.04), ("bnpo", "sequence", 0.04), ("dr_grpo", "sequence", 0.0),
+                ("dapo", "sequence", 0.04)]
+    old_seq = lp + 0.02 * torch.randn(B, T, generator=g)  # sequence means of the token ratios stay near the clip range
+    for lt, level, beta in variants:
+        for bias_kl in (False, True):
+            o = old_seq if level == "sequence" or lt == "vespo" else old
+            kw = dict(entropies=ent, old_per_token_logps=o, ref_per_token_logps=ref, loss_type=lt, epsilon_low=0.002,
+                      epsilon_high=1.05 if lt == "cispo" else 0.003, beta=beta, max_completion_length=T,
+                      num_items_in_batch=n_items, grad_accum_steps=2.0, entropy_coef=0.01,
+                      importance_sampling_level=level, use_bias_correction_kl=bias_kl)
+            olp = lp.clone().requires_grad_(True)
+            oloss, ometrics = oracle.grpo_loss(olp, adv, mask, **kw)
+            oloss.backward()
+            dlp = lp.to(DEV).requires_grad_(True)
+            dkw = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in kw.items()}
+            loss, metrics = amd.grpo_loss(dlp, adv.to(DEV), mask.to(DEV), **dkw)
+            loss.backward()
+            tag = (lt, level, bias_kl)
+            assert abs(float(loss) - float(oloss)) <= 1e-5 * max(1.0, abs(float(oloss))), tag
+            assert _rel_l2(dlp.grad, olp.grad) < 1e-5, tag
+            md = amd.trainer.metrics_to_dict(metrics, beta, loss_type=lt)
+            for name, want in ometrics.items():
+                if name == "entropy_coef":
+                    continue
+                assert abs(md[name] - want) <= 1e-5 * max(1.0, abs(want)), (tag, name, md[name], want)
+    with pytest.raises(NotImplementedError):
+        amd.grpo_loss(lp.to(DEV), adv.to(DEV), mask.to(DEV), loss_type="luspo", old_per_token_logps=old.to(DEV))
     # determinism: identical bits on a second call
     a = amd.grpo_loss(lp.to(DEV), adv.to(DEV), mask.to(DEV), loss_type="grpo", old_per_token_logps=old.to(DEV))
     b = amd.grpo_loss(lp.to(DEV), adv.to(DEV), mask.to(DEV), loss_type="grpo", old_per_token_logps=old.to(DEV))

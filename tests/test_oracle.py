@@ -208,7 +208,7 @@ def _grpo_case(case, g):
 
 def test_golden_grpo_compute_loss():
     cases, g = load_golden("grpo_compute_loss")
-    assert len(cases) >= 16
+    assert len(cases) >= 27
     for case in cases:
         c = f"c{case['id']}_"
         logits, logps, ent, loss, metrics = _grpo_case(case, g)

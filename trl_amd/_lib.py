@@ -17,7 +17,8 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 LIB_PATH = os.environ.get("TRLK_LIBRARY_PATH") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libtrlk.so")
 
 F32, BF16, F16 = 0, 1, 2
-GRPO, BNPO, DR_GRPO, DAPO = 0, 1, 2, 3
+GRPO, BNPO, DR_GRPO, DAPO, LUSPO = 0, 1, 2, 3, 4
+TERM_CLIP, TERM_CISPO, TERM_SAPO, TERM_WEIGHTED_LOGP = 0, 1, 2, 3
 SCALE_GROUP, SCALE_BATCH, SCALE_NONE = 0, 1, 2
 FLAG_INDEX_OUT_OF_RANGE = 1
 GRPO_NUM_METRICS = 16
@@ -42,9 +43,10 @@ SIGNATURES = {
     "trlk_grpo_workspace_bytes": (c_size_t, [c_int64]),
     "trlk_grpo_loss": (
         c_int32,
-        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int64,
-         c_int64, c_int32, c_float, c_float, c_float, c_float, c_int32, c_float, c_float, c_void_p, c_float, c_float,
-         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_int64, c_int32, c_int32, c_int32, c_float, c_float, c_float, c_float, c_int32, c_float, c_float,
+         c_void_p, c_float, c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+         c_void_p],
     ),
     "trlk_dpo_loss": (
         c_int32,

@@ -11,7 +11,7 @@ namespace trlk {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kRowStats = 12;  // floats of workspace per sequence
+constexpr int kRowStats = 16;  // floats of workspace per sequence
 
 enum RowStat { RS_MASK = 0, RS_LOSS, RS_KL, RS_ENT, RS_LOW, RS_HIGH, RS_REGION, RS_ENT_EFF, RS_EFF, RS_QUOT };
 
@@ -70,17 +70,71 @@ __global__ __launch_bounds__(kThreads) void group_advantages_kernel(const float*
 
 // ------------------------------------------------------------------------------ GRPO
 struct GrpoArgs {
-    const float *logp, *old_logp, *ref_logp, *entropy, *adv, *mask, *token_weight, *entropy_mask;
+    const float *logp, *old_logp, *ref_logp, *entropy, *adv, *mask, *token_weight, *entropy_mask, *seq_coef;
     int64_t adv_stride_b, adv_stride_t;
     int64_t B, T;
-    int loss_type;
+    int loss_type, policy_term, seq_level;
     float eps_low, eps_high, delta, beta;
     int bias_kl;
     float grad_accum, dr_denominator;
     const float* dapo_normalizer;
-    float num_processes, entropy_coef;
+    float num_processes, entropy_coef, sapo_tau_pos, sapo_tau_neg;
     float *out_loss, *out_metrics, *out_dlogp, *out_dentropy, *ws;
 };
+
+constexpr int kRowStatsUsed = 13;
+enum RowStat2 { RS_CLIP_CNT = 10, RS_AUX = 11, RS_AUX_CNT = 12 };
+static_assert(kRowStatsUsed <= 16, "row stats");
+
+// Policy term f(c, A, logp) of one token (or one sequence) and its two partial derivatives:
+// through the log importance ratio ln c, and directly through logp (terms that multiply logp itself).
+struct PolicyTerm {
+    float f, d_lnc, d_logp, low, high, aux;
+};
+
+__device__ __forceinline__ PolicyTerm policy_term(const GrpoArgs& a, float c_raw, float A, float lp, float coef) {
+    PolicyTerm r{0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const float lo = 1.f - a.eps_low, hi = 1.f + a.eps_high;
+    switch (a.policy_term) {
+        case TRLK_TERM_CLIP: {  // -min(c' A, clamp(c, lo, hi) A), c' = min(c, delta)   (grpo_trainer.py:3083-3091)
+            const bool has_delta = a.delta == a.delta;
+            const float c2 = fminf(fmaxf(c_raw, lo), hi);
+            const float c1 = has_delta ? fminf(c_raw, a.delta) : c_raw;
+            const float l1 = c1 * A, l2 = c2 * A;
+            // d c / d ln c = c; clamp passes the gradient on the closed interval
+            const float d1 = (!has_delta || c_raw <= a.delta) ? A * c_raw : 0.f;
+            const float d2 = (c_raw >= lo && c_raw <= hi) ? A * c_raw : 0.f;
+            // min(l1, l2): the gradient goes to the smaller operand, half to each on a tie
+            const float w1 = (l1 < l2) ? 1.f : ((l1 == l2) ? 0.5f : 0.f);
+            r.f = -fminf(l1, l2);
+            r.d_lnc = -(w1 * d1 + (1.f - w1) * d2);
+            r.low = (c1 < lo && A < 0.f) ? 1.f : 0.f;
+            r.high = (c1 > hi && A > 0.f) ? 1.f : 0.f;
+            break;
+        }
+        case TRLK_TERM_CISPO: {  // -min(c, eps_high).detach() * A * logp   (:3080-3082)
+            const float cl = fminf(c_raw, a.eps_high);
+            r.f = -cl * A * lp;
+            r.d_logp = -cl * A;
+            r.aux = (c_raw > a.eps_high && A > 0.f) ? 1.f : 0.f;
+            break;
+        }
+        case TRLK_TERM_SAPO: {  // -sigmoid(tau (c - 1)) * 4 / tau * A   (:3092-3095)
+            const float tau = A > 0.f ? a.sapo_tau_pos : a.sapo_tau_neg;
+            const float sg = 1.f / (1.f + expf(-tau * (c_raw - 1.f)));
+            r.f = -sg * 4.f / tau * A;
+            r.d_lnc = -4.f * A * sg * (1.f - sg) * c_raw;
+            break;
+        }
+        default: {  // TRLK_TERM_WEIGHTED_LOGP: -coef * A * logp with a given, detached per-sequence coef (:3096-3107)
+            r.f = -coef * A * lp;
+            r.d_logp = -coef * A;
+            r.aux = coef;
+            break;
+        }
+    }
+    return r;
+}
 
 // Pass 1: one workgroup per sequence.  Writes d(per-token loss)/d(logp) * mask (not yet
 // normalised) and the sequence's masked sums.
@@ -89,10 +143,25 @@ __global__ __launch_bounds__(kThreads) void grpo_rows_kernel(GrpoArgs a) {
     const int64_t b = blockIdx.x;
     const int tid = threadIdx.x;
     const int64_t off = b * a.T;
-    const bool has_delta = a.delta == a.delta;
-    const float lo = 1.f - a.eps_low, hi = 1.f + a.eps_high;
+    const float coef = a.seq_coef ? a.seq_coef[b] : 0.f;
+
+    // sequence-level importance weight: exp(masked mean of the token log-ratios)   (:3057-3059)
+    float n_b = 0.f, c_seq = 1.f;
+    if (a.seq_level) {
+        float s1 = 0.f, s0 = 0.f;
+        for (int64_t t = tid; t < a.T; t += kThreads) {
+            const float m = a.mask[off + t];
+            if (m == 0.f) continue;
+            s0 += m;
+            if (a.old_logp) s1 += (a.logp[off + t] - a.old_logp[off + t]) * m;
+        }
+        s1 = block_sum<kThreads>(s1, scratch);
+        n_b = block_sum<kThreads>(s0, scratch);
+        c_seq = expf(s1 / fmaxf(n_b, 1.f));
+    }
 
     float s_mask = 0, s_loss = 0, s_kl = 0, s_ent = 0, s_low = 0, s_high = 0, s_reg = 0, s_ent_eff = 0, s_eff = 0;
+    float s_aux = 0, s_glnc = 0;
     for (int64_t t = tid; t < a.T; t += kThreads) {
         const float m = a.mask[off + t];
         if (m == 0.f) {  // a masked token contributes exactly nothing, whatever its (possibly skipped) inputs hold
@@ -101,60 +170,80 @@ __global__ __launch_bounds__(kThreads) void grpo_rows_kernel(GrpoArgs a) {
         }
         const float lp = a.logp[off + t];
         const float A = a.adv[b * a.adv_stride_b + t * a.adv_stride_t];
-        const float c1_raw = a.old_logp ? expf(lp - a.old_logp[off + t]) : 1.f;
-        const float c2 = fminf(fmaxf(c1_raw, lo), hi);
-        const float c1 = has_delta ? fminf(c1_raw, a.delta) : c1_raw;
-        const float l1 = c1 * A, l2 = c2 * A;
-        // d c1_raw / d logp = c1_raw; clamp passes the gradient on the closed interval
-        const float d1 = (!has_delta || c1_raw <= a.delta) ? A * c1_raw : 0.f;
-        const float d2 = (c1_raw >= lo && c1_raw <= hi) ? A * c1_raw : 0.f;
-        // min(l1, l2): the gradient goes to the smaller operand, half to each on a tie
-        const float w1 = (l1 < l2) ? 1.f : ((l1 == l2) ? 0.5f : 0.f);
-        float pl = -fminf(l1, l2);
-        float dpl = -(w1 * d1 + (1.f - w1) * d2);
+        const float c_raw = a.seq_level ? c_seq : (a.old_logp ? expf(lp - a.old_logp[off + t]) : 1.f);
+        const PolicyTerm p = policy_term(a, c_raw, A, lp, coef);
+        float pl = p.f, g_lnc = p.d_lnc, g_lp = p.d_logp;
         if (a.token_weight) {
             const float w = a.token_weight[off + t];
             pl *= w;
-            dpl *= w;
+            g_lnc *= w;
+            g_lp *= w;
         }
         float kl = 0.f;
-        if (a.beta != 0.f) {
+        if (a.beta != 0.f) {  // k3 estimator exp(d) - d - 1, d = ref - logp   (:3069-3076)
             const float d = a.ref_logp[off + t] - lp;
             const float e = expf(d);
             kl = e - d - 1.f;
             float dkl = 1.f - e;
-            if (a.bias_kl) {
-                dkl = (dkl + kl) * c1_raw;
-                kl *= c1_raw;
+            if (a.bias_kl) {  // kl * c: the factor c is differentiated through ln c
+                g_lnc += a.beta * kl * c_raw;
+                dkl *= c_raw;
+                kl *= c_raw;
             }
             pl += a.beta * kl;
-            dpl += a.beta * dkl;
+            g_lp += a.beta * dkl;
         }
         const float H = a.entropy ? a.entropy[off + t] : 0.f;
-        const float is_low = (c1 < lo && A < 0.f) ? 1.f : 0.f;
-        const float is_high = (c1 > hi && A > 0.f) ? 1.f : 0.f;
         const float eff = a.entropy_mask ? m * a.entropy_mask[off + t] : m;
         s_mask += m;
         s_loss += pl * m;
         s_kl += kl * m;
         s_ent += H * m;
-        s_low += is_low * m;
-        s_high += is_high * m;
-        s_reg += fmaxf(is_low, is_high) * m;
+        s_low += p.low * m;
+        s_high += p.high * m;
+        s_reg += fmaxf(p.low, p.high) * m;
+        s_aux += p.aux * m;
         s_ent_eff += H * eff;
         s_eff += eff;
-        a.out_dlogp[off + t] = dpl * m;
+        if (a.seq_level) {
+            s_glnc += g_lnc * m;
+            a.out_dlogp[off + t] = g_lp * m;
+        } else {
+            a.out_dlogp[off + t] = (g_lp + g_lnc) * m;
+        }
     }
     float* ws = a.ws + b * kRowStats;
     const float r_mask = block_sum<kThreads>(s_mask, scratch);
     const float r_loss = block_sum<kThreads>(s_loss, scratch);
     const float r_kl = block_sum<kThreads>(s_kl, scratch);
     const float r_ent = block_sum<kThreads>(s_ent, scratch);
-    const float r_low = block_sum<kThreads>(s_low, scratch);
-    const float r_high = block_sum<kThreads>(s_high, scratch);
-    const float r_reg = block_sum<kThreads>(s_reg, scratch);
+    float r_low = block_sum<kThreads>(s_low, scratch);
+    float r_high = block_sum<kThreads>(s_high, scratch);
+    float r_reg = block_sum<kThreads>(s_reg, scratch);
+    float r_aux = block_sum<kThreads>(s_aux, scratch);
     const float r_ent_eff = block_sum<kThreads>(s_ent_eff, scratch);
     const float r_eff = block_sum<kThreads>(s_eff, scratch);
+    float clip_cnt = r_mask, aux_cnt = r_mask;
+    if (a.seq_level) {
+        // the ratio-dependent part of every token's loss pulls on all tokens of the sequence through the mean
+        const float g_seq = block_sum<kThreads>(s_glnc, scratch) / fmaxf(n_b, 1.f);
+        for (int64_t t = tid; t < a.T; t += kThreads) {
+            const float m = a.mask[off + t];
+            if (m != 0.f) a.out_dlogp[off + t] += g_seq * m;
+        }
+        // clip flags are per sequence: one value each, also for a sequence without active tokens
+        const PolicyTerm p = policy_term(a, c_seq, a.adv[b * a.adv_stride_b], 0.f, coef);
+        r_low = p.low;
+        r_high = p.high;
+        r_reg = fmaxf(p.low, p.high);
+        r_aux = p.aux;
+        clip_cnt = 1.f;
+        aux_cnt = 1.f;
+    }
+    if (a.policy_term == TRLK_TERM_WEIGHTED_LOGP) {  // the logged quantity is the per-sequence coefficient
+        r_aux = coef;
+        aux_cnt = 1.f;
+    }
     if (tid == 0) {
         ws[RS_MASK] = r_mask;
         ws[RS_LOSS] = r_loss;
@@ -166,6 +255,9 @@ __global__ __launch_bounds__(kThreads) void grpo_rows_kernel(GrpoArgs a) {
         ws[RS_ENT_EFF] = r_ent_eff;
         ws[RS_EFF] = r_eff;
         ws[RS_QUOT] = r_loss / fmaxf(r_mask, 1.f);
+        ws[RS_CLIP_CNT] = clip_cnt;
+        ws[RS_AUX] = r_aux;
+        ws[RS_AUX_CNT] = aux_cnt;
     }
 }
 
@@ -176,20 +268,20 @@ __global__ __launch_bounds__(kThreads) void grpo_finish_kernel(GrpoArgs a) {
     __shared__ float scratch[kThreads / kWave];
     const int64_t b = blockIdx.x;
     const int tid = threadIdx.x;
-    float tot[kRowStats];
+    float tot[kRowStatsUsed];
 #pragma unroll
-    for (int j = 0; j < kRowStats; ++j) tot[j] = 0.f;
+    for (int j = 0; j < kRowStatsUsed; ++j) tot[j] = 0.f;
     float low_min = INFINITY, high_max = -INFINITY;
     for (int64_t r = tid; r < a.B; r += kThreads) {
         const float* ws = a.ws + r * kRowStats;
 #pragma unroll
-        for (int j = 0; j <= RS_QUOT; ++j) tot[j] += ws[j];
-        const float lm = ws[RS_LOW] / ws[RS_MASK], hm = ws[RS_HIGH] / ws[RS_MASK];  // NaN for an empty sequence
+        for (int j = 0; j < kRowStatsUsed; ++j) tot[j] += ws[j];
+        const float lm = ws[RS_LOW] / ws[RS_CLIP_CNT], hm = ws[RS_HIGH] / ws[RS_CLIP_CNT];  // NaN for an empty sequence
         if (lm == lm) low_min = fminf(low_min, lm);
         if (hm == hm) high_max = fmaxf(high_max, hm);
     }
 #pragma unroll
-    for (int j = 0; j <= RS_QUOT; ++j) tot[j] = block_sum<kThreads>(tot[j], scratch);
+    for (int j = 0; j < kRowStatsUsed; ++j) tot[j] = block_sum<kThreads>(tot[j], scratch);
     low_min = wave_min(low_min);
     high_max = wave_max(high_max);
     __shared__ float s_min[kThreads / kWave], s_max[kThreads / kWave];
@@ -211,6 +303,10 @@ __global__ __launch_bounds__(kThreads) void grpo_finish_kernel(GrpoArgs a) {
         case TRLK_GRPO:
             loss = tot[RS_QUOT] / Bf;
             norm_rows = 1.f / Bf;  // times 1 / max(mask_sum_b, 1) per row
+            break;
+        case TRLK_LUSPO:  // mean over sequences of (per-sequence loss * active tokens)   (:3143-3148)
+            loss = tot[RS_LOSS] / Bf;
+            norm_rows = 1.f / Bf;
             break;
         case TRLK_BNPO:
             loss = tot[RS_LOSS] / fmaxf(tot[RS_MASK], 1.f);
@@ -243,20 +339,25 @@ __global__ __launch_bounds__(kThreads) void grpo_finish_kernel(GrpoArgs a) {
     }
     if (b == 0 && tid == 0) {
         const float cnt = fmaxf(tot[RS_MASK], 1.f);
+        const float clip_cnt = fmaxf(tot[RS_CLIP_CNT], 1.f);
         a.out_loss[0] = loss;
         float* mt = a.out_metrics;
         for (int j = 0; j < TRLK_GRPO_NUM_METRICS; ++j) mt[j] = 0.f;
         mt[TRLK_M_KL_MEAN] = (a.beta != 0.f) ? tot[RS_KL] / cnt : NAN;
         mt[TRLK_M_ENTROPY_MEAN] = a.entropy ? tot[RS_ENT] / cnt : NAN;
-        mt[TRLK_M_CLIP_LOW_MEAN] = tot[RS_LOW] / cnt;
-        mt[TRLK_M_CLIP_HIGH_MEAN] = tot[RS_HIGH] / cnt;
-        mt[TRLK_M_CLIP_REGION_MEAN] = tot[RS_REGION] / cnt;
+        mt[TRLK_M_CLIP_LOW_MEAN] = tot[RS_LOW] / clip_cnt;
+        mt[TRLK_M_CLIP_HIGH_MEAN] = tot[RS_HIGH] / clip_cnt;
+        mt[TRLK_M_CLIP_REGION_MEAN] = tot[RS_REGION] / clip_cnt;
         mt[TRLK_M_CLIP_LOW_MIN] = (low_min == INFINITY) ? NAN : low_min;
         mt[TRLK_M_CLIP_HIGH_MAX] = (high_max == -INFINITY) ? NAN : high_max;
         mt[TRLK_M_POLICY_LOSS] = policy_loss;
         mt[TRLK_M_MASK_SUM] = tot[RS_MASK];
         mt[TRLK_M_KL_SUM] = tot[RS_KL];
         mt[TRLK_M_ENTROPY_SUM] = tot[RS_ENT];
+        mt[TRLK_M_AUX_MEAN] = tot[RS_AUX] / fmaxf(tot[RS_AUX_CNT], 1.f);
+        mt[TRLK_M_CLIP_COUNT] = tot[RS_CLIP_CNT];
+        mt[TRLK_M_AUX_SUM] = tot[RS_AUX];
+        mt[TRLK_M_AUX_COUNT] = tot[RS_AUX_CNT];
     }
     const float row_scale =
         (a.loss_type == TRLK_GRPO) ? norm_rows / fmaxf(a.ws[b * kRowStats + RS_MASK], 1.f) : norm_rows;
@@ -423,18 +524,30 @@ extern "C" size_t trlk_grpo_workspace_bytes(int64_t n_seq) {
 extern "C" int trlk_grpo_loss(const float* d_logp, const float* d_old_logp, const float* d_ref_logp,
                               const float* d_entropy, const float* d_advantages, int64_t adv_stride_b,
                               int64_t adv_stride_t, const float* d_mask, const float* d_token_weight,
-                              const float* d_entropy_mask, int64_t n_seq, int64_t seq_len, int32_t loss_type,
-                              float epsilon_low, float epsilon_high, float delta, float beta,
-                              int32_t use_bias_correction_kl, float grad_accum_steps, float dr_grpo_denominator,
-                              const float* d_dapo_normalizer, float num_processes, float entropy_coef,
-                              float* d_out_loss, float* d_out_metrics, float* d_out_dlogp, float* d_out_dentropy,
-                              void* d_workspace, size_t workspace_bytes, trlk_stream_t stream) {
+                              const float* d_entropy_mask, const float* d_seq_coef, int64_t n_seq, int64_t seq_len,
+                              int32_t loss_type, int32_t policy_term, int32_t sequence_level, float epsilon_low,
+                              float epsilon_high, float delta, float beta, int32_t use_bias_correction_kl,
+                              float grad_accum_steps, float dr_grpo_denominator, const float* d_dapo_normalizer,
+                              float num_processes, float entropy_coef, float sapo_temperature_pos,
+                              float sapo_temperature_neg, float* d_out_loss, float* d_out_metrics, float* d_out_dlogp,
+                              float* d_out_dentropy, void* d_workspace, size_t workspace_bytes, trlk_stream_t stream) {
     clear_error();
     TRLK_REQUIRE(n_seq >= 1 && seq_len >= 1, TRLK_ERR_BAD_SHAPE, "grpo_loss: need n_seq >= 1 and seq_len >= 1 (got %lld x %lld)",
                  (long long)n_seq, (long long)seq_len);
     TRLK_REQUIRE(n_seq < (int64_t(1) << 31), TRLK_ERR_BAD_SHAPE, "grpo_loss: too many sequences");
-    TRLK_REQUIRE(loss_type >= TRLK_GRPO && loss_type <= TRLK_DAPO, TRLK_ERR_BAD_VALUE, "grpo_loss: unknown loss_type %d",
+    TRLK_REQUIRE(loss_type >= TRLK_GRPO && loss_type <= TRLK_LUSPO, TRLK_ERR_BAD_VALUE, "grpo_loss: unknown loss_type %d",
                  loss_type);
+    TRLK_REQUIRE(policy_term >= TRLK_TERM_CLIP && policy_term <= TRLK_TERM_WEIGHTED_LOGP, TRLK_ERR_BAD_VALUE,
+                 "grpo_loss: unknown policy_term %d", policy_term);
+    TRLK_REQUIRE(policy_term != TRLK_TERM_WEIGHTED_LOGP || d_seq_coef != nullptr, TRLK_ERR_NULL_POINTER,
+                 "grpo_loss: the weighted-logp policy term needs the per-sequence coefficients");
+    TRLK_REQUIRE(policy_term != TRLK_TERM_SAPO || (sapo_temperature_pos > 0.f && sapo_temperature_neg > 0.f),
+                 TRLK_ERR_BAD_VALUE, "grpo_loss: SAPO temperatures must be positive");
+    TRLK_REQUIRE(loss_type != TRLK_LUSPO || (sequence_level && beta == 0.f && d_token_weight == nullptr),
+                 TRLK_ERR_UNSUPPORTED,
+                 "grpo_loss: LUSPO is built for sequence-level importance weights without KL term or token weights");
+    TRLK_REQUIRE(!sequence_level || adv_stride_t == 0, TRLK_ERR_UNSUPPORTED,
+                 "grpo_loss: sequence-level importance weights need one advantage per sequence");
     TRLK_REQUIRE(d_logp && d_advantages && d_mask && d_out_loss && d_out_metrics && d_out_dlogp, TRLK_ERR_NULL_POINTER,
                  "grpo_loss: a required pointer is null");
     TRLK_REQUIRE(beta == 0.f || d_ref_logp != nullptr, TRLK_ERR_NULL_POINTER,
@@ -451,9 +564,10 @@ extern "C" int trlk_grpo_loss(const float* d_logp, const float* d_old_logp, cons
     TRLK_REQUIRE(d_workspace != nullptr && workspace_bytes >= trlk_grpo_workspace_bytes(n_seq), TRLK_ERR_WORKSPACE,
                  "grpo_loss: workspace of %zu bytes needed, %zu given", trlk_grpo_workspace_bytes(n_seq), workspace_bytes);
     GrpoArgs a{d_logp, d_old_logp, d_ref_logp, d_entropy, d_advantages, d_mask, d_token_weight, d_entropy_mask,
-               adv_stride_b, adv_stride_t, n_seq, seq_len, loss_type, epsilon_low, epsilon_high, delta, beta,
-               use_bias_correction_kl, grad_accum_steps, dr_grpo_denominator, d_dapo_normalizer, num_processes,
-               entropy_coef, d_out_loss, d_out_metrics, d_out_dlogp, d_out_dentropy, static_cast<float*>(d_workspace)};
+               d_seq_coef, adv_stride_b, adv_stride_t, n_seq, seq_len, loss_type, policy_term, sequence_level != 0,
+               epsilon_low, epsilon_high, delta, beta, use_bias_correction_kl, grad_accum_steps, dr_grpo_denominator,
+               d_dapo_normalizer, num_processes, entropy_coef, sapo_temperature_pos, sapo_temperature_neg, d_out_loss,
+               d_out_metrics, d_out_dlogp, d_out_dentropy, static_cast<float*>(d_workspace)};
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipLaunchKernelGGL(grpo_rows_kernel, dim3((unsigned)n_seq), dim3(kThreads), 0, s, a);
     if (int rc = launch_status("grpo_loss (rows)")) return rc;

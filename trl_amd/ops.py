@@ -193,7 +193,17 @@ def group_advantages(rewards: Tensor, num_generations: int, scale_rewards: str =
 # --------------------------------------------------------------------------------------------
 # GRPO loss (K2)
 # --------------------------------------------------------------------------------------------
-LOSS_TYPES = {"grpo": _lib.GRPO, "bnpo": _lib.BNPO, "dr_grpo": _lib.DR_GRPO, "dapo": _lib.DAPO}
+# reference loss_type -> (normalisation, per-token policy term)   (trl/trainer/grpo_trainer.py:3080-3148)
+LOSS_TYPES = {
+    "grpo": (_lib.GRPO, _lib.TERM_CLIP),
+    "bnpo": (_lib.BNPO, _lib.TERM_CLIP),
+    "dr_grpo": (_lib.DR_GRPO, _lib.TERM_CLIP),
+    "dapo": (_lib.DAPO, _lib.TERM_CLIP),
+    "luspo": (_lib.LUSPO, _lib.TERM_CLIP),
+    "cispo": (_lib.DAPO, _lib.TERM_CISPO),
+    "sapo": (_lib.GRPO, _lib.TERM_SAPO),
+    "vespo": (_lib.DAPO, _lib.TERM_WEIGHTED_LOGP),
+}
 
 
 def _f32c(t: Optional[Tensor]) -> Optional[Tensor]:
@@ -206,7 +216,8 @@ def grpo_loss_op(
     advantages: Tensor, mask: Tensor, token_weight: Optional[Tensor], entropy_mask: Optional[Tensor],
     dapo_normalizer: Optional[Tensor], loss_type: int, epsilon_low: float, epsilon_high: float, delta: float,
     beta: float, use_bias_correction_kl: bool, grad_accum_steps: float, dr_grpo_denominator: float,
-    num_processes: float, entropy_coef: float,
+    num_processes: float, entropy_coef: float, policy_term: int = 0, sequence_level: bool = False,
+    seq_coef: Optional[Tensor] = None, sapo_temperature_pos: float = 1.0, sapo_temperature_neg: float = 1.05,
 ) -> tuple[Tensor, Tensor, Tensor, Tensor]:
     """Returns (loss [], metrics [16], d loss/d logp [B,T], d loss/d entropy [B,T])."""
     if logp.dim() != 2:
@@ -229,6 +240,10 @@ def grpo_loss_op(
         if t is not None and tuple(t.shape) != (B, T):
             raise ValueError(f"grpo_loss: {name} has shape {tuple(t.shape)}, expected {(B, T)}")
     dapo_normalizer = None if dapo_normalizer is None else dapo_normalizer.reshape(1).contiguous().float()
+    if seq_coef is not None:
+        if seq_coef.numel() != B:
+            raise ValueError("grpo_loss: seq_coef must have one entry per sequence")
+        seq_coef = seq_coef.reshape(B).contiguous().float()
     loss = torch.empty((), dtype=torch.float32, device=dev)
     metrics = torch.empty((_lib.GRPO_NUM_METRICS,), dtype=torch.float32, device=dev)
     dlogp = torch.empty((B, T), dtype=torch.float32, device=dev)
@@ -239,10 +254,11 @@ def grpo_loss_op(
         check(
             lib.trlk_grpo_loss(
                 ptr(logp), ptr(old_logp), ptr(ref_logp), ptr(entropy), ptr(advantages), sb, st, ptr(mask),
-                ptr(token_weight), ptr(entropy_mask), B, T, loss_type, epsilon_low, epsilon_high, delta, beta,
-                int(use_bias_correction_kl), grad_accum_steps, dr_grpo_denominator, ptr(dapo_normalizer),
-                num_processes, entropy_coef, ptr(loss), ptr(metrics), ptr(dlogp), ptr(dent), ptr(ws), ws_bytes,
-                current_stream(dev),
+                ptr(token_weight), ptr(entropy_mask), ptr(seq_coef), B, T, loss_type, policy_term,
+                int(sequence_level), epsilon_low, epsilon_high, delta, beta, int(use_bias_correction_kl),
+                grad_accum_steps, dr_grpo_denominator, ptr(dapo_normalizer), num_processes, entropy_coef,
+                sapo_temperature_pos, sapo_temperature_neg, ptr(loss), ptr(metrics), ptr(dlogp), ptr(dent), ptr(ws),
+                ws_bytes, current_stream(dev),
             )
         )
     if dent is None:
@@ -253,7 +269,8 @@ def grpo_loss_op(
 @grpo_loss_op.register_fake
 def _(logp, old_logp, ref_logp, entropy, advantages, mask, token_weight, entropy_mask, dapo_normalizer, loss_type,
       epsilon_low, epsilon_high, delta, beta, use_bias_correction_kl, grad_accum_steps, dr_grpo_denominator,
-      num_processes, entropy_coef):
+      num_processes, entropy_coef, policy_term=0, sequence_level=False, seq_coef=None, sapo_temperature_pos=1.0,
+      sapo_temperature_neg=1.05):
     f = lambda *s: torch.empty(s, dtype=torch.float32, device=logp.device)  # noqa: E731
     return f(), f(_lib.GRPO_NUM_METRICS), f(*logp.shape), (f(*logp.shape) if entropy_coef != 0.0 else f(0))
 
@@ -268,7 +285,7 @@ def _grpo_setup(ctx, inputs, output):
 
 def _grpo_backward(ctx, g_loss, g_metrics, g_dlogp, g_dent):
     dlogp, dent = ctx.saved_tensors
-    grads = [None] * 19
+    grads = [None] * 24
     if g_loss is not None:
         grads[0] = (g_loss * dlogp).to(ctx.logp_dtype)
         if ctx.has_ent_grad:

@@ -25,6 +25,7 @@ __all__ = [
     "group_advantages",
     "get_off_policy_mask",
     "get_high_entropy_mask",
+    "get_gamma_weights",
     "GRPOLossMixin",
 ]
 
@@ -78,6 +79,24 @@ def get_high_entropy_mask(entropies, mask, threshold, accelerator=None):
     return ((entropies * mask.float()) >= cut) & mask.bool()
 
 
+@torch.no_grad()
+def get_gamma_weights(advantages, log_ratio_per_token, mask, importance_sampling_ratio=None, k_pos=2.0,
+                      lambda_pos=3.0, k_neg=3.0, lambda_neg=2.0):
+    """VESPO's detached `(B, 1)` sequence coefficients phi(w) = e^lambda w^k e^(-lambda w), evaluated in
+    log space with w = exp(sum over active tokens of the clamped log-ratios), optionally times the
+    sampler correction (trl/trainer/grpo_trainer.py:2941-2989).  `[B, T]`-sized torch ops."""
+    floor = math.log(1e-8)
+    log_w = (log_ratio_per_token.clamp(-20.0, 20.0) * mask).sum(dim=-1, keepdim=True)
+    if importance_sampling_ratio is not None:
+        log_w = log_w + torch.log(importance_sampling_ratio).clamp(floor, 20.0).sum(dim=-1, keepdim=True)
+    log_w = log_w.clamp(floor, 20.0)
+    nonneg = advantages >= 0
+    k = torch.where(nonneg, k_pos, k_neg)
+    lam = torch.where(nonneg, lambda_pos, lambda_neg).clamp(min=1e-4)
+    phi = torch.exp(lam + k * log_w - lam * torch.exp(log_w))
+    return phi.nan_to_num(nan=0.0, posinf=0.0, neginf=0.0)
+
+
 def grpo_loss(
     per_token_logps: Tensor,
     advantages: Tensor,
@@ -99,20 +118,51 @@ def grpo_loss(
     token_weight: Tensor | None = None,
     entropy_mask: Tensor | None = None,
     entropy_coef: float = 0.0,
+    importance_sampling_level: str = "token",
+    sapo_temperature_pos: float = 1.0,
+    sapo_temperature_neg: float = 1.05,
+    vespo_params: tuple[float, float, float, float] = (2.0, 3.0, 3.0, 2.0),
+    importance_sampling_ratio: Tensor | None = None,
 ) -> tuple[Tensor, Tensor]:
-    """Fused GRPO-family loss (token-level importance weights) on `[B, T]` log-probs.
+    """Fused GRPO-family loss on `[B, T]` log-probs: loss types grpo, bnpo, dr_grpo, dapo, luspo, cispo,
+    sapo and vespo, token- or sequence-level importance weights.
+
+    `token_weight` is the product of every `[B, T]` factor the reference multiplies onto the policy term
+    (off-policy mask, entropy mask, sampler importance ratio).  `importance_sampling_ratio` is only read
+    by vespo, whose sequence coefficients `(k_pos, lambda_pos, k_neg, lambda_neg) = vespo_params` absorb it.
 
     Returns `(loss, metrics)`; `metrics` is the fp32 device vector indexed by
     `trl_amd._lib`'s `trlk_grpo_metric` order (see include/trlk.h).  Differentiable w.r.t.
     `per_token_logps` (and `entropies` when `entropy_coef != 0`)."""
     if loss_type not in ops.LOSS_TYPES:
         raise ValueError(f"Unknown loss type: {loss_type}")
+    if importance_sampling_level not in ("token", "sequence"):
+        raise ValueError(
+            f"Unknown importance sampling level: {importance_sampling_level}. Possible values are 'token' "
+            "and 'sequence'."
+        )
     if beta != 0.0 and ref_per_token_logps is None:
         raise KeyError("ref_per_token_logps")
+    seq_level = importance_sampling_level == "sequence"
+    if seq_level and advantages.dim() == 2 and advantages.shape[1] != 1:
+        raise NotImplementedError("sequence-level importance weights with per-token advantages are not implemented")
+    if loss_type == "luspo" and (not seq_level or beta != 0.0 or token_weight is not None):
+        # the reference then averages a [B, T] tensor over padding as well; only the (B, 1) form is built here
+        raise NotImplementedError(
+            "luspo is implemented for importance_sampling_level='sequence' without KL term or per-token weights")
+    reduce_code, term_code = ops.LOSS_TYPES[loss_type]
     dev = per_token_logps.device
+    seq_coef = None
+    if loss_type == "vespo":
+        old = per_token_logps.detach() if old_per_token_logps is None else old_per_token_logps
+        adv2 = advantages.unsqueeze(1) if advantages.dim() == 1 else advantages
+        if adv2.shape[1] != 1:
+            raise NotImplementedError("vespo with per-token advantages is not implemented")
+        seq_coef = get_gamma_weights(adv2.float(), per_token_logps.detach().float() - old.float(), mask.float(),
+                                     importance_sampling_ratio, *vespo_params)
     dapo_norm = None
     dr_denominator = 1.0
-    if loss_type == "dapo":
+    if reduce_code == _lib.DAPO:
         if num_items_in_batch is None:
             raise KeyError("num_items_in_batch")
         dapo_norm = (
@@ -126,9 +176,10 @@ def grpo_loss(
         dr_denominator = float(per_token_logps.shape[0] * max_completion_length)
     loss, metrics, _, _ = ops.grpo_loss_op(
         per_token_logps, old_per_token_logps, ref_per_token_logps if beta != 0.0 else None, entropies, advantages,
-        mask, token_weight, entropy_mask, dapo_norm, ops.LOSS_TYPES[loss_type], float(epsilon_low),
+        mask, token_weight, entropy_mask, dapo_norm, reduce_code, float(epsilon_low),
         float(epsilon_high), math.nan if delta is None else float(delta), float(beta), bool(use_bias_correction_kl),
-        float(grad_accum_steps), dr_denominator, float(num_processes), float(entropy_coef),
+        float(grad_accum_steps), dr_denominator, float(num_processes), float(entropy_coef), term_code, seq_level,
+        seq_coef, float(sapo_temperature_pos), float(sapo_temperature_neg),
     )
     return loss, metrics
 
@@ -174,12 +225,10 @@ class GRPOLossMixin:
         return logps, entropies, aux_loss
 
     def _compute_loss(self, model, inputs):
-        """Reference: trl/trainer/grpo_trainer.py:2991-3260 for loss types grpo / bnpo / dr_grpo / dapo
-        with token-level importance weights."""
+        """Reference: trl/trainer/grpo_trainer.py:2991-3260, every loss type, token- and sequence-level
+        importance weights; adaptive entropy control is left to the reference."""
         if self.loss_type not in ops.LOSS_TYPES:
-            raise NotImplementedError(f"loss_type={self.loss_type!r} is not implemented by trl_amd")
-        if self.importance_sampling_level != "token":
-            raise NotImplementedError("importance_sampling_level='sequence' is not implemented by trl_amd")
+            raise ValueError(f"Unknown loss type: {self.loss_type}")
         if getattr(self, "use_adaptive_entropy", False):
             raise NotImplementedError("adaptive entropy control is not implemented by trl_amd")
         prompt_ids, prompt_mask = inputs["prompt_ids"], inputs["prompt_mask"]
@@ -212,7 +261,7 @@ class GRPOLossMixin:
         if entropy_mask is not None:
             em = entropy_mask.float()
             token_weight = em if token_weight is None else token_weight * em
-        if self.use_vllm and self.vllm_importance_sampling_correction:
+        if self.use_vllm and self.vllm_importance_sampling_correction and self.loss_type != "vespo":
             isr = inputs["importance_sampling_ratio"].float().expand_as(per_token_logps)
             token_weight = isr if token_weight is None else token_weight * isr
 
@@ -228,6 +277,12 @@ class GRPOLossMixin:
             grad_accum_steps=grad_accum, use_bias_correction_kl=self.args.use_bias_correction_kl,
             token_weight=token_weight, entropy_mask=None if entropy_mask is None else entropy_mask.float(),
             entropy_coef=self.entropy_coef if bonus else 0.0,
+            importance_sampling_level=self.importance_sampling_level,
+            sapo_temperature_pos=getattr(self.args, "sapo_temperature_pos", 1.0),
+            sapo_temperature_neg=getattr(self.args, "sapo_temperature_neg", 1.05),
+            vespo_params=(getattr(self.args, "vespo_k_pos", 2.0), getattr(self.args, "vespo_lambda_pos", 3.0),
+                          getattr(self.args, "vespo_k_neg", 3.0), getattr(self.args, "vespo_lambda_neg", 2.0)),
+            importance_sampling_ratio=inputs.get("importance_sampling_ratio"),
         )
         if aux_enabled:
             loss = loss + self.router_aux_loss_coef * aux_loss / grad_accum
@@ -235,14 +290,15 @@ class GRPOLossMixin:
 
         # metrics: cross-process sums of (sum, count) pairs, then one host copy
         m = metrics.detach()
-        sums = torch.stack([m[_lib_metric("KL_SUM")], m[_lib_metric("ENTROPY_SUM")], m[_lib_metric("MASK_SUM")]])
-        clip = m[2:5] * m[_lib_metric("MASK_SUM")].clamp(min=1.0)
+        i = _METRIC_INDEX
+        sums = m[[i["KL_SUM"], i["ENTROPY_SUM"], i["MASK_SUM"], i["CLIP_COUNT"], i["AUX_SUM"], i["AUX_COUNT"]]]
+        clip = m[2:5] * m[i["CLIP_COUNT"]].clamp(min=1.0)
         totals = self.accelerator.reduce(torch.cat([sums, clip]), reduction="sum")
         low_min = nanmin(self.accelerator.gather(m[5:6]))
         high_max = nanmax(self.accelerator.gather(m[6:7]))
         host = torch.cat([totals, low_min.reshape(1), high_max.reshape(1), m[7:8]]).tolist()
-        kl_sum, ent_sum, cnt, low, high, region, lmin, hmax, policy_loss = host
-        cnt = max(cnt, 1.0)
+        kl_sum, ent_sum, cnt, clip_cnt, aux_sum, aux_cnt, low, high, region, lmin, hmax, policy_loss = host
+        cnt, clip_cnt, aux_cnt = max(cnt, 1.0), max(clip_cnt, 1.0), max(aux_cnt, 1.0)
         log = self._metrics[mode]
         if bonus:
             log["policy_loss"].append(policy_loss)
@@ -251,34 +307,42 @@ class GRPOLossMixin:
         if self.beta != 0.0:
             log["kl"].append(kl_sum / cnt)
         log["entropy"].append(ent_sum / cnt)
-        log["clip_ratio/low_mean"].append(low / cnt)
-        log["clip_ratio/high_mean"].append(high / cnt)
-        log["clip_ratio/region_mean"].append(region / cnt)
-        log["clip_ratio/low_min"].append(lmin)
-        log["clip_ratio/high_max"].append(hmax)
+        if self.loss_type in ("grpo", "bnpo", "dr_grpo", "dapo", "luspo"):
+            log["clip_ratio/low_mean"].append(low / clip_cnt)
+            log["clip_ratio/high_mean"].append(high / clip_cnt)
+            log["clip_ratio/region_mean"].append(region / clip_cnt)
+            log["clip_ratio/low_min"].append(lmin)
+            log["clip_ratio/high_max"].append(hmax)
+        elif self.loss_type == "cispo":
+            log["cispo_clip_ratio"].append(aux_sum / aux_cnt)
+        elif self.loss_type == "vespo":
+            log["vespo/phi_seq_mean"].append(aux_sum / aux_cnt)
         return loss
 
 
 _METRIC_INDEX = {"KL_MEAN": 0, "ENTROPY_MEAN": 1, "CLIP_LOW_MEAN": 2, "CLIP_HIGH_MEAN": 3, "CLIP_REGION_MEAN": 4,
-                 "CLIP_LOW_MIN": 5, "CLIP_HIGH_MAX": 6, "POLICY_LOSS": 7, "MASK_SUM": 8, "KL_SUM": 9, "ENTROPY_SUM": 10}
+                 "CLIP_LOW_MIN": 5, "CLIP_HIGH_MAX": 6, "POLICY_LOSS": 7, "MASK_SUM": 8, "KL_SUM": 9, "ENTROPY_SUM": 10,
+                 "AUX_MEAN": 11, "CLIP_COUNT": 12, "AUX_SUM": 13, "AUX_COUNT": 14}
 
 
-def _lib_metric(name: str) -> int:
-    return _METRIC_INDEX[name]
-
-
-def metrics_to_dict(metrics: Tensor, beta: float, has_entropy: bool = True) -> dict[str, float]:
+def metrics_to_dict(metrics: Tensor, beta: float, has_entropy: bool = True, loss_type: str = "dapo") -> dict[str, float]:
     """Host dictionary with the reference's metric names (single device->host copy)."""
     m = metrics.detach().tolist()
+    i = _METRIC_INDEX
     out = {}
     if beta != 0.0:
-        out["kl"] = m[0]
+        out["kl"] = m[i["KL_MEAN"]]
     if has_entropy:
-        out["entropy"] = m[1]
-    out["clip_ratio/low_mean"] = m[2]
-    out["clip_ratio/high_mean"] = m[3]
-    out["clip_ratio/region_mean"] = m[4]
-    out["clip_ratio/low_min"] = m[5]
-    out["clip_ratio/high_max"] = m[6]
-    out["policy_loss"] = m[7]
+        out["entropy"] = m[i["ENTROPY_MEAN"]]
+    if loss_type == "cispo":
+        out["cispo_clip_ratio"] = m[i["AUX_MEAN"]]
+    elif loss_type == "vespo":
+        out["vespo/phi_seq_mean"] = m[i["AUX_MEAN"]]
+    elif loss_type != "sapo":
+        out["clip_ratio/low_mean"] = m[i["CLIP_LOW_MEAN"]]
+        out["clip_ratio/high_mean"] = m[i["CLIP_HIGH_MEAN"]]
+        out["clip_ratio/region_mean"] = m[i["CLIP_REGION_MEAN"]]
+        out["clip_ratio/low_min"] = m[i["CLIP_LOW_MIN"]]
+        out["clip_ratio/high_max"] = m[i["CLIP_HIGH_MAX"]]
+    out["policy_loss"] = m[i["POLICY_LOSS"]]
     return out
