@@ -23,6 +23,8 @@
 // registers, so dz goes through a chunk-sized workspace (never the whole [N, V] matrix).
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace trlk {
 namespace {
 
@@ -57,8 +59,10 @@ constexpr int kRowStep = kHeadThreads / kCpr;       // rows staged per pass of t
 constexpr int kLoadsA = BM / kRowStep, kLoadsB = BN / kRowStep;
 constexpr int kTileABytes = BM * kLdsRow * 2, kTileBBytes = BN * kLdsRow * 2;
 constexpr int kStageBytes = kTileABytes + kTileBBytes;
-constexpr int kHeadLdsBytes = 2 * kStageBytes;  // two stages
+constexpr int kDirectLdsBytesDecl = 2 * (BM + BN) * 64 * 2;  // direct-to-LDS tile ring: 4 x 32-wide or 2 x 64-wide stages
 constexpr int kDzLdsRow = BM * 2 + 16;     // bytes per token row of the dz tile staged in LDS by the backward
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
+constexpr int kHeadLdsBytes = cmax(cmax(2 * kStageBytes, kDirectLdsBytesDecl), BN * kDzLdsRow);
 static_assert(BN * kDzLdsRow <= kHeadLdsBytes, "dz staging tile");
 static_assert(2 * WGM * BN * 4 * 4 <= kHeadLdsBytes && BN <= kHeadThreads, "merge scratch");
 static_assert(BM % kRowStep == 0 && BN % kRowStep == 0 && WM % 32 == 0 && WN % 32 == 0 && BK % 16 == 0, "tile shape");
@@ -87,66 +91,106 @@ struct Operand {
 #ifndef TRLK_HEAD_DIRECT_LDS
 #define TRLK_HEAD_DIRECT_LDS 1
 #endif
+// k-step width of the direct-to-LDS loop per kernel: the short contraction over the hidden size
+// (forward, recompute) gains from the deeper ring of 32-wide steps, the long contractions of the
+// two backward products from 64-wide steps with half as many barriers.
+#ifndef TRLK_HEAD_BK_FWD
+#define TRLK_HEAD_BK_FWD 32
+#endif
+#ifndef TRLK_HEAD_BK_DZ
+#define TRLK_HEAD_BK_DZ 32
+#endif
+#ifndef TRLK_HEAD_BK_GEMM
+#define TRLK_HEAD_BK_GEMM 64
+#endif
 
-// Direct-to-LDS variant of the tile loop (K % 64 == 0): `global_load_lds_dwordx4` moves 16 bytes per
-// lane from memory straight into LDS, 1 KiB contiguous per wave instruction = 8 tile rows of 128
-// bytes, with no register staging and no ds_write.  Rows are dense (no padding is possible inside a
+// Direct-to-LDS variant of the tile loop (K % BK == 0): `global_load_lds_dwordx4` moves 16 bytes per
+// lane from memory straight into LDS, 1 KiB contiguous per wave instruction = 1024 / (2 BK) tile
+// rows, with no register staging and no ds_write.  Rows are dense (no padding is possible inside a
 // wave's 1 KiB), so bank conflicts are avoided by an XOR swizzle of the 16-byte chunk index: the
-// chunk at physical position pc of row r holds logical chunk pc ^ (r & 7) ^ ((r >> 3) & 1).  The
-// lane fetches that logical chunk from memory (a permutation inside one 128-byte line, still
-// coalesced) and the fragment reads apply the same XOR.
-template <int DT>
+// chunk at physical position pc of row r holds logical chunk pc ^ swz(r), with
+//   BK = 64 (128-byte rows): swz(r) = (r & 7) ^ ((r >> 3) & 1),   BK = 32 (64-byte rows): swz(r) = (r >> 2) & 3,
+// which makes the 16 rows that one ds_read_b128 phase touches cover all 64 banks once.  The lane
+// fetches that logical chunk from memory (a permutation inside one row, still coalesced) and the
+// fragment reads apply the same XOR.
+//
+// The loop keeps kStages tiles in LDS (4 x 32 KiB for BK = 32, 2 x 64 KiB for BK = 64).  A stage is
+// refilled as soon as the barrier that ends its last use has passed, kStages - 1 steps before it
+// is needed again: the transfer of one stage through the CU's vector memory path (64 bytes per
+// clock) takes longer than half a k step of MFMAs, so with only two stages every barrier waits
+// for data in flight.
+template <int BKT>
+struct DirectCfg {
+    static_assert(BKT == 32 || BKT == 64, "direct-to-LDS layouts exist for 32- and 64-wide k steps");
+    static constexpr int kStages = BKT == 32 ? 4 : 2;
+    static constexpr int kRowBytes = BKT * 2;                // dense LDS row
+    static constexpr int kRowsPerBlk = 1024 / kRowBytes;     // rows one wave instruction fills
+    static constexpr int kChunks = kRowBytes / 16;
+    static constexpr int kDenseA = BM * kRowBytes, kDenseStage = (BM + BN) * kRowBytes;
+    static constexpr int kLdsBytes = kStages * kDenseStage;
+    static __device__ __forceinline__ int swizzle(int r) {
+        return BKT == 64 ? ((r & 7) ^ ((r >> 3) & 1)) : ((r >> 2) & 3);
+    }
+};
+static_assert(DirectCfg<32>::kLdsBytes <= kHeadLdsBytes && DirectCfg<64>::kLdsBytes <= kHeadLdsBytes, "LDS budget");
+
+template <int DT, int BKT>
 __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, const Operand B, int n0, int K,
                                                     f32x16 (&acc)[MB][NB], char* smem) {
-    static_assert(BK == 64, "the direct-to-LDS layout assumes 128-byte tile rows");
+    typedef DirectCfg<BKT> C;
+    constexpr int kStages = C::kStages, kRowBytes = C::kRowBytes, kRowsPerBlk = C::kRowsPerBlk, kChunks = C::kChunks;
+    constexpr int kDenseA = C::kDenseA, kDenseStage = C::kDenseStage;
     constexpr int kWaves = kHeadThreads / 64;
-    constexpr int kBlkA = BM / 8 / kWaves, kBlkB = BN / 8 / kWaves;  // 8-row blocks per wave and stage
-    constexpr int kDenseA = BM * BK * 2, kDenseStage = (BM + BN) * BK * 2;
-    static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0, "blocks per wave");
+    constexpr int kBlkA = BM / kRowsPerBlk / kWaves, kBlkB = BN / kRowsPerBlk / kWaves;  // blocks per wave and stage
+    static_assert(BM % (kRowsPerBlk * kWaves) == 0 && BN % (kRowsPerBlk * kWaves) == 0, "blocks per wave");
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: LDS targets stay scalar
     const int wm = wave / WGN, wn = wave % WGN;
 
     // --- loader side: this lane's row inside a block and the logical chunk it fetches
-    const int rr = lane >> 3, pc = lane & 7;
-    const int kc = pc ^ rr ^ (wave & 1);  // blocks of a wave all have the parity of the wave index
+    const int rr = lane / kChunks, pc = lane % kChunks;
     const char* abase = reinterpret_cast<const char*>(A.p + int64_t(m0) * A.ld);
     const char* bbase = reinterpret_cast<const char*>(B.p + int64_t(n0) * B.ld);
     uint32_t ao[kBlkA], bo[kBlkB];
 #pragma unroll
     for (int j = 0; j < kBlkA; ++j) {
-        int r = (wave + kWaves * j) * 8 + rr;
-        r = m0 + r < A.rows ? r : A.rows - 1 - m0;
+        const int row = (wave + kWaves * j) * kRowsPerBlk + rr;
+        const int kc = pc ^ C::swizzle(row);
+        const int r = m0 + row < A.rows ? row : A.rows - 1 - m0;
         ao[j] = uint32_t((int64_t(r) * A.ld + kc * 8) * 2);
     }
 #pragma unroll
     for (int j = 0; j < kBlkB; ++j) {
-        int r = (wave + kWaves * j) * 8 + rr;
-        r = n0 + r < B.rows ? r : B.rows - 1 - n0;
+        const int row = (wave + kWaves * j) * kRowsPerBlk + rr;
+        const int kc = pc ^ C::swizzle(row);
+        const int r = n0 + row < B.rows ? row : B.rows - 1 - n0;
         bo[j] = uint32_t((int64_t(r) * B.ld + kc * 8) * 2);
     }
     typedef __attribute__((address_space(1))) const void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    auto issue_stage = [&](int buf, int k0) {
+    auto issue_a = [&](int buf, int k0) {
         const char* ap = abase + int64_t(k0) * 2;
-        const char* bp = bbase + int64_t(k0) * 2;
         char* sa = smem + buf * kDenseStage;
-        char* sb = sa + kDenseA;
 #pragma unroll
         for (int j = 0; j < kBlkA; ++j)
             __builtin_amdgcn_global_load_lds((gptr_t)(ap + ao[j]), (lptr_t)(sa + (wave + kWaves * j) * 1024), 16, 0, 0);
+    };
+    auto issue_b = [&](int buf, int k0) {
+        const char* bp = bbase + int64_t(k0) * 2;
+        char* sb = smem + buf * kDenseStage + kDenseA;
 #pragma unroll
         for (int j = 0; j < kBlkB; ++j)
             __builtin_amdgcn_global_load_lds((gptr_t)(bp + bo[j]), (lptr_t)(sb + (wave + kWaves * j) * 1024), 16, 0, 0);
     };
 
-    // --- fragment side
-    const int swz = (lane & 7) ^ ((lane >> 3) & 1);
+    // --- fragment side (tile rows of a wave start at multiples of 32, so the swizzle depends on the lane only)
+    const int swz = C::swizzle(lane & 31);
     const int hl = lane >> 5;
-    const int fa_row = (wm * WM + (lane & 31)) * 128, fb_row = (wn * WN + (lane & 31)) * 128;
-    int koff[BK / 16];
+    const int fa_row = (wm * WM + (lane & 31)) * kRowBytes, fb_row = (wn * WN + (lane & 31)) * kRowBytes;
+    constexpr int KS = BKT / 16;
+    int koff[KS];
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) koff[ks] = ((ks * 2 + hl) ^ swz) * 16;
+    for (int ks = 0; ks < KS; ++ks) koff[ks] = ((ks * 2 + hl) ^ swz) * 16;
 
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -155,42 +199,107 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0.f;
 
-    // Fragment loads run one 16-wide k slice ahead of the MFMAs that consume them, so the LDS
-    // latency of slice ks+1 hides behind the 8 MFMAs of slice ks.
-    auto load_frags = [&](const char* sa, const char* sb, int ks, u32x4(&fa)[MB], u32x4(&fb)[NB]) {
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-            fa[mb] = *reinterpret_cast<const u32x4*>(sa + fa_row + mb * 32 * 128 + koff[ks]);
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-            fb[nb] = *reinterpret_cast<const u32x4*>(sb + fb_row + nb * 32 * 128 + koff[ks]);
-    };
-    auto compute = [&](int buf) {
+    // Software pipeline.  Fragment loads run one 16-wide k slice ahead of the MFMAs that consume them,
+    // across the barrier too: the last slice of a stage is already in registers when the workgroup
+    // synchronises, so its MFMAs cover the refill of the freed stage and the first fragment reads of
+    // the next one.  The compiler's own scheduler sinks every ds_read next to its first use (one
+    // exposed LDS latency per MFMA pair); the sched_group_barrier sequences pin the interleaving.
+    constexpr int kStageLoads = kBlkA + kBlkB;
+    auto load_frags = [&](int buf, int ks, u32x4(&fa)[MB], u32x4(&fb)[NB]) {
         const char* sa = smem + buf * kDenseStage;
         const char* sb = sa + kDenseA;
-        u32x4 fa[2][MB], fb[2][NB];
-        load_frags(sa, sb, 0, fa[0], fb[0]);
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            if (ks + 1 < BK / 16) load_frags(sa, sb, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+        for (int mb = 0; mb < MB; ++mb)
+            fa[mb] = *reinterpret_cast<const u32x4*>(sa + fa_row + mb * 32 * kRowBytes + koff[ks]);
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
+        for (int nb = 0; nb < NB; ++nb)
+            fb[nb] = *reinterpret_cast<const u32x4*>(sb + fb_row + nb * 32 * kRowBytes + koff[ks]);
+    };
+    auto mfma_all = [&](u32x4(&fa)[MB], u32x4(&fb)[NB]) {
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = mfma<DT>(fa[ks & 1][mb], fb[ks & 1][nb], acc[mb][nb]);
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = mfma<DT>(fa[mb], fb[nb], acc[mb][nb]);
+    };
+    // Issue order of one slice: an MFMA, a fragment read, ... with the slice's `loads` tile transfers
+    // spread evenly between the MFMAs (a burst of transfers would block the wave, and with it its
+    // MFMAs, until the vector memory path has taken them all: it accepts one per 16 clocks).
+    auto interleave = [&](auto reads_tag, auto loads_tag) {
+        constexpr int R = decltype(reads_tag)::value, L = decltype(loads_tag)::value, M = MB * NB;
+#pragma unroll
+        for (int i = 0; i < M; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // MFMA
+            if (i < R) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+            if (L > 0 && (i + 1) * L / M > i * L / M) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);  // VMEM
         }
     };
+    typedef std::integral_constant<int, MB + NB> reads_t;
+    typedef std::integral_constant<int, kStageLoads> loads_t;
+    typedef std::integral_constant<int, 0> none_t;
+    u32x4 fa[2][MB], fb[2][NB];
+    // One k step.  ISSUE: the stage this step frees at its barrier is refilled, right behind that
+    // barrier, with the tile kStages steps ahead.  FULL: kStages - 2 younger stages are in flight
+    // behind the one the next step needs.  NEXT: there is a following step.
+    auto step = [&](int kt, auto issue_tag, auto full_tag, auto next_tag) {
+        constexpr bool ISSUE = decltype(issue_tag)::value, FULL = decltype(full_tag)::value;
+        constexpr bool NEXT = decltype(next_tag)::value;
+        const int cur = kt & (kStages - 1);
+#pragma unroll
+        for (int ks = 0; ks + 1 < KS; ++ks) {
+            load_frags(cur, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+            mfma_all(fa[ks & 1], fb[ks & 1]);
+            interleave(reads_t{}, none_t{});
+        }
+        // every fragment read of this stage has returned and the next stage has landed
+        if constexpr (FULL)
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((kStages - 2) * kStageLoads) : "memory");
+        else
+            __builtin_amdgcn_s_waitcnt(0);
+        // A bare s_barrier: __syncthreads() carries release/acquire fences, for which the compiler
+        // drains every outstanding transfer (vmcnt(0)), younger stages included.  The waits above
+        // are the ones this exchange needs; nothing may move across the barrier.
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("" ::: "memory");
+        if constexpr (NEXT) load_frags((kt + 1) & (kStages - 1), 0, fa[0], fb[0]);
+        mfma_all(fa[(KS - 1) & 1], fb[(KS - 1) & 1]);
+        if constexpr (ISSUE) {
+            issue_a(cur, (kt + kStages) * BKT);
+            issue_b(cur, (kt + kStages) * BKT);
+        }
+        if constexpr (NEXT && ISSUE)
+            interleave(reads_t{}, loads_t{});
+        else if constexpr (NEXT)
+            interleave(reads_t{}, none_t{});
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    static_assert(KS % 2 == 0 && MB * NB > MB + NB && (kStages - 2) * kStageLoads < 64, "pipeline shape");
+    constexpr std::true_type T{};
+    constexpr std::false_type F{};
 
-    const int nk = K / BK;
-    issue_stage(0, 0);
-    __builtin_amdgcn_s_waitcnt(0);
+    const int nk = K / BKT;
+#pragma unroll
+    for (int st = 0; st < kStages; ++st)
+        if (st < nk) {
+            issue_a(st, st * BKT);
+            issue_b(st, st * BKT);
+        }
+    if (nk >= kStages)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 1) * kStageLoads) : "memory");
+    else
+        __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        // the other buffer was last read before the previous barrier: refill it asynchronously now
-        if (kt + 1 < nk) issue_stage((kt + 1) & 1, (kt + 1) * BK);
-        compute(kt & 1);
-        __builtin_amdgcn_s_waitcnt(0);  // this wave's transfers have landed in LDS
-        __syncthreads();                // ... and so have everyone else's; all reads of this buffer are done
+    load_frags(0, 0, fa[0], fb[0]);
+    int kt = 0;
+    if (nk >= kStages) {
+        for (; kt + kStages < nk; ++kt) step(kt, T, T, T);
+        step(kt++, F, T, T);  // kt = nk - kStages: every stage has been requested
     }
+    for (; kt + 1 < nk; ++kt) step(kt, F, F, T);
+    step(kt, F, F, F);
+    // every LDS read of this tile completed before the last barrier: the caller may reuse the LDS right away
 }
 
 // acc[mb][nb] = sum_k A[m0 + .., k] * B[n0 + .., k].  Rows beyond the operand's end are clamped to
@@ -291,12 +400,12 @@ __device__ __forceinline__ void gemm_tile_nt_staged(const Operand A, int m0, con
     }
 }
 
-template <int DT>
+template <int DT, int BKT>
 __device__ __forceinline__ void gemm_tile_nt(const Operand A, int m0, const Operand B, int n0, int K,
                                              f32x16 (&acc)[MB][NB], char* smem) {
 #if TRLK_HEAD_DIRECT_LDS
-    if ((K & (BK - 1)) == 0)
-        gemm_tile_nt_direct<DT>(A, m0, B, n0, K, acc, smem);
+    if ((K & (BKT - 1)) == 0)
+        gemm_tile_nt_direct<DT, BKT>(A, m0, B, n0, K, acc, smem);
     else
 #endif
         gemm_tile_nt_staged<DT>(A, m0, B, n0, K, acc, smem);
@@ -382,20 +491,33 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
     for (int vt = vt0; vt < vt1; ++vt) {
         const int m0 = vt * BM;
         f32x16 acc[MB][NB];
-        gemm_tile_nt<DT>(W, m0, Hd, n0, a.H, acc, smem);
+        gemm_tile_nt<DT, TRLK_HEAD_BK_FWD>(W, m0, Hd, n0, a.H, acc, smem);
         const bool partial_tile = m0 + BM > a.V;
+        // Common case (no soft-capping, tile inside the vocabulary): z = y * zs with one positive
+        // scale, so the maximum is taken on the raw accumulators and the scale is folded into the
+        // exponent's multiplier; sum(e * z) is accumulated as zs * sum(e * y).
+        const float zs = a.logit_scale * a.inv_t, zs2 = zs * kLog2e;
+        const bool plain = a.softcap <= 0.f && !partial_tile && zs > 0.f;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             float bm = -INFINITY;
+            if (plain) {
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
+                for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    float z = head_z(acc[mb][nb][r], a);
-                    if (partial_tile && m0 + acc_row(wm, mb, r, lane) >= a.V) z = -INFINITY;
-                    acc[mb][nb][r] = z;
-                    bm = fmaxf(bm, z);
-                }
+                    for (int r = 0; r < 16; ++r) bm = fmaxf(bm, acc[mb][nb][r]);
+                bm *= zs;
+            } else {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        float z = head_z(acc[mb][nb][r], a);
+                        if (partial_tile && m0 + acc_row(wm, mb, r, lane) >= a.V) z = -INFINITY;
+                        acc[mb][nb][r] = z;
+                        bm = fmaxf(bm, z);
+                    }
+            }
             zmax[nb] = fmaxf(zmax[nb], bm);
             const float need = ceilf(bm * kLog2e);
             if (need > ref[nb]) {
@@ -406,15 +528,28 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
                 rr[nb] = need;
             }
             float s = 0.f, u = 0.f;
+            if (plain) {
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
+                for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float z = acc[mb][nb][r];
-                    const float e = fast_exp2(fmaf(z, kLog2e, -rr[nb]));
-                    s += e;
-                    u = (z == -INFINITY) ? u : fmaf(e, z, u);
-                }
+                    for (int r = 0; r < 16; ++r) {
+                        const float y = acc[mb][nb][r];
+                        const float e = fast_exp2(fmaf(y, zs2, -rr[nb]));
+                        s += e;
+                        u = fmaf(e, y, u);
+                    }
+                u *= zs;
+            } else {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const float z = acc[mb][nb][r];
+                        const float e = fast_exp2(fmaf(z, kLog2e, -rr[nb]));
+                        s += e;
+                        u = (z == -INFINITY) ? u : fmaf(e, z, u);
+                    }
+            }
             S[nb] += s;
             U[nb] += u;
             // target logit: rarely inside this wave's 128 vocabulary rows
@@ -424,7 +559,8 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
-                        if (acc_row(0, mb, r, lane) == int(rel)) a.tgt[n0 + acc_col(wn, nb, lane)] = acc[mb][nb][r];
+                        if (acc_row(0, mb, r, lane) == int(rel))
+                            a.tgt[n0 + acc_col(wn, nb, lane)] = plain ? acc[mb][nb][r] * zs : acc[mb][nb][r];
             }
         }
     }
@@ -518,7 +654,7 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
     const int n0 = tb * BN, m0 = a.c0 + vt * BM;
     const Operand W{a.weight, a.ldw, a.V}, Hd{a.hidden, a.ldh, a.N};
     f32x16 acc[MB][NB];
-    gemm_tile_nt<DT>(W, m0, Hd, n0, a.H, acc, smem);
+    gemm_tile_nt<DT, TRLK_HEAD_BK_DZ>(W, m0, Hd, n0, a.H, acc, smem);
 
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
@@ -601,7 +737,7 @@ TRLK_HEAD_KERNEL void gemm_nt_kernel(GemmArgs a) {
     const int wm = wave / WGN, wn = wave % WGN;
     const int m0 = tm * BM, n0 = tn * BN;
     f32x16 acc[MB][NB];
-    gemm_tile_nt<DT>(a.A, m0, a.B, n0, a.K, acc, smem);
+    gemm_tile_nt<DT, TRLK_HEAD_BK_GEMM>(a.A, m0, a.B, n0, a.K, acc, smem);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
