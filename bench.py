@@ -108,6 +108,12 @@ def cpu_baseline(w, loss_type, rows_per_seq=512, n_seq=32, repeats=2):
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
 
 
+# Vocabulary rows per backward chunk of the fused head.  The operator's `chunk_size` only sizes the
+# dz workspace (2 x N x chunk bf16); 32768 rows = 4.3 GB at this shape, a small share of the card's
+# HBM, and leaves 5 chunks instead of 19 (fewer partial waves and dHidden accumulation passes).
+HEAD_CHUNK = 32768
+
+
 def bench_head(args, w):
     """BASELINE.json config 5: the logits are never materialised.  Step = fused head forward, GRPO loss,
     fused head backward (dHidden and dW)."""
@@ -133,7 +139,7 @@ def bench_head(args, w):
 
     def step():
         hidden.grad = weight.grad = None
-        lp, ent = trl_amd._ChunkedLogProbFunction.apply(hidden, weight, targets, w["temperature"], 8192)
+        lp, ent = trl_amd._ChunkedLogProbFunction.apply(hidden, weight, targets, w["temperature"], HEAD_CHUNK)
         loss, _ = trl_amd.grpo_loss(lp.view(B, T), adv, mask, entropies=ent.view(B, T), old_per_token_logps=old,
                                     ref_per_token_logps=ref, loss_type=args.loss_type, epsilon_low=w["eps_low"],
                                     epsilon_high=w["eps_high"], beta=w["beta"], max_completion_length=T,
@@ -168,7 +174,7 @@ def bench_head(args, w):
         _, _, log_z, _ = ops.fused_head_fwd(hidden, weight, targets, w["temperature"], 0.0, 1.0)
         gl = torch.randn((N,), generator=g, device=dev)
         fwd_ms = time_op(lambda: ops.fused_head_fwd(hidden, weight, targets, w["temperature"], 0.0, 1.0))
-        bwd_ms = time_op(lambda: ops.fused_head_bwd(hidden, weight, targets, w["temperature"], 0.0, 1.0, log_z, gl, 8192))
+        bwd_ms = time_op(lambda: ops.fused_head_bwd(hidden, weight, targets, w["temperature"], 0.0, 1.0, log_z, gl, HEAD_CHUNK))
     flop = 2.0 * N * H * V
     fwd_tf, bwd_tf = flop / (fwd_ms * 1e-3) / 1e12, 3 * flop / (bwd_ms * 1e-3) / 1e12
     total_tf = 4 * flop / ((fwd_ms + bwd_ms) * 1e-3) / 1e12
@@ -178,6 +184,7 @@ def bench_head(args, w):
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": args.workload, "description": w["desc"], "tokens": N, "hidden": H, "vocab": V,
+                   "backward_chunk_rows": HEAD_CHUNK,
                    "loss_type": args.loss_type, "loss": float(loss.detach())},
         "roofline": {"bound": "mfma", "kernel": "fused head forward + backward (all MFMA kernels)",
                      "achieved": total_tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",

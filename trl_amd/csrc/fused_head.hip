@@ -134,54 +134,76 @@ struct DirectCfg {
 };
 static_assert(DirectCfg<32>::kLdsBytes <= kHeadLdsBytes && DirectCfg<64>::kLdsBytes <= kHeadLdsBytes, "LDS budget");
 
-template <int DT, int BKT>
-__device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, const Operand B, int n0, int K,
-                                                    f32x16 (&acc)[MB][NB], char* smem) {
+// Loader side of the direct-to-LDS loop: per-lane source offsets of the wave's tile blocks and the
+// transfer of one stage.
+template <int BKT>
+struct DirectLoader {
     typedef DirectCfg<BKT> C;
-    constexpr int kStages = C::kStages, kRowBytes = C::kRowBytes, kRowsPerBlk = C::kRowsPerBlk, kChunks = C::kChunks;
-    constexpr int kDenseA = C::kDenseA, kDenseStage = C::kDenseStage;
-    constexpr int kWaves = kHeadThreads / 64;
-    constexpr int kBlkA = BM / kRowsPerBlk / kWaves, kBlkB = BN / kRowsPerBlk / kWaves;  // blocks per wave and stage
-    static_assert(BM % (kRowsPerBlk * kWaves) == 0 && BN % (kRowsPerBlk * kWaves) == 0, "blocks per wave");
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: LDS targets stay scalar
-    const int wm = wave / WGN, wn = wave % WGN;
-
-    // --- loader side: this lane's row inside a block and the logical chunk it fetches
-    const int rr = lane / kChunks, pc = lane % kChunks;
-    const char* abase = reinterpret_cast<const char*>(A.p + int64_t(m0) * A.ld);
-    const char* bbase = reinterpret_cast<const char*>(B.p + int64_t(n0) * B.ld);
+    static constexpr int kWaves = kHeadThreads / 64;
+    static constexpr int kBlkA = BM / C::kRowsPerBlk / kWaves, kBlkB = BN / C::kRowsPerBlk / kWaves;  // per wave and stage
+    static constexpr int kStageLoads = kBlkA + kBlkB;
+    static_assert(BM % (C::kRowsPerBlk * kWaves) == 0 && BN % (C::kRowsPerBlk * kWaves) == 0, "blocks per wave");
+    const char *abase, *bbase;
+    char* smem;
+    int wave;
     uint32_t ao[kBlkA], bo[kBlkB];
+
+    __device__ __forceinline__ DirectLoader(const Operand A, int m0, const Operand B, int n0, char* lds) : smem(lds) {
+        const int lane = threadIdx.x & 63;
+        wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: LDS targets stay scalar
+        const int rr = lane / C::kChunks, pc = lane % C::kChunks;  // row inside a block, chunk position
+        abase = reinterpret_cast<const char*>(A.p + int64_t(m0) * A.ld);
+        bbase = reinterpret_cast<const char*>(B.p + int64_t(n0) * B.ld);
 #pragma unroll
-    for (int j = 0; j < kBlkA; ++j) {
-        const int row = (wave + kWaves * j) * kRowsPerBlk + rr;
-        const int kc = pc ^ C::swizzle(row);
-        const int r = m0 + row < A.rows ? row : A.rows - 1 - m0;
-        ao[j] = uint32_t((int64_t(r) * A.ld + kc * 8) * 2);
-    }
+        for (int j = 0; j < kBlkA; ++j) {
+            const int row = (wave + kWaves * j) * C::kRowsPerBlk + rr;
+            const int kc = pc ^ C::swizzle(row);  // the logical chunk this lane fetches
+            const int r = m0 + row < A.rows ? row : A.rows - 1 - m0;
+            ao[j] = uint32_t((int64_t(r) * A.ld + kc * 8) * 2);
+        }
 #pragma unroll
-    for (int j = 0; j < kBlkB; ++j) {
-        const int row = (wave + kWaves * j) * kRowsPerBlk + rr;
-        const int kc = pc ^ C::swizzle(row);
-        const int r = n0 + row < B.rows ? row : B.rows - 1 - n0;
-        bo[j] = uint32_t((int64_t(r) * B.ld + kc * 8) * 2);
+        for (int j = 0; j < kBlkB; ++j) {
+            const int row = (wave + kWaves * j) * C::kRowsPerBlk + rr;
+            const int kc = pc ^ C::swizzle(row);
+            const int r = n0 + row < B.rows ? row : B.rows - 1 - n0;
+            bo[j] = uint32_t((int64_t(r) * B.ld + kc * 8) * 2);
+        }
     }
-    typedef __attribute__((address_space(1))) const void* gptr_t;
-    typedef __attribute__((address_space(3))) void* lptr_t;
-    auto issue_a = [&](int buf, int k0) {
+    __device__ __forceinline__ void issue(int buf, int k0) const {
+        typedef __attribute__((address_space(1))) const void* gptr_t;
+        typedef __attribute__((address_space(3))) void* lptr_t;
         const char* ap = abase + int64_t(k0) * 2;
-        char* sa = smem + buf * kDenseStage;
+        const char* bp = bbase + int64_t(k0) * 2;
+        char* sa = smem + buf * C::kDenseStage;
+        char* sb = sa + C::kDenseA;
 #pragma unroll
         for (int j = 0; j < kBlkA; ++j)
             __builtin_amdgcn_global_load_lds((gptr_t)(ap + ao[j]), (lptr_t)(sa + (wave + kWaves * j) * 1024), 16, 0, 0);
-    };
-    auto issue_b = [&](int buf, int k0) {
-        const char* bp = bbase + int64_t(k0) * 2;
-        char* sb = smem + buf * kDenseStage + kDenseA;
 #pragma unroll
         for (int j = 0; j < kBlkB; ++j)
             __builtin_amdgcn_global_load_lds((gptr_t)(bp + bo[j]), (lptr_t)(sb + (wave + kWaves * j) * 1024), 16, 0, 0);
-    };
+    }
+    // the first kStages tiles of a product; every stage must be free (all reads of the LDS done)
+    __device__ __forceinline__ void prologue(int K) const {
+        const int nk = K / BKT;
+#pragma unroll
+        for (int st = 0; st < C::kStages; ++st)
+            if (st < nk) issue(st, st * BKT);
+    }
+};
+
+// `prefetched`: the caller has already run DirectLoader::prologue for this tile (and nothing has
+// touched the LDS since).
+template <int DT, int BKT>
+__device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, const Operand B, int n0, int K,
+                                                    f32x16 (&acc)[MB][NB], char* smem, bool prefetched) {
+    typedef DirectCfg<BKT> C;
+    constexpr int kStages = C::kStages, kRowBytes = C::kRowBytes;
+    constexpr int kDenseA = C::kDenseA, kDenseStage = C::kDenseStage;
+    const DirectLoader<BKT> loader(A, m0, B, n0, smem);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = loader.wave;
+    const int wm = wave / WGN, wn = wave % WGN;
 
     // --- fragment side (tile rows of a wave start at multiples of 32, so the swizzle depends on the lane only)
     const int swz = C::swizzle(lane & 31);
@@ -204,7 +226,7 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
     // synchronises, so its MFMAs cover the refill of the freed stage and the first fragment reads of
     // the next one.  The compiler's own scheduler sinks every ds_read next to its first use (one
     // exposed LDS latency per MFMA pair); the sched_group_barrier sequences pin the interleaving.
-    constexpr int kStageLoads = kBlkA + kBlkB;
+    constexpr int kStageLoads = DirectLoader<BKT>::kStageLoads;
     auto load_frags = [&](int buf, int ks, u32x4(&fa)[MB], u32x4(&fb)[NB]) {
         const char* sa = smem + buf * kDenseStage;
         const char* sb = sa + kDenseA;
@@ -265,10 +287,7 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
         asm volatile("" ::: "memory");
         if constexpr (NEXT) load_frags((kt + 1) & (kStages - 1), 0, fa[0], fb[0]);
         mfma_all(fa[(KS - 1) & 1], fb[(KS - 1) & 1]);
-        if constexpr (ISSUE) {
-            issue_a(cur, (kt + kStages) * BKT);
-            issue_b(cur, (kt + kStages) * BKT);
-        }
+        if constexpr (ISSUE) loader.issue(cur, (kt + kStages) * BKT);
         if constexpr (NEXT && ISSUE)
             interleave(reads_t{}, loads_t{});
         else if constexpr (NEXT)
@@ -280,12 +299,7 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
     constexpr std::false_type F{};
 
     const int nk = K / BKT;
-#pragma unroll
-    for (int st = 0; st < kStages; ++st)
-        if (st < nk) {
-            issue_a(st, st * BKT);
-            issue_b(st, st * BKT);
-        }
+    if (!prefetched) loader.prologue(K);
     if (nk >= kStages)
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 1) * kStageLoads) : "memory");
     else
@@ -402,13 +416,22 @@ __device__ __forceinline__ void gemm_tile_nt_staged(const Operand A, int m0, con
 
 template <int DT, int BKT>
 __device__ __forceinline__ void gemm_tile_nt(const Operand A, int m0, const Operand B, int n0, int K,
-                                             f32x16 (&acc)[MB][NB], char* smem) {
+                                             f32x16 (&acc)[MB][NB], char* smem, bool prefetched = false) {
 #if TRLK_HEAD_DIRECT_LDS
     if ((K & (BKT - 1)) == 0)
-        gemm_tile_nt_direct<DT, BKT>(A, m0, B, n0, K, acc, smem);
+        gemm_tile_nt_direct<DT, BKT>(A, m0, B, n0, K, acc, smem, prefetched);
     else
 #endif
         gemm_tile_nt_staged<DT>(A, m0, B, n0, K, acc, smem);
+}
+
+// Starts the transfers of a tile's first stages so that they overlap whatever the caller does
+// before gemm_tile_nt(..., prefetched = true); the LDS must be free and stay untouched until then.
+template <int BKT>
+__device__ __forceinline__ void gemm_tile_prefetch(const Operand A, int m0, const Operand B, int n0, int K, char* smem) {
+#if TRLK_HEAD_DIRECT_LDS
+    if ((K & (BKT - 1)) == 0) DirectLoader<BKT>(A, m0, B, n0, smem).prologue(K);
+#endif
 }
 
 // Row (M index) inside the workgroup tile of accumulator element r of block mb, for this lane.
@@ -488,10 +511,13 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
     }
     const Operand W{a.weight, a.ldw, a.V}, Hd{a.hidden, a.ldh, a.N};
 
+    if (vt0 < vt1) gemm_tile_prefetch<TRLK_HEAD_BK_FWD>(W, vt0 * BM, Hd, n0, a.H, smem);
     for (int vt = vt0; vt < vt1; ++vt) {
         const int m0 = vt * BM;
         f32x16 acc[MB][NB];
-        gemm_tile_nt<DT, TRLK_HEAD_BK_FWD>(W, m0, Hd, n0, a.H, acc, smem);
+        gemm_tile_nt<DT, TRLK_HEAD_BK_FWD>(W, m0, Hd, n0, a.H, acc, smem, true);
+        // the next tile's first stages travel while this tile's logits are reduced (registers only)
+        if (vt + 1 < vt1) gemm_tile_prefetch<TRLK_HEAD_BK_FWD>(W, m0 + BM, Hd, n0, a.H, smem);
         const bool partial_tile = m0 + BM > a.V;
         // Common case (no soft-capping, tile inside the vocabulary): z = y * zs with one positive
         // scale, so the maximum is taken on the raw accumulators and the scale is folded into the
@@ -656,37 +682,47 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
     f32x16 acc[MB][NB];
     gemm_tile_nt<DT, TRLK_HEAD_BK_DZ>(W, m0, Hd, n0, a.H, acc, smem);
 
+    // Common case (no soft-capping, tile inside the chunk): dz = -(g * chain) * exp2(y * zs2 - lzc)
+    // with one scale folded into the exponent; the target's one-hot term is patched afterwards.
+    const float zs = a.logit_scale * a.inv_t, zs2 = zs * kLog2e;
+    const bool plain = a.softcap <= 0.f && m0 + BM <= a.c1;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         const int tok = n0 + acc_col(wn, nb, lane);
         const bool tok_ok = tok < a.N;
         const float g = tok_ok ? a.g[tok] : 0.f;
-        const float lzc = tok_ok ? a.log_z[tok] * kLog2e : 0.f;
+        const float lzc = tok_ok ? a.log_z[tok] * kLog2e : INFINITY;  // rows beyond N: exp2(-inf) = 0
         const int64_t tg = tok_ok ? a.targets[tok] : -1;
+        const int64_t rel = tg - (m0 + wm * WM);  // target row relative to this wave's rows
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
             float d[16];
+            if (plain) {
+                const float ngc = -g * zs;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int v = m0 + acc_row(wm, mb, r, lane);
-                float y = acc[mb][nb][r] * a.logit_scale;
-                float chain = a.inv_t * a.logit_scale;
-                if (a.softcap > 0.f) {
-                    const float th = tanhf(y / a.softcap);
-                    y = th * a.softcap;
-                    chain *= 1.f - th * th;
+                for (int r = 0; r < 16; ++r) d[r] = ngc * fast_exp2(fmaf(acc[mb][nb][r], zs2, -lzc));
+                if (rel >= mb * 32 && rel < mb * 32 + 32) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (acc_row(0, mb, r, lane) == int(rel)) d[r] -= ngc;
                 }
-                const float z = y * a.inv_t;
-                const float p = fast_exp2(fmaf(z, kLog2e, -lzc));
-                float dzv = -g * p;
-                if (v == tg) dzv += g;
-                d[r] = (v < a.c1 && tok_ok) ? dzv * chain : 0.f;
-            }
-            // dz^T [chunk row][token]: lanes = consecutive tokens -> 64-byte runs per vocabulary row
+            } else {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int vrow = vt * BM + acc_row(wm, mb, r, lane);  // chunk-local (padding rows are written as 0)
-                E::store1(a.dzT + int64_t(vrow) * a.ldzt + (n0 + acc_col(wn, nb, lane)), d[r]);
+                for (int r = 0; r < 16; ++r) {
+                    const int v = m0 + acc_row(wm, mb, r, lane);
+                    float y = acc[mb][nb][r] * a.logit_scale;
+                    float chain = a.inv_t * a.logit_scale;
+                    if (a.softcap > 0.f) {
+                        const float th = tanhf(y / a.softcap);
+                        y = th * a.softcap;
+                        chain *= 1.f - th * th;
+                    }
+                    const float z = y * a.inv_t;
+                    const float p = fast_exp2(fmaf(z, kLog2e, -lzc));
+                    float dzv = -g * p;
+                    if (v == tg) dzv += g;
+                    d[r] = (v < a.c1 && tok_ok) ? dzv * chain : 0.f;
+                }
             }
             // dz [token][chunk column] goes through LDS: a lane owns scattered 8-byte pieces of 32
             // different token rows, which would reach memory as partial sectors; staged as a
@@ -698,16 +734,48 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
                 w.y = E::pack2(d[q * 4 + 2], d[q * 4 + 3]);
                 *reinterpret_cast<uint2*>(smem + acc_col(wn, nb, lane) * kDzLdsRow + acc_row(wm, mb, q * 4, lane) * 2) = w;
             }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mb][nb][r] = d[r];  // kept for the transposed copy
         }
     }
     __syncthreads();
-    constexpr int kChunksPerRow = BM / 8;  // 16-byte pieces per token row of the tile
+    constexpr int kChunksPerRow = BM / 8;  // 16-byte pieces per row of the staged tile (BM == BN)
+    static_assert(BM == BN, "the two staged copies of the dz tile share one LDS layout");
 #pragma unroll 4
     for (int c = tid; c < BN * kChunksPerRow; c += kHeadThreads) {
         const int tok_local = c / kChunksPerRow, vc = c % kChunksPerRow;
         if (n0 + tok_local < a.N)
             *reinterpret_cast<u32x4*>(a.dz + int64_t(n0 + tok_local) * a.ldz + vt * BM + vc * 8) =
                 *reinterpret_cast<const u32x4*>(smem + tok_local * kDzLdsRow + vc * 16);
+    }
+    __syncthreads();
+    // dz^T [chunk row][token]: the lanes of a block hold consecutive tokens of one vocabulary row.
+    // Neighbouring lanes swap one value each, so that the even lane owns two tokens of row r and
+    // the odd lane two tokens of row r + 1; the 4-byte pieces are staged as a [vocabulary][token]
+    // tile and leave as 512-byte runs as well.
+    const int odd = lane & 1;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int tcol = (acc_col(wn, nb, lane) & ~1) * 2;  // byte offset of the token pair inside a staged row
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                const float mine0 = acc[mb][nb][r], mine1 = acc[mb][nb][r + 1];
+                const float give = odd ? mine0 : mine1;
+                const float got = __builtin_bit_cast(
+                    float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, give), 0xB1 /* quad_perm 1,0,3,2 */, 0xf, 0xf, true));
+                const uint32_t w = odd ? E::pack2(got, mine1) : E::pack2(mine0, got);
+                const int vrow = acc_row(wm, mb, r, lane) + odd;
+                *reinterpret_cast<uint32_t*>(smem + vrow * kDzLdsRow + tcol) = w;
+            }
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int c = tid; c < BM * kChunksPerRow; c += kHeadThreads) {
+        const int vrow = c / kChunksPerRow, tc = c % kChunksPerRow;  // chunk-local row (padding rows are written as 0)
+        *reinterpret_cast<u32x4*>(a.dzT + int64_t(vt * BM + vrow) * a.ldzt + n0 + tc * 8) =
+            *reinterpret_cast<const u32x4*>(smem + vrow * kDzLdsRow + tc * 16);
     }
 }
 
@@ -758,9 +826,9 @@ TRLK_HEAD_KERNEL void gemm_nt_kernel(GemmArgs a) {
         }
 }
 
-// [R, C] (ld) -> [C, ldo] with columns >= R zero-filled up to ldo: 64 x 64 tiles through LDS.
+// [R, C] (ld) -> [C, ldo] with columns >= R zero-filled up to `fill`: 64 x 64 tiles through LDS.
 __global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* in, int64_t ld, int R, int C, uint16_t* out,
-                                                          int64_t ldo) {
+                                                          int64_t ldo, int64_t fill) {
     __shared__ uint16_t tile[64][66];
     const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
@@ -771,14 +839,19 @@ __global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* in, in
     __syncthreads();
     for (int i = ty; i < 64; i += 4) {
         const int c = c0 + i, r = r0 + tx;
-        if (c < C && r < ldo) out[int64_t(c) * ldo + r] = tile[tx][i];
+        if (c < C && r < fill) out[int64_t(c) * ldo + r] = tile[tx][i];
     }
 }
 
 int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
+// Row strides of the workspace matrices carry 128 extra bytes: their padded extents are multiples
+// of large powers of two (tokens, chunk), and with such a stride the 256 rows of a tile step all
+// fall into the same memory channels.
+constexpr int64_t kLdSkew = 64;
 struct BwdLayout {
-    int64_t vpad, npad, cpad;
+    int64_t vpad, npad, cpad;    // padded extents (zero-filled)
+    int64_t ld_v, ld_n, ld_c;    // row strides of [*, vpad], [*, npad], [*, cpad] matrices
     size_t off_wt, off_ht, off_dz, off_dzt, off_dh, total;
 };
 BwdLayout bwd_layout(int64_t N, int64_t V, int64_t H, int64_t chunk) {
@@ -786,16 +859,19 @@ BwdLayout bwd_layout(int64_t N, int64_t V, int64_t H, int64_t chunk) {
     l.vpad = round_up(V, BK);
     l.npad = round_up(N, BN);
     l.cpad = round_up(chunk < V ? chunk : V, BM);
+    l.ld_v = l.vpad + kLdSkew;
+    l.ld_n = l.npad + kLdSkew;
+    l.ld_c = l.cpad + kLdSkew;
     size_t o = 0;
     auto take = [&](size_t bytes) {
         const size_t at = o;
         o += (bytes + 255) / 256 * 256;
         return at;
     };
-    l.off_wt = take(size_t(H) * l.vpad * 2);
-    l.off_ht = take(size_t(H) * l.npad * 2);
-    l.off_dz = take(size_t(N) * l.cpad * 2);
-    l.off_dzt = take(size_t(l.cpad) * l.npad * 2);
+    l.off_wt = take(size_t(H) * l.ld_v * 2);
+    l.off_ht = take(size_t(H) * l.ld_n * 2);
+    l.off_dz = take(size_t(N) * l.ld_c * 2);
+    l.off_dzt = take(size_t(l.cpad) * l.ld_n * 2);
     l.off_dh = take(size_t(N) * H * 4);
     l.total = o;
     return l;
@@ -929,18 +1005,18 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     TRLK_REQUIRE(d_workspace && workspace_bytes >= l.total, TRLK_ERR_WORKSPACE,
                  "fused_head_bwd: workspace of %zu bytes needed, %zu given", l.total, workspace_bytes);
     char* ws = static_cast<char*>(d_workspace);
-    uint16_t* wt = reinterpret_cast<uint16_t*>(ws + l.off_wt);    // [H, vpad]
-    uint16_t* ht = reinterpret_cast<uint16_t*>(ws + l.off_ht);    // [H, npad]
-    uint16_t* dz = reinterpret_cast<uint16_t*>(ws + l.off_dz);    // [N, cpad]
-    uint16_t* dzt = reinterpret_cast<uint16_t*>(ws + l.off_dzt);  // [cpad, npad]
+    uint16_t* wt = reinterpret_cast<uint16_t*>(ws + l.off_wt);    // [H, vpad], row stride ld_v
+    uint16_t* ht = reinterpret_cast<uint16_t*>(ws + l.off_ht);    // [H, npad], row stride ld_n
+    uint16_t* dz = reinterpret_cast<uint16_t*>(ws + l.off_dz);    // [N, cpad], row stride ld_c
+    uint16_t* dzt = reinterpret_cast<uint16_t*>(ws + l.off_dzt);  // [cpad, npad], row stride ld_n
     float* dh = reinterpret_cast<float*>(ws + l.off_dh);          // [N, H]
     (void)es;
     const int H = int(hidden_size), N = int(n_tokens), V = int(vocab);
     hipLaunchKernelGGL(transpose16_kernel, dim3((H + 63) / 64, unsigned((l.vpad + 63) / 64)), dim3(256), 0, s,
-                       static_cast<const uint16_t*>(d_weight), weight_stride, V, H, wt, l.vpad);
+                       static_cast<const uint16_t*>(d_weight), weight_stride, V, H, wt, l.ld_v, l.vpad);
     if (int rc = launch_status("fused_head_bwd (W^T)")) return rc;
     hipLaunchKernelGGL(transpose16_kernel, dim3((H + 63) / 64, unsigned((l.npad + 63) / 64)), dim3(256), 0, s,
-                       static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.npad);
+                       static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.ld_n, l.npad);
     if (int rc = launch_status("fused_head_bwd (hidden^T)")) return rc;
 
     HeadArgs a{};
@@ -959,8 +1035,8 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     a.g = d_g_logp;
     a.dz = dz;
     a.dzT = dzt;
-    a.ldz = l.cpad;
-    a.ldzt = l.npad;
+    a.ldz = l.ld_c;
+    a.ldzt = l.ld_n;
     const int n_tb = int((n_tokens + BN - 1) / BN);
     const int n_ht = (H + BN - 1) / BN;
     for (int64_t c0 = 0; c0 < vocab; c0 += chunk) {
@@ -977,8 +1053,8 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         const bool first = c0 == 0, last = c1 == vocab;
         // dHidden[N, H] += dz[N, chunk] * (W^T[H, chunk])^T ; W^T columns beyond V are zero and so is dz there
         GemmArgs gh{};
-        gh.A = Operand{dz, l.cpad, N};
-        gh.B = Operand{wt + c0, l.vpad, H};
+        gh.A = Operand{dz, l.ld_c, N};
+        gh.B = Operand{wt + c0, l.ld_v, H};
         gh.M = N;
         gh.N = H;
         gh.K = int(c0 + kpad <= l.vpad ? kpad : l.vpad - c0);
@@ -997,8 +1073,8 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         if (rc) return rc;
         // dW[chunk, H] = dz^T[chunk, N] * (hidden^T[H, N])^T
         GemmArgs gw{};
-        gw.A = Operand{dzt, l.npad, kpad};
-        gw.B = Operand{ht, l.npad, H};
+        gw.A = Operand{dzt, l.ld_n, kpad};
+        gw.B = Operand{ht, l.ld_n, H};
         gw.M = rows;
         gw.N = H;
         gw.K = int(l.npad);
