@@ -26,6 +26,11 @@ Pinning status (what checks each function against something other than itself):
                               autograd of it (reference test tests/test_utils.py:1161-1232)
   chunked_cross_entropy_loss: golden vectors from the reference's `_chunked_cross_entropy_loss`,
                               `F.cross_entropy` library routine
+  fused_linear_grpo_loss / fused_linear_dpo_loss : PARITY UNPINNED against the third-party operators
+                              they stand in for (liger-kernel >=0.8.0,<0.8.1 is not importable here and no
+                              reference test holds their numbers); they compose pinned pieces only -- the naive
+                              head routine + `grpo_loss` / `dpo_sigmoid_loss` -- in the metric order the
+                              reference's call sites read (grpo_trainer.py:2900-2901, dpo_trainer.py:1293-1301)
   get_off_policy_mask       : reference unit-test vectors (tests/test_grpo_trainer.py:1456-1520)
   get_high_entropy_mask     : reference unit-test vectors (tests/test_grpo_trainer.py:110-160)
 """
@@ -60,6 +65,8 @@ __all__ = [
     "ChunkedLogProbOracle",
     "patch_chunked_rows",
     "chunked_cross_entropy_loss",
+    "fused_linear_grpo_loss",
+    "fused_linear_dpo_loss",
 ]
 
 
@@ -365,7 +372,7 @@ def grpo_loss(
         per_token_loss = per_token_loss * off_mask
     if entropy_mask is not None:
         per_token_loss = per_token_loss * entropy_mask
-    if importance_sampling_ratio is not None:
+    if importance_sampling_ratio is not None and loss_type != "vespo":  # vespo folds it into phi (:3117)
         per_token_loss = per_token_loss * importance_sampling_ratio
     if beta != 0.0:
         per_token_loss = per_token_loss + beta * per_token_kl
@@ -659,3 +666,52 @@ def chunked_cross_entropy_loss(hidden_states, lm_head_weight, chunk_size, labels
         entropy_sum = entropy_sum + (-(lp.exp() * lp).sum(-1)).sum()
     denom = n_valid if num_items_in_batch is None else num_items_in_batch
     return loss / denom, correct, entropy_sum, n_valid
+
+
+# --------------------------------------------------------------------------------------
+# Fused-linear operator contracts          trl/trainer/grpo_trainer.py:2885-2907, dpo_trainer.py:1287-1327
+# --------------------------------------------------------------------------------------
+def fused_linear_grpo_loss(hidden, weight, selected_token_ids, loss_mask, advantages, temperature=1.0,
+                           old_per_token_logps=None, ref_per_token_logps=None, vllm_is_ratio=None, **loss_kwargs):
+    """What `compute_liger_loss` expects of `self.liger_loss` (grpo_trainer.py:2885-2901), stated with the
+    reference's own arithmetic: logits `(hidden @ W.T).float() / T` of every position (utils.py:1328-1337 without
+    chunking), `selective_log_softmax`, then `_compute_loss`'s loss (`grpo_loss` above, not divided by the
+    accumulation steps, dapo normaliser = active tokens of the batch).  Returns `(loss, [mean_kl]? + [clip_ratio])`
+    with clip_ratio = the region clip ratio."""
+    b, t, h = hidden.shape
+    logits = (hidden.reshape(b * t, h) @ weight.t()).float() / temperature
+    logps = selective_log_softmax(logits, selected_token_ids.reshape(b * t)).view(b, t)
+    beta = loss_kwargs.get("beta", 0.0)
+    loss, metrics = grpo_loss(
+        logps, advantages, loss_mask, old_per_token_logps=old_per_token_logps,
+        ref_per_token_logps=ref_per_token_logps, num_items_in_batch=loss_mask.sum().float(),
+        importance_sampling_ratio=vllm_is_ratio, grad_accum_steps=1.0, **loss_kwargs)
+    out = [metrics["kl"]] if beta != 0.0 else []
+    out.append(metrics.get("clip_ratio/region_mean", float("nan")))
+    return loss, out
+
+
+def fused_linear_dpo_loss(weight, hidden, target, ref_hidden, ref_weight, beta, ignore_index=-100):
+    """What `_compute_loss_liger` expects of `self.liger_loss` (dpo_trainer.py:1287-1301) for the sigmoid loss:
+    summed log-probs of the non-ignored targets (as dpo_trainer.py:1347-1350), reference ones without grad,
+    `dpo_sigmoid_loss` above.  Returns `(loss, (chosen_logps, rejected_logps, chosen_logits_mean,
+    rejected_logits_mean, nll_loss, chosen_rewards, rejected_rewards))`; the logits means run over all
+    positions and the whole vocabulary."""
+    b, t, h = hidden.shape
+    keep = target != ignore_index
+    labels = torch.where(keep, target, torch.zeros_like(target))
+
+    def seq_logps(hs, w):
+        logits = (hs.reshape(b * t, h) @ w.t()).float()
+        tok = selective_log_softmax(logits, labels.reshape(b * t)).view(b, t)
+        return (tok * keep).sum(-1), logits.view(b, t, -1)
+
+    seq, logits = seq_logps(hidden, weight)
+    with torch.no_grad():
+        ref_seq, _ = seq_logps(ref_hidden, ref_weight)
+    pairs = b // 2
+    loss, _ = dpo_sigmoid_loss(seq, ref_seq[:pairs], ref_seq[pairs:], beta)
+    rewards = beta * (seq.detach() - ref_seq)
+    metrics = (seq.detach()[:pairs], seq.detach()[pairs:], logits.detach()[:pairs].mean(), logits.detach()[pairs:].mean(),
+               torch.zeros(()), rewards[:pairs], rewards[pairs:])
+    return loss, metrics

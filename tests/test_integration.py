@@ -35,3 +35,36 @@ def test_patch_trl_rebinds_every_importer():
         assert ref_grpo.selective_log_softmax is orig and ref_grpo.GRPOTrainer._compute_loss is orig_loss
     finally:
         sys.path.remove(REFERENCE)
+
+
+@pytest.mark.skipif(not os.path.isdir(os.path.join(REFERENCE, "trl")), reason="reference tree not present")
+def test_patch_trl_binds_the_fused_linear_operators():
+    """`liger=True` puts the fused-linear operators under the names the reference's trainers construct
+    (trl/trainer/grpo_trainer.py:1027, trl/trainer/dpo_trainer.py:834) and removes them again."""
+    sys.path.insert(0, REFERENCE)
+    try:
+        import trl.trainer.dpo_trainer as ref_dpo
+        import trl.trainer.grpo_trainer as ref_grpo
+
+        import trl_amd
+        from trl_amd import integration
+
+        had = hasattr(ref_grpo, "LigerFusedLinearGRPOLoss")
+        integration.patch_trl(grpo=False, liger=True)
+        try:
+            assert ref_grpo.LigerFusedLinearGRPOLoss is trl_amd.FusedLinearGRPOLoss
+            assert ref_dpo.LigerFusedLinearDPOLoss is trl_amd.FusedLinearDPOLoss
+            assert ref_grpo.is_liger_kernel_available() and ref_dpo.is_liger_kernel_available()
+            # the constructor calls of the reference (keyword sets at grpo_trainer.py:1027-1044, dpo_trainer.py:834)
+            op = ref_grpo.LigerFusedLinearGRPOLoss(
+                beta=0.04, epsilon_low=0.2, epsilon_high=0.2, temperature=1.0, use_ref_model=True, loss_type="dapo",
+                max_completion_length=16, importance_sampling_level="token", delta=None, use_bias_correction_kl=False,
+                sapo_temperature_pos=1.0, sapo_temperature_neg=1.05, vespo_k_pos=2.0, vespo_lambda_pos=3.0,
+                vespo_k_neg=3.0, vespo_lambda_neg=2.0)
+            assert op.beta == 0.04
+            ref_dpo.LigerFusedLinearDPOLoss(beta=0.1, loss_type="sigmoid")
+        finally:
+            integration.unpatch_trl()
+        assert hasattr(ref_grpo, "LigerFusedLinearGRPOLoss") == had
+    finally:
+        sys.path.remove(REFERENCE)

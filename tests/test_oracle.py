@@ -380,3 +380,31 @@ def test_golden_sft_chunked_nll():
     loss, correct, ent, nv = oracle.chunked_cross_entropy_loss(hs, w, 4, labels=torch.full((2, 7), -100))
     loss.backward()
     assert float(loss) == 0.0 and int(nv) == 0 and torch.count_nonzero(hs.grad) == 0
+
+
+def test_fused_linear_contracts_reduce_to_closed_forms():
+    """The fused-linear oracle functions only compose pinned pieces; what is checked here is the contract of
+    the call sites: metric positions (grpo_trainer.py:2900-2901, dpo_trainer.py:1293-1301) and two closed forms
+    (policy == reference gives ln 2 and zero rewards; on-policy GRPO has clip ratio 0 and kl 0 when ref == logps)."""
+    g = torch.Generator().manual_seed(5)
+    P, T, H, V = 3, 7, 16, 29
+    hidden = torch.randn(2 * P, T, H, generator=g)
+    weight = torch.randn(V, H, generator=g) * 0.3
+    target = torch.randint(0, V, (2 * P, T), generator=g)
+    target[:, :2] = -100
+    loss, m = oracle.fused_linear_dpo_loss(weight, hidden, target, hidden, weight, beta=0.1)
+    assert abs(float(loss) - math.log(2.0)) < 1e-6 and len(m) == 7
+    assert torch.equal(m[5], torch.zeros(P)) and torch.equal(m[6], torch.zeros(P)) and float(m[4]) == 0.0
+    logits = hidden.reshape(-1, H) @ weight.t()
+    assert abs(float(m[2]) - float(logits.view(2 * P, T, V)[:P].mean())) < 1e-6
+
+    ids = torch.randint(0, V, (2 * P, T), generator=g)
+    mask = torch.ones(2 * P, T, dtype=torch.long)
+    adv = torch.randn(2 * P, generator=g)
+    logps = oracle.selective_log_softmax(logits.float(), ids.reshape(-1)).view(2 * P, T)
+    loss, m = oracle.fused_linear_grpo_loss(hidden, weight, ids, mask, adv, 1.0, None, logps, None, beta=0.04,
+                                            loss_type="bnpo")
+    assert len(m) == 2 and abs(m[0]) < 1e-7 and m[1] == 0.0
+    assert abs(float(loss) + float(adv.mean())) < 1e-6  # -(sum A * 1) / tokens
+    loss, m = oracle.fused_linear_grpo_loss(hidden, weight, ids, mask, adv, 1.0, beta=0.0, loss_type="bnpo")
+    assert len(m) == 1

@@ -5,7 +5,11 @@ every trainer module, and the loss is a trainer method.  `patch_trl()` therefore
   * `selective_log_softmax`, `entropy_from_logits`, `_ChunkedLogProbFunction`, `patch_chunked_lm_head`
     in `trl.trainer.utils` **and** in every already-imported `trl.*` module that holds its own reference;
   * `trl.trainer.sft_trainer._chunked_cross_entropy_loss` (the default SFT loss);
-  * `GRPOTrainer._get_per_token_logps_and_entropies` / `_compute_loss` (optional, `grpo=True`).
+  * `GRPOTrainer._get_per_token_logps_and_entropies` / `_compute_loss` (optional, `grpo=True`);
+  * the fused-linear loss operators behind `use_liger_kernel` (optional, `liger=True`): the names
+    `LigerFusedLinearGRPOLoss` / `LigerFusedLinearDPOLoss` and `is_liger_kernel_available` in
+    `trl.trainer.grpo_trainer` / `trl.trainer.dpo_trainer` (trl/trainer/grpo_trainer.py:1020-1044,
+    trl/trainer/dpo_trainer.py:834), so that `compute_liger_loss` / `_compute_loss_liger` call the fused head.
 `unpatch_trl()` restores the originals.
 """
 from __future__ import annotations
@@ -19,7 +23,15 @@ _FUNCTIONS = ("selective_log_softmax", "entropy_from_logits", "_ChunkedLogProbFu
 _saved: list[tuple[object, str, object]] = []
 
 
-def patch_trl(grpo: bool = True) -> int:
+_MISSING = object()
+
+
+def _set(mod, name, value) -> None:
+    _saved.append((mod, name, getattr(mod, name, _MISSING)))
+    setattr(mod, name, value)
+
+
+def patch_trl(grpo: bool = True, liger: bool = False) -> int:
     """Returns the number of names rebound.  Needs `trl` to be importable."""
     import trl.trainer.utils as ref_utils
 
@@ -53,10 +65,24 @@ def patch_trl(grpo: bool = True) -> int:
             _saved.append((GRPOTrainer, name, GRPOTrainer.__dict__[name]))
             setattr(GRPOTrainer, name, getattr(_grpo.GRPOLossMixin, name))
             count += 1
+    if liger:
+        import trl.trainer.dpo_trainer as ref_dpo
+        import trl.trainer.grpo_trainer as ref_grpo
+
+        from .trainer.fused_linear import FusedLinearDPOLoss, FusedLinearGRPOLoss
+
+        _set(ref_grpo, "LigerFusedLinearGRPOLoss", FusedLinearGRPOLoss)
+        _set(ref_grpo, "is_liger_kernel_available", lambda *a, **k: True)
+        _set(ref_dpo, "LigerFusedLinearDPOLoss", FusedLinearDPOLoss)
+        _set(ref_dpo, "is_liger_kernel_available", lambda *a, **k: True)
+        count += 4
     return count
 
 
 def unpatch_trl() -> None:
     while _saved:
         obj, name, orig = _saved.pop()
-        setattr(obj, name, orig)
+        if orig is _MISSING:
+            delattr(obj, name)
+        else:
+            setattr(obj, name, orig)
