@@ -76,14 +76,21 @@ const char* trlk_last_error(void);
  *   out_lse[r]     = logsumexp(z[r, :])            (the only state the backward needs)
  * All arithmetic is fp32 whatever `dtype` is; outputs are fp32.
  * d_index: int64 [rows, n_index].  d_row_mask (optional, uint8 [rows]): rows whose mask is 0
- * are not read and get 0 in every output.  d_out_entropy / d_out_lse / d_error_flag may be
- * NULL.  An index outside [0, vocab) yields NaN for that entry and sets
+ * are not read and get 0 in every output.  d_out_entropy / d_out_lse / d_out_row_stats /
+ * d_error_flag may be NULL.
+ * d_out_row_stats (optional, fp32 [rows, 4]) takes what DPOTrainer._compute_loss derives from
+ * three more passes over the logits (trl/trainer/dpo_trainer.py:1563-1574 WPO weights, :1605-1618
+ * logits means, :1620-1631 token accuracy):
+ *   [0] mean_v logits[r, v]                       (raw logits, not divided by the temperature)
+ *   [1] log sum_v softmax(z[r])_v^2 = logsumexp(2 z) - 2 logsumexp(z)
+ *   [2] 1 if index[r, 0] is the row's arg-max (the FIRST maximal position, as torch.argmax), else 0
+ *   [3] 0 (reserved)  An index outside [0, vocab) yields NaN for that entry and sets
  * TRLK_FLAG_INDEX_OUT_OF_RANGE in *d_error_flag.
  */
 int trlk_logp_entropy_fwd(const void* d_logits, int dtype, int64_t n_seq, int64_t rows_per_seq, int64_t vocab,
                           int64_t seq_stride, int64_t row_stride, const int64_t* d_index, int32_t n_index,
                           float temperature, const uint8_t* d_row_mask, float* d_out_logp, float* d_out_entropy,
-                          float* d_out_lse, int32_t* d_error_flag, trlk_stream_t stream);
+                          float* d_out_lse, float* d_out_row_stats, int32_t* d_error_flag, trlk_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------
  * K3  backward of K1 by recomputation from the saved lse: one read and one write of the

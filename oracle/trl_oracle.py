@@ -20,7 +20,8 @@ Pinning status (what checks each function against something other than itself):
                               `GRPOTrainer._compute_loss` on a mocked trainer
                               (tests/golden/), closed forms (on-policy, ref == logps)
   dpo_*                     : golden vectors from the reference's
-                              `DPOTrainer._compute_loss` (mocked), closed form ln 2
+                              `DPOTrainer._compute_loss` (mocked; all fifteen loss types, ld_alpha, WPO
+                              weighting, f-divergences, arg-max ties), closed form ln 2
   rloo_loss                 : golden vectors from `RLOOTrainer._compute_loss` (mocked)
   chunked_logprob           : naive `(h @ W.T).float()/T -> log_softmax` routine and
                               autograd of it (reference test tests/test_utils.py:1161-1232)
@@ -58,6 +59,7 @@ __all__ = [
     "grpo_loss",
     "dpo_sequence_logps",
     "dpo_sigmoid_loss",
+    "dpo_compute_loss",
     "rloo_loss",
     "chunked_logprob_naive",
     "chunked_logprob_online",
@@ -475,6 +477,128 @@ def dpo_sigmoid_loss(seq_logps: torch.Tensor, ref_chosen_logps: torch.Tensor, re
     c_rew = beta * chosen_lr.detach()
     r_rew = beta * rejected_lr.detach()
     metrics = {
+        "rewards/chosen": float(c_rew.mean()),
+        "rewards/rejected": float(r_rew.mean()),
+        "rewards/accuracies": float((c_rew > r_rew).float().mean()),
+        "rewards/margins": float((c_rew - r_rew).mean()),
+        "logps/chosen": float(chosen.detach().mean()),
+        "logps/rejected": float(rejected.detach().mean()),
+    }
+    return loss, metrics
+
+
+def _dpo_scores(chosen_lr, rejected_lr, f_divergence_type, f_alpha):
+    """f-divergence scores of the log-ratios (dpo_trainer.py:1402-1429)."""
+    if f_divergence_type == "reverse_kl" or (f_divergence_type == "alpha_divergence" and abs(f_alpha - 1.0) < 1e-6):
+        return chosen_lr, rejected_lr
+    if f_divergence_type == "forward_kl":
+        return -torch.exp(-chosen_lr), -torch.exp(-rejected_lr)
+    if f_divergence_type == "js_divergence":
+        return F.logsigmoid(chosen_lr), F.logsigmoid(rejected_lr)
+    if f_divergence_type == "alpha_divergence":
+        cap = {torch.float16: 11.0, torch.bfloat16: 80.0, torch.float32: 80.0}[chosen_lr.dtype]
+        k = f_alpha - 1.0
+        out = []
+        for lr in (chosen_lr, rejected_lr):
+            out.append(torch.exp(torch.clamp((k * lr).float(), max=cap)).to(lr.dtype) / k)
+        return tuple(out)
+    raise ValueError(f"Unknown f_divergence_type: {f_divergence_type}")
+
+
+def dpo_compute_loss(logits, input_ids, completion_mask, ref_chosen_logps, ref_rejected_logps, beta, loss_types=("sigmoid",),
+                     loss_weights=None, label_smoothing=0.0, ld_alpha=None, use_weighting=False,
+                     f_divergence_type="reverse_kl", f_alpha=1.0, discopop_tau=0.05):
+    """`DPOTrainer._compute_loss` after the model call with precomputed reference log-probs
+    (dpo_trainer.py:1342-1362 sequence log-probs incl. the `ld_alpha` split, :1397-1431 scores, :1433-1561 the
+    fifteen per-pair losses, :1563-1574 WPO weights, :1584-1653 metrics).  Returns `(loss, metrics)`."""
+    shift_logits = logits[..., :-1, :]
+    labels = input_ids[..., 1:]
+    smask = completion_mask[..., 1:]
+    tok = selective_log_softmax(shift_logits, labels)
+    tok = torch.where(smask == 0, torch.zeros_like(tok), tok)
+    if ld_alpha is None:
+        seq = tok.sum(dim=1)
+    else:  # tokens beyond the shorter completion of the pair count with weight ld_alpha
+        pos = smask.cumsum(dim=1)
+        lens = smask.sum(dim=1).long()
+        c_len, r_len = lens.chunk(2)
+        shared = torch.minimum(c_len, r_len).repeat(2).unsqueeze(1)
+        head = (pos > 0) & (pos <= shared)
+        tail = pos > shared
+        seq = (tok * head).sum(dim=1) + ld_alpha * (tok * tail).sum(dim=1)
+    chosen, rejected = seq.chunk(2)
+    c_lr, r_lr = chosen - ref_chosen_logps, rejected - ref_rejected_logps
+    c_sc, r_sc = _dpo_scores(c_lr, r_lr, f_divergence_type, f_alpha)
+    d = c_sc - r_sc
+    c_n, r_n = (m.sum(dim=1).clamp(min=1.0) for m in completion_mask.chunk(2))
+    ls = label_smoothing
+
+    def smoothed(delta):
+        return -F.logsigmoid(beta * delta) * (1 - ls) - F.logsigmoid(-beta * delta) * ls
+
+    def sft_loss():
+        cm = smask.chunk(2)[0].bool()
+        ce = F.cross_entropy(shift_logits.chunk(2)[0][cm], labels.chunk(2)[0][cm])
+        return ce.expand(chosen.shape[0])
+
+    def exo():
+        eps = torch.tensor(ls)
+        qw, ql = torch.sigmoid(beta * d), torch.sigmoid(-beta * d)
+        return qw * (F.logsigmoid(beta * d) - torch.log1p(-eps)) + ql * (F.logsigmoid(-beta * d) - torch.log(eps))
+
+    def discopop():
+        x = beta * d
+        mix = torch.sigmoid(x / discopop_tau)
+        return -F.logsigmoid(x) * (1 - mix) + torch.exp(-x) * mix
+
+    per_pair = {
+        "sigmoid": lambda: -F.logsigmoid(beta * d),
+        "hinge": lambda: torch.relu(1 - beta * d),
+        "ipo": lambda: ((c_sc / c_n - r_sc / r_n) - 1 / (2 * beta)) ** 2,
+        "exo_pair": exo,
+        "nca_pair": lambda: -F.logsigmoid(beta * c_sc) - 0.5 * F.logsigmoid(-beta * c_sc) - 0.5 * F.logsigmoid(-beta * r_sc),
+        "robust": lambda: (-(1 - ls) * F.logsigmoid(beta * d) + ls * F.logsigmoid(-beta * d)) / (1 - 2 * ls),
+        "bco_pair": lambda: -F.logsigmoid(beta * c_sc) - F.logsigmoid(-beta * r_sc),
+        "sppo_hard": lambda: (c_sc - 0.5 / beta) ** 2 + (r_sc + 0.5 / beta) ** 2,
+        "aot": lambda: smoothed(torch.sort(chosen - rejected, dim=0)[0]
+                                - torch.sort(ref_chosen_logps - ref_rejected_logps, dim=0)[0]),
+        "aot_unpaired": lambda: smoothed(torch.sort(c_lr, dim=0)[0] - torch.sort(r_lr, dim=0)[0]),
+        "apo_zero": lambda: 1 - torch.sigmoid(beta * c_lr) + torch.sigmoid(beta * r_lr),
+        "apo_down": lambda: torch.sigmoid(beta * c_lr) + 1 - torch.sigmoid(beta * d),
+        "discopop": discopop,
+        "sft": sft_loss,
+        "sigmoid_norm": lambda: -F.logsigmoid(beta * (c_sc / c_n - r_sc / r_n)),
+    }
+    weights = None
+    if use_weighting:  # WPO: exp(mean over the completion of logp - log sum_v p_v^2), product over the pair (:1563-1574)
+        with torch.no_grad():
+            log_denom = torch.logsumexp(2.0 * shift_logits, dim=-1) - 2.0 * torch.logsumexp(shift_logits, dim=-1)
+            aligned = (tok - log_denom) * smask
+        w = torch.exp(aligned.sum(dim=1) / smask.sum(dim=1).clamp_min(1))
+        weights = w.chunk(2)[0] * w.chunk(2)[1]
+    loss_weights = [1.0] * len(loss_types) if loss_weights is None else loss_weights
+    loss = 0.0
+    for name, lw in zip(loss_types, loss_weights):
+        if name not in per_pair:
+            raise ValueError(f"Unknown loss type: {name}")
+        term = per_pair[name]()
+        if weights is not None:
+            term = term * weights
+        loss = loss + term.mean() * lw
+
+    det = shift_logits.detach()
+    ent = entropy_from_logits(det)
+    n_tok = smask.sum()
+    c_logits, r_logits = det.chunk(2)
+    c_m, r_m = (m.bool() for m in smask.chunk(2))
+    c_rew, r_rew = beta * c_lr.detach(), beta * r_lr.detach()
+    hits = (c_logits.argmax(dim=-1) == labels.chunk(2)[0]) & c_m
+    metrics = {
+        "entropy": float((ent * smask).sum() / n_tok) if n_tok > 0 else 0.0,
+        # sums leave the device in the logits dtype, the division happens on the host (:1609-1616)
+        "logits/chosen": float(c_logits[c_m].mean(-1).sum()) / float(c_m.sum()) if c_m.any() else 0.0,
+        "logits/rejected": float(r_logits[r_m].mean(-1).sum()) / float(r_m.sum()) if r_m.any() else 0.0,
+        "mean_token_accuracy": float(hits.sum() / c_m.sum()) if c_m.any() else 0.0,
         "rewards/chosen": float(c_rew.mean()),
         "rewards/rejected": float(r_rew.mean()),
         "rewards/accuracies": float((c_rew > r_rew).float().mean()),

@@ -217,6 +217,29 @@ DPO_CASES = [
     dict(name="sigmoid_beta05", beta=0.5, dtype="float32"),
     dict(name="sigmoid_bf16", beta=0.1, dtype="bfloat16"),
     dict(name="sigmoid_ref_equal", beta=0.1, dtype="float32", ref_equal=True),
+    dict(name="hinge", beta=0.1, dtype="float32", loss_types=["hinge"]),
+    dict(name="ipo", beta=0.1, dtype="float32", loss_types=["ipo"]),
+    dict(name="exo_pair", beta=0.1, dtype="float32", loss_types=["exo_pair"], label_smoothing=0.1),
+    dict(name="nca_pair", beta=0.1, dtype="float32", loss_types=["nca_pair"]),
+    dict(name="robust", beta=0.1, dtype="float32", loss_types=["robust"], label_smoothing=0.1),
+    dict(name="bco_pair", beta=0.1, dtype="float32", loss_types=["bco_pair"]),
+    dict(name="sppo_hard", beta=0.1, dtype="float32", loss_types=["sppo_hard"]),
+    dict(name="aot", beta=0.1, dtype="float32", loss_types=["aot"], label_smoothing=0.05),
+    dict(name="aot_unpaired", beta=0.1, dtype="float32", loss_types=["aot_unpaired"]),
+    dict(name="apo_zero", beta=0.1, dtype="float32", loss_types=["apo_zero"]),
+    dict(name="apo_down", beta=0.1, dtype="float32", loss_types=["apo_down"]),
+    dict(name="discopop", beta=0.1, dtype="float32", loss_types=["discopop"]),
+    dict(name="sft", beta=0.1, dtype="float32", loss_types=["sft"]),
+    dict(name="sigmoid_norm", beta=0.1, dtype="float32", loss_types=["sigmoid_norm"]),
+    dict(name="sigmoid_plus_sft", beta=0.1, dtype="float32", loss_types=["sigmoid", "sft"], loss_weights=[1.0, 0.5]),
+    dict(name="ld_alpha", beta=0.1, dtype="float32", ld_alpha=0.5),
+    dict(name="wpo", beta=0.1, dtype="float32", use_weighting=True),
+    dict(name="wpo_bf16", beta=0.1, dtype="bfloat16", use_weighting=True),
+    dict(name="forward_kl", beta=0.1, dtype="float32", f_divergence_type="forward_kl"),
+    dict(name="js_divergence", beta=0.1, dtype="float32", f_divergence_type="js_divergence"),
+    dict(name="alpha_divergence", beta=0.1, dtype="float32", f_divergence_type="alpha_divergence", f_alpha=0.5),
+    dict(name="ipo_ld_alpha_wpo", beta=0.2, dtype="float32", loss_types=["ipo"], ld_alpha=0.3, use_weighting=True),
+    dict(name="argmax_ties", beta=0.1, dtype="float32", ties=True),
 ]
 
 
@@ -229,6 +252,15 @@ def make_dpo(DPOTrainer, out_dir):
         dtype = getattr(torch, case["dtype"])
         logits = (2.0 * torch.randn(B, L, V, generator=g)).to(dtype)
         input_ids = torch.randint(0, V, (B, L), generator=g)
+        if ci >= 4:  # later cases: a third of the labels are the arg-max token, so the accuracy metric is exercised
+            g2 = torch.Generator().manual_seed(2500 + ci)
+            pick = torch.rand(B, L - 1, generator=g2) < 0.33
+            input_ids[:, 1:] = torch.where(pick, logits[:, :-1].float().argmax(-1), input_ids[:, 1:])
+        if case.get("ties"):  # two equal maxima per row: arg-max is the first one
+            top = logits.float().amax(-1) + 1.0
+            logits[..., 5] = top.to(dtype)
+            logits[..., 20] = top.to(dtype)
+            input_ids[:, 1:] = torch.where(torch.arange(L - 1)[None] % 2 == 0, 5, 20)
         prompt_len = [2, 3, 4]
         comp_len = [5, 4, 6, 8, 3, 2]
         completion_mask = torch.zeros(B, L, dtype=torch.long)
@@ -241,14 +273,16 @@ def make_dpo(DPOTrainer, out_dir):
         trainer = Mock(spec=DPOTrainer)
         trainer.accelerator = _fake_accelerator()
         trainer.aux_loss_enabled = False
-        trainer.ld_alpha = None
+        trainer.ld_alpha = case.get("ld_alpha")
         trainer.precompute_ref_logps = True
-        trainer.f_divergence_type = "reverse_kl"
-        trainer.loss_types = ["sigmoid"]
-        trainer.loss_weights = [1.0]
+        trainer.f_divergence_type = case.get("f_divergence_type", "reverse_kl")
+        trainer.f_alpha_divergence_coef = case.get("f_alpha", 1.0)
+        trainer.loss_types = case.get("loss_types", ["sigmoid"])
+        trainer.loss_weights = case.get("loss_weights", [1.0] * len(trainer.loss_types))
         trainer.beta = case["beta"]
-        trainer.label_smoothing = 0.0
-        trainer.use_weighting = False
+        trainer.label_smoothing = case.get("label_smoothing", 0.0)
+        trainer.use_weighting = case.get("use_weighting", False)
+        trainer.args = SimpleNamespace(discopop_tau=0.05)
         trainer._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
         trainer._total_train_tokens = 0
         trainer.model = SimpleNamespace(training=True)

@@ -277,3 +277,41 @@ def test_full_size_properties_config3_shape(amd):
     want_g = gl[pick_b][:, pick_t].cpu().unsqueeze(-1) * (onehot - p) / temp
     got_g = grad[pick_b][:, pick_t].float().cpu()
     assert _rel_l2(got_g, want_g) < 3e-3
+
+
+def test_row_statistics_of_the_same_pass():
+    """`logp_entropy_stats_fwd`: mean logit, log sum_v p_v^2 and the arg-max flag (first maximal position, as
+    `torch.argmax`) against torch on the same values, at a real vocabulary size, with ties and masked rows."""
+    import trl_amd
+    from trl_amd import ops
+
+    g = torch.Generator().manual_seed(77)
+    for dtype, V, tol in ((torch.bfloat16, 128256, 2e-3), (torch.float32, 32000, 1e-5), (torch.float16, 1003, 2e-3)):
+        B, L = 2, 9
+        logits = (2.0 * torch.randn(B, L, V, generator=g)).to(dtype)
+        ids = torch.randint(0, V, (B, L), generator=g)
+        top = logits.float().argmax(-1)
+        ids[:, 1::3] = top[:, 1::3]                      # every third target is the arg-max
+        logits[0, 2, 7] = logits[0, 2, 11] = logits[0, 2].max() + 1   # tie: position 7 wins
+        ids[0, 2] = 11
+        logits[1, 4, 3] = logits[1, 4, 900] = logits[1, 4].max() + 1  # tie, target is the first one
+        ids[1, 4] = 3
+        mask = torch.ones(B, L, dtype=torch.uint8)
+        mask[1, 6] = 0
+        x = logits.float()
+        want_mean = x.mean(-1)
+        want_lsp2 = torch.logsumexp(2 * x, -1) - 2 * torch.logsumexp(x, -1)
+        want_hit = (x.argmax(-1) == ids).float()
+        logp, ent, lse, stats = ops.logp_entropy_stats_fwd(logits.to(DEV), ids.reshape(-1, 1).to(DEV), 1.0, 0, L,
+                                                           mask.reshape(-1).to(DEV))
+        stats = stats.cpu().view(B, L, 4)
+        keep = mask.bool()
+        torch.testing.assert_close(stats[..., 0][keep], want_mean[keep], atol=tol, rtol=0)
+        torch.testing.assert_close(stats[..., 1][keep], want_lsp2[keep], atol=10 * tol, rtol=0)
+        assert torch.equal(stats[..., 2][keep], want_hit[keep])
+        assert want_hit[0, 2] == 0 and want_hit[1, 4] == 1 and want_hit[:, 1].sum() == B
+        assert torch.equal(stats[1, 6], torch.zeros(4)) and float(logp.view(B, L)[1, 6]) == 0.0
+        # the other outputs are those of the plain forward
+        lp2, ent2, lse2 = ops.logp_entropy_fwd(logits.to(DEV), ids.reshape(-1, 1).to(DEV), 1.0, 0, L,
+                                               mask.reshape(-1).to(DEV))
+        assert torch.equal(logp, lp2) and torch.equal(ent, ent2) and torch.equal(lse, lse2)

@@ -242,9 +242,88 @@ def test_group_advantages(amd):
     torch.testing.assert_close(amd.group_advantages(rb.to(DEV), 16).cpu(), oracle.group_advantages(rb, 16), rtol=1e-5, atol=1e-6)
 
 
-def test_golden_dpo_compute_loss(amd):
+def _dpo_kwargs(case):
+    return dict(loss_types=case.get("loss_types", ["sigmoid"]), loss_weights=case.get("loss_weights"),
+                label_smoothing=case.get("label_smoothing", 0.0), ld_alpha=case.get("ld_alpha"),
+                use_weighting=case.get("use_weighting", False), f_divergence_type=case.get("f_divergence_type", "reverse_kl"),
+                f_alpha_divergence_coef=case.get("f_alpha", 1.0), discopop_tau=0.05)
+
+
+@pytest.mark.parametrize("skip_masked", [False, True])
+def test_golden_dpo_compute_loss_all_loss_types(amd, skip_masked):
+    """Every case the reference's `DPOTrainer._compute_loss` ran on a mocked trainer (fifteen loss types, ld_alpha,
+    WPO weighting, f-divergences, arg-max ties): loss, dlogits and the ten logged metrics, from one pass over the
+    logits.  bf16 cases: the reference rounds log-probs, entropies and the WPO log-sum-exps to bf16, hence 2e-2."""
     cases, g = load_golden("dpo_compute_loss")
     for case in cases:
+        c = f"c{case['id']}_"
+        dtype = getattr(torch, case["dtype"])
+        low = dtype != torch.float32
+        leaf = _t(g[c + "logits"], dtype).to(DEV).requires_grad_(True)
+        loss, parts = amd.dpo_compute_loss(
+            leaf, _t(g[c + "input_ids"]).to(DEV), _t(g[c + "completion_mask"]).to(DEV),
+            _t(g[c + "ref_chosen_logps"]).to(DEV), _t(g[c + "ref_rejected_logps"]).to(DEV), beta=case["beta"],
+            skip_masked_rows=skip_masked, **_dpo_kwargs(case))
+        loss.backward()
+        want = float(g[c + "out_loss"])
+        rel = 5e-2 if low else 1e-5
+        assert abs(float(loss) - want) <= rel * max(1.0, abs(want)), (case["name"], float(loss), want)
+        assert _rel_l2(leaf.grad.float(), _t(g[c + "out_dlogits"])) < (5e-2 if low else 1e-4), case["name"]
+        got = amd.dpo_metrics_to_dict(parts)
+        for name, want_m in case["metrics"].items():
+            if name == "num_tokens" or (name == "rewards/accuracies" and (low or case.get("ref_equal"))):
+                continue  # accuracies: ties / near-ties between the rewards are decided by rounding noise
+            tol = (0.15 if low else 1e-5) * max(1.0, abs(want_m))
+            if name in ("logits/chosen", "logits/rejected"):
+                tol = max(tol, 2e-6)  # means of ~N(0, 4) logits over V: absolute fp32 summation noise
+            assert abs(got[name] - want_m) <= tol, (case["name"], name, got[name], want_m)
+
+
+def test_dpo_mixin_compute_loss(amd):
+    """The mix-in method with the reference's signature on a mocked trainer (wpo + ld_alpha + ipo case)."""
+    cases, g = load_golden("dpo_compute_loss")
+    case = next(c for c in cases if c["name"] == "ipo_ld_alpha_wpo")
+    c = f"c{case['id']}_"
+
+    class Trainer(amd.DPOLossMixin):
+        pass
+
+    tr = Trainer()
+    tr.accelerator = _Identity()
+    tr.accelerator.gather_for_metrics = lambda x: x
+    tr.model = SimpleNamespace(training=True)
+    tr.aux_loss_enabled = False
+    tr.precompute_ref_logps = True
+    tr.beta, tr.loss_types, tr.loss_weights = case["beta"], case["loss_types"], [1.0]
+    tr.label_smoothing, tr.ld_alpha, tr.use_weighting = 0.0, case["ld_alpha"], True
+    tr.f_divergence_type, tr.f_alpha_divergence_coef = "reverse_kl", 1.0
+    tr.args = SimpleNamespace(discopop_tau=0.05)
+    tr._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
+    tr._total_train_tokens = 0
+    leaf = _t(g[c + "logits"]).to(DEV).requires_grad_(True)
+    inputs = dict(input_ids=_t(g[c + "input_ids"]).to(DEV), attention_mask=_t(g[c + "attention_mask"]).to(DEV),
+                  completion_mask=_t(g[c + "completion_mask"]).to(DEV),
+                  ref_chosen_logps=_t(g[c + "ref_chosen_logps"]).to(DEV),
+                  ref_rejected_logps=_t(g[c + "ref_rejected_logps"]).to(DEV))
+    loss = tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None), inputs, False)
+    loss.backward()
+    assert abs(float(loss) - float(g[c + "out_loss"])) <= 1e-5 * max(1.0, abs(float(g[c + "out_loss"])))
+    assert _rel_l2(leaf.grad, _t(g[c + "out_dlogits"])) < 1e-4
+    got = {k: v[-1] for k, v in tr._metrics["train"].items()}
+    for name, want in case["metrics"].items():
+        assert abs(got[name] - want) <= 1e-5 * max(1.0, abs(want)), (name, got[name], want)
+    # the reference-model pass: sequence log-probs of the same logits, with and without the ld_alpha split
+    seq = amd.dpo_sequence_logps(leaf.detach(), inputs["input_ids"], inputs["completion_mask"])
+    oseq, _ = oracle.dpo_sequence_logps(_t(g[c + "logits"]), _t(g[c + "input_ids"]), _t(g[c + "completion_mask"]))
+    torch.testing.assert_close(seq.cpu(), oseq, rtol=1e-5, atol=1e-5)
+
+
+def test_golden_dpo_compute_loss(amd):
+    """The fused sigmoid path (one loss kernel) on the plain sigmoid cases."""
+    cases, g = load_golden("dpo_compute_loss")
+    plain = [c for c in cases if not ({"loss_types", "ld_alpha", "use_weighting", "f_divergence_type"} & set(c))]
+    assert len(plain) >= 5
+    for case in plain:
         c = f"c{case['id']}_"
         dtype = getattr(torch, case["dtype"])
         low = dtype != torch.float32

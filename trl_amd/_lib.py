@@ -32,7 +32,7 @@ SIGNATURES = {
     "trlk_logp_entropy_fwd": (
         c_int32,
         [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int32, c_float, c_void_p,
-         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     ),
     "trlk_logp_entropy_bwd": (
         c_int32,

@@ -64,6 +64,7 @@ struct FwdArgs {
     float* out_logp;
     float* out_entropy;
     float* out_lse;
+    float* out_stats;  // [rows, 4] or null: mean logit, log sum_v p_v^2, first index is the arg-max, 0
     int32_t* error_flag;
 };
 
@@ -93,6 +94,23 @@ struct OnlineLse {
     }
 };
 
+// Extra per-lane row statistics of the STATS variant (what the DPO metrics and the WPO weights
+// need on top of log-prob and entropy, so that no further pass over the logits is necessary):
+// sum of exp2(x*c - r)^2 (same reference as OnlineLse), sum of x, and the number of elements that
+// come before the target in arg-max order (larger value, or equal value at a smaller position).
+struct RowStats {
+    float s2 = 0.f, sx = 0.f;
+    int beats = 0;
+};
+
+// Next float below x (x itself for -inf and NaN).
+__device__ __forceinline__ float prev_float(float x) {
+    if (!(x > -INFINITY)) return x;
+    const uint32_t b = __builtin_bit_cast(uint32_t, x);
+    if ((b << 1) == 0u) return __builtin_bit_cast(float, 0x80000001u);  // +-0 -> smallest negative denormal
+    return __builtin_bit_cast(float, (b >> 31) ? b + 1u : b - 1u);
+}
+
 template <int N>
 __device__ __forceinline__ float max_of(const float* x) {
     float a = x[0];
@@ -102,12 +120,13 @@ __device__ __forceinline__ float max_of(const float* x) {
 }
 
 // VEC: rows are 16-byte aligned and vocab is a multiple of the vector width.
-template <int DT, bool VEC>
+// STATS: also produce the row statistics of `out_stats`.
+template <int DT, bool VEC, bool STATS>
 __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
     typedef Elem<DT> E;
     typedef typename E::type T;
     constexpr int NW = kThreads / kWave;
-    __shared__ float red[3][NW];
+    __shared__ float red[STATS ? 6 : 3][NW];
     __shared__ float bcast[2];
 
     const int64_t row = blockIdx.x;
@@ -118,6 +137,7 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
             if (a.out_entropy) a.out_entropy[row] = 0.f;
             if (a.out_lse) a.out_lse[row] = 0.f;
         }
+        if (STATS && tid < 4) a.out_stats[row * 4 + tid] = 0.f;
         return;
     }
     const int64_t b = row / a.rows_per_seq;
@@ -127,6 +147,57 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
     const int64_t V = a.vocab;
 
     OnlineLse acc;
+    RowStats st;
+    // arg-max order against the target (first index of the row): an element before the target's
+    // position beats it with x >= xt, one behind it with x > xt; x >= xt is tested as x > xt_prev
+    // with the next smaller float (the logits are exact in fp32).
+    int64_t tpos = -1;
+    float xt = INFINITY, xt_prev = INFINITY;
+    if constexpr (STATS) {
+        const int64_t idx = a.n_index > 0 ? a.index[row * a.n_index] : -1;
+        if (idx >= 0 && idx < V) {
+            tpos = idx;
+            xt = E::load1(base + idx);
+            xt_prev = prev_float(xt);
+        }
+    }
+    // one element with its position e (stats only)
+    auto stat_elem = [&](float x, int64_t e) {
+        st.sx += x;
+        st.beats += x > (e < tpos ? xt_prev : xt) ? 1 : 0;
+    };
+    // EPV elements starting at position e0: one threshold for the whole vector unless it holds the target
+    auto stat_vec = [&](const float* x, int64_t e0, int n) {
+        if (e0 <= tpos && tpos < e0 + n) {
+            for (int i = 0; i < n; ++i) stat_elem(x[i], e0 + i);
+        } else {
+            const float thr = e0 < tpos ? xt_prev : xt;
+            for (int i = 0; i < n; ++i) {
+                st.sx += x[i];
+                st.beats += x[i] > thr ? 1 : 0;
+            }
+        }
+    };
+    auto raise = [&](float bm) {
+        if constexpr (STATS) {
+            const float need = ceilf(bm * c);
+            if (need > acc.r) {
+                const float sc = fast_exp2(acc.r - need);
+                st.s2 *= sc * sc;
+            }
+        }
+        acc.raise(bm, c);
+    };
+    auto add = [&](float x) {
+        if constexpr (STATS) {
+            const float e = fast_exp2(fmaf(x, c, -acc.rr));
+            acc.s += e;
+            acc.u = fmaf(e, x, acc.u);
+            st.s2 = fmaf(e, e, st.s2);
+        } else {
+            acc.add(x, c);
+        }
+    };
     if constexpr (VEC) {
         constexpr int EPV = E::EPV;
         const u32x4* vp = reinterpret_cast<const u32x4*>(base);
@@ -139,22 +210,28 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
             float x[kUnroll * EPV];
 #pragma unroll
             for (int j = 0; j < kUnroll; ++j) E::unpack(q[j], x + j * EPV);
-            acc.raise(max_of<kUnroll * EPV>(x), c);
+            raise(max_of<kUnroll * EPV>(x));
 #pragma unroll
-            for (int i = 0; i < kUnroll * EPV; ++i) acc.add(x[i], c);
+            for (int i = 0; i < kUnroll * EPV; ++i) add(x[i]);
+            if constexpr (STATS) {
+#pragma unroll
+                for (int j = 0; j < kUnroll; ++j) stat_vec(x + j * EPV, int64_t(v + j * kThreads) * EPV, EPV);
+            }
         }
         for (; v < nvec; v += kThreads) {
             float x[EPV];
             E::unpack(stream_load<kFwdNt>(vp + v), x);
-            acc.raise(max_of<EPV>(x), c);
+            raise(max_of<EPV>(x));
 #pragma unroll
-            for (int i = 0; i < EPV; ++i) acc.add(x[i], c);
+            for (int i = 0; i < EPV; ++i) add(x[i]);
+            if constexpr (STATS) stat_vec(x, int64_t(v) * EPV, EPV);
         }
     } else {
         for (int64_t v = tid; v < V; v += kThreads) {
             const float x = E::load1(base + v);
-            acc.raise(x, c);
-            acc.add(x, c);
+            raise(x);
+            add(x);
+            if constexpr (STATS) stat_elem(x, v);
         }
     }
 
@@ -174,6 +251,16 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
         red[1][wave] = s;
         red[2][wave] = u;
     }
+    if constexpr (STATS) {
+        const float s2 = wave_sum(st.s2 * sc * sc);
+        const float sx = wave_sum(st.sx);
+        const float beats = wave_sum(float(st.beats));  // exact: the host admits vocab < 2^24 only
+        if (lane == 0) {
+            red[3][wave] = s2;
+            red[4][wave] = sx;
+            red[5][wave] = beats;
+        }
+    }
     __syncthreads();
     if (tid == 0) {
         float S = 0.f, U = 0.f;
@@ -181,6 +268,20 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
         for (int w = 0; w < NW; ++w) {
             S += red[1][w];
             U += red[2][w];
+        }
+        if constexpr (STATS) {
+            float S2 = 0.f, SX = 0.f, beats = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                S2 += red[3][w];
+                SX += red[4][w];
+                beats += red[5][w];
+            }
+            float* o = a.out_stats + row * 4;
+            o[0] = SX / float(V);
+            o[1] = logf(S2) - 2.f * logf(S);  // log sum_v softmax(z)_v^2: the common reference cancels
+            o[2] = (tpos >= 0 && beats == 0.f) ? 1.f : 0.f;
+            o[3] = 0.f;
         }
         // lse = R*ln2 + ln S with ln2 split in two so that the product carries no rounding of ln2
         constexpr float kLn2Hi = 0.693145751953125f, kLn2Lo = 1.42860677e-06f;
@@ -365,7 +466,7 @@ extern "C" int trlk_logp_entropy_fwd(const void* d_logits, int dtype, int64_t n_
                                      int64_t vocab, int64_t seq_stride, int64_t row_stride, const int64_t* d_index,
                                      int32_t n_index, float temperature, const uint8_t* d_row_mask,
                                      float* d_out_logp, float* d_out_entropy, float* d_out_lse,
-                                     int32_t* d_error_flag, trlk_stream_t stream) {
+                                     float* d_out_row_stats, int32_t* d_error_flag, trlk_stream_t stream) {
     clear_error();
     if (int rc = check_view("logp_entropy_fwd: logits", d_logits, dtype, n_seq, rows_per_seq, vocab, seq_stride,
                             row_stride))
@@ -377,21 +478,28 @@ extern "C" int trlk_logp_entropy_fwd(const void* d_logits, int dtype, int64_t n_
     if (rows == 0) return TRLK_OK;
     TRLK_REQUIRE(n_index == 0 || (d_index != nullptr && d_out_logp != nullptr), TRLK_ERR_NULL_POINTER,
                  "logp_entropy_fwd: index / out_logp pointer is null");
-    TRLK_REQUIRE(n_index > 0 || d_out_entropy != nullptr || d_out_lse != nullptr, TRLK_ERR_NULL_POINTER,
-                 "logp_entropy_fwd: no output requested");
+    TRLK_REQUIRE(n_index > 0 || d_out_entropy != nullptr || d_out_lse != nullptr || d_out_row_stats != nullptr,
+                 TRLK_ERR_NULL_POINTER, "logp_entropy_fwd: no output requested");
+    TRLK_REQUIRE(d_out_row_stats == nullptr || vocab < (int64_t(1) << 24), TRLK_ERR_UNSUPPORTED,
+                 "logp_entropy_fwd: row statistics need vocab < 2^24 (got %lld)", (long long)vocab);
 
     FwdArgs a{d_logits,    rows_per_seq, vocab,         seq_stride, row_stride,  d_index,
               n_index,     temperature,  d_row_mask,    d_out_logp, d_out_entropy, d_out_lse,
-              d_error_flag};
+              d_out_row_stats, d_error_flag};
     const size_t es = elem_size(dtype);
     const bool vec = aligned16(d_logits, es, {seq_stride, row_stride}) && vocab % int64_t(16 / es) == 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)rows), block(kThreads);
-#define TRLK_LAUNCH_FWD(DT)                                                             \
-    if (vec)                                                                            \
-        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, true>), grid, block, 0, s, a);  \
-    else                                                                                \
-        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, false>), grid, block, 0, s, a);
+    const bool stats = d_out_row_stats != nullptr;
+#define TRLK_LAUNCH_FWD(DT)                                                                    \
+    if (vec && stats)                                                                          \
+        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, true, true>), grid, block, 0, s, a);   \
+    else if (vec)                                                                              \
+        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, true, false>), grid, block, 0, s, a);  \
+    else if (stats)                                                                            \
+        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, false, true>), grid, block, 0, s, a);  \
+    else                                                                                       \
+        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, false, false>), grid, block, 0, s, a);
     if (dtype == TRLK_F32) {
         TRLK_LAUNCH_FWD(TRLK_F32)
     } else if (dtype == TRLK_BF16) {

@@ -6,6 +6,7 @@ every trainer module, and the loss is a trainer method.  `patch_trl()` therefore
     in `trl.trainer.utils` **and** in every already-imported `trl.*` module that holds its own reference;
   * `trl.trainer.sft_trainer._chunked_cross_entropy_loss` (the default SFT loss);
   * `GRPOTrainer._get_per_token_logps_and_entropies` / `_compute_loss` (optional, `grpo=True`);
+  * `DPOTrainer._compute_loss` (optional, `dpo=True`): one pass over the logits instead of six;
   * the fused-linear loss operators behind `use_liger_kernel` (optional, `liger=True`): the names
     `LigerFusedLinearGRPOLoss` / `LigerFusedLinearDPOLoss` and `is_liger_kernel_available` in
     `trl.trainer.grpo_trainer` / `trl.trainer.dpo_trainer` (trl/trainer/grpo_trainer.py:1020-1044,
@@ -31,7 +32,7 @@ def _set(mod, name, value) -> None:
     setattr(mod, name, value)
 
 
-def patch_trl(grpo: bool = True, liger: bool = False) -> int:
+def patch_trl(grpo: bool = True, liger: bool = False, dpo: bool = False) -> int:
     """Returns the number of names rebound.  Needs `trl` to be importable."""
     import trl.trainer.utils as ref_utils
 
@@ -65,6 +66,14 @@ def patch_trl(grpo: bool = True, liger: bool = False) -> int:
             _saved.append((GRPOTrainer, name, GRPOTrainer.__dict__[name]))
             setattr(GRPOTrainer, name, getattr(_grpo.GRPOLossMixin, name))
             count += 1
+    if dpo:
+        from trl.trainer.dpo_trainer import DPOTrainer
+
+        from .trainer.dpo_trainer import DPOLossMixin
+
+        _saved.append((DPOTrainer, "_compute_loss", DPOTrainer.__dict__["_compute_loss"]))
+        DPOTrainer._compute_loss = DPOLossMixin._compute_loss
+        count += 1
     if liger:
         import trl.trainer.dpo_trainer as ref_dpo
         import trl.trainer.grpo_trainer as ref_grpo

@@ -62,13 +62,7 @@ def _check_logits3d(logits: Tensor) -> None:
         raise ValueError("the vocabulary axis of the logits must be contiguous")
 
 
-@torch.library.custom_op("trl_amd::logp_entropy_fwd", mutates_args=(), device_types="cuda")
-def logp_entropy_fwd(
-    logits: Tensor, index: Tensor, temperature: float, keep_start: int, keep_len: int, row_mask: Optional[Tensor]
-) -> tuple[Tensor, Tensor, Tensor]:
-    """logits [n_seq, L, V] (strided view, last axis contiguous); rows keep_start..keep_start+keep_len
-    of every sequence are processed.  index int64 [n_seq*keep_len, K].  Returns fp32
-    (logp [rows, K], entropy [rows], lse [rows])."""
+def _run_logp_entropy_fwd(logits, index, temperature, keep_start, keep_len, row_mask, with_stats):
     _check_logits3d(logits)
     n_seq, _, vocab = logits.shape
     rows = n_seq * keep_len
@@ -77,21 +71,32 @@ def logp_entropy_fwd(
     logp = torch.empty((rows, k), dtype=torch.float32, device=dev)
     ent = torch.empty((rows,), dtype=torch.float32, device=dev)
     lse = torch.empty((rows,), dtype=torch.float32, device=dev)
+    stats = torch.empty((rows, 4), dtype=torch.float32, device=dev) if with_stats else None
     if rows == 0:
-        return logp, ent, lse
+        return logp, ent, lse, stats
     index = index.contiguous()
     view = logits[:, keep_start : keep_start + keep_len]
     with torch.cuda.device(dev):
         check(
             lib.trlk_logp_entropy_fwd(
                 view.data_ptr(), dtype_code(logits.dtype), n_seq, keep_len, vocab, view.stride(0), view.stride(1),
-                ptr(index), k, temperature, ptr(row_mask), ptr(logp), ptr(ent), ptr(lse), ptr(_error_flag(dev)),
-                current_stream(dev),
+                ptr(index), k, temperature, ptr(row_mask), ptr(logp), ptr(ent), ptr(lse), ptr(stats),
+                ptr(_error_flag(dev)), current_stream(dev),
             )
         )
     if _SYNC_CHECKS:
         check_device_errors()
-    return logp, ent, lse
+    return logp, ent, lse, stats
+
+
+@torch.library.custom_op("trl_amd::logp_entropy_fwd", mutates_args=(), device_types="cuda")
+def logp_entropy_fwd(
+    logits: Tensor, index: Tensor, temperature: float, keep_start: int, keep_len: int, row_mask: Optional[Tensor]
+) -> tuple[Tensor, Tensor, Tensor]:
+    """logits [n_seq, L, V] (strided view, last axis contiguous); rows keep_start..keep_start+keep_len
+    of every sequence are processed.  index int64 [n_seq*keep_len, K].  Returns fp32
+    (logp [rows, K], entropy [rows], lse [rows])."""
+    return _run_logp_entropy_fwd(logits, index, temperature, keep_start, keep_len, row_mask, False)[:3]
 
 
 @logp_entropy_fwd.register_fake
@@ -99,6 +104,22 @@ def _(logits, index, temperature, keep_start, keep_len, row_mask):
     rows = logits.shape[0] * keep_len
     f = lambda *s: torch.empty(s, dtype=torch.float32, device=logits.device)  # noqa: E731
     return f(rows, index.shape[-1]), f(rows), f(rows)
+
+
+@torch.library.custom_op("trl_amd::logp_entropy_stats_fwd", mutates_args=(), device_types="cuda")
+def logp_entropy_stats_fwd(
+    logits: Tensor, index: Tensor, temperature: float, keep_start: int, keep_len: int, row_mask: Optional[Tensor]
+) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    """As `logp_entropy_fwd`, plus the fp32 row statistics `[rows, 4]` of the same pass: mean logit,
+    log sum_v p_v^2, whether index[:, 0] is the row's arg-max (first maximal position), 0."""
+    return _run_logp_entropy_fwd(logits, index, temperature, keep_start, keep_len, row_mask, True)
+
+
+@logp_entropy_stats_fwd.register_fake
+def _(logits, index, temperature, keep_start, keep_len, row_mask):
+    rows = logits.shape[0] * keep_len
+    f = lambda *s: torch.empty(s, dtype=torch.float32, device=logits.device)  # noqa: E731
+    return f(rows, index.shape[-1]), f(rows), f(rows), f(rows, 4)
 
 
 @torch.library.custom_op("trl_amd::logp_entropy_bwd", mutates_args=(), device_types="cuda")
@@ -138,13 +159,13 @@ def _(logits, index, temperature, keep_start, keep_len, lse, entropy, g_logp, g_
 
 def _lpe_setup(ctx, inputs, output):
     logits, index, temperature, keep_start, keep_len, row_mask = inputs
-    _, ent, lse = output
+    _, ent, lse = output[:3]
     ctx.save_for_backward(logits, index, lse, ent)
     ctx.cfg = (temperature, keep_start, keep_len)
     ctx.set_materialize_grads(False)
 
 
-def _lpe_backward(ctx, g_logp, g_ent, g_lse):
+def _lpe_backward(ctx, g_logp, g_ent, g_lse, g_stats=None):
     logits, index, lse, ent = ctx.saved_tensors
     temperature, keep_start, keep_len = ctx.cfg
     # the lse output only exists to be saved for this backward; a gradient arriving there is ignored
@@ -157,6 +178,7 @@ def _lpe_backward(ctx, g_logp, g_ent, g_lse):
 
 
 logp_entropy_fwd.register_autograd(_lpe_backward, setup_context=_lpe_setup)
+logp_entropy_stats_fwd.register_autograd(_lpe_backward, setup_context=_lpe_setup)
 
 
 # --------------------------------------------------------------------------------------------

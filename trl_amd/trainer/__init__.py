@@ -1,4 +1,5 @@
-from .dpo_trainer import dpo_loss_from_logits, dpo_per_token_logps, dpo_sigmoid_loss
+from .dpo_trainer import (DPOLossMixin, dpo_compute_loss, dpo_loss_from_logits, dpo_metrics_to_dict, dpo_per_token_logps,
+                          dpo_sequence_logps, dpo_sigmoid_loss)
 from .grpo_trainer import (GRPOLossMixin, get_high_entropy_mask, get_off_policy_mask, group_advantages, grpo_loss,
                            metrics_to_dict, per_token_logps_and_entropies)
 from .rloo_trainer import rloo_advantages, rloo_loss
