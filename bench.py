@@ -43,6 +43,9 @@ WORKLOADS = {
     "head_c5": dict(B=16, T=2048, V=151936, H=3584, temperature=1.0, G=8, min_len=64, beta=0.04, eps_low=0.2,
                     eps_high=0.2, rewards="normal", head=True,
                     desc="fused lm_head + log-prob + GRPO loss fwd+bwd, hidden bf16 [16x2048,3584], W bf16 [151936,3584]"),
+    "dpo_c2": dict(B=64, T=2048, V=128256, beta=0.1, dpo=True,
+                   desc="DPO sequence log-probs + sigmoid loss fwd+bwd, bf16 logits [64,2048,128256], 32 pairs, "
+                        "prompt~U[64,512], completion~U[128,1536]"),
     "tiny": dict(B=8, T=64, V=151936, temperature=0.9, G=8, min_len=8, beta=0.04, eps_low=0.2, eps_high=0.2,
                  rewards="normal", desc="reduced-size functional check (not a benchmark configuration)"),
 }
@@ -197,6 +200,95 @@ def bench_head(args, w):
     print(json.dumps(result))
 
 
+def bench_dpo(args, w):
+    """Config 2: `DPOTrainer._compute_loss` arithmetic (sigmoid loss, given reference log-probs) forward + backward
+    to dlogits.  Headline = every shifted row computed; `mask_aware` = only the completion rows are read."""
+    import trl_amd
+    from trl_amd import ops
+
+    dev = torch.device("cuda:0")
+    B, L, V = w["B"], w["T"], w["V"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    logits = torch.empty((B, L, V), dtype=torch.bfloat16, device=dev)
+    for b in range(B):
+        logits[b] = (2.0 * torch.randn((L, V), generator=g, device=dev)).bfloat16()
+    ids = torch.randint(0, V, (B, L), generator=g, device=dev)
+    prompt = torch.randint(64, 513, (B // 2,), generator=g, device=dev).repeat(2)
+    comp = torch.randint(128, 1537, (B,), generator=g, device=dev)
+    pos = torch.arange(L, device=dev)[None]
+    cmask = ((pos >= prompt[:, None]) & (pos < (prompt + comp)[:, None])).long()
+    with torch.no_grad():
+        seq = trl_amd.dpo_sequence_logps(logits, ids, cmask)
+    ref = seq + 0.5 * torch.randn((B,), generator=g, device=dev)
+    leaf = logits.requires_grad_(True)
+    R = B * (L - 1)
+
+    def step(skip):
+        leaf.grad = None
+        loss, _ = trl_amd.dpo_compute_loss(leaf, ids, cmask, ref[: B // 2], ref[B // 2:], beta=w["beta"],
+                                           skip_masked_rows=skip)
+        loss.backward()
+        return loss
+
+    def timed(skip):
+        for _ in range(args.warmup):
+            step(skip)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            loss = step(skip)
+        e1.record()
+        torch.cuda.synchronize()
+        return max((time.perf_counter() - t0) * 1e3, e0.elapsed_time(e1)) / args.steps, float(loss.detach())
+
+    ms_dense, loss_dense = timed(False)
+    ms_aware, loss_aware = timed(True)
+    assert abs(loss_dense - loss_aware) <= 1e-6 * max(1.0, abs(loss_dense)), "mask-aware loss differs"
+    idx = ids[:, 1:].reshape(R, 1).contiguous()
+    active = int(cmask[:, 1:].sum())
+    with torch.no_grad():
+        _, _, lse, _ = ops.logp_entropy_stats_fwd(logits.detach(), idx, 1.0, 0, L - 1, None)
+        g_logp = (cmask[:, 1:].reshape(R, 1) * 0.01).float().contiguous()
+
+        def time_kernel(fn, reps=5):
+            fn()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                out = fn()
+                del out
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / reps
+
+        fwd_ms = time_kernel(lambda: ops.logp_entropy_stats_fwd(logits.detach(), idx, 1.0, 0, L - 1, None))
+        bwd_ms = time_kernel(lambda: ops.logp_entropy_bwd(logits.detach(), idx, 1.0, 0, L - 1, lse, None, g_logp, None))
+    row_bytes = V * 2
+    fwd_bytes = R * row_bytes
+    bwd_bytes = active * 2 * row_bytes + (B * L - active) * row_bytes  # masked rows and the last position: zero fill
+    result = {
+        "metric": "tokens/sec + achieved HBM TB/s (% of peak) for DPO sequence logps + sigmoid loss fwd+bwd",
+        "value": R / (ms_dense * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_dense, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "description": w["desc"], "rows": R, "vocab": V, "active_rows": active,
+                   "loss": loss_dense},
+        "roofline": {"bound": "hbm", "kernel": "logp_entropy_bwd_kernel (K3)", "achieved": bwd_bytes / (bwd_ms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": None, "algorithmic_bytes": bwd_bytes, "avg_launch_ms": bwd_ms},
+        "kernels": {"logp_entropy_fwd_kernel with row statistics (K1)": {
+            "avg_launch_ms": fwd_ms, "algorithmic_bytes": fwd_bytes, "achieved_GBps": fwd_bytes / (fwd_ms * 1e-3) / 1e9,
+            "frac": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}},
+        "mask_aware": {"ms_per_step": ms_aware, "tokens_per_s": R / (ms_aware * 1e-3),
+                       "note": "only rows inside the completion mask are read; loss, metrics and dlogits identical"},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -221,6 +313,9 @@ def main():
     if w.get("head"):
         torch.cuda.set_device(0)
         return bench_head(args, w)
+    if w.get("dpo"):
+        torch.cuda.set_device(0)
+        return bench_dpo(args, w)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     B, T, V = w["B"], w["T"], w["V"]
