@@ -396,3 +396,38 @@ def test_golden_rloo_compute_loss(amd):
             assert abs(float(metrics[i]) - case["metrics"][name]) <= 1e-6, name
     r = torch.tensor([1.0, 2.0, 4.0, 0.5, float("nan"), 2.5])
     torch.testing.assert_close(amd.rloo_advantages(r.to(DEV), 3).cpu(), oracle.rloo_advantages(r, 3))
+
+
+@pytest.mark.parametrize("skip_masked", [False, True])
+def test_rloo_mixin_compute_loss(amd, skip_masked):
+    """`RLOOLossMixin._compute_loss` on the mocked trainer the reference's own method ran on."""
+    cases, g = load_golden("rloo_compute_loss")
+    for case in cases:
+        c = f"c{case['id']}_"
+        B, P, T, V = case["shape"]
+
+        class Trainer(amd.RLOOLossMixin):
+            pass
+
+        tr = Trainer()
+        tr.accelerator = _Identity()
+        tr.temperature = case["temperature"]
+        tr.model_kwarg_keys = set()
+        tr.aux_loss_enabled = False
+        tr.epsilon_low, tr.epsilon_high = case["eps_low"], case["eps_high"]
+        tr._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
+        tr.model = SimpleNamespace(training=True)
+        tr.trl_amd_skip_masked_rows = skip_masked
+        leaf = _t(g[c + "logits"]).to(DEV).requires_grad_(True)
+        inputs = dict(
+            prompt_ids=_t(g[c + "prompt_ids"]).to(DEV), prompt_mask=torch.ones(B, P, dtype=torch.long, device=DEV),
+            completion_ids=_t(g[c + "completion_ids"]).to(DEV), completion_mask=_t(g[c + "completion_mask"]).to(DEV),
+            old_logps=_t(g[c + "old_logps"]).to(DEV), advantages=_t(g[c + "advantages"]).to(DEV))
+        loss = tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None), inputs)
+        loss.backward()
+        want = float(g[c + "out_loss"])
+        assert abs(float(loss) - want) <= 1e-5 * max(1.0, abs(want))
+        assert _rel_l2(leaf.grad, _t(g[c + "out_dlogits"])) < 1e-4
+        got = {k: v[-1] for k, v in tr._metrics["train"].items()}
+        for name, want_m in case["metrics"].items():
+            assert abs(got[name] - want_m) <= 1e-5 * max(1.0, abs(want_m)), (name, got[name], want_m)

@@ -7,6 +7,7 @@ every trainer module, and the loss is a trainer method.  `patch_trl()` therefore
   * `trl.trainer.sft_trainer._chunked_cross_entropy_loss` (the default SFT loss);
   * `GRPOTrainer._get_per_token_logps_and_entropies` / `_compute_loss` (optional, `grpo=True`);
   * `DPOTrainer._compute_loss` (optional, `dpo=True`): one pass over the logits instead of six;
+  * `RLOOTrainer._get_per_token_logps_and_entropies` / `_compute_loss` (optional, `rloo=True`);
   * the fused-linear loss operators behind `use_liger_kernel` (optional, `liger=True`): the names
     `LigerFusedLinearGRPOLoss` / `LigerFusedLinearDPOLoss` and `is_liger_kernel_available` in
     `trl.trainer.grpo_trainer` / `trl.trainer.dpo_trainer` (trl/trainer/grpo_trainer.py:1020-1044,
@@ -32,7 +33,7 @@ def _set(mod, name, value) -> None:
     setattr(mod, name, value)
 
 
-def patch_trl(grpo: bool = True, liger: bool = False, dpo: bool = False) -> int:
+def patch_trl(grpo: bool = True, liger: bool = False, dpo: bool = False, rloo: bool = False) -> int:
     """Returns the number of names rebound.  Needs `trl` to be importable."""
     import trl.trainer.utils as ref_utils
 
@@ -65,6 +66,15 @@ def patch_trl(grpo: bool = True, liger: bool = False, dpo: bool = False) -> int:
         for name in ("_get_per_token_logps_and_entropies", "_compute_loss"):
             _saved.append((GRPOTrainer, name, GRPOTrainer.__dict__[name]))
             setattr(GRPOTrainer, name, getattr(_grpo.GRPOLossMixin, name))
+            count += 1
+    if rloo:
+        from trl.trainer.rloo_trainer import RLOOTrainer
+
+        from .trainer.rloo_trainer import RLOOLossMixin
+
+        for name in ("_get_per_token_logps_and_entropies", "_compute_loss"):
+            _saved.append((RLOOTrainer, name, RLOOTrainer.__dict__[name]))
+            setattr(RLOOTrainer, name, getattr(RLOOLossMixin, name))
             count += 1
     if dpo:
         from trl.trainer.dpo_trainer import DPOTrainer
