@@ -311,6 +311,7 @@ def grpo_loss(
     top_entropy_quantile: float = 1.0,
     importance_sampling_ratio: torch.Tensor | None = None,
     entropy_coef: float = 0.0,
+    adaptive_entropy: dict | None = None,
     sapo_temperature_pos: float = 1.0,
     sapo_temperature_neg: float = 1.05,
     vespo_params: tuple[float, float, float, float] = (2.0, 3.0, 3.0, 2.0),
@@ -365,7 +366,7 @@ def grpo_loss(
         temps = torch.where(adv > 0, sapo_temperature_pos, sapo_temperature_neg)
         per_token_loss = -(torch.sigmoid(temps * (coef_1 - 1)) * 4 / temps) * adv
     elif loss_type == "vespo":  # (:3096-3107)
-        phi_seq = get_gamma_weights(adv, log_ratio, mask, None, *vespo_params)
+        phi_seq = get_gamma_weights(adv, log_ratio, mask, importance_sampling_ratio, *vespo_params)
         per_token_loss = -phi_seq * adv * per_token_logps
     else:
         raise ValueError(f"Unknown loss type: {loss_type}")
@@ -409,15 +410,35 @@ def grpo_loss(
         policy_loss = loss.detach()
 
     metrics: dict[str, float] = {}
-    if entropy_coef != 0.0:
+    ad = adaptive_entropy
+    if entropy_coef != 0.0 or ad is not None:
         eff = mask if entropy_mask is None else mask * entropy_mask
         if loss_type in ("dapo", "cispo", "vespo"):
             ent_term = (entropies * eff).sum() / normalizer
         else:
             ent_term = (entropies * eff).sum() / eff.sum().clamp(min=1.0) / normalizer
-        loss = loss - entropy_coef * ent_term
+        # adaptive control applies the coefficient only while the last window's entropy is at or below the target (:3176-3179)
+        apply_coef = entropy_coef if ad is None or ad["last_world_entropy"] <= ad["target"] else 0.0
+        loss = loss - apply_coef * ent_term
         metrics["policy_loss"] = float(policy_loss)
-        metrics["entropy_coef"] = float(entropy_coef)  # logged at optimizer-step boundaries (:3214-3215)
+        coef_after = entropy_coef
+        sync = True if ad is None else ad.get("sync_gradients", True)
+        if ad is not None and ad.get("train", True):  # window accumulation and update at the step boundary (:3186-3210)
+            stats = torch.stack([(entropies * eff).sum(), eff.sum().float()]).detach()
+            window = stats if ad.get("window") is None else torch.as_tensor(ad["window"], dtype=stats.dtype) + stats
+            last = ad["last_world_entropy"]
+            if sync:
+                last = float(window[0] / window[1].clamp(min=1.0))
+                if last <= ad["target"]:
+                    coef_after = min(entropy_coef + ad["delta"], ad["max"])
+                else:
+                    coef_after = max(entropy_coef - ad["delta"], ad["min"])
+                window = None
+            metrics["state/entropy_coef"] = float(coef_after)
+            metrics["state/last_world_entropy"] = float(last)
+            metrics["state/window"] = None if window is None else [float(x) for x in window]
+        if sync:
+            metrics["entropy_coef"] = float(coef_after)  # logged at optimizer-step boundaries (:3214-3215)
 
     def seq_mean(x):
         if x.shape[1] == 1:

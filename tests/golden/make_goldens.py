@@ -97,6 +97,16 @@ GRPO_CASES = [
     dict(name="bnpo_seq_delta", loss_type="bnpo", beta=0.0, eps_low=0.03, eps_high=0.04, is_level="sequence", delta=1.02),
     dict(name="grpo_seq_offpolicy_entq", loss_type="grpo", beta=0.04, eps_low=0.05, eps_high=0.05, is_level="sequence",
          off_policy=0.02, top_entropy_quantile=0.5),
+    dict(name="adaptive_below_target", loss_type="grpo", beta=0.04, eps_low=0.2, eps_high=0.2, entropy_coef=0.01,
+         adaptive=dict(target=5.0, delta=0.005, max=0.012, min=0.0, last=1.0, sync=True)),
+    dict(name="adaptive_above_target", loss_type="dapo", beta=0.0, eps_low=0.2, eps_high=0.2, entropy_coef=0.02,
+         adaptive=dict(target=0.5, delta=0.005, max=0.1, min=0.0, last=float("inf"), sync=True)),
+    dict(name="adaptive_accumulating", loss_type="bnpo", beta=0.0, eps_low=0.2, eps_high=0.2, entropy_coef=0.02,
+         grad_accum=2, adaptive=dict(target=5.0, delta=0.005, max=0.1, min=0.0, last=2.0, sync=False, window=[3.0, 2.0])),
+    dict(name="adaptive_window_close", loss_type="dr_grpo", beta=0.0, eps_low=0.2, eps_high=0.2, entropy_coef=0.0,
+         grad_accum=2, adaptive=dict(target=5.0, delta=0.005, max=0.1, min=0.0, last=9.0, sync=True, window=[30.0, 12.0])),
+    dict(name="vllm_is_ratio", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, is_ratio=True),
+    dict(name="vespo_is_ratio", loss_type="vespo", beta=0.0, eps_low=0.2, eps_high=0.2, is_ratio=True),
 ]
 
 
@@ -123,9 +133,14 @@ def make_grpo(GRPOTrainer, out_dir):
         trainer.accelerator = _fake_accelerator()
         trainer.temperature = temperature
         trainer.model_kwarg_keys = set()
-        trainer._entropy_bonus_enabled = case.get("entropy_coef", 0.0) != 0.0
+        ad = case.get("adaptive")
+        trainer._entropy_bonus_enabled = case.get("entropy_coef", 0.0) != 0.0 or ad is not None
         trainer.entropy_coef = case.get("entropy_coef", 0.0)
-        trainer.use_adaptive_entropy = False
+        trainer.use_adaptive_entropy = ad is not None
+        if ad is not None:
+            trainer._last_world_entropy = ad["last"]
+            trainer._entropy_window_stats = torch.tensor(ad["window"]) if "window" in ad else None
+            trainer.accelerator.sync_gradients = ad["sync"]
         trainer.aux_loss_enabled = False
         trainer.top_entropy_quantile = case.get("top_entropy_quantile", 1.0)
         trainer.off_policy_mask_threshold = case.get("off_policy")
@@ -134,13 +149,16 @@ def make_grpo(GRPOTrainer, out_dir):
         trainer.loss_type = case["loss_type"]
         trainer.epsilon_low = case["eps_low"]
         trainer.epsilon_high = case["eps_high"]
-        trainer.use_vllm = False
-        trainer.vllm_importance_sampling_correction = False
+        trainer.use_vllm = bool(case.get("is_ratio"))
+        trainer.vllm_importance_sampling_correction = bool(case.get("is_ratio"))
         trainer.max_completion_length = T
         trainer.current_gradient_accumulation_steps = case.get("grad_accum", 1)
         trainer.args = SimpleNamespace(delta=case.get("delta"), use_bias_correction_kl=case.get("bias_kl", False),
                                        sapo_temperature_pos=1.0, sapo_temperature_neg=1.05, vespo_k_pos=2.0,
                                        vespo_lambda_pos=3.0, vespo_k_neg=3.0, vespo_lambda_neg=2.0)
+        if ad is not None:
+            trainer.args.entropy_target, trainer.args.entropy_coef_delta = ad["target"], ad["delta"]
+            trainer.args.entropy_coef_max, trainer.args.entropy_coef_min = ad["max"], ad["min"]
         trainer.get_gamma_weights = GRPOTrainer.get_gamma_weights
         trainer._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
         trainer.model = SimpleNamespace(training=True)
@@ -170,6 +188,8 @@ def make_grpo(GRPOTrainer, out_dir):
             inputs["old_per_token_logps"] = base_logps + 0.15 * torch.randn(B, T, generator=g)
         if case["beta"] != 0.0:
             inputs["ref_per_token_logps"] = base_logps + 0.3 * torch.randn(B, T, generator=g)
+        if case.get("is_ratio"):
+            inputs["importance_sampling_ratio"] = 0.5 + torch.rand(B, T, generator=g)
 
         leaf = logits.clone().requires_grad_(True)
 
@@ -200,12 +220,20 @@ def make_grpo(GRPOTrainer, out_dir):
             arrays[pre + "old_per_token_logps"] = _np(inputs["old_per_token_logps"])
         if "ref_per_token_logps" in inputs:
             arrays[pre + "ref_per_token_logps"] = _np(inputs["ref_per_token_logps"])
+        if "importance_sampling_ratio" in inputs:
+            arrays[pre + "importance_sampling_ratio"] = _np(inputs["importance_sampling_ratio"])
         arrays[pre + "out_logps"] = _np(captured["logps"])
         arrays[pre + "out_entropies"] = _np(captured["entropies"])
         arrays[pre + "out_loss"] = _np(loss)
         arrays[pre + "out_dlogits"] = _np(leaf.grad)
         metrics = {k: float(v[-1]) for k, v in trainer._metrics["train"].items()}
-        index.append(dict(case, id=ci, shape=[B, P, T, V], metrics=metrics))
+        entry = dict(case, id=ci, shape=[B, P, T, V], metrics=metrics)
+        if ad is not None:  # the controller's state after the call
+            win = trainer._entropy_window_stats
+            entry["state_after"] = dict(entropy_coef=float(trainer.entropy_coef),
+                                        last_world_entropy=float(trainer._last_world_entropy),
+                                        window=None if win is None else [float(x) for x in win])
+        index.append(entry)
     np.savez_compressed(os.path.join(out_dir, "grpo_compute_loss.npz"), **arrays)
     with open(os.path.join(out_dir, "grpo_compute_loss.json"), "w") as f:
         json.dump(index, f, indent=1)

@@ -57,9 +57,14 @@ def _fake_trainer(amd, case, T, skip_masked=False):
     tr.accelerator = _Identity()
     tr.temperature = case.get("temperature", 1.0)
     tr.model_kwarg_keys = set()
-    tr._entropy_bonus_enabled = case.get("entropy_coef", 0.0) != 0.0
+    ad = case.get("adaptive")
+    tr._entropy_bonus_enabled = case.get("entropy_coef", 0.0) != 0.0 or ad is not None
     tr.entropy_coef = case.get("entropy_coef", 0.0)
-    tr.use_adaptive_entropy = False
+    tr.use_adaptive_entropy = ad is not None
+    if ad is not None:
+        tr._last_world_entropy = ad["last"]
+        tr._entropy_window_stats = torch.tensor(ad["window"]) if "window" in ad else None
+        tr.accelerator.sync_gradients = ad["sync"]
     tr.aux_loss_enabled = False
     tr.top_entropy_quantile = case.get("top_entropy_quantile", 1.0)
     tr.off_policy_mask_threshold = case.get("off_policy")
@@ -67,11 +72,14 @@ def _fake_trainer(amd, case, T, skip_masked=False):
     tr.beta = case["beta"]
     tr.loss_type = case["loss_type"]
     tr.epsilon_low, tr.epsilon_high = case["eps_low"], case["eps_high"]
-    tr.use_vllm = False
-    tr.vllm_importance_sampling_correction = False
+    tr.use_vllm = bool(case.get("is_ratio"))
+    tr.vllm_importance_sampling_correction = bool(case.get("is_ratio"))
     tr.max_completion_length = T
     tr.current_gradient_accumulation_steps = case.get("grad_accum", 1)
     tr.args = SimpleNamespace(delta=case.get("delta"), use_bias_correction_kl=case.get("bias_kl", False))
+    if ad is not None:
+        tr.args.entropy_target, tr.args.entropy_coef_delta = ad["target"], ad["delta"]
+        tr.args.entropy_coef_max, tr.args.entropy_coef_min = ad["max"], ad["min"]
     tr._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
     tr.model = SimpleNamespace(training=True)
     tr.trl_amd_skip_masked_rows = skip_masked
@@ -96,7 +104,7 @@ def test_golden_grpo_compute_loss_through_trainer_methods(amd, skip_masked):
             completion_ids=_t(g[c + "completion_ids"]).to(DEV), completion_mask=_t(g[c + "completion_mask"]).to(DEV),
             advantages=_t(g[c + "advantages"]).to(DEV), num_items_in_batch=_t(g[c + "num_items_in_batch"]).to(DEV),
         )
-        for key in ("old_per_token_logps", "ref_per_token_logps"):
+        for key in ("old_per_token_logps", "ref_per_token_logps", "importance_sampling_ratio"):
             if c + key in g:
                 inputs[key] = _t(g[c + key]).to(DEV)
         model = lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None)  # noqa: E731
@@ -134,8 +142,17 @@ def test_golden_grpo_compute_loss_through_trainer_methods(amd, skip_masked):
             got = got_metrics[name]
             ok = (math.isnan(got) and math.isnan(want)) or abs(got - want) <= (2e-2 if low else 1e-5) * max(1.0, abs(want))
             assert ok, (case["name"], name, got, want)
+        if "state_after" in case:  # the adaptive entropy controller's state after the call
+            want = case["state_after"]
+            assert abs(tr.entropy_coef - want["entropy_coef"]) < 1e-9, case["name"]
+            assert abs(tr._last_world_entropy - want["last_world_entropy"]) < 1e-4, case["name"]
+            if want["window"] is None:
+                assert tr._entropy_window_stats is None
+            else:
+                torch.testing.assert_close(tr._entropy_window_stats.cpu(), torch.tensor(want["window"]), rtol=1e-5, atol=1e-4)
+            assert ("entropy_coef" in got_metrics) == ("entropy_coef" in case["metrics"]), case["name"]
         ran += 1
-    assert ran >= 27
+    assert ran >= 33
 
 
 def test_grpo_loss_against_oracle_random(amd):

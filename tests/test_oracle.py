@@ -187,7 +187,8 @@ def _grpo_case(case, g):
     logits = _t(g[c + "logits"], dtype).requires_grad_(True)
     input_ids = torch.cat([_t(g[c + "prompt_ids"]), _t(g[c + "completion_ids"])], 1)
     mask = _t(g[c + "completion_mask"])
-    ent_bonus = case.get("entropy_coef", 0.0) != 0.0
+    ad = case.get("adaptive")
+    ent_bonus = case.get("entropy_coef", 0.0) != 0.0 or ad is not None
     logps, ent = oracle.logps_and_entropies_from_logits(
         logits, input_ids, T, case.get("temperature", 1.0), True, entropy_requires_grad=ent_bonus
     )
@@ -200,7 +201,11 @@ def _grpo_case(case, g):
         grad_accum_steps=case.get("grad_accum", 1), importance_sampling_level=case.get("is_level", "token"),
         use_bias_correction_kl=case.get("bias_kl", False), off_policy_mask_threshold=case.get("off_policy"),
         top_entropy_quantile=case.get("top_entropy_quantile", 1.0), entropy_coef=case.get("entropy_coef", 0.0),
+        importance_sampling_ratio=_t(g[c + "importance_sampling_ratio"]) if c + "importance_sampling_ratio" in g else None,
     )
+    if ad is not None:
+        kw["adaptive_entropy"] = dict(last_world_entropy=ad["last"], window=ad.get("window"), target=ad["target"],
+                                      delta=ad["delta"], max=ad["max"], min=ad["min"], sync_gradients=ad["sync"])
     loss, metrics = oracle.grpo_loss(logps, _t(g[c + "advantages"]), mask, **kw)
     loss.backward()
     return logits, logps, ent, loss, metrics
@@ -208,10 +213,19 @@ def _grpo_case(case, g):
 
 def test_golden_grpo_compute_loss():
     cases, g = load_golden("grpo_compute_loss")
-    assert len(cases) >= 27
+    assert len(cases) >= 33
     for case in cases:
         c = f"c{case['id']}_"
         logits, logps, ent, loss, metrics = _grpo_case(case, g)
+        if "state_after" in case:  # adaptive entropy controller (grpo_trainer.py:3176-3215)
+            want = case["state_after"]
+            assert abs(metrics["state/entropy_coef"] - want["entropy_coef"]) < 1e-9, case["name"]
+            assert abs(metrics["state/last_world_entropy"] - want["last_world_entropy"]) < 1e-5, case["name"]
+            if want["window"] is None:
+                assert metrics["state/window"] is None
+            else:
+                assert max(abs(a - b) for a, b in zip(metrics["state/window"], want["window"])) < 1e-4
+            assert ("entropy_coef" in metrics) == ("entropy_coef" in case["metrics"]), case["name"]
         tol = dict(rtol=1e-5, atol=1e-6)
         torch.testing.assert_close(logps.detach().float(), _t(g[c + "out_logps"]), **tol)
         torch.testing.assert_close(ent.detach().float(), _t(g[c + "out_entropies"]), **tol)

@@ -225,12 +225,10 @@ class GRPOLossMixin:
         return logps, entropies, aux_loss
 
     def _compute_loss(self, model, inputs):
-        """Reference: trl/trainer/grpo_trainer.py:2991-3260, every loss type, token- and sequence-level
-        importance weights; adaptive entropy control is left to the reference."""
+        """Reference: trl/trainer/grpo_trainer.py:2991-3260: every loss type, token- and sequence-level
+        importance weights, static and adaptive entropy bonus."""
         if self.loss_type not in ops.LOSS_TYPES:
             raise ValueError(f"Unknown loss type: {self.loss_type}")
-        if getattr(self, "use_adaptive_entropy", False):
-            raise NotImplementedError("adaptive entropy control is not implemented by trl_amd")
         prompt_ids, prompt_mask = inputs["prompt_ids"], inputs["prompt_mask"]
         completion_ids, completion_mask = inputs["completion_ids"], inputs["completion_mask"]
         input_ids = torch.cat([prompt_ids, completion_ids], dim=1)
@@ -268,6 +266,12 @@ class GRPOLossMixin:
         mode = "train" if self.model.training else "eval"
         grad_accum = self.current_gradient_accumulation_steps if mode == "train" else 1.0
         bonus = bool(getattr(self, "_entropy_bonus_enabled", False))
+        adaptive = bonus and bool(getattr(self, "use_adaptive_entropy", False))
+        # the coefficient of the end of the previous optimizer step applies to the whole accumulation window;
+        # under adaptive control only while the last window's entropy was at or below the target (:3173-3179)
+        apply_coef = self.entropy_coef if bonus else 0.0
+        if adaptive and not (self._last_world_entropy <= self.args.entropy_target):
+            apply_coef = 0.0
         loss, metrics = grpo_loss(
             per_token_logps, advantages, mask, entropies=entropies, old_per_token_logps=old,
             ref_per_token_logps=inputs["ref_per_token_logps"] if self.beta != 0.0 else None,
@@ -276,7 +280,7 @@ class GRPOLossMixin:
             num_items_in_batch=inputs.get("num_items_in_batch"), num_processes=self.accelerator.num_processes,
             grad_accum_steps=grad_accum, use_bias_correction_kl=self.args.use_bias_correction_kl,
             token_weight=token_weight, entropy_mask=None if entropy_mask is None else entropy_mask.float(),
-            entropy_coef=self.entropy_coef if bonus else 0.0,
+            entropy_coef=apply_coef,
             importance_sampling_level=self.importance_sampling_level,
             sapo_temperature_pos=getattr(self.args, "sapo_temperature_pos", 1.0),
             sapo_temperature_neg=getattr(self.args, "sapo_temperature_neg", 1.05),
@@ -302,6 +306,20 @@ class GRPOLossMixin:
         log = self._metrics[mode]
         if bonus:
             log["policy_loss"].append(policy_loss)
+            if adaptive and mode == "train":  # window-global entropy drives the coefficient of the next step (:3186-3210)
+                eff = mask.float() if entropy_mask is None else mask.float() * entropy_mask.float()
+                stats = torch.stack([(entropies.detach() * eff).sum(), eff.sum()])
+                window = getattr(self, "_entropy_window_stats", None)
+                self._entropy_window_stats = stats if window is None else window.to(stats.device) + stats
+                if self.accelerator.sync_gradients:
+                    total = self.accelerator.reduce(self._entropy_window_stats, reduction="sum")
+                    world_entropy = (total[0] / total[1].clamp(min=1.0)).item()
+                    if world_entropy <= self.args.entropy_target:
+                        self.entropy_coef = min(self.entropy_coef + self.args.entropy_coef_delta, self.args.entropy_coef_max)
+                    else:
+                        self.entropy_coef = max(self.entropy_coef - self.args.entropy_coef_delta, self.args.entropy_coef_min)
+                    self._last_world_entropy = world_entropy
+                    self._entropy_window_stats = None
             if mode == "train" and self.accelerator.sync_gradients:
                 log["entropy_coef"].append(self.entropy_coef)
         if self.beta != 0.0:
