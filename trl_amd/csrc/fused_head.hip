@@ -169,19 +169,32 @@ struct DirectLoader {
             bo[j] = uint32_t((int64_t(r) * B.ld + kc * 8) * 2);
         }
     }
+    // One 1 KiB transfer: 16 bytes per lane from `src` to LDS offset `lds` + 16 * lane.  Issued as
+    // inline assembly on purpose: the compiler books a global_load_lds as an access of both memory
+    // and LDS, after which every wait on a fragment read becomes lgkmcnt(0) (it stalls on the
+    // reads just issued); the loop keeps its own vmcnt bookkeeping for these transfers anyway.
+    // (m0 is a reserved register; naming it as clobbered is what tells the compiler not to keep a value there)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+    static __device__ __forceinline__ void transfer(const char* src, uint32_t lds) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds),
+                     "v"(reinterpret_cast<uint64_t>(src))
+                     : "memory", "m0");
+    }
+#pragma clang diagnostic pop
+    __device__ __forceinline__ uint32_t lds_base(int buf) const {
+        return uint32_t(reinterpret_cast<uintptr_t>(smem)) + uint32_t(buf * C::kDenseStage);
+    }
+    // transfer j of a stage (A blocks first, then B blocks)
+    __device__ __forceinline__ void issue_one(int buf, int k0, int j) const {
+        if (j < kBlkA)
+            transfer(abase + int64_t(k0) * 2 + ao[j], lds_base(buf) + (wave + kWaves * j) * 1024);
+        else
+            transfer(bbase + int64_t(k0) * 2 + bo[j - kBlkA], lds_base(buf) + C::kDenseA + (wave + kWaves * (j - kBlkA)) * 1024);
+    }
     __device__ __forceinline__ void issue(int buf, int k0) const {
-        typedef __attribute__((address_space(1))) const void* gptr_t;
-        typedef __attribute__((address_space(3))) void* lptr_t;
-        const char* ap = abase + int64_t(k0) * 2;
-        const char* bp = bbase + int64_t(k0) * 2;
-        char* sa = smem + buf * C::kDenseStage;
-        char* sb = sa + C::kDenseA;
 #pragma unroll
-        for (int j = 0; j < kBlkA; ++j)
-            __builtin_amdgcn_global_load_lds((gptr_t)(ap + ao[j]), (lptr_t)(sa + (wave + kWaves * j) * 1024), 16, 0, 0);
-#pragma unroll
-        for (int j = 0; j < kBlkB; ++j)
-            __builtin_amdgcn_global_load_lds((gptr_t)(bp + bo[j]), (lptr_t)(sb + (wave + kWaves * j) * 1024), 16, 0, 0);
+        for (int j = 0; j < kStageLoads; ++j) issue_one(buf, k0, j);
     }
     // the first kStages tiles of a product; every stage must be free (all reads of the LDS done)
     __device__ __forceinline__ void prologue(int K) const {
@@ -225,7 +238,7 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
     // across the barrier too: the last slice of a stage is already in registers when the workgroup
     // synchronises, so its MFMAs cover the refill of the freed stage and the first fragment reads of
     // the next one.  The compiler's own scheduler sinks every ds_read next to its first use (one
-    // exposed LDS latency per MFMA pair); the sched_group_barrier sequences pin the interleaving.
+    // exposed LDS latency per MFMA pair), so the issue order is pinned explicitly below.
     constexpr int kStageLoads = DirectLoader<BKT>::kStageLoads;
     auto load_frags = [&](int buf, int ks, u32x4(&fa)[MB], u32x4(&fb)[NB]) {
         const char* sa = smem + buf * kDenseStage;
@@ -237,40 +250,69 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
         for (int nb = 0; nb < NB; ++nb)
             fb[nb] = *reinterpret_cast<const u32x4*>(sb + fb_row + nb * 32 * kRowBytes + koff[ks]);
     };
-    auto mfma_all = [&](u32x4(&fa)[MB], u32x4(&fb)[NB]) {
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = mfma<DT>(fa[mb], fb[nb], acc[mb][nb]);
-    };
-    // Issue order of one slice: an MFMA, a fragment read, ... with the slice's `loads` tile transfers
-    // spread evenly between the MFMAs (a burst of transfers would block the wave, and with it its
-    // MFMAs, until the vector memory path has taken them all: it accepts one per 16 clocks).
-    auto interleave = [&](auto reads_tag, auto loads_tag) {
-        constexpr int R = decltype(reads_tag)::value, L = decltype(loads_tag)::value, M = MB * NB;
+    u32x4 fa[2][MB], fb[2][NB];
+    static_assert(KS % 2 == 0 && MB * NB > MB + NB && (kStages - 2) * kStageLoads < 64, "pipeline shape");
+    constexpr std::true_type T{};
+    constexpr std::false_type F{};
+    const int nk = K / BKT;
+    if (!prefetched) loader.prologue(K);
+    if (nk >= kStages)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 1) * kStageLoads) : "memory");
+    else
+        __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    load_frags(0, 0, fa[0], fb[0]);
+    // Exact issue order, pinned instruction by instruction (sched_barrier(0) between the groups):
+    // MFMA i of the slice, then at most one fragment read of the next slice and at most one tile
+    // transfer.  Fragments are read in the order the mb-major MFMA sequence needs them (fa0, fb*,
+    // fa1, ...), so every read has most of a slice between its issue and its first use.  The refill
+    // of a stage is split: the first half of its transfers goes behind the barrier that frees it, the
+    // second half into the first slice of the following step.
+    constexpr int M = MB * NB, R = MB + NB;
+    constexpr int kLoadsPost = (kStageLoads + 1) / 2, kLoadsPre = kStageLoads - kLoadsPost;
+    auto slice = [&](u32x4(&ca)[MB], u32x4(&cb)[NB], auto read_tag, int rbuf, int rks, u32x4(&na)[MB], u32x4(&nb_)[NB],
+                     auto nload_tag, int lbuf, int lk0, int lfirst) {
+        constexpr bool READ = decltype(read_tag)::value;
+        constexpr int NL = decltype(nload_tag)::value;
+        const char* sa = smem + rbuf * kDenseStage;
+        const char* sb = sa + kDenseA;
+        int issued = 0;
 #pragma unroll
         for (int i = 0; i < M; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // MFMA
-            if (i < R) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-            if (L > 0 && (i + 1) * L / M > i * L / M) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);  // VMEM
+            const int mb = i / NB, nb = i % NB;
+            acc[mb][nb] = mfma<DT>(ca[mb], cb[nb], acc[mb][nb]);
+            if (READ && i < R) {
+                // read order: fa[0], fb[0..NB-1], fa[1..MB-1]
+                if (i == 0)
+                    na[0] = *reinterpret_cast<const u32x4*>(sa + fa_row + koff[rks]);
+                else if (i <= NB)
+                    nb_[i - 1] = *reinterpret_cast<const u32x4*>(sb + fb_row + (i - 1) * 32 * kRowBytes + koff[rks]);
+                else
+                    na[i - NB] = *reinterpret_cast<const u32x4*>(sa + fa_row + (i - NB) * 32 * kRowBytes + koff[rks]);
+            }
+            if (NL > 0 && (i + 1) * NL / M > i * NL / M) {
+                loader.issue_one(lbuf, lk0, lfirst + issued);
+                ++issued;
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
-    typedef std::integral_constant<int, MB + NB> reads_t;
-    typedef std::integral_constant<int, kStageLoads> loads_t;
-    typedef std::integral_constant<int, 0> none_t;
-    u32x4 fa[2][MB], fb[2][NB];
-    // One k step.  ISSUE: the stage this step frees at its barrier is refilled, right behind that
-    // barrier, with the tile kStages steps ahead.  FULL: kStages - 2 younger stages are in flight
-    // behind the one the next step needs.  NEXT: there is a following step.
-    auto step = [&](int kt, auto issue_tag, auto full_tag, auto next_tag) {
-        constexpr bool ISSUE = decltype(issue_tag)::value, FULL = decltype(full_tag)::value;
-        constexpr bool NEXT = decltype(next_tag)::value;
-        const int cur = kt & (kStages - 1);
+    typedef std::integral_constant<int, kLoadsPost> post_t;
+    typedef std::integral_constant<int, kLoadsPre> pre_t;
+    typedef std::integral_constant<int, 0> zero_t;
+    // POST / PRE: this step issues the first half of the refill of the stage it frees / the second
+    // half of the refill the previous step started.  FULL, NEXT as above.
+    auto xstep = [&](int kt, auto post_tag, auto pre_tag, auto full_tag, auto next_tag) {
+        constexpr bool POST = decltype(post_tag)::value, PRE = decltype(pre_tag)::value;
+        constexpr bool FULL = decltype(full_tag)::value, NEXT = decltype(next_tag)::value;
+        const int cur = kt & (kStages - 1), prev = (kt - 1) & (kStages - 1);
 #pragma unroll
         for (int ks = 0; ks + 1 < KS; ++ks) {
-            load_frags(cur, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
-            mfma_all(fa[ks & 1], fb[ks & 1]);
-            interleave(reads_t{}, none_t{});
+            if (PRE && ks == 0)
+                slice(fa[ks & 1], fb[ks & 1], T, cur, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1], pre_t{}, prev,
+                      (kt - 1 + kStages) * BKT, kLoadsPost);
+            else
+                slice(fa[ks & 1], fb[ks & 1], T, cur, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1], zero_t{}, 0, 0, 0);
         }
         // every fragment read of this stage has returned and the next stage has landed
         if constexpr (FULL)
@@ -285,34 +327,26 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("" ::: "memory");
-        if constexpr (NEXT) load_frags((kt + 1) & (kStages - 1), 0, fa[0], fb[0]);
-        mfma_all(fa[(KS - 1) & 1], fb[(KS - 1) & 1]);
-        if constexpr (ISSUE) loader.issue(cur, (kt + kStages) * BKT);
-        if constexpr (NEXT && ISSUE)
-            interleave(reads_t{}, loads_t{});
+        constexpr int L = (KS - 1) & 1;
+        const int nxt = (kt + 1) & (kStages - 1);
+        if constexpr (NEXT && POST)
+            slice(fa[L], fb[L], T, nxt, 0, fa[0], fb[0], post_t{}, cur, (kt + kStages) * BKT, 0);
         else if constexpr (NEXT)
-            interleave(reads_t{}, none_t{});
-        __builtin_amdgcn_sched_barrier(0);
+            slice(fa[L], fb[L], T, nxt, 0, fa[0], fb[0], zero_t{}, 0, 0, 0);
+        else
+            slice(fa[L], fb[L], F, 0, 0, fa[0], fb[0], zero_t{}, 0, 0, 0);
     };
-    static_assert(KS % 2 == 0 && MB * NB > MB + NB && (kStages - 2) * kStageLoads < 64, "pipeline shape");
-    constexpr std::true_type T{};
-    constexpr std::false_type F{};
-
-    const int nk = K / BKT;
-    if (!prefetched) loader.prologue(K);
-    if (nk >= kStages)
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 1) * kStageLoads) : "memory");
-    else
-        __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    load_frags(0, 0, fa[0], fb[0]);
+    static_assert(((KS - 1) & 1) == 1, "the last slice of a stage sits in fragment buffer 1, the next stage's first in 0");
     int kt = 0;
-    if (nk >= kStages) {
-        for (; kt + kStages < nk; ++kt) step(kt, T, T, T);
-        step(kt++, F, T, T);  // kt = nk - kStages: every stage has been requested
+    if (nk > kStages) {
+        xstep(kt++, T, F, T, T);
+        for (; kt + kStages < nk; ++kt) xstep(kt, T, T, T, T);
+        xstep(kt++, F, T, T, T);  // kt = nk - kStages: completes the last refill
+    } else if (nk == kStages) {
+        xstep(kt++, F, F, T, T);
     }
-    for (; kt + 1 < nk; ++kt) step(kt, F, F, T);
-    step(kt, F, F, F);
+    for (; kt + 1 < nk; ++kt) xstep(kt, F, F, F, T);
+    xstep(kt, F, F, F, F);
     // every LDS read of this tile completed before the last barrier: the caller may reuse the LDS right away
 }
 
