@@ -214,7 +214,9 @@ int trlk_rloo_loss(const float* d_token_logp, const float* d_mask, const float* 
 /* ---------------------------------------------------------------------------------------
  * K5 / K6  lm_head fused with the log-prob / entropy reduction; the [N, V] logits are never
  * written to memory.  Replaces _ChunkedLogProbFunction (trl/trainer/utils.py:1291-1424):
- *   y = hidden @ weight^T   (bf16/fp16 operands on the matrix cores, fp32 accumulation)
+ *   y = hidden @ weight^T (+ bias)  (bf16/fp16 operands on the matrix cores, fp32 accumulation;
+ *       d_bias: optional fp32 [vocab], the lm_head bias the fused-linear operators behind
+ *       use_liger_kernel take, trl/trainer/grpo_trainer.py:2885-2896, dpo_trainer.py:1287-1289)
  *   z = softcap(y * logit_scale) / temperature,  softcap(x) = cap * tanh(x / cap) if cap > 0
  *   out_logp[n] = z[n, targets[n]] - logsumexp(z[n, :]);  out_entropy[n] = logsumexp - E_p[z];
  *   out_log_z[n] = logsumexp(z[n, :])   (saved for the backward)
@@ -231,8 +233,9 @@ size_t trlk_fused_head_fwd_workspace_bytes(int64_t n_tokens);
 int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, const int64_t* d_targets, int dtype,
                         int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                         int64_t weight_stride, float temperature, float final_logit_softcapping, float logit_scale,
-                        float* d_out_logp, float* d_out_entropy, float* d_out_log_z, float* d_out_target_is_max,
-                        int32_t* d_error_flag, void* d_workspace, size_t workspace_bytes, trlk_stream_t stream);
+                        const float* d_bias, float* d_out_logp, float* d_out_entropy, float* d_out_log_z,
+                        float* d_out_target_is_max, int32_t* d_error_flag, void* d_workspace, size_t workspace_bytes,
+                        trlk_stream_t stream);
 
 /* Backward of the above w.r.t. hidden and weight for an upstream gradient on the log-probs
  * (the entropy output carries no gradient, as in the reference, utils.py:1368):
@@ -241,14 +244,16 @@ int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, const int64_
  *   dense [n_tokens, hidden_size] and [vocab, hidden_size]).
  * The vocabulary is processed in chunks of `chunk_size` rows (rounded up to 256); dz exists only
  * for one chunk at a time, in bf16/fp16, inside the workspace.
+ * d_out_dbias (optional, fp32 [vocab]): sum over tokens of dz, the gradient of d_bias.
  */
 size_t trlk_fused_head_bwd_workspace_bytes(int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t chunk_size);
 
 int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, const int64_t* d_targets, int dtype,
                         int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                         int64_t weight_stride, float temperature, float final_logit_softcapping, float logit_scale,
-                        const float* d_log_z, const float* d_g_logp, int64_t chunk_size, void* d_out_dhidden,
-                        void* d_out_dweight, void* d_workspace, size_t workspace_bytes, trlk_stream_t stream);
+                        const float* d_bias, const float* d_log_z, const float* d_g_logp, int64_t chunk_size,
+                        void* d_out_dhidden, void* d_out_dweight, float* d_out_dbias, void* d_workspace,
+                        size_t workspace_bytes, trlk_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -817,14 +817,18 @@ def chunked_cross_entropy_loss(hidden_states, lm_head_weight, chunk_size, labels
 # Fused-linear operator contracts          trl/trainer/grpo_trainer.py:2885-2907, dpo_trainer.py:1287-1327
 # --------------------------------------------------------------------------------------
 def fused_linear_grpo_loss(hidden, weight, selected_token_ids, loss_mask, advantages, temperature=1.0,
-                           old_per_token_logps=None, ref_per_token_logps=None, vllm_is_ratio=None, **loss_kwargs):
+                           old_per_token_logps=None, ref_per_token_logps=None, vllm_is_ratio=None, bias=None,
+                           **loss_kwargs):
     """What `compute_liger_loss` expects of `self.liger_loss` (grpo_trainer.py:2885-2901), stated with the
     reference's own arithmetic: logits `(hidden @ W.T).float() / T` of every position (utils.py:1328-1337 without
     chunking), `selective_log_softmax`, then `_compute_loss`'s loss (`grpo_loss` above, not divided by the
     accumulation steps, dapo normaliser = active tokens of the batch).  Returns `(loss, [mean_kl]? + [clip_ratio])`
-    with clip_ratio = the region clip ratio."""
+    with clip_ratio = the region clip ratio.  `bias` is the `lm_head` bias (`nn.Linear`: `x @ W.T + b`)."""
     b, t, h = hidden.shape
-    logits = (hidden.reshape(b * t, h) @ weight.t()).float() / temperature
+    logits = hidden.reshape(b * t, h) @ weight.t()
+    if bias is not None:
+        logits = logits + bias
+    logits = logits.float() / temperature
     logps = selective_log_softmax(logits, selected_token_ids.reshape(b * t)).view(b, t)
     beta = loss_kwargs.get("beta", 0.0)
     loss, metrics = grpo_loss(
@@ -836,7 +840,8 @@ def fused_linear_grpo_loss(hidden, weight, selected_token_ids, loss_mask, advant
     return loss, out
 
 
-def fused_linear_dpo_loss(weight, hidden, target, ref_hidden, ref_weight, beta, ignore_index=-100):
+def fused_linear_dpo_loss(weight, hidden, target, ref_hidden, ref_weight, beta, ignore_index=-100, bias=None,
+                          ref_bias=None):
     """What `_compute_loss_liger` expects of `self.liger_loss` (dpo_trainer.py:1287-1301) for the sigmoid loss:
     summed log-probs of the non-ignored targets (as dpo_trainer.py:1347-1350), reference ones without grad,
     `dpo_sigmoid_loss` above.  Returns `(loss, (chosen_logps, rejected_logps, chosen_logits_mean,
@@ -846,14 +851,17 @@ def fused_linear_dpo_loss(weight, hidden, target, ref_hidden, ref_weight, beta, 
     keep = target != ignore_index
     labels = torch.where(keep, target, torch.zeros_like(target))
 
-    def seq_logps(hs, w):
-        logits = (hs.reshape(b * t, h) @ w.t()).float()
+    def seq_logps(hs, w, bi):
+        logits = hs.reshape(b * t, h) @ w.t()
+        if bi is not None:
+            logits = logits + bi
+        logits = logits.float()
         tok = selective_log_softmax(logits, labels.reshape(b * t)).view(b, t)
         return (tok * keep).sum(-1), logits.view(b, t, -1)
 
-    seq, logits = seq_logps(hidden, weight)
+    seq, logits = seq_logps(hidden, weight, bias)
     with torch.no_grad():
-        ref_seq, _ = seq_logps(ref_hidden, ref_weight)
+        ref_seq, _ = seq_logps(ref_hidden, ref_weight, ref_bias)
     pairs = b // 2
     loss, _ = dpo_sigmoid_loss(seq, ref_seq[:pairs], ref_seq[pairs:], beta)
     rewards = beta * (seq.detach() - ref_seq)

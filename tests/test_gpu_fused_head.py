@@ -113,6 +113,34 @@ def test_fused_head_against_fp32_reference(amd, dtype, n, h, v, chunk, temperatu
     torch.testing.assert_close(ent, oent, atol=2e-3, rtol=0)
 
 
+@pytest.mark.parametrize("n,h,v,chunk,softcap,scale", [(300, 256, 1000, 256, None, 1.0), (257, 136, 777, 512, 5.0, 0.5)])
+def test_fused_head_with_bias(amd, n, h, v, chunk, softcap, scale):
+    """z = softcap((hidden @ W.T + bias) * scale) / T: outputs, and the gradients of all three operands."""
+    g = torch.Generator().manual_seed(n + v)
+    hidden = torch.randn(n, h, generator=g).bfloat16()
+    weight = (torch.randn(v, h, generator=g) * (2.0 / h**0.5)).bfloat16()
+    bias = (2.0 * torch.randn(v, generator=g)).bfloat16()
+    labels = torch.randint(0, v, (n,), generator=g)
+    gout = torch.randn(n, generator=g)
+    temperature = 0.8
+    rh, rw, rb = (x.float().requires_grad_(True) for x in (hidden, weight, bias))
+    y = (rh @ rw.t() + rb) * scale
+    if softcap:
+        y = torch.tanh(y / softcap) * softcap
+    lp_all = F.log_softmax(y / temperature, -1)
+    rlp = lp_all.gather(-1, labels[:, None]).squeeze(-1)
+    rent = -(lp_all.exp() * lp_all).sum(-1)
+    (rlp * gout).sum().backward()
+    dh, dw, db = (x.to(DEV).requires_grad_(True) for x in (hidden, weight, bias))
+    lp, ent = amd._ChunkedLogProbFunction.apply(dh, dw, labels.to(DEV), temperature, chunk, softcap, scale, db)
+    (lp * gout.to(DEV)).sum().backward()
+    torch.testing.assert_close(lp.detach().cpu(), rlp.detach(), atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent.cpu(), rent.detach(), atol=2e-3, rtol=0)
+    assert db.grad.dtype == torch.bfloat16
+    for got, want in ((dh, rh), (dw, rw), (db, rb)):
+        assert _rel_l2(got.grad.float(), want.grad) < 1e-2, _rel_l2(got.grad.float(), want.grad)
+
+
 def test_masked_rows_and_scatter(amd):
     # reference tests/test_utils.py:1338-1398: masked == unmasked on completion rows, exact zeros elsewhere,
     # and the lm_head gradient only sees completion rows

@@ -71,9 +71,9 @@ def test_fused_linear_grpo_loss(amd, loss_type, level, beta):
     assert torch.count_nonzero(dh.grad.float().cpu()[mask == 0]) == 0
     assert _rel_l2(dh.grad.float(), oh.grad) < 1e-2
     assert _rel_l2(dw.grad.float(), ow.grad) < 1e-2
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError):  # a bias of the wrong length
         op(_input=dh, lin_weight=dw, selected_token_ids=ids.to(DEV), attention_mask=mask.to(DEV),
-           advantages=adv.to(DEV), bias=torch.zeros(V, device=DEV))
+           advantages=adv.to(DEV), bias=torch.zeros(V + 1, device=DEV))
 
 
 def test_fused_linear_dpo_loss(amd):
@@ -105,3 +105,44 @@ def test_fused_linear_dpo_loss(amd):
     assert _rel_l2(dw.grad.float(), ow.grad) < 1e-2
     with pytest.raises(NotImplementedError):
         amd.FusedLinearDPOLoss(beta=beta, loss_type="ipo")
+
+
+def test_fused_linear_losses_with_lm_head_bias(amd):
+    """`bias` of both operators (`nn.Linear` form `x @ W.T + b`): loss, metrics and the three gradients."""
+    B, T, H, V = 6, 20, 64, 389
+    g, hidden, weight, ids, mask = _problem(33, B, T, H, V)
+    bias = torch.randn(V, generator=g).bfloat16()
+    ref_bias = (bias.float() + 0.1 * torch.randn(V, generator=g)).bfloat16()
+    temperature = 0.9
+    adv = torch.randn(B, generator=g)
+    kw = dict(beta=0.0, epsilon_low=0.2, epsilon_high=0.2, loss_type="dapo", max_completion_length=T)
+    oh, ow, ob = (x.float().requires_grad_(True) for x in (hidden, weight, bias))
+    oloss, om = oracle.fused_linear_grpo_loss(oh, ow, ids, mask, adv, temperature, bias=ob, **kw)
+    oloss.backward()
+    op = amd.FusedLinearGRPOLoss(temperature=temperature, use_ref_model=False, **kw)
+    dh, dw, db = (x.to(DEV).requires_grad_(True) for x in (hidden, weight, bias))
+    loss, m = op(dh, dw, ids.to(DEV), mask.to(DEV), adv.to(DEV), db)
+    loss.backward()
+    assert abs(float(loss) - float(oloss)) <= 1e-3 * max(1.0, abs(float(oloss)))
+    assert db.grad.dtype == torch.bfloat16 and db.grad.shape == (V,)
+    for got, want in ((dh, oh), (dw, ow), (db, ob)):
+        assert _rel_l2(got.grad.float(), want.grad) < 1e-2
+
+    target = torch.where(mask == 1, ids, torch.full_like(ids, -100))
+    ref_hidden = (hidden.float() + 0.1 * torch.randn(B, T, H, generator=g)).bfloat16()
+    ref_weight = (weight.float() + 0.02 * torch.randn(V, H, generator=g)).bfloat16()
+    oh, ow, ob = (x.float().requires_grad_(True) for x in (hidden, weight, bias))
+    oloss, om = oracle.fused_linear_dpo_loss(ow, oh, target, ref_hidden.float(), ref_weight.float(), 0.1, bias=ob,
+                                             ref_bias=ref_bias.float())
+    oloss.backward()
+    dh, dw, db = (x.to(DEV).requires_grad_(True) for x in (hidden, weight, bias))
+    loss, m = amd.FusedLinearDPOLoss(beta=0.1)(dw, dh, target.to(DEV), db, ref_hidden.to(DEV), ref_weight.to(DEV),
+                                                ref_bias.to(DEV))
+    loss.backward()
+    assert abs(float(loss) - float(oloss)) <= 1e-3 * max(1.0, abs(float(oloss)))
+    for i in (0, 1, 5, 6):
+        torch.testing.assert_close(m[i].cpu(), om[i], rtol=1e-3, atol=2e-3)
+    for i in (2, 3):
+        assert abs(float(m[i]) - float(om[i])) <= 1e-3
+    for got, want in ((dh, oh), (dw, ow), (db, ob)):
+        assert _rel_l2(got.grad.float(), want.grad) < 1e-2

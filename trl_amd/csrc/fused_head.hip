@@ -493,6 +493,7 @@ struct HeadArgs {
     const uint16_t* hidden;  // [N, H]
     const uint16_t* weight;  // [V, H]
     const int64_t* targets;  // [N]
+    const float* bias;       // [V] added to hidden . weight[v] before scaling, or null
     int N, V, H;
     int64_t ldh, ldw;
     float logit_scale, inv_t, softcap;  // softcap <= 0: none
@@ -557,7 +558,7 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
         // scale, so the maximum is taken on the raw accumulators and the scale is folded into the
         // exponent's multiplier; sum(e * z) is accumulated as zs * sum(e * y).
         const float zs = a.logit_scale * a.inv_t, zs2 = zs * kLog2e;
-        const bool plain = a.softcap <= 0.f && !partial_tile && zs > 0.f;
+        const bool plain = a.softcap <= 0.f && !partial_tile && zs > 0.f && a.bias == nullptr;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             float bm = -INFINITY;
@@ -572,8 +573,11 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        float z = head_z(acc[mb][nb][r], a);
-                        if (partial_tile && m0 + acc_row(wm, mb, r, lane) >= a.V) z = -INFINITY;
+                        const int v = m0 + acc_row(wm, mb, r, lane);
+                        float y = acc[mb][nb][r];
+                        if (a.bias != nullptr && v < a.V) y += a.bias[v];
+                        float z = head_z(y, a);
+                        if (partial_tile && v >= a.V) z = -INFINITY;
                         acc[mb][nb][r] = z;
                         bm = fmaxf(bm, z);
                     }
@@ -719,7 +723,7 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
     // Common case (no soft-capping, tile inside the chunk): dz = -(g * chain) * exp2(y * zs2 - lzc)
     // with one scale folded into the exponent; the target's one-hot term is patched afterwards.
     const float zs = a.logit_scale * a.inv_t, zs2 = zs * kLog2e;
-    const bool plain = a.softcap <= 0.f && m0 + BM <= a.c1;
+    const bool plain = a.softcap <= 0.f && m0 + BM <= a.c1 && a.bias == nullptr;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         const int tok = n0 + acc_col(wn, nb, lane);
@@ -744,7 +748,9 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int v = m0 + acc_row(wm, mb, r, lane);
-                    float y = acc[mb][nb][r] * a.logit_scale;
+                    float y = acc[mb][nb][r];
+                    if (a.bias != nullptr && v < a.c1) y += a.bias[v];
+                    y *= a.logit_scale;
                     float chain = a.inv_t * a.logit_scale;
                     if (a.softcap > 0.f) {
                         const float th = tanhf(y / a.softcap);
@@ -879,6 +885,27 @@ __global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* in, in
 
 int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
+// d bias[v] = sum over tokens of dz[token, v]: row sums of the transposed dz copy (padding columns are zero).
+template <int DT>
+__global__ __launch_bounds__(256) void dz_row_sum_kernel(const uint16_t* dzT, int64_t ld, int n_cols8, float* out) {
+    typedef Elem<DT> E;
+    const uint16_t* row = dzT + int64_t(blockIdx.x) * ld;
+    float acc = 0.f;
+    for (int c = threadIdx.x; c < n_cols8; c += 256) {
+        const u32x4 w = *reinterpret_cast<const u32x4*>(row + c * 8);
+        float x[8];
+        E::unpack(w, x);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) acc += x[q];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    __shared__ float part[4];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) out[blockIdx.x] = part[0] + part[1] + part[2] + part[3];
+}
+
 // Row strides of the workspace matrices carry 128 extra bytes: their padded extents are multiples
 // of large powers of two (tokens, chunk), and with such a stride the 256 rows of a tile step all
 // fall into the same memory channels.
@@ -971,9 +998,9 @@ extern "C" size_t trlk_fused_head_bwd_workspace_bytes(int64_t n_tokens, int64_t 
 extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, const int64_t* d_targets, int dtype,
                                    int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                                    int64_t weight_stride, float temperature, float final_logit_softcapping,
-                                   float logit_scale, float* d_out_logp, float* d_out_entropy, float* d_out_log_z,
-                                   float* d_out_target_is_max, int32_t* d_error_flag, void* d_workspace,
-                                   size_t workspace_bytes, trlk_stream_t stream) {
+                                   float logit_scale, const float* d_bias, float* d_out_logp, float* d_out_entropy,
+                                   float* d_out_log_z, float* d_out_target_is_max, int32_t* d_error_flag,
+                                   void* d_workspace, size_t workspace_bytes, trlk_stream_t stream) {
     clear_error();
     if (int rc = check_head("fused_head_fwd", d_hidden, d_weight, d_targets, dtype, n_tokens, vocab, hidden_size,
                             hidden_stride, weight_stride, temperature))
@@ -988,6 +1015,7 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
     a.hidden = static_cast<const uint16_t*>(d_hidden);
     a.weight = static_cast<const uint16_t*>(d_weight);
     a.targets = d_targets;
+    a.bias = d_bias;
     a.N = int(n_tokens);
     a.V = int(vocab);
     a.H = int(hidden_size);
@@ -1017,9 +1045,9 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
 extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, const int64_t* d_targets, int dtype,
                                    int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                                    int64_t weight_stride, float temperature, float final_logit_softcapping,
-                                   float logit_scale, const float* d_log_z, const float* d_g_logp, int64_t chunk_size,
-                                   void* d_out_dhidden, void* d_out_dweight, void* d_workspace, size_t workspace_bytes,
-                                   trlk_stream_t stream) {
+                                   float logit_scale, const float* d_bias, const float* d_log_z, const float* d_g_logp,
+                                   int64_t chunk_size, void* d_out_dhidden, void* d_out_dweight, float* d_out_dbias,
+                                   void* d_workspace, size_t workspace_bytes, trlk_stream_t stream) {
     clear_error();
     if (int rc = check_head("fused_head_bwd", d_hidden, d_weight, d_targets, dtype, n_tokens, vocab, hidden_size,
                             hidden_stride, weight_stride, temperature))
@@ -1031,6 +1059,8 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     if (n_tokens == 0) {  // no tokens: both gradients are zero
         hipLaunchKernelGGL(head_fill_kernel, dim3(unsigned((vocab * hidden_size / 2 + 255) / 256)), dim3(256), 0, s,
                            static_cast<float*>(d_out_dweight), vocab * hidden_size / 2, 0.f);
+        if (d_out_dbias)
+            hipLaunchKernelGGL(head_fill_kernel, dim3(unsigned((vocab + 255) / 256)), dim3(256), 0, s, d_out_dbias, vocab, 0.f);
         return launch_status("fused_head_bwd (zero dW)");
     }
     TRLK_REQUIRE(d_log_z && d_g_logp, TRLK_ERR_NULL_POINTER, "fused_head_bwd: log_z / g_logp pointer is null");
@@ -1057,6 +1087,7 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     a.hidden = static_cast<const uint16_t*>(d_hidden);
     a.weight = static_cast<const uint16_t*>(d_weight);
     a.targets = d_targets;
+    a.bias = d_bias;
     a.N = N;
     a.V = V;
     a.H = H;
@@ -1084,6 +1115,15 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
                      ? launch_head(fused_head_dz_kernel<TRLK_BF16>, xcd_patch_grid(n_tb, n_vt), a, s, "fused_head_bwd (dz)")
                      : launch_head(fused_head_dz_kernel<TRLK_F16>, xcd_patch_grid(n_tb, n_vt), a, s, "fused_head_bwd (dz)");
         if (rc) return rc;
+        if (d_out_dbias) {
+            if (dtype == TRLK_BF16)
+                hipLaunchKernelGGL(dz_row_sum_kernel<TRLK_BF16>, dim3(rows), dim3(256), 0, s, dzt, l.ld_n, int(l.npad / 8),
+                                   d_out_dbias + c0);
+            else
+                hipLaunchKernelGGL(dz_row_sum_kernel<TRLK_F16>, dim3(rows), dim3(256), 0, s, dzt, l.ld_n, int(l.npad / 8),
+                                   d_out_dbias + c0);
+            if (int rc2 = launch_status("fused_head_bwd (dBias)")) return rc2;
+        }
         const bool first = c0 == 0, last = c1 == vocab;
         // dHidden[N, H] += dz[N, chunk] * (W^T[H, chunk])^T ; W^T columns beyond V are zero and so is dz there
         GemmArgs gh{};

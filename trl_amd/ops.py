@@ -440,15 +440,25 @@ def _head_operands(hidden: Tensor, weight: Tensor, targets: Tensor):
     return hidden, weight, targets.contiguous()
 
 
+def _head_bias(bias, vocab):
+    if bias is None:
+        return None
+    if bias.shape != (vocab,):
+        raise ValueError(f"fused head: bias must have shape [{vocab}], got {tuple(bias.shape)}")
+    return bias.detach().float().contiguous()
+
+
 @torch.library.custom_op("trl_amd::fused_head_fwd", mutates_args=(), device_types="cuda")
 def fused_head_fwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature: float, softcap: float,
-                   logit_scale: float) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+                   logit_scale: float, bias: Optional[Tensor] = None) -> tuple[Tensor, Tensor, Tensor, Tensor]:
     """hidden [N, H], weight [V, H] (bf16/fp16), targets int64 [N] -> fp32 (logp, entropy, log_z, target_is_max),
-    each [N]; target_is_max is 1 where argmax(logits) == target.  `softcap <= 0` means no soft-capping."""
+    each [N]; target_is_max is 1 where argmax(logits) == target.  `softcap <= 0` means no soft-capping.
+    `bias` [V] (any float dtype) is added to `hidden @ weight.T` before scaling."""
     hidden, weight, targets = _head_operands(hidden, weight, targets)
     n, h = hidden.shape
     v = weight.shape[0]
     dev = hidden.device
+    bias32 = _head_bias(bias, v)
     logp = torch.empty((n,), dtype=torch.float32, device=dev)
     ent = torch.empty((n,), dtype=torch.float32, device=dev)
     log_z = torch.empty((n,), dtype=torch.float32, device=dev)
@@ -459,24 +469,25 @@ def fused_head_fwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         check(lib.trlk_fused_head_fwd(ptr(hidden), ptr(weight), ptr(targets), dtype_code(hidden.dtype), n, v, h,
-                                      hidden.stride(0), weight.stride(0), temperature, softcap, logit_scale, ptr(logp),
-                                      ptr(ent), ptr(log_z), ptr(hit), ptr(_error_flag(dev)), ptr(ws), ws_bytes,
-                                      current_stream(dev)))
+                                      hidden.stride(0), weight.stride(0), temperature, softcap, logit_scale,
+                                      ptr(bias32), ptr(logp), ptr(ent), ptr(log_z), ptr(hit), ptr(_error_flag(dev)),
+                                      ptr(ws), ws_bytes, current_stream(dev)))
     if _SYNC_CHECKS:
         check_device_errors()
     return logp, ent, log_z, hit
 
 
 @fused_head_fwd.register_fake
-def _(hidden, weight, targets, temperature, softcap, logit_scale):
+def _(hidden, weight, targets, temperature, softcap, logit_scale, bias=None):
     f = lambda: torch.empty((hidden.shape[0],), dtype=torch.float32, device=hidden.device)  # noqa: E731
     return f(), f(), f(), f()
 
 
 @torch.library.custom_op("trl_amd::fused_head_bwd", mutates_args=(), device_types="cuda")
 def fused_head_bwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature: float, softcap: float,
-                   logit_scale: float, log_z: Tensor, g_logp: Tensor, chunk_size: int) -> tuple[Tensor, Tensor]:
-    """Returns (d hidden [N, H], d weight [V, H]) in the operand dtype."""
+                   logit_scale: float, log_z: Tensor, g_logp: Tensor, chunk_size: int,
+                   bias: Optional[Tensor] = None) -> tuple[Tensor, Tensor, Tensor]:
+    """Returns (d hidden [N, H], d weight [V, H]) in the operand dtype and d bias (fp32 [V]; empty without a bias)."""
     w_dtype = weight.dtype
     hidden, weight, targets = _head_operands(hidden, weight, targets)
     n, h = hidden.shape
@@ -485,19 +496,22 @@ def fused_head_bwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
     d_hidden = torch.empty((n, h), dtype=hidden.dtype, device=dev)
     d_weight = torch.empty((v, h), dtype=hidden.dtype, device=dev)
     g = g_logp.contiguous().float()
+    bias32 = _head_bias(bias, v)
+    d_bias = torch.empty((v if bias is not None else 0,), dtype=torch.float32, device=dev)
     ws_bytes = lib.trlk_fused_head_bwd_workspace_bytes(max(n, 1), v, h, chunk_size)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         check(lib.trlk_fused_head_bwd(ptr(hidden), ptr(weight), ptr(targets), dtype_code(hidden.dtype), n, v, h,
-                                      hidden.stride(0), weight.stride(0), temperature, softcap, logit_scale, ptr(log_z),
-                                      ptr(g), chunk_size, ptr(d_hidden), ptr(d_weight), ptr(ws), ws_bytes,
-                                      current_stream(dev)))
-    return d_hidden, (d_weight if w_dtype == d_weight.dtype else d_weight.to(w_dtype))
+                                      hidden.stride(0), weight.stride(0), temperature, softcap, logit_scale,
+                                      ptr(bias32), ptr(log_z), ptr(g), chunk_size, ptr(d_hidden), ptr(d_weight),
+                                      ptr(d_bias) if bias is not None else None, ptr(ws), ws_bytes, current_stream(dev)))
+    return d_hidden, (d_weight if w_dtype == d_weight.dtype else d_weight.to(w_dtype)), d_bias
 
 
 @fused_head_bwd.register_fake
-def _(hidden, weight, targets, temperature, softcap, logit_scale, log_z, g_logp, chunk_size):
-    return torch.empty_like(hidden), torch.empty_like(weight)
+def _(hidden, weight, targets, temperature, softcap, logit_scale, log_z, g_logp, chunk_size, bias=None):
+    return (torch.empty_like(hidden), torch.empty_like(weight),
+            torch.empty((weight.shape[0] if bias is not None else 0,), dtype=torch.float32, device=hidden.device))
 
 
 NAN = math.nan

@@ -7,8 +7,7 @@ Those operators live in the third-party `liger-kernel` package (pinned `>=0.8.0,
 reference, not importable here), so what is mirrored is the call contract the reference relies on:
 argument names and meaning, the `(loss, metrics)` return and the position of each metric.  The
 arithmetic is the reference's own `_compute_loss` (same kernels as `GRPOLossMixin._compute_loss` /
-`dpo_sigmoid_loss`), fed by the fused head instead of materialised logits.  An `lm_head` bias is
-not supported (`NotImplementedError`).
+`dpo_sigmoid_loss`), fed by the fused head instead of materialised logits.
 """
 from __future__ import annotations
 
@@ -23,14 +22,15 @@ __all__ = ["FusedLinearGRPOLoss", "FusedLinearDPOLoss"]
 
 
 def _head_logps(hidden: Tensor, weight: Tensor, targets: Tensor, keep: Tensor, temperature: float,
-                chunk_size: int) -> Tensor:
-    """fp32 log-probs of `targets` `[B, T]` under `softmax(hidden @ weight.T / temperature)`; only the
+                chunk_size: int, bias: Tensor | None = None) -> Tensor:
+    """fp32 log-probs of `targets` `[B, T]` under `softmax((hidden @ weight.T + bias) / temperature)`; only the
     rows with `keep != 0` go through the head, the others are 0 (and receive no gradient)."""
     b, t, h = hidden.shape
     sel = keep.reshape(b * t) != 0
     flat_h = hidden.reshape(b * t, h)[sel]
     flat_t = targets.reshape(b * t)[sel]
-    lp_v, _ = _ChunkedLogProbFunction.apply(flat_h, weight, flat_t, float(temperature), int(chunk_size))
+    lp_v, _ = _ChunkedLogProbFunction.apply(flat_h, weight, flat_t, float(temperature), int(chunk_size), None, 1.0,
+                                            bias)
     lp = torch.zeros(b * t, dtype=torch.float32, device=hidden.device)
     lp[sel] = lp_v
     return lp.view(b, t)
@@ -70,14 +70,12 @@ class FusedLinearGRPOLoss(torch.nn.Module):
     def forward(self, _input: Tensor, lin_weight: Tensor, selected_token_ids: Tensor, attention_mask: Tensor,
                 advantages: Tensor, bias: Tensor | None = None, old_per_token_logps: Tensor | None = None,
                 ref_per_token_logps: Tensor | None = None, vllm_is_ratio: Tensor | None = None):
-        if bias is not None:
-            raise NotImplementedError("an lm_head bias is not supported by the fused head")
         if _input.dim() != 3:
             raise ValueError("_input must be [B, T, H] hidden states")
         if self.beta != 0.0 and ref_per_token_logps is None:
             raise ValueError("ref_per_token_logps is required when beta != 0")
         mask = attention_mask
-        logps = _head_logps(_input, lin_weight, selected_token_ids, mask, self.temperature, self.chunk_size)
+        logps = _head_logps(_input, lin_weight, selected_token_ids, mask, self.temperature, self.chunk_size, bias)
         n_items = mask.sum().float()
         n_proc = 1
         if torch.distributed.is_available() and torch.distributed.is_initialized():
@@ -108,7 +106,7 @@ class FusedLinearGRPOLoss(torch.nn.Module):
 class FusedLinearDPOLoss(torch.nn.Module):
     """`loss, metrics = op(lin_weight [V, H], _input [2P, T, H], target [2P, T] (-100 = ignored),
     bias=None, ref_input=None, ref_weight=None, ref_bias=None)`; rows `[0, P)` are the chosen, `[P, 2P)`
-    the rejected sequences.  `metrics = (chosen_logps [P], rejected_logps [P], chosen_logits_mean,
+    the rejected sequences; without `ref_weight` the reference model shares `lin_weight` and `bias`.  `metrics = (chosen_logps [P], rejected_logps [P], chosen_logits_mean,
     rejected_logits_mean, nll_loss, chosen_rewards [P], rejected_rewards [P])`, the order
     `_compute_loss_liger` unpacks (dpo_trainer.py:1293-1301).  Sigmoid loss only; the logits means are
     taken over every position and the whole vocabulary, computed as `hidden . sum_v W[v]` (no logits)."""
@@ -125,20 +123,18 @@ class FusedLinearDPOLoss(torch.nn.Module):
 
     def forward(self, lin_weight: Tensor, _input: Tensor, target: Tensor, bias: Tensor | None = None,
                 ref_input: Tensor | None = None, ref_weight: Tensor | None = None, ref_bias: Tensor | None = None):
-        if bias is not None or ref_bias is not None:
-            raise NotImplementedError("an lm_head bias is not supported by the fused head")
         if _input.dim() != 3 or _input.shape[0] % 2:
             raise ValueError("_input must be [2P, T, H]: chosen sequences first, rejected second")
         pairs = _input.shape[0] // 2
         keep = target != self.ignore_index
         labels = torch.where(keep, target, torch.zeros_like(target))
-        logps = _head_logps(_input, lin_weight, labels, keep, 1.0, self.chunk_size)
+        logps = _head_logps(_input, lin_weight, labels, keep, 1.0, self.chunk_size, bias)
         if self.use_ref_model:
             if ref_input is None:
                 raise ValueError("ref_input is required when use_ref_model=True")
             with torch.no_grad():
                 ref_logps = _head_logps(ref_input, lin_weight if ref_weight is None else ref_weight, labels, keep, 1.0,
-                                        self.chunk_size)
+                                        self.chunk_size, bias if ref_weight is None else ref_bias)
                 ref_seq = (ref_logps * keep).sum(-1)
         else:
             ref_seq = torch.zeros(2 * pairs, dtype=torch.float32, device=_input.device)
@@ -147,6 +143,8 @@ class FusedLinearDPOLoss(torch.nn.Module):
             seq = seq.detach()
             wsum = lin_weight.float().sum(0)
             logits_mean = (_input.float() @ wsum).mean(dim=1) / lin_weight.shape[0]  # [2P], over T and V
+            if bias is not None:
+                logits_mean = logits_mean + bias.float().mean()
             rewards = self.beta * (seq - ref_seq)
             nll = torch.zeros((), dtype=torch.float32, device=_input.device)
         metrics = (seq[:pairs], seq[pairs:], logits_mean[:pairs].mean(), logits_mean[pairs:].mean(), nll,

@@ -26,7 +26,7 @@ class _FusedNLLFunction(torch.autograd.Function):
     def backward(ctx, g_logp, g_ent, g_hit):
         hidden, weight, labels, log_z = ctx.saved_tensors
         chunk_size, softcap, logit_scale = ctx.cfg
-        d_hidden, d_weight = ops.fused_head_bwd(hidden, weight, labels, 1.0, softcap, logit_scale, log_z, g_logp,
+        d_hidden, d_weight, _ = ops.fused_head_bwd(hidden, weight, labels, 1.0, softcap, logit_scale, log_z, g_logp,
                                                 chunk_size)
         return d_hidden, d_weight, None, None, None, None
 
