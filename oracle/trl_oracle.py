@@ -55,6 +55,7 @@ __all__ = [
     "get_off_policy_mask",
     "get_high_entropy_mask",
     "get_gamma_weights",
+    "vllm_importance_sampling_ratio",
     "logps_and_entropies_from_logits",
     "grpo_loss",
     "dpo_sequence_logps",
@@ -224,6 +225,22 @@ def get_off_policy_mask(advantages, per_token_logps, sampling_per_token_logps, m
     gap = sampling_per_token_logps - per_token_logps.detach()
     mean_gap = (gap * mask).sum(1, keepdim=True) / mask.sum(1, keepdim=True).clamp(min=1.0)
     return ((advantages >= 0) | (mean_gap <= off_policy_threshold)).to(mask.dtype)
+
+
+def vllm_importance_sampling_ratio(old_logps, sampling_logps, completion_mask, tool_mask, mode, clip_min, clip_max):
+    """Sampler/trainer mismatch correction, trl/trainer/grpo_trainer.py:2578-2623, one branch per mode."""
+    mask = completion_mask if tool_mask is None else completion_mask * tool_mask
+    d = (old_logps - sampling_logps) * mask
+    if mode in ("sequence_mask", "sequence_truncate"):
+        d = d.sum(dim=-1, keepdim=True)
+    r = torch.exp(d)
+    if mode in ("sequence_truncate", "token_truncate"):
+        return torch.clamp(r, min=clip_min, max=clip_max)
+    if mode in ("sequence_mask", "token_mask"):
+        lo = -math.inf if clip_min is None else clip_min
+        hi = math.inf if clip_max is None else clip_max
+        return torch.where((r < lo) | (r > hi), torch.zeros_like(r), r)
+    raise ValueError(mode)
 
 
 def get_high_entropy_mask(entropies, mask, threshold):

@@ -26,6 +26,7 @@ __all__ = [
     "get_off_policy_mask",
     "get_high_entropy_mask",
     "get_gamma_weights",
+    "vllm_importance_sampling_ratio",
     "GRPOLossMixin",
 ]
 
@@ -60,6 +61,43 @@ def get_off_policy_mask(advantages, per_token_logps, sampling_per_token_logps, m
     gap = sampling_per_token_logps - per_token_logps.detach()
     mean_gap = (gap * mask).sum(dim=1, keepdim=True) / mask.sum(dim=1, keepdim=True).clamp(min=1.0)
     return ((advantages >= 0) | (mean_gap <= off_policy_threshold)).to(dtype=mask.dtype)
+
+
+_IS_MODES = ("token_truncate", "token_mask", "sequence_truncate", "sequence_mask")
+
+
+def vllm_importance_sampling_ratio(old_per_token_logps, sampling_per_token_logps, completion_mask, tool_mask=None,
+                                   mode="sequence_mask", clip_min=None, clip_max=None):
+    """Correction factor for the sampler/trainer distribution mismatch (trl/trainer/grpo_trainer.py:2578-2623):
+    `exp((old - sampling) * mask)` per token (`token_*` modes, `(B, T)`) or of the per-sequence sum
+    (`sequence_*`, `(B, 1)`), clamped to `[clip_min, clip_max]` (`*_truncate`) or zeroed outside it (`*_mask`).
+    Also returns the five logged statistics (:2779-2813) as 0-d tensors of this process's batch:
+    `sampling_logp_difference/{mean,max}`, `importance_sampling_ratio/{min,mean,max}` (0 when no token is active)."""
+    if mode not in _IS_MODES:
+        raise ValueError(f"Unknown vLLM importance sampling level: {mode}. Possible values are 'token_truncate', "
+                         "'token_mask', 'sequence_truncate', and 'sequence_mask'.")
+    mask = completion_mask if tool_mask is None else completion_mask * tool_mask
+    diff = (old_per_token_logps - sampling_per_token_logps) * mask
+    sequence_level = mode.startswith("sequence")
+    ratio = torch.exp(diff.sum(dim=-1, keepdim=True) if sequence_level else diff)
+    if mode.endswith("truncate"):
+        ratio = torch.clamp(ratio, min=clip_min, max=clip_max)
+    else:
+        lo = -math.inf if clip_min is None else clip_min
+        hi = math.inf if clip_max is None else clip_max
+        ratio = ratio.masked_fill((ratio < lo) | (ratio > hi), 0.0)
+    keep = mask.bool()
+    delta = torch.abs(old_per_token_logps - sampling_per_token_logps)[keep]
+    flat = ratio.flatten() if sequence_level else ratio[keep]
+    zero = torch.zeros((), dtype=ratio.dtype, device=ratio.device)
+    stats = {
+        "sampling/sampling_logp_difference/mean": delta.mean() if delta.numel() else zero,
+        "sampling/sampling_logp_difference/max": delta.max() if delta.numel() else zero,
+        "sampling/importance_sampling_ratio/min": flat.min() if flat.numel() else zero,
+        "sampling/importance_sampling_ratio/mean": flat.mean() if flat.numel() else zero,
+        "sampling/importance_sampling_ratio/max": flat.max() if flat.numel() else zero,
+    }
+    return ratio, stats
 
 
 def get_high_entropy_mask(entropies, mask, threshold, accelerator=None):
