@@ -23,6 +23,9 @@ Pinning status (what checks each function against something other than itself):
                               `DPOTrainer._compute_loss` (mocked; all fifteen loss types, ld_alpha, WPO
                               weighting, f-divergences, arg-max ties), closed form ln 2
   rloo_loss                 : golden vectors from `RLOOTrainer._compute_loss` (mocked)
+  kto_*                     : golden vectors from `KTOTrainer._compute_loss` (mocked, KL pass included),
+                              closed form 1/2 at policy == reference
+  vllm_importance_sampling_ratio : hand-computed values per mode (no reference test holds numbers for it)
   chunked_logprob           : naive `(h @ W.T).float()/T -> log_softmax` routine and
                               autograd of it (reference test tests/test_utils.py:1161-1232)
   chunked_cross_entropy_loss: golden vectors from the reference's `_chunked_cross_entropy_loss`,
@@ -62,6 +65,8 @@ __all__ = [
     "dpo_sigmoid_loss",
     "dpo_compute_loss",
     "rloo_loss",
+    "kto_sequence_logps",
+    "kto_compute_loss",
     "chunked_logprob_naive",
     "chunked_logprob_online",
     "chunked_logprob_backward",
@@ -667,6 +672,61 @@ def rloo_loss(per_token_logps, completion_mask, old_logps, advantages, epsilon_l
         "clip_ratio/high_max": float(nanmax(high)),
         "clip_ratio/region_mean": float(region.mean()),
     }
+    return loss, metrics
+
+
+# --------------------------------------------------------------------------------------
+# KTO  sequence log-probs, KL baseline, loss and logged metrics   trl/trainer/kto_trainer.py:1478-1663
+# --------------------------------------------------------------------------------------
+def kto_sequence_logps(logits, input_ids, completion_mask):
+    """Masked sum of the shifted per-token log-probs in the logits dtype (kto_trainer.py:1506-1509; the same four
+    lines serve the KL-estimate and reference passes, :1265-1276, :1323-1327)."""
+    tok = selective_log_softmax(logits[:, :-1, :], input_ids[:, 1:])
+    tok = torch.where(completion_mask[:, 1:] == 0, torch.zeros_like(tok), tok)
+    return tok.sum(-1)
+
+
+def kto_compute_loss(logits, input_ids, completion_mask, label, ref_logps, kl_logps=None, ref_kl_logps=None, beta=0.1,
+                     loss_type="kto", desirable_weight=1.0, undesirable_weight=1.0):
+    """`KTOTrainer._compute_loss` (kto_trainer.py:1506-1663) for one process with precomputed reference log-probs.
+    Returns `(loss, metrics)` with the logged names."""
+    seq = kto_sequence_logps(logits, input_ids, completion_mask)
+    lab = torch.as_tensor(label, dtype=torch.bool)
+    ci, ri = torch.nonzero(lab).view(-1), torch.nonzero(~lab).view(-1)
+    c_lp, r_lp = seq[ci], seq[ri]
+    if kl_logps is not None:  # :1549-1553
+        kl = (kl_logps - ref_kl_logps).mean().detach().clamp(min=0)
+    else:
+        kl = torch.zeros(1)
+    c_lr, r_lr = c_lp - ref_logps[ci], r_lp - ref_logps[ri]
+    if loss_type == "kto":  # :1558-1560, :1576-1577
+        c_loss = 1 - torch.sigmoid(beta * (c_lr - kl))
+        r_loss = 1 - torch.sigmoid(beta * (kl - r_lr))
+    elif loss_type == "apo_zero_unpaired":  # :1561-1564, :1578-1579
+        c_loss = 1 - torch.sigmoid(beta * c_lr)
+        r_loss = torch.sigmoid(beta * r_lr)
+    else:
+        raise ValueError(loss_type)
+    loss = torch.cat((desirable_weight * c_loss, undesirable_weight * r_loss), 0).nanmean()  # :1586-1589, :1655
+    metrics = {"kl": float(kl)}
+    with torch.no_grad():
+        shift = logits[:, :-1, :].detach()
+        mask = completion_mask[:, 1:]
+        ent = entropy_from_logits(shift)  # :1594-1603
+        total = mask.sum()
+        metrics["entropy"] = float((ent * mask).sum() / total) if total > 0 else 0.0
+        for name, idx in (("chosen", ci), ("rejected", ri)):  # :1612-1628
+            mk = mask[idx]
+            if mk.sum() > 0:
+                metrics["logits/" + name] = float(shift[idx][mk.bool()].mean(-1).sum()) / float(mk.sum())
+        if len(ci) > 0:  # :1633-1647
+            metrics["rewards/chosen"] = float((beta * c_lr).nansum()) / len(ci)
+            metrics["logps/chosen"] = float(c_lp.nansum()) / len(ci)
+        if len(ri) > 0:
+            metrics["rewards/rejected"] = float((beta * r_lr).nansum()) / len(ri)
+            metrics["logps/rejected"] = float(r_lp.nansum()) / len(ri)
+        if len(ci) > 0 and len(ri) > 0:
+            metrics["rewards/margins"] = metrics["rewards/chosen"] - metrics["rewards/rejected"]
     return loss, metrics
 
 

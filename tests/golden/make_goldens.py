@@ -356,6 +356,96 @@ def make_dpo(DPOTrainer, out_dir):
         json.dump(index, f, indent=1)
 
 
+# ------------------------------------------------------------------------------------ KTO
+KTO_CASES = [
+    dict(name="kto_fp32", dtype="float32", loss_type="kto", beta=0.1, labels=[1, 0, 1, 1, 0, 0], kl=True),
+    dict(name="kto_weights", dtype="float32", loss_type="kto", beta=0.25, labels=[1, 0, 0, 1, 0, 0], kl=True,
+         desirable_weight=1.33, undesirable_weight=0.8),
+    dict(name="kto_negative_kl", dtype="float32", loss_type="kto", beta=0.1, labels=[0, 1, 1, 0, 1, 0], kl=True, kl_shift=-3.0),
+    dict(name="apo_zero_unpaired", dtype="float32", loss_type="apo_zero_unpaired", beta=0.1, labels=[1, 0, 1, 0, 1, 0], kl=False),
+    dict(name="kto_all_chosen", dtype="float32", loss_type="kto", beta=0.1, labels=[1, 1, 1, 1, 1, 1], kl=True),
+    dict(name="kto_all_rejected", dtype="float32", loss_type="apo_zero_unpaired", beta=0.1, labels=[0, 0, 0, 0, 0, 0], kl=False),
+    dict(name="kto_bf16", dtype="bfloat16", loss_type="kto", beta=0.1, labels=[1, 0, 1, 1, 0, 0], kl=True),
+]
+
+
+def make_kto(KTOTrainer, out_dir):
+    from trl.trainer.utils import selective_log_softmax as ref_sls
+
+    index, arrays = [], {}
+    for ci, case in enumerate(KTO_CASES):
+        g = torch.Generator().manual_seed(4000 + ci)
+        B, L, LK, V = 6, 10, 12, 37
+        dtype = getattr(torch, case["dtype"])
+        logits = (2.0 * torch.randn(B, L, V, generator=g)).to(dtype)
+        kl_logits = (2.0 * torch.randn(B, LK, V, generator=g)).to(dtype)
+        input_ids = torch.randint(0, V, (B, L), generator=g)
+        kl_input_ids = torch.randint(0, V, (B, LK), generator=g)
+        prompt_len, comp_len, kl_comp_len = [2, 3, 4, 1, 2, 5], [5, 4, 6, 8, 3, 2], [4, 7, 3, 9, 5, 6]
+        completion_mask = torch.zeros(B, L, dtype=torch.long)
+        attention_mask = torch.zeros(B, L, dtype=torch.long)
+        kl_completion_mask = torch.zeros(B, LK, dtype=torch.long)
+        kl_attention_mask = torch.zeros(B, LK, dtype=torch.long)
+        for i in range(B):
+            lp = prompt_len[i]
+            completion_mask[i, lp : lp + comp_len[i]] = 1
+            attention_mask[i, : lp + comp_len[i]] = 1
+            kl_completion_mask[i, lp : lp + kl_comp_len[i]] = 1
+            kl_attention_mask[i, : lp + kl_comp_len[i]] = 1
+
+        def seq_logps(lg, ids, cm):
+            with torch.no_grad():
+                tok = ref_sls(lg[:, :-1, :], ids[:, 1:]).float()
+                return (tok * cm[:, 1:]).sum(1)
+
+        ref_logps = seq_logps(logits, input_ids, completion_mask) + 0.7 * torch.randn(B, generator=g)
+        ref_kl_logps = (seq_logps(kl_logits, kl_input_ids, kl_completion_mask) + 0.3 * torch.randn(B, generator=g)
+                        - case.get("kl_shift", 1.5))
+
+        trainer = Mock(spec=KTOTrainer)
+        trainer.accelerator = _fake_accelerator()
+        trainer.aux_loss_enabled = False
+        trainer.use_liger_kernel = False
+        trainer.calculate_KL = case["kl"]
+        trainer.precompute_ref_logps = True
+        trainer.loss_type = case["loss_type"]
+        trainer.beta = case["beta"]
+        trainer.desirable_weight = case.get("desirable_weight", 1.0)
+        trainer.undesirable_weight = case.get("undesirable_weight", 1.0)
+        trainer._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
+        trainer._total_train_tokens = 0
+        trainer.model = SimpleNamespace(training=True)
+        trainer._compute_kl_logps = lambda model, batch, t=trainer: KTOTrainer._compute_kl_logps(t, model, batch)
+
+        leaf = logits.clone().requires_grad_(True)
+
+        def model(input_ids=None, **kw):  # the KL pass is told apart by its sequence length
+            if input_ids.shape[1] == LK:
+                return SimpleNamespace(logits=kl_logits.clone(), aux_loss=None)
+            return SimpleNamespace(logits=leaf * 1.0, aux_loss=None)
+
+        inputs = dict(
+            input_ids=input_ids, attention_mask=attention_mask, completion_mask=completion_mask,
+            label=torch.tensor(case["labels"], dtype=torch.bool), ref_logps=ref_logps,
+        )
+        if case["kl"]:
+            inputs.update(KL_input_ids=kl_input_ids, KL_attention_mask=kl_attention_mask,
+                          KL_completion_mask=kl_completion_mask, ref_KL_logps=ref_kl_logps)
+        loss = KTOTrainer._compute_loss(trainer, model, inputs, False)
+        loss.backward()
+        pre = f"c{ci}_"
+        for key, val in dict(logits=logits, kl_logits=kl_logits, input_ids=input_ids, kl_input_ids=kl_input_ids,
+                             completion_mask=completion_mask, attention_mask=attention_mask,
+                             kl_completion_mask=kl_completion_mask, kl_attention_mask=kl_attention_mask,
+                             ref_logps=ref_logps, ref_kl_logps=ref_kl_logps, out_loss=loss, out_dlogits=leaf.grad).items():
+            arrays[pre + key] = _np(val)
+        metrics = {k: float(v[-1]) for k, v in trainer._metrics["train"].items()}
+        index.append(dict(case, id=ci, shape=[B, L, V], kl_len=LK, metrics=metrics))
+    np.savez_compressed(os.path.join(out_dir, "kto_compute_loss.npz"), **arrays)
+    with open(os.path.join(out_dir, "kto_compute_loss.json"), "w") as f:
+        json.dump(index, f, indent=1)
+
+
 # ------------------------------------------------------------------------------------ RLOO
 RLOO_CASES = [
     dict(name="rloo_sym", eps_low=0.2, eps_high=0.2, temperature=1.0),
@@ -518,6 +608,7 @@ def main():
     import trl.trainer.utils as ref_utils
     from trl.trainer.dpo_trainer import DPOTrainer
     from trl.trainer.grpo_trainer import GRPOTrainer
+    from trl.trainer.kto_trainer import KTOTrainer
     from trl.trainer.rloo_trainer import RLOOTrainer
 
     from trl.trainer.sft_trainer import _chunked_cross_entropy_loss
@@ -528,6 +619,7 @@ def main():
     make_grpo(GRPOTrainer, args.out)
     make_dpo(DPOTrainer, args.out)
     make_rloo(RLOOTrainer, args.out)
+    make_kto(KTOTrainer, args.out)
     print("golden fixtures written to", args.out)
 
 

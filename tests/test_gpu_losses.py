@@ -335,6 +335,67 @@ def test_dpo_mixin_compute_loss(amd):
     torch.testing.assert_close(seq.cpu(), oseq, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("skip_masked", [True, False])
+def test_golden_kto_compute_loss(amd, skip_masked):
+    """The reference's `KTOTrainer._compute_loss` cases: loss, dlogits and the logged metrics through the mix-in
+    method on a mocked trainer (KL pass included).  bf16: the reference sums bf16-rounded log-probs, hence 5e-2."""
+    cases, g = load_golden("kto_compute_loss")
+    for case in cases:
+        c = f"c{case['id']}_"
+        dtype = getattr(torch, case["dtype"])
+        low = dtype != torch.float32
+
+        class Trainer(amd.KTOLossMixin):
+            pass
+
+        tr = Trainer()
+        tr.accelerator = _Identity()
+        tr.accelerator.gather_for_metrics = lambda x: x
+        tr.accelerator.device = torch.device(DEV)
+        tr.model = SimpleNamespace(training=True)
+        tr.aux_loss_enabled = False
+        tr.precompute_ref_logps, tr.calculate_KL = True, case["kl"]
+        tr.beta, tr.loss_type = case["beta"], case["loss_type"]
+        tr.desirable_weight = case.get("desirable_weight", 1.0)
+        tr.undesirable_weight = case.get("undesirable_weight", 1.0)
+        tr._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
+        tr._total_train_tokens = 0
+        leaf = _t(g[c + "logits"], dtype).to(DEV).requires_grad_(True)
+        kl_logits = _t(g[c + "kl_logits"], dtype).to(DEV)
+        kl_len = case["kl_len"]
+
+        def model(input_ids=None, **kw):
+            return SimpleNamespace(logits=kl_logits if input_ids.shape[1] == kl_len else leaf, aux_loss=None)
+
+        inputs = dict(input_ids=_t(g[c + "input_ids"]), attention_mask=_t(g[c + "attention_mask"]),
+                      completion_mask=_t(g[c + "completion_mask"]), label=torch.tensor(case["labels"], dtype=torch.bool),
+                      ref_logps=_t(g[c + "ref_logps"]))
+        if case["kl"]:
+            inputs.update(KL_input_ids=_t(g[c + "kl_input_ids"]), KL_attention_mask=_t(g[c + "kl_attention_mask"]),
+                          KL_completion_mask=_t(g[c + "kl_completion_mask"]), ref_KL_logps=_t(g[c + "ref_kl_logps"]))
+        if skip_masked:
+            loss = tr._compute_loss(model, inputs, False)
+            got = {k: v[-1] for k, v in tr._metrics["train"].items()}
+        else:
+            dev = {k: v.to(DEV) for k, v in inputs.items()}
+            kl = amd.kto_sequence_logps(kl_logits, dev["KL_input_ids"], dev["KL_completion_mask"], False) if case["kl"] else None
+            loss, parts = amd.kto_compute_loss(
+                leaf, dev["input_ids"], dev["completion_mask"], dev["label"], dev["ref_logps"], kl,
+                dev.get("ref_KL_logps"), case["beta"], case["loss_type"], tr.desirable_weight, tr.undesirable_weight,
+                skip_masked_rows=False)
+            got = {"kl": float(parts["kl"])}
+        loss.backward()
+        want = float(g[c + "out_loss"])
+        assert abs(float(loss) - want) <= (5e-2 if low else 1e-5) * max(1.0, abs(want)), (case["name"], float(loss), want)
+        assert _rel_l2(leaf.grad.float(), _t(g[c + "out_dlogits"])) < (5e-2 if low else 1e-4), case["name"]
+        if skip_masked:
+            assert set(got) == set(case["metrics"]), (case["name"], sorted(got))
+        for name, value in got.items():
+            want_m = case["metrics"][name]
+            tol = max((0.15 if low else 1e-5) * max(1.0, abs(want_m)), 2e-6)
+            assert abs(value - want_m) <= tol, (case["name"], name, value, want_m)
+
+
 def test_golden_dpo_compute_loss(amd):
     """The fused sigmoid path (one loss kernel) on the plain sigmoid cases."""
     cases, g = load_golden("dpo_compute_loss")

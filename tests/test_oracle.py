@@ -347,6 +347,40 @@ def test_golden_dpo_compute_loss():
             assert abs(float(l2) - float(loss)) < 1e-7
 
 
+def test_golden_kto_compute_loss():
+    """Every case the reference's `KTOTrainer._compute_loss` ran (mocked trainer): kto with the KL baseline (also
+    one clamped at 0), weights, apo_zero_unpaired, all-desirable and all-undesirable batches, bf16."""
+    cases, g = load_golden("kto_compute_loss")
+    assert len(cases) >= 7
+    for case in cases:
+        c = f"c{case['id']}_"
+        dtype = getattr(torch, case["dtype"])
+        low = dtype != torch.float32
+        logits = _t(g[c + "logits"], dtype).requires_grad_(True)
+        kl = ref_kl = None
+        if case["kl"]:
+            kl = oracle.kto_sequence_logps(_t(g[c + "kl_logits"], dtype), _t(g[c + "kl_input_ids"]),
+                                           _t(g[c + "kl_completion_mask"]))
+            ref_kl = _t(g[c + "ref_kl_logps"])
+        loss, metrics = oracle.kto_compute_loss(
+            logits, _t(g[c + "input_ids"]), _t(g[c + "completion_mask"]), case["labels"], _t(g[c + "ref_logps"]), kl,
+            ref_kl, case["beta"], case["loss_type"], case.get("desirable_weight", 1.0), case.get("undesirable_weight", 1.0))
+        loss.backward()
+        torch.testing.assert_close(loss.detach().float(), _t(g[c + "out_loss"]).float(), rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(logits.grad.float(), _t(g[c + "out_dlogits"]), rtol=1e-5, atol=1e-8)
+        assert set(metrics) == set(case["metrics"]) - {"num_tokens"}, case["name"]
+        for name, got in metrics.items():
+            want = case["metrics"][name]
+            assert abs(got - want) <= 1e-6 + (1e-2 if low else 1e-5) * abs(want), (case["name"], name, got, want)
+        if case["name"] == "kto_negative_kl":
+            assert metrics["kl"] == 0.0
+    # closed form: policy == reference and KL = 0 -> every loss is 1 - sigmoid(0) = 1/2
+    logits = _t(g["c0_logits"])
+    seq = oracle.kto_sequence_logps(logits, _t(g["c0_input_ids"]), _t(g["c0_completion_mask"]))
+    loss, _ = oracle.kto_compute_loss(logits, _t(g["c0_input_ids"]), _t(g["c0_completion_mask"]), [1, 0, 1, 1, 0, 0], seq)
+    assert abs(float(loss) - 0.5) < 1e-7
+
+
 def test_golden_rloo_compute_loss():
     cases, g = load_golden("rloo_compute_loss")
     for case in cases:

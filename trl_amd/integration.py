@@ -33,7 +33,7 @@ def _set(mod, name, value) -> None:
     setattr(mod, name, value)
 
 
-def patch_trl(grpo: bool = True, liger: bool = False, dpo: bool = False, rloo: bool = False) -> int:
+def patch_trl(grpo: bool = True, liger: bool = False, dpo: bool = False, rloo: bool = False, kto: bool = False) -> int:
     """Returns the number of names rebound.  Needs `trl` to be importable."""
     import trl.trainer.utils as ref_utils
 
@@ -76,6 +76,16 @@ def patch_trl(grpo: bool = True, liger: bool = False, dpo: bool = False, rloo: b
             _saved.append((RLOOTrainer, name, RLOOTrainer.__dict__[name]))
             setattr(RLOOTrainer, name, getattr(RLOOLossMixin, name))
             count += 1
+    if kto:
+        from trl.trainer.kto_trainer import KTOTrainer
+
+        from .trainer.kto_trainer import KTOLossMixin
+
+        for name in ("_compute_kl_logps", "_compute_loss"):
+            _saved.append((KTOTrainer, name, KTOTrainer.__dict__[name]))
+            setattr(KTOTrainer, name, getattr(KTOLossMixin, name))
+            count += 1
+        _set(KTOTrainer, "_NON_MODEL_KEYS", KTOLossMixin._NON_MODEL_KEYS)
     if dpo:
         from trl.trainer.dpo_trainer import DPOTrainer
 
