@@ -230,12 +230,22 @@ int trlk_rloo_loss(const float* d_token_logp, const float* d_mask, const float* 
  */
 size_t trlk_fused_head_fwd_workspace_bytes(int64_t n_tokens);
 
+/* Optional stash of the forward's raw products y = hidden @ weight^T (fp32, vocabulary-major:
+ * [vocab rounded up to 256, *out_ld], *out_ld = n_tokens rounded up to 256).  A forward that is given
+ * the buffer (d_out_stash, stash_ld) fills it; a backward that is given the same buffer (d_stash)
+ * derives dz from it in one memory-bound sweep instead of recomputing the chunk's logits on the
+ * matrix cores (a third of the backward's work).  No counterpart in the reference, which always
+ * recomputes (trl/trainer/utils.py:1385-1399): it trades vocab * n_tokens * 4 bytes held between
+ * forward and backward for that recompute.  Returns the buffer size in bytes.
+ */
+size_t trlk_fused_head_stash_bytes(int64_t n_tokens, int64_t vocab, int64_t* out_ld);
+
 int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, const int64_t* d_targets, int dtype,
                         int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                         int64_t weight_stride, float temperature, float final_logit_softcapping, float logit_scale,
                         const float* d_bias, float* d_out_logp, float* d_out_entropy, float* d_out_log_z,
-                        float* d_out_target_is_max, int32_t* d_error_flag, void* d_workspace, size_t workspace_bytes,
-                        trlk_stream_t stream);
+                        float* d_out_target_is_max, float* d_out_stash, int64_t stash_ld, int32_t* d_error_flag,
+                        void* d_workspace, size_t workspace_bytes, trlk_stream_t stream);
 
 /* Backward of the above w.r.t. hidden and weight for an upstream gradient on the log-probs
  * (the entropy output carries no gradient, as in the reference, utils.py:1368):
@@ -252,8 +262,8 @@ int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, const int64_
                         int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                         int64_t weight_stride, float temperature, float final_logit_softcapping, float logit_scale,
                         const float* d_bias, const float* d_log_z, const float* d_g_logp, int64_t chunk_size,
-                        void* d_out_dhidden, void* d_out_dweight, float* d_out_dbias, void* d_workspace,
-                        size_t workspace_bytes, trlk_stream_t stream);
+                        const float* d_stash, int64_t stash_ld, void* d_out_dhidden, void* d_out_dweight,
+                        float* d_out_dbias, void* d_workspace, size_t workspace_bytes, trlk_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -141,6 +141,43 @@ def test_fused_head_with_bias(amd, n, h, v, chunk, softcap, scale):
         assert _rel_l2(got.grad.float(), want.grad) < 1e-2, _rel_l2(got.grad.float(), want.grad)
 
 
+@pytest.mark.parametrize("n,h,v,chunk,softcap,scale,bias", [
+    (300, 256, 1000, 256, None, 1.0, False),   # ragged tokens and vocabulary, four chunks
+    (257, 136, 777, 512, 5.0, 0.5, True),      # soft-capping + logit_scale + bias (general epilogue)
+    (600, 512, 2304, 1024, None, 1.0, False),  # several token blocks x several vocabulary tiles
+    (1, 8, 3, 8192, None, 1.0, False),
+])
+def test_backward_from_stashed_products_equals_recompute(amd, monkeypatch, n, h, v, chunk, softcap, scale, bias):
+    """The backward fed by the forward's stashed products gives the recompute path's gradients (same
+    accumulators, same dz arithmetic: equal up to the order of fp32 operations), and the forward's outputs do
+    not depend on stashing."""
+    g = torch.Generator().manual_seed(n * 3 + v)
+    hidden = torch.randn(n, h, generator=g).bfloat16().to(DEV)
+    weight = (torch.randn(v, h, generator=g) * (2.0 / h**0.5)).bfloat16().to(DEV)
+    b = (2.0 * torch.randn(v, generator=g)).bfloat16().to(DEV) if bias else None
+    labels = torch.randint(0, v, (n,), generator=g).to(DEV)
+    gout = torch.randn(n, generator=g).to(DEV)
+    gout[::7] = 0.0  # rows without an upstream gradient
+    out = {}
+    for mode, gib in (("stash", "1"), ("recompute", "0")):
+        monkeypatch.setenv("TRL_AMD_HEAD_STASH_GIB", gib)
+        assert amd.ops.head_stash_fits(n, v) == (mode == "stash")
+        hh, ww = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+        bb = b.clone().requires_grad_(True) if bias else None
+        lp, ent = amd._ChunkedLogProbFunction.apply(hh, ww, labels, 0.9, chunk, softcap, scale, bb)
+        (lp * gout).sum().backward()
+        out[mode] = (lp.detach(), ent, hh.grad, ww.grad, bb.grad if bias else None)
+    assert torch.equal(out["stash"][0], out["recompute"][0]) and torch.equal(out["stash"][1], out["recompute"][1])
+    for got, want in zip(out["stash"][2:], out["recompute"][2:]):
+        if want is not None:
+            assert _rel_l2(got.float(), want.float()) < 2e-3, _rel_l2(got.float(), want.float())
+    # the op rejects a stash of the wrong shape
+    lp, ent, log_z, _, saved = amd.ops.fused_head_fwd(hidden, weight, labels, 0.9, 0.0, 1.0, None, True)
+    assert saved.shape == ((v + 255) // 256 * 256, (n + 255) // 256 * 256)
+    with pytest.raises(ValueError):
+        amd.ops.fused_head_bwd(hidden, weight, labels, 0.9, 0.0, 1.0, log_z, gout, chunk, None, saved[:, :128])
+
+
 def test_masked_rows_and_scatter(amd):
     # reference tests/test_utils.py:1338-1398: masked == unmasked on completion rows, exact zeros elsewhere,
     # and the lm_head gradient only sees completion rows

@@ -5,9 +5,9 @@
 // row-major and K contiguous, which is the layout the MFMA A/B fragments want (a lane holds 8
 // consecutive k of one row), so fragments come straight out of LDS with 16-byte reads and nothing
 // is ever transposed on the fly.  512 threads = 8 waves as 2 (M) x 4 (N); a wave owns 128 x 64 of
-// the tile = 4 x 2 MFMA blocks = 128 accumulator registers per lane.  Two LDS stages, one barrier
-// per 64-wide k step; tiles go from memory straight into LDS (global_load_lds_dwordx4) when K is a
-// multiple of 64, through registers otherwise.
+// the tile = 4 x 2 MFMA blocks = 128 accumulator registers per lane.  Tiles go from memory
+// straight into a ring of LDS stages (global_load_lds_dwordx4) when K is a multiple of the k step,
+// through registers otherwise.
 //
 // Forward (K5): the tile is computed TRANSPOSED -- M = vocabulary rows of W, N = tokens -- so that
 // a lane of the accumulator layout holds 16 vocabulary entries of ONE token per block.  The online
@@ -15,8 +15,9 @@
 // epilogue needs no cross-lane traffic; a workgroup keeps 256 tokens and walks over its share of
 // the vocabulary tiles, the logits exist only as accumulators.
 //
-// Backward (K6), per vocabulary chunk: (1) recompute the chunk's logits the same way and turn
-// them into dz = dL/dlogits (bf16), written both as [tokens, chunk] and as [chunk, tokens];
+// Backward (K6), per vocabulary chunk: (1) dz = dL/dlogits (bf16), written both as [tokens, chunk]
+// and as [chunk, tokens] -- from a recompute of the chunk's logits (same tile loop), or, when the
+// forward was asked to stash its raw products, from one elementwise sweep over that stash;
 // (2) dHidden += dz * W_chunk as an NT product against W^T; (3) dW_chunk = dz^T * hidden as an NT
 // product against hidden^T.  The contraction of (2)/(3) is over a different axis than the
 // recompute, and with H in the thousands the output tile of a fused kernel cannot stay in
@@ -70,6 +71,7 @@ static_assert(BM % kRowStep == 0 && BN % kRowStep == 0 && WM % 32 == 0 && WN % 3
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 template <int DT>
 __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
@@ -505,6 +507,9 @@ struct HeadArgs {
     const float* log_z;  // [N]
     const float* g;      // [N] upstream d loss / d logp
     int c0, c1;          // vocabulary rows of this chunk
+    float* stash;        // forward: raw products y[v][n], [V padded to BM, ld_stash] (vocabulary-major), or null
+    const float* stash_in;  // backward: the same buffer, or null (recompute)
+    int64_t ld_stash;
     uint16_t* dz;        // [N, ldz]   (columns = chunk-local vocabulary index)
     uint16_t* dzT;       // [chunk rows padded, ldzt]
     int64_t ldz, ldzt;
@@ -553,6 +558,23 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
         gemm_tile_nt<DT, TRLK_HEAD_BK_FWD>(W, m0, Hd, n0, a.H, acc, smem, true);
         // the next tile's first stages travel while this tile's logits are reduced (registers only)
         if (vt + 1 < vt1) gemm_tile_prefetch<TRLK_HEAD_BK_FWD>(W, m0 + BM, Hd, n0, a.H, smem);
+        if (a.stash != nullptr) {
+            // The tile's raw products go to memory for the backward (vocabulary-major, fp32): for one
+            // accumulator register the 32 lanes of a half-wave hold 32 consecutive tokens of one
+            // vocabulary row = one 128-byte line per store.  The buffer is padded to whole tiles.
+            const int uw = __builtin_amdgcn_readfirstlane(wave);
+            const int uwm = uw / WGN, uwn = uw % WGN;
+            const uint32_t lane_off = uint32_t((lane >> 5) * 4) * uint32_t(a.ld_stash) + uint32_t(lane & 31);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                    float* blk = a.stash + int64_t(m0 + uwm * WM + mb * 32) * a.ld_stash + (n0 + uwn * WN + nb * 32);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        __builtin_nontemporal_store(acc[mb][nb][r], blk + int64_t((r >> 2) * 8 + (r & 3)) * a.ld_stash + lane_off);
+                }
+        }
         const bool partial_tile = m0 + BM > a.V;
         // Common case (no soft-capping, tile inside the vocabulary): z = y * zs with one positive
         // scale, so the maximum is taken on the raw accumulators and the scale is folded into the
@@ -819,6 +841,86 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
     }
 }
 
+// dz pass of the backward from the forward's stashed products instead of a recompute: an
+// elementwise sweep over y[v][n] (memory bound: 4 bytes read, 2 x 2 bytes written per logit).
+// One workgroup = 64 vocabulary rows x 256 tokens.  A lane owns 4 consecutive tokens; a wave walks
+// over row pairs.  dz^T (vocabulary-major, like the stash) is written directly, dz (token-major)
+// through an LDS transpose.  Rows beyond the chunk and tokens beyond N are written as zeros.
+constexpr int kSdzRows = 64, kSdzTokens = 256, kSdzLdsRow = kSdzRows * 2 + 4;  // bytes per staged token row
+template <int DT>
+__global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
+    typedef Elem<DT> E;
+    __shared__ __attribute__((aligned(16))) char lds[kSdzTokens * kSdzLdsRow];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // consecutive workgroups take consecutive row groups of one token block: their 128-byte pieces of
+    // the token-major dz rows are neighbours in memory
+    const int n0 = blockIdx.y * kSdzTokens, r0 = blockIdx.x * kSdzRows;  // r0: chunk-local row
+    const int rows = a.c1 - a.c0;
+    const float zs = a.logit_scale * a.inv_t, zs2 = zs * kLog2e;
+    const bool plain = a.softcap <= 0.f && a.bias == nullptr;
+    float g[4], lzc[4];
+    int64_t tg[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int tok = n0 + lane * 4 + j;
+        const bool ok = tok < a.N;
+        g[j] = ok ? a.g[tok] : 0.f;
+        lzc[j] = ok ? a.log_z[tok] * kLog2e : INFINITY;
+        tg[j] = ok ? a.targets[tok] - a.c0 : -1;  // chunk-local target row
+    }
+#pragma unroll
+    for (int i = 0; i < kSdzRows / 8; ++i) {
+        const int rl = 2 * (wave + 4 * i);  // row pair rl, rl + 1 of this workgroup's 64
+        float d[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int row = r0 + rl + h;
+            const f32x4 y4 = __builtin_nontemporal_load(
+                reinterpret_cast<const f32x4*>(a.stash_in + int64_t(a.c0 + row) * a.ld_stash + n0 + lane * 4));
+            const float bias = (!plain && a.bias != nullptr && row < rows) ? a.bias[a.c0 + row] : 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float dv;
+                if (plain) {
+                    const float ngc = -g[j] * zs;
+                    dv = ngc * fast_exp2(fmaf(y4[j], zs2, -lzc[j]));
+                    if (tg[j] == row) dv -= ngc;
+                } else {
+                    float y = (y4[j] + bias) * a.logit_scale;
+                    float chain = zs;
+                    if (a.softcap > 0.f) {
+                        const float th = tanhf(y / a.softcap);
+                        y = th * a.softcap;
+                        chain *= 1.f - th * th;
+                    }
+                    dv = -g[j] * fast_exp2(fmaf(y * a.inv_t, kLog2e, -lzc[j]));
+                    if (tg[j] == row) dv += g[j];
+                    dv *= chain;
+                }
+                d[h][j] = (row < rows && g[j] != 0.f) ? dv : 0.f;
+            }
+            uint2 w;
+            w.x = E::pack2(d[h][0], d[h][1]);
+            w.y = E::pack2(d[h][2], d[h][3]);
+            *reinterpret_cast<uint2*>(a.dzT + int64_t(row) * a.ldzt + n0 + lane * 4) = w;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            *reinterpret_cast<uint32_t*>(lds + (lane * 4 + j) * kSdzLdsRow + rl * 2) = E::pack2(d[0][j], d[1][j]);
+    }
+    __syncthreads();
+    constexpr int kPieces = kSdzRows / 8;  // 16-byte pieces per staged token row
+#pragma unroll 2
+    for (int c = tid; c < kSdzTokens * kPieces; c += 256) {
+        const int tl = c / kPieces, pc = c % kPieces;
+        if (n0 + tl < a.N) {
+            const uint32_t* src = reinterpret_cast<const uint32_t*>(lds + tl * kSdzLdsRow + pc * 16);
+            u32x4 w = {src[0], src[1], src[2], src[3]};
+            *reinterpret_cast<u32x4*>(a.dz + int64_t(n0 + tl) * a.ldz + r0 + pc * 8) = w;
+        }
+    }
+}
+
 // Plain NT product with an output epilogue: C[M, N] (+)= A[M, K] * B[N, K]^T.
 //   MODE 0: store to `out_lp` in the storage dtype.
 //   MODE 1: fp32 accumulate into `out_f32` (first = overwrite).
@@ -989,6 +1091,13 @@ extern "C" size_t trlk_fused_head_fwd_workspace_bytes(int64_t n_tokens) {
     return n_tokens > 0 ? size_t(n_tokens) * (kFwdSplits * 4 + 1) * sizeof(float) : 0;
 }
 
+extern "C" size_t trlk_fused_head_stash_bytes(int64_t n_tokens, int64_t vocab, int64_t* out_ld) {
+    if (n_tokens <= 0 || vocab <= 0) return 0;
+    const int64_t ld = round_up(n_tokens, BN);
+    if (out_ld) *out_ld = ld;
+    return size_t(round_up(vocab, BM)) * size_t(ld) * sizeof(float);
+}
+
 extern "C" size_t trlk_fused_head_bwd_workspace_bytes(int64_t n_tokens, int64_t vocab, int64_t hidden_size,
                                                       int64_t chunk_size) {
     if (n_tokens <= 0 || vocab <= 0 || hidden_size <= 0 || chunk_size <= 0) return 0;
@@ -999,8 +1108,9 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
                                    int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                                    int64_t weight_stride, float temperature, float final_logit_softcapping,
                                    float logit_scale, const float* d_bias, float* d_out_logp, float* d_out_entropy,
-                                   float* d_out_log_z, float* d_out_target_is_max, int32_t* d_error_flag,
-                                   void* d_workspace, size_t workspace_bytes, trlk_stream_t stream) {
+                                   float* d_out_log_z, float* d_out_target_is_max, float* d_out_stash,
+                                   int64_t stash_ld, int32_t* d_error_flag, void* d_workspace, size_t workspace_bytes,
+                                   trlk_stream_t stream) {
     clear_error();
     if (int rc = check_head("fused_head_fwd", d_hidden, d_weight, d_targets, dtype, n_tokens, vocab, hidden_size,
                             hidden_stride, weight_stride, temperature))
@@ -1010,12 +1120,19 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
     TRLK_REQUIRE(d_workspace && workspace_bytes >= trlk_fused_head_fwd_workspace_bytes(n_tokens), TRLK_ERR_WORKSPACE,
                  "fused_head_fwd: workspace of %zu bytes needed, %zu given", trlk_fused_head_fwd_workspace_bytes(n_tokens),
                  workspace_bytes);
+    TRLK_REQUIRE(d_out_stash == nullptr || (stash_ld >= round_up(n_tokens, BN) && stash_ld % 4 == 0 &&
+                                            stash_ld < (int64_t(1) << 31) / 16 &&
+                                            reinterpret_cast<uintptr_t>(d_out_stash) % 16 == 0),
+                 TRLK_ERR_BAD_STRIDE, "fused_head_fwd: the stash needs a 16-byte aligned buffer with a row stride >= %lld (got %lld)",
+                 (long long)round_up(n_tokens, BN), (long long)stash_ld);
     hipStream_t s = static_cast<hipStream_t>(stream);
     HeadArgs a{};
     a.hidden = static_cast<const uint16_t*>(d_hidden);
     a.weight = static_cast<const uint16_t*>(d_weight);
     a.targets = d_targets;
     a.bias = d_bias;
+    a.stash = d_out_stash;
+    a.ld_stash = stash_ld;
     a.N = int(n_tokens);
     a.V = int(vocab);
     a.H = int(hidden_size);
@@ -1046,8 +1163,9 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
                                    int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                                    int64_t weight_stride, float temperature, float final_logit_softcapping,
                                    float logit_scale, const float* d_bias, const float* d_log_z, const float* d_g_logp,
-                                   int64_t chunk_size, void* d_out_dhidden, void* d_out_dweight, float* d_out_dbias,
-                                   void* d_workspace, size_t workspace_bytes, trlk_stream_t stream) {
+                                   int64_t chunk_size, const float* d_stash, int64_t stash_ld, void* d_out_dhidden,
+                                   void* d_out_dweight, float* d_out_dbias, void* d_workspace, size_t workspace_bytes,
+                                   trlk_stream_t stream) {
     clear_error();
     if (int rc = check_head("fused_head_bwd", d_hidden, d_weight, d_targets, dtype, n_tokens, vocab, hidden_size,
                             hidden_stride, weight_stride, temperature))
@@ -1064,6 +1182,12 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         return launch_status("fused_head_bwd (zero dW)");
     }
     TRLK_REQUIRE(d_log_z && d_g_logp, TRLK_ERR_NULL_POINTER, "fused_head_bwd: log_z / g_logp pointer is null");
+    TRLK_REQUIRE(d_stash == nullptr || n_tokens <= int64_t(65535) * kSdzTokens, TRLK_ERR_BAD_SHAPE,
+                 "fused_head_bwd: too many tokens for the stash path (%lld)", (long long)n_tokens);
+    TRLK_REQUIRE(d_stash == nullptr || (stash_ld >= round_up(n_tokens, BN) && stash_ld % 4 == 0 &&
+                                        reinterpret_cast<uintptr_t>(d_stash) % 16 == 0),
+                 TRLK_ERR_BAD_STRIDE, "fused_head_bwd: the stash needs a 16-byte aligned buffer with a row stride >= %lld (got %lld)",
+                 (long long)round_up(n_tokens, BN), (long long)stash_ld);
     const int64_t chunk = round_up(chunk_size < vocab ? chunk_size : vocab, BM);
     const BwdLayout l = bwd_layout(n_tokens, vocab, hidden_size, chunk);
     TRLK_REQUIRE(d_workspace && workspace_bytes >= l.total, TRLK_ERR_WORKSPACE,
@@ -1098,6 +1222,8 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     a.softcap = final_logit_softcapping > 0.f ? final_logit_softcapping : 0.f;
     a.log_z = d_log_z;
     a.g = d_g_logp;
+    a.stash_in = d_stash;
+    a.ld_stash = stash_ld;
     a.dz = dz;
     a.dzT = dzt;
     a.ldz = l.ld_c;
@@ -1111,9 +1237,19 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         a.c0 = int(c0);
         a.c1 = int(c1);
         const int n_vt = (rows + BM - 1) / BM;
-        int rc = dtype == TRLK_BF16
+        int rc;
+        if (d_stash != nullptr) {
+            const dim3 grid(unsigned(kpad / kSdzRows), unsigned(l.npad / kSdzTokens));
+            if (dtype == TRLK_BF16)
+                hipLaunchKernelGGL(head_dz_from_stash_kernel<TRLK_BF16>, grid, dim3(256), 0, s, a);
+            else
+                hipLaunchKernelGGL(head_dz_from_stash_kernel<TRLK_F16>, grid, dim3(256), 0, s, a);
+            rc = launch_status("fused_head_bwd (dz from the stash)");
+        } else {
+            rc = dtype == TRLK_BF16
                      ? launch_head(fused_head_dz_kernel<TRLK_BF16>, xcd_patch_grid(n_tb, n_vt), a, s, "fused_head_bwd (dz)")
                      : launch_head(fused_head_dz_kernel<TRLK_F16>, xcd_patch_grid(n_tb, n_vt), a, s, "fused_head_bwd (dz)");
+        }
         if (rc) return rc;
         if (d_out_dbias) {
             if (dtype == TRLK_BF16)

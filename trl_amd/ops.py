@@ -11,6 +11,7 @@ tensor).
 """
 from __future__ import annotations
 
+import ctypes
 import math
 import os
 from typing import Optional
@@ -440,6 +441,14 @@ def _head_operands(hidden: Tensor, weight: Tensor, targets: Tensor):
     return hidden, weight, targets.contiguous()
 
 
+def head_stash_fits(n_tokens: int, vocab: int) -> bool:
+    """Whether the forward should keep its raw products for the backward: the fp32 `[vocab, n_tokens]` buffer
+    (both padded to 256) must fit the budget `TRL_AMD_HEAD_STASH_GIB` (GiB, default 24; 0 = always recompute)."""
+    budget = float(os.environ.get("TRL_AMD_HEAD_STASH_GIB", "24"))
+    need = ((vocab + 255) // 256 * 256) * ((n_tokens + 255) // 256 * 256) * 4
+    return n_tokens > 0 and need <= budget * 2**30
+
+
 def _head_bias(bias, vocab):
     if bias is None:
         return None
@@ -450,10 +459,12 @@ def _head_bias(bias, vocab):
 
 @torch.library.custom_op("trl_amd::fused_head_fwd", mutates_args=(), device_types="cuda")
 def fused_head_fwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature: float, softcap: float,
-                   logit_scale: float, bias: Optional[Tensor] = None) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+                   logit_scale: float, bias: Optional[Tensor] = None,
+                   stash: bool = False) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor]:
     """hidden [N, H], weight [V, H] (bf16/fp16), targets int64 [N] -> fp32 (logp, entropy, log_z, target_is_max),
     each [N]; target_is_max is 1 where argmax(logits) == target.  `softcap <= 0` means no soft-capping.
-    `bias` [V] (any float dtype) is added to `hidden @ weight.T` before scaling."""
+    `bias` [V] (any float dtype) is added to `hidden @ weight.T` before scaling.  With `stash` the fifth
+    output holds the raw products (fp32 `[V padded, N padded]`) for `fused_head_bwd`; it is empty otherwise."""
     hidden, weight, targets = _head_operands(hidden, weight, targets)
     n, h = hidden.shape
     v = weight.shape[0]
@@ -464,30 +475,39 @@ def fused_head_fwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
     log_z = torch.empty((n,), dtype=torch.float32, device=dev)
     hit = torch.empty((n,), dtype=torch.float32, device=dev)
     if n == 0:
-        return logp, ent, log_z, hit
+        return logp, ent, log_z, hit, torch.empty((0, 0), dtype=torch.float32, device=dev)
+    if stash:
+        ld = ctypes.c_int64(0)
+        nbytes = lib.trlk_fused_head_stash_bytes(n, v, ctypes.addressof(ld))
+        saved = torch.empty((nbytes // (4 * ld.value), ld.value), dtype=torch.float32, device=dev)
+    else:
+        saved = torch.empty((0, 0), dtype=torch.float32, device=dev)
     ws_bytes = lib.trlk_fused_head_fwd_workspace_bytes(n)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         check(lib.trlk_fused_head_fwd(ptr(hidden), ptr(weight), ptr(targets), dtype_code(hidden.dtype), n, v, h,
                                       hidden.stride(0), weight.stride(0), temperature, softcap, logit_scale,
-                                      ptr(bias32), ptr(logp), ptr(ent), ptr(log_z), ptr(hit), ptr(_error_flag(dev)),
-                                      ptr(ws), ws_bytes, current_stream(dev)))
+                                      ptr(bias32), ptr(logp), ptr(ent), ptr(log_z), ptr(hit),
+                                      ptr(saved) if stash else None, saved.stride(0) if stash else 0,
+                                      ptr(_error_flag(dev)), ptr(ws), ws_bytes, current_stream(dev)))
     if _SYNC_CHECKS:
         check_device_errors()
-    return logp, ent, log_z, hit
+    return logp, ent, log_z, hit, saved
 
 
 @fused_head_fwd.register_fake
-def _(hidden, weight, targets, temperature, softcap, logit_scale, bias=None):
+def _(hidden, weight, targets, temperature, softcap, logit_scale, bias=None, stash=False):
     f = lambda: torch.empty((hidden.shape[0],), dtype=torch.float32, device=hidden.device)  # noqa: E731
-    return f(), f(), f(), f()
+    rows, cols = ((weight.shape[0] + 255) // 256 * 256, (hidden.shape[0] + 255) // 256 * 256) if stash else (0, 0)
+    return f(), f(), f(), f(), torch.empty((rows, cols), dtype=torch.float32, device=hidden.device)
 
 
 @torch.library.custom_op("trl_amd::fused_head_bwd", mutates_args=(), device_types="cuda")
 def fused_head_bwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature: float, softcap: float,
                    logit_scale: float, log_z: Tensor, g_logp: Tensor, chunk_size: int,
-                   bias: Optional[Tensor] = None) -> tuple[Tensor, Tensor, Tensor]:
-    """Returns (d hidden [N, H], d weight [V, H]) in the operand dtype and d bias (fp32 [V]; empty without a bias)."""
+                   bias: Optional[Tensor] = None, stash: Optional[Tensor] = None) -> tuple[Tensor, Tensor, Tensor]:
+    """Returns (d hidden [N, H], d weight [V, H]) in the operand dtype and d bias (fp32 [V]; empty without a bias).
+    `stash`: the fifth output of a `fused_head_fwd(..., stash=True)` on the same operands (skips the recompute)."""
     w_dtype = weight.dtype
     hidden, weight, targets = _head_operands(hidden, weight, targets)
     n, h = hidden.shape
@@ -498,18 +518,24 @@ def fused_head_bwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
     g = g_logp.contiguous().float()
     bias32 = _head_bias(bias, v)
     d_bias = torch.empty((v if bias is not None else 0,), dtype=torch.float32, device=dev)
+    if stash is not None and stash.numel() == 0:
+        stash = None
+    if stash is not None and (stash.dtype != torch.float32 or stash.stride(1) != 1 or
+                              stash.shape[0] < (v + 255) // 256 * 256 or stash.shape[1] < (n + 255) // 256 * 256):
+        raise ValueError("fused head: the stash does not belong to these operands")
     ws_bytes = lib.trlk_fused_head_bwd_workspace_bytes(max(n, 1), v, h, chunk_size)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         check(lib.trlk_fused_head_bwd(ptr(hidden), ptr(weight), ptr(targets), dtype_code(hidden.dtype), n, v, h,
                                       hidden.stride(0), weight.stride(0), temperature, softcap, logit_scale,
-                                      ptr(bias32), ptr(log_z), ptr(g), chunk_size, ptr(d_hidden), ptr(d_weight),
+                                      ptr(bias32), ptr(log_z), ptr(g), chunk_size, ptr(stash),
+                                      stash.stride(0) if stash is not None else 0, ptr(d_hidden), ptr(d_weight),
                                       ptr(d_bias) if bias is not None else None, ptr(ws), ws_bytes, current_stream(dev)))
     return d_hidden, (d_weight if w_dtype == d_weight.dtype else d_weight.to(w_dtype)), d_bias
 
 
 @fused_head_bwd.register_fake
-def _(hidden, weight, targets, temperature, softcap, logit_scale, log_z, g_logp, chunk_size, bias=None):
+def _(hidden, weight, targets, temperature, softcap, logit_scale, log_z, g_logp, chunk_size, bias=None, stash=None):
     return (torch.empty_like(hidden), torch.empty_like(weight),
             torch.empty((weight.shape[0] if bias is not None else 0,), dtype=torch.float32, device=hidden.device))
 

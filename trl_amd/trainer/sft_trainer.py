@@ -12,22 +12,24 @@ __all__ = ["_chunked_cross_entropy_loss"]
 
 class _FusedNLLFunction(torch.autograd.Function):
     """(hidden [N, H], weight [V, H], labels [N]) -> fp32 per-token (log-prob, entropy, argmax-hit); only the
-    log-prob is differentiable.  One matrix-core sweep forward, chunked recompute backward."""
+    log-prob is differentiable.  One matrix-core sweep forward; the backward works from the forward's stashed
+    products when they fit `ops.head_stash_fits`, from a chunked recompute otherwise."""
 
     @staticmethod
     def forward(ctx, hidden, weight, labels, chunk_size, softcap, logit_scale):
-        logp, ent, log_z, hit = ops.fused_head_fwd(hidden, weight, labels, 1.0, softcap, logit_scale)
-        ctx.save_for_backward(hidden, weight, labels, log_z)
+        stash = any(ctx.needs_input_grad[:2]) and ops.head_stash_fits(hidden.shape[0], weight.shape[0])
+        logp, ent, log_z, hit, saved = ops.fused_head_fwd(hidden, weight, labels, 1.0, softcap, logit_scale, None, stash)
+        ctx.save_for_backward(hidden, weight, labels, log_z, saved)
         ctx.cfg = (int(chunk_size), softcap, logit_scale)
         ctx.mark_non_differentiable(ent, hit)
         return logp, ent, hit
 
     @staticmethod
     def backward(ctx, g_logp, g_ent, g_hit):
-        hidden, weight, labels, log_z = ctx.saved_tensors
+        hidden, weight, labels, log_z, saved = ctx.saved_tensors
         chunk_size, softcap, logit_scale = ctx.cfg
         d_hidden, d_weight, _ = ops.fused_head_bwd(hidden, weight, labels, 1.0, softcap, logit_scale, log_z, g_logp,
-                                                chunk_size)
+                                                   chunk_size, None, saved)
         return d_hidden, d_weight, None, None, None, None
 
 

@@ -147,26 +147,30 @@ class _ChunkedLogProbFunction(torch.autograd.Function):
     chunk_size, final_logit_softcapping=None, logit_scale=1.0) -> (logprobs fp32 [N], entropy fp32 [N])`.
 
     The forward is one matrix-core kernel sweep (no vocabulary chunking is needed, `chunk_size` only
-    sizes the backward's dz workspace).  The entropy output is not differentiable, as in the reference.
+    sizes the backward's dz workspace).  When a gradient is required and the fp32 `[V, N]` products fit
+    `ops.head_stash_fits` (24 GiB by default), the forward keeps them and the backward skips the
+    reference's recompute of the logits; otherwise it recomputes them chunk by chunk as the reference does.
+    The entropy output is not differentiable, as in the reference.
     One argument beyond the reference's: `bias` [V], the `lm_head` bias the fused-linear losses take."""
 
     @staticmethod
     def forward(ctx, last_hidden, weight, targets, temperature, chunk_size, final_logit_softcapping=None,
                 logit_scale=1.0, bias=None):
         cap = 0.0 if final_logit_softcapping is None else float(final_logit_softcapping)
-        logp, ent, log_z, _ = ops.fused_head_fwd(last_hidden, weight, targets, float(temperature), cap,
-                                                 float(logit_scale), bias)
-        ctx.save_for_backward(last_hidden, weight, targets, log_z, bias)
+        stash = any(ctx.needs_input_grad[:2]) and ops.head_stash_fits(last_hidden.shape[0], weight.shape[0])
+        logp, ent, log_z, _, saved = ops.fused_head_fwd(last_hidden, weight, targets, float(temperature), cap,
+                                                        float(logit_scale), bias, stash)
+        ctx.save_for_backward(last_hidden, weight, targets, log_z, bias, saved)
         ctx.cfg = (float(temperature), int(chunk_size), cap, float(logit_scale))
         ctx.mark_non_differentiable(ent)
         return logp, ent
 
     @staticmethod
     def backward(ctx, grad_logprobs, grad_entropy):
-        hidden, weight, targets, log_z, bias = ctx.saved_tensors
+        hidden, weight, targets, log_z, bias, saved = ctx.saved_tensors
         temperature, chunk_size, cap, logit_scale = ctx.cfg
         d_hidden, d_weight, d_bias = ops.fused_head_bwd(hidden, weight, targets, temperature, cap, logit_scale,
-                                                        log_z, grad_logprobs, chunk_size, bias)
+                                                        log_z, grad_logprobs, chunk_size, bias, saved)
         return (d_hidden, d_weight, None, None, None, None, None,
                 None if bias is None else d_bias.to(bias.dtype))
 
