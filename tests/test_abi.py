@@ -88,6 +88,23 @@ def test_host_side_argument_validation():
     # dpo: odd batch
     assert lib.trlk_dpo_loss(fake, fake, fake, fake, 3, 8, 0.1, fake, fake, fake, fake, None) == -2
     assert lib.trlk_rloo_loss(fake, fake, fake, fake, 0, 8, 0.2, 0.2, fake, fake, fake, fake, None) == -2
+    # fused head: fp32 operands, ragged hidden size, a stash whose rows are too short, missing workspace
+    fake16 = 0x1000
+
+    def head_fwd(dtype=_lib.BF16, h=64, stash=None, stash_ld=0, ws=fake16, ws_bytes=1 << 30):
+        return lib.trlk_fused_head_fwd(fake16, fake16, fake, dtype, 300, 1000, h, h, h, 1.0, 0.0, 1.0, None, fake, fake,
+                                       fake, None, stash, stash_ld, None, ws, ws_bytes, None)
+
+    assert head_fwd(dtype=_lib.F32) == -3 and "bf16 or fp16" in _lib.last_error()
+    assert head_fwd(h=60) == -4
+    assert head_fwd(stash=fake16, stash_ld=300) == -4 and "stash" in _lib.last_error()
+    assert head_fwd(ws_bytes=16) == -6
+    ld = ctypes.c_int64(0)
+    assert lib.trlk_fused_head_stash_bytes(300, 1000, ctypes.addressof(ld)) == 1024 * 512 * 4 and ld.value == 512
+    assert lib.trlk_fused_head_bwd(fake16, fake16, fake, _lib.BF16, 300, 1000, 64, 64, 64, 1.0, 0.0, 1.0, None, fake, fake,
+                                   256, fake16, 256, fake16, fake16, None, fake16, 1 << 40, None) == -4
+    assert lib.trlk_fused_head_bwd(fake16, fake16, fake, _lib.BF16, 300, 1000, 64, 64, 64, 1.0, 0.0, 1.0, None, fake, fake,
+                                   0, None, 0, fake16, fake16, None, fake16, 1 << 40, None) == -5  # chunk_size
     # an empty problem is a successful no-op
     assert lib.trlk_logp_entropy_fwd(None, _lib.F32, 0, 4, 8, 32, 8, None, 1, 1.0, None, None, None, None, None, None, None) == 0
     assert _lib.last_error() == ""
