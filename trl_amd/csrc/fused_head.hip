@@ -1031,7 +1031,7 @@ BwdLayout bwd_layout(int64_t N, int64_t V, int64_t H, int64_t chunk) {
         o += (bytes + 255) / 256 * 256;
         return at;
     };
-    l.off_wt = take(size_t(H) * l.ld_v * 2);
+    l.off_wt = take(size_t(H) * l.ld_c * 2);
     l.off_ht = take(size_t(H) * l.ld_n * 2);
     l.off_dz = take(size_t(N) * l.ld_c * 2);
     l.off_dzt = take(size_t(l.cpad) * l.ld_n * 2);
@@ -1193,16 +1193,13 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     TRLK_REQUIRE(d_workspace && workspace_bytes >= l.total, TRLK_ERR_WORKSPACE,
                  "fused_head_bwd: workspace of %zu bytes needed, %zu given", l.total, workspace_bytes);
     char* ws = static_cast<char*>(d_workspace);
-    uint16_t* wt = reinterpret_cast<uint16_t*>(ws + l.off_wt);    // [H, vpad], row stride ld_v
+    uint16_t* wt = reinterpret_cast<uint16_t*>(ws + l.off_wt);    // [H, cpad], row stride ld_c (one chunk at a time)
     uint16_t* ht = reinterpret_cast<uint16_t*>(ws + l.off_ht);    // [H, npad], row stride ld_n
     uint16_t* dz = reinterpret_cast<uint16_t*>(ws + l.off_dz);    // [N, cpad], row stride ld_c
     uint16_t* dzt = reinterpret_cast<uint16_t*>(ws + l.off_dzt);  // [cpad, npad], row stride ld_n
     float* dh = reinterpret_cast<float*>(ws + l.off_dh);          // [N, H]
     (void)es;
     const int H = int(hidden_size), N = int(n_tokens), V = int(vocab);
-    hipLaunchKernelGGL(transpose16_kernel, dim3((H + 63) / 64, unsigned((l.vpad + 63) / 64)), dim3(256), 0, s,
-                       static_cast<const uint16_t*>(d_weight), weight_stride, V, H, wt, l.ld_v, l.vpad);
-    if (int rc = launch_status("fused_head_bwd (W^T)")) return rc;
     hipLaunchKernelGGL(transpose16_kernel, dim3((H + 63) / 64, unsigned((l.npad + 63) / 64)), dim3(256), 0, s,
                        static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.ld_n, l.npad);
     if (int rc = launch_status("fused_head_bwd (hidden^T)")) return rc;
@@ -1261,13 +1258,19 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
             if (int rc2 = launch_status("fused_head_bwd (dBias)")) return rc2;
         }
         const bool first = c0 == 0, last = c1 == vocab;
-        // dHidden[N, H] += dz[N, chunk] * (W^T[H, chunk])^T ; W^T columns beyond V are zero and so is dz there
+        // W_chunk^T [H, kpad] (columns beyond the chunk's rows are zero): the chunk's own transposed copy keeps the
+        // row stride of this operand as short as that of the other three
+        hipLaunchKernelGGL(transpose16_kernel, dim3((H + 63) / 64, unsigned((kpad + 63) / 64)), dim3(256), 0, s,
+                           static_cast<const uint16_t*>(d_weight) + c0 * weight_stride, weight_stride, rows, H, wt, l.ld_c,
+                           int64_t(kpad));
+        if (int rc2 = launch_status("fused_head_bwd (W^T)")) return rc2;
+        // dHidden[N, H] += dz[N, chunk] * (W_chunk^T[H, chunk])^T
         GemmArgs gh{};
         gh.A = Operand{dz, l.ld_c, N};
-        gh.B = Operand{wt + c0, l.ld_v, H};
+        gh.B = Operand{wt, l.ld_c, H};
         gh.M = N;
         gh.N = H;
-        gh.K = int(c0 + kpad <= l.vpad ? kpad : l.vpad - c0);
+        gh.K = kpad;
         gh.out_f32 = dh;
         gh.ld_f32 = H;
         gh.out_lp = static_cast<uint16_t*>(d_out_dhidden);
