@@ -108,6 +108,75 @@ def cpu_baseline(w, loss_type, rows_per_seq=512, n_seq=32, repeats=2):
     }
 
 
+def cpu_baseline_head(w, rows=128, chunk=8192):
+    """The oracle's chunked lm_head + log-prob operator (the reference's algorithm: vocabulary slabs, online
+    log-sum-exp, recompute backward with fp32 products) forward + backward on `rows` tokens of the workload's
+    hidden size and vocabulary."""
+    import oracle
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    g = torch.Generator().manual_seed(0)
+    H, V = w["H"], w["V"]
+    # a 2048-row random block repeated down the vocabulary: the timing does not depend on the values, and drawing
+    # 5.4e8 normals on the host would take longer than the measurement
+    block = (0.02 * torch.randn(2048, H, generator=g)).bfloat16()
+    weight = block.repeat((V + 2047) // 2048, 1)[:V].contiguous().requires_grad_(True)
+
+    def run(n):
+        hid = torch.randn(n, H, generator=g).bfloat16().requires_grad_(True)
+        targets = torch.randint(0, V, (n,), generator=g)
+        gout = torch.randn(n, generator=g)
+        weight.grad = None
+        t0 = time.perf_counter()
+        lp, _ = oracle.ChunkedLogProbOracle.apply(hid, weight, targets, w["temperature"], chunk)
+        (lp * gout).sum().backward()
+        return time.perf_counter() - t0
+
+    dt = run(rows)
+    if dt < 5.0:  # a fast host: grow the sample towards ~10 s of work
+        rows = int(min(4096, rows * 10.0 / max(dt, 1e-3))) // 64 * 64
+        dt = run(rows)
+    return {"value": rows / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle chunked head fwd+bwd on hidden bf16 [{rows},{H}], W bf16 [{V},{H}], chunk {chunk}, one run, "
+                      f"{dt:.2f} s; torch {torch.__version__} CPU"}
+
+
+def cpu_baseline_dpo(w, n_pairs=2, length=257):
+    """The oracle's `DPOTrainer._compute_loss` restatement (sigmoid loss, all logged metrics) forward + backward on
+    `2 * n_pairs` sequences of `length` tokens at the workload's vocabulary."""
+    import oracle
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    g = torch.Generator().manual_seed(0)
+    V = w["V"]
+
+    def run(pairs):
+        B = 2 * pairs
+        logits = (2.0 * torch.randn(B, length, V, generator=g)).bfloat16()
+        ids = torch.randint(0, V, (B, length), generator=g)
+        cm = torch.zeros(B, length, dtype=torch.long)
+        cm[:, length // 8:] = 1
+        ref = -8.0 * (length - length // 8) + torch.randn(B, generator=g)
+        best = float("inf")
+        for _ in range(2):
+            leaf = logits.clone().requires_grad_(True)
+            t0 = time.perf_counter()
+            loss, _ = oracle.dpo_compute_loss(leaf, ids, cm, ref[:pairs], ref[pairs:], w["beta"])
+            loss.backward()
+            best = min(best, time.perf_counter() - t0)
+        return best
+
+    best = run(n_pairs)
+    if best < 2.0:  # a fast host: grow the sample towards ~5 s per run
+        n_pairs = int(min(16, max(n_pairs, n_pairs * 5.0 / max(best, 1e-3))))
+        best = run(n_pairs)
+    B = 2 * n_pairs
+    rows = B * length
+    return {"value": rows / best, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle DPO loss fwd+bwd on bf16 logits [{B},{length},{V}] ({rows} token rows), best of 2, "
+                      f"{best:.2f} s; torch {torch.__version__} CPU"}
+
+
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
 
 
@@ -215,7 +284,7 @@ def bench_head(args, w):
             "fused_head_fwd": {"avg_ms": fwd_ms, "TFLOPs": fwd_tf, "frac": fwd_tf / MFMA_BF16_PEAK_TFLOPS},
             "fused_head_bwd": {"avg_ms": bwd_ms, "TFLOPs": bwd_tf, "frac": bwd_tf / MFMA_BF16_PEAK_TFLOPS,
                                "products": 2 if stash else 3}}),
-        "cpu_baseline": None,
+        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_head(w),
     }
     print(json.dumps(result))
 
@@ -304,7 +373,7 @@ def bench_dpo(args, w):
             "frac": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}},
         "mask_aware": {"ms_per_step": ms_aware, "tokens_per_s": R / (ms_aware * 1e-3),
                        "note": "only rows inside the completion mask are read; loss, metrics and dlogits identical"},
-        "cpu_baseline": None,
+        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_dpo(w),
     }
     print(json.dumps(result))
 
