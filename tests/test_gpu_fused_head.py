@@ -206,9 +206,57 @@ def test_masked_rows_and_scatter(amd):
     assert torch.count_nonzero(lp_e) == 0
 
 
-def test_fp32_operands_are_rejected_loudly(amd):
+def test_golden_chunked_logprob_fp32(amd):
+    """fp32 operands (the dtype of the reference's own unit test, tests/test_utils.py:1161-1232) at its tolerance:
+    forward and backward within 1e-5 of what the reference operator wrote."""
+    cases, g = load_golden("chunked_logprob")
+    ran = 0
+    for case in cases:
+        if case["dtype"] != "float32":
+            continue
+        c = f"c{case['id']}_"
+        hidden, weight = _t(g[c + "hidden"]), _t(g[c + "weight"])
+        labels, gout = _t(g[c + "labels"]), _t(g[c + "grad_out"])
+        lp, ent, dh, dw = _run_device(amd, hidden, weight, labels, case["temperature"], case["chunk"], case["softcap"],
+                                      case["logit_scale"], gout)
+        assert dh.dtype == torch.float32 and dw.dtype == torch.float32
+        torch.testing.assert_close(lp, _t(g[c + "out_logprobs"]), atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(ent, _t(g[c + "out_entropy"]), atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(dh, _t(g[c + "out_dhidden"]), atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(dw, _t(g[c + "out_dweight"]), atol=1e-5, rtol=1e-5)
+        ran += 1
+    assert ran >= 1
+
+
+def test_fp32_operands_blocks_bias_and_ragged_shapes(amd, monkeypatch):
+    """The fp32-operand path over several token blocks, with bias, soft-capping and odd sizes, against autograd."""
+    from trl_amd.trainer import utils as tu
+
+    monkeypatch.setattr(tu, "_fp32_head_block_rows", lambda vocab: 64)
+    g = torch.Generator().manual_seed(91)
+    n, h, v = 150, 37, 301
+    hidden, weight, bias = torch.randn(n, h, generator=g), 0.3 * torch.randn(v, h, generator=g), torch.randn(v, generator=g)
+    labels, gout = torch.randint(0, v, (n,), generator=g), torch.randn(n, generator=g)
+    rh, rw, rb = (x.clone().requires_grad_(True) for x in (hidden, weight, bias))
+    y = (rh @ rw.t() + rb) * 0.5
+    y = torch.tanh(y / 5.0) * 5.0
+    lp_all = F.log_softmax(y / 0.8, -1)
+    rlp = lp_all.gather(-1, labels[:, None]).squeeze(-1)
+    rent = -(lp_all.exp() * lp_all).sum(-1)
+    (rlp * gout).sum().backward()
+    dh, dw, db = (x.to(DEV).requires_grad_(True) for x in (hidden, weight, bias))
+    lp, ent = amd._ChunkedLogProbFunction.apply(dh, dw, labels.to(DEV), 0.8, 64, 5.0, 0.5, db)
+    (lp * gout.to(DEV)).sum().backward()
+    torch.testing.assert_close(lp.detach().cpu(), rlp.detach(), atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(ent.cpu(), rent.detach(), atol=1e-5, rtol=1e-5)
+    for got, want in ((dh, rh), (dw, rw), (db, rb)):
+        torch.testing.assert_close(got.grad.cpu(), want.grad, atol=2e-5, rtol=1e-4)
+
+
+def test_fp64_operands_are_rejected_loudly(amd):
     with pytest.raises(TypeError):
-        amd._ChunkedLogProbFunction.apply(torch.randn(4, 8, device=DEV), torch.randn(16, 8, device=DEV),
+        amd._ChunkedLogProbFunction.apply(torch.randn(4, 8, device=DEV, dtype=torch.float64),
+                                          torch.randn(16, 8, device=DEV, dtype=torch.float64),
                                           torch.zeros(4, dtype=torch.long, device=DEV), 1.0, 8)
 
 
@@ -255,6 +303,15 @@ def test_golden_sft_chunked_nll(amd):
         assert _rel_l2(dhs.grad.float(), ohs.grad) < 1e-2 and _rel_l2(dw.grad.float(), ow.grad) < 1e-2
         if case["dtype"] == "float32":  # and loosely against the reference's own fp32 numbers (bf16 operand rounding)
             assert abs(float(loss) - float(g[c + "out_loss"])) <= 2e-2 * abs(float(g[c + "out_loss"]))
+            # fp32 operands: the reference's numbers at fp32 accuracy
+            fhs, fw = _t(g[c + "hidden"]).to(DEV).requires_grad_(True), _t(g[c + "weight"]).to(DEV).requires_grad_(True)
+            loss, correct, ent, nv = _chunked_cross_entropy_loss(fhs, fw, 256, **common, **dkw)
+            loss.backward()
+            assert abs(float(loss) - float(g[c + "out_loss"])) <= 1e-5 * max(1.0, abs(float(g[c + "out_loss"])))
+            assert float(correct) == float(g[c + "out_correct"])
+            assert abs(float(ent) - float(g[c + "out_entropy_sum"])) <= 1e-4 * abs(float(g[c + "out_entropy_sum"]))
+            torch.testing.assert_close(fhs.grad.cpu(), _t(g[c + "out_dhidden"]), atol=1e-6, rtol=1e-4)
+            torch.testing.assert_close(fw.grad.cpu(), _t(g[c + "out_dweight"]), atol=1e-6, rtol=1e-4)
     # all positions masked: zero loss that still backpropagates
     dhs = torch.randn(2, 5, 32, device=DEV).bfloat16().requires_grad_(True)
     dw = torch.randn(64, 32, device=DEV).bfloat16().requires_grad_(True)

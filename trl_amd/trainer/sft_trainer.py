@@ -6,6 +6,7 @@ import torch
 from torch import Tensor
 
 from .. import ops
+from .utils import _fp32_head_backward, _fp32_head_forward
 
 __all__ = ["_chunked_cross_entropy_loss"]
 
@@ -16,21 +17,35 @@ class _FusedNLLFunction(torch.autograd.Function):
     products when they fit `ops.head_stash_fits`, from a chunked recompute otherwise."""
 
     @staticmethod
-    def forward(ctx, hidden, weight, labels, chunk_size, softcap, logit_scale):
-        stash = any(ctx.needs_input_grad[:2]) and ops.head_stash_fits(hidden.shape[0], weight.shape[0])
-        logp, ent, log_z, hit, saved = ops.fused_head_fwd(hidden, weight, labels, 1.0, softcap, logit_scale, None, stash)
-        ctx.save_for_backward(hidden, weight, labels, log_z, saved)
+    def forward(ctx, hidden, weight, labels, chunk_size, softcap, logit_scale, bias=None):
         ctx.cfg = (int(chunk_size), softcap, logit_scale)
+        if hidden.dtype == torch.float32:  # fp32 operands: library GEMMs around the streaming kernels
+            if not hidden.is_cuda:
+                raise NotImplementedError("the fused head runs on the GPU only")
+            logp, ent, log_z, hit = _fp32_head_forward(hidden, weight.float(), labels.long(), 1.0, softcap, logit_scale,
+                                                       None if bias is None else bias.float(), True)
+            ctx.save_for_backward(hidden, weight, labels, log_z, None, bias)
+            ctx.mark_non_differentiable(ent, hit)
+            return logp, ent, hit
+        stash = any(ctx.needs_input_grad[:2]) and ops.head_stash_fits(hidden.shape[0], weight.shape[0])
+        logp, ent, log_z, hit, saved = ops.fused_head_fwd(hidden, weight, labels, 1.0, softcap, logit_scale, bias, stash)
+        ctx.save_for_backward(hidden, weight, labels, log_z, saved, bias)
         ctx.mark_non_differentiable(ent, hit)
         return logp, ent, hit
 
     @staticmethod
     def backward(ctx, g_logp, g_ent, g_hit):
-        hidden, weight, labels, log_z, saved = ctx.saved_tensors
+        hidden, weight, labels, log_z, saved, bias = ctx.saved_tensors
         chunk_size, softcap, logit_scale = ctx.cfg
-        d_hidden, d_weight, _ = ops.fused_head_bwd(hidden, weight, labels, 1.0, softcap, logit_scale, log_z, g_logp,
-                                                   chunk_size, None, saved)
-        return d_hidden, d_weight, None, None, None, None
+        if hidden.dtype == torch.float32:
+            d_hidden, d_weight, d_bias = _fp32_head_backward(hidden, weight.float(), labels.long(), 1.0, softcap,
+                                                             logit_scale, None if bias is None else bias.float(), log_z,
+                                                             g_logp)
+            d_weight = d_weight.to(weight.dtype)
+        else:
+            d_hidden, d_weight, d_bias = ops.fused_head_bwd(hidden, weight, labels, 1.0, softcap, logit_scale, log_z,
+                                                            g_logp, chunk_size, bias, saved)
+        return d_hidden, d_weight, None, None, None, None, None if bias is None else d_bias.to(bias.dtype)
 
 
 def _chunked_cross_entropy_loss(
@@ -53,8 +68,6 @@ def _chunked_cross_entropy_loss(
     the kernels need no token chunking).  `correct_count` counts tokens whose label holds the row maximum."""
     if labels is None and shift_labels is None:
         raise ValueError("At least one of `labels` or `shift_labels` must be provided.")
-    if lm_head_bias is not None:
-        raise NotImplementedError("lm_head_bias is not implemented by the trl_amd fused head")
     if shift_labels is not None:
         hidden = hidden_states.reshape(-1, hidden_states.size(-1))
         flat_labels = shift_labels.reshape(-1)
@@ -66,11 +79,13 @@ def _chunked_cross_entropy_loss(
     if int(n_valid) == 0:
         # whole micro-batch masked: keep the loss attached to every trainable input (sft_trainer.py:186-195)
         loss = (hidden_states.float().sum() + lm_head_weight.float().sum()) * 0.0
+        if lm_head_bias is not None:
+            loss = loss + lm_head_bias.float().sum() * 0.0
         zero = hidden.new_zeros((), dtype=torch.float32)
         return loss, zero, zero.clone(), n_valid
     cap = 0.0 if final_logit_softcapping is None else float(final_logit_softcapping)
     logp, ent, hit = _FusedNLLFunction.apply(hidden[valid], lm_head_weight, flat_labels[valid], chunk_size, cap,
-                                             float(logit_scale))
+                                             float(logit_scale), lm_head_bias)
     loss = -logp.sum()
     if num_items_in_batch is None:
         loss = loss / n_valid

@@ -140,6 +140,72 @@ def nanmax(tensor: Tensor) -> Tensor:
 # ----------------------------------------------------------------------------------------------
 # fused lm_head + log-prob (reference: trl/trainer/utils.py:1291-1517)
 # ----------------------------------------------------------------------------------------------
+def _fp32_head_block_rows(vocab: int) -> int:
+    """Token rows per block of the fp32-operand path: about 1 GiB of fp32 logits at a time."""
+    return max(64, min(8192, (1 << 28) // max(vocab, 1)))
+
+
+def _fp32_head_logits(hidden_blk, weight, bias, cap, logit_scale):
+    """fp32 `[rows, V]` logits of a block of tokens before the temperature, and the soft-cap's tanh (or None)."""
+    y = hidden_blk @ weight.t()
+    if bias is not None:
+        y += bias
+    if logit_scale != 1.0:
+        y *= logit_scale
+    th = None
+    if cap > 0.0:
+        th = torch.tanh(y / cap)
+        y = th * cap
+    return y, th
+
+
+def _fp32_head_forward(hidden, weight, targets, temperature, cap, logit_scale, bias, want_hit=False):
+    """fp32 operands: the products come from the fp32 GEMM library one block of tokens at a time, the log-sum-exp,
+    entropy and gather of each block from the streaming log-prob kernel (whole vocabulary rows, so no online merge)."""
+    n, v = hidden.shape[0], weight.shape[0]
+    logp = torch.empty(n, dtype=torch.float32, device=hidden.device)
+    ent = torch.empty_like(logp)
+    lse = torch.empty_like(logp)
+    hit = torch.empty_like(logp) if want_hit else None
+    step = _fp32_head_block_rows(v)
+    for r0 in range(0, n, step):
+        r1 = min(r0 + step, n)
+        z, _ = _fp32_head_logits(hidden[r0:r1], weight, bias, cap, logit_scale)
+        idx = targets[r0:r1].reshape(-1, 1)
+        if want_hit:  # the row statistics carry the arg-max flag of the target
+            lp, e, l, st = ops.logp_entropy_stats_fwd(z.unsqueeze(0), idx, temperature, 0, r1 - r0, None)
+            hit[r0:r1] = st[:, 2]
+        else:
+            lp, e, l = ops.logp_entropy_fwd(z.unsqueeze(0), idx, temperature, 0, r1 - r0, None)
+        logp[r0:r1], ent[r0:r1], lse[r0:r1] = lp.view(-1), e, l
+    return (logp, ent, lse, hit) if want_hit else (logp, ent, lse)
+
+
+def _fp32_head_backward(hidden, weight, targets, temperature, cap, logit_scale, bias, lse, grad_logprobs):
+    """Recompute per block of tokens, d logits from the streaming backward kernel, the two products from the GEMM
+    library; everything in fp32."""
+    n, v = hidden.shape[0], weight.shape[0]
+    d_hidden = torch.empty_like(hidden)
+    d_weight = torch.zeros_like(weight)
+    d_bias = torch.zeros(v, dtype=torch.float32, device=hidden.device) if bias is not None else None
+    g = grad_logprobs.contiguous().float()
+    step = _fp32_head_block_rows(v)
+    for r0 in range(0, n, step):
+        r1 = min(r0 + step, n)
+        z, th = _fp32_head_logits(hidden[r0:r1], weight, bias, cap, logit_scale)
+        dz = ops.logp_entropy_bwd(z.unsqueeze(0), targets[r0:r1].reshape(-1, 1), temperature, 0, r1 - r0, lse[r0:r1], None,
+                                  g[r0:r1].reshape(-1, 1), None).squeeze(0)
+        if th is not None:
+            dz *= 1.0 - th * th
+        if logit_scale != 1.0:
+            dz *= logit_scale
+        d_hidden[r0:r1] = dz @ weight
+        d_weight.addmm_(dz.t(), hidden[r0:r1])
+        if d_bias is not None:
+            d_bias += dz.sum(0)
+    return d_hidden, d_weight, d_bias
+
+
 class _ChunkedLogProbFunction(torch.autograd.Function):
     """Per-token log-probs and entropy of `softmax((hidden @ weight.T) / temperature)` without ever
     materialising the `[N, V]` logits.  Same call signature as the reference operator
@@ -150,6 +216,8 @@ class _ChunkedLogProbFunction(torch.autograd.Function):
     sizes the backward's dz workspace).  When a gradient is required and the fp32 `[V, N]` products fit
     `ops.head_stash_fits` (24 GiB by default), the forward keeps them and the backward skips the
     reference's recompute of the logits; otherwise it recomputes them chunk by chunk as the reference does.
+    fp32 operands take a separate path: fp32 library GEMMs over blocks of tokens around the streaming log-prob
+    kernels (the matrix-core kernels take 16-bit operands only); fp64 is rejected.
     The entropy output is not differentiable, as in the reference.
     One argument beyond the reference's: `bias` [V], the `lm_head` bias the fused-linear losses take."""
 
@@ -157,6 +225,16 @@ class _ChunkedLogProbFunction(torch.autograd.Function):
     def forward(ctx, last_hidden, weight, targets, temperature, chunk_size, final_logit_softcapping=None,
                 logit_scale=1.0, bias=None):
         cap = 0.0 if final_logit_softcapping is None else float(final_logit_softcapping)
+        if last_hidden.dtype == torch.float32:
+            if not last_hidden.is_cuda:
+                raise NotImplementedError("the fused head runs on the GPU only")
+            w32 = weight.float()
+            logp, ent, log_z = _fp32_head_forward(last_hidden, w32, targets.long(), float(temperature), cap,
+                                                  float(logit_scale), None if bias is None else bias.float())
+            ctx.save_for_backward(last_hidden, weight, targets, log_z, bias, None)
+            ctx.cfg = (float(temperature), int(chunk_size), cap, float(logit_scale))
+            ctx.mark_non_differentiable(ent)
+            return logp, ent
         stash = any(ctx.needs_input_grad[:2]) and ops.head_stash_fits(last_hidden.shape[0], weight.shape[0])
         logp, ent, log_z, _, saved = ops.fused_head_fwd(last_hidden, weight, targets, float(temperature), cap,
                                                         float(logit_scale), bias, stash)
@@ -169,6 +247,12 @@ class _ChunkedLogProbFunction(torch.autograd.Function):
     def backward(ctx, grad_logprobs, grad_entropy):
         hidden, weight, targets, log_z, bias, saved = ctx.saved_tensors
         temperature, chunk_size, cap, logit_scale = ctx.cfg
+        if hidden.dtype == torch.float32:
+            d_hidden, d_weight, d_bias = _fp32_head_backward(hidden, weight.float(), targets.long(), temperature, cap,
+                                                             logit_scale, None if bias is None else bias.float(), log_z,
+                                                             grad_logprobs)
+            return (d_hidden, d_weight.to(weight.dtype), None, None, None, None, None,
+                    None if bias is None else d_bias.to(bias.dtype))
         d_hidden, d_weight, d_bias = ops.fused_head_bwd(hidden, weight, targets, temperature, cap, logit_scale,
                                                         log_z, grad_logprobs, chunk_size, bias, saved)
         return (d_hidden, d_weight, None, None, None, None, None,
