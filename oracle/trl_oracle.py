@@ -856,7 +856,7 @@ def patch_chunked_rows(hidden_states, labels, completion_mask, weight, temperatu
 # SFT chunked cross-entropy              trl/trainer/sft_trainer.py:99-234
 # --------------------------------------------------------------------------------------
 def chunked_cross_entropy_loss(hidden_states, lm_head_weight, chunk_size, labels=None, shift_labels=None,
-                               num_items_in_batch=None, logit_scale=1.0, final_logit_softcapping=None):
+                               num_items_in_batch=None, logit_scale=1.0, final_logit_softcapping=None, lm_head_bias=None):
     """Shift (or take pre-shifted labels) (sft_trainer.py:175-180), drop `-100` rows, and over token
     chunks of `chunk_size` accumulate fp32 NLL sum, argmax hits and entropy sum (`_chunk`, :99-114);
     loss = sum / num_items_in_batch, or / n_valid (:228-233).  Returns (loss, correct, entropy_sum, n_valid)."""
@@ -870,13 +870,18 @@ def chunked_cross_entropy_loss(hidden_states, lm_head_weight, chunk_size, labels
     n_valid = keep.sum()
     if int(n_valid) == 0:
         zero = torch.zeros((), dtype=torch.float32)
-        return (hidden_states.float().sum() + lm_head_weight.float().sum()) * 0.0, zero, zero.clone(), n_valid
+        loss = (hidden_states.float().sum() + lm_head_weight.float().sum()) * 0.0
+        if lm_head_bias is not None:
+            loss = loss + lm_head_bias.float().sum() * 0.0
+        return loss, zero, zero.clone(), n_valid
     hidden, lab = hidden[keep], lab[keep]
     loss = torch.zeros((), dtype=torch.float32)
     correct = torch.zeros((), dtype=torch.float32)
     entropy_sum = torch.zeros((), dtype=torch.float32)
     for lo in range(0, hidden.shape[0], chunk_size):
         z = hidden[lo : lo + chunk_size].float() @ lm_head_weight.float().t()
+        if lm_head_bias is not None:  # sft_trainer.py:102-103
+            z = z + lm_head_bias.float()
         if logit_scale != 1.0:
             z = z * logit_scale
         if final_logit_softcapping is not None:

@@ -549,6 +549,8 @@ SFT_CASES = [
     dict(name="shift_labels_nitems", dtype="float32", chunk=7, shift=True, nitems=50.0, softcap=None, scale=1.0),
     dict(name="softcap_scale", dtype="float32", chunk=32, shift=False, nitems=None, softcap=4.0, scale=0.5),
     dict(name="bf16", dtype="bfloat16", chunk=16, shift=False, nitems=None, softcap=None, scale=1.0),
+    dict(name="bias", dtype="float32", chunk=16, shift=False, nitems=None, softcap=None, scale=1.0, bias=True),
+    dict(name="bias_softcap_bf16", dtype="bfloat16", chunk=8, shift=True, nitems=None, softcap=6.0, scale=0.7, bias=True),
 ]
 
 
@@ -565,6 +567,10 @@ def make_sft(chunked_ce, out_dir):
         labels[1, 7:] = -100
         labels[2, 5] = -100
         kw = dict(shift_labels=labels) if case["shift"] else dict(labels=labels)
+        bias = None
+        if case.get("bias"):  # drawn after everything else, so the earlier cases keep their arrays
+            bias = torch.randn(V, generator=g).to(dtype).requires_grad_(True)
+            kw["lm_head_bias"] = bias
         loss, correct, ent, nv = chunked_ce(hs, w, case["chunk"], num_items_in_batch=case["nitems"],
                                             logit_scale=case["scale"], final_logit_softcapping=case["softcap"], **kw)
         loss.backward()
@@ -572,6 +578,8 @@ def make_sft(chunked_ce, out_dir):
         for k, v in dict(hidden=hs, weight=w, labels=labels, out_loss=loss, out_correct=correct, out_entropy_sum=ent,
                          out_n_valid=nv, out_dhidden=hs.grad, out_dweight=w.grad).items():
             arrays[pre + k] = _np(v)
+        if bias is not None:
+            arrays[pre + "bias"], arrays[pre + "out_dbias"] = _np(bias), _np(bias.grad)
         index.append(dict(case, id=ci, shape=[B, S, H, V]))
     np.savez_compressed(os.path.join(out_dir, "sft_chunked_nll.npz"), **arrays)
     with open(os.path.join(out_dir, "sft_chunked_nll.json"), "w") as f:

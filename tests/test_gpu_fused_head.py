@@ -289,13 +289,19 @@ def test_golden_sft_chunked_nll(amd):
         labels = _t(g[c + "labels"])
         kw = dict(shift_labels=labels) if case["shift"] else dict(labels=labels)
         common = dict(num_items_in_batch=case["nitems"], logit_scale=case["scale"], final_logit_softcapping=case["softcap"])
+        has_bias = bool(case.get("bias"))
+        b = _t(g[c + "bias"]).bfloat16() if has_bias else None
         ohs, ow = hs.float().requires_grad_(True), w.float().requires_grad_(True)
-        oloss, ocorrect, oent, onv = oracle.chunked_cross_entropy_loss(ohs, ow, case["chunk"], **common, **kw)
+        ob = b.float().requires_grad_(True) if has_bias else None
+        oloss, ocorrect, oent, onv = oracle.chunked_cross_entropy_loss(ohs, ow, case["chunk"], lm_head_bias=ob, **common, **kw)
         oloss.backward()
         dhs, dw = hs.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+        db = b.to(DEV).requires_grad_(True) if has_bias else None
         dkw = {k: v.to(DEV) for k, v in kw.items()}
-        loss, correct, ent, nv = _chunked_cross_entropy_loss(dhs, dw, 256, **common, **dkw)
+        loss, correct, ent, nv = _chunked_cross_entropy_loss(dhs, dw, 256, lm_head_bias=db, **common, **dkw)
         loss.backward()
+        if has_bias:
+            assert _rel_l2(db.grad.float(), ob.grad) < 1e-2
         assert int(nv) == int(onv) == int(g[c + "out_n_valid"])
         assert abs(float(loss) - float(oloss)) <= 1e-3 * abs(float(oloss))
         assert abs(float(correct) - float(ocorrect)) <= 1.0  # a near-tie between the two largest logits may flip
@@ -305,8 +311,11 @@ def test_golden_sft_chunked_nll(amd):
             assert abs(float(loss) - float(g[c + "out_loss"])) <= 2e-2 * abs(float(g[c + "out_loss"]))
             # fp32 operands: the reference's numbers at fp32 accuracy
             fhs, fw = _t(g[c + "hidden"]).to(DEV).requires_grad_(True), _t(g[c + "weight"]).to(DEV).requires_grad_(True)
-            loss, correct, ent, nv = _chunked_cross_entropy_loss(fhs, fw, 256, **common, **dkw)
+            fb = _t(g[c + "bias"]).to(DEV).requires_grad_(True) if has_bias else None
+            loss, correct, ent, nv = _chunked_cross_entropy_loss(fhs, fw, 256, lm_head_bias=fb, **common, **dkw)
             loss.backward()
+            if has_bias:
+                torch.testing.assert_close(fb.grad.cpu(), _t(g[c + "out_dbias"]), atol=1e-6, rtol=1e-4)
             assert abs(float(loss) - float(g[c + "out_loss"])) <= 1e-5 * max(1.0, abs(float(g[c + "out_loss"])))
             assert float(correct) == float(g[c + "out_correct"])
             assert abs(float(ent) - float(g[c + "out_entropy_sum"])) <= 1e-4 * abs(float(g[c + "out_entropy_sum"]))

@@ -464,9 +464,10 @@ def test_golden_sft_chunked_nll():
         w = _t(g[c + "weight"], dtype).requires_grad_(True)
         labels = _t(g[c + "labels"])
         kw = dict(shift_labels=labels) if case["shift"] else dict(labels=labels)
+        bias = _t(g[c + "bias"], dtype).requires_grad_(True) if case.get("bias") else None
         loss, correct, ent, nv = oracle.chunked_cross_entropy_loss(
             hs, w, case["chunk"], num_items_in_batch=case["nitems"], logit_scale=case["scale"],
-            final_logit_softcapping=case["softcap"], **kw)
+            final_logit_softcapping=case["softcap"], lm_head_bias=bias, **kw)
         loss.backward()
         tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
         torch.testing.assert_close(loss.detach().float(), _t(g[c + "out_loss"]).float(), **tol)
@@ -474,6 +475,9 @@ def test_golden_sft_chunked_nll():
         torch.testing.assert_close(ent.detach(), _t(g[c + "out_entropy_sum"]), rtol=1e-5, atol=1e-4)
         torch.testing.assert_close(hs.grad.float(), _t(g[c + "out_dhidden"]), **tol)
         torch.testing.assert_close(w.grad.float(), _t(g[c + "out_dweight"]), **tol)
+        if bias is not None:
+            torch.testing.assert_close(bias.grad.float(), _t(g[c + "out_dbias"]), **tol)
+    assert sum(bool(c.get("bias")) for c in cases) >= 2
     # library routine: mean cross-entropy over the valid positions
     torch.manual_seed(9)
     hs, w = torch.randn(2, 7, 16), torch.randn(40, 16)
