@@ -206,6 +206,47 @@ def test_masked_rows_and_scatter(amd):
     assert torch.count_nonzero(lp_e) == 0
 
 
+def test_patch_chunked_lm_head_with_router_logits(amd):
+    """The patched forward on a stand-in MoE model: log-probs as the unpatched pieces give them, and the
+    auxiliary loss equal to transformers' load-balancing loss of the backbone's router logits."""
+    from types import SimpleNamespace
+
+    from transformers.models.mixtral.modeling_mixtral import load_balancing_loss_func
+
+    g = torch.Generator().manual_seed(6)
+    B, S, H, V, E = 2, 9, 32, 120, 4
+    hs = torch.randn(B, S, H, generator=g).bfloat16().to(DEV)
+    router = tuple(torch.randn(B * S, E, generator=g).to(DEV) for _ in range(2))
+    seen = {}
+
+    class Backbone(torch.nn.Module):
+        def forward(self, input_ids=None, attention_mask=None, use_cache=False, **kw):
+            seen.update(kw)
+            return SimpleNamespace(last_hidden_state=hs, router_logits=router)
+
+    class Model(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.model = Backbone()
+            self.lm_head = torch.nn.Linear(H, V, bias=False, device=DEV, dtype=torch.bfloat16)
+            self.config = SimpleNamespace(num_experts=E, num_experts_per_tok=2, logit_scale=0.5)
+
+    model = Model()
+    amd.patch_chunked_lm_head(model, chunk_size=64, temperature=0.9, output_router_logits=True)
+    ids = torch.randint(0, V, (B, S), generator=g).to(DEV)
+    am = torch.ones(B, S, dtype=torch.long, device=DEV)
+    am[1, 6:] = 0
+    cm = am.clone()
+    cm[:, :3] = 0
+    out = model(input_ids=ids, attention_mask=am, labels=ids, completion_mask=cm)
+    assert seen.get("output_router_logits") is True
+    want_aux = load_balancing_loss_func(router, E, 2, am)
+    torch.testing.assert_close(out["aux_loss"], want_aux)
+    lp, ent = amd.chunked_logprobs_from_hidden(hs, model.lm_head.weight, ids, cm, 0.9, 64, None, 0.5)
+    assert torch.equal(out["log_probs"], lp) and torch.equal(out["entropy"], ent)
+    assert out["log_probs"].shape == (B, S - 1)
+
+
 def test_golden_chunked_logprob_fp32(amd):
     """fp32 operands (the dtype of the reference's own unit test, tests/test_utils.py:1161-1232) at its tolerance:
     forward and backward within 1e-5 of what the reference operator wrote."""

@@ -290,21 +290,30 @@ def patch_chunked_lm_head(model: torch.nn.Module, chunk_size: int, temperature: 
                           output_router_logits: bool = False) -> None:
     """Replaces `model.forward` by one that runs the backbone, then the fused head, and returns
     `{"log_probs" [B, S-1], "entropy" [B, S-1], "aux_loss"}` (reference: utils.py:1427-1517).
-    The MoE load-balancing auxiliary loss of the reference is not reproduced here."""
+    With `output_router_logits` the backbone is asked for its router logits and `aux_loss` is the transformers
+    load-balancing loss of them (the function every MoE family shares), as in the reference (:1484-1508)."""
     import types
 
-    if output_router_logits:
-        raise NotImplementedError("patch_chunked_lm_head(output_router_logits=True) is not implemented by trl_amd")
     final_logit_softcapping = getattr(model.config, "final_logit_softcapping", None)
 
     def _chunked_forward(self, input_ids=None, attention_mask=None, labels=None, completion_mask=None,
                          use_cache=False, **kwargs):
         assert labels is not None, "requires labels to not be None for logprob computation"
-        outputs = self.model(input_ids=input_ids, attention_mask=attention_mask, use_cache=use_cache, **kwargs)
+        decoder_kwargs = {"output_router_logits": True} if output_router_logits else {}
+        outputs = self.model(input_ids=input_ids, attention_mask=attention_mask, use_cache=use_cache, **decoder_kwargs,
+                             **kwargs)
         logit_scale = getattr(self.config, "logit_scale", 1.0)
         log_probs, entropy = chunked_logprobs_from_hidden(
             outputs.last_hidden_state, self.lm_head.weight, labels, completion_mask, temperature, chunk_size,
             final_logit_softcapping, logit_scale)
-        return {"log_probs": log_probs, "entropy": entropy, "aux_loss": None}
+        aux_loss = None
+        if output_router_logits:
+            from transformers.models.mixtral.modeling_mixtral import load_balancing_loss_func
+
+            # the expert counts live on the config (on the module itself for some families / older transformers)
+            num_experts = getattr(self.config, "num_experts", None) or getattr(self, "num_experts")
+            top_k = getattr(self.config, "num_experts_per_tok", None) or getattr(self, "num_experts_per_tok")
+            aux_loss = load_balancing_loss_func(outputs.router_logits, num_experts, top_k, attention_mask)
+        return {"log_probs": log_probs, "entropy": entropy, "aux_loss": aux_loss}
 
     model.forward = types.MethodType(_chunked_forward, model)
