@@ -923,10 +923,10 @@ def fused_linear_grpo_loss(hidden, weight, selected_token_ids, loss_mask, advant
 
 
 def fused_linear_dpo_loss(weight, hidden, target, ref_hidden, ref_weight, beta, ignore_index=-100, bias=None,
-                          ref_bias=None):
-    """What `_compute_loss_liger` expects of `self.liger_loss` (dpo_trainer.py:1287-1301) for the sigmoid loss:
+                          ref_bias=None, loss_type="sigmoid"):
+    """What `_compute_loss_liger` expects of `self.liger_loss` (dpo_trainer.py:1287-1301):
     summed log-probs of the non-ignored targets (as dpo_trainer.py:1347-1350), reference ones without grad,
-    `dpo_sigmoid_loss` above.  Returns `(loss, (chosen_logps, rejected_logps, chosen_logits_mean,
+    `dpo_sigmoid_loss` above (other loss types: `dpo_compute_loss` above on the same logits).  Returns `(loss, (chosen_logps, rejected_logps, chosen_logits_mean,
     rejected_logits_mean, nll_loss, chosen_rewards, rejected_rewards))`; the logits means run over all
     positions and the whole vocabulary."""
     b, t, h = hidden.shape
@@ -945,7 +945,14 @@ def fused_linear_dpo_loss(weight, hidden, target, ref_hidden, ref_weight, beta, 
     with torch.no_grad():
         ref_seq, _ = seq_logps(ref_hidden, ref_weight, ref_bias)
     pairs = b // 2
-    loss, _ = dpo_sigmoid_loss(seq, ref_seq[:pairs], ref_seq[pairs:], beta)
+    if loss_type == "sigmoid":
+        loss, _ = dpo_sigmoid_loss(seq, ref_seq[:pairs], ref_seq[pairs:], beta)
+    else:  # undo the shift `dpo_compute_loss` applies: a dummy last position, a dummy first label
+        pad_l = torch.zeros(b, 1, logits.shape[-1], dtype=logits.dtype)
+        pad_i = torch.zeros(b, 1, dtype=labels.dtype)
+        loss, _ = dpo_compute_loss(torch.cat([logits, pad_l], 1), torch.cat([pad_i, labels], 1),
+                                   torch.cat([pad_i, keep.to(labels.dtype)], 1), ref_seq[:pairs], ref_seq[pairs:], beta,
+                                   loss_types=(loss_type,))
     rewards = beta * (seq.detach() - ref_seq)
     metrics = (seq.detach()[:pairs], seq.detach()[pairs:], logits.detach()[:pairs].mean(), logits.detach()[pairs:].mean(),
                torch.zeros(()), rewards[:pairs], rewards[pairs:])

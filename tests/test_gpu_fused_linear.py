@@ -76,7 +76,8 @@ def test_fused_linear_grpo_loss(amd, loss_type, level, beta):
            advantages=adv.to(DEV), bias=torch.zeros(V + 1, device=DEV))
 
 
-def test_fused_linear_dpo_loss(amd):
+@pytest.mark.parametrize("loss_type", ["sigmoid", "apo_zero", "apo_down", "sppo_hard", "nca_pair"])
+def test_fused_linear_dpo_loss(amd, loss_type):
     P, T, H, V = 4, 20, 64, 389
     g, hidden, weight, ids, mask = _problem(32, 2 * P, T, H, V)
     ref_hidden = (hidden.float() + 0.1 * torch.randn(2 * P, T, H, generator=g)).bfloat16()
@@ -86,10 +87,11 @@ def test_fused_linear_dpo_loss(amd):
     beta = 0.1
     oh = hidden.float().requires_grad_(True)
     ow = weight.float().requires_grad_(True)
-    oloss, om = oracle.fused_linear_dpo_loss(ow, oh, target, ref_hidden.float(), ref_weight.float(), beta)
+    oloss, om = oracle.fused_linear_dpo_loss(ow, oh, target, ref_hidden.float(), ref_weight.float(), beta,
+                                             loss_type=loss_type)
     oloss.backward()
 
-    op = amd.FusedLinearDPOLoss(beta=beta, loss_type="sigmoid")
+    op = amd.FusedLinearDPOLoss(beta=beta, loss_type=loss_type)
     dh = hidden.to(DEV).requires_grad_(True)
     dw = weight.to(DEV).requires_grad_(True)
     loss, m = op(dw, dh, target.to(DEV), None, ref_hidden.to(DEV), ref_weight.to(DEV), None)

@@ -12,6 +12,7 @@ arithmetic is the reference's own `_compute_loss` (same kernels as `GRPOLossMixi
 from __future__ import annotations
 
 import torch
+import torch.nn.functional as F
 from torch import Tensor
 
 from .. import ops
@@ -108,14 +109,19 @@ class FusedLinearDPOLoss(torch.nn.Module):
     bias=None, ref_input=None, ref_weight=None, ref_bias=None)`; rows `[0, P)` are the chosen, `[P, 2P)`
     the rejected sequences; without `ref_weight` the reference model shares `lin_weight` and `bias`.  `metrics = (chosen_logps [P], rejected_logps [P], chosen_logits_mean,
     rejected_logits_mean, nll_loss, chosen_rewards [P], rejected_rewards [P])`, the order
-    `_compute_loss_liger` unpacks (dpo_trainer.py:1293-1301).  Sigmoid loss only; the logits means are
-    taken over every position and the whole vocabulary, computed as `hidden . sum_v W[v]` (no logits)."""
+    `_compute_loss_liger` unpacks (dpo_trainer.py:1293-1301).  Loss types: `sigmoid` (one fused loss kernel) and
+    the other pair losses of the third-party operator, `apo_zero`, `apo_down`, `sppo_hard`, `nca_pair`, with the
+    reference's own formulas (dpo_trainer.py:1396-1519).  The logits means are taken over every position and the
+    whole vocabulary, computed as `hidden . sum_v W[v]` (no logits)."""
+
+    LOSS_TYPES = ("sigmoid", "apo_zero", "apo_down", "sppo_hard", "nca_pair")
 
     def __init__(self, ignore_index: int = -100, beta: float = 0.1, loss_type: str = "sigmoid", use_ref_model: bool = True,
                  chunk_size: int = 32768):
         super().__init__()
-        if loss_type != "sigmoid":
-            raise NotImplementedError(f"loss_type={loss_type!r}: only the sigmoid DPO loss is fused")
+        if loss_type not in self.LOSS_TYPES:
+            raise NotImplementedError(f"loss_type={loss_type!r}: the fused-linear DPO loss has {self.LOSS_TYPES}")
+        self.loss_type = loss_type
         self.ignore_index = int(ignore_index)
         self.beta = float(beta)
         self.use_ref_model = bool(use_ref_model)
@@ -138,7 +144,21 @@ class FusedLinearDPOLoss(torch.nn.Module):
                 ref_seq = (ref_logps * keep).sum(-1)
         else:
             ref_seq = torch.zeros(2 * pairs, dtype=torch.float32, device=_input.device)
-        loss, seq, _, _ = ops.dpo_loss_op(logps, keep, ref_seq[:pairs], ref_seq[pairs:], self.beta)
+        if self.loss_type == "sigmoid":
+            loss, seq, _, _ = ops.dpo_loss_op(logps, keep, ref_seq[:pairs], ref_seq[pairs:], self.beta)
+        else:  # [P]-sized fp32 arithmetic on the sequence log-ratios
+            seq = (logps * keep).sum(-1)
+            c_lr, r_lr = seq[:pairs] - ref_seq[:pairs], seq[pairs:] - ref_seq[pairs:]
+            b = self.beta
+            if self.loss_type == "apo_zero":
+                per_pair = 1 - torch.sigmoid(b * c_lr) + torch.sigmoid(b * r_lr)
+            elif self.loss_type == "apo_down":
+                per_pair = torch.sigmoid(b * c_lr) + 1 - torch.sigmoid(b * (c_lr - r_lr))
+            elif self.loss_type == "sppo_hard":
+                per_pair = (c_lr - 0.5 / b) ** 2 + (r_lr + 0.5 / b) ** 2
+            else:  # nca_pair
+                per_pair = (-F.logsigmoid(b * c_lr) - 0.5 * F.logsigmoid(-b * c_lr) - 0.5 * F.logsigmoid(-b * r_lr))
+            loss = per_pair.mean()
         with torch.no_grad():
             seq = seq.detach()
             wsum = lin_weight.float().sum(0)
