@@ -30,7 +30,7 @@ Pinning status (what checks each function against something other than itself):
                               autograd of it (reference test tests/test_utils.py:1161-1232)
   chunked_cross_entropy_loss: golden vectors from the reference's `_chunked_cross_entropy_loss`,
                               `F.cross_entropy` library routine
-  fused_linear_grpo_loss / fused_linear_dpo_loss : PARITY UNPINNED against the third-party operators
+  fused_linear_grpo_loss / fused_linear_dpo_loss / fused_linear_kto_loss : PARITY UNPINNED against the third-party operators
                               they stand in for (liger-kernel >=0.8.0,<0.8.1 is not importable here and no
                               reference test holds their numbers); they compose pinned pieces only -- the naive
                               head routine + `grpo_loss` / `dpo_sigmoid_loss` -- in the metric order the
@@ -75,6 +75,7 @@ __all__ = [
     "chunked_cross_entropy_loss",
     "fused_linear_grpo_loss",
     "fused_linear_dpo_loss",
+    "fused_linear_kto_loss",
 ]
 
 
@@ -957,3 +958,36 @@ def fused_linear_dpo_loss(weight, hidden, target, ref_hidden, ref_weight, beta, 
     metrics = (seq.detach()[:pairs], seq.detach()[pairs:], logits.detach()[:pairs].mean(), logits.detach()[pairs:].mean(),
                torch.zeros(()), rewards[:pairs], rewards[pairs:])
     return loss, metrics
+
+
+def fused_linear_kto_loss(weight, hidden, target, preference_labels, ref_hidden, ref_weight, beta, kl=None,
+                          ignore_index=-100, bias=None, ref_bias=None):
+    """What `KTOTrainer._compute_loss_liger` expects of `self.liger_loss` (kto_trainer.py:1415-1435), stated with the
+    reference's own `kto` arithmetic (`kto_compute_loss` above, unit class weights) on naive logits.  Returns
+    `(loss, (chosen_logps_sum, rejected_logps_sum, chosen_logits_sum, rejected_logits_sum, chosen_rewards_sum,
+    rejected_rewards_sum))`; a sequence's logits entry is its mean logit over positions and vocabulary."""
+    b, t, h = hidden.shape
+    keep = target != ignore_index
+    labels = torch.where(keep, target, torch.zeros_like(target))
+
+    def logits_of(hs, w, bi):
+        z = hs.reshape(b * t, h) @ w.t()
+        return (z if bi is None else z + bi).float().view(b, t, -1)
+
+    logits = logits_of(hidden, weight, bias)
+    pad_l = torch.zeros(b, 1, logits.shape[-1])
+    pad_i = torch.zeros(b, 1, dtype=labels.dtype)
+    ids, cm = torch.cat([pad_i, labels], 1), torch.cat([pad_i, keep.to(labels.dtype)], 1)
+    with torch.no_grad():
+        ref_seq = kto_sequence_logps(torch.cat([logits_of(ref_hidden, ref_weight, ref_bias), pad_l], 1), ids, cm)
+    zero = torch.zeros(b)
+    kl_pair = (None, None) if kl is None else (zero + kl, zero)  # mean(kl_logps - ref_kl_logps) = kl
+    loss, _ = kto_compute_loss(torch.cat([logits, pad_l], 1), ids, cm, preference_labels, ref_seq, *kl_pair, beta=beta)
+    with torch.no_grad():
+        seq = kto_sequence_logps(torch.cat([logits, pad_l], 1), ids, cm)
+        c = torch.as_tensor(preference_labels, dtype=torch.bool).float()
+        lm = logits.mean(dim=(1, 2))
+        rew = beta * (seq - ref_seq)
+        sums = ((seq * c).sum(), (seq * (1 - c)).sum(), (lm * c).sum(), (lm * (1 - c)).sum(), (rew * c).sum(),
+                (rew * (1 - c)).sum())
+    return loss, sums

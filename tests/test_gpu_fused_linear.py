@@ -148,3 +148,30 @@ def test_fused_linear_losses_with_lm_head_bias(amd):
         assert abs(float(m[i]) - float(om[i])) <= 1e-3
     for got, want in ((dh, oh), (dw, ow), (db, ob)):
         assert _rel_l2(got.grad.float(), want.grad) < 1e-2
+
+
+@pytest.mark.parametrize("kl", [None, 0.7])
+def test_fused_linear_kto_loss(amd, kl):
+    B, T, H, V = 6, 18, 64, 389
+    g, hidden, weight, ids, mask = _problem(34, B, T, H, V)
+    ref_hidden = (hidden.float() + 0.1 * torch.randn(B, T, H, generator=g)).bfloat16()
+    ref_weight = (weight.float() + 0.02 * torch.randn(V, H, generator=g)).bfloat16()
+    bias = torch.randn(V, generator=g).bfloat16()
+    target = torch.where(mask == 1, ids, torch.full_like(ids, -100))
+    pref = torch.tensor([1, 0, 1, 1, 0, 0], dtype=torch.bool)
+    oh, ow, ob = (x.float().requires_grad_(True) for x in (hidden, weight, bias))
+    oloss, osums = oracle.fused_linear_kto_loss(ow, oh, target, pref, ref_hidden.float(), ref_weight.float(), 0.2, kl,
+                                                bias=ob, ref_bias=bias.float())
+    oloss.backward()
+    dh, dw, db = (x.to(DEV).requires_grad_(True) for x in (hidden, weight, bias))
+    op = amd.FusedLinearKTOLoss(beta=0.2, use_ref_model=True)
+    loss, sums = op(_input=dh, lin_weight=dw, target=target.to(DEV), bias=db, preference_labels=pref.to(DEV),
+                    ref_input=ref_hidden.to(DEV), ref_weight=ref_weight.to(DEV), ref_bias=bias.to(DEV),
+                    kl=None if kl is None else torch.tensor([kl], device=DEV))
+    loss.backward()
+    assert abs(float(loss) - float(oloss)) <= 1e-3 * max(1.0, abs(float(oloss)))
+    assert len(sums) == 6
+    for got, want in zip(sums, osums):
+        assert abs(float(got) - float(want)) <= 2e-3 * max(1.0, abs(float(want))), (float(got), float(want))
+    for got, want in ((dh, oh), (dw, ow), (db, ob)):
+        assert _rel_l2(got.grad.float(), want.grad) < 1e-2

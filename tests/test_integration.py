@@ -63,6 +63,10 @@ def test_patch_trl_binds_the_fused_linear_operators():
                 vespo_k_neg=3.0, vespo_lambda_neg=2.0)
             assert op.beta == 0.04
             ref_dpo.LigerFusedLinearDPOLoss(beta=0.1, loss_type="sigmoid")
+            import trl.trainer.kto_trainer as ref_kto
+
+            assert ref_kto.LigerFusedLinearKTOLoss is trl_amd.FusedLinearKTOLoss
+            ref_kto.LigerFusedLinearKTOLoss(beta=0.1, use_ref_model=True)  # kto_trainer.py:978
         finally:
             integration.unpatch_trl()
         assert hasattr(ref_grpo, "LigerFusedLinearGRPOLoss") == had

@@ -103,6 +103,15 @@ def patch_trl(grpo: bool = True, liger: bool = False, dpo: bool = False, rloo: b
         _set(ref_grpo, "LigerFusedLinearGRPOLoss", FusedLinearGRPOLoss)
         _set(ref_grpo, "is_liger_kernel_available", lambda *a, **k: True)
         _set(ref_dpo, "LigerFusedLinearDPOLoss", FusedLinearDPOLoss)
+        try:
+            import trl.trainer.kto_trainer as ref_kto
+
+            from .trainer.fused_linear import FusedLinearKTOLoss
+
+            _set(ref_kto, "LigerFusedLinearKTOLoss", FusedLinearKTOLoss)
+            _set(ref_kto, "is_liger_kernel_available", lambda *a, **k: True)
+        except ImportError:
+            pass
         _set(ref_dpo, "is_liger_kernel_available", lambda *a, **k: True)
         count += 4
     return count

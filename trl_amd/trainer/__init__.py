@@ -7,4 +7,4 @@ from .rloo_trainer import RLOOLossMixin, rloo_advantages, rloo_loss
 from .utils import (_ChunkedLogProbFunction, chunked_logprobs_from_hidden, entropy_from_logits, logps_and_entropies,
                     nanmax, nanmin, nanstd, patch_chunked_lm_head, selective_log_softmax)
 from .sft_trainer import _chunked_cross_entropy_loss
-from .fused_linear import FusedLinearDPOLoss, FusedLinearGRPOLoss
+from .fused_linear import FusedLinearDPOLoss, FusedLinearGRPOLoss, FusedLinearKTOLoss

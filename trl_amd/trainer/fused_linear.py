@@ -1,7 +1,8 @@
 """Fused-linear losses: lm_head + log-prob + policy loss from the last hidden states, with the call
 signatures of the operators the reference plugs in behind `use_liger_kernel`
 (`LigerFusedLinearGRPOLoss`, trl/trainer/grpo_trainer.py:1027-1044, 2885-2907;
-`LigerFusedLinearDPOLoss`, trl/trainer/dpo_trainer.py:834, 1287-1327).
+`LigerFusedLinearDPOLoss`, trl/trainer/dpo_trainer.py:834, 1287-1327;
+`LigerFusedLinearKTOLoss`, trl/trainer/kto_trainer.py:978, 1415-1435).
 
 Those operators live in the third-party `liger-kernel` package (pinned `>=0.8.0,<0.8.1` by the
 reference, not importable here), so what is mirrored is the call contract the reference relies on:
@@ -19,7 +20,7 @@ from .. import ops
 from .grpo_trainer import _METRIC_INDEX, grpo_loss
 from .utils import _ChunkedLogProbFunction
 
-__all__ = ["FusedLinearGRPOLoss", "FusedLinearDPOLoss"]
+__all__ = ["FusedLinearGRPOLoss", "FusedLinearDPOLoss", "FusedLinearKTOLoss"]
 
 
 def _head_logps(hidden: Tensor, weight: Tensor, targets: Tensor, keep: Tensor, temperature: float,
@@ -170,3 +171,57 @@ class FusedLinearDPOLoss(torch.nn.Module):
         metrics = (seq[:pairs], seq[pairs:], logits_mean[:pairs].mean(), logits_mean[pairs:].mean(), nll,
                    rewards[:pairs], rewards[pairs:])
         return loss, metrics
+
+
+class FusedLinearKTOLoss(torch.nn.Module):
+    """`loss, sums = op(_input [B, T, H], lin_weight [V, H], target [B, T] (-100 = ignored), bias=None,
+    preference_labels [B] (true = desirable), ref_input=None, ref_weight=None, ref_bias=None, kl=None)` with
+    `sums = (chosen_logps_sum, rejected_logps_sum, chosen_logits_sum, rejected_logits_sum, chosen_rewards_sum,
+    rejected_rewards_sum)`, the order `_compute_loss_liger` unpacks (kto_trainer.py:1415-1424); the caller divides
+    each by the number of desirable / undesirable examples.  The loss is the reference's `kto` loss with unit
+    class weights (kto_trainer.py:1558-1560, 1576-1577, 1586-1589, 1655); a sequence's "logits" entry is its mean
+    logit over positions and vocabulary."""
+
+    def __init__(self, ignore_index: int = -100, beta: float = 0.1, use_ref_model: bool = True, chunk_size: int = 32768):
+        super().__init__()
+        self.ignore_index = int(ignore_index)
+        self.beta = float(beta)
+        self.use_ref_model = bool(use_ref_model)
+        self.chunk_size = int(chunk_size)
+
+    def forward(self, _input: Tensor, lin_weight: Tensor, target: Tensor, bias: Tensor | None = None,
+                preference_labels: Tensor | None = None, ref_input: Tensor | None = None,
+                ref_weight: Tensor | None = None, ref_bias: Tensor | None = None, kl: Tensor | None = None):
+        if _input.dim() != 3:
+            raise ValueError("_input must be [B, T, H] hidden states")
+        if preference_labels is None or len(preference_labels) != _input.shape[0]:
+            raise ValueError("preference_labels must hold one entry per sequence")
+        dev = _input.device
+        keep = target != self.ignore_index
+        labels = torch.where(keep, target, torch.zeros_like(target))
+        seq = (_head_logps(_input, lin_weight, labels, keep, 1.0, self.chunk_size, bias) * keep).sum(-1)
+        if self.use_ref_model:
+            if ref_input is None:
+                raise ValueError("ref_input is required when use_ref_model=True")
+            with torch.no_grad():
+                ref_seq = (_head_logps(ref_input, lin_weight if ref_weight is None else ref_weight, labels, keep, 1.0,
+                                       self.chunk_size, bias if ref_weight is None else ref_bias) * keep).sum(-1)
+        else:
+            ref_seq = torch.zeros_like(seq)
+        chosen = torch.as_tensor(preference_labels, dtype=torch.bool, device=dev)
+        kl_term = torch.zeros((), device=dev) if kl is None else kl.to(dev).float().reshape(-1)[0].detach()
+        lr = seq - ref_seq
+        per_example = torch.where(chosen, 1 - torch.sigmoid(self.beta * (lr - kl_term)),
+                                  1 - torch.sigmoid(self.beta * (kl_term - lr)))
+        loss = per_example.mean()
+        with torch.no_grad():
+            c = chosen.to(torch.float32)
+            wsum = lin_weight.float().sum(0)
+            logits_mean = (_input.float() @ wsum).mean(dim=1) / lin_weight.shape[0]
+            if bias is not None:
+                logits_mean = logits_mean + bias.float().mean()
+            rewards = self.beta * lr.detach()
+            s = seq.detach()
+            sums = ((s * c).sum(), (s * (1 - c)).sum(), (logits_mean * c).sum(), (logits_mean * (1 - c)).sum(),
+                    (rewards * c).sum(), (rewards * (1 - c)).sum())
+        return loss, sums
