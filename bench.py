@@ -252,6 +252,10 @@ def bench_head(args, w):
         del out
         fwd_ms = time_op(lambda: ops.fused_head_fwd(*fwd_args, None, stash))
         bwd_ms = time_op(lambda: ops.fused_head_bwd(*fwd_args, log_z, gl, HEAD_CHUNK, None, saved))
+        # the step's backward: the loss gives the tokens outside the completion mask an upstream gradient of exactly
+        # zero, and those tokens are dropped before the two products (their dz rows are zero)
+        g_step = gl * mask.reshape(-1).float()
+        bwd_step_ms = time_op(lambda: ops.head_backward(*fwd_args, log_z, g_step, HEAD_CHUNK, None, saved))
         kernels = {}
         if stash:  # the reference's scheme (recompute the logits in the backward) on the same kernels, for comparison
             del saved
@@ -272,6 +276,7 @@ def bench_head(args, w):
         "config": {"workload": args.workload, "description": w["desc"], "tokens": N, "hidden": H, "vocab": V,
                    "backward_chunk_rows": HEAD_CHUNK,
                    "backward_logits": "stashed by the forward (fp32 [V, N])" if stash else "recomputed per chunk",
+                   "tokens_with_gradient": int(mask.sum()),
                    "loss_type": args.loss_type, "loss": float(loss.detach())},
         # the dominant kernel: the forward sweep (2*N*H*V flop per launch; the event-timed interval also holds its
         # two sub-0.1 ms helper kernels)
@@ -283,7 +288,10 @@ def bench_head(args, w):
         "kernels": dict(kernels, **{
             "fused_head_fwd": {"avg_ms": fwd_ms, "TFLOPs": fwd_tf, "frac": fwd_tf / MFMA_BF16_PEAK_TFLOPS},
             "fused_head_bwd": {"avg_ms": bwd_ms, "TFLOPs": bwd_tf, "frac": bwd_tf / MFMA_BF16_PEAK_TFLOPS,
-                               "products": 2 if stash else 3}}),
+                               "products": 2 if stash else 3, "note": "every token with an upstream gradient"},
+            "fused_head_bwd_step": {"avg_ms": bwd_step_ms, "tokens": int(mask.sum()),
+                                    "note": "as in the step: tokens whose upstream gradient is zero are dropped"},
+            "step_if_every_token_had_a_gradient_ms": ms_per_step - bwd_step_ms + bwd_ms}),
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_head(w),
     }
     print(json.dumps(result))

@@ -255,6 +255,9 @@ int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, const int64_
  * The vocabulary is processed in chunks of `chunk_size` rows (rounded up to 256); dz exists only
  * for one chunk at a time, in bf16/fp16, inside the workspace.
  * d_out_dbias (optional, fp32 [vocab]): sum over tokens of dz, the gradient of d_bias.
+ * d_stash_cols (optional, int32 [n_tokens]): the stash column of each token, for a caller that dropped tokens
+ * since the forward (those without an upstream gradient contribute nothing to either product); values in
+ * [0, stash_ld).
  */
 size_t trlk_fused_head_bwd_workspace_bytes(int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t chunk_size);
 
@@ -262,8 +265,9 @@ int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, const int64_
                         int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                         int64_t weight_stride, float temperature, float final_logit_softcapping, float logit_scale,
                         const float* d_bias, const float* d_log_z, const float* d_g_logp, int64_t chunk_size,
-                        const float* d_stash, int64_t stash_ld, void* d_out_dhidden, void* d_out_dweight,
-                        float* d_out_dbias, void* d_workspace, size_t workspace_bytes, trlk_stream_t stream);
+                        const float* d_stash, int64_t stash_ld, const int32_t* d_stash_cols, void* d_out_dhidden,
+                        void* d_out_dweight, float* d_out_dbias, void* d_workspace, size_t workspace_bytes,
+                        trlk_stream_t stream);
 
 #ifdef __cplusplus
 }

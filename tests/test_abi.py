@@ -102,9 +102,11 @@ def test_host_side_argument_validation():
     ld = ctypes.c_int64(0)
     assert lib.trlk_fused_head_stash_bytes(300, 1000, ctypes.addressof(ld)) == 1024 * 512 * 4 and ld.value == 512
     assert lib.trlk_fused_head_bwd(fake16, fake16, fake, _lib.BF16, 300, 1000, 64, 64, 64, 1.0, 0.0, 1.0, None, fake, fake,
-                                   256, fake16, 256, fake16, fake16, None, fake16, 1 << 40, None) == -4
+                                   256, fake16, 256, None, fake16, fake16, None, fake16, 1 << 40, None) == -4
     assert lib.trlk_fused_head_bwd(fake16, fake16, fake, _lib.BF16, 300, 1000, 64, 64, 64, 1.0, 0.0, 1.0, None, fake, fake,
-                                   0, None, 0, fake16, fake16, None, fake16, 1 << 40, None) == -5  # chunk_size
+                                   0, None, 0, None, fake16, fake16, None, fake16, 1 << 40, None) == -5  # chunk_size
+    assert lib.trlk_fused_head_bwd(fake16, fake16, fake, _lib.BF16, 300, 1000, 64, 64, 64, 1.0, 0.0, 1.0, None, fake, fake,
+                                   256, None, 0, fake16, fake16, fake16, None, fake16, 1 << 40, None) == -1  # columns, no stash
     # an empty problem is a successful no-op
     assert lib.trlk_logp_entropy_fwd(None, _lib.F32, 0, 4, 8, 32, 8, None, 1, 1.0, None, None, None, None, None, None, None) == 0
     assert _lib.last_error() == ""

@@ -157,20 +157,30 @@ def test_backward_from_stashed_products_equals_recompute(amd, monkeypatch, n, h,
     b = (2.0 * torch.randn(v, generator=g)).bfloat16().to(DEV) if bias else None
     labels = torch.randint(0, v, (n,), generator=g).to(DEV)
     gout = torch.randn(n, generator=g).to(DEV)
-    gout[::7] = 0.0  # rows without an upstream gradient
+    gout[torch.rand(n, generator=g).to(DEV) < 0.45] = 0.0  # rows without an upstream gradient (masked positions)
     out = {}
     for mode, gib in (("stash", "1"), ("recompute", "0")):
-        monkeypatch.setenv("TRL_AMD_HEAD_STASH_GIB", gib)
-        assert amd.ops.head_stash_fits(n, v) == (mode == "stash")
-        hh, ww = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
-        bb = b.clone().requires_grad_(True) if bias else None
-        lp, ent = amd._ChunkedLogProbFunction.apply(hh, ww, labels, 0.9, chunk, softcap, scale, bb)
-        (lp * gout).sum().backward()
-        out[mode] = (lp.detach(), ent, hh.grad, ww.grad, bb.grad if bias else None)
-    assert torch.equal(out["stash"][0], out["recompute"][0]) and torch.equal(out["stash"][1], out["recompute"][1])
-    for got, want in zip(out["stash"][2:], out["recompute"][2:]):
-        if want is not None:
-            assert _rel_l2(got.float(), want.float()) < 2e-3, _rel_l2(got.float(), want.float())
+        for drop in ("1", "0"):  # with and without dropping the zero-gradient tokens before the backward
+            monkeypatch.setenv("TRL_AMD_HEAD_STASH_GIB", gib)
+            monkeypatch.setenv("TRL_AMD_HEAD_DROP_ZERO_GRAD", drop)
+            assert amd.ops.head_stash_fits(n, v) == (mode == "stash")
+            hh, ww = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+            bb = b.clone().requires_grad_(True) if bias else None
+            lp, ent = amd._ChunkedLogProbFunction.apply(hh, ww, labels, 0.9, chunk, softcap, scale, bb)
+            (lp * gout).sum().backward()
+            out[mode, drop] = (lp.detach(), ent, hh.grad, ww.grad, bb.grad if bias else None)
+    want_all = out["recompute", "0"]
+    for key, got_all in out.items():
+        assert torch.equal(got_all[0], want_all[0]) and torch.equal(got_all[1], want_all[1]), key
+        assert torch.count_nonzero(got_all[2][gout == 0]) == 0, key  # no gradient for tokens without an upstream one
+        for got, want in zip(got_all[2:], want_all[2:]):
+            if want is not None:
+                assert _rel_l2(got.float(), want.float()) < 2e-3, (key, _rel_l2(got.float(), want.float()))
+    monkeypatch.setenv("TRL_AMD_HEAD_DROP_ZERO_GRAD", "1")
+    hh, ww = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+    lp, _ = amd._ChunkedLogProbFunction.apply(hh, ww, labels, 0.9, chunk, softcap, scale)
+    (lp * 0.0).sum().backward()  # no token has a gradient
+    assert torch.count_nonzero(hh.grad) == 0 and torch.count_nonzero(ww.grad) == 0
     # the op rejects a stash of the wrong shape
     lp, ent, log_z, _, saved = amd.ops.fused_head_fwd(hidden, weight, labels, 0.9, 0.0, 1.0, None, True)
     assert saved.shape == ((v + 255) // 256 * 256, (n + 255) // 256 * 256)

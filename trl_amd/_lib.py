@@ -65,7 +65,7 @@ SIGNATURES = {
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64, c_float, c_float,
          c_float, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
-         c_size_t, c_void_p],
+         c_void_p, c_size_t, c_void_p],
     ),
     "trlk_fused_head_stash_bytes": (c_size_t, [c_int64, c_int64, c_void_p]),
     "trlk_rloo_loss": (

@@ -509,6 +509,7 @@ struct HeadArgs {
     int c0, c1;          // vocabulary rows of this chunk
     float* stash;        // forward: raw products y[v][n], [V padded to BM, ld_stash] (vocabulary-major), or null
     const float* stash_in;  // backward: the same buffer, or null (recompute)
+    const int32_t* stash_cols;  // backward: stash column of token n (tokens were compacted since the forward), or null
     int64_t ld_stash;
     uint16_t* dz;        // [N, ldz]   (columns = chunk-local vocabulary index)
     uint16_t* dzT;       // [chunk rows padded, ldzt]
@@ -860,10 +861,12 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
     const bool plain = a.softcap <= 0.f && a.bias == nullptr;
     float g[4], lzc[4];
     int64_t tg[4];
+    int col[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int tok = n0 + lane * 4 + j;
         const bool ok = tok < a.N;
+        col[j] = (ok && a.stash_cols != nullptr) ? a.stash_cols[tok] : -1;
         g[j] = ok ? a.g[tok] : 0.f;
         lzc[j] = ok ? a.log_z[tok] * kLog2e : INFINITY;
         tg[j] = ok ? a.targets[tok] - a.c0 : -1;  // chunk-local target row
@@ -875,8 +878,14 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int row = r0 + rl + h;
-            const f32x4 y4 = __builtin_nontemporal_load(
-                reinterpret_cast<const f32x4*>(a.stash_in + int64_t(a.c0 + row) * a.ld_stash + n0 + lane * 4));
+            const float* srow = a.stash_in + int64_t(a.c0 + row) * a.ld_stash;
+            f32x4 y4;
+            if (a.stash_cols == nullptr) {
+                y4 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(srow + n0 + lane * 4));
+            } else {  // compacted tokens: runs of neighbours in the stash stay neighbours, so this still coalesces
+#pragma unroll
+                for (int j = 0; j < 4; ++j) y4[j] = col[j] >= 0 ? __builtin_nontemporal_load(srow + col[j]) : 0.f;
+            }
             const float bias = (!plain && a.bias != nullptr && row < rows) ? a.bias[a.c0 + row] : 0.f;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -1163,9 +1172,9 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
                                    int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                                    int64_t weight_stride, float temperature, float final_logit_softcapping,
                                    float logit_scale, const float* d_bias, const float* d_log_z, const float* d_g_logp,
-                                   int64_t chunk_size, const float* d_stash, int64_t stash_ld, void* d_out_dhidden,
-                                   void* d_out_dweight, float* d_out_dbias, void* d_workspace, size_t workspace_bytes,
-                                   trlk_stream_t stream) {
+                                   int64_t chunk_size, const float* d_stash, int64_t stash_ld, const int32_t* d_stash_cols,
+                                   void* d_out_dhidden, void* d_out_dweight, float* d_out_dbias, void* d_workspace,
+                                   size_t workspace_bytes, trlk_stream_t stream) {
     clear_error();
     if (int rc = check_head("fused_head_bwd", d_hidden, d_weight, d_targets, dtype, n_tokens, vocab, hidden_size,
                             hidden_stride, weight_stride, temperature))
@@ -1184,7 +1193,9 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     TRLK_REQUIRE(d_log_z && d_g_logp, TRLK_ERR_NULL_POINTER, "fused_head_bwd: log_z / g_logp pointer is null");
     TRLK_REQUIRE(d_stash == nullptr || n_tokens <= int64_t(65535) * kSdzTokens, TRLK_ERR_BAD_SHAPE,
                  "fused_head_bwd: too many tokens for the stash path (%lld)", (long long)n_tokens);
-    TRLK_REQUIRE(d_stash == nullptr || (stash_ld >= round_up(n_tokens, BN) && stash_ld % 4 == 0 &&
+    TRLK_REQUIRE(d_stash_cols == nullptr || d_stash != nullptr, TRLK_ERR_NULL_POINTER,
+                 "fused_head_bwd: stash columns given without a stash");
+    TRLK_REQUIRE(d_stash == nullptr || ((d_stash_cols != nullptr || stash_ld >= round_up(n_tokens, BN)) && stash_ld % 4 == 0 &&
                                         reinterpret_cast<uintptr_t>(d_stash) % 16 == 0),
                  TRLK_ERR_BAD_STRIDE, "fused_head_bwd: the stash needs a 16-byte aligned buffer with a row stride >= %lld (got %lld)",
                  (long long)round_up(n_tokens, BN), (long long)stash_ld);
@@ -1220,6 +1231,7 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     a.log_z = d_log_z;
     a.g = d_g_logp;
     a.stash_in = d_stash;
+    a.stash_cols = d_stash_cols;
     a.ld_stash = stash_ld;
     a.dz = dz;
     a.dzT = dzt;

@@ -505,9 +505,11 @@ def _(hidden, weight, targets, temperature, softcap, logit_scale, bias=None, sta
 @torch.library.custom_op("trl_amd::fused_head_bwd", mutates_args=(), device_types="cuda")
 def fused_head_bwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature: float, softcap: float,
                    logit_scale: float, log_z: Tensor, g_logp: Tensor, chunk_size: int,
-                   bias: Optional[Tensor] = None, stash: Optional[Tensor] = None) -> tuple[Tensor, Tensor, Tensor]:
+                   bias: Optional[Tensor] = None, stash: Optional[Tensor] = None,
+                   stash_cols: Optional[Tensor] = None) -> tuple[Tensor, Tensor, Tensor]:
     """Returns (d hidden [N, H], d weight [V, H]) in the operand dtype and d bias (fp32 [V]; empty without a bias).
-    `stash`: the fifth output of a `fused_head_fwd(..., stash=True)` on the same operands (skips the recompute)."""
+    `stash`: the fifth output of a `fused_head_fwd(..., stash=True)` on the same operands (skips the recompute);
+    `stash_cols` (int32 [N]): the forward's row of each token when rows were dropped since (see `head_backward`)."""
     w_dtype = weight.dtype
     hidden, weight, targets = _head_operands(hidden, weight, targets)
     n, h = hidden.shape
@@ -520,8 +522,15 @@ def fused_head_bwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
     d_bias = torch.empty((v if bias is not None else 0,), dtype=torch.float32, device=dev)
     if stash is not None and stash.numel() == 0:
         stash = None
+    if stash is None:
+        stash_cols = None
+    if stash_cols is not None:
+        if stash_cols.dtype != torch.int32 or stash_cols.shape != (n,):
+            raise ValueError("fused head: stash_cols must be int32 [N]")
+        stash_cols = stash_cols.contiguous()
     if stash is not None and (stash.dtype != torch.float32 or stash.stride(1) != 1 or
-                              stash.shape[0] < (v + 255) // 256 * 256 or stash.shape[1] < (n + 255) // 256 * 256):
+                              stash.shape[0] < (v + 255) // 256 * 256 or
+                              (stash_cols is None and stash.shape[1] < (n + 255) // 256 * 256)):
         raise ValueError("fused head: the stash does not belong to these operands")
     ws_bytes = lib.trlk_fused_head_bwd_workspace_bytes(max(n, 1), v, h, chunk_size)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
@@ -529,15 +538,45 @@ def fused_head_bwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
         check(lib.trlk_fused_head_bwd(ptr(hidden), ptr(weight), ptr(targets), dtype_code(hidden.dtype), n, v, h,
                                       hidden.stride(0), weight.stride(0), temperature, softcap, logit_scale,
                                       ptr(bias32), ptr(log_z), ptr(g), chunk_size, ptr(stash),
-                                      stash.stride(0) if stash is not None else 0, ptr(d_hidden), ptr(d_weight),
+                                      stash.stride(0) if stash is not None else 0, ptr(stash_cols), ptr(d_hidden),
+                                      ptr(d_weight),
                                       ptr(d_bias) if bias is not None else None, ptr(ws), ws_bytes, current_stream(dev)))
     return d_hidden, (d_weight if w_dtype == d_weight.dtype else d_weight.to(w_dtype)), d_bias
 
 
 @fused_head_bwd.register_fake
-def _(hidden, weight, targets, temperature, softcap, logit_scale, log_z, g_logp, chunk_size, bias=None, stash=None):
+def _(hidden, weight, targets, temperature, softcap, logit_scale, log_z, g_logp, chunk_size, bias=None, stash=None,
+      stash_cols=None):
     return (torch.empty_like(hidden), torch.empty_like(weight),
             torch.empty((weight.shape[0] if bias is not None else 0,), dtype=torch.float32, device=hidden.device))
+
+
+def head_backward(hidden: Tensor, weight: Tensor, targets: Tensor, temperature: float, softcap: float,
+                  logit_scale: float, log_z: Tensor, g_logp: Tensor, chunk_size: int, bias: Optional[Tensor] = None,
+                  stash: Optional[Tensor] = None) -> tuple[Tensor, Tensor, Tensor]:
+    """`fused_head_bwd` that first drops the tokens whose upstream gradient is exactly zero (masked positions of
+    a policy loss): their dz row is zero, so they add nothing to d weight and their d hidden row is zero.  Both
+    products shrink with the share of such tokens; one host synchronisation (the count) per call.  Tokens are only
+    dropped when at least a tenth of them can go."""
+    n = hidden.shape[0]
+    g = g_logp.reshape(-1)
+    if n == 0 or os.environ.get("TRL_AMD_HEAD_DROP_ZERO_GRAD", "1") == "0":
+        return fused_head_bwd(hidden, weight, targets, temperature, softcap, logit_scale, log_z, g, chunk_size, bias, stash)
+    active = g != 0
+    n_active = int(active.sum())
+    if n_active > 0.9 * n:
+        return fused_head_bwd(hidden, weight, targets, temperature, softcap, logit_scale, log_z, g, chunk_size, bias, stash)
+    idx = active.nonzero().squeeze(1)
+    d_hidden = torch.zeros_like(hidden)
+    if n_active == 0:
+        d_bias = torch.zeros((weight.shape[0] if bias is not None else 0,), dtype=torch.float32, device=hidden.device)
+        return d_hidden, torch.zeros_like(weight), d_bias
+    cols = idx.to(torch.int32) if stash is not None and stash.numel() else None
+    d_h, d_weight, d_bias = fused_head_bwd(
+        hidden.index_select(0, idx), weight, targets.index_select(0, idx), temperature, softcap, logit_scale,
+        log_z.index_select(0, idx), g.index_select(0, idx), chunk_size, bias, stash, cols)
+    d_hidden.index_copy_(0, idx, d_h)
+    return d_hidden, d_weight, d_bias
 
 
 NAN = math.nan

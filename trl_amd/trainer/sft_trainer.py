@@ -43,7 +43,7 @@ class _FusedNLLFunction(torch.autograd.Function):
                                                              g_logp)
             d_weight = d_weight.to(weight.dtype)
         else:
-            d_hidden, d_weight, d_bias = ops.fused_head_bwd(hidden, weight, labels, 1.0, softcap, logit_scale, log_z,
+            d_hidden, d_weight, d_bias = ops.head_backward(hidden, weight, labels, 1.0, softcap, logit_scale, log_z,
                                                             g_logp, chunk_size, bias, saved)
         return d_hidden, d_weight, None, None, None, None, None if bias is None else d_bias.to(bias.dtype)
 

@@ -253,7 +253,7 @@ class _ChunkedLogProbFunction(torch.autograd.Function):
                                                              grad_logprobs)
             return (d_hidden, d_weight.to(weight.dtype), None, None, None, None, None,
                     None if bias is None else d_bias.to(bias.dtype))
-        d_hidden, d_weight, d_bias = ops.fused_head_bwd(hidden, weight, targets, temperature, cap, logit_scale,
+        d_hidden, d_weight, d_bias = ops.head_backward(hidden, weight, targets, temperature, cap, logit_scale,
                                                         log_z, grad_logprobs, chunk_size, bias, saved)
         return (d_hidden, d_weight, None, None, None, None, None,
                 None if bias is None else d_bias.to(bias.dtype))
