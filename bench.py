@@ -242,6 +242,21 @@ def bench_head(args, w):
         torch.cuda.synchronize()
         return a.elapsed_time(b) / reps
 
+    # the same loss through the fused-linear operator (the call behind `use_liger_kernel`): it compacts the hidden
+    # states to the rows of the completion mask before the head, so forward and backward both run on those rows only
+    fl = trl_amd.FusedLinearGRPOLoss(beta=w["beta"], epsilon_low=w["eps_low"], epsilon_high=w["eps_high"],
+                                     temperature=w["temperature"], use_ref_model=w["beta"] != 0.0,
+                                     loss_type=args.loss_type, max_completion_length=T, chunk_size=HEAD_CHUNK)
+    h3, t3 = hidden.view(B, T, H), targets.view(B, T)
+
+    def fl_step():
+        hidden.grad = weight.grad = None
+        loss_fl, _ = fl(h3, weight, t3, mask, adv, None, old, ref if w["beta"] else None)
+        loss_fl.backward()
+        return loss_fl
+
+    fl_ms = time_op(fl_step, reps=max(2, args.steps // 2))
+    fl_loss = float(fl_step().detach())
     stash = ops.head_stash_fits(N, V)  # what the step above did: keep the forward's products, or recompute them
     flop = 2.0 * N * H * V
     with torch.no_grad():
@@ -292,6 +307,9 @@ def bench_head(args, w):
             "fused_head_bwd_step": {"avg_ms": bwd_step_ms, "tokens": int(mask.sum()),
                                     "note": "as in the step: tokens whose upstream gradient is zero are dropped"},
             "step_if_every_token_had_a_gradient_ms": ms_per_step - bwd_step_ms + bwd_ms}),
+        "mask_aware": {"ms_per_step": fl_ms, "tokens_per_s": N / (fl_ms * 1e-3), "loss": fl_loss,
+                       "note": "FusedLinearGRPOLoss: only the rows of the completion mask go through the head, forward "
+                               "and backward; same loss"},
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_head(w),
     }
     print(json.dumps(result))
