@@ -34,6 +34,7 @@ namespace {
 #endif
 constexpr int kThreads = TRLK_THREADS;
 constexpr int kUnroll = TRLK_FWD_UNROLL;
+static_assert(kUnroll >= 2, "the row tail of the forward holds up to kUnroll - 1 vectors per lane");
 constexpr int kBwdUnroll = TRLK_BWD_UNROLL;
 
 template <bool NT>
@@ -96,19 +97,25 @@ struct OnlineLse {
 
 // Extra per-lane row statistics of the STATS variant (what the DPO metrics and the WPO weights
 // need on top of log-prob and entropy, so that no further pass over the logits is necessary):
-// sum of exp2(x*c - r)^2 (same reference as OnlineLse), sum of x, and the number of elements that
-// come before the target in arg-max order (larger value, or equal value at a smaller position).
+// sum of exp2(x*c - r)^2 (same reference as OnlineLse), sum of x, and the lane's running maximum
+// with the FIRST position that holds it (a lane visits its positions in increasing order and only
+// a strictly larger value moves the position, so ties keep the earliest one, as torch.argmax does).
 struct RowStats {
     float s2 = 0.f, sx = 0.f;
-    int beats = 0;
+    float vmax = -INFINITY;
+    float vpos = 3.0e38f;  // position as a float: exact below 2^24, which the host guarantees
 };
 
-// Next float below x (x itself for -inf and NaN).
-__device__ __forceinline__ float prev_float(float x) {
-    if (!(x > -INFINITY)) return x;
-    const uint32_t b = __builtin_bit_cast(uint32_t, x);
-    if ((b << 1) == 0u) return __builtin_bit_cast(float, 0x80000001u);  // +-0 -> smallest negative denormal
-    return __builtin_bit_cast(float, (b >> 31) ? b + 1u : b - 1u);
+// sum of the two 16-bit floats packed in w, added to acc (one dot-product instruction against (1, 1))
+template <int DT>
+__device__ __forceinline__ float add_pair(uint32_t w, float acc) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+    if constexpr (DT == TRLK_BF16)
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), __builtin_bit_cast(bf16x2_t, 0x3F803F80u),
+                                               acc, false);
+    else
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, w), __builtin_bit_cast(f16x2_t, 0x3C003C00u), acc, false);
 }
 
 template <int N>
@@ -126,7 +133,7 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
     typedef Elem<DT> E;
     typedef typename E::type T;
     constexpr int NW = kThreads / kWave;
-    __shared__ float red[STATS ? 6 : 3][NW];
+    __shared__ float red[STATS ? 7 : 3][NW];
     __shared__ float bcast[2];
 
     const int64_t row = blockIdx.x;
@@ -148,34 +155,32 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
 
     OnlineLse acc;
     RowStats st;
-    // arg-max order against the target (first index of the row): an element before the target's
-    // position beats it with x >= xt, one behind it with x > xt; x >= xt is tested as x > xt_prev
-    // with the next smaller float (the logits are exact in fp32).
-    int64_t tpos = -1;
-    float xt = INFINITY, xt_prev = INFINITY;
-    if constexpr (STATS) {
-        const int64_t idx = a.n_index > 0 ? a.index[row * a.n_index] : -1;
-        if (idx >= 0 && idx < V) {
-            tpos = idx;
-            xt = E::load1(base + idx);
-            xt_prev = prev_float(xt);
-        }
-    }
     // one element with its position e (stats only)
     auto stat_elem = [&](float x, int64_t e) {
         st.sx += x;
-        st.beats += x > (e < tpos ? xt_prev : xt) ? 1 : 0;
+        if (x > st.vmax) {
+            st.vmax = x;
+            st.vpos = float(e);
+        }
     };
-    // EPV elements starting at position e0: one threshold for the whole vector unless it holds the target
-    auto stat_vec = [&](const float* x, int64_t e0, int n) {
-        if (e0 <= tpos && tpos < e0 + n) {
-            for (int i = 0; i < n; ++i) stat_elem(x[i], e0 + i);
+    // N elements starting at position e0 whose maximum is bm (q: their packed form, 16-bit types only).  The
+    // running maximum moves a few times per row only, so the position search sits in a rarely taken branch.
+    // (the sum is taken from the packed form first, so that it need not stay in registers beside the unpacked one)
+    auto stat_sum = [&](u32x4 q) {
+        if constexpr (DT == TRLK_F32) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) st.sx += __uint_as_float(q[w]);
         } else {
-            const float thr = e0 < tpos ? xt_prev : xt;
-            for (int i = 0; i < n; ++i) {
-                st.sx += x[i];
-                st.beats += x[i] > thr ? 1 : 0;
-            }
+#pragma unroll
+            for (int w = 0; w < 4; ++w) st.sx = add_pair<DT>(q[w], st.sx);
+        }
+    };
+    auto stat_vec = [&](const float* x, int64_t e0, int n, float bm) {
+        if (bm > st.vmax) {
+            st.vmax = bm;
+            int first = n - 1;
+            for (int i = n - 2; i >= 0; --i) first = x[i] == bm ? i : first;
+            st.vpos = float(e0 + first);
         }
     };
     auto raise = [&](float bm) {
@@ -207,24 +212,45 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
             u32x4 q[kUnroll];
 #pragma unroll
             for (int j = 0; j < kUnroll; ++j) q[j] = stream_load<kFwdNt>(vp + v + j * kThreads);
+            if constexpr (STATS) {
+#pragma unroll
+                for (int j = 0; j < kUnroll; ++j) stat_sum(q[j]);
+            }
             float x[kUnroll * EPV];
 #pragma unroll
             for (int j = 0; j < kUnroll; ++j) E::unpack(q[j], x + j * EPV);
-            raise(max_of<kUnroll * EPV>(x));
+            float bmj[kUnroll];  // per-vector maxima (the statistics need them), then the maximum of all
+#pragma unroll
+            for (int j = 0; j < kUnroll; ++j) bmj[j] = max_of<EPV>(x + j * EPV);
+            raise(max_of<kUnroll>(bmj));
 #pragma unroll
             for (int i = 0; i < kUnroll * EPV; ++i) add(x[i]);
             if constexpr (STATS) {
 #pragma unroll
-                for (int j = 0; j < kUnroll; ++j) stat_vec(x + j * EPV, int64_t(v + j * kThreads) * EPV, EPV);
+                for (int j = 0; j < kUnroll; ++j)  // increasing positions: j-th vector before the (j+1)-th
+                    stat_vec(x + j * EPV, int64_t(v + j * kThreads) * EPV, EPV, bmj[j]);
             }
         }
-        for (; v < nvec; v += kThreads) {
-            float x[EPV];
-            E::unpack(stream_load<kFwdNt>(vp + v), x);
-            raise(max_of<EPV>(x));
+        // the row's tail: fewer than kUnroll vectors are left for this lane; their loads go out together
+        // (one after the other they would cost a memory round trip each, at the end of every row)
+        {
+            u32x4 q[kUnroll - 1];
 #pragma unroll
-            for (int i = 0; i < EPV; ++i) add(x[i]);
-            if constexpr (STATS) stat_vec(x, int64_t(v) * EPV, EPV);
+            for (int j = 0; j < kUnroll - 1; ++j)
+                if (v + j * kThreads < nvec) q[j] = stream_load<kFwdNt>(vp + v + j * kThreads);
+#pragma unroll
+            for (int j = 0; j < kUnroll - 1; ++j) {
+                if (v + j * kThreads < nvec) {
+                    if constexpr (STATS) stat_sum(q[j]);
+                    float x[EPV];
+                    E::unpack(q[j], x);
+                    const float bm = max_of<EPV>(x);
+                    raise(bm);
+#pragma unroll
+                    for (int i = 0; i < EPV; ++i) add(x[i]);
+                    if constexpr (STATS) stat_vec(x, int64_t(v + j * kThreads) * EPV, EPV, bm);
+                }
+            }
         }
     } else {
         for (int64_t v = tid; v < V; v += kThreads) {
@@ -254,11 +280,14 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
     if constexpr (STATS) {
         const float s2 = wave_sum(st.s2 * sc * sc);
         const float sx = wave_sum(st.sx);
-        const float beats = wave_sum(float(st.beats));  // exact: the host admits vocab < 2^24 only
+        // the row maximum and the smallest position among the lanes that hold it
+        const float wmax = wave_max(st.vmax);
+        const float wpos = wave_min(st.vmax == wmax ? st.vpos : 3.0e38f);
         if (lane == 0) {
             red[3][wave] = s2;
             red[4][wave] = sx;
-            red[5][wave] = beats;
+            red[5][wave] = wmax;
+            red[6][wave] = wpos;
         }
     }
     __syncthreads();
@@ -270,17 +299,21 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
             U += red[2][w];
         }
         if constexpr (STATS) {
-            float S2 = 0.f, SX = 0.f, beats = 0.f;
+            float S2 = 0.f, SX = 0.f, vmax = -INFINITY, vpos = 3.0e38f;
 #pragma unroll
             for (int w = 0; w < NW; ++w) {
                 S2 += red[3][w];
                 SX += red[4][w];
-                beats += red[5][w];
+                if (red[5][w] > vmax || (red[5][w] == vmax && red[6][w] < vpos)) {
+                    vmax = red[5][w];
+                    vpos = red[6][w];
+                }
             }
+            const int64_t tpos = a.n_index > 0 ? a.index[row * a.n_index] : -1;
             float* o = a.out_stats + row * 4;
             o[0] = SX / float(V);
             o[1] = logf(S2) - 2.f * logf(S);  // log sum_v softmax(z)_v^2: the common reference cancels
-            o[2] = (tpos >= 0 && beats == 0.f) ? 1.f : 0.f;
+            o[2] = (tpos >= 0 && tpos < V && float(tpos) == vpos) ? 1.f : 0.f;
             o[3] = 0.f;
         }
         // lse = R*ln2 + ln S with ln2 split in two so that the product carries no rounding of ln2
