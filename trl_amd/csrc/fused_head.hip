@@ -945,12 +945,11 @@ struct GemmArgs {
 };
 
 template <int DT, int MODE>
-TRLK_HEAD_KERNEL void gemm_nt_kernel(GemmArgs a) {
-    extern __shared__ __attribute__((aligned(16))) char smem[];
+__device__ __forceinline__ void gemm_nt_body(const GemmArgs& a, int block, char* smem) {
     typedef Elem<DT> E;
     const int n_mt = (a.M + BM - 1) / BM, n_nt = (a.N + BN - 1) / BN;
     int tm, tn;
-    xcd_patch(blockIdx.x, n_nt, tm, tn);
+    xcd_patch(block, n_nt, tm, tn);
     if (tm >= n_mt || tn >= n_nt) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -975,6 +974,24 @@ TRLK_HEAD_KERNEL void gemm_nt_kernel(GemmArgs a) {
                     E::store1(a.out_lp + int64_t(row) * a.ld_lp + col, v);
             }
         }
+}
+
+template <int DT, int MODE>
+TRLK_HEAD_KERNEL void gemm_nt_kernel(GemmArgs a) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    gemm_nt_body<DT, MODE>(a, blockIdx.x, smem);
+}
+
+// Two independent products in one launch: workgroups [0, grid_a) take `a` (epilogue MODE_A), the rest take `b`
+// (epilogue 0).  When the tile count of one product is not a multiple of the CU count, the other product's
+// tiles fill the CUs its last round leaves idle.  grid_a is a multiple of 8 (the XCD mapping of `b` is kept).
+template <int DT, int MODE_A>
+TRLK_HEAD_KERNEL void gemm_nt_pair_kernel(GemmArgs a, int grid_a, GemmArgs b) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    if (int(blockIdx.x) < grid_a)
+        gemm_nt_body<DT, MODE_A>(a, blockIdx.x, smem);
+    else
+        gemm_nt_body<DT, 0>(b, int(blockIdx.x) - grid_a, smem);
 }
 
 // [R, C] (ld) -> [C, ldo] with columns >= R zero-filled up to `fill`: 64 x 64 tiles through LDS.
@@ -1071,8 +1088,26 @@ int check_head(const char* what, const void* hidden, const void* weight, const i
     return TRLK_OK;
 }
 
+template <typename Kern>
+int reserve_head_lds(Kern kern, const char* what);
+
+template <typename Kern>
+int launch_head_pair(Kern kern, int grid_a, const GemmArgs& a, int grid_b, const GemmArgs& b, hipStream_t s,
+                     const char* what) {
+    if (int rc = reserve_head_lds(kern, what)) return rc;
+    hipLaunchKernelGGL(kern, dim3(grid_a + grid_b), dim3(kHeadThreads), kHeadLdsBytes, s, a, grid_a, b);
+    return launch_status(what);
+}
+
 template <typename Kern, typename Args>
 int launch_head(Kern kern, int grid, const Args& a, hipStream_t s, const char* what) {
+    if (int rc = reserve_head_lds(kern, what)) return rc;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kHeadThreads), kHeadLdsBytes, s, a);
+    return launch_status(what);
+}
+
+template <typename Kern>
+int reserve_head_lds(Kern kern, const char* what) {
     static thread_local const void* configured[16] = {};
     // dynamic LDS above 64 KiB has to be allowed per kernel once
     bool done = false;
@@ -1087,8 +1122,7 @@ int launch_head(Kern kern, int grid, const Args& a, hipStream_t s, const char* w
                 break;
             }
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kHeadThreads), kHeadLdsBytes, s, a);
-    return launch_status(what);
+    return TRLK_OK;
 }
 
 }  // namespace
@@ -1289,13 +1323,6 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         gh.ld_lp = H;
         gh.first = first;
         const int ghgrid = xcd_patch_grid(n_tb, n_ht);
-        if (last)
-            rc = dtype == TRLK_BF16 ? launch_head(gemm_nt_kernel<TRLK_BF16, 2>, ghgrid, gh, s, "fused_head_bwd (dHidden)")
-                                    : launch_head(gemm_nt_kernel<TRLK_F16, 2>, ghgrid, gh, s, "fused_head_bwd (dHidden)");
-        else
-            rc = dtype == TRLK_BF16 ? launch_head(gemm_nt_kernel<TRLK_BF16, 1>, ghgrid, gh, s, "fused_head_bwd (dHidden)")
-                                    : launch_head(gemm_nt_kernel<TRLK_F16, 1>, ghgrid, gh, s, "fused_head_bwd (dHidden)");
-        if (rc) return rc;
         // dW[chunk, H] = dz^T[chunk, N] * (hidden^T[H, N])^T
         GemmArgs gw{};
         gw.A = Operand{dzt, l.ld_n, kpad};
@@ -1306,9 +1333,15 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         gw.out_lp = static_cast<uint16_t*>(d_out_dweight) + c0 * hidden_size;
         gw.ld_lp = hidden_size;
         gw.first = 1;
-        rc = dtype == TRLK_BF16
-                 ? launch_head(gemm_nt_kernel<TRLK_BF16, 0>, xcd_patch_grid(n_vt, n_ht), gw, s, "fused_head_bwd (dW)")
-                 : launch_head(gemm_nt_kernel<TRLK_F16, 0>, xcd_patch_grid(n_vt, n_ht), gw, s, "fused_head_bwd (dW)");
+        // both products of the chunk in one launch (dHidden's workgroups first)
+        const int gwgrid = xcd_patch_grid(n_vt, n_ht);
+        const char* what = "fused_head_bwd (dHidden, dW)";
+        if (last)
+            rc = dtype == TRLK_BF16 ? launch_head_pair(gemm_nt_pair_kernel<TRLK_BF16, 2>, ghgrid, gh, gwgrid, gw, s, what)
+                                    : launch_head_pair(gemm_nt_pair_kernel<TRLK_F16, 2>, ghgrid, gh, gwgrid, gw, s, what);
+        else
+            rc = dtype == TRLK_BF16 ? launch_head_pair(gemm_nt_pair_kernel<TRLK_BF16, 1>, ghgrid, gh, gwgrid, gw, s, what)
+                                    : launch_head_pair(gemm_nt_pair_kernel<TRLK_F16, 1>, ghgrid, gh, gwgrid, gw, s, what);
         if (rc) return rc;
     }
     return TRLK_OK;
