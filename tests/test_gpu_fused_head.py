@@ -327,6 +327,38 @@ def test_real_head_shape_row_subsample(amd):
     assert _rel_l2(dw.float(), rdw) < 1e-2
 
 
+def test_real_head_shape_paths_agree(amd, monkeypatch):
+    """BASELINE config 5's head shape on 4096 tokens (16 token blocks, 594 vocabulary tiles, 5 backward chunks, a
+    prefix mask on the upstream gradient): the stash + token-dropping path gives the recompute path's results, and
+    size-independent properties hold -- rows without an upstream gradient get none, dW sums to zero over the
+    vocabulary (softmax gradients are orthogonal to the constant shift) and the probabilities behind the entropy are
+    normalised (0 <= H <= ln V)."""
+    gdev = torch.Generator(device=DEV).manual_seed(77)
+    n, h, v = 4096, 3584, 151936
+    hidden = torch.randn(n, h, generator=gdev, device=DEV).bfloat16()
+    weight = (0.02 * torch.randn(v, h, generator=gdev, device=DEV)).bfloat16()
+    labels = torch.randint(0, v, (n,), generator=gdev, device=DEV)
+    lengths = torch.randint(16, 257, (16,), generator=gdev, device=DEV)
+    active = (torch.arange(256, device=DEV)[None] < lengths[:, None]).reshape(-1)
+    gout = torch.randn(n, generator=gdev, device=DEV) * active
+    out = {}
+    for mode, gib, drop in (("stash", "24", "1"), ("recompute", "0", "0")):
+        monkeypatch.setenv("TRL_AMD_HEAD_STASH_GIB", gib)
+        monkeypatch.setenv("TRL_AMD_HEAD_DROP_ZERO_GRAD", drop)
+        hh, ww = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+        lp, ent = amd._ChunkedLogProbFunction.apply(hh, ww, labels, 1.0, 32768)
+        (lp * gout).sum().backward()
+        out[mode] = (lp.detach(), ent, hh.grad, ww.grad)
+    a, b = out["stash"], out["recompute"]
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    assert _rel_l2(a[2].float(), b[2].float()) < 2e-3 and _rel_l2(a[3].float(), b[3].float()) < 2e-3
+    assert torch.count_nonzero(a[2][~active]) == 0 and torch.count_nonzero(a[2][active]) > 0
+    col_sum = a[3].float().sum(0)  # sum_v dW[v, :] = sum_n (sum_v dz[n, v]) hidden[n, :] = 0
+    assert float(col_sum.abs().max()) < 2e-2 * float(a[3].float().abs().sum(0).max())
+    assert float(a[1].min()) >= 0.0 and float(a[1].max()) <= float(torch.log(torch.tensor(float(v)))) + 1e-3
+    assert float(a[0].max()) <= 0.0
+
+
 def test_golden_sft_chunked_nll(amd):
     """The reference's `_chunked_cross_entropy_loss` wrote these; fp32 cases are run in bf16 on the device
     (the matrix-core kernels take bf16/fp16) and compared with the oracle on the bf16-rounded operands."""
