@@ -417,7 +417,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs on ONE GPU; rows are independent, so N GPUs would each run this same "
-                 "kernel on B/N sequences (see DESIGN.md). Run with --gpus 1.")
+                 "kernel on B/N sequences and exchange a handful of scalars per step. Run with --gpus 1.")
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the hot path has no CPU fallback.")
 
