@@ -1216,7 +1216,6 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     TRLK_REQUIRE(chunk_size >= 1, TRLK_ERR_BAD_VALUE, "fused_head_bwd: chunk_size must be >= 1");
     TRLK_REQUIRE(d_out_dhidden && d_out_dweight, TRLK_ERR_NULL_POINTER, "fused_head_bwd: null output pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const size_t es = 2;
     if (n_tokens == 0) {  // no tokens: both gradients are zero
         hipLaunchKernelGGL(head_fill_kernel, dim3(unsigned((vocab * hidden_size / 2 + 255) / 256)), dim3(256), 0, s,
                            static_cast<float*>(d_out_dweight), vocab * hidden_size / 2, 0.f);
@@ -1243,7 +1242,6 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     uint16_t* dz = reinterpret_cast<uint16_t*>(ws + l.off_dz);    // [N, cpad], row stride ld_c
     uint16_t* dzt = reinterpret_cast<uint16_t*>(ws + l.off_dzt);  // [cpad, npad], row stride ld_n
     float* dh = reinterpret_cast<float*>(ws + l.off_dh);          // [N, H]
-    (void)es;
     const int H = int(hidden_size), N = int(n_tokens), V = int(vocab);
     hipLaunchKernelGGL(transpose16_kernel, dim3((H + 63) / 64, unsigned((l.npad + 63) / 64)), dim3(256), 0, s,
                        static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.ld_n, l.npad);
