@@ -279,6 +279,46 @@ def test_full_size_properties_config3_shape(amd):
     assert _rel_l2(got_g, want_g) < 3e-3
 
 
+def test_long_context_config4_saved_state_and_properties(amd):
+    """BASELINE config 4 (32 x 4096 rows, V = 151936, bf16: 39.8 GB of logits): what the forward keeps for the
+    backward is a few bytes per row (the reference keeps a [T, V] log-softmax per sequence), masked rows and the
+    dropped last position get exactly zero gradient, and sum_v dlogits = 0 on the active rows."""
+    B, T, V = 32, 4096, 151936
+    g = torch.Generator(device=DEV).manual_seed(4)
+    logits = torch.empty(B, T + 1, V, dtype=torch.bfloat16, device=DEV)
+    for b in range(B):
+        for t0 in range(0, T + 1, 1024):  # blocks keep the fp32 temporary small
+            t1 = min(t0 + 1024, T + 1)
+            logits[b, t0:t1] = (2.0 * torch.randn(t1 - t0, V, generator=g, device=DEV)).bfloat16()
+    ids = torch.randint(0, V, (B, T + 1), generator=g, device=DEV)
+    lengths = torch.randint(512, T + 1, (B,), generator=g, device=DEV)
+    mask = (torch.arange(T, device=DEV)[None] < lengths[:, None]).float()
+    logits.requires_grad_(True)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    lp, ent = amd.per_token_logps_and_entropies(logits, ids, T, 1.0, True)
+    torch.cuda.synchronize()
+    held = torch.cuda.memory_allocated() - before
+    rows = B * T
+    # outputs (lp, ent: fp32 per row) + saved for backward (lse, entropy: fp32 per row) + int64 index per row
+    assert held <= rows * (4 * 4 + 8) + (1 << 20), held
+    assert (lp <= 0).all() and (ent >= 0).all() and (ent <= math.log(V) + 1e-3).all()
+    gl = torch.randn(B, T, generator=g, device=DEV) * mask
+    (lp * gl).sum().backward()
+    grad = logits.grad
+    row_nonzero = torch.stack([(grad[b] != 0).any(-1) for b in range(B)])
+    assert not row_nonzero[:, -1].any() and torch.equal(row_nonzero[:, :T], gl != 0)
+    row_sum = torch.stack([grad[b, :T].float().sum(-1) for b in range(B)])
+    assert (row_sum.abs() <= 2e-2 * gl.abs() + 1e-6).all()
+    # a few rows against fp32 op-math on the same stored values
+    pick_b, pick_t = torch.tensor([0, 31]), torch.tensor([0, 2047, 4095])
+    sub = logits.detach()[pick_b][:, pick_t].cpu()
+    sub_ids = ids[pick_b][:, pick_t + 1].cpu()
+    torch.testing.assert_close(lp.detach()[pick_b][:, pick_t].cpu(), oracle.selective_log_softmax_f32(sub, sub_ids, 1.0),
+                               atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent[pick_b][:, pick_t].cpu(), oracle.entropy_from_logits_f32(sub, 1.0), atol=2e-3, rtol=0)
+
+
 def test_row_statistics_of_the_same_pass():
     """`logp_entropy_stats_fwd`: mean logit, log sum_v p_v^2 and the arg-max flag (first maximal position, as
     `torch.argmax`) against torch on the same values, at a real vocabulary size, with ties and masked rows."""
