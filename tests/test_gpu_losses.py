@@ -454,6 +454,43 @@ def test_dpo_against_oracle_config2_shape_subsample(amd):
         assert abs(float(named[name]) - want) <= 1e-3 * max(1.0, abs(want)), name
 
 
+def test_dpo_full_size_config2_closed_form_and_properties(amd):
+    """BASELINE config 2 at full size (64 x 2048 x 128256 bf16, 32 pairs, prompt + right padding): with the
+    reference log-probs equal to the policy's the loss is ln 2 and every pair carries the gradient -beta/(2P) on
+    the chosen and +beta/(2P) on the rejected sequence; rows outside the shifted completion mask and the last
+    position get exactly zero gradient; sum_v dlogits = 0 on the others."""
+    B, L, V, beta = 64, 2048, 128256, 0.1
+    P = B // 2
+    g = torch.Generator(device=DEV).manual_seed(2)
+    logits = torch.empty(B, L, V, dtype=torch.bfloat16, device=DEV)
+    for b in range(B):
+        for t0 in range(0, L, 1024):
+            logits[b, t0 : t0 + 1024] = (2.0 * torch.randn(1024, V, generator=g, device=DEV)).bfloat16()
+    ids = torch.randint(0, V, (B, L), generator=g, device=DEV)
+    lp_len = torch.randint(64, 513, (P,), generator=g, device=DEV).repeat(2)
+    lc_len = torch.randint(128, 1537, (B,), generator=g, device=DEV)
+    pos = torch.arange(L, device=DEV)[None]
+    cm = ((pos >= lp_len[:, None]) & (pos < (lp_len + lc_len)[:, None])).long()
+    seq = amd.dpo_sequence_logps(logits, ids, cm)
+    logits.requires_grad_(True)
+    loss, parts = amd.dpo_compute_loss(logits, ids, cm, seq[:P], seq[P:], beta=beta)
+    assert abs(float(loss) - math.log(2.0)) < 1e-6
+    loss.backward()
+    grad = logits.grad
+    shift = cm[:, 1:].bool()
+    row_nonzero = torch.stack([(grad[b] != 0).any(-1) for b in range(B)])
+    assert not row_nonzero[:, -1].any() and torch.equal(row_nonzero[:, :-1], shift)
+    row_sum = torch.stack([grad[b, :-1].float().sum(-1) for b in range(B)])
+    coef = beta / (2 * P)
+    assert (row_sum.abs() <= 2e-2 * coef).all()
+    # the target's entry: -/+ coef * (1 - p_target) on chosen / rejected rows
+    tgt = torch.stack([grad[b, :-1].gather(-1, ids[b, 1:, None]).squeeze(-1).float() for b in range(B)])
+    assert (tgt[:P][shift[:P]] < 0).all() and (tgt[P:][shift[P:]] > 0).all()
+    assert (tgt.abs() <= coef * (1 + 2e-2)).all()
+    m = amd.dpo_metrics_to_dict(parts)
+    assert abs(m["rewards/margins"]) < 1e-6 and 0.0 < m["entropy"] <= math.log(V)
+
+
 def test_golden_rloo_compute_loss(amd):
     cases, g = load_golden("rloo_compute_loss")
     for case in cases:
