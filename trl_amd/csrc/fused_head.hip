@@ -847,8 +847,14 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
 // One workgroup = 64 vocabulary rows x 256 tokens.  A lane owns 4 consecutive tokens; a wave walks
 // over row pairs.  dz^T (vocabulary-major, like the stash) is written directly, dz (token-major)
 // through an LDS transpose.  Rows beyond the chunk and tokens beyond N are written as zeros.
-constexpr int kSdzRows = 64, kSdzTokens = 256, kSdzLdsRow = kSdzRows * 2 + 4;  // bytes per staged token row
-template <int DT>
+#ifndef TRLK_SDZ_TOKENS
+#define TRLK_SDZ_TOKENS 256
+#endif
+constexpr int kSdzRows = 64, kSdzTokens = TRLK_SDZ_TOKENS, kSdzLdsRow = kSdzRows * 2 + 4;  // bytes per staged token row
+constexpr int kSdzLanesPerRow = kSdzTokens / 4, kSdzPairsPerWave = 64 / kSdzLanesPerRow;
+static_assert(kSdzTokens == 256 || kSdzTokens == 128, "a row of the tile is one wave or half a wave wide");
+// COLS: the tokens were compacted since the forward, a.stash_cols maps them to their stash columns.
+template <int DT, bool COLS>
 __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
     typedef Elem<DT> E;
     __shared__ __attribute__((aligned(16))) char lds[kSdzTokens * kSdzLdsRow];
@@ -862,27 +868,32 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
     float g[4], lzc[4];
     int64_t tg[4];
     int col[4];
+    const int tl0 = (lane % kSdzLanesPerRow) * 4, sub = lane / kSdzLanesPerRow;  // first token of the lane, row pair
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int tok = n0 + lane * 4 + j;
+        const int tok = n0 + tl0 + j;
         const bool ok = tok < a.N;
-        col[j] = (ok && a.stash_cols != nullptr) ? a.stash_cols[tok] : -1;
+        col[j] = (COLS && ok) ? a.stash_cols[tok] : -1;
         g[j] = ok ? a.g[tok] : 0.f;
         lzc[j] = ok ? a.log_z[tok] * kLog2e : INFINITY;
         tg[j] = ok ? a.targets[tok] - a.c0 : -1;  // chunk-local target row
     }
+    const bool contiguous = COLS && col[0] >= 0 && col[1] == col[0] + 1 && col[2] == col[0] + 2 && col[3] == col[0] + 3;
 #pragma unroll
-    for (int i = 0; i < kSdzRows / 8; ++i) {
-        const int rl = 2 * (wave + 4 * i);  // row pair rl, rl + 1 of this workgroup's 64
+    for (int i = 0; i < kSdzRows / (8 * kSdzPairsPerWave); ++i) {
+        const int rl = 2 * (wave * kSdzPairsPerWave + sub + 4 * kSdzPairsPerWave * i);  // row pair rl, rl + 1 of the 64
         float d[2][4];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int row = r0 + rl + h;
             const float* srow = a.stash_in + int64_t(a.c0 + row) * a.ld_stash;
             f32x4 y4;
-            if (a.stash_cols == nullptr) {
-                y4 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(srow + n0 + lane * 4));
-            } else {  // compacted tokens: runs of neighbours in the stash stay neighbours, so this still coalesces
+            if constexpr (!COLS) {
+                y4 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(srow + n0 + tl0));
+            } else if (contiguous) {  // the usual case: the lane's 4 tokens were neighbours in the forward too
+                typedef float f32x4_dword_aligned __attribute__((ext_vector_type(4), aligned(4)));
+                y4 = *reinterpret_cast<const f32x4_dword_aligned*>(srow + col[0]);
+            } else {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) y4[j] = col[j] >= 0 ? __builtin_nontemporal_load(srow + col[j]) : 0.f;
             }
@@ -911,11 +922,11 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
             uint2 w;
             w.x = E::pack2(d[h][0], d[h][1]);
             w.y = E::pack2(d[h][2], d[h][3]);
-            *reinterpret_cast<uint2*>(a.dzT + int64_t(row) * a.ldzt + n0 + lane * 4) = w;
+            *reinterpret_cast<uint2*>(a.dzT + int64_t(row) * a.ldzt + n0 + tl0) = w;
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            *reinterpret_cast<uint32_t*>(lds + (lane * 4 + j) * kSdzLdsRow + rl * 2) = E::pack2(d[0][j], d[1][j]);
+            *reinterpret_cast<uint32_t*>(lds + (tl0 + j) * kSdzLdsRow + rl * 2) = E::pack2(d[0][j], d[1][j]);
     }
     __syncthreads();
     constexpr int kPieces = kSdzRows / 8;  // 16-byte pieces per staged token row
@@ -1281,10 +1292,14 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         int rc;
         if (d_stash != nullptr) {
             const dim3 grid(unsigned(kpad / kSdzRows), unsigned(l.npad / kSdzTokens));
-            if (dtype == TRLK_BF16)
-                hipLaunchKernelGGL(head_dz_from_stash_kernel<TRLK_BF16>, grid, dim3(256), 0, s, a);
+            if (dtype == TRLK_BF16 && d_stash_cols)
+                hipLaunchKernelGGL((head_dz_from_stash_kernel<TRLK_BF16, true>), grid, dim3(256), 0, s, a);
+            else if (dtype == TRLK_BF16)
+                hipLaunchKernelGGL((head_dz_from_stash_kernel<TRLK_BF16, false>), grid, dim3(256), 0, s, a);
+            else if (d_stash_cols)
+                hipLaunchKernelGGL((head_dz_from_stash_kernel<TRLK_F16, true>), grid, dim3(256), 0, s, a);
             else
-                hipLaunchKernelGGL(head_dz_from_stash_kernel<TRLK_F16>, grid, dim3(256), 0, s, a);
+                hipLaunchKernelGGL((head_dz_from_stash_kernel<TRLK_F16, false>), grid, dim3(256), 0, s, a);
             rc = launch_status("fused_head_bwd (dz from the stash)");
         } else {
             rc = dtype == TRLK_BF16
