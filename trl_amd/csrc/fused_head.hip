@@ -477,18 +477,32 @@ __device__ __forceinline__ int acc_row(int wm, int mb, int r, int lane) {
 // Column (N index) inside the workgroup tile of block nb, for this lane.
 __device__ __forceinline__ int acc_col(int wn, int nb, int lane) { return wn * WN + nb * 32 + (lane & 31); }
 
-// Workgroup id -> (tile along N-like axis `a`, tile along the other axis `b`) such that the
-// workgroups that run together on one XCD (ids congruent mod 8, dispatched round-robin) form
-// 4 x 8 patches: they share operand slabs through that XCD's L2.
-__device__ __forceinline__ void xcd_patch(int w, int n_b, int& ta, int& tb) {
+// Workgroup id -> (tile along axis `a`, tile along axis `b`) such that the workgroups that run
+// together on one XCD (ids congruent mod 8, dispatched round-robin) form 4 x 8 patches: they share
+// operand slabs through that XCD's L2.  An XCD owns the `a` tiles congruent to its number mod 8, in
+// bands of 4; inside a band it walks b with the band's a tiles innermost.  The last band holds only
+// as many a tiles per XCD as n_a needs, so that (almost) no workgroup of the grid is empty: the
+// hardware deals workgroups to the CUs in order, and with empty ones interleaved at a fixed stride
+// the real ones end up on a fraction of the CUs (measured: a third more time for 65 instead of 64
+// a tiles with a grid padded to whole bands).  The caller skips ta >= n_a.
+__device__ __forceinline__ void xcd_patch(int w, int n_a, int n_b, int& ta, int& tb) {
     const int xcd = w & 7, q = w >> 3;
-    const int nb4 = (n_b + 7) / 8 * 8;  // b tiles padded to a multiple of 8 (callers skip the excess)
-    tb = (q >> 2) % nb4;
-    ta = ((q & 3) + 4 * (q / (4 * nb4))) * 8 + xcd;
+    const int bands = n_a >> 5;                    // full bands of 32 a tiles
+    const int full = bands * 4 * n_b;              // workgroups of this XCD in the full bands
+    if (q < full) {
+        const int rem = q % (4 * n_b);
+        tb = rem >> 2;
+        ta = ((q / (4 * n_b)) * 4 + (rem & 3)) * 8 + xcd;
+    } else {
+        const int m = (n_a - bands * 32 + 7) >> 3;  // a tiles per XCD in the last band (1..4; 0 = no last band)
+        const int qq = q - full;
+        tb = m > 0 ? qq / m : n_b;
+        ta = (bands * 4 + (m > 0 ? qq % m : 0)) * 8 + xcd;
+    }
 }
 inline int xcd_patch_grid(int n_a, int n_b) {
-    const int na32 = (n_a + 31) / 32 * 32, nb8 = (n_b + 7) / 8 * 8;
-    return na32 * nb8;
+    const int bands = n_a / 32, m = (n_a - bands * 32 + 7) / 8;
+    return 8 * (bands * 4 + m) * n_b;
 }
 
 struct HeadArgs {
@@ -528,7 +542,7 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int n_tb = (a.N + BN - 1) / BN;
     int tb, vs;
-    xcd_patch(blockIdx.x, a.v_splits, tb, vs);
+    xcd_patch(blockIdx.x, n_tb, a.v_splits, tb, vs);
     if (tb >= n_tb || vs >= a.v_splits) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -734,7 +748,7 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
     const int n_tb = (a.N + BN - 1) / BN;
     const int n_vt = (a.c1 - a.c0 + BM - 1) / BM;
     int tb, vt;
-    xcd_patch(blockIdx.x, n_vt, tb, vt);
+    xcd_patch(blockIdx.x, n_tb, n_vt, tb, vt);
     if (tb >= n_tb || vt >= n_vt) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -960,7 +974,7 @@ __device__ __forceinline__ void gemm_nt_body(const GemmArgs& a, int block, char*
     typedef Elem<DT> E;
     const int n_mt = (a.M + BM - 1) / BM, n_nt = (a.N + BN - 1) / BN;
     int tm, tn;
-    xcd_patch(block, n_nt, tm, tn);
+    xcd_patch(block, n_mt, n_nt, tm, tn);
     if (tm >= n_mt || tn >= n_nt) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
