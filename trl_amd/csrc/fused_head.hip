@@ -1091,7 +1091,25 @@ BwdLayout bwd_layout(int64_t N, int64_t V, int64_t H, int64_t chunk) {
     return l;
 }
 
-constexpr int kFwdSplits = 8;
+// Vocabulary splits of the forward.  A workgroup keeps one token block and walks over 1/splits of the
+// vocabulary tiles, so the grid is token blocks x splits workgroups of equal length, one per CU at a
+// time: the splits are chosen so that they fill whole rounds of the 256 CUs (65 token blocks x 8 splits
+// would run 3 rounds for 2.03 rounds of work), preferring few splits.
+constexpr int kCus = 256, kMinFwdSplits = 8, kMaxFwdSplits = 128;
+int fwd_splits(int64_t n_tokens) {
+    const int64_t n_tb = (n_tokens + BN - 1) / BN;
+    int best = kMinFwdSplits;
+    double best_cost = 1e30;
+    for (int sp = kMinFwdSplits; sp <= kMaxFwdSplits; sp *= 2) {
+        const double rounds = double(n_tb * sp) / kCus;
+        const double cost = double((n_tb * sp + kCus - 1) / kCus) / rounds;
+        if (cost < best_cost - 0.02) {  // more splits only for a gain of 2 % or more
+            best_cost = cost;
+            best = sp;
+        }
+    }
+    return best;
+}
 
 int check_head(const char* what, const void* hidden, const void* weight, const int64_t* targets, int dtype, int64_t N,
                int64_t V, int64_t H, int64_t ldh, int64_t ldw, float temperature) {
@@ -1156,7 +1174,7 @@ int reserve_head_lds(Kern kern, const char* what) {
 using namespace trlk;
 
 extern "C" size_t trlk_fused_head_fwd_workspace_bytes(int64_t n_tokens) {
-    return n_tokens > 0 ? size_t(n_tokens) * (kFwdSplits * 4 + 1) * sizeof(float) : 0;
+    return n_tokens > 0 ? size_t(n_tokens) * (fwd_splits(n_tokens) * 4 + 1) * sizeof(float) : 0;
 }
 
 extern "C" size_t trlk_fused_head_stash_bytes(int64_t n_tokens, int64_t vocab, int64_t* out_ld) {
@@ -1210,19 +1228,21 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
     a.inv_t = 1.f / temperature;
     a.softcap = final_logit_softcapping > 0.f ? final_logit_softcapping : 0.f;
     const int n_vt = int((vocab + BM - 1) / BM);
-    a.v_splits = kFwdSplits;
-    a.tiles_per_split = (n_vt + kFwdSplits - 1) / kFwdSplits;
+    int splits = fwd_splits(n_tokens);  // what the workspace was sized for
+    while (splits > 1 && n_vt < 4 * splits) splits /= 2;  // at least 4 vocabulary tiles per workgroup
+    a.v_splits = splits;
+    a.tiles_per_split = (n_vt + splits - 1) / splits;
     a.partial = static_cast<float*>(d_workspace);
-    a.tgt = a.partial + size_t(n_tokens) * kFwdSplits * 4;
+    a.tgt = a.partial + size_t(n_tokens) * splits * 4;
     hipLaunchKernelGGL(head_fill_kernel, dim3(unsigned((n_tokens + 255) / 256)), dim3(256), 0, s, a.tgt, n_tokens, NAN);
     if (int rc = launch_status("fused_head_fwd (fill)")) return rc;
     const int n_tb = int((n_tokens + BN - 1) / BN);
-    const int grid = xcd_patch_grid(n_tb, kFwdSplits);
+    const int grid = xcd_patch_grid(n_tb, splits);
     int rc = dtype == TRLK_BF16 ? launch_head(fused_head_fwd_kernel<TRLK_BF16>, grid, a, s, "fused_head_fwd")
                                 : launch_head(fused_head_fwd_kernel<TRLK_F16>, grid, a, s, "fused_head_fwd");
     if (rc) return rc;
     hipLaunchKernelGGL(head_merge_kernel, dim3(unsigned((n_tokens + 255) / 256)), dim3(256), 0, s, a.partial, a.tgt,
-                       d_targets, int(n_tokens), int(vocab), kFwdSplits, d_out_logp, d_out_entropy, d_out_log_z,
+                       d_targets, int(n_tokens), int(vocab), splits, d_out_logp, d_out_entropy, d_out_log_z,
                        d_out_target_is_max, d_error_flag);
     return launch_status("fused_head_fwd (merge)");
 }
