@@ -559,7 +559,11 @@ def main():
     if not args.no_cpu_baseline:
         del leaf, logits
         torch.cuda.empty_cache()
-        result["cpu_baseline"] = cpu_baseline(w, args.loss_type)
+        base = cpu_baseline(w, args.loss_type, repeats=1)
+        secs = 32 * 512 / base["value"]
+        if secs < 5.0:  # a fast host: the sample grows towards ~10 s of work per run
+            base = cpu_baseline(w, args.loss_type, n_seq=int(min(96, max(32, 32 * 10.0 / secs))) // 8 * 8)
+        result["cpu_baseline"] = base
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))
