@@ -312,6 +312,13 @@ def bench_head(args, w):
                                "and backward; same loss"},
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_head(w),
     }
+    if args.calibrate_copy:
+        dst = torch.empty_like(weight)
+        for _ in range(3):
+            dst.copy_(weight.detach())  # reads and writes V*H*2 bytes each
+        torch.cuda.synchronize()
+        result["calibration_copy_bytes_each_way"] = V * H * 2
+        del dst
     print(json.dumps(result))
 
 

@@ -653,15 +653,23 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
             }
             S[nb] += s;
             U[nb] += u;
-            // target logit: rarely inside this wave's 128 vocabulary rows
+            // target logit: rarely inside this wave's 128 vocabulary rows.  It is selected into one register
+            // and stored once: a conditional store per accumulator held the wave for about 20 us, and a
+            // workgroup that falls behind the others no longer finds the tiles they share in the L2.
             const int64_t rel = tg[nb] - (m0 + wm * WM);
             if (rel >= 0 && rel < WM) {
+                const int want = int(rel) - (lane >> 5) * 4;  // acc_row() without this lane's half-wave offset
+                float tv = 0.f;
+                bool mine = false;
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        if (acc_row(0, mb, r, lane) == int(rel))
-                            a.tgt[n0 + acc_col(wn, nb, lane)] = plain ? acc[mb][nb][r] * zs : acc[mb][nb][r];
+                    for (int r = 0; r < 16; ++r) {
+                        const bool m = (mb * 32 + (r >> 2) * 8 + (r & 3)) == want;
+                        tv = m ? acc[mb][nb][r] : tv;
+                        mine |= m;
+                    }
+                if (mine) a.tgt[n0 + acc_col(wn, nb, lane)] = plain ? tv * zs : tv;
             }
         }
     }
