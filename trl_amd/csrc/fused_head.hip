@@ -93,14 +93,14 @@ struct Operand {
 #ifndef TRLK_HEAD_DIRECT_LDS
 #define TRLK_HEAD_DIRECT_LDS 1
 #endif
-// k-step width of the direct-to-LDS loop per kernel: the short contraction over the hidden size
-// (forward, recompute) gains from the deeper ring of 32-wide steps, the long contractions of the
-// two backward products from 64-wide steps with half as many barriers.
+// k-step width of the direct-to-LDS loop per kernel.  All three use 64-wide steps (two 64 KiB stages, half as
+// many barriers, whole 128-byte lines per row and step); the 32-wide, four-stage ring was only ahead for the
+// short contraction over the hidden size while the forward's workgroups still ran out of step with each other.
 #ifndef TRLK_HEAD_BK_FWD
-#define TRLK_HEAD_BK_FWD 32
+#define TRLK_HEAD_BK_FWD 64
 #endif
 #ifndef TRLK_HEAD_BK_DZ
-#define TRLK_HEAD_BK_DZ 32
+#define TRLK_HEAD_BK_DZ 64
 #endif
 #ifndef TRLK_HEAD_BK_GEMM
 #define TRLK_HEAD_BK_GEMM 64
