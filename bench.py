@@ -33,6 +33,11 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # HBM bytes per K3 launch from rocprofv3 FETCH_SIZE / WRITE_SIZE (two --pmc runs of this file, scaled by a plain
 # device copy of known size: FETCH x 2.000, WRITE x 1.000 KiB); the inputs are seeded, so the figure is stable.
 MEASURED_K3_TRAFFIC_BYTES = {("grpo_c3", "dapo"): (10116130 + 19461194) * 1024}
+# The same two counters for one forward launch of the fused head with its stash stores (FETCH_SIZE varies between
+# 36.6e6 and 44.0e6 over the launches of a run; the mean is used): what leaves the L2s towards memory.  The writes
+# are the stash plus the partial results; the reads are the operand tiles that miss the L2 of their XCD, about 60
+# times the 1.3 GB of the two operands.
+MEASURED_HEAD_FWD_TRAFFIC_BYTES = {"head_c5": (2 * 40600000 + 19497000) * 1024}
 
 WORKLOADS = {
     # name: (n_seq, completion_len, vocab, temperature, group_size, min_len)
@@ -297,7 +302,8 @@ def bench_head(args, w):
         # two sub-0.1 ms helper kernels)
         "roofline": {"bound": "mfma", "kernel": "fused_head_fwd_kernel", "achieved": fwd_tf,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": fwd_tf / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None, "algorithmic_flop": flop, "avg_launch_ms": fwd_ms,
+                     "traffic": MEASURED_HEAD_FWD_TRAFFIC_BYTES.get(args.workload) if stash else None,
+                     "algorithmic_flop": flop, "avg_launch_ms": fwd_ms,
                      "forward_plus_backward": {"achieved": total_tf, "frac": total_tf / MFMA_BF16_PEAK_TFLOPS,
                                                "executed_flop": flop + bwd_flop, "ms": fwd_ms + bwd_ms}},
         "kernels": dict(kernels, **{
