@@ -901,24 +901,39 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
         tg[j] = ok ? a.targets[tok] - a.c0 : -1;  // chunk-local target row
     }
     const bool contiguous = COLS && col[0] >= 0 && col[1] == col[0] + 1 && col[2] == col[0] + 2 && col[3] == col[0] + 3;
+    // The loads of kSdzBatch row pairs are issued before any of their results is used or stored: with
+    // one pair (32 bytes per lane) in flight the sweep is bound by memory latency, not bandwidth.
+    constexpr int kIters = kSdzRows / (8 * kSdzPairsPerWave), kSdzBatch = 4;
+    static_assert(kIters % kSdzBatch == 0, "row pairs per lane");
+    f32x4 yb[kSdzBatch][2];
 #pragma unroll
-    for (int i = 0; i < kSdzRows / (8 * kSdzPairsPerWave); ++i) {
+    for (int i = 0; i < kIters; ++i) {
+        if (i % kSdzBatch == 0) {
+#pragma unroll
+            for (int ii = 0; ii < kSdzBatch; ++ii)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int row = r0 + 2 * (wave * kSdzPairsPerWave + sub + 4 * kSdzPairsPerWave * (i + ii)) + h;
+                    const float* srow = a.stash_in + int64_t(a.c0 + row) * a.ld_stash;
+                    f32x4 y4;
+                    if constexpr (!COLS) {
+                        y4 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(srow + n0 + tl0));
+                    } else if (contiguous) {  // the usual case: the lane's 4 tokens were neighbours in the forward too
+                        typedef float f32x4_dword_aligned __attribute__((ext_vector_type(4), aligned(4)));
+                        y4 = *reinterpret_cast<const f32x4_dword_aligned*>(srow + col[0]);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) y4[j] = col[j] >= 0 ? __builtin_nontemporal_load(srow + col[j]) : 0.f;
+                    }
+                    yb[ii][h] = y4;
+                }
+        }
         const int rl = 2 * (wave * kSdzPairsPerWave + sub + 4 * kSdzPairsPerWave * i);  // row pair rl, rl + 1 of the 64
         float d[2][4];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int row = r0 + rl + h;
-            const float* srow = a.stash_in + int64_t(a.c0 + row) * a.ld_stash;
-            f32x4 y4;
-            if constexpr (!COLS) {
-                y4 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(srow + n0 + tl0));
-            } else if (contiguous) {  // the usual case: the lane's 4 tokens were neighbours in the forward too
-                typedef float f32x4_dword_aligned __attribute__((ext_vector_type(4), aligned(4)));
-                y4 = *reinterpret_cast<const f32x4_dword_aligned*>(srow + col[0]);
-            } else {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) y4[j] = col[j] >= 0 ? __builtin_nontemporal_load(srow + col[j]) : 0.f;
-            }
+            const f32x4 y4 = yb[i % kSdzBatch][h];
             const float bias = (!plain && a.bias != nullptr && row < rows) ? a.bias[a.c0 + row] : 0.f;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
