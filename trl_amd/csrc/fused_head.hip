@@ -1182,20 +1182,25 @@ int launch_head(Kern kern, int grid, const Args& a, hipStream_t s, const char* w
 
 template <typename Kern>
 int reserve_head_lds(Kern kern, const char* what) {
-    static thread_local const void* configured[16] = {};
-    // dynamic LDS above 64 KiB has to be allowed per kernel once
-    bool done = false;
-    for (const void* c : configured) done |= (c == reinterpret_cast<const void*>(kern));
-    if (!done) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kHeadLdsBytes);
-        if (e != hipSuccess) return fail(int(e), "%s: cannot reserve %d bytes of LDS: %s", what, kHeadLdsBytes, hipGetErrorString(e));
-        for (const void*& c : configured)
-            if (c == nullptr) {
-                c = reinterpret_cast<const void*>(kern);
-                break;
-            }
-    }
+    // dynamic LDS above 64 KiB has to be allowed per kernel and device once
+    struct Done {
+        const void* kern;
+        int device;
+    };
+    static thread_local Done configured[32] = {};
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) device = 0;
+    const void* key = reinterpret_cast<const void*>(kern);
+    for (const Done& c : configured)
+        if (c.kern == key && c.device == device) return TRLK_OK;
+    const hipError_t e = hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, kHeadLdsBytes);
+    if (e != hipSuccess) return fail(int(e), "%s: cannot reserve %d bytes of LDS: %s", what, kHeadLdsBytes, hipGetErrorString(e));
+    for (Done& c : configured)
+        if (c.kern == nullptr) {
+            c.kern = key;
+            c.device = device;
+            break;
+        }
     return TRLK_OK;
 }
 
