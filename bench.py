@@ -5,7 +5,7 @@ One "step" = one pass of the hot path over one synthetic batch that is already r
   K1  log-prob + entropy forward over bf16 logits [64, 1024, 151936] (temperature 0.9)
   K2  GRPO loss + metrics + d loss/d logp on [64, 1024]
   K3  recompute backward writing dlogits [64, 1024, 151936] bf16
-(BASELINE.json config "GRPO loss fwd+bwd").  Prints ONE JSON line.
+(benchmark configuration "GRPO loss fwd+bwd").  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--loss-type dapo] [--no-cpu-baseline]
 
@@ -192,7 +192,7 @@ HEAD_CHUNK = 32768
 
 
 def bench_head(args, w):
-    """BASELINE.json config 5: the logits are never materialised.  Step = fused head forward, GRPO loss,
+    """benchmark configuration 5: the logits are never materialised.  Step = fused head forward, GRPO loss,
     fused head backward (dHidden and dW)."""
     import trl_amd
     from trl_amd import ops

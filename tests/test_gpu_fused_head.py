@@ -312,7 +312,7 @@ def test_fp64_operands_are_rejected_loudly(amd):
 
 
 def test_real_head_shape_row_subsample(amd):
-    """Qwen2.5-7B head shape of BASELINE config 5 (H = 3584, V = 151936) on 256 tokens."""
+    """Qwen2.5-7B head shape of benchmark configuration 5 (H = 3584, V = 151936) on 256 tokens."""
     g = torch.Generator().manual_seed(55)
     n, h, v = 256, 3584, 151936
     hidden = torch.randn(n, h, generator=g).bfloat16()
@@ -328,7 +328,7 @@ def test_real_head_shape_row_subsample(amd):
 
 
 def test_real_head_shape_paths_agree(amd, monkeypatch):
-    """BASELINE config 5's head shape on 4096 tokens (16 token blocks, 594 vocabulary tiles, 5 backward chunks, a
+    """benchmark configuration 5's head shape on 4096 tokens (16 token blocks, 594 vocabulary tiles, 5 backward chunks, a
     prefix mask on the upstream gradient): the stash + token-dropping path gives the recompute path's results, and
     size-independent properties hold -- rows without an upstream gradient get none, dW sums to zero over the
     vocabulary (softmax gradients are orthogonal to the constant shift) and the probabilities behind the entropy are

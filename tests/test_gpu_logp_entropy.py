@@ -99,7 +99,7 @@ def test_entropy_reference_unit_test_shapes(amd, dtype, shape):
                                    rtol=1e-5, atol=1e-5)
 
 
-# ------------------------------------------------------------------ BASELINE config 1 at full size
+# ------------------------------------------------------------------ benchmark configuration 1 at full size
 def test_config1_full_size_fp32(amd):
     g = torch.Generator().manual_seed(0)
     logits = 3.0 * torch.randn(8, 256, 32000, generator=g)
@@ -238,7 +238,7 @@ def test_bitwise_reproducible(amd):
 
 # ------------------------------------------------------------------ properties at the benchmark shape
 def test_full_size_properties_config3_shape(amd):
-    """BASELINE config 3 shape (64 x 1024 rows, V = 151936, bf16) is too large for the CPU oracle:
+    """benchmark configuration 3 shape (64 x 1024 rows, V = 151936, bf16) is too large for the CPU oracle:
     check a row subsample against the oracle and size-independent properties on all rows."""
     B, T, V, temp = 64, 1024, 151936, 0.9
     g = torch.Generator(device=DEV).manual_seed(3)
@@ -280,7 +280,7 @@ def test_full_size_properties_config3_shape(amd):
 
 
 def test_long_context_config4_saved_state_and_properties(amd):
-    """BASELINE config 4 (32 x 4096 rows, V = 151936, bf16: 39.8 GB of logits): what the forward keeps for the
+    """benchmark configuration 4 (32 x 4096 rows, V = 151936, bf16: 39.8 GB of logits): what the forward keeps for the
     backward is a few bytes per row (the reference keeps a [T, V] log-softmax per sequence), masked rows and the
     dropped last position get exactly zero gradient, and sum_v dlogits = 0 on the active rows."""
     B, T, V = 32, 4096, 151936

@@ -254,7 +254,7 @@ def test_group_advantages(amd):
             want = oracle.group_advantages(r, G, mode)
             torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
     assert torch.equal(amd.group_advantages(r.to(DEV), 8, "group").cpu()[8:24], torch.zeros(16))
-    # Bernoulli rewards of BASELINE config 4 (G = 16): all-equal groups give exactly zero
+    # Bernoulli rewards of benchmark configuration 4 (G = 16): all-equal groups give exactly zero
     rb = (torch.rand(32, generator=g) < 0.3).float()
     torch.testing.assert_close(amd.group_advantages(rb.to(DEV), 16).cpu(), oracle.group_advantages(rb, 16), rtol=1e-5, atol=1e-6)
 
@@ -425,7 +425,7 @@ def test_golden_dpo_compute_loss(amd):
 
 
 def test_dpo_against_oracle_config2_shape_subsample(amd):
-    """BASELINE config 2 layout (prompt mask + right padding, [chosen; rejected]) on a reduced
+    """benchmark configuration 2 layout (prompt mask + right padding, [chosen; rejected]) on a reduced
     sequence count/length at the real vocabulary; bf16 logits vs fp32-op-math oracle."""
     g = torch.Generator().manual_seed(24)
     P, L, V = 2, 48, 128256
@@ -455,7 +455,7 @@ def test_dpo_against_oracle_config2_shape_subsample(amd):
 
 
 def test_dpo_full_size_config2_closed_form_and_properties(amd):
-    """BASELINE config 2 at full size (64 x 2048 x 128256 bf16, 32 pairs, prompt + right padding): with the
+    """benchmark configuration 2 at full size (64 x 2048 x 128256 bf16, 32 pairs, prompt + right padding): with the
     reference log-probs equal to the policy's the loss is ln 2 and every pair carries the gradient -beta/(2P) on
     the chosen and +beta/(2P) on the rejected sequence; rows outside the shifted completion mask and the last
     position get exactly zero gradient; sum_v dlogits = 0 on the others."""
