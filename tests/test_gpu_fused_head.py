@@ -410,3 +410,26 @@ def test_golden_sft_chunked_nll(amd):
     loss, correct, ent, nv = _chunked_cross_entropy_loss(dhs, dw, 256, labels=torch.full((2, 5), -100, device=DEV))
     loss.backward()
     assert float(loss) == 0.0 and int(nv) == 0 and torch.count_nonzero(dw.grad) == 0
+
+
+def test_target_logit_every_tile_position(amd):
+    """The forward picks the target's logit out of the accumulators of the tile that holds it.  Every pair of
+    (token position inside its 256-token block, vocabulary row inside its 256-row tile) occurs once here, in both
+    vocabulary tiles and in a ragged last tile; a wrong accumulator would be off by the spread of the logits
+    (about 1), the bar is the 2e-3 of bf16 operands against fp32 op-math."""
+    from trl_amd import ops
+
+    n_blocks, H, V = 256, 64, 512 + 40
+    N = 256 * n_blocks
+    g = torch.Generator().manual_seed(11)
+    hidden = torch.randn(N, H, generator=g).bfloat16()
+    weight = (0.2 * torch.randn(V, H, generator=g)).bfloat16()
+    n = torch.arange(N)
+    col, blk = n % 256, n // 256
+    labels = (col + blk) % 256 + 256 * (blk % 2)          # every (column, row) pair, alternating tiles
+    labels[::517] = 512 + (n[::517] % 40)                 # and some targets in the ragged third tile
+    want = F.log_softmax(hidden.double() @ weight.double().t(), -1).gather(-1, labels[:, None]).squeeze(-1).float()
+    for stash in (False, True):
+        out = ops.fused_head_fwd(hidden.to(DEV), weight.to(DEV), labels.to(DEV), 1.0, 0.0, 1.0, None, stash)
+        torch.testing.assert_close(out[0].cpu(), want, atol=2e-3, rtol=0)
+    amd.check_device_errors()  # no index was out of range
