@@ -269,6 +269,35 @@ int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, const int64_
                         void* d_out_dweight, float* d_out_dbias, void* d_workspace, size_t workspace_bytes,
                         trlk_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------
+ * K7  GRPO loss gradient straight from the logits: one read and one write of the logits-sized
+ * data instead of K1 + K3's two reads and one write.  Stands in for the whole chain
+ * `_get_per_token_logps_and_entropies` -> `_compute_loss` -> `loss.backward()` down to dlogits
+ * (trl/trainer/grpo_trainer.py:1514-1532, 3026-3150) for the token-level loss types, where the
+ * gradient coefficient of a token depends only on its own log-prob, on per-token inputs and on
+ * normalisers known from the mask:
+ *   d_row_scale fp32 [n_seq] = d loss / d (masked token loss of that sequence), e.g. 1 / num_items for dapo;
+ *   the other per-token inputs, the policy terms and their parameters are those of trlk_grpo_loss.
+ * 16-bit logits only, vocab % 8 == 0 and vocab <= trlk_grpo_fused_max_vocab(dtype) (a row is held
+ * in the registers of one workgroup), rows 16-byte aligned.  Outputs: log-prob, entropy and lse of
+ * every row of the completion mask (0 for the others, which are not read), and the full
+ * [n_seq, out_rows_per_seq, vocab] gradient laid out as trlk_logp_entropy_bwd writes it, for an
+ * upstream gradient of 1 on the loss.  trlk_scale_unless_one multiplies such a buffer by a device
+ * scalar, and launches an empty kernel when that scalar is exactly 1.
+ */
+int64_t trlk_grpo_fused_max_vocab(int dtype);
+int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t n_seq, int64_t rows_per_seq, int64_t vocab,
+                            int64_t seq_stride, int64_t row_stride, const int64_t* d_index, float temperature,
+                            const float* d_old_logp, const float* d_ref_logp, const float* d_advantages,
+                            int64_t adv_stride_b, int64_t adv_stride_t, const float* d_mask,
+                            const float* d_token_weight, const float* d_seq_coef, const float* d_row_scale,
+                            int policy_term, float epsilon_low, float epsilon_high, float delta, float beta,
+                            int use_bias_correction_kl, float sapo_temperature_pos, float sapo_temperature_neg,
+                            float* d_out_logp, float* d_out_entropy, float* d_out_lse, void* d_dlogits,
+                            int64_t out_rows_per_seq, int64_t out_row_offset, int64_t out_seq_stride,
+                            int64_t out_row_stride, int32_t* d_error_flag, trlk_stream_t stream);
+int trlk_scale_unless_one(void* d_data, int dtype, int64_t n_elems, const float* d_scale, trlk_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,161 @@
+"""GPU parity of the single-pass GRPO operator (logits -> loss + dlogits in one kernel pass) against the
+two-pass path (K1 log-probs, [B, T] loss kernel, K3 gradient), which the other GPU tests pin to the golden
+vectors and the oracle.  Bars: loss and metrics 1e-5 relative, log-probs / entropies 1e-5 abs on the rows of the
+mask (the other rows are 0 by contract), dlogits 2e-3 relative L2 (both sides round to bf16) with the rows
+outside the mask exactly zero."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def amd():
+    import trl_amd
+
+    return trl_amd
+
+
+def _inputs(B, K, V, dtype=torch.bfloat16, seed=0, extra_rows=3):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    L = K + extra_rows
+    logits = (2.0 * torch.randn((B, L, V), generator=g, device=DEV)).to(dtype)
+    ids = torch.randint(0, V, (B, K), generator=g, device=DEV)
+    lengths = torch.randint(1, K + 1, (B,), generator=g, device=DEV)
+    lengths[0] = 0  # a sequence without any active token
+    mask = (torch.arange(K, device=DEV)[None] < lengths[:, None]).long()
+    adv = torch.randn((B,), generator=g, device=DEV)
+    return logits, ids, mask, adv, g
+
+
+def _two_pass(amd, logits, ids, mask, adv, temperature, **kw):
+    leaf = logits.detach().clone().requires_grad_(True)
+    logp, ent = amd.per_token_logps_and_entropies(leaf, ids, ids.shape[1], temperature)
+    loss, metrics = amd.grpo_loss(logp, adv, mask, entropies=ent, **kw)
+    return leaf, loss, metrics, logp.detach(), ent.detach()
+
+
+def _rel_l2(a, b):
+    a, b = a.double(), b.double()
+    return float((a - b).norm() / b.norm().clamp(min=1e-30))
+
+
+@pytest.mark.parametrize("loss_type", ["dapo", "grpo", "bnpo", "dr_grpo", "cispo", "sapo"])
+@pytest.mark.parametrize("beta", [0.0, 0.04])
+def test_matches_two_pass(amd, loss_type, beta):
+    B, K, V, T = 8, 32, 4096, 0.9
+    logits, ids, mask, adv, g = _inputs(B, K, V, seed=3)
+    with torch.no_grad():
+        base, _ = amd.per_token_logps_and_entropies(logits, ids, K, T)
+    old = base + 0.3 * torch.randn(base.shape, generator=g, device=DEV)
+    ref = base + 0.1 * torch.randn(base.shape, generator=g, device=DEV)
+    kw = dict(old_per_token_logps=old, ref_per_token_logps=ref if beta else None, loss_type=loss_type, epsilon_low=0.2,
+              epsilon_high=0.28, beta=beta, max_completion_length=K, num_items_in_batch=mask.sum().float(),
+              grad_accum_steps=2.0)
+    leaf, loss2, met2, lp2, ent2 = _two_pass(amd, logits, ids, mask, adv, T, **kw)
+    loss2.backward()
+    leaf1 = logits.detach().clone().requires_grad_(True)
+    loss1, met1, lp1, ent1 = amd.grpo_loss_from_logits(leaf1, ids, adv, mask, temperature=T, **kw)
+    loss1.backward()
+    torch.testing.assert_close(loss1, loss2, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(met1, met2, rtol=1e-5, atol=1e-6, equal_nan=True)
+    m = mask.bool()
+    torch.testing.assert_close(lp1[m], lp2[m], rtol=0, atol=1e-5)
+    torch.testing.assert_close(ent1[m], ent2[m], rtol=0, atol=1e-5)
+    assert float(lp1[~m].abs().max()) == 0.0 and float(ent1[~m].abs().max()) == 0.0
+    g1, g2 = leaf1.grad, leaf.grad
+    assert g1.shape == logits.shape and g1.dtype == logits.dtype
+    assert _rel_l2(g1, g2) < 2e-3
+    # rows outside the window or the mask: exactly zero on both sides
+    full_mask = torch.zeros(logits.shape[:2], dtype=torch.bool, device=DEV)
+    start = logits.shape[1] - 1 - K
+    full_mask[:, start:start + K] = m
+    assert float(g1[~full_mask].abs().max()) == 0.0 and float(g2[~full_mask].abs().max()) == 0.0
+    # every gradient row sums to zero up to the rounding of its 4096 bf16 entries
+    assert float(g1.float().sum(-1).abs().max()) < 1e-3
+    amd.check_device_errors()
+
+
+def test_upstream_gradient_scales(amd):
+    B, K, V = 4, 16, 2048
+    logits, ids, mask, adv, _ = _inputs(B, K, V, seed=5)
+    kw = dict(loss_type="dapo", num_items_in_batch=mask.sum().float(), temperature=1.0)
+    a = logits.detach().clone().requires_grad_(True)
+    amd.grpo_loss_from_logits(a, ids, adv, mask, **kw)[0].backward()
+    b = logits.detach().clone().requires_grad_(True)
+    (amd.grpo_loss_from_logits(b, ids, adv, mask, **kw)[0] * 0.25).backward()
+    torch.testing.assert_close(b.grad.float(), a.grad.float() * 0.25, rtol=1e-2, atol=0)  # 0.25 is exact in bf16
+    assert _rel_l2(b.grad.float(), a.grad.float() * 0.25) == 0.0
+
+
+def test_fp16_and_token_weight_and_per_token_advantages(amd):
+    B, K, V = 4, 24, 1024
+    logits, ids, mask, _, g = _inputs(B, K, V, dtype=torch.float16, seed=7)
+    adv = torch.randn((B, K), generator=g, device=DEV)
+    tw = torch.rand((B, K), generator=g, device=DEV)
+    kw = dict(loss_type="grpo", token_weight=tw, delta=1.5, epsilon_low=0.1, epsilon_high=0.3)
+    with torch.no_grad():
+        base, _ = amd.per_token_logps_and_entropies(logits, ids, K, 0.7)
+    kw["old_per_token_logps"] = base + 0.5 * torch.randn(base.shape, generator=g, device=DEV)
+    leaf, loss2, met2, _, _ = _two_pass(amd, logits, ids, mask, adv, 0.7, **kw)
+    loss2.backward()
+    leaf1 = logits.detach().clone().requires_grad_(True)
+    loss1, met1, _, _ = amd.grpo_loss_from_logits(leaf1, ids, adv, mask, temperature=0.7, **kw)
+    loss1.backward()
+    torch.testing.assert_close(loss1, loss2, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(met1, met2, rtol=1e-5, atol=1e-6, equal_nan=True)
+    assert _rel_l2(leaf1.grad, leaf.grad) < 2e-3
+
+
+def test_real_vocabulary_and_limits(amd):
+    """A row of 151936 logits (19 vectors per lane, the last one ragged) and the largest supported row."""
+    for V in (151936, 163840):
+        B, K = 2, 6
+        logits, ids, mask, adv, _ = _inputs(B, K, V, seed=V % 97, extra_rows=1)
+        mask[:] = 1
+        mask[1, 4:] = 0
+        ids[0, 0], ids[0, 1] = 0, V - 1
+        kw = dict(loss_type="bnpo", beta=0.0)
+        leaf, loss2, met2, lp2, ent2 = _two_pass(amd, logits, ids, mask, adv, 0.9, **kw)
+        loss2.backward()
+        leaf1 = logits.detach().clone().requires_grad_(True)
+        loss1, met1, lp1, ent1 = amd.grpo_loss_from_logits(leaf1, ids, adv, mask, temperature=0.9, **kw)
+        loss1.backward()
+        m = mask.bool()
+        torch.testing.assert_close(loss1, loss2, rtol=1e-5, atol=1e-7)
+        torch.testing.assert_close(lp1[m], lp2[m], rtol=0, atol=1e-5)
+        torch.testing.assert_close(ent1[m], ent2[m], rtol=0, atol=1e-5)
+        assert _rel_l2(leaf1.grad, leaf.grad) < 2e-3
+    amd.check_device_errors()
+
+
+def test_unsupported_configurations_raise(amd):
+    logits, ids, mask, adv, _ = _inputs(2, 4, 1024)
+    assert amd.grpo_single_pass_supported(logits)
+    assert not amd.grpo_single_pass_supported(logits.float())
+    assert not amd.grpo_single_pass_supported(logits, "vespo")
+    assert not amd.grpo_single_pass_supported(logits, "dapo", "sequence")
+    assert not amd.grpo_single_pass_supported(logits, entropy_coef=0.01)
+    assert not amd.grpo_single_pass_supported(logits[..., :1020])
+    big = torch.empty((1, 2, amd.ops.grpo_fused_max_vocab(torch.bfloat16) + 8), dtype=torch.bfloat16, device=DEV)
+    assert not amd.grpo_single_pass_supported(big)
+    with pytest.raises(NotImplementedError):
+        amd.grpo_loss_from_logits(logits.float(), ids, adv, mask, loss_type="bnpo")
+    with pytest.raises(KeyError):
+        amd.grpo_loss_from_logits(logits, ids, adv, mask, loss_type="dapo")
+    with pytest.raises(KeyError):
+        amd.grpo_loss_from_logits(logits, ids, adv, mask, loss_type="bnpo", beta=0.1)
+
+
+def test_index_out_of_range_is_flagged(amd):
+    logits, ids, mask, adv, _ = _inputs(2, 4, 1024, seed=9)
+    mask[:] = 1
+    ids[1, 2] = 1024
+    leaf = logits.detach().clone().requires_grad_(True)
+    loss, _, lp, _ = amd.grpo_loss_from_logits(leaf, ids, adv, mask, loss_type="bnpo")
+    assert math.isnan(float(lp[1, 2]))
+    with pytest.raises(IndexError):
+        amd.check_device_errors()

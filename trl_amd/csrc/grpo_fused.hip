@@ -1,0 +1,292 @@
+// K7: from the logits straight to the GRPO loss gradient, one read and one write of the logits-sized data.
+//
+// The two-pass path reads the logits twice (K1 for the log-probs, K3 for the gradient) because the loss sits
+// between them.  For the token-level GRPO losses the gradient coefficient of a token depends only on that
+// token's own log-prob, on per-token inputs (old / reference log-probs, advantage, mask, weight) and on
+// normalisers that are known from the mask before any logit is read.  A 1024-lane workgroup can hold a whole
+// vocabulary row of 16-bit logits in registers (up to kMaxVec 16-byte vectors per lane), so one workgroup
+// per row loads the row once, reduces it to (lse, entropy, target logit), evaluates the token's loss terms
+// with the same device functions as the [B, T]-sized loss kernel, and writes the row's dlogits from the
+// registers.  Rows outside the completion mask are never read: their gradient row is zero-filled and their
+// outputs are 0.
+#include "common.hpp"
+#include "grpo_token.hpp"
+
+namespace trlk {
+namespace {
+
+constexpr int kFThreads = 1024;
+constexpr int kFWaves = kFThreads / kWave;
+constexpr int kMaxVec = 20;  // 16-byte vectors of a row per lane: rows of up to 20 * 1024 * 8 = 163840 logits
+
+struct FusedArgs {
+    const void* logits;
+    int64_t rows_per_seq, vocab, seq_stride, row_stride;
+    const int64_t* index;  // [n_seq * rows_per_seq]
+    float temperature;
+    const float *old_logp, *ref_logp, *adv, *mask, *token_weight, *row_scale, *seq_coef;
+    int64_t adv_stride_b, adv_stride_t;
+    int policy_term;
+    float eps_low, eps_high, delta, beta;
+    int bias_kl;
+    float sapo_tau_pos, sapo_tau_neg;
+    float *out_logp, *out_entropy, *out_lse;
+    void* dlogits;
+    int64_t out_rows_per_seq, out_row_offset, out_seq_stride, out_row_stride;
+    int32_t* error_flag;
+};
+
+template <int DT>
+__global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
+    typedef Elem<DT> E;
+    typedef typename E::type T;
+    constexpr int EPV = E::EPV;
+    __shared__ float red[3][kFWaves];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int64_t orow = blockIdx.x;
+    const int64_t b = orow / a.out_rows_per_seq;
+    const int64_t to = orow - b * a.out_rows_per_seq;
+    const int64_t t = to - a.out_row_offset;
+    const bool inside = t >= 0 && t < a.rows_per_seq;
+    const int64_t row = b * a.rows_per_seq + (inside ? t : 0);
+    const int nv = int(a.vocab / EPV);
+    u32x4* op = reinterpret_cast<u32x4*>(static_cast<T*>(a.dlogits) + b * a.out_seq_stride + to * a.out_row_stride);
+    const float m = inside ? a.mask[row] : 0.f;
+    if (m == 0.f) {  // no gradient reaches this row: zero-fill, nothing is read
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        for (int v = tid; v < nv; v += kFThreads) __builtin_nontemporal_store(z, op + v);
+        if (inside && tid == 0) {
+            a.out_logp[row] = 0.f;
+            a.out_entropy[row] = 0.f;
+            a.out_lse[row] = 0.f;
+        }
+        return;
+    }
+    const T* base = static_cast<const T*>(a.logits) + b * a.seq_stride + t * a.row_stride;
+    const u32x4* vp = reinterpret_cast<const u32x4*>(base);
+    u32x4 q[kMaxVec];
+#pragma unroll
+    for (int j = 0; j < kMaxVec; ++j) {
+        const int v = j * kFThreads + tid;
+        if (v < nv) q[j] = __builtin_nontemporal_load(vp + v);
+    }
+    // the per-row scalars travel while the row does
+    const int64_t idx = a.index[row];
+    const bool idx_ok = idx >= 0 && idx < a.vocab;
+    const float x_t = idx_ok ? E::load1(base + idx) : NAN;
+    const float A = a.adv[b * a.adv_stride_b + t * a.adv_stride_t];
+    const float old_lp = a.old_logp ? a.old_logp[row] : 0.f;
+    const float ref_lp = a.beta != 0.f ? a.ref_logp[row] : 0.f;
+    const float w = a.token_weight ? a.token_weight[row] : 1.f;
+    const float coef = a.seq_coef ? a.seq_coef[b] : 0.f;
+    const float scale = a.row_scale[b];
+    const float inv_t = 1.f / a.temperature, c = kLog2e * inv_t;
+
+    // lane maximum, then the lane's sums relative to it
+    float lm = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < kMaxVec; ++j)
+        if (j * kFThreads + tid < nv) {
+            float x[EPV];
+            E::unpack(q[j], x);
+#pragma unroll
+            for (int i = 0; i < EPV; ++i) lm = fmaxf(lm, x[i]);
+        }
+    // (the compiler must not keep the unpacked values of one pass alive for the next: 152 floats per lane)
+#pragma unroll
+    for (int j = 0; j < kMaxVec; ++j) asm volatile("" : "+v"(q[j]));
+    float M = wave_max(lm);
+    if (lane == 0) red[0][wave] = M;
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kFWaves; ++k) M = fmaxf(M, red[0][k]);
+    const float mc = M * c;
+    float s = 0.f, u = 0.f;
+#pragma unroll
+    for (int j = 0; j < kMaxVec; ++j)
+        if (j * kFThreads + tid < nv) {
+            float x[EPV];
+            E::unpack(q[j], x);
+#pragma unroll
+            for (int i = 0; i < EPV; ++i) {
+                const float e = fast_exp2(fmaf(x[i], c, -mc));
+                s += e;
+                u = fmaf(e, x[i], u);
+            }
+        }
+#pragma unroll
+    for (int j = 0; j < kMaxVec; ++j) asm volatile("" : "+v"(q[j]));
+    s = wave_sum(s);
+    u = wave_sum(u);
+    if (lane == 0) {
+        red[1][wave] = s;
+        red[2][wave] = u;
+    }
+    __syncthreads();
+    float S = 0.f, U = 0.f;
+#pragma unroll
+    for (int k = 0; k < kFWaves; ++k) {
+        S += red[1][k];
+        U += red[2][k];
+    }
+    const float lse2 = mc + __builtin_amdgcn_logf(S);  // log2 of sum exp(z), z = x / T
+    const float lse = lse2 * kLn2;
+    const float ent = lse - (U / S) * inv_t;
+    const float lp = x_t * inv_t - lse;
+    if (tid == 0) {
+        a.out_logp[row] = lp;
+        a.out_entropy[row] = ent;
+        a.out_lse[row] = lse;
+        if (!idx_ok && a.error_flag) atomicOr(a.error_flag, TRLK_FLAG_INDEX_OUT_OF_RANGE);
+    }
+    // the token's loss terms -> d loss / d logp, already normalised
+    const float c_raw = a.old_logp ? expf(lp - old_lp) : 1.f;
+    const PolicyTerm p = policy_term(a, c_raw, A, lp, coef);
+    float pl, kl, g_lnc, g_lp;
+    grpo_token_terms(a, p, c_raw, lp, w, ref_lp, pl, kl, g_lnc, g_lp);
+    float g = (g_lp + g_lnc) * m * scale;
+    if (!idx_ok) g = 0.f;  // an invalid index leaves a zero row (its log-prob is NaN and the flag is set)
+    const float a0 = -g * inv_t;
+    // dlogits[v] = -g p_v / T (+ g / T at the target), p_v = 2^(x c - lse2)
+#pragma unroll
+    for (int j = 0; j < kMaxVec; ++j) {
+        const int v = j * kFThreads + tid;
+        if (v < nv) {
+            float x[EPV], d[EPV];
+            E::unpack(q[j], x);
+#pragma unroll
+            for (int i = 0; i < EPV; ++i) d[i] = a0 * fast_exp2(fmaf(x[i], c, -lse2));
+            __builtin_nontemporal_store(E::pack(d), op + v);
+        }
+    }
+    // one-hot term: the lane that stored the target's vector rewrites that element (same lane, same
+    // address: ordered after its first store)
+    if (idx_ok && int((idx / EPV) % kFThreads) == tid) {
+        T* out = reinterpret_cast<T*>(op);
+        E::store1(out + idx, a0 * fast_exp2(fmaf(x_t, c, -lse2)) + g * inv_t);
+    }
+}
+
+// data *= *scale over 16-byte vectors, unless the scale is exactly 1 (then nothing is read or written).
+template <int DT>
+__global__ __launch_bounds__(256) void scale_unless_one_kernel(u32x4* data, int64_t n_vec, const float* scale) {
+    typedef Elem<DT> E;
+    const float sc = *scale;
+    if (sc == 1.f) return;
+    for (int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x; v < n_vec; v += int64_t(gridDim.x) * 256) {
+        float x[E::EPV];
+        E::unpack(data[v], x);
+#pragma unroll
+        for (int i = 0; i < E::EPV; ++i) x[i] *= sc;
+        data[v] = E::pack(x);
+    }
+}
+
+}  // namespace
+}  // namespace trlk
+
+using namespace trlk;
+
+extern "C" int trlk_scale_unless_one(void* d_data, int dtype, int64_t n_elems, const float* d_scale, trlk_stream_t stream) {
+    clear_error();
+    TRLK_REQUIRE(dtype == TRLK_BF16 || dtype == TRLK_F16, TRLK_ERR_BAD_DTYPE, "scale_unless_one: 16-bit data only");
+    TRLK_REQUIRE(n_elems >= 0 && n_elems % 8 == 0, TRLK_ERR_BAD_SHAPE, "scale_unless_one: element count must be a multiple of 8");
+    if (n_elems == 0) return TRLK_OK;
+    TRLK_REQUIRE(d_data && d_scale && reinterpret_cast<uintptr_t>(d_data) % 16 == 0, TRLK_ERR_NULL_POINTER,
+                 "scale_unless_one: null or misaligned pointer");
+    const int64_t n_vec = n_elems / 8;
+    const unsigned grid = unsigned(n_vec < 256 * 8192 ? (n_vec + 255) / 256 : 8192);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == TRLK_BF16)
+        hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_BF16>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, d_scale);
+    else
+        hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_F16>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, d_scale);
+    return launch_status("scale_unless_one");
+}
+
+extern "C" int64_t trlk_grpo_fused_max_vocab(int dtype) {
+    return dtype == TRLK_BF16 || dtype == TRLK_F16 ? int64_t(kMaxVec) * kFThreads * 8 : 0;
+}
+
+extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t n_seq, int64_t rows_per_seq, int64_t vocab,
+                                       int64_t seq_stride, int64_t row_stride, const int64_t* d_index, float temperature,
+                                       const float* d_old_logp, const float* d_ref_logp, const float* d_advantages,
+                                       int64_t adv_stride_b, int64_t adv_stride_t, const float* d_mask,
+                                       const float* d_token_weight, const float* d_seq_coef, const float* d_row_scale,
+                                       int policy_term, float epsilon_low, float epsilon_high, float delta, float beta,
+                                       int use_bias_correction_kl, float sapo_temperature_pos, float sapo_temperature_neg,
+                                       float* d_out_logp, float* d_out_entropy, float* d_out_lse, void* d_dlogits,
+                                       int64_t out_rows_per_seq, int64_t out_row_offset, int64_t out_seq_stride,
+                                       int64_t out_row_stride, int32_t* d_error_flag, trlk_stream_t stream) {
+    clear_error();
+    TRLK_REQUIRE(dtype == TRLK_BF16 || dtype == TRLK_F16, TRLK_ERR_BAD_DTYPE,
+                 "grpo_fused: 16-bit logits only (dtype code %d); use the two-pass path", dtype);
+    TRLK_REQUIRE(n_seq >= 0 && rows_per_seq >= 0 && vocab >= 1, TRLK_ERR_BAD_SHAPE, "grpo_fused: bad sizes");
+    TRLK_REQUIRE(vocab % 8 == 0 && vocab <= trlk_grpo_fused_max_vocab(dtype), TRLK_ERR_UNSUPPORTED,
+                 "grpo_fused: vocab must be a multiple of 8 and at most %lld (got %lld); use the two-pass path",
+                 (long long)trlk_grpo_fused_max_vocab(dtype), (long long)vocab);
+    TRLK_REQUIRE(out_row_offset >= 0 && out_row_offset + rows_per_seq <= out_rows_per_seq, TRLK_ERR_BAD_SHAPE,
+                 "grpo_fused: input rows [%lld, %lld) do not fit the %lld output rows per sequence",
+                 (long long)out_row_offset, (long long)(out_row_offset + rows_per_seq), (long long)out_rows_per_seq);
+    TRLK_REQUIRE(temperature > 0.f && temperature < INFINITY, TRLK_ERR_BAD_VALUE,
+                 "grpo_fused: temperature must be positive and finite (got %g)", (double)temperature);
+    TRLK_REQUIRE(policy_term >= TRLK_TERM_CLIP && policy_term <= TRLK_TERM_WEIGHTED_LOGP, TRLK_ERR_BAD_VALUE,
+                 "grpo_fused: unknown policy term %d", policy_term);
+    const int64_t orows = n_seq * out_rows_per_seq;
+    if (orows == 0) return TRLK_OK;
+    TRLK_REQUIRE(orows < (int64_t(1) << 31), TRLK_ERR_BAD_SHAPE, "grpo_fused: too many rows (%lld)", (long long)orows);
+    TRLK_REQUIRE(d_dlogits != nullptr, TRLK_ERR_NULL_POINTER, "grpo_fused: dlogits pointer is null");
+    if (n_seq * rows_per_seq > 0) {
+        TRLK_REQUIRE(d_logits && d_index && d_advantages && d_mask && d_row_scale && d_out_logp && d_out_entropy && d_out_lse,
+                     TRLK_ERR_NULL_POINTER, "grpo_fused: a required pointer is null");
+        TRLK_REQUIRE(beta == 0.f || d_ref_logp != nullptr, TRLK_ERR_NULL_POINTER, "grpo_fused: beta != 0 needs ref_logp");
+        TRLK_REQUIRE(policy_term != TRLK_TERM_WEIGHTED_LOGP || d_seq_coef != nullptr, TRLK_ERR_NULL_POINTER,
+                     "grpo_fused: the weighted log-prob term needs seq_coef");
+        TRLK_REQUIRE(row_stride >= vocab || rows_per_seq <= 1, TRLK_ERR_BAD_STRIDE, "grpo_fused: rows overlap");
+    }
+    const auto al16 = [](const void* p, int64_t s0, int64_t s1) {
+        return reinterpret_cast<uintptr_t>(p) % 16 == 0 && (s0 * 2) % 16 == 0 && (s1 * 2) % 16 == 0;
+    };
+    TRLK_REQUIRE(al16(d_logits, seq_stride, row_stride) && al16(d_dlogits, out_seq_stride, out_row_stride),
+                 TRLK_ERR_BAD_STRIDE, "grpo_fused: logits and dlogits rows must be 16-byte aligned; use the two-pass path");
+    FusedArgs a{};
+    a.logits = d_logits;
+    a.rows_per_seq = rows_per_seq;
+    a.vocab = vocab;
+    a.seq_stride = seq_stride;
+    a.row_stride = row_stride;
+    a.index = d_index;
+    a.temperature = temperature;
+    a.old_logp = d_old_logp;
+    a.ref_logp = d_ref_logp;
+    a.adv = d_advantages;
+    a.mask = d_mask;
+    a.token_weight = d_token_weight;
+    a.row_scale = d_row_scale;
+    a.seq_coef = d_seq_coef;
+    a.adv_stride_b = adv_stride_b;
+    a.adv_stride_t = adv_stride_t;
+    a.policy_term = policy_term;
+    a.eps_low = epsilon_low;
+    a.eps_high = epsilon_high;
+    a.delta = delta;
+    a.beta = beta;
+    a.bias_kl = use_bias_correction_kl;
+    a.sapo_tau_pos = sapo_temperature_pos;
+    a.sapo_tau_neg = sapo_temperature_neg;
+    a.out_logp = d_out_logp;
+    a.out_entropy = d_out_entropy;
+    a.out_lse = d_out_lse;
+    a.dlogits = d_dlogits;
+    a.out_rows_per_seq = out_rows_per_seq;
+    a.out_row_offset = out_row_offset;
+    a.out_seq_stride = out_seq_stride;
+    a.out_row_stride = out_row_stride;
+    a.error_flag = d_error_flag;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == TRLK_BF16)
+        hipLaunchKernelGGL(grpo_fused_kernel<TRLK_BF16>, dim3((unsigned)orows), dim3(kFThreads), 0, s, a);
+    else
+        hipLaunchKernelGGL(grpo_fused_kernel<TRLK_F16>, dim3((unsigned)orows), dim3(kFThreads), 0, s, a);
+    return launch_status("grpo_fused");
+}

@@ -6,6 +6,7 @@
 // sequence, and the final cross-sequence reduction is recomputed identically by every
 // workgroup instead of being passed through a third launch.
 #include "common.hpp"
+#include "grpo_token.hpp"
 
 namespace trlk {
 namespace {
@@ -86,56 +87,6 @@ constexpr int kRowStatsUsed = 13;
 enum RowStat2 { RS_CLIP_CNT = 10, RS_AUX = 11, RS_AUX_CNT = 12 };
 static_assert(kRowStatsUsed <= 16, "row stats");
 
-// Policy term f(c, A, logp) of one token (or one sequence) and its two partial derivatives:
-// through the log importance ratio ln c, and directly through logp (terms that multiply logp itself).
-struct PolicyTerm {
-    float f, d_lnc, d_logp, low, high, aux;
-};
-
-__device__ __forceinline__ PolicyTerm policy_term(const GrpoArgs& a, float c_raw, float A, float lp, float coef) {
-    PolicyTerm r{0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    const float lo = 1.f - a.eps_low, hi = 1.f + a.eps_high;
-    switch (a.policy_term) {
-        case TRLK_TERM_CLIP: {  // -min(c' A, clamp(c, lo, hi) A), c' = min(c, delta)   (grpo_trainer.py:3083-3091)
-            const bool has_delta = a.delta == a.delta;
-            const float c2 = fminf(fmaxf(c_raw, lo), hi);
-            const float c1 = has_delta ? fminf(c_raw, a.delta) : c_raw;
-            const float l1 = c1 * A, l2 = c2 * A;
-            // d c / d ln c = c; clamp passes the gradient on the closed interval
-            const float d1 = (!has_delta || c_raw <= a.delta) ? A * c_raw : 0.f;
-            const float d2 = (c_raw >= lo && c_raw <= hi) ? A * c_raw : 0.f;
-            // min(l1, l2): the gradient goes to the smaller operand, half to each on a tie
-            const float w1 = (l1 < l2) ? 1.f : ((l1 == l2) ? 0.5f : 0.f);
-            r.f = -fminf(l1, l2);
-            r.d_lnc = -(w1 * d1 + (1.f - w1) * d2);
-            r.low = (c1 < lo && A < 0.f) ? 1.f : 0.f;
-            r.high = (c1 > hi && A > 0.f) ? 1.f : 0.f;
-            break;
-        }
-        case TRLK_TERM_CISPO: {  // -min(c, eps_high).detach() * A * logp   (:3080-3082)
-            const float cl = fminf(c_raw, a.eps_high);
-            r.f = -cl * A * lp;
-            r.d_logp = -cl * A;
-            r.aux = (c_raw > a.eps_high && A > 0.f) ? 1.f : 0.f;
-            break;
-        }
-        case TRLK_TERM_SAPO: {  // -sigmoid(tau (c - 1)) * 4 / tau * A   (:3092-3095)
-            const float tau = A > 0.f ? a.sapo_tau_pos : a.sapo_tau_neg;
-            const float sg = 1.f / (1.f + expf(-tau * (c_raw - 1.f)));
-            r.f = -sg * 4.f / tau * A;
-            r.d_lnc = -4.f * A * sg * (1.f - sg) * c_raw;
-            break;
-        }
-        default: {  // TRLK_TERM_WEIGHTED_LOGP: -coef * A * logp with a given, detached per-sequence coef (:3096-3107)
-            r.f = -coef * A * lp;
-            r.d_logp = -coef * A;
-            r.aux = coef;
-            break;
-        }
-    }
-    return r;
-}
-
 // Pass 1: one workgroup per sequence.  Writes d(per-token loss)/d(logp) * mask (not yet
 // normalised) and the sequence's masked sums.
 __global__ __launch_bounds__(kThreads) void grpo_rows_kernel(GrpoArgs a) {
@@ -172,27 +123,9 @@ __global__ __launch_bounds__(kThreads) void grpo_rows_kernel(GrpoArgs a) {
         const float A = a.adv[b * a.adv_stride_b + t * a.adv_stride_t];
         const float c_raw = a.seq_level ? c_seq : (a.old_logp ? expf(lp - a.old_logp[off + t]) : 1.f);
         const PolicyTerm p = policy_term(a, c_raw, A, lp, coef);
-        float pl = p.f, g_lnc = p.d_lnc, g_lp = p.d_logp;
-        if (a.token_weight) {
-            const float w = a.token_weight[off + t];
-            pl *= w;
-            g_lnc *= w;
-            g_lp *= w;
-        }
-        float kl = 0.f;
-        if (a.beta != 0.f) {  // k3 estimator exp(d) - d - 1, d = ref - logp   (:3069-3076)
-            const float d = a.ref_logp[off + t] - lp;
-            const float e = expf(d);
-            kl = e - d - 1.f;
-            float dkl = 1.f - e;
-            if (a.bias_kl) {  // kl * c: the factor c is differentiated through ln c
-                g_lnc += a.beta * kl * c_raw;
-                dkl *= c_raw;
-                kl *= c_raw;
-            }
-            pl += a.beta * kl;
-            g_lp += a.beta * dkl;
-        }
+        float pl, kl, g_lnc, g_lp;
+        grpo_token_terms(a, p, c_raw, lp, a.token_weight ? a.token_weight[off + t] : 1.f,
+                         a.beta != 0.f ? a.ref_logp[off + t] : 0.f, pl, kl, g_lnc, g_lp);
         const float H = a.entropy ? a.entropy[off + t] : 0.f;
         const float eff = a.entropy_mask ? m * a.entropy_mask[off + t] : m;
         s_mask += m;

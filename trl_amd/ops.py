@@ -320,6 +320,81 @@ grpo_loss_op.register_autograd(_grpo_backward, setup_context=_grpo_setup)
 
 
 # --------------------------------------------------------------------------------------------
+# GRPO gradient straight from the logits (K7)
+# --------------------------------------------------------------------------------------------
+def grpo_fused_max_vocab(dtype: torch.dtype) -> int:
+    """Largest vocabulary the single-pass kernel takes for this dtype (0: not supported)."""
+    return int(lib.trlk_grpo_fused_max_vocab(dtype_code(dtype))) if dtype in (torch.bfloat16, torch.float16) else 0
+
+
+def grpo_fused_fwd_bwd(
+    logits: Tensor, index: Tensor, temperature: float, keep_start: int, keep_len: int, mask: Tensor, advantages: Tensor,
+    row_scale: Tensor, old_logp: Optional[Tensor], ref_logp: Optional[Tensor], token_weight: Optional[Tensor],
+    seq_coef: Optional[Tensor], policy_term: int, epsilon_low: float, epsilon_high: float, delta: float, beta: float,
+    use_bias_correction_kl: bool, sapo_temperature_pos: float, sapo_temperature_neg: float,
+) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    """One pass over `logits[:, keep_start : keep_start + keep_len]` (`[B, L, V]`, 16-bit): returns
+    `(logp [B, K], entropy [B, K], lse [B, K], dlogits [B, L, V])`, the gradient for an upstream gradient of 1 on
+    the loss whose per-sequence normalisation is `row_scale [B]`.  Rows with `mask == 0` are not read (outputs 0)."""
+    _check_logits3d(logits)
+    n_seq, length, vocab = logits.shape
+    dev = logits.device
+    if tuple(index.shape) != (n_seq, keep_len) or tuple(mask.shape) != (n_seq, keep_len):
+        raise ValueError(f"grpo_fused: index and mask must be [{n_seq}, {keep_len}]")
+    index = index.contiguous()
+    if index.dtype != torch.int64:
+        index = index.long()
+    mask, old_logp, ref_logp, token_weight = _f32c(mask), _f32c(old_logp), _f32c(ref_logp), _f32c(token_weight)
+    for name, t in (("old_logp", old_logp), ("ref_logp", ref_logp), ("token_weight", token_weight)):
+        if t is not None and tuple(t.shape) != (n_seq, keep_len):
+            raise ValueError(f"grpo_fused: {name} has shape {tuple(t.shape)}, expected {(n_seq, keep_len)}")
+    advantages = _f32c(advantages)
+    if advantages.dim() == 1 or (advantages.dim() == 2 and advantages.shape[1] == 1):
+        if advantages.numel() != n_seq:
+            raise ValueError("grpo_fused: advantages must have one entry per sequence")
+        sb, st = 1, 0
+    elif tuple(advantages.shape) == (n_seq, keep_len):
+        sb, st = keep_len, 1
+    else:
+        raise ValueError(f"grpo_fused: advantages of shape {tuple(advantages.shape)} do not match [B] or [B, K]")
+    row_scale = row_scale.reshape(n_seq).contiguous().float()
+    seq_coef = None if seq_coef is None else seq_coef.reshape(n_seq).contiguous().float()
+    logp = torch.empty((n_seq, keep_len), dtype=torch.float32, device=dev)
+    ent = torch.empty_like(logp)
+    lse = torch.empty_like(logp)
+    dlogits = torch.empty((n_seq, length, vocab), dtype=logits.dtype, device=dev)
+    if dlogits.numel() == 0:
+        return logp, ent, lse, dlogits
+    view = logits[:, keep_start : keep_start + keep_len]
+    with torch.cuda.device(dev):
+        check(
+            lib.trlk_grpo_fused_fwd_bwd(
+                view.data_ptr(), dtype_code(logits.dtype), n_seq, keep_len, vocab, view.stride(0), view.stride(1),
+                ptr(index), temperature, ptr(old_logp), ptr(ref_logp), ptr(advantages), sb, st, ptr(mask),
+                ptr(token_weight), ptr(seq_coef), ptr(row_scale), policy_term, epsilon_low, epsilon_high, delta, beta,
+                int(use_bias_correction_kl), sapo_temperature_pos, sapo_temperature_neg, ptr(logp), ptr(ent), ptr(lse),
+                ptr(dlogits), length, keep_start, dlogits.stride(0), dlogits.stride(1), ptr(_error_flag(dev)),
+                current_stream(dev),
+            )
+        )
+    if _SYNC_CHECKS:
+        check_device_errors()
+    return logp, ent, lse, dlogits
+
+
+def scale_unless_one_(data: Tensor, scale: Tensor) -> Tensor:
+    """In place `data *= scale` for a contiguous 16-bit tensor and a one-element device scalar; when the scalar is
+    exactly 1 the launched kernel touches nothing (no host synchronisation either way)."""
+    if not data.is_contiguous() or data.dtype not in (torch.bfloat16, torch.float16):
+        raise ValueError("scale_unless_one_: contiguous bf16/fp16 data expected")
+    scale = scale.reshape(1).to(device=data.device, dtype=torch.float32)
+    with torch.cuda.device(data.device):
+        check(lib.trlk_scale_unless_one(data.data_ptr(), dtype_code(data.dtype), data.numel(), ptr(scale),
+                                        current_stream(data.device)))
+    return data
+
+
+# --------------------------------------------------------------------------------------------
 # DPO / RLOO sequence losses (K4)
 # --------------------------------------------------------------------------------------------
 @torch.library.custom_op("trl_amd::dpo_loss", mutates_args=(), device_types="cuda")

@@ -22,6 +22,8 @@ from .utils import logps_and_entropies, nanmax, nanmin  # noqa: F401  (re-export
 __all__ = [
     "per_token_logps_and_entropies",
     "grpo_loss",
+    "grpo_loss_from_logits",
+    "grpo_single_pass_supported",
     "group_advantages",
     "get_off_policy_mask",
     "get_high_entropy_mask",
@@ -220,6 +222,135 @@ def grpo_loss(
         seq_coef, float(sapo_temperature_pos), float(sapo_temperature_neg),
     )
     return loss, metrics
+
+
+_SINGLE_PASS_LOSS_TYPES = ("grpo", "bnpo", "dr_grpo", "dapo", "cispo", "sapo")
+
+
+def grpo_single_pass_supported(logits: Tensor, loss_type: str = "dapo", importance_sampling_level: str = "token",
+                               entropy_coef: float = 0.0, entropy_mask: Tensor | None = None) -> bool:
+    """Whether `grpo_loss_from_logits` can go from these logits to their gradient in one pass: a token-level
+    loss type without entropy term (the gradient coefficient of a token then depends on nothing but that
+    token), 16-bit logits whose rows fit one workgroup's registers and are 16-byte aligned."""
+    if loss_type not in _SINGLE_PASS_LOSS_TYPES or importance_sampling_level != "token":
+        return False
+    if entropy_coef != 0.0 or entropy_mask is not None:
+        return False
+    if logits.dim() != 3 or not logits.is_cuda or logits.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    vocab = logits.shape[-1]
+    if vocab % 8 != 0 or vocab > ops.grpo_fused_max_vocab(logits.dtype) or (vocab > 1 and logits.stride(-1) != 1):
+        return False
+    return logits.data_ptr() % 16 == 0 and logits.stride(0) % 8 == 0 and logits.stride(1) % 8 == 0
+
+
+class _GRPOFromLogits(torch.autograd.Function):
+    """loss (and the detached log-probs / entropies) from the logits; the gradient w.r.t. the logits was
+    written by the same pass and is only scaled by the upstream gradient in `backward`."""
+
+    @staticmethod
+    def forward(ctx, logits, completion_ids, advantages, mask, temperature, kw):
+        length = logits.shape[1]
+        keep_len = min(completion_ids.shape[1], length - 1)
+        keep_start = length - 1 - keep_len
+        ids = completion_ids[:, -keep_len:] if keep_len > 0 else completion_ids[:, :0]
+        mask_f = mask[:, -keep_len:].float() if keep_len > 0 else mask[:, :0].float()
+        n_seq = logits.shape[0]
+        reduce_code, term_code = ops.LOSS_TYPES[kw["loss_type"]]
+        ga = 1.0 if reduce_code == _lib.DAPO else float(kw["grad_accum_steps"])
+        # d loss / d (masked token loss of sequence b): what the loss kernel's second pass applies to its rows
+        if reduce_code == _lib.GRPO:
+            row_scale = (1.0 / n_seq) / ga / mask_f.sum(dim=1).clamp(min=1.0)
+        elif reduce_code == _lib.BNPO:
+            row_scale = ((1.0 / mask_f.sum().clamp(min=1.0)) / ga).expand(n_seq)
+        elif reduce_code == _lib.DR_GRPO:
+            row_scale = torch.full((n_seq,), (1.0 / float(n_seq * kw["max_completion_length"])) / ga, device=logits.device)
+        else:  # DAPO
+            n_items = kw["num_items_in_batch"]
+            n_items = (n_items.to(device=logits.device, dtype=torch.float32) if torch.is_tensor(n_items)
+                       else torch.tensor(float(n_items), dtype=torch.float32, device=logits.device))
+            row_scale = (1.0 / (n_items.clamp(min=1.0) / float(kw["num_processes"]))).reshape(1).expand(n_seq)
+        delta = kw["delta"]
+        logp, ent, _, dlogits = ops.grpo_fused_fwd_bwd(
+            logits, ids, float(temperature), keep_start, keep_len, mask_f, advantages, row_scale,
+            kw["old_per_token_logps"], kw["ref_per_token_logps"] if kw["beta"] != 0.0 else None, kw["token_weight"],
+            None, term_code, float(kw["epsilon_low"]), float(kw["epsilon_high"]),
+            math.nan if delta is None else float(delta), float(kw["beta"]), bool(kw["use_bias_correction_kl"]),
+            float(kw["sapo_temperature_pos"]), float(kw["sapo_temperature_neg"]))
+        # loss value and every metric from the [B, K]-sized kernel, on the log-probs of the same pass
+        loss, metrics = grpo_loss(
+            logp, advantages, mask_f, entropies=ent, old_per_token_logps=kw["old_per_token_logps"],
+            ref_per_token_logps=kw["ref_per_token_logps"], loss_type=kw["loss_type"], epsilon_low=kw["epsilon_low"],
+            epsilon_high=kw["epsilon_high"], beta=kw["beta"], delta=delta,
+            max_completion_length=kw["max_completion_length"], num_items_in_batch=kw["num_items_in_batch"],
+            num_processes=kw["num_processes"], grad_accum_steps=kw["grad_accum_steps"],
+            use_bias_correction_kl=kw["use_bias_correction_kl"], token_weight=kw["token_weight"],
+            sapo_temperature_pos=kw["sapo_temperature_pos"], sapo_temperature_neg=kw["sapo_temperature_neg"])
+        ctx.save_for_backward(dlogits)
+        ctx.mark_non_differentiable(metrics, logp, ent)
+        return loss, metrics, logp, ent
+
+    @staticmethod
+    def backward(ctx, g_loss, g_metrics, g_logp, g_ent):
+        (dlogits,) = ctx.saved_tensors
+        if g_loss is None:
+            return None, None, None, None, None, None
+        # in place: the buffer belongs to this node and is handed on once
+        return ops.scale_unless_one_(dlogits, g_loss), None, None, None, None, None
+
+
+def grpo_loss_from_logits(
+    logits: Tensor,
+    completion_ids: Tensor,
+    advantages: Tensor,
+    mask: Tensor,
+    *,
+    temperature: float = 1.0,
+    old_per_token_logps: Tensor | None = None,
+    ref_per_token_logps: Tensor | None = None,
+    loss_type: str = "dapo",
+    epsilon_low: float = 0.2,
+    epsilon_high: float = 0.2,
+    beta: float = 0.0,
+    delta: float | None = None,
+    max_completion_length: int | None = None,
+    num_items_in_batch: Tensor | float | None = None,
+    num_processes: int = 1,
+    grad_accum_steps: float = 1.0,
+    use_bias_correction_kl: bool = False,
+    token_weight: Tensor | None = None,
+    sapo_temperature_pos: float = 1.0,
+    sapo_temperature_neg: float = 1.05,
+) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    """`[B, L, V]` model logits -> `(loss, metrics, per_token_logps [B, K], entropies [B, K])` with ONE pass over
+    the logits: what `per_token_logps_and_entropies` + `grpo_loss` + `loss.backward()` do with two reads and a
+    write of the logits-sized data (trl/trainer/grpo_trainer.py:1514-1532, 3026-3150) costs one read and one
+    write here, because the pass that computes a row's log-prob also writes that row's gradient.
+
+    Same window as the reference (`logits[:, :-1][:, -K:]`, `K = completion_ids.shape[1]`), same arguments
+    as `grpo_loss`.  Only for `grpo_single_pass_supported(...)` configurations; the rows outside `mask` are
+    never read and their log-prob / entropy come back as 0.  `loss.backward()` hands the `[B, L, V]` gradient
+    to the graph behind `logits`; the returned log-probs and entropies are detached."""
+    if loss_type not in ops.LOSS_TYPES:
+        raise ValueError(f"Unknown loss type: {loss_type}")
+    if not grpo_single_pass_supported(logits, loss_type):
+        raise NotImplementedError(
+            "grpo_loss_from_logits: this configuration needs the two-pass path (per_token_logps_and_entropies + "
+            "grpo_loss): token-level loss types, 16-bit logits, vocab % 8 == 0 and at most "
+            f"{ops.grpo_fused_max_vocab(logits.dtype) if logits.dtype in (torch.bfloat16, torch.float16) else 0}")
+    if beta != 0.0 and ref_per_token_logps is None:
+        raise KeyError("ref_per_token_logps")
+    if ops.LOSS_TYPES[loss_type][0] == _lib.DAPO and num_items_in_batch is None:
+        raise KeyError("num_items_in_batch")
+    if loss_type == "dr_grpo" and max_completion_length is None:
+        raise ValueError("dr_grpo needs max_completion_length")
+    kw = dict(old_per_token_logps=old_per_token_logps, ref_per_token_logps=ref_per_token_logps, loss_type=loss_type,
+              epsilon_low=epsilon_low, epsilon_high=epsilon_high, beta=beta, delta=delta,
+              max_completion_length=max_completion_length, num_items_in_batch=num_items_in_batch,
+              num_processes=num_processes, grad_accum_steps=grad_accum_steps,
+              use_bias_correction_kl=use_bias_correction_kl, token_weight=token_weight,
+              sapo_temperature_pos=sapo_temperature_pos, sapo_temperature_neg=sapo_temperature_neg)
+    return _GRPOFromLogits.apply(logits, completion_ids, advantages, mask, temperature, kw)
 
 
 class GRPOLossMixin:
