@@ -159,3 +159,47 @@ def test_index_out_of_range_is_flagged(amd):
     assert math.isnan(float(lp[1, 2]))
     with pytest.raises(IndexError):
         amd.check_device_errors()
+
+
+@pytest.mark.parametrize("loss_type,beta,is_ratio", [("dapo", 0.04, False), ("grpo", 0.0, True), ("cispo", 0.0, False)])
+def test_trainer_method_takes_the_single_pass(amd, loss_type, beta, is_ratio):
+    """`GRPOLossMixin._compute_loss` on a mocked trainer: with 16-bit logits and a token-level loss it goes
+    through the one-pass operator (the log-prob method is never called) and logs the same metrics, returns
+    the same loss and leaves the same gradient as with `trl_amd_single_pass = False`."""
+    from types import SimpleNamespace
+
+    from test_gpu_losses import _fake_trainer
+
+    B, P, K, V = 6, 3, 20, 1024
+    g = torch.Generator(device=DEV).manual_seed(13)
+    logits = (2.0 * torch.randn((B, P + K, V), generator=g, device=DEV)).bfloat16()
+    completion_ids = torch.randint(0, V, (B, K), generator=g, device=DEV)
+    lengths = torch.randint(1, K + 1, (B,), generator=g, device=DEV)
+    cmask = (torch.arange(K, device=DEV)[None] < lengths[:, None]).long()
+    with torch.no_grad():
+        ids_all = torch.cat([torch.zeros((B, P), dtype=torch.long, device=DEV), completion_ids], 1)
+        base, _ = amd.per_token_logps_and_entropies(logits, ids_all, K, 0.8)
+    inputs = dict(
+        prompt_ids=torch.zeros((B, P), dtype=torch.long, device=DEV), prompt_mask=torch.ones((B, P), dtype=torch.long, device=DEV),
+        completion_ids=completion_ids, completion_mask=cmask, advantages=torch.randn((B,), generator=g, device=DEV),
+        num_items_in_batch=cmask.sum().float(), old_per_token_logps=base + 0.3 * torch.randn(base.shape, generator=g, device=DEV),
+        ref_per_token_logps=base + 0.1 * torch.randn(base.shape, generator=g, device=DEV),
+        importance_sampling_ratio=0.5 + torch.rand((B, K), generator=g, device=DEV))
+    case = dict(temperature=0.8, beta=beta, loss_type=loss_type, eps_low=0.2, eps_high=0.28, is_ratio=is_ratio, grad_accum=2)
+    results = []
+    for single in (False, True):
+        tr = _fake_trainer(amd, case, K, skip_masked=True, single_pass=single)
+        leaf = logits.detach().clone().requires_grad_(True)
+        calls = []
+        inner = tr._get_per_token_logps_and_entropies
+        tr._get_per_token_logps_and_entropies = lambda *a, _i=inner, **k: (calls.append(1), _i(*a, **k))[1]
+        loss = tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None), inputs)
+        loss.backward()
+        assert bool(calls) == (not single)
+        results.append((loss.detach(), leaf.grad, {k: v[-1] for k, v in tr._metrics["train"].items()}))
+    (l2, g2, m2), (l1, g1, m1) = results
+    torch.testing.assert_close(l1, l2, rtol=1e-5, atol=1e-7)
+    assert _rel_l2(g1, g2) < 2e-3
+    assert m1.keys() == m2.keys()
+    for k in m2:
+        assert (math.isnan(m1[k]) and math.isnan(m2[k])) or abs(m1[k] - m2[k]) <= 1e-5 * max(1.0, abs(m2[k])), k

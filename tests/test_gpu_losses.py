@@ -49,7 +49,7 @@ class _Identity:
         return x
 
 
-def _fake_trainer(amd, case, T, skip_masked=False):
+def _fake_trainer(amd, case, T, skip_masked=False, single_pass=False):
     class Trainer(amd.GRPOLossMixin):
         pass
 
@@ -83,21 +83,24 @@ def _fake_trainer(amd, case, T, skip_masked=False):
     tr._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
     tr.model = SimpleNamespace(training=True)
     tr.trl_amd_skip_masked_rows = skip_masked
+    tr.trl_amd_single_pass = single_pass
     return tr
 
 
-@pytest.mark.parametrize("skip_masked", [False, True])
-def test_golden_grpo_compute_loss_through_trainer_methods(amd, skip_masked):
+@pytest.mark.parametrize("skip_masked,single_pass", [(False, False), (True, False), (True, True)])
+def test_golden_grpo_compute_loss_through_trainer_methods(amd, skip_masked, single_pass):
     """The reference's `GRPOTrainer._compute_loss` ran these inputs on a mocked trainer; the same
     mock drives our mix-in methods on the device.  With `skip_masked` the forward kernel skips the
-    rows the completion mask zeroes; loss, metrics and gradients must not change."""
+    rows the completion mask zeroes; loss, metrics and gradients must not change.  With `single_pass`
+    the cases the one-pass kernel takes (16-bit logits, token-level loss) go through it, the others
+    fall back to the two kernels on the logits of the same model call."""
     cases, g = load_golden("grpo_compute_loss")
     ran = 0
     for case in cases:
         c = f"c{case['id']}_"
         B, P, T, V = case["shape"]
         dtype = getattr(torch, case.get("dtype", "float32"))
-        tr = _fake_trainer(amd, case, T, skip_masked)
+        tr = _fake_trainer(amd, case, T, skip_masked, single_pass)
         leaf = _t(g[c + "logits"], dtype).to(DEV).requires_grad_(True)
         inputs = dict(
             prompt_ids=_t(g[c + "prompt_ids"]).to(DEV), prompt_mask=torch.ones(B, P, dtype=torch.long, device=DEV),
@@ -131,8 +134,9 @@ def test_golden_grpo_compute_loss_through_trainer_methods(amd, skip_masked):
         else:
             want_lp, want_ent = _t(g[c + "out_logps"]), _t(g[c + "out_entropies"])
         keep = _t(g[c + "completion_mask"]).float() if skip_masked else torch.ones_like(want_lp)
-        torch.testing.assert_close(captured["lp"].detach().cpu(), want_lp * keep, atol=tol, rtol=0)
-        torch.testing.assert_close(captured["ent"].detach().cpu(), want_ent * keep, atol=tol, rtol=0)
+        if captured:  # (the one-pass branch does not go through the log-prob method)
+            torch.testing.assert_close(captured["lp"].detach().cpu(), want_lp * keep, atol=tol, rtol=0)
+            torch.testing.assert_close(captured["ent"].detach().cpu(), want_ent * keep, atol=tol, rtol=0)
         want_loss = float(g[c + "out_loss"])
         assert abs(float(loss) - want_loss) <= (2e-2 if low else 1e-5) * max(1.0, abs(want_loss)), case["name"]
         rel = _rel_l2(leaf.grad.float(), _t(g[c + "out_dlogits"]))

@@ -410,11 +410,53 @@ class GRPOLossMixin:
         # Every use of the log-probs and entropies below is multiplied by `mask`, so rows with mask == 0
         # need not be computed at all (set `trl_amd_skip_masked_rows = False` on the trainer to compute them).
         skip = mask if getattr(self, "trl_amd_skip_masked_rows", True) else None
-        per_token_logps, entropies, aux_loss = self._get_per_token_logps_and_entropies(
-            model, input_ids, attention_mask, logits_to_keep, compute_entropy=True, compute_aux_loss=aux_enabled,
-            skip_rows_mask=skip, **{k: inputs.get(k) for k in extra_keys},
-        )
         advantages = inputs["advantages"]
+        mode = "train" if self.model.training else "eval"
+        grad_accum = self.current_gradient_accumulation_steps if mode == "train" else 1.0
+        bonus = bool(getattr(self, "_entropy_bonus_enabled", False))
+        # One pass over the logits (log-probs and gradient from the same read) when nothing between the two
+        # needs the log-probs of other tokens: token-level weights, no entropy term, no mask derived from the
+        # log-probs or entropies.  `trl_amd_single_pass = False` on the trainer keeps the two-pass path.
+        single_pass = (
+            getattr(self, "trl_amd_single_pass", True) and skip is not None and not bonus
+            and self.loss_type in _SINGLE_PASS_LOSS_TYPES and self.importance_sampling_level == "token"
+            and self.top_entropy_quantile >= 1.0 and self.off_policy_mask_threshold is None
+        )
+        if single_pass:
+            model_inputs = {"input_ids": input_ids, "attention_mask": attention_mask, "use_cache": False,
+                            **{k: inputs[k] for k in extra_keys if inputs.get(k) is not None}}
+            if "logits_to_keep" in getattr(self, "model_kwarg_keys", ()):
+                model_inputs["logits_to_keep"] = logits_to_keep + 1
+            if aux_enabled:
+                model_inputs["output_router_logits"] = True
+            outputs = model(**model_inputs)
+            aux_loss = outputs.aux_loss if aux_enabled else None
+            logits = outputs.logits
+            if logits.shape[-1] > 1 and logits.stride(-1) != 1:
+                logits = logits.contiguous()
+            if grpo_single_pass_supported(logits, self.loss_type):
+                token_weight = None
+                if self.use_vllm and self.vllm_importance_sampling_correction:
+                    token_weight = inputs["importance_sampling_ratio"].float().expand(mask.shape)
+                loss, metrics, per_token_logps, entropies = grpo_loss_from_logits(
+                    logits, completion_ids, advantages, mask, temperature=self.temperature,
+                    old_per_token_logps=inputs.get("old_per_token_logps"),
+                    ref_per_token_logps=inputs["ref_per_token_logps"] if self.beta != 0.0 else None,
+                    loss_type=self.loss_type, epsilon_low=self.epsilon_low, epsilon_high=self.epsilon_high,
+                    beta=self.beta, delta=self.args.delta, max_completion_length=self.max_completion_length,
+                    num_items_in_batch=inputs.get("num_items_in_batch"), num_processes=self.accelerator.num_processes,
+                    grad_accum_steps=grad_accum, use_bias_correction_kl=self.args.use_bias_correction_kl,
+                    token_weight=token_weight, sapo_temperature_pos=getattr(self.args, "sapo_temperature_pos", 1.0),
+                    sapo_temperature_neg=getattr(self.args, "sapo_temperature_neg", 1.05))
+                return self._finish_loss(loss, metrics, entropies, mask, None, aux_loss, aux_enabled, grad_accum, mode, bonus)
+            # these logits need the two-pass kernels (fp32, a vocabulary too large for one workgroup, ...)
+            per_token_logps, entropies = per_token_logps_and_entropies(
+                logits, input_ids, logits_to_keep, self.temperature, True, False, skip)
+        else:
+            per_token_logps, entropies, aux_loss = self._get_per_token_logps_and_entropies(
+                model, input_ids, attention_mask, logits_to_keep, compute_entropy=True, compute_aux_loss=aux_enabled,
+                skip_rows_mask=skip, **{k: inputs.get(k) for k in extra_keys},
+            )
         entropy_mask = None
         if self.top_entropy_quantile < 1.0:
             entropy_mask = get_high_entropy_mask(entropies.detach(), mask, 1 - self.top_entropy_quantile, self.accelerator)
@@ -432,9 +474,6 @@ class GRPOLossMixin:
             isr = inputs["importance_sampling_ratio"].float().expand_as(per_token_logps)
             token_weight = isr if token_weight is None else token_weight * isr
 
-        mode = "train" if self.model.training else "eval"
-        grad_accum = self.current_gradient_accumulation_steps if mode == "train" else 1.0
-        bonus = bool(getattr(self, "_entropy_bonus_enabled", False))
         adaptive = bonus and bool(getattr(self, "use_adaptive_entropy", False))
         # the coefficient of the end of the previous optimizer step applies to the whole accumulation window;
         # under adaptive control only while the last window's entropy was at or below the target (:3173-3179)
@@ -457,6 +496,11 @@ class GRPOLossMixin:
                           getattr(self.args, "vespo_k_neg", 3.0), getattr(self.args, "vespo_lambda_neg", 2.0)),
             importance_sampling_ratio=inputs.get("importance_sampling_ratio"),
         )
+        return self._finish_loss(loss, metrics, entropies, mask, entropy_mask, aux_loss, aux_enabled, grad_accum, mode, bonus)
+
+    def _finish_loss(self, loss, metrics, entropies, mask, entropy_mask, aux_loss, aux_enabled, grad_accum, mode, bonus):
+        """Auxiliary loss, the adaptive entropy controller and the logged metrics (grpo_trainer.py:3152-3258)."""
+        adaptive = bonus and bool(getattr(self, "use_adaptive_entropy", False))
         if aux_enabled:
             loss = loss + self.router_aux_loss_coef * aux_loss / grad_accum
             self._metrics[mode]["aux_loss"].append(self.accelerator.gather_for_metrics(aux_loss).mean().item())
