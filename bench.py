@@ -37,6 +37,8 @@ MEASURED_K3_TRAFFIC_BYTES = {("grpo_c3", "dapo"): (10116130 + 19461194) * 1024}
 # 36.6e6 and 44.0e6 over the launches of a run; the mean is used): what leaves the L2s towards memory.  The writes
 # are the stash plus the partial results; the reads are the operand tiles that miss the L2 of their XCD, about 60
 # times the 1.3 GB of the two operands.
+# The same for one launch of the single-pass kernel with every row read (FETCH 9731350 x 2 KiB, WRITE 19470000 KiB).
+MEASURED_K7_TRAFFIC_BYTES = {("grpo_c3", "dapo"): (2 * 9731350 + 19470000) * 1024}
 MEASURED_HEAD_FWD_TRAFFIC_BYTES = {"head_c5": (2 * 40600000 + 19497000) * 1024}
 
 WORKLOADS = {
@@ -467,27 +469,49 @@ def main():
         loss.backward()
         return loss, metrics
 
-    def timed(row_mask):
+    def timed(fn):
         for _ in range(args.warmup):
-            step(row_mask)
+            fn()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(args.steps):
-            loss, _ = step(row_mask)
+            loss, _ = fn()
         e1.record()
         torch.cuda.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3
         return max(wall_ms, e0.elapsed_time(e1)) / args.steps, float(loss.detach())
 
-    # headline: every row's log-prob and entropy is produced (the configuration's stated outputs)
-    ms_per_step, loss_value = timed(None)
-    tokens_per_s = R / (ms_per_step * 1e-3)
+    # two passes over the logits (log-prob kernel, [B, T] loss kernel, gradient kernel); every row's log-prob and
+    # entropy is produced (the configuration's stated outputs)
+    ms_two_pass, loss_value = timed(lambda: step(None))
     assert loss_value == loss_value, "loss is NaN"
-    # secondary: the forward also skips the rows the completion mask zeroes (what `_compute_loss` does by default)
-    ms_mask_aware, loss_mask_aware = timed(mask)
+    # the forward also skips the rows the completion mask zeroes (what `_compute_loss` does by default)
+    ms_mask_aware, loss_mask_aware = timed(lambda: step(mask))
     assert abs(loss_mask_aware - loss_value) <= 1e-6 * max(1.0, abs(loss_value)), "mask-aware loss differs"
+
+    # one pass over the logits: the kernel that computes a row's log-prob also writes that row's gradient
+    single = None
+    if trl_amd.grpo_single_pass_supported(leaf, args.loss_type):
+        def sp_step(skip):
+            leaf.grad = None
+            loss, metrics, _, _ = trl_amd.grpo_loss_from_logits(
+                leaf, ids, adv, mask, temperature=w["temperature"], old_per_token_logps=old, ref_per_token_logps=ref,
+                loss_type=args.loss_type, epsilon_low=w["eps_low"], epsilon_high=w["eps_high"], beta=w["beta"],
+                max_completion_length=T, num_items_in_batch=n_items, keep_start=0, skip_masked_rows=skip)
+            loss.backward()
+            return loss, metrics
+
+        ms_sp_all, loss_sp = timed(lambda: sp_step(False))
+        assert abs(loss_sp - loss_value) <= 1e-6 * max(1.0, abs(loss_value)), "single-pass loss differs"
+        ms_sp_skip, loss_sp2 = timed(lambda: sp_step(True))
+        assert abs(loss_sp2 - loss_value) <= 1e-6 * max(1.0, abs(loss_value)), "single-pass (mask-aware) loss differs"
+        single = {"all_rows_ms": ms_sp_all, "mask_aware_ms": ms_sp_skip}
+    # headline: the fastest path that produces every stated output (log-prob and entropy of every row, loss, dlogits)
+    ms_per_step = min(ms_two_pass, single["all_rows_ms"]) if single else ms_two_pass
+    headline_single = single is not None and single["all_rows_ms"] <= ms_two_pass
+    tokens_per_s = R / (ms_per_step * 1e-3)
 
     # ---- per-kernel timing: each kernel alone, events around `reps` back-to-back launches -----------
     idx = ids.reshape(R, 1)
@@ -524,6 +548,48 @@ def main():
     bwd_bytes = active_rows * 2 * row_bytes + (R - active_rows) * row_bytes  # masked rows: zero-fill write only
     fwd_gbps = fwd_bytes / (fwd_ms * 1e-3) / 1e9
     bwd_gbps = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+    roofline = {
+        "bound": "hbm", "kernel": "logp_entropy_bwd_kernel (K3)", "achieved": bwd_gbps, "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s", "frac": bwd_gbps / HBM_PEAK_GBPS,
+        "traffic": MEASURED_K3_TRAFFIC_BYTES.get((args.workload, args.loss_type)), "algorithmic_bytes": bwd_bytes,
+        "avg_launch_ms": bwd_ms,
+    }
+    kernels = {}
+    if single:
+        reduce_code, term_code = ops.LOSS_TYPES[args.loss_type]
+        if reduce_code == 0:  # per-sequence mean
+            row_scale = 1.0 / B / mask.float().sum(1).clamp(min=1.0)
+        elif args.loss_type == "dr_grpo":
+            row_scale = torch.full((B,), 1.0 / (B * T), device=dev)
+        elif args.loss_type == "bnpo":
+            row_scale = (1.0 / n_items.clamp(min=1.0)).expand(B)
+        else:
+            row_scale = (1.0 / n_items.clamp(min=1.0)).expand(B)
+
+        def fused(all_rows):
+            return ops.grpo_fused_fwd_bwd(logits.detach(), ids, w["temperature"], 0, T, mask, adv, row_scale, old, ref, None,
+                                          None, term_code, w["eps_low"], w["eps_high"], float("nan"), w["beta"], False,
+                                          1.0, 1.05, all_rows)
+
+        with torch.no_grad():
+            sp_all_ms = time_kernel(lambda: fused(True))
+            sp_skip_ms = time_kernel(lambda: fused(False))
+        sp_all_bytes = 2 * R * row_bytes                              # every row read, every gradient row written
+        sp_skip_bytes = active_rows * 2 * row_bytes + (R - active_rows) * row_bytes
+        for name, ms_k, nbytes in (("grpo_fused_kernel (K7), every row read", sp_all_ms, sp_all_bytes),
+                                   ("grpo_fused_kernel (K7), masked rows not read", sp_skip_ms, sp_skip_bytes)):
+            kernels[name] = {"avg_launch_ms": ms_k, "algorithmic_bytes": nbytes,
+                             "achieved_GBps": nbytes / (ms_k * 1e-3) / 1e9,
+                             "frac": nbytes / (ms_k * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+        if headline_single:
+            gbps = sp_all_bytes / (sp_all_ms * 1e-3) / 1e9
+            roofline = {"bound": "hbm", "kernel": "grpo_fused_kernel (K7)", "achieved": gbps, "peak": HBM_PEAK_GBPS,
+                        "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+                        "traffic": MEASURED_K7_TRAFFIC_BYTES.get((args.workload, args.loss_type)),
+                        "algorithmic_bytes": sp_all_bytes, "avg_launch_ms": sp_all_ms,
+                        # the work of this launch priced as the two-pass kernels' bytes (forward read of every row,
+                        # backward read + write): what the launch replaces, not what it moves
+                        "two_pass_equivalent_GBps": (fwd_bytes + bwd_bytes) / (sp_all_ms * 1e-3) / 1e9}
 
     result = {
         "metric": "tokens/sec + achieved HBM TB/s (% of peak) for GRPO logprob+loss fwd+bwd",
@@ -539,25 +605,26 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": args.workload, "description": w["desc"], "rows": R, "vocab": V,
-                   "loss_type": args.loss_type, "active_rows": active_rows, "loss": loss_value},
-        "roofline": {
-            "bound": "hbm",
-            "kernel": "logp_entropy_bwd_kernel (K3)",
-            "achieved": bwd_gbps,
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": bwd_gbps / HBM_PEAK_GBPS,
-            "traffic": MEASURED_K3_TRAFFIC_BYTES.get((args.workload, args.loss_type)),
-            "algorithmic_bytes": bwd_bytes,
-            "avg_launch_ms": bwd_ms,
-        },
-        "kernels": {
+                   "loss_type": args.loss_type, "active_rows": active_rows, "loss": loss_value,
+                   "path": "single pass over the logits (K7), every row computed" if headline_single
+                           else "two passes over the logits (K1, K3)"},
+        "roofline": roofline,
+        "kernels": dict(kernels, **{
             "logp_entropy_fwd_kernel (K1)": {"avg_launch_ms": fwd_ms, "algorithmic_bytes": fwd_bytes,
                                              "achieved_GBps": fwd_gbps, "frac": fwd_gbps / HBM_PEAK_GBPS},
             "logp_entropy_bwd_kernel (K3)": {"avg_launch_ms": bwd_ms, "algorithmic_bytes": bwd_bytes,
                                              "achieved_GBps": bwd_gbps, "frac": bwd_gbps / HBM_PEAK_GBPS},
-            "step_hbm_GBps": (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9,
-        },
+            "two_pass_step_hbm_GBps": (fwd_bytes + bwd_bytes) / (ms_two_pass * 1e-3) / 1e9,
+        }),
+        "two_pass": {"ms_per_step": ms_two_pass, "tokens_per_s": R / (ms_two_pass * 1e-3),
+                     "note": "log-prob kernel (K1), [B, T] loss kernel, gradient kernel (K3): two reads and one write "
+                             "of the logits-sized data; the path of every configuration the single pass does not take"},
+        "single_pass": None if single is None else {
+            "ms_per_step": single["all_rows_ms"], "tokens_per_s": R / (single["all_rows_ms"] * 1e-3),
+            "mask_aware_ms_per_step": single["mask_aware_ms"],
+            "mask_aware_tokens_per_s": R / (single["mask_aware_ms"] * 1e-3),
+            "note": "grpo_loss_from_logits: one read and one write; same loss, log-probs, entropies and dlogits; "
+                    "mask-aware = rows with completion_mask == 0 are not read (what `_compute_loss` does by default)"},
         "mask_aware": {"ms_per_step": ms_mask_aware, "tokens_per_s": R / (ms_mask_aware * 1e-3),
                        "note": "forward also skips rows with completion_mask == 0 (their outputs are 0); "
                                "loss, metrics and dlogits identical"},

@@ -280,7 +280,8 @@ int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, const int64_
  *   the other per-token inputs, the policy terms and their parameters are those of trlk_grpo_loss.
  * 16-bit logits only, vocab % 8 == 0 and vocab <= trlk_grpo_fused_max_vocab(dtype) (a row is held
  * in the registers of one workgroup), rows 16-byte aligned.  Outputs: log-prob, entropy and lse of
- * every row of the completion mask (0 for the others, which are not read), and the full
+ * every row of the completion mask (the others are not read and yield 0, unless compute_masked_rows
+ * asks for their outputs too), and the full
  * [n_seq, out_rows_per_seq, vocab] gradient laid out as trlk_logp_entropy_bwd writes it, for an
  * upstream gradient of 1 on the loss.  trlk_scale_unless_one multiplies such a buffer by a device
  * scalar, and launches an empty kernel when that scalar is exactly 1.
@@ -295,7 +296,8 @@ int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t n_seq, int6
                             int use_bias_correction_kl, float sapo_temperature_pos, float sapo_temperature_neg,
                             float* d_out_logp, float* d_out_entropy, float* d_out_lse, void* d_dlogits,
                             int64_t out_rows_per_seq, int64_t out_row_offset, int64_t out_seq_stride,
-                            int64_t out_row_stride, int32_t* d_error_flag, trlk_stream_t stream);
+                            int64_t out_row_stride, int compute_masked_rows, int32_t* d_error_flag,
+                            trlk_stream_t stream);
 int trlk_scale_unless_one(void* d_data, int dtype, int64_t n_elems, const float* d_scale, trlk_stream_t stream);
 
 #ifdef __cplusplus

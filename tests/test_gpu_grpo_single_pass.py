@@ -76,7 +76,32 @@ def test_matches_two_pass(amd, loss_type, beta):
     assert float(g1[~full_mask].abs().max()) == 0.0 and float(g2[~full_mask].abs().max()) == 0.0
     # every gradient row sums to zero up to the rounding of its 4096 bf16 entries
     assert float(g1.float().sum(-1).abs().max()) < 1e-3
+    # with the rows outside the mask computed too: their outputs match the two-pass values, nothing else moves
+    leaf3 = logits.detach().clone().requires_grad_(True)
+    loss3, met3, lp3, ent3 = amd.grpo_loss_from_logits(leaf3, ids, adv, mask, temperature=T, skip_masked_rows=False, **kw)
+    loss3.backward()
+    torch.testing.assert_close(lp3, lp2, rtol=0, atol=1e-5)
+    torch.testing.assert_close(ent3, ent2, rtol=0, atol=1e-5)
+    assert torch.equal(loss3, loss1) and torch.equal(leaf3.grad, g1)
     amd.check_device_errors()
+
+
+def test_window_given_by_keep_start(amd):
+    """`keep_start` places the K-row window anywhere in the logits (here: all rows, no position dropped)."""
+    B, K, V = 3, 8, 512
+    logits, ids, mask, adv, _ = _inputs(B, K, V, seed=17, extra_rows=0)
+    leaf = logits.detach().clone().requires_grad_(True)
+    lp2, ent2 = amd.logps_and_entropies(leaf, ids, 1.0)
+    loss2, _ = amd.grpo_loss(lp2, adv, mask, entropies=ent2.detach(), loss_type="bnpo")
+    loss2.backward()
+    leaf1 = logits.detach().clone().requires_grad_(True)
+    loss1, _, lp1, _ = amd.grpo_loss_from_logits(leaf1, ids, adv, mask, loss_type="bnpo", keep_start=0, skip_masked_rows=False)
+    loss1.backward()
+    torch.testing.assert_close(loss1, loss2, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(lp1, lp2.detach(), rtol=0, atol=1e-5)
+    assert _rel_l2(leaf1.grad, leaf.grad) < 2e-3
+    with pytest.raises(ValueError):
+        amd.grpo_loss_from_logits(leaf1, ids, adv, mask, loss_type="bnpo", keep_start=1)
 
 
 def test_upstream_gradient_scales(amd):

@@ -34,6 +34,7 @@ struct FusedArgs {
     void* dlogits;
     int64_t out_rows_per_seq, out_row_offset, out_seq_stride, out_row_stride;
     int32_t* error_flag;
+    int all_rows;  // also read the rows with mask == 0 for their log-prob and entropy (their gradient is zero either way)
 };
 
 template <int DT>
@@ -52,9 +53,11 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     const int nv = int(a.vocab / EPV);
     u32x4* op = reinterpret_cast<u32x4*>(static_cast<T*>(a.dlogits) + b * a.out_seq_stride + to * a.out_row_stride);
     const float m = inside ? a.mask[row] : 0.f;
-    if (m == 0.f) {  // no gradient reaches this row: zero-fill, nothing is read
+    if (m == 0.f) {  // no gradient reaches this row: zero-fill
         const u32x4 z = {0u, 0u, 0u, 0u};
         for (int v = tid; v < nv; v += kFThreads) __builtin_nontemporal_store(z, op + v);
+    }
+    if (m == 0.f && !(inside && a.all_rows)) {  // and nothing is read
         if (inside && tid == 0) {
             a.out_logp[row] = 0.f;
             a.out_entropy[row] = 0.f;
@@ -139,6 +142,7 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
         a.out_lse[row] = lse;
         if (!idx_ok && a.error_flag) atomicOr(a.error_flag, TRLK_FLAG_INDEX_OUT_OF_RANGE);
     }
+    if (m == 0.f) return;  // (all_rows) the row was read for its outputs only
     // the token's loss terms -> d loss / d logp, already normalised
     const float c_raw = a.old_logp ? expf(lp - old_lp) : 1.f;
     const PolicyTerm p = policy_term(a, c_raw, A, lp, coef);
@@ -217,7 +221,8 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
                                        int use_bias_correction_kl, float sapo_temperature_pos, float sapo_temperature_neg,
                                        float* d_out_logp, float* d_out_entropy, float* d_out_lse, void* d_dlogits,
                                        int64_t out_rows_per_seq, int64_t out_row_offset, int64_t out_seq_stride,
-                                       int64_t out_row_stride, int32_t* d_error_flag, trlk_stream_t stream) {
+                                       int64_t out_row_stride, int compute_masked_rows, int32_t* d_error_flag,
+                                       trlk_stream_t stream) {
     clear_error();
     TRLK_REQUIRE(dtype == TRLK_BF16 || dtype == TRLK_F16, TRLK_ERR_BAD_DTYPE,
                  "grpo_fused: 16-bit logits only (dtype code %d); use the two-pass path", dtype);
@@ -283,6 +288,7 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
     a.out_seq_stride = out_seq_stride;
     a.out_row_stride = out_row_stride;
     a.error_flag = d_error_flag;
+    a.all_rows = compute_masked_rows != 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == TRLK_BF16)
         hipLaunchKernelGGL(grpo_fused_kernel<TRLK_BF16>, dim3((unsigned)orows), dim3(kFThreads), 0, s, a);

@@ -332,10 +332,12 @@ def grpo_fused_fwd_bwd(
     row_scale: Tensor, old_logp: Optional[Tensor], ref_logp: Optional[Tensor], token_weight: Optional[Tensor],
     seq_coef: Optional[Tensor], policy_term: int, epsilon_low: float, epsilon_high: float, delta: float, beta: float,
     use_bias_correction_kl: bool, sapo_temperature_pos: float, sapo_temperature_neg: float,
+    compute_masked_rows: bool = False,
 ) -> tuple[Tensor, Tensor, Tensor, Tensor]:
     """One pass over `logits[:, keep_start : keep_start + keep_len]` (`[B, L, V]`, 16-bit): returns
     `(logp [B, K], entropy [B, K], lse [B, K], dlogits [B, L, V])`, the gradient for an upstream gradient of 1 on
-    the loss whose per-sequence normalisation is `row_scale [B]`.  Rows with `mask == 0` are not read (outputs 0)."""
+    the loss whose per-sequence normalisation is `row_scale [B]`.  Rows with `mask == 0` are not read (outputs 0)
+    unless `compute_masked_rows`."""
     _check_logits3d(logits)
     n_seq, length, vocab = logits.shape
     dev = logits.device
@@ -373,8 +375,8 @@ def grpo_fused_fwd_bwd(
                 ptr(index), temperature, ptr(old_logp), ptr(ref_logp), ptr(advantages), sb, st, ptr(mask),
                 ptr(token_weight), ptr(seq_coef), ptr(row_scale), policy_term, epsilon_low, epsilon_high, delta, beta,
                 int(use_bias_correction_kl), sapo_temperature_pos, sapo_temperature_neg, ptr(logp), ptr(ent), ptr(lse),
-                ptr(dlogits), length, keep_start, dlogits.stride(0), dlogits.stride(1), ptr(_error_flag(dev)),
-                current_stream(dev),
+                ptr(dlogits), length, keep_start, dlogits.stride(0), dlogits.stride(1), int(compute_masked_rows),
+                ptr(_error_flag(dev)), current_stream(dev),
             )
         )
     if _SYNC_CHECKS:

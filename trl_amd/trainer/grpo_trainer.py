@@ -251,8 +251,13 @@ class _GRPOFromLogits(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, completion_ids, advantages, mask, temperature, kw):
         length = logits.shape[1]
-        keep_len = min(completion_ids.shape[1], length - 1)
-        keep_start = length - 1 - keep_len
+        if kw["keep_start"] is None:
+            keep_len = min(completion_ids.shape[1], length - 1)
+            keep_start = length - 1 - keep_len
+        else:
+            keep_len, keep_start = completion_ids.shape[1], int(kw["keep_start"])
+            if keep_start < 0 or keep_start + keep_len > length:
+                raise ValueError("grpo_loss_from_logits: keep_start + K exceeds the logits' rows")
         ids = completion_ids[:, -keep_len:] if keep_len > 0 else completion_ids[:, :0]
         mask_f = mask[:, -keep_len:].float() if keep_len > 0 else mask[:, :0].float()
         n_seq = logits.shape[0]
@@ -276,7 +281,7 @@ class _GRPOFromLogits(torch.autograd.Function):
             kw["old_per_token_logps"], kw["ref_per_token_logps"] if kw["beta"] != 0.0 else None, kw["token_weight"],
             None, term_code, float(kw["epsilon_low"]), float(kw["epsilon_high"]),
             math.nan if delta is None else float(delta), float(kw["beta"]), bool(kw["use_bias_correction_kl"]),
-            float(kw["sapo_temperature_pos"]), float(kw["sapo_temperature_neg"]))
+            float(kw["sapo_temperature_pos"]), float(kw["sapo_temperature_neg"]), not kw["skip_masked_rows"])
         # loss value and every metric from the [B, K]-sized kernel, on the log-probs of the same pass
         loss, metrics = grpo_loss(
             logp, advantages, mask_f, entropies=ent, old_per_token_logps=kw["old_per_token_logps"],
@@ -321,6 +326,8 @@ def grpo_loss_from_logits(
     token_weight: Tensor | None = None,
     sapo_temperature_pos: float = 1.0,
     sapo_temperature_neg: float = 1.05,
+    skip_masked_rows: bool = True,
+    keep_start: int | None = None,
 ) -> tuple[Tensor, Tensor, Tensor, Tensor]:
     """`[B, L, V]` model logits -> `(loss, metrics, per_token_logps [B, K], entropies [B, K])` with ONE pass over
     the logits: what `per_token_logps_and_entropies` + `grpo_loss` + `loss.backward()` do with two reads and a
@@ -328,8 +335,9 @@ def grpo_loss_from_logits(
     write here, because the pass that computes a row's log-prob also writes that row's gradient.
 
     Same window as the reference (`logits[:, :-1][:, -K:]`, `K = completion_ids.shape[1]`), same arguments
-    as `grpo_loss`.  Only for `grpo_single_pass_supported(...)` configurations; the rows outside `mask` are
-    never read and their log-prob / entropy come back as 0.  `loss.backward()` hands the `[B, L, V]` gradient
+    as `grpo_loss`; `keep_start` names another first row of the window.  Only for
+    `grpo_single_pass_supported(...)` configurations.  The rows outside `mask` are never read and their log-prob /
+    entropy come back as 0, unless `skip_masked_rows=False` asks for them (their gradient is zero either way).  `loss.backward()` hands the `[B, L, V]` gradient
     to the graph behind `logits`; the returned log-probs and entropies are detached."""
     if loss_type not in ops.LOSS_TYPES:
         raise ValueError(f"Unknown loss type: {loss_type}")
@@ -349,7 +357,8 @@ def grpo_loss_from_logits(
               max_completion_length=max_completion_length, num_items_in_batch=num_items_in_batch,
               num_processes=num_processes, grad_accum_steps=grad_accum_steps,
               use_bias_correction_kl=use_bias_correction_kl, token_weight=token_weight,
-              sapo_temperature_pos=sapo_temperature_pos, sapo_temperature_neg=sapo_temperature_neg)
+              sapo_temperature_pos=sapo_temperature_pos, sapo_temperature_neg=sapo_temperature_neg,
+              skip_masked_rows=skip_masked_rows, keep_start=keep_start)
     return _GRPOFromLogits.apply(logits, completion_ids, advantages, mask, temperature, kw)
 
 
