@@ -228,3 +228,38 @@ def test_trainer_method_takes_the_single_pass(amd, loss_type, beta, is_ratio):
     assert m1.keys() == m2.keys()
     for k in m2:
         assert (math.isnan(m1[k]) and math.isnan(m2[k])) or abs(m1[k] - m2[k]) <= 1e-5 * max(1.0, abs(m2[k])), k
+
+
+@pytest.mark.parametrize("loss_type", ["dapo", "grpo", "dr_grpo", "bnpo"])
+def test_against_the_oracle_autograd(amd, loss_type):
+    """Independent of the two-pass kernels: the CPU oracle's log-probs, loss and autograd gradient on the same
+    stored bf16 logits (fp32 op-math).  Log-probs 2e-3 abs, loss 1e-3 relative, dlogits 5e-3 relative L2 (the
+    output is rounded to bf16)."""
+    import oracle
+
+    B, L, K, V, temp = 4, 9, 6, 4096, 0.9
+    g = torch.Generator().manual_seed(2)
+    logits = (2.0 * torch.randn(B, L, V, generator=g)).bfloat16()
+    ids = torch.randint(0, V, (B, L), generator=g)
+    mask = (torch.arange(K)[None] < torch.tensor([6, 3, 0, 5])[:, None]).long()
+    adv = torch.randn(B, generator=g)
+    with torch.no_grad():
+        base, _ = oracle.logps_and_entropies_from_logits(logits.float(), ids, K, temp, False)
+    old, ref = base + 0.2 * torch.randn(base.shape, generator=g), base - 0.1
+    kw = dict(loss_type=loss_type, epsilon_low=0.2, epsilon_high=0.28, beta=0.04, max_completion_length=K,
+              num_items_in_batch=mask.sum().float(), grad_accum_steps=2.0)
+    cpu_leaf = logits.float().requires_grad_(True)
+    lp, ent = oracle.logps_and_entropies_from_logits(cpu_leaf, ids, K, temp, True)
+    want_loss, _ = oracle.grpo_loss(lp, adv, mask, entropies=ent, old_per_token_logps=old, ref_per_token_logps=ref, **kw)
+    want_loss.backward()
+    leaf = logits.to(DEV).requires_grad_(True)
+    kw["num_items_in_batch"] = kw["num_items_in_batch"].to(DEV)
+    loss, _, got_lp, got_ent = amd.grpo_loss_from_logits(
+        leaf, ids[:, -K:].to(DEV), adv.to(DEV), mask.to(DEV), temperature=temp, old_per_token_logps=old.to(DEV),
+        ref_per_token_logps=ref.to(DEV), **kw)
+    loss.backward()
+    m = mask.bool()
+    torch.testing.assert_close(got_lp.cpu()[m], lp.detach()[m], atol=2e-3, rtol=0)
+    torch.testing.assert_close(got_ent.cpu()[m], ent.detach()[m], atol=2e-3, rtol=0)
+    torch.testing.assert_close(loss.detach().cpu(), want_loss.detach(), atol=1e-6, rtol=1e-3)
+    assert _rel_l2(leaf.grad.float().cpu(), cpu_leaf.grad) < 5e-3
