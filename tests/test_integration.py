@@ -29,10 +29,12 @@ def test_patch_trl_rebinds_every_importer():
             assert ref_grpo.entropy_from_logits is trl_amd.entropy_from_logits
             assert ref_utils._ChunkedLogProbFunction is trl_amd._ChunkedLogProbFunction
             assert ref_grpo.GRPOTrainer._compute_loss is trl_amd.GRPOLossMixin._compute_loss
+            assert ref_grpo.GRPOTrainer._finish_loss is trl_amd.GRPOLossMixin._finish_loss
             assert integration.patch_trl() == 0  # idempotent
         finally:
             integration.unpatch_trl()
         assert ref_grpo.selective_log_softmax is orig and ref_grpo.GRPOTrainer._compute_loss is orig_loss
+        assert not hasattr(ref_grpo.GRPOTrainer, "_finish_loss")
     finally:
         sys.path.remove(REFERENCE)
 

@@ -67,6 +67,9 @@ def patch_trl(grpo: bool = True, liger: bool = False, dpo: bool = False, rloo: b
             _saved.append((GRPOTrainer, name, GRPOTrainer.__dict__[name]))
             setattr(GRPOTrainer, name, getattr(_grpo.GRPOLossMixin, name))
             count += 1
+        # helper of the mix-in's `_compute_loss` (no method of that name in the reference class)
+        _saved.append((GRPOTrainer, "_finish_loss", GRPOTrainer.__dict__.get("_finish_loss", _MISSING)))
+        GRPOTrainer._finish_loss = _grpo.GRPOLossMixin._finish_loss
     if rloo:
         from trl.trainer.rloo_trainer import RLOOTrainer
 
