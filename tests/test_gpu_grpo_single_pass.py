@@ -263,3 +263,23 @@ def test_against_the_oracle_autograd(amd, loss_type):
     torch.testing.assert_close(got_ent.cpu()[m], ent.detach()[m], atol=2e-3, rtol=0)
     torch.testing.assert_close(loss.detach().cpu(), want_loss.detach(), atol=1e-6, rtol=1e-3)
     assert _rel_l2(leaf.grad.float().cpu(), cpu_leaf.grad) < 5e-3
+
+
+def test_without_gradient_only_the_forward_runs(amd):
+    """Under `no_grad` (evaluation) the operator returns the same loss, metrics, log-probs and entropies without
+    writing a logits-sized gradient."""
+    B, K, V = 4, 16, 2048
+    logits, ids, mask, adv, _ = _inputs(B, K, V, seed=23)
+    kw = dict(loss_type="dapo", num_items_in_batch=mask.sum().float(), temperature=0.9)
+    leaf = logits.detach().clone().requires_grad_(True)
+    want = amd.grpo_loss_from_logits(leaf, ids, adv, mask, **kw)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    with torch.no_grad():
+        got = amd.grpo_loss_from_logits(leaf, ids, adv, mask, **kw)
+    assert torch.cuda.memory_allocated() - before < logits.numel()  # no [B, L, V] buffer was kept
+    assert not got[0].requires_grad
+    torch.testing.assert_close(got[0], want[0].detach(), rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(got[1], want[1], rtol=1e-5, atol=1e-6, equal_nan=True)
+    torch.testing.assert_close(got[2], want[2], rtol=0, atol=1e-5)
+    torch.testing.assert_close(got[3], want[3], rtol=0, atol=1e-5)

@@ -352,6 +352,24 @@ def grpo_loss_from_logits(
         raise KeyError("num_items_in_batch")
     if loss_type == "dr_grpo" and max_completion_length is None:
         raise ValueError("dr_grpo needs max_completion_length")
+    if not (torch.is_grad_enabled() and logits.requires_grad):
+        # nobody will ask for the gradient: the forward kernel alone (one read, nothing logits-sized written)
+        length = logits.shape[1]
+        keep_len = completion_ids.shape[1] if keep_start is not None else min(completion_ids.shape[1], length - 1)
+        start = int(keep_start) if keep_start is not None else length - 1 - keep_len
+        if start < 0 or start + keep_len > length:
+            raise ValueError("grpo_loss_from_logits: keep_start + K exceeds the logits' rows")
+        ids = completion_ids[:, -keep_len:] if keep_len > 0 else completion_ids[:, :0]
+        m = mask[:, -keep_len:] if keep_len > 0 else mask[:, :0]
+        logp, ent = logps_and_entropies(logits, ids, temperature, start, keep_len, m if skip_masked_rows else None)
+        loss, metrics = grpo_loss(
+            logp, advantages, m, entropies=ent, old_per_token_logps=old_per_token_logps,
+            ref_per_token_logps=ref_per_token_logps, loss_type=loss_type, epsilon_low=epsilon_low,
+            epsilon_high=epsilon_high, beta=beta, delta=delta, max_completion_length=max_completion_length,
+            num_items_in_batch=num_items_in_batch, num_processes=num_processes, grad_accum_steps=grad_accum_steps,
+            use_bias_correction_kl=use_bias_correction_kl, token_weight=token_weight,
+            sapo_temperature_pos=sapo_temperature_pos, sapo_temperature_neg=sapo_temperature_neg)
+        return loss, metrics, logp.detach(), ent.detach()
     kw = dict(old_per_token_logps=old_per_token_logps, ref_per_token_logps=ref_per_token_logps, loss_type=loss_type,
               epsilon_low=epsilon_low, epsilon_high=epsilon_high, beta=beta, delta=delta,
               max_completion_length=max_completion_length, num_items_in_batch=num_items_in_batch,
