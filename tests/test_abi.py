@@ -88,8 +88,26 @@ def test_host_side_argument_validation():
     # dpo: odd batch
     assert lib.trlk_dpo_loss(fake, fake, fake, fake, 3, 8, 0.1, fake, fake, fake, fake, None) == -2
     assert lib.trlk_rloo_loss(fake, fake, fake, fake, 0, 8, 0.2, 0.2, fake, fake, fake, fake, None) == -2
-    # fused head: fp32 operands, ragged hidden size, a stash whose rows are too short, missing workspace
+    # single-pass GRPO: fp32 logits, a vocabulary that does not fit one workgroup, ragged or misaligned rows,
+    # beta != 0 without reference log-probs, a window that does not fit the output rows
     fake16 = 0x1000
+
+    def fused(dtype=_lib.BF16, vocab=4096, logits=fake16, row_stride=None, beta=0.0, ref=None, out_rows=4, offset=0,
+              term=_lib.TERM_CLIP):
+        rs = vocab if row_stride is None else row_stride
+        return lib.trlk_grpo_fused_fwd_bwd(logits, dtype, 2, 4, vocab, 4 * rs, rs, fake, 1.0, None, ref, fake, 1, 0, fake,
+                                           None, None, fake, term, 0.2, 0.2, float("nan"), beta, 0, 1.0, 1.05, fake, fake,
+                                           fake, fake16, out_rows, offset, out_rows * vocab, vocab, 0, None, None)
+
+    assert lib.trlk_grpo_fused_max_vocab(_lib.BF16) == 20 * 1024 * 8 and lib.trlk_grpo_fused_max_vocab(_lib.F32) == 0
+    assert fused(dtype=_lib.F32) == -3 and "two-pass" in _lib.last_error()
+    assert fused(vocab=4100) == -7 and fused(vocab=20 * 1024 * 8 + 8) == -7
+    assert fused(logits=fake16 + 2) == -4 and fused(row_stride=4100) == -4
+    assert fused(beta=0.1) == -1 and fused(term=9) == -5
+    assert fused(out_rows=3) == -2 and fused(out_rows=8, offset=5) == -2
+    assert lib.trlk_scale_unless_one(fake16, _lib.F32, 64, fake, None) == -3
+    assert lib.trlk_scale_unless_one(fake16, _lib.BF16, 60, fake, None) == -2
+    # fused head: fp32 operands, ragged hidden size, a stash whose rows are too short, missing workspace
 
     def head_fwd(dtype=_lib.BF16, h=64, stash=None, stash_ld=0, ws=fake16, ws_bytes=1 << 30):
         return lib.trlk_fused_head_fwd(fake16, fake16, fake, dtype, 300, 1000, h, h, h, 1.0, 0.0, 1.0, None, fake, fake,
