@@ -277,6 +277,8 @@ int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, const int64_
  * gradient coefficient of a token depends only on its own log-prob, on per-token inputs and on
  * normalisers known from the mask:
  *   d_row_scale fp32 [n_seq] = d loss / d (masked token loss of that sequence), e.g. 1 / num_items for dapo;
+ *   d_entropy_weight fp32 [n_seq, rows_per_seq] or NULL = d loss / d entropy of each token (the entropy bonus of
+ *   grpo_trainer.py:3155-3181 with its normaliser folded in);
  *   the other per-token inputs, the policy terms and their parameters are those of trlk_grpo_loss.
  * 16-bit logits only, vocab % 8 == 0 and vocab <= trlk_grpo_fused_max_vocab(dtype) (a row is held
  * in the registers of one workgroup), rows 16-byte aligned.  Outputs: log-prob, entropy and lse of
@@ -292,7 +294,7 @@ int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t n_seq, int6
                             const float* d_old_logp, const float* d_ref_logp, const float* d_advantages,
                             int64_t adv_stride_b, int64_t adv_stride_t, const float* d_mask,
                             const float* d_token_weight, const float* d_seq_coef, const float* d_row_scale,
-                            int policy_term, float epsilon_low, float epsilon_high, float delta, float beta,
+                            const float* d_entropy_weight, int policy_term, float epsilon_low, float epsilon_high, float delta, float beta,
                             int use_bias_correction_kl, float sapo_temperature_pos, float sapo_temperature_neg,
                             float* d_out_logp, float* d_out_entropy, float* d_out_lse, void* d_dlogits,
                             int64_t out_rows_per_seq, int64_t out_row_offset, int64_t out_seq_stride,

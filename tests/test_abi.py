@@ -96,7 +96,7 @@ def test_host_side_argument_validation():
               term=_lib.TERM_CLIP):
         rs = vocab if row_stride is None else row_stride
         return lib.trlk_grpo_fused_fwd_bwd(logits, dtype, 2, 4, vocab, 4 * rs, rs, fake, 1.0, None, ref, fake, 1, 0, fake,
-                                           None, None, fake, term, 0.2, 0.2, float("nan"), beta, 0, 1.0, 1.05, fake, fake,
+                                           None, None, fake, None, term, 0.2, 0.2, float("nan"), beta, 0, 1.0, 1.05, fake, fake,
                                            fake, fake16, out_rows, offset, out_rows * vocab, vocab, 0, None, None)
 
     assert lib.trlk_grpo_fused_max_vocab(_lib.BF16) == 20 * 1024 * 8 and lib.trlk_grpo_fused_max_vocab(_lib.F32) == 0

@@ -104,6 +104,31 @@ def test_window_given_by_keep_start(amd):
         amd.grpo_loss_from_logits(leaf1, ids, adv, mask, loss_type="bnpo", keep_start=1)
 
 
+@pytest.mark.parametrize("loss_type", ["dapo", "grpo", "bnpo"])
+def test_entropy_bonus_matches_two_pass(amd, loss_type):
+    """With an entropy bonus the gradient also has the entropy's own term (through every logit of the row)."""
+    B, K, V, T = 6, 24, 2048, 0.8
+    logits, ids, mask, adv, g = _inputs(B, K, V, seed=31)
+    with torch.no_grad():
+        base, _ = amd.per_token_logps_and_entropies(logits, ids, K, T)
+    kw = dict(old_per_token_logps=base + 0.2 * torch.randn(base.shape, generator=g, device=DEV), loss_type=loss_type,
+              num_items_in_batch=mask.sum().float() * 2, grad_accum_steps=2.0, entropy_coef=0.05)
+    leaf = logits.detach().clone().requires_grad_(True)
+    logp, ent = amd.per_token_logps_and_entropies(leaf, ids, K, T, True, True)
+    loss2, met2 = amd.grpo_loss(logp, adv, mask, entropies=ent, **kw)
+    loss2.backward()
+    leaf1 = logits.detach().clone().requires_grad_(True)
+    loss1, met1, _, _ = amd.grpo_loss_from_logits(leaf1, ids, adv, mask, temperature=T, **kw)
+    loss1.backward()
+    torch.testing.assert_close(loss1, loss2, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(met1, met2, rtol=1e-5, atol=1e-6, equal_nan=True)
+    assert _rel_l2(leaf1.grad, leaf.grad) < 2e-3
+    # the entropy term is really there: without it the gradient is a different one
+    leaf0 = logits.detach().clone().requires_grad_(True)
+    amd.grpo_loss_from_logits(leaf0, ids, adv, mask, temperature=T, **dict(kw, entropy_coef=0.0))[0].backward()
+    assert _rel_l2(leaf0.grad, leaf.grad) > 1e-2
+
+
 def test_upstream_gradient_scales(amd):
     B, K, V = 4, 16, 2048
     logits, ids, mask, adv, _ = _inputs(B, K, V, seed=5)
@@ -163,7 +188,8 @@ def test_unsupported_configurations_raise(amd):
     assert not amd.grpo_single_pass_supported(logits.float())
     assert not amd.grpo_single_pass_supported(logits, "vespo")
     assert not amd.grpo_single_pass_supported(logits, "dapo", "sequence")
-    assert not amd.grpo_single_pass_supported(logits, entropy_coef=0.01)
+    assert amd.grpo_single_pass_supported(logits, entropy_coef=0.01)
+    assert not amd.grpo_single_pass_supported(logits, entropy_mask=mask)
     assert not amd.grpo_single_pass_supported(logits[..., :1020])
     big = torch.empty((1, 2, amd.ops.grpo_fused_max_vocab(torch.bfloat16) + 8), dtype=torch.bfloat16, device=DEV)
     assert not amd.grpo_single_pass_supported(big)
@@ -186,8 +212,9 @@ def test_index_out_of_range_is_flagged(amd):
         amd.check_device_errors()
 
 
-@pytest.mark.parametrize("loss_type,beta,is_ratio", [("dapo", 0.04, False), ("grpo", 0.0, True), ("cispo", 0.0, False)])
-def test_trainer_method_takes_the_single_pass(amd, loss_type, beta, is_ratio):
+@pytest.mark.parametrize("loss_type,beta,is_ratio,ent_coef", [("dapo", 0.04, False, 0.0), ("grpo", 0.0, True, 0.0),
+                                                              ("cispo", 0.0, False, 0.0), ("dapo", 0.0, False, 0.02)])
+def test_trainer_method_takes_the_single_pass(amd, loss_type, beta, is_ratio, ent_coef):
     """`GRPOLossMixin._compute_loss` on a mocked trainer: with 16-bit logits and a token-level loss it goes
     through the one-pass operator (the log-prob method is never called) and logs the same metrics, returns
     the same loss and leaves the same gradient as with `trl_amd_single_pass = False`."""
@@ -210,7 +237,8 @@ def test_trainer_method_takes_the_single_pass(amd, loss_type, beta, is_ratio):
         num_items_in_batch=cmask.sum().float(), old_per_token_logps=base + 0.3 * torch.randn(base.shape, generator=g, device=DEV),
         ref_per_token_logps=base + 0.1 * torch.randn(base.shape, generator=g, device=DEV),
         importance_sampling_ratio=0.5 + torch.rand((B, K), generator=g, device=DEV))
-    case = dict(temperature=0.8, beta=beta, loss_type=loss_type, eps_low=0.2, eps_high=0.28, is_ratio=is_ratio, grad_accum=2)
+    case = dict(temperature=0.8, beta=beta, loss_type=loss_type, eps_low=0.2, eps_high=0.28, is_ratio=is_ratio, grad_accum=2,
+                entropy_coef=ent_coef)
     results = []
     for single in (False, True):
         tr = _fake_trainer(amd, case, K, skip_masked=True, single_pass=single)

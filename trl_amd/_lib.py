@@ -52,8 +52,8 @@ SIGNATURES = {
     "trlk_grpo_fused_fwd_bwd": (
         c_int32,
         [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
-         c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_float, c_float, c_float, c_float, c_int32,
-         c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int32,
+         c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_float, c_float, c_float, c_float,
+         c_int32, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int32,
          c_void_p, c_void_p],
     ),
     "trlk_scale_unless_one": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),

@@ -25,6 +25,7 @@ struct FusedArgs {
     const int64_t* index;  // [n_seq * rows_per_seq]
     float temperature;
     const float *old_logp, *ref_logp, *adv, *mask, *token_weight, *row_scale, *seq_coef;
+    const float* ent_weight;  // [rows] d loss / d entropy of the token, already normalised, or null
     int64_t adv_stride_b, adv_stride_t;
     int policy_term;
     float eps_low, eps_high, delta, beta;
@@ -83,6 +84,7 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     const float w = a.token_weight ? a.token_weight[row] : 1.f;
     const float coef = a.seq_coef ? a.seq_coef[b] : 0.f;
     const float scale = a.row_scale[b];
+    const float h = a.ent_weight ? a.ent_weight[row] : 0.f;
     const float inv_t = 1.f / a.temperature, c = kLog2e * inv_t;
 
     // lane maximum, then the lane's sums relative to it
@@ -150,8 +152,10 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     grpo_token_terms(a, p, c_raw, lp, w, ref_lp, pl, kl, g_lnc, g_lp);
     float g = (g_lp + g_lnc) * m * scale;
     if (!idx_ok) g = 0.f;  // an invalid index leaves a zero row (its log-prob is NaN and the flag is set)
-    const float a0 = -g * inv_t;
-    // dlogits[v] = -g p_v / T (+ g / T at the target), p_v = 2^(x c - lse2)
+    // dlogits[v] = p_v (a0 + b0 tt_v) (+ g / T at the target), p_v = 2^tt_v, tt_v = x c - lse2 = (z_v - lse) log2(e):
+    // -g p_v / T from the log-prob, -h p_v ((z_v - lse) + H) / T from the entropy
+    const float a0 = (-g - h * ent) * inv_t;
+    const float b0 = -h * kLn2 * inv_t;
 #pragma unroll
     for (int j = 0; j < kMaxVec; ++j) {
         const int v = j * kFThreads + tid;
@@ -159,7 +163,10 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
             float x[EPV], d[EPV];
             E::unpack(q[j], x);
 #pragma unroll
-            for (int i = 0; i < EPV; ++i) d[i] = a0 * fast_exp2(fmaf(x[i], c, -lse2));
+            for (int i = 0; i < EPV; ++i) {
+                const float tt = fmaf(x[i], c, -lse2);
+                d[i] = fast_exp2(tt) * fmaf(b0, tt, a0);
+            }
             __builtin_nontemporal_store(E::pack(d), op + v);
         }
     }
@@ -167,7 +174,8 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     // address: ordered after its first store)
     if (idx_ok && int((idx / EPV) % kFThreads) == tid) {
         T* out = reinterpret_cast<T*>(op);
-        E::store1(out + idx, a0 * fast_exp2(fmaf(x_t, c, -lse2)) + g * inv_t);
+        const float tt = fmaf(x_t, c, -lse2);
+        E::store1(out + idx, fast_exp2(tt) * fmaf(b0, tt, a0) + g * inv_t);
     }
 }
 
@@ -217,7 +225,7 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
                                        const float* d_old_logp, const float* d_ref_logp, const float* d_advantages,
                                        int64_t adv_stride_b, int64_t adv_stride_t, const float* d_mask,
                                        const float* d_token_weight, const float* d_seq_coef, const float* d_row_scale,
-                                       int policy_term, float epsilon_low, float epsilon_high, float delta, float beta,
+                                       const float* d_entropy_weight, int policy_term, float epsilon_low, float epsilon_high, float delta, float beta,
                                        int use_bias_correction_kl, float sapo_temperature_pos, float sapo_temperature_neg,
                                        float* d_out_logp, float* d_out_entropy, float* d_out_lse, void* d_dlogits,
                                        int64_t out_rows_per_seq, int64_t out_row_offset, int64_t out_seq_stride,
@@ -268,6 +276,7 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
     a.mask = d_mask;
     a.token_weight = d_token_weight;
     a.row_scale = d_row_scale;
+    a.ent_weight = d_entropy_weight;
     a.seq_coef = d_seq_coef;
     a.adv_stride_b = adv_stride_b;
     a.adv_stride_t = adv_stride_t;

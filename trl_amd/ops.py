@@ -332,12 +332,12 @@ def grpo_fused_fwd_bwd(
     row_scale: Tensor, old_logp: Optional[Tensor], ref_logp: Optional[Tensor], token_weight: Optional[Tensor],
     seq_coef: Optional[Tensor], policy_term: int, epsilon_low: float, epsilon_high: float, delta: float, beta: float,
     use_bias_correction_kl: bool, sapo_temperature_pos: float, sapo_temperature_neg: float,
-    compute_masked_rows: bool = False,
+    compute_masked_rows: bool = False, entropy_weight: Optional[Tensor] = None,
 ) -> tuple[Tensor, Tensor, Tensor, Tensor]:
     """One pass over `logits[:, keep_start : keep_start + keep_len]` (`[B, L, V]`, 16-bit): returns
     `(logp [B, K], entropy [B, K], lse [B, K], dlogits [B, L, V])`, the gradient for an upstream gradient of 1 on
     the loss whose per-sequence normalisation is `row_scale [B]`.  Rows with `mask == 0` are not read (outputs 0)
-    unless `compute_masked_rows`."""
+    unless `compute_masked_rows`.  `entropy_weight [B, K]` is d loss / d entropy per token (entropy bonus)."""
     _check_logits3d(logits)
     n_seq, length, vocab = logits.shape
     dev = logits.device
@@ -347,7 +347,9 @@ def grpo_fused_fwd_bwd(
     if index.dtype != torch.int64:
         index = index.long()
     mask, old_logp, ref_logp, token_weight = _f32c(mask), _f32c(old_logp), _f32c(ref_logp), _f32c(token_weight)
-    for name, t in (("old_logp", old_logp), ("ref_logp", ref_logp), ("token_weight", token_weight)):
+    entropy_weight = _f32c(entropy_weight)
+    for name, t in (("old_logp", old_logp), ("ref_logp", ref_logp), ("token_weight", token_weight),
+                    ("entropy_weight", entropy_weight)):
         if t is not None and tuple(t.shape) != (n_seq, keep_len):
             raise ValueError(f"grpo_fused: {name} has shape {tuple(t.shape)}, expected {(n_seq, keep_len)}")
     advantages = _f32c(advantages)
@@ -373,7 +375,7 @@ def grpo_fused_fwd_bwd(
             lib.trlk_grpo_fused_fwd_bwd(
                 view.data_ptr(), dtype_code(logits.dtype), n_seq, keep_len, vocab, view.stride(0), view.stride(1),
                 ptr(index), temperature, ptr(old_logp), ptr(ref_logp), ptr(advantages), sb, st, ptr(mask),
-                ptr(token_weight), ptr(seq_coef), ptr(row_scale), policy_term, epsilon_low, epsilon_high, delta, beta,
+                ptr(token_weight), ptr(seq_coef), ptr(row_scale), ptr(entropy_weight), policy_term, epsilon_low, epsilon_high, delta, beta,
                 int(use_bias_correction_kl), sapo_temperature_pos, sapo_temperature_neg, ptr(logp), ptr(ent), ptr(lse),
                 ptr(dlogits), length, keep_start, dlogits.stride(0), dlogits.stride(1), int(compute_masked_rows),
                 ptr(_error_flag(dev)), current_stream(dev),

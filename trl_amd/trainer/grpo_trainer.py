@@ -230,11 +230,12 @@ _SINGLE_PASS_LOSS_TYPES = ("grpo", "bnpo", "dr_grpo", "dapo", "cispo", "sapo")
 def grpo_single_pass_supported(logits: Tensor, loss_type: str = "dapo", importance_sampling_level: str = "token",
                                entropy_coef: float = 0.0, entropy_mask: Tensor | None = None) -> bool:
     """Whether `grpo_loss_from_logits` can go from these logits to their gradient in one pass: a token-level
-    loss type without entropy term (the gradient coefficient of a token then depends on nothing but that
-    token), 16-bit logits whose rows fit one workgroup's registers and are 16-byte aligned."""
+    loss type, with or without entropy bonus but without an entropy-quantile mask (the gradient coefficients of
+    a token then depend on nothing but that token), 16-bit logits whose rows fit one workgroup's registers and
+    are 16-byte aligned."""
     if loss_type not in _SINGLE_PASS_LOSS_TYPES or importance_sampling_level != "token":
         return False
-    if entropy_coef != 0.0 or entropy_mask is not None:
+    if entropy_mask is not None:  # (a mask derived from every token's entropy needs the forward pass first)
         return False
     if logits.dim() != 3 or not logits.is_cuda or logits.dtype not in (torch.bfloat16, torch.float16):
         return False
@@ -275,13 +276,19 @@ class _GRPOFromLogits(torch.autograd.Function):
             n_items = (n_items.to(device=logits.device, dtype=torch.float32) if torch.is_tensor(n_items)
                        else torch.tensor(float(n_items), dtype=torch.float32, device=logits.device))
             row_scale = (1.0 / (n_items.clamp(min=1.0) / float(kw["num_processes"]))).reshape(1).expand(n_seq)
+        ent_weight = None
+        if kw["entropy_coef"] != 0.0:  # d loss / d entropy = -coef * mask / normaliser (grpo_trainer.py:3155-3181)
+            if reduce_code == _lib.DAPO:
+                ent_weight = mask_f * (-float(kw["entropy_coef"]) * row_scale[0])
+            else:
+                ent_weight = mask_f * (-float(kw["entropy_coef"]) / mask_f.sum().clamp(min=1.0) / ga)
         delta = kw["delta"]
         logp, ent, _, dlogits = ops.grpo_fused_fwd_bwd(
             logits, ids, float(temperature), keep_start, keep_len, mask_f, advantages, row_scale,
             kw["old_per_token_logps"], kw["ref_per_token_logps"] if kw["beta"] != 0.0 else None, kw["token_weight"],
             None, term_code, float(kw["epsilon_low"]), float(kw["epsilon_high"]),
             math.nan if delta is None else float(delta), float(kw["beta"]), bool(kw["use_bias_correction_kl"]),
-            float(kw["sapo_temperature_pos"]), float(kw["sapo_temperature_neg"]), not kw["skip_masked_rows"])
+            float(kw["sapo_temperature_pos"]), float(kw["sapo_temperature_neg"]), not kw["skip_masked_rows"], ent_weight)
         # loss value and every metric from the [B, K]-sized kernel, on the log-probs of the same pass
         loss, metrics = grpo_loss(
             logp, advantages, mask_f, entropies=ent, old_per_token_logps=kw["old_per_token_logps"],
@@ -290,6 +297,7 @@ class _GRPOFromLogits(torch.autograd.Function):
             max_completion_length=kw["max_completion_length"], num_items_in_batch=kw["num_items_in_batch"],
             num_processes=kw["num_processes"], grad_accum_steps=kw["grad_accum_steps"],
             use_bias_correction_kl=kw["use_bias_correction_kl"], token_weight=kw["token_weight"],
+            entropy_coef=kw["entropy_coef"],
             sapo_temperature_pos=kw["sapo_temperature_pos"], sapo_temperature_neg=kw["sapo_temperature_neg"])
         ctx.save_for_backward(dlogits)
         ctx.mark_non_differentiable(metrics, logp, ent)
@@ -324,6 +332,7 @@ def grpo_loss_from_logits(
     grad_accum_steps: float = 1.0,
     use_bias_correction_kl: bool = False,
     token_weight: Tensor | None = None,
+    entropy_coef: float = 0.0,
     sapo_temperature_pos: float = 1.0,
     sapo_temperature_neg: float = 1.05,
     skip_masked_rows: bool = True,
@@ -367,14 +376,14 @@ def grpo_loss_from_logits(
             ref_per_token_logps=ref_per_token_logps, loss_type=loss_type, epsilon_low=epsilon_low,
             epsilon_high=epsilon_high, beta=beta, delta=delta, max_completion_length=max_completion_length,
             num_items_in_batch=num_items_in_batch, num_processes=num_processes, grad_accum_steps=grad_accum_steps,
-            use_bias_correction_kl=use_bias_correction_kl, token_weight=token_weight,
+            use_bias_correction_kl=use_bias_correction_kl, token_weight=token_weight, entropy_coef=entropy_coef,
             sapo_temperature_pos=sapo_temperature_pos, sapo_temperature_neg=sapo_temperature_neg)
         return loss, metrics, logp.detach(), ent.detach()
     kw = dict(old_per_token_logps=old_per_token_logps, ref_per_token_logps=ref_per_token_logps, loss_type=loss_type,
               epsilon_low=epsilon_low, epsilon_high=epsilon_high, beta=beta, delta=delta,
               max_completion_length=max_completion_length, num_items_in_batch=num_items_in_batch,
               num_processes=num_processes, grad_accum_steps=grad_accum_steps,
-              use_bias_correction_kl=use_bias_correction_kl, token_weight=token_weight,
+              use_bias_correction_kl=use_bias_correction_kl, token_weight=token_weight, entropy_coef=entropy_coef,
               sapo_temperature_pos=sapo_temperature_pos, sapo_temperature_neg=sapo_temperature_neg,
               skip_masked_rows=skip_masked_rows, keep_start=keep_start)
     return _GRPOFromLogits.apply(logits, completion_ids, advantages, mask, temperature, kw)
@@ -442,10 +451,16 @@ class GRPOLossMixin:
         grad_accum = self.current_gradient_accumulation_steps if mode == "train" else 1.0
         bonus = bool(getattr(self, "_entropy_bonus_enabled", False))
         # One pass over the logits (log-probs and gradient from the same read) when nothing between the two
-        # needs the log-probs of other tokens: token-level weights, no entropy term, no mask derived from the
-        # log-probs or entropies.  `trl_amd_single_pass = False` on the trainer keeps the two-pass path.
+        # needs the log-probs of other tokens: token-level weights, no mask derived from the log-probs or
+        # entropies.  `trl_amd_single_pass = False` on the trainer keeps the two-pass path.
+        adaptive = bonus and bool(getattr(self, "use_adaptive_entropy", False))
+        # the coefficient of the end of the previous optimizer step applies to the whole accumulation window;
+        # under adaptive control only while the last window's entropy was at or below the target (:3173-3179)
+        apply_coef = self.entropy_coef if bonus else 0.0
+        if adaptive and not (self._last_world_entropy <= self.args.entropy_target):
+            apply_coef = 0.0
         single_pass = (
-            getattr(self, "trl_amd_single_pass", True) and skip is not None and not bonus
+            getattr(self, "trl_amd_single_pass", True) and skip is not None
             and self.loss_type in _SINGLE_PASS_LOSS_TYPES and self.importance_sampling_level == "token"
             and self.top_entropy_quantile >= 1.0 and self.off_policy_mask_threshold is None
         )
@@ -473,12 +488,13 @@ class GRPOLossMixin:
                     beta=self.beta, delta=self.args.delta, max_completion_length=self.max_completion_length,
                     num_items_in_batch=inputs.get("num_items_in_batch"), num_processes=self.accelerator.num_processes,
                     grad_accum_steps=grad_accum, use_bias_correction_kl=self.args.use_bias_correction_kl,
-                    token_weight=token_weight, sapo_temperature_pos=getattr(self.args, "sapo_temperature_pos", 1.0),
+                    token_weight=token_weight, entropy_coef=apply_coef,
+                    sapo_temperature_pos=getattr(self.args, "sapo_temperature_pos", 1.0),
                     sapo_temperature_neg=getattr(self.args, "sapo_temperature_neg", 1.05))
                 return self._finish_loss(loss, metrics, entropies, mask, None, aux_loss, aux_enabled, grad_accum, mode, bonus)
             # these logits need the two-pass kernels (fp32, a vocabulary too large for one workgroup, ...)
             per_token_logps, entropies = per_token_logps_and_entropies(
-                logits, input_ids, logits_to_keep, self.temperature, True, False, skip)
+                logits, input_ids, logits_to_keep, self.temperature, True, bonus, skip)
         else:
             per_token_logps, entropies, aux_loss = self._get_per_token_logps_and_entropies(
                 model, input_ids, attention_mask, logits_to_keep, compute_entropy=True, compute_aux_loss=aux_enabled,
@@ -501,12 +517,6 @@ class GRPOLossMixin:
             isr = inputs["importance_sampling_ratio"].float().expand_as(per_token_logps)
             token_weight = isr if token_weight is None else token_weight * isr
 
-        adaptive = bonus and bool(getattr(self, "use_adaptive_entropy", False))
-        # the coefficient of the end of the previous optimizer step applies to the whole accumulation window;
-        # under adaptive control only while the last window's entropy was at or below the target (:3173-3179)
-        apply_coef = self.entropy_coef if bonus else 0.0
-        if adaptive and not (self._last_world_entropy <= self.args.entropy_target):
-            apply_coef = 0.0
         loss, metrics = grpo_loss(
             per_token_logps, advantages, mask, entropies=entropies, old_per_token_logps=old,
             ref_per_token_logps=inputs["ref_per_token_logps"] if self.beta != 0.0 else None,
