@@ -311,3 +311,23 @@ def test_without_gradient_only_the_forward_runs(amd):
     torch.testing.assert_close(got[1], want[1], rtol=1e-5, atol=1e-6, equal_nan=True)
     torch.testing.assert_close(got[2], want[2], rtol=0, atol=1e-5)
     torch.testing.assert_close(got[3], want[3], rtol=0, atol=1e-5)
+
+
+def test_kernel_reads_masked_rows_when_asked(amd):
+    """`compute_masked_rows` of the C entry point (the Python operator fills those outputs with the streaming
+    forward kernel instead): log-prob and entropy of every row, the same gradient."""
+    from trl_amd import ops
+
+    B, K, V = 4, 12, 1024
+    logits, ids, mask, adv, _ = _inputs(B, K, V, seed=41, extra_rows=0)
+    scale = torch.full((B,), 0.01, device=DEV)
+    args = (logits, ids, 0.9, 0, K, mask.float(), adv, scale, None, None, None, None, 0, 0.2, 0.2, float("nan"), 0.0, False,
+            1.0, 1.05)
+    lp_a, ent_a, lse_a, g_a = ops.grpo_fused_fwd_bwd(*args, True)
+    lp_s, ent_s, lse_s, g_s = ops.grpo_fused_fwd_bwd(*args, False)
+    want_lp, want_ent = amd.logps_and_entropies(logits, ids, 0.9)
+    torch.testing.assert_close(lp_a, want_lp, rtol=0, atol=1e-5)
+    torch.testing.assert_close(ent_a, want_ent, rtol=0, atol=1e-5)
+    m = mask.bool()
+    assert torch.equal(lp_a[m], lp_s[m]) and float(lp_s[~m].abs().max()) == 0.0
+    assert torch.equal(g_a, g_s)

@@ -288,7 +288,15 @@ class _GRPOFromLogits(torch.autograd.Function):
             kw["old_per_token_logps"], kw["ref_per_token_logps"] if kw["beta"] != 0.0 else None, kw["token_weight"],
             None, term_code, float(kw["epsilon_low"]), float(kw["epsilon_high"]),
             math.nan if delta is None else float(delta), float(kw["beta"]), bool(kw["use_bias_correction_kl"]),
-            float(kw["sapo_temperature_pos"]), float(kw["sapo_temperature_neg"]), not kw["skip_masked_rows"], ent_weight)
+            float(kw["sapo_temperature_pos"]), float(kw["sapo_temperature_neg"]), False, ent_weight)
+        if not kw["skip_masked_rows"] and keep_len > 0:
+            # the outputs of the rows without gradient come from the streaming forward kernel, which reads them
+            # faster than the one-workgroup-per-CU kernel would (its `compute_masked_rows` mode)
+            rest = (mask_f == 0).to(torch.uint8)
+            lp0, ent0, _ = ops.logp_entropy_fwd(logits.detach(), ids.reshape(-1, 1), float(temperature), keep_start,
+                                                keep_len, rest.reshape(-1).contiguous())
+            logp = torch.where(rest.bool(), lp0.view_as(logp), logp)
+            ent = torch.where(rest.bool(), ent0.view_as(ent), ent)
         # loss value and every metric from the [B, K]-sized kernel, on the log-probs of the same pass
         loss, metrics = grpo_loss(
             logp, advantages, mask_f, entropies=ent, old_per_token_logps=kw["old_per_token_logps"],
