@@ -167,7 +167,7 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
                 const float tt = fmaf(x[i], c, -lse2);
                 d[i] = fast_exp2(tt) * fmaf(b0, tt, a0);
             }
-            __builtin_nontemporal_store(E::pack(d), op + v);
+            op[v] = E::pack(d);  // (plain: measured 3 % faster than non-temporal here; the zero-fill above is faster non-temporal)
         }
     }
     // one-hot term: the lane that stored the target's vector rewrites that element (same lane, same
