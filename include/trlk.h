@@ -175,6 +175,27 @@ int trlk_grpo_loss(const float* d_logp, const float* d_old_logp, const float* d_
                    float* d_out_dlogp, float* d_out_dentropy, void* d_workspace, size_t workspace_bytes,
                    trlk_stream_t stream);
 
+/* trlk_grpo_loss_static: trlk_grpo_loss without the workspace argument, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The per-sequence partial sums live in a device array built into the library
+ * (512 KiB per GPU, held until the process ends), so n_seq is limited to trlk_grpo_loss_static_max_seq() = 8192;
+ * more sequences are rejected with TRLK_ERR_WORKSPACE.  The call allocates and frees nothing.  All calls on one GPU
+ * share that GPU's array: calls that overlap on one GPU (different streams or threads) race and must be serialised by
+ * the caller.  Same arguments, outputs and bit-exact results as trlk_grpo_loss.
+ * trlk_init looks up the array's address on the current device (once per device); a caller that captures graphs
+ * calls it beforehand, with each device current -- otherwise the first trlk_grpo_loss_static call on a device does it. */
+int trlk_init(void);
+int64_t trlk_grpo_loss_static_max_seq(void);
+int trlk_grpo_loss_static(const float* d_logp, const float* d_old_logp, const float* d_ref_logp, const float* d_entropy,
+                          const float* d_advantages, int64_t adv_stride_b, int64_t adv_stride_t, const float* d_mask,
+                          const float* d_token_weight, const float* d_entropy_mask, const float* d_seq_coef,
+                          int64_t n_seq, int64_t seq_len, int32_t loss_type, int32_t policy_term, int32_t sequence_level,
+                          float epsilon_low, float epsilon_high, float delta, float beta, int32_t use_bias_correction_kl,
+                          float grad_accum_steps, float dr_grpo_denominator, const float* d_dapo_normalizer,
+                          float num_processes, float entropy_coef, float sapo_temperature_pos,
+                          float sapo_temperature_neg, float* d_out_loss, float* d_out_metrics, float* d_out_dlogp,
+                          float* d_out_dentropy, trlk_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------
  * K4  sequence-level losses on top of per-token log-probs.
  *

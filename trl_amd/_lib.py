@@ -48,6 +48,14 @@ SIGNATURES = {
          c_void_p, c_float, c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
          c_void_p],
     ),
+    "trlk_init": (c_int32, []),
+    "trlk_grpo_loss_static_max_seq": (c_int64, []),
+    "trlk_grpo_loss_static": (
+        c_int32,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_int64, c_int32, c_int32, c_int32, c_float, c_float, c_float, c_float, c_int32, c_float, c_float,
+         c_void_p, c_float, c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
     "trlk_grpo_fused_max_vocab": (c_int64, [c_int32]),
     "trlk_grpo_fused_fwd_bwd": (
         c_int32,

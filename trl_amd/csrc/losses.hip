@@ -5,6 +5,8 @@
 // every reduction has a fixed combination order (no float atomics), one workgroup owns one
 // sequence, and the final cross-sequence reduction is recomputed identically by every
 // workgroup instead of being passed through a third launch.
+#include <mutex>
+
 #include "common.hpp"
 #include "grpo_token.hpp"
 
@@ -454,6 +456,74 @@ extern "C" size_t trlk_grpo_workspace_bytes(int64_t n_seq) {
     return n_seq > 0 ? size_t(n_seq) * kRowStats * sizeof(float) : 0;
 }
 
+namespace {
+
+struct GrpoLossCall {
+    const float *d_logp, *d_old_logp, *d_ref_logp, *d_entropy, *d_advantages;
+    int64_t adv_stride_b, adv_stride_t;
+    const float *d_mask, *d_token_weight, *d_entropy_mask, *d_seq_coef;
+    int64_t n_seq, seq_len;
+    int32_t loss_type, policy_term, sequence_level;
+    float epsilon_low, epsilon_high, delta, beta;
+    int32_t use_bias_correction_kl;
+    float grad_accum_steps, dr_grpo_denominator;
+    const float* d_dapo_normalizer;
+    float num_processes, entropy_coef, sapo_temperature_pos, sapo_temperature_neg;
+    float *d_out_loss, *d_out_metrics, *d_out_dlogp, *d_out_dentropy;
+};
+
+// Argument checks shared by the two GRPO-loss entry points (everything but the workspace).
+int grpo_loss_validate(const GrpoLossCall& c) {
+    TRLK_REQUIRE(c.n_seq >= 1 && c.seq_len >= 1, TRLK_ERR_BAD_SHAPE, "grpo_loss: need n_seq >= 1 and seq_len >= 1 (got %lld x %lld)",
+                 (long long)c.n_seq, (long long)c.seq_len);
+    TRLK_REQUIRE(c.n_seq < (int64_t(1) << 31), TRLK_ERR_BAD_SHAPE, "grpo_loss: too many sequences");
+    TRLK_REQUIRE(c.loss_type >= TRLK_GRPO && c.loss_type <= TRLK_LUSPO, TRLK_ERR_BAD_VALUE, "grpo_loss: unknown loss_type %d",
+                 c.loss_type);
+    TRLK_REQUIRE(c.policy_term >= TRLK_TERM_CLIP && c.policy_term <= TRLK_TERM_WEIGHTED_LOGP, TRLK_ERR_BAD_VALUE,
+                 "grpo_loss: unknown policy_term %d", c.policy_term);
+    TRLK_REQUIRE(c.policy_term != TRLK_TERM_WEIGHTED_LOGP || c.d_seq_coef != nullptr, TRLK_ERR_NULL_POINTER,
+                 "grpo_loss: the weighted-logp policy term needs the per-sequence coefficients");
+    TRLK_REQUIRE(c.policy_term != TRLK_TERM_SAPO || (c.sapo_temperature_pos > 0.f && c.sapo_temperature_neg > 0.f),
+                 TRLK_ERR_BAD_VALUE, "grpo_loss: SAPO temperatures must be positive");
+    TRLK_REQUIRE(c.loss_type != TRLK_LUSPO || (c.sequence_level && c.beta == 0.f && c.d_token_weight == nullptr),
+                 TRLK_ERR_UNSUPPORTED,
+                 "grpo_loss: LUSPO is built for sequence-level importance weights without KL term or token weights");
+    TRLK_REQUIRE(!c.sequence_level || c.adv_stride_t == 0, TRLK_ERR_UNSUPPORTED,
+                 "grpo_loss: sequence-level importance weights need one advantage per sequence");
+    TRLK_REQUIRE(c.d_logp && c.d_advantages && c.d_mask && c.d_out_loss && c.d_out_metrics && c.d_out_dlogp, TRLK_ERR_NULL_POINTER,
+                 "grpo_loss: a required pointer is null");
+    TRLK_REQUIRE(c.beta == 0.f || c.d_ref_logp != nullptr, TRLK_ERR_NULL_POINTER,
+                 "grpo_loss: beta != 0 needs the reference log-probs");
+    TRLK_REQUIRE(c.entropy_coef == 0.f || (c.d_entropy != nullptr && c.d_out_dentropy != nullptr), TRLK_ERR_NULL_POINTER,
+                 "grpo_loss: entropy_coef != 0 needs entropy and out_dentropy");
+    TRLK_REQUIRE(c.loss_type != TRLK_DAPO || c.d_dapo_normalizer != nullptr, TRLK_ERR_NULL_POINTER,
+                 "grpo_loss: the DAPO loss needs the num_items_in_batch device scalar");
+    TRLK_REQUIRE(c.loss_type != TRLK_DR_GRPO || c.dr_grpo_denominator > 0.f, TRLK_ERR_BAD_VALUE,
+                 "grpo_loss: dr_grpo_denominator must be positive");
+    TRLK_REQUIRE(c.grad_accum_steps > 0.f && c.num_processes > 0.f, TRLK_ERR_BAD_VALUE,
+                 "grpo_loss: grad_accum_steps and num_processes must be positive");
+    TRLK_REQUIRE(c.epsilon_low == c.epsilon_low && c.epsilon_high == c.epsilon_high, TRLK_ERR_BAD_VALUE, "grpo_loss: epsilon is NaN");
+    return TRLK_OK;
+}
+
+// The two launches of the GRPO loss; `ws` holds kRowStats floats per sequence, all of which the first
+// kernel writes before the second reads them (nothing has to be cleared).
+int grpo_loss_launch(const GrpoLossCall& c, float* ws, trlk_stream_t stream) {
+    GrpoArgs a{c.d_logp, c.d_old_logp, c.d_ref_logp, c.d_entropy, c.d_advantages, c.d_mask, c.d_token_weight,
+               c.d_entropy_mask, c.d_seq_coef, c.adv_stride_b, c.adv_stride_t, c.n_seq, c.seq_len, c.loss_type,
+               c.policy_term, c.sequence_level != 0, c.epsilon_low, c.epsilon_high, c.delta, c.beta,
+               c.use_bias_correction_kl, c.grad_accum_steps, c.dr_grpo_denominator, c.d_dapo_normalizer,
+               c.num_processes, c.entropy_coef, c.sapo_temperature_pos, c.sapo_temperature_neg, c.d_out_loss,
+               c.d_out_metrics, c.d_out_dlogp, c.d_out_dentropy, ws};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(grpo_rows_kernel, dim3((unsigned)c.n_seq), dim3(kThreads), 0, s, a);
+    if (int rc = launch_status("grpo_loss (rows)")) return rc;
+    hipLaunchKernelGGL(grpo_finish_kernel, dim3((unsigned)c.n_seq), dim3(kThreads), 0, s, a);
+    return launch_status("grpo_loss (finish)");
+}
+
+}  // namespace
+
 extern "C" int trlk_grpo_loss(const float* d_logp, const float* d_old_logp, const float* d_ref_logp,
                               const float* d_entropy, const float* d_advantages, int64_t adv_stride_b,
                               int64_t adv_stride_t, const float* d_mask, const float* d_token_weight,
@@ -465,47 +535,85 @@ extern "C" int trlk_grpo_loss(const float* d_logp, const float* d_old_logp, cons
                               float sapo_temperature_neg, float* d_out_loss, float* d_out_metrics, float* d_out_dlogp,
                               float* d_out_dentropy, void* d_workspace, size_t workspace_bytes, trlk_stream_t stream) {
     clear_error();
-    TRLK_REQUIRE(n_seq >= 1 && seq_len >= 1, TRLK_ERR_BAD_SHAPE, "grpo_loss: need n_seq >= 1 and seq_len >= 1 (got %lld x %lld)",
-                 (long long)n_seq, (long long)seq_len);
-    TRLK_REQUIRE(n_seq < (int64_t(1) << 31), TRLK_ERR_BAD_SHAPE, "grpo_loss: too many sequences");
-    TRLK_REQUIRE(loss_type >= TRLK_GRPO && loss_type <= TRLK_LUSPO, TRLK_ERR_BAD_VALUE, "grpo_loss: unknown loss_type %d",
-                 loss_type);
-    TRLK_REQUIRE(policy_term >= TRLK_TERM_CLIP && policy_term <= TRLK_TERM_WEIGHTED_LOGP, TRLK_ERR_BAD_VALUE,
-                 "grpo_loss: unknown policy_term %d", policy_term);
-    TRLK_REQUIRE(policy_term != TRLK_TERM_WEIGHTED_LOGP || d_seq_coef != nullptr, TRLK_ERR_NULL_POINTER,
-                 "grpo_loss: the weighted-logp policy term needs the per-sequence coefficients");
-    TRLK_REQUIRE(policy_term != TRLK_TERM_SAPO || (sapo_temperature_pos > 0.f && sapo_temperature_neg > 0.f),
-                 TRLK_ERR_BAD_VALUE, "grpo_loss: SAPO temperatures must be positive");
-    TRLK_REQUIRE(loss_type != TRLK_LUSPO || (sequence_level && beta == 0.f && d_token_weight == nullptr),
-                 TRLK_ERR_UNSUPPORTED,
-                 "grpo_loss: LUSPO is built for sequence-level importance weights without KL term or token weights");
-    TRLK_REQUIRE(!sequence_level || adv_stride_t == 0, TRLK_ERR_UNSUPPORTED,
-                 "grpo_loss: sequence-level importance weights need one advantage per sequence");
-    TRLK_REQUIRE(d_logp && d_advantages && d_mask && d_out_loss && d_out_metrics && d_out_dlogp, TRLK_ERR_NULL_POINTER,
-                 "grpo_loss: a required pointer is null");
-    TRLK_REQUIRE(beta == 0.f || d_ref_logp != nullptr, TRLK_ERR_NULL_POINTER,
-                 "grpo_loss: beta != 0 needs the reference log-probs");
-    TRLK_REQUIRE(entropy_coef == 0.f || (d_entropy != nullptr && d_out_dentropy != nullptr), TRLK_ERR_NULL_POINTER,
-                 "grpo_loss: entropy_coef != 0 needs entropy and out_dentropy");
-    TRLK_REQUIRE(loss_type != TRLK_DAPO || d_dapo_normalizer != nullptr, TRLK_ERR_NULL_POINTER,
-                 "grpo_loss: the DAPO loss needs the num_items_in_batch device scalar");
-    TRLK_REQUIRE(loss_type != TRLK_DR_GRPO || dr_grpo_denominator > 0.f, TRLK_ERR_BAD_VALUE,
-                 "grpo_loss: dr_grpo_denominator must be positive");
-    TRLK_REQUIRE(grad_accum_steps > 0.f && num_processes > 0.f, TRLK_ERR_BAD_VALUE,
-                 "grpo_loss: grad_accum_steps and num_processes must be positive");
-    TRLK_REQUIRE(epsilon_low == epsilon_low && epsilon_high == epsilon_high, TRLK_ERR_BAD_VALUE, "grpo_loss: epsilon is NaN");
+    const GrpoLossCall c{d_logp, d_old_logp, d_ref_logp, d_entropy, d_advantages, adv_stride_b, adv_stride_t, d_mask,
+                         d_token_weight, d_entropy_mask, d_seq_coef, n_seq, seq_len, loss_type, policy_term,
+                         sequence_level, epsilon_low, epsilon_high, delta, beta, use_bias_correction_kl,
+                         grad_accum_steps, dr_grpo_denominator, d_dapo_normalizer, num_processes, entropy_coef,
+                         sapo_temperature_pos, sapo_temperature_neg, d_out_loss, d_out_metrics, d_out_dlogp,
+                         d_out_dentropy};
+    if (int rc = grpo_loss_validate(c)) return rc;
     TRLK_REQUIRE(d_workspace != nullptr && workspace_bytes >= trlk_grpo_workspace_bytes(n_seq), TRLK_ERR_WORKSPACE,
                  "grpo_loss: workspace of %zu bytes needed, %zu given", trlk_grpo_workspace_bytes(n_seq), workspace_bytes);
-    GrpoArgs a{d_logp, d_old_logp, d_ref_logp, d_entropy, d_advantages, d_mask, d_token_weight, d_entropy_mask,
-               d_seq_coef, adv_stride_b, adv_stride_t, n_seq, seq_len, loss_type, policy_term, sequence_level != 0,
-               epsilon_low, epsilon_high, delta, beta, use_bias_correction_kl, grad_accum_steps, dr_grpo_denominator,
-               d_dapo_normalizer, num_processes, entropy_coef, sapo_temperature_pos, sapo_temperature_neg, d_out_loss,
-               d_out_metrics, d_out_dlogp, d_out_dentropy, static_cast<float*>(d_workspace)};
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(grpo_rows_kernel, dim3((unsigned)n_seq), dim3(kThreads), 0, s, a);
-    if (int rc = launch_status("grpo_loss (rows)")) return rc;
-    hipLaunchKernelGGL(grpo_finish_kernel, dim3((unsigned)n_seq), dim3(kThreads), 0, s, a);
-    return launch_status("grpo_loss (finish)");
+    return grpo_loss_launch(c, static_cast<float*>(d_workspace), stream);
+}
+
+// ---- the GRPO loss for callers that cannot allocate: its per-sequence partial sums live in a file-scope device
+// array instead of a caller workspace.  Every GPU the library runs on holds its own copy of the array (at its own
+// address) until the process ends; every call on a GPU shares that GPU's copy, so calls that overlap on one GPU
+// (two streams, two threads) race.  The array keeps the previous call's contents; nothing needs clearing because
+// the first kernel writes every float the second one reads.
+constexpr int64_t kStaticMaxSeq = 8192;  // 8192 sequences * 16 floats = 512 KiB per GPU
+static __device__ __align__(256) float grpo_static_scratch[kStaticMaxSeq * kRowStats];
+
+namespace {
+constexpr int kMaxDevices = 64;
+float* g_static_scratch_ptr[kMaxDevices] = {};  // device address of grpo_static_scratch per GPU (0 = not yet asked)
+std::mutex g_static_scratch_mutex;
+
+// The array's name is a host-side handle, not a device address: the address on the current device comes from
+// hipGetSymbolAddress, once per device, and is what kernels get.
+int static_scratch_for_current_device(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(int(e), "grpo_loss_static: hipGetDevice failed: %s", hipGetErrorString(e));
+    TRLK_REQUIRE(dev >= 0 && dev < kMaxDevices, TRLK_ERR_UNSUPPORTED, "grpo_loss_static: device ordinal %d is out of range", dev);
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (g_static_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(grpo_static_scratch));
+        if (e != hipSuccess || p == nullptr)
+            return fail(e != hipSuccess ? int(e) : int(hipErrorInvalidSymbol), "grpo_loss_static: hipGetSymbolAddress failed: %s",
+                        hipGetErrorString(e));
+        g_static_scratch_ptr[dev] = static_cast<float*>(p);
+    }
+    *out = g_static_scratch_ptr[dev];
+    return TRLK_OK;
+}
+}  // namespace
+
+extern "C" int trlk_init(void) {
+    clear_error();
+    float* p = nullptr;
+    return static_scratch_for_current_device(&p);
+}
+
+extern "C" int64_t trlk_grpo_loss_static_max_seq(void) { return kStaticMaxSeq; }
+
+extern "C" int trlk_grpo_loss_static(const float* d_logp, const float* d_old_logp, const float* d_ref_logp,
+                                     const float* d_entropy, const float* d_advantages, int64_t adv_stride_b,
+                                     int64_t adv_stride_t, const float* d_mask, const float* d_token_weight,
+                                     const float* d_entropy_mask, const float* d_seq_coef, int64_t n_seq,
+                                     int64_t seq_len, int32_t loss_type, int32_t policy_term, int32_t sequence_level,
+                                     float epsilon_low, float epsilon_high, float delta, float beta,
+                                     int32_t use_bias_correction_kl, float grad_accum_steps, float dr_grpo_denominator,
+                                     const float* d_dapo_normalizer, float num_processes, float entropy_coef,
+                                     float sapo_temperature_pos, float sapo_temperature_neg, float* d_out_loss,
+                                     float* d_out_metrics, float* d_out_dlogp, float* d_out_dentropy,
+                                     trlk_stream_t stream) {
+    clear_error();
+    const GrpoLossCall c{d_logp, d_old_logp, d_ref_logp, d_entropy, d_advantages, adv_stride_b, adv_stride_t, d_mask,
+                         d_token_weight, d_entropy_mask, d_seq_coef, n_seq, seq_len, loss_type, policy_term,
+                         sequence_level, epsilon_low, epsilon_high, delta, beta, use_bias_correction_kl,
+                         grad_accum_steps, dr_grpo_denominator, d_dapo_normalizer, num_processes, entropy_coef,
+                         sapo_temperature_pos, sapo_temperature_neg, d_out_loss, d_out_metrics, d_out_dlogp,
+                         d_out_dentropy};
+    if (int rc = grpo_loss_validate(c)) return rc;
+    TRLK_REQUIRE(n_seq <= kStaticMaxSeq, TRLK_ERR_WORKSPACE,
+                 "grpo_loss_static: %lld sequences exceed the built-in scratch of %lld; use trlk_grpo_loss with a workspace",
+                 (long long)n_seq, (long long)kStaticMaxSeq);
+    float* ws = nullptr;
+    if (int rc = static_scratch_for_current_device(&ws)) return rc;
+    return grpo_loss_launch(c, ws, stream);
 }
 
 extern "C" int trlk_dpo_loss(const float* d_token_logp, const float* d_mask, const float* d_ref_chosen,

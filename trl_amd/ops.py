@@ -319,6 +319,56 @@ def _grpo_backward(ctx, g_loss, g_metrics, g_dlogp, g_dent):
 grpo_loss_op.register_autograd(_grpo_backward, setup_context=_grpo_setup)
 
 
+def grpo_loss_static_max_seq() -> int:
+    """Most sequences `grpo_loss_static_` takes (the size of the scratch array built into the library)."""
+    return int(lib.trlk_grpo_loss_static_max_seq())
+
+
+def grpo_loss_static_(
+    out_loss: Tensor, out_metrics: Tensor, out_dlogp: Tensor, out_dentropy: Optional[Tensor], logp: Tensor,
+    old_logp: Optional[Tensor], ref_logp: Optional[Tensor], entropy: Optional[Tensor], advantages: Tensor, mask: Tensor,
+    token_weight: Optional[Tensor], entropy_mask: Optional[Tensor], dapo_normalizer: Optional[Tensor], loss_type: int,
+    epsilon_low: float, epsilon_high: float, delta: float, beta: float, use_bias_correction_kl: bool,
+    grad_accum_steps: float, dr_grpo_denominator: float, num_processes: float, entropy_coef: float,
+    policy_term: int = 0, sequence_level: bool = False, seq_coef: Optional[Tensor] = None,
+    sapo_temperature_pos: float = 1.0, sapo_temperature_neg: float = 1.05,
+) -> None:
+    """The GRPO loss (`grpo_loss_op`'s arithmetic, bit for bit) for callers that must not allocate: every operand
+    is a contiguous fp32 device tensor the caller owns (`logp`, `mask`, ... `[B, T]`; `advantages` `[B]` or
+    `[B, T]`; outputs `out_loss []`, `out_metrics [16]`, `out_dlogp [B, T]`, `out_dentropy [B, T]` when
+    `entropy_coef != 0`), nothing is converted or copied, and the kernels' partial sums go to a scratch array built
+    into the library instead of a workspace tensor.  At most `grpo_loss_static_max_seq()` sequences; calls that
+    overlap on one GPU race (they share the array).  No autograd."""
+    B, T = logp.shape
+    for name, t in (("logp", logp), ("old_logp", old_logp), ("ref_logp", ref_logp), ("entropy", entropy),
+                    ("mask", mask), ("token_weight", token_weight), ("entropy_mask", entropy_mask),
+                    ("out_dlogp", out_dlogp), ("out_dentropy", out_dentropy)):
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape) != (B, T)):
+            raise ValueError(f"grpo_loss_static_: {name} must be a contiguous fp32 [{B}, {T}] tensor")
+    if advantages.dtype != torch.float32 or not advantages.is_contiguous():
+        raise ValueError("grpo_loss_static_: advantages must be contiguous fp32")
+    if advantages.numel() == B:
+        sb, st = 1, 0
+    elif tuple(advantages.shape) == (B, T):
+        sb, st = T, 1
+    else:
+        raise ValueError(f"grpo_loss_static_: advantages of shape {tuple(advantages.shape)} do not match [B] or [B, T]")
+    if out_loss.dtype != torch.float32 or out_metrics.dtype != torch.float32 or out_metrics.numel() < _lib.GRPO_NUM_METRICS:
+        raise ValueError("grpo_loss_static_: out_loss / out_metrics must be fp32 ([] and [16])")
+    dev = logp.device
+    with torch.cuda.device(dev):
+        check(
+            lib.trlk_grpo_loss_static(
+                ptr(logp), ptr(old_logp), ptr(ref_logp), ptr(entropy), ptr(advantages), sb, st, ptr(mask),
+                ptr(token_weight), ptr(entropy_mask), ptr(seq_coef), B, T, loss_type, policy_term,
+                int(sequence_level), epsilon_low, epsilon_high, delta, beta, int(use_bias_correction_kl),
+                grad_accum_steps, dr_grpo_denominator, ptr(dapo_normalizer), num_processes, entropy_coef,
+                sapo_temperature_pos, sapo_temperature_neg, ptr(out_loss), ptr(out_metrics), ptr(out_dlogp),
+                ptr(out_dentropy), current_stream(dev),
+            )
+        )
+
+
 # --------------------------------------------------------------------------------------------
 # GRPO gradient straight from the logits (K7)
 # --------------------------------------------------------------------------------------------
