@@ -110,132 +110,217 @@ GRPO_CASES = [
 ]
 
 
+def _grpo_case(GRPOTrainer, case, seed, dims, lengths, adv_2d=False):
+    """Runs the reference's `_compute_loss` (+ backward) on one mocked trainer; returns (arrays, index entry).
+    `case["values"]` (optional) names a 16-bit dtype whose values the fp32 logits are rounded to: the reference
+    then does fp32 arithmetic on numbers a bf16 / fp16 tensor holds exactly, so a kernel that reads that 16-bit
+    tensor and accumulates in fp32 can be compared with these outputs at fp32 tolerance."""
+    g = torch.Generator().manual_seed(seed)
+    B, P, T, V = dims
+    dtype = getattr(torch, case.get("dtype", "float32"))
+    temperature = case.get("temperature", 1.0)
+    logits = (2.0 * torch.randn(B, P + T, V, generator=g)).to(dtype)
+    if case.get("values"):
+        logits = logits.to(getattr(torch, case["values"])).to(dtype)
+    prompt_ids = torch.randint(0, V, (B, P), generator=g)
+    completion_ids = torch.randint(0, V, (B, T), generator=g)
+    lengths = list(lengths)
+    if case.get("empty_row"):
+        lengths[3] = 0
+    completion_mask = _lengths_mask(lengths, T)
+    prompt_mask = torch.ones(B, P, dtype=torch.long)
+    advantages = torch.randn(B, generator=g)
+    advantages[1] = 0.0
+
+    trainer = Mock(spec=GRPOTrainer)
+    trainer.accelerator = _fake_accelerator()
+    trainer.temperature = temperature
+    trainer.model_kwarg_keys = set()
+    ad = case.get("adaptive")
+    trainer._entropy_bonus_enabled = case.get("entropy_coef", 0.0) != 0.0 or ad is not None
+    trainer.entropy_coef = case.get("entropy_coef", 0.0)
+    trainer.use_adaptive_entropy = ad is not None
+    if ad is not None:
+        trainer._last_world_entropy = ad["last"]
+        trainer._entropy_window_stats = torch.tensor(ad["window"]) if "window" in ad else None
+        trainer.accelerator.sync_gradients = ad["sync"]
+    trainer.aux_loss_enabled = False
+    trainer.top_entropy_quantile = case.get("top_entropy_quantile", 1.0)
+    trainer.off_policy_mask_threshold = case.get("off_policy")
+    trainer.importance_sampling_level = case.get("is_level", "token")
+    trainer.beta = case["beta"]
+    trainer.loss_type = case["loss_type"]
+    trainer.epsilon_low = case["eps_low"]
+    trainer.epsilon_high = case["eps_high"]
+    trainer.use_vllm = bool(case.get("is_ratio"))
+    trainer.vllm_importance_sampling_correction = bool(case.get("is_ratio"))
+    trainer.max_completion_length = T
+    trainer.current_gradient_accumulation_steps = case.get("grad_accum", 1)
+    trainer.args = SimpleNamespace(delta=case.get("delta"), use_bias_correction_kl=case.get("bias_kl", False),
+                                   sapo_temperature_pos=1.0, sapo_temperature_neg=1.05, vespo_k_pos=2.0,
+                                   vespo_lambda_pos=3.0, vespo_k_neg=3.0, vespo_lambda_neg=2.0)
+    if ad is not None:
+        trainer.args.entropy_target, trainer.args.entropy_coef_delta = ad["target"], ad["delta"]
+        trainer.args.entropy_coef_max, trainer.args.entropy_coef_min = ad["max"], ad["min"]
+    trainer.get_gamma_weights = GRPOTrainer.get_gamma_weights
+    trainer._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
+    trainer.model = SimpleNamespace(training=True)
+    trainer._get_per_token_logps_and_entropies = (
+        lambda *a, **k: GRPOTrainer._get_per_token_logps_and_entropies(trainer, *a, **k)
+    )
+    trainer.get_high_entropy_mask = lambda *a, **k: GRPOTrainer.get_high_entropy_mask(trainer, *a, **k)
+    trainer.get_off_policy_mask = GRPOTrainer.get_off_policy_mask
+
+    # old / ref log-probs: perturbations of the no-grad policy log-probs
+    input_ids = torch.cat([prompt_ids, completion_ids], 1)
+    attn = torch.cat([prompt_mask, completion_mask], 1)
+    with torch.no_grad():
+        base_logps, _, _ = GRPOTrainer._get_per_token_logps_and_entropies(
+            trainer, _FixedLogitsModel(logits), input_ids, attn, T, compute_entropy=False
+        )
+    base_logps = base_logps.float()
+    inputs = dict(
+        prompt_ids=prompt_ids,
+        prompt_mask=prompt_mask,
+        completion_ids=completion_ids,
+        completion_mask=completion_mask,
+        advantages=advantages,
+        num_items_in_batch=completion_mask.sum().float() * 2.0,  # as if a second, equal micro-batch existed
+    )
+    if not case.get("on_policy"):
+        inputs["old_per_token_logps"] = base_logps + case.get("old_noise", 0.15) * torch.randn(B, T, generator=g)
+    if case["beta"] != 0.0:
+        inputs["ref_per_token_logps"] = base_logps + 0.3 * torch.randn(B, T, generator=g)
+    if case.get("is_ratio"):
+        inputs["importance_sampling_ratio"] = 0.5 + torch.rand(B, T, generator=g)
+    if case.get("adv_2d"):  # per-token advantages, as subclasses of the trainer provide them (grpo_trainer.py:3026-3030)
+        inputs["advantages"] = advantages[:, None] * (0.5 + torch.rand(B, T, generator=g)) - 0.3 * torch.rand(B, T, generator=g)
+
+    leaf = logits.clone().requires_grad_(True)
+
+    class _Model(_FixedLogitsModel):
+        def __call__(self, input_ids=None, **kw):
+            return SimpleNamespace(logits=leaf[: input_ids.shape[0]] * 1.0, aux_loss=None)
+
+    captured = {}
+    real = GRPOTrainer._get_per_token_logps_and_entropies
+
+    def spy(*a, **k):
+        out = real(trainer, *a, **k)
+        captured["logps"], captured["entropies"] = out[0], out[1]
+        return out
+
+    trainer._get_per_token_logps_and_entropies = spy
+    loss = GRPOTrainer._compute_loss(trainer, _Model(logits), inputs)
+    loss.backward()
+
+    arrays = {}
+    arrays["logits"] = _np(logits)
+    arrays["prompt_ids"] = _np(prompt_ids)
+    arrays["completion_ids"] = _np(completion_ids)
+    arrays["completion_mask"] = _np(completion_mask)
+    arrays["advantages"] = _np(inputs["advantages"])
+    arrays["num_items_in_batch"] = _np(inputs["num_items_in_batch"])
+    if "old_per_token_logps" in inputs:
+        arrays["old_per_token_logps"] = _np(inputs["old_per_token_logps"])
+    if "ref_per_token_logps" in inputs:
+        arrays["ref_per_token_logps"] = _np(inputs["ref_per_token_logps"])
+    if "importance_sampling_ratio" in inputs:
+        arrays["importance_sampling_ratio"] = _np(inputs["importance_sampling_ratio"])
+    arrays["out_logps"] = _np(captured["logps"])
+    arrays["out_entropies"] = _np(captured["entropies"])
+    arrays["out_loss"] = _np(loss)
+    arrays["out_dlogits"] = _np(leaf.grad)
+    metrics = {k: float(v[-1]) for k, v in trainer._metrics["train"].items()}
+    entry = dict(case, id=None, shape=[B, P, T, V], metrics=metrics)
+    if ad is not None:  # the controller's state after the call
+        win = trainer._entropy_window_stats
+        entry["state_after"] = dict(entropy_coef=float(trainer.entropy_coef),
+                                    last_world_entropy=float(trainer._last_world_entropy),
+                                    window=None if win is None else [float(x) for x in win])
+    return arrays, entry
+
+
 def make_grpo(GRPOTrainer, out_dir):
     index = []
     arrays = {}
     for ci, case in enumerate(GRPO_CASES):
-        g = torch.Generator().manual_seed(1000 + ci)
-        B, P, T, V = 6, 3, 7, 41
-        dtype = getattr(torch, case.get("dtype", "float32"))
-        temperature = case.get("temperature", 1.0)
-        logits = (2.0 * torch.randn(B, P + T, V, generator=g)).to(dtype)
-        prompt_ids = torch.randint(0, V, (B, P), generator=g)
-        completion_ids = torch.randint(0, V, (B, T), generator=g)
-        lengths = [7, 3, 5, 1, 6, 4]
-        if case.get("empty_row"):
-            lengths[3] = 0
-        completion_mask = _lengths_mask(lengths, T)
-        prompt_mask = torch.ones(B, P, dtype=torch.long)
-        advantages = torch.randn(B, generator=g)
-        advantages[1] = 0.0
-
-        trainer = Mock(spec=GRPOTrainer)
-        trainer.accelerator = _fake_accelerator()
-        trainer.temperature = temperature
-        trainer.model_kwarg_keys = set()
-        ad = case.get("adaptive")
-        trainer._entropy_bonus_enabled = case.get("entropy_coef", 0.0) != 0.0 or ad is not None
-        trainer.entropy_coef = case.get("entropy_coef", 0.0)
-        trainer.use_adaptive_entropy = ad is not None
-        if ad is not None:
-            trainer._last_world_entropy = ad["last"]
-            trainer._entropy_window_stats = torch.tensor(ad["window"]) if "window" in ad else None
-            trainer.accelerator.sync_gradients = ad["sync"]
-        trainer.aux_loss_enabled = False
-        trainer.top_entropy_quantile = case.get("top_entropy_quantile", 1.0)
-        trainer.off_policy_mask_threshold = case.get("off_policy")
-        trainer.importance_sampling_level = case.get("is_level", "token")
-        trainer.beta = case["beta"]
-        trainer.loss_type = case["loss_type"]
-        trainer.epsilon_low = case["eps_low"]
-        trainer.epsilon_high = case["eps_high"]
-        trainer.use_vllm = bool(case.get("is_ratio"))
-        trainer.vllm_importance_sampling_correction = bool(case.get("is_ratio"))
-        trainer.max_completion_length = T
-        trainer.current_gradient_accumulation_steps = case.get("grad_accum", 1)
-        trainer.args = SimpleNamespace(delta=case.get("delta"), use_bias_correction_kl=case.get("bias_kl", False),
-                                       sapo_temperature_pos=1.0, sapo_temperature_neg=1.05, vespo_k_pos=2.0,
-                                       vespo_lambda_pos=3.0, vespo_k_neg=3.0, vespo_lambda_neg=2.0)
-        if ad is not None:
-            trainer.args.entropy_target, trainer.args.entropy_coef_delta = ad["target"], ad["delta"]
-            trainer.args.entropy_coef_max, trainer.args.entropy_coef_min = ad["max"], ad["min"]
-        trainer.get_gamma_weights = GRPOTrainer.get_gamma_weights
-        trainer._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
-        trainer.model = SimpleNamespace(training=True)
-        trainer._get_per_token_logps_and_entropies = (
-            lambda *a, **k: GRPOTrainer._get_per_token_logps_and_entropies(trainer, *a, **k)
-        )
-        trainer.get_high_entropy_mask = lambda *a, **k: GRPOTrainer.get_high_entropy_mask(trainer, *a, **k)
-        trainer.get_off_policy_mask = GRPOTrainer.get_off_policy_mask
-
-        # old / ref log-probs: perturbations of the no-grad policy log-probs
-        input_ids = torch.cat([prompt_ids, completion_ids], 1)
-        attn = torch.cat([prompt_mask, completion_mask], 1)
-        with torch.no_grad():
-            base_logps, _, _ = GRPOTrainer._get_per_token_logps_and_entropies(
-                trainer, _FixedLogitsModel(logits), input_ids, attn, T, compute_entropy=False
-            )
-        base_logps = base_logps.float()
-        inputs = dict(
-            prompt_ids=prompt_ids,
-            prompt_mask=prompt_mask,
-            completion_ids=completion_ids,
-            completion_mask=completion_mask,
-            advantages=advantages,
-            num_items_in_batch=completion_mask.sum().float() * 2.0,  # as if a second, equal micro-batch existed
-        )
-        if not case.get("on_policy"):
-            inputs["old_per_token_logps"] = base_logps + 0.15 * torch.randn(B, T, generator=g)
-        if case["beta"] != 0.0:
-            inputs["ref_per_token_logps"] = base_logps + 0.3 * torch.randn(B, T, generator=g)
-        if case.get("is_ratio"):
-            inputs["importance_sampling_ratio"] = 0.5 + torch.rand(B, T, generator=g)
-
-        leaf = logits.clone().requires_grad_(True)
-
-        class _Model(_FixedLogitsModel):
-            def __call__(self, input_ids=None, **kw):
-                return SimpleNamespace(logits=leaf[: input_ids.shape[0]] * 1.0, aux_loss=None)
-
-        captured = {}
-        real = GRPOTrainer._get_per_token_logps_and_entropies
-
-        def spy(*a, **k):
-            out = real(trainer, *a, **k)
-            captured["logps"], captured["entropies"] = out[0], out[1]
-            return out
-
-        trainer._get_per_token_logps_and_entropies = spy
-        loss = GRPOTrainer._compute_loss(trainer, _Model(logits), inputs)
-        loss.backward()
-
-        pre = f"c{ci}_"
-        arrays[pre + "logits"] = _np(logits)
-        arrays[pre + "prompt_ids"] = _np(prompt_ids)
-        arrays[pre + "completion_ids"] = _np(completion_ids)
-        arrays[pre + "completion_mask"] = _np(completion_mask)
-        arrays[pre + "advantages"] = _np(advantages)
-        arrays[pre + "num_items_in_batch"] = _np(inputs["num_items_in_batch"])
-        if "old_per_token_logps" in inputs:
-            arrays[pre + "old_per_token_logps"] = _np(inputs["old_per_token_logps"])
-        if "ref_per_token_logps" in inputs:
-            arrays[pre + "ref_per_token_logps"] = _np(inputs["ref_per_token_logps"])
-        if "importance_sampling_ratio" in inputs:
-            arrays[pre + "importance_sampling_ratio"] = _np(inputs["importance_sampling_ratio"])
-        arrays[pre + "out_logps"] = _np(captured["logps"])
-        arrays[pre + "out_entropies"] = _np(captured["entropies"])
-        arrays[pre + "out_loss"] = _np(loss)
-        arrays[pre + "out_dlogits"] = _np(leaf.grad)
-        metrics = {k: float(v[-1]) for k, v in trainer._metrics["train"].items()}
-        entry = dict(case, id=ci, shape=[B, P, T, V], metrics=metrics)
-        if ad is not None:  # the controller's state after the call
-            win = trainer._entropy_window_stats
-            entry["state_after"] = dict(entropy_coef=float(trainer.entropy_coef),
-                                        last_world_entropy=float(trainer._last_world_entropy),
-                                        window=None if win is None else [float(x) for x in win])
+        got, entry = _grpo_case(GRPOTrainer, case, 1000 + ci, (6, 3, 7, 41), [7, 3, 5, 1, 6, 4])
+        for k, v in got.items():
+            arrays[f"c{ci}_{k}"] = v
+        entry["id"] = ci
         index.append(entry)
     np.savez_compressed(os.path.join(out_dir, "grpo_compute_loss.npz"), **arrays)
     with open(os.path.join(out_dir, "grpo_compute_loss.json"), "w") as f:
+        json.dump(index, f, indent=1)
+
+
+# Configurations that one pass over 16-bit logits can serve (a token-level loss type, no mask derived from other
+# tokens' log-probs or entropies), on vocabularies that are multiples of 8.  Each runs twice: on logits holding
+# bf16-exact values and on logits holding fp16-exact values (fp32 arithmetic in the reference both times).
+SINGLE_PASS_CASES = [
+    dict(name="dapo_beta0", loss_type="dapo", beta=0.0, eps_low=0.2, eps_high=0.2),
+    dict(name="dapo_beta_temp", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.28, temperature=0.9),
+    dict(name="grpo_beta_ga", loss_type="grpo", beta=0.04, eps_low=0.2, eps_high=0.2, grad_accum=2, temperature=0.9),
+    dict(name="dr_grpo_beta_ga", loss_type="dr_grpo", beta=0.04, eps_low=0.1, eps_high=0.3, grad_accum=4, temperature=0.9),
+    dict(name="bnpo_beta", loss_type="bnpo", beta=0.1, eps_low=0.2, eps_high=0.2),
+    dict(name="grpo_beta0", loss_type="grpo", beta=0.0, eps_low=0.2, eps_high=0.2),
+    dict(name="dr_grpo_beta0", loss_type="dr_grpo", beta=0.0, eps_low=0.2, eps_high=0.2),
+    dict(name="bnpo_beta0_ga", loss_type="bnpo", beta=0.0, eps_low=0.05, eps_high=0.05, grad_accum=2),
+    dict(name="grpo_onpolicy", loss_type="grpo", beta=0.0, eps_low=0.2, eps_high=0.2, on_policy=True),
+    dict(name="dapo_onpolicy_beta", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, on_policy=True, temperature=0.7),
+    dict(name="dapo_delta", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, delta=1.05),
+    dict(name="bnpo_delta_beta0", loss_type="bnpo", beta=0.0, eps_low=0.03, eps_high=0.04, delta=1.02),
+    dict(name="dapo_biaskl", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, bias_kl=True),
+    dict(name="grpo_biaskl_delta_temp", loss_type="grpo", beta=0.1, eps_low=0.1, eps_high=0.1, bias_kl=True, delta=1.1,
+         temperature=0.8, grad_accum=2),
+    dict(name="grpo_entbonus", loss_type="grpo", beta=0.04, eps_low=0.2, eps_high=0.2, entropy_coef=0.01),
+    dict(name="dapo_entbonus", loss_type="dapo", beta=0.0, eps_low=0.2, eps_high=0.2, entropy_coef=0.02, temperature=0.9),
+    dict(name="bnpo_entbonus_ga", loss_type="bnpo", beta=0.0, eps_low=0.2, eps_high=0.2, entropy_coef=0.02, grad_accum=2),
+    dict(name="dr_grpo_entbonus_ga", loss_type="dr_grpo", beta=0.04, eps_low=0.2, eps_high=0.2, entropy_coef=0.02, grad_accum=2),
+    dict(name="dapo_emptyrow", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, empty_row=True),
+    dict(name="grpo_emptyrow_entbonus", loss_type="grpo", beta=0.0, eps_low=0.2, eps_high=0.2, empty_row=True, entropy_coef=0.01),
+    dict(name="cispo_beta", loss_type="cispo", beta=0.04, eps_low=0.2, eps_high=1.1),
+    dict(name="cispo_beta0_temp", loss_type="cispo", beta=0.0, eps_low=0.2, eps_high=1.05, temperature=0.9),
+    dict(name="cispo_entbonus", loss_type="cispo", beta=0.0, eps_low=0.2, eps_high=1.1, entropy_coef=0.02),
+    dict(name="sapo_beta0_ga", loss_type="sapo", beta=0.0, eps_low=0.2, eps_high=0.2, grad_accum=2),
+    dict(name="sapo_beta_temp", loss_type="sapo", beta=0.04, eps_low=0.2, eps_high=0.2, temperature=0.9),
+    dict(name="adaptive_below_target", loss_type="grpo", beta=0.04, eps_low=0.2, eps_high=0.2, entropy_coef=0.01,
+         adaptive=dict(target=5.0, delta=0.005, max=0.012, min=0.0, last=1.0, sync=True)),
+    dict(name="adaptive_above_target", loss_type="dapo", beta=0.0, eps_low=0.2, eps_high=0.2, entropy_coef=0.02,
+         adaptive=dict(target=0.5, delta=0.005, max=0.1, min=0.0, last=float("inf"), sync=True)),
+    dict(name="adaptive_accumulating", loss_type="bnpo", beta=0.0, eps_low=0.2, eps_high=0.2, entropy_coef=0.02,
+         grad_accum=2, adaptive=dict(target=5.0, delta=0.005, max=0.1, min=0.0, last=2.0, sync=False, window=[3.0, 2.0])),
+    dict(name="vllm_is_ratio_dapo", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, is_ratio=True),
+    dict(name="vllm_is_ratio_cispo", loss_type="cispo", beta=0.0, eps_low=0.2, eps_high=1.1, is_ratio=True, temperature=0.9),
+    dict(name="vllm_is_ratio_sapo_entbonus", loss_type="sapo", beta=0.04, eps_low=0.2, eps_high=0.2, is_ratio=True,
+         entropy_coef=0.01),
+    dict(name="dapo_per_token_advantages", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.28, adv_2d=True),
+    # the reference's own 16-bit arithmetic (log-probs rounded to the logits dtype): comparable at 2e-2 only
+    dict(name="dapo_true_bf16", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, dtype="bfloat16", temperature=0.9),
+    dict(name="grpo_true_fp16_entbonus", loss_type="grpo", beta=0.04, eps_low=0.2, eps_high=0.2, dtype="float16",
+         entropy_coef=0.01),
+]
+
+
+def make_grpo_single_pass(GRPOTrainer, out_dir):
+    index, arrays = [], {}
+    vocabs = (48, 264, 56, 72)
+    ci = 0
+    for k, case in enumerate(SINGLE_PASS_CASES):
+        variants = ([None] if "dtype" in case else ["bfloat16", "float16"])
+        for j, values in enumerate(variants):
+            c = dict(case) if values is None else dict(case, values=values)
+            V = vocabs[(k + j) % len(vocabs)]
+            got, entry = _grpo_case(GRPOTrainer, c, 6000 + ci, (6, 2, 6, V), [6, 3, 5, 1, 6, 4])
+            got["logits"] = got["logits"].astype(np.float32)
+            for key, v in got.items():
+                arrays[f"c{ci}_{key}"] = v
+            entry["id"] = ci
+            index.append(entry)
+            ci += 1
+    np.savez_compressed(os.path.join(out_dir, "grpo_single_pass.npz"), **arrays)
+    with open(os.path.join(out_dir, "grpo_single_pass.json"), "w") as f:
         json.dump(index, f, indent=1)
 
 
@@ -625,6 +710,7 @@ def main():
     make_utils(ref_utils, args.out)
     make_head(ref_utils._ChunkedLogProbFunction, args.out)
     make_grpo(GRPOTrainer, args.out)
+    make_grpo_single_pass(GRPOTrainer, args.out)
     make_dpo(DPOTrainer, args.out)
     make_rloo(RLOOTrainer, args.out)
     make_kto(KTOTrainer, args.out)

@@ -331,3 +331,237 @@ def test_kernel_reads_masked_rows_when_asked(amd):
     m = mask.bool()
     assert torch.equal(lp_a[m], lp_s[m]) and float(lp_s[~m].abs().max()) == 0.0
     assert torch.equal(g_a, g_s)
+
+
+# ------------------------------------------------------------------ vectors written by the reference
+def _round_to(t, dtype):
+    return t.to(dtype).float()
+
+
+def test_golden_vectors_go_through_the_single_pass_kernel(amd, monkeypatch):
+    """`tests/golden/grpo_single_pass.*`: the reference's `GRPOTrainer._compute_loss` + backward on a mocked trainer
+    (trl/trainer/grpo_trainer.py:2991-3260), for every configuration the one-pass kernel takes, on vocabularies
+    that are multiples of 8.  The fixture's fp32 logits hold bf16-exact (or fp16-exact) values, so the reference did
+    fp32 arithmetic on exactly the numbers the kernel reads from the 16-bit tensor: loss, metrics, log-probs and
+    entropies are held to fp32 bars, and the gradient to the reference's gradient ROUNDED to the 16-bit dtype (what
+    an exact kernel would store).  Two cases ran the reference in true bf16 / fp16 arithmetic (its log-probs are
+    rounded to 16 bits) and are comparable at 2e-2 only.  The call into the one-pass kernel is counted: a case
+    that falls back to the two-pass path fails."""
+    from conftest import fake_grpo_trainer, load_golden
+    from types import SimpleNamespace
+
+    import numpy as np
+
+    from trl_amd import ops
+
+    calls = []
+    real = ops.grpo_fused_fwd_bwd
+
+    def spy(*a, **k):
+        out = real(*a, **k)
+        calls.append(out[3])
+        return out
+
+    monkeypatch.setattr(ops, "grpo_fused_fwd_bwd", spy)
+    cases, g = load_golden("grpo_single_pass")
+    assert len(cases) >= 60
+    seen = set()
+    for case in cases:
+        c = f"c{case['id']}_"
+        B, P, T, V = case["shape"]
+        true_low = "dtype" in case
+        dtype = getattr(torch, case["dtype"] if true_low else case["values"])
+        logits32 = torch.from_numpy(g[c + "logits"])
+        assert torch.equal(logits32.to(dtype).float(), logits32)  # the 16-bit tensor holds the reference's inputs exactly
+        tr = fake_grpo_trainer(amd, case, T, skip_masked=True, single_pass=True)
+        leaf = logits32.to(dtype).to(DEV).requires_grad_(True)
+        dev = lambda key: torch.from_numpy(np.asarray(g[c + key])).to(DEV)  # noqa: E731
+        inputs = dict(prompt_ids=dev("prompt_ids"), prompt_mask=torch.ones(B, P, dtype=torch.long, device=DEV),
+                      completion_ids=dev("completion_ids"), completion_mask=dev("completion_mask"),
+                      advantages=dev("advantages"), num_items_in_batch=dev("num_items_in_batch"))
+        for key in ("old_per_token_logps", "ref_per_token_logps", "importance_sampling_ratio"):
+            if c + key in g:
+                inputs[key] = dev(key)
+        n_before = len(calls)
+        loss = tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None), inputs)
+        loss.backward()
+        assert len(calls) == n_before + 1, f"{case['name']}: the one-pass kernel was not taken"
+        assert leaf.grad.data_ptr() == calls[-1].data_ptr() or torch.equal(leaf.grad, calls[-1])
+        name = (case["name"], str(dtype))
+        rtol = 2e-2 if true_low else 2e-5
+        want_loss = float(g[c + "out_loss"])
+        assert abs(float(loss) - want_loss) <= rtol * max(1.0, abs(want_loss)), (name, float(loss), want_loss)
+        got_metrics = {k: v[-1] for k, v in tr._metrics["train"].items()}
+        assert set(case["metrics"]) <= set(got_metrics), (name, set(case["metrics"]) - set(got_metrics))
+        for key, want in case["metrics"].items():
+            got = got_metrics[key]
+            ok = (math.isnan(got) and math.isnan(want)) or abs(got - want) <= rtol * max(1.0, abs(want))
+            assert ok, (name, key, got, want)
+        want_g = torch.from_numpy(g[c + "out_dlogits"]).float()
+        got_g = leaf.grad.float().cpu()
+        mask = torch.from_numpy(g[c + "completion_mask"]).bool()
+        full = torch.zeros(B, P + T, dtype=torch.bool)
+        full[:, P - 1 : P - 1 + T] = mask
+        assert float(got_g[~full].abs().max()) == 0.0 and float(want_g[~full].abs().max()) == 0.0, name
+        if true_low:
+            assert _rel_l2(got_g, want_g) < 2e-2, (name, _rel_l2(got_g, want_g))
+        else:
+            # against what an exact kernel would store: the fp32 gradient rounded once to the logits dtype
+            exact = _round_to(want_g, dtype)
+            rel = _rel_l2(got_g, exact)
+            assert rel < 5e-4, (name, rel)
+            assert float((got_g == exact).float().mean()) > 0.98, name
+            assert _rel_l2(got_g, want_g) < (3e-3 if dtype == torch.bfloat16 else 6e-4), name
+        if "state_after" in case:
+            want = case["state_after"]
+            assert abs(tr.entropy_coef - want["entropy_coef"]) < 1e-9, name
+            assert abs(tr._last_world_entropy - want["last_world_entropy"]) < 1e-4, name
+            if want["window"] is None:
+                assert tr._entropy_window_stats is None
+            else:
+                torch.testing.assert_close(tr._entropy_window_stats.cpu(), torch.tensor(want["window"]), rtol=1e-5, atol=1e-4)
+        seen.add((case["loss_type"], str(dtype)))
+    for lt in ("dapo", "grpo", "dr_grpo", "bnpo", "cispo", "sapo"):
+        assert (lt, "torch.bfloat16") in seen and (lt, "torch.float16") in seen
+    amd.check_device_errors()
+
+
+def test_golden_vectors_functional_form_logps_and_entropies(amd):
+    """The same fixture through `grpo_loss_from_logits` directly: per-token log-probs and entropies of the active
+    rows against the reference's (fp32 arithmetic on the same 16-bit values), 1e-5 absolute."""
+    from conftest import load_golden
+
+    cases, g = load_golden("grpo_single_pass")
+    for case in cases:
+        if "dtype" in case or case.get("is_ratio") or case.get("adaptive"):
+            continue
+        c = f"c{case['id']}_"
+        B, P, T, V = case["shape"]
+        dtype = getattr(torch, case["values"])
+        leaf = torch.from_numpy(g[c + "logits"]).to(dtype).to(DEV).requires_grad_(True)
+        t = lambda key: torch.from_numpy(g[c + key]).to(DEV) if c + key in g else None  # noqa: E731
+        loss, _, lp, ent = amd.grpo_loss_from_logits(
+            leaf, t("completion_ids"), t("advantages"), t("completion_mask"), temperature=case.get("temperature", 1.0),
+            old_per_token_logps=t("old_per_token_logps"), ref_per_token_logps=t("ref_per_token_logps"),
+            loss_type=case["loss_type"], epsilon_low=case["eps_low"], epsilon_high=case["eps_high"], beta=case["beta"],
+            delta=case.get("delta"), max_completion_length=T, num_items_in_batch=t("num_items_in_batch"),
+            grad_accum_steps=float(case.get("grad_accum", 1)), use_bias_correction_kl=case.get("bias_kl", False),
+            entropy_coef=case.get("entropy_coef", 0.0), skip_masked_rows=False)
+        torch.testing.assert_close(lp.cpu(), torch.from_numpy(g[c + "out_logps"]), atol=1e-5, rtol=0)
+        torch.testing.assert_close(ent.cpu(), torch.from_numpy(g[c + "out_entropies"]), atol=1e-5, rtol=0)
+        want_loss = float(g[c + "out_loss"])
+        assert abs(float(loss) - want_loss) <= 2e-5 * max(1.0, abs(want_loss)), case["name"]
+
+
+# ------------------------------------------------------------------ the benchmark shapes through the single pass
+def _big_logits(B, L, V, seed):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    logits = torch.empty(B, L, V, dtype=torch.bfloat16, device=DEV)
+    for b in range(B):
+        for t0 in range(0, L, 1024):  # blocks keep the fp32 temporary small
+            t1 = min(t0 + 1024, L)
+            logits[b, t0:t1] = (2.0 * torch.randn(t1 - t0, V, generator=g, device=DEV)).bfloat16()
+    return logits, g
+
+
+def _full_size_check(amd, monkeypatch, logits, g, K, temperature, lengths_lo, adv, pick_b, pick_t, **kw):
+    """`grpo_loss_from_logits` on benchmark-sized logits: the call reaches the one-pass kernel; rows without gradient
+    are exactly zero; every gradient row sums to zero; a row subsample of log-prob, entropy and dlogits equals the
+    CPU oracle's autograd on the same stored values; the loss equals the oracle's loss on the forward kernel's
+    log-probs of all rows."""
+    import oracle
+    from trl_amd import ops
+
+    B, L, V = logits.shape
+    calls = []
+    real = ops.grpo_fused_fwd_bwd
+    monkeypatch.setattr(ops, "grpo_fused_fwd_bwd", lambda *a, **k: calls.append(1) or real(*a, **k))
+    ids = torch.randint(0, V, (B, K), generator=g, device=DEV)
+    lengths = torch.randint(lengths_lo, K + 1, (B,), generator=g, device=DEV)
+    mask = (torch.arange(K, device=DEV)[None] < lengths[:, None]).long()
+    with torch.no_grad():
+        base, base_ent = amd.per_token_logps_and_entropies(logits, torch.cat([ids[:, :1], ids], 1), K, temperature)
+    old = base + 0.05 * torch.randn(base.shape, generator=g, device=DEV)
+    ref = base + 0.1 * torch.randn(base.shape, generator=g, device=DEV)
+    beta = kw["beta"]
+    kw = dict(kw, old_per_token_logps=old, ref_per_token_logps=ref if beta else None, max_completion_length=K,
+              num_items_in_batch=mask.sum().float())
+    logits.requires_grad_(True)
+    logits.grad = None
+    loss, metrics, lp, ent = amd.grpo_loss_from_logits(logits, ids, adv, mask, temperature=temperature,
+                                                       skip_masked_rows=False, **kw)
+    loss.backward()
+    assert len(calls) == 1
+    grad = logits.grad
+    assert grad.shape == logits.shape and grad.dtype == logits.dtype
+    start = L - 1 - K
+    # (1) rows outside the window or the mask: exactly zero; active rows: not all zero
+    nz = torch.stack([(grad[b] != 0).any(-1) for b in range(B)])
+    want_nz = torch.zeros(B, L, dtype=torch.bool, device=DEV)
+    if beta:  # the KL term moves every active token, whatever its advantage
+        want_nz[:, start:start + K] = mask.bool()
+        assert torch.equal(nz, want_nz)
+    else:  # a token whose ratio left the clip range on the clipped side has no gradient either (a handful of rows)
+        want_nz[:, start:start + K] = mask.bool() & (adv.reshape(B, -1) != 0)
+        assert not bool((nz & ~want_nz).any())
+        assert int((want_nz & ~nz).sum()) <= 2e-3 * int(want_nz.sum())
+        assert int(want_nz.sum()) > 0.2 * B * K
+    # (2) sum_v dlogits = 0 up to the bf16 rounding of the row's entries
+    for b in range(B):
+        gb = grad[b, start:start + K].float()
+        assert bool((gb.sum(-1).abs() <= 3e-3 * gb.abs().sum(-1) + 1e-12).all()), b
+    # (3) every row's log-prob and entropy: the forward kernel's (all rows were asked for)
+    torch.testing.assert_close(lp, base, atol=1e-5, rtol=0)
+    torch.testing.assert_close(ent, base_ent, atol=1e-4, rtol=0)  # (entropies of ~7 nats from differently ordered sums)
+    # (4) the loss: the oracle's arithmetic on the forward kernel's log-probs of all rows
+    okw = {k: (v.cpu() if torch.is_tensor(v) else v) for k, v in kw.items()}
+    o_lp = base.cpu().clone().requires_grad_(True)
+    o_loss, o_metrics = oracle.grpo_loss(o_lp, adv.cpu(), mask.cpu(), entropies=base_ent.cpu(), **okw)
+    assert abs(float(loss) - float(o_loss)) <= 2e-6 + 1e-4 * abs(float(o_loss)), (float(loss), float(o_loss))
+    md = amd.trainer.metrics_to_dict(metrics, beta, loss_type=kw["loss_type"])
+    for name, want in o_metrics.items():
+        if name in md:
+            assert abs(md[name] - want) <= 1e-4 * max(1.0, abs(want)), (name, md[name], want)
+    # (5) a row subsample through the oracle's autograd, from the stored logits to dlogits
+    pb, pt = torch.tensor(pick_b), torch.tensor(pick_t)
+    sub = logits.detach()[pb.to(DEV)][:, (start + pt).to(DEV)].cpu().float().requires_grad_(True)
+    sub_ids = ids[pb.to(DEV)][:, pt.to(DEV)].cpu()
+    sub_lp = oracle.selective_log_softmax_f32(sub, sub_ids, temperature)
+    sub_ent = oracle.entropy_from_logits_f32(sub, temperature)
+    torch.testing.assert_close(lp[pb.to(DEV)][:, pt.to(DEV)].cpu(), sub_lp.detach(), atol=2e-3, rtol=0)
+    torch.testing.assert_close(ent[pb.to(DEV)][:, pt.to(DEV)].cpu(), sub_ent.detach(), atol=2e-3, rtol=0)
+    spliced = base.cpu().index_put((pb[:, None], pt[None, :]), sub_lp)
+    o_loss2, _ = oracle.grpo_loss(spliced, adv.cpu(), mask.cpu(), entropies=base_ent.cpu(), **okw)
+    o_loss2.backward()
+    got = grad[pb.to(DEV)][:, (start + pt).to(DEV)].float().cpu()
+    active = mask.cpu()[pb][:, pt].bool()
+    assert int(active.sum()) >= 4
+    assert _rel_l2(got[active], sub.grad[active]) < 3e-3, _rel_l2(got[active], sub.grad[active])
+    assert _rel_l2(got[active], sub.grad[active].bfloat16().float()) < 1e-3
+    assert float(got[~active].abs().max() if (~active).any() else 0.0) == 0.0
+    logits.requires_grad_(False)
+    amd.check_device_errors()
+
+
+def test_full_size_config3_single_pass(amd, monkeypatch):
+    """Benchmark configuration 3 (64 sequences x 1024 completion tokens, V = 151936, bf16, T = 0.9, G = 8,
+    eps = 0.2, beta = 0.04) through `grpo_loss_from_logits` for loss_type grpo, dapo and dr_grpo."""
+    B, K, V = 64, 1024, 151936
+    logits, g = _big_logits(B, K + 1, V, seed=33)
+    rewards = torch.randn(B, generator=g, device=DEV)
+    adv = amd.group_advantages(rewards, 8)
+    for lt in ("grpo", "dapo", "dr_grpo"):
+        _full_size_check(amd, monkeypatch, logits, g, K, 0.9, 64, adv, [0, 17, 63], [0, 1, 40, 500, 1023],
+                         loss_type=lt, epsilon_low=0.2, epsilon_high=0.2, beta=0.04)
+        monkeypatch.undo()
+
+
+def test_full_size_config4_single_pass(amd, monkeypatch):
+    """Benchmark configuration 4 (32 sequences x 4096 completion tokens, V = 151936, 39.8 GB of bf16 logits, G = 16,
+    Bernoulli(0.3) rewards, eps_low = 0.2, eps_high = 0.28, beta = 0) through `grpo_loss_from_logits`."""
+    B, K, V = 32, 4096, 151936
+    logits, g = _big_logits(B, K + 1, V, seed=44)
+    rewards = (torch.rand(B, generator=g, device=DEV) < 0.3).float()
+    adv = amd.group_advantages(rewards, 16)
+    _full_size_check(amd, monkeypatch, logits, g, K, 1.0, 512, adv, [0, 13, 31], [0, 300, 511, 2047, 4095],
+                     loss_type="dapo", epsilon_low=0.2, epsilon_high=0.28, beta=0.0)

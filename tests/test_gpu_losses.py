@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import oracle
-from conftest import load_golden
+from conftest import fake_grpo_trainer as _fake_trainer, load_golden
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -33,67 +33,15 @@ def amd():
     return trl_amd
 
 
-class _Identity:
-    num_processes = 1
-    sync_gradients = True
-
-    def gather(self, x):
-        return x
-
-    gather_for_metrics = reduce = gather
-
-    def reduce(self, x, reduction="sum"):
-        return x
-
-    def pad_across_processes(self, x, dim=0, pad_index=0):
-        return x
-
-
-def _fake_trainer(amd, case, T, skip_masked=False, single_pass=False):
-    class Trainer(amd.GRPOLossMixin):
-        pass
-
-    tr = Trainer()
-    tr.accelerator = _Identity()
-    tr.temperature = case.get("temperature", 1.0)
-    tr.model_kwarg_keys = set()
-    ad = case.get("adaptive")
-    tr._entropy_bonus_enabled = case.get("entropy_coef", 0.0) != 0.0 or ad is not None
-    tr.entropy_coef = case.get("entropy_coef", 0.0)
-    tr.use_adaptive_entropy = ad is not None
-    if ad is not None:
-        tr._last_world_entropy = ad["last"]
-        tr._entropy_window_stats = torch.tensor(ad["window"]) if "window" in ad else None
-        tr.accelerator.sync_gradients = ad["sync"]
-    tr.aux_loss_enabled = False
-    tr.top_entropy_quantile = case.get("top_entropy_quantile", 1.0)
-    tr.off_policy_mask_threshold = case.get("off_policy")
-    tr.importance_sampling_level = case.get("is_level", "token")
-    tr.beta = case["beta"]
-    tr.loss_type = case["loss_type"]
-    tr.epsilon_low, tr.epsilon_high = case["eps_low"], case["eps_high"]
-    tr.use_vllm = bool(case.get("is_ratio"))
-    tr.vllm_importance_sampling_correction = bool(case.get("is_ratio"))
-    tr.max_completion_length = T
-    tr.current_gradient_accumulation_steps = case.get("grad_accum", 1)
-    tr.args = SimpleNamespace(delta=case.get("delta"), use_bias_correction_kl=case.get("bias_kl", False))
-    if ad is not None:
-        tr.args.entropy_target, tr.args.entropy_coef_delta = ad["target"], ad["delta"]
-        tr.args.entropy_coef_max, tr.args.entropy_coef_min = ad["max"], ad["min"]
-    tr._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
-    tr.model = SimpleNamespace(training=True)
-    tr.trl_amd_skip_masked_rows = skip_masked
-    tr.trl_amd_single_pass = single_pass
-    return tr
-
-
 @pytest.mark.parametrize("skip_masked,single_pass", [(False, False), (True, False), (True, True)])
 def test_golden_grpo_compute_loss_through_trainer_methods(amd, skip_masked, single_pass):
     """The reference's `GRPOTrainer._compute_loss` ran these inputs on a mocked trainer; the same
     mock drives our mix-in methods on the device.  With `skip_masked` the forward kernel skips the
-    rows the completion mask zeroes; loss, metrics and gradients must not change.  With `single_pass`
-    the cases the one-pass kernel takes (16-bit logits, token-level loss) go through it, the others
-    fall back to the two kernels on the logits of the same model call."""
+    rows the completion mask zeroes; loss, metrics and gradients must not change.  With `single_pass` the
+    trainer asks for the one-pass kernel, which none of these cases can take (V = 41 is no multiple of 8, most
+    logits are fp32): this leg checks the fall-back to the two kernels on the logits of the same model call.
+    The reference-written vectors that DO go through the one-pass kernel are `grpo_single_pass.*`
+    (tests/test_gpu_grpo_single_pass.py)."""
     cases, g = load_golden("grpo_compute_loss")
     ran = 0
     for case in cases:
