@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import oracle
-from conftest import fake_grpo_trainer as _fake_trainer, load_golden
+from conftest import IdentityAccelerator as _Identity, fake_grpo_trainer as _fake_trainer, load_golden
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"

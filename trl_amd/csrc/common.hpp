@@ -79,6 +79,7 @@ struct Elem<TRLK_F32> {
         u32x4 q = {__float_as_uint(x[0]), __float_as_uint(x[1]), __float_as_uint(x[2]), __float_as_uint(x[3])};
         return q;
     }
+    static __device__ __forceinline__ float to_float(type v) { return v; }
     static __device__ __forceinline__ float load1(const type* p) { return *p; }
     static __device__ __forceinline__ void store1(type* p, float v) { *p = v; }
 };
@@ -105,7 +106,8 @@ struct Elem<TRLK_BF16> {
         u32x4 q = {pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
         return q;
     }
-    static __device__ __forceinline__ float load1(const type* p) { return __uint_as_float(uint32_t(*p) << 16); }
+    static __device__ __forceinline__ float to_float(type v) { return __uint_as_float(uint32_t(v) << 16); }
+    static __device__ __forceinline__ float load1(const type* p) { return to_float(*p); }
     static __device__ __forceinline__ void store1(type* p, float v) { *p = uint16_t(pack2(v, 0.f) & 0xffffu); }
 };
 
@@ -132,9 +134,8 @@ struct Elem<TRLK_F16> {
         u32x4 q = {pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7])};
         return q;
     }
-    static __device__ __forceinline__ float load1(const type* p) {
-        return float(__builtin_bit_cast(_Float16, *p));
-    }
+    static __device__ __forceinline__ float to_float(type v) { return float(__builtin_bit_cast(_Float16, v)); }
+    static __device__ __forceinline__ float load1(const type* p) { return to_float(*p); }
     static __device__ __forceinline__ void store1(type* p, float v) {
         *p = __builtin_bit_cast(uint16_t, _Float16(v));
     }

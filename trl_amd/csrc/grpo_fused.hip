@@ -18,6 +18,10 @@ namespace {
 constexpr int kFThreads = 1024;
 constexpr int kFWaves = kFThreads / kWave;
 constexpr int kMaxVec = 20;  // 16-byte vectors of a row per lane: rows of up to 20 * 1024 * 8 = 163840 logits
+constexpr int kVecStep = 4;  // the kernel is built for 4, 8, ... kMaxVec vectors per lane; the host picks the smallest that holds the row
+
+typedef __attribute__((address_space(1))) const u32x4 GlobalVecIn;
+typedef __attribute__((address_space(1))) u32x4 GlobalVecOut;
 
 struct FusedArgs {
     const void* logits;
@@ -38,12 +42,23 @@ struct FusedArgs {
     int all_rows;  // also read the rows with mask == 0 for their log-prob and entropy (their gradient is zero either way)
 };
 
-template <int DT>
+// One workgroup of 1024 lanes per output row; NVEC = 16-byte vectors of the row a lane holds (the last kVecStep of
+// them may lie beyond the row's end for some lanes).  A workgroup fills its CU's register file, so nothing else
+// runs beside it: the arithmetic has to overlap the row's own memory traffic.  Hence
+//   * the per-row scalars are loaded first, from uniform addresses before any store: scalar loads, which return
+//     long before (and independently of) the row's vector loads; the target's logit is requested right behind the row;
+//   * the exponentials are summed while the row arrives: a lane takes its reference exponent r0 from its FIRST
+//     vector (an integer, so bringing the lanes' sums to a common exponent afterwards is exact) and consumes each
+//     vector as its load retires.  Later logits may exceed the first vector's by 128 / (log2(e) / T) before a
+//     term overflows; a row where that happens (or one that holds inf / NaN) is detected by its non-finite sums
+//     and takes the exact two-sweep reduction over the registers instead.
+template <int DT, int NVEC>
 __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     typedef Elem<DT> E;
     typedef typename E::type T;
     constexpr int EPV = E::EPV;
-    __shared__ float red[3][kFWaves];
+    constexpr int kTail = NVEC - kVecStep;
+    __shared__ float red[7][kFWaves];
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int64_t orow = blockIdx.x;
     const int64_t b = orow / a.out_rows_per_seq;
@@ -52,8 +67,20 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     const bool inside = t >= 0 && t < a.rows_per_seq;
     const int64_t row = b * a.rows_per_seq + (inside ? t : 0);
     const int nv = int(a.vocab / EPV);
+    float m = 0.f, A = 0.f, old_lp = 0.f, ref_lp = 0.f, w = 1.f, coef = 0.f, scale = 0.f, h = 0.f;
+    int64_t idx = -1;
+    if (inside) {
+        m = a.mask[row];
+        idx = a.index[row];
+        A = a.adv[b * a.adv_stride_b + t * a.adv_stride_t];
+        if (a.old_logp) old_lp = a.old_logp[row];
+        if (a.beta != 0.f) ref_lp = a.ref_logp[row];
+        if (a.token_weight) w = a.token_weight[row];
+        if (a.seq_coef) coef = a.seq_coef[b];
+        scale = a.row_scale[b];
+        if (a.ent_weight) h = a.ent_weight[row];
+    }
     u32x4* op = reinterpret_cast<u32x4*>(static_cast<T*>(a.dlogits) + b * a.out_seq_stride + to * a.out_row_stride);
-    const float m = inside ? a.mask[row] : 0.f;
     if (m == 0.f) {  // no gradient reaches this row: zero-fill
         const u32x4 z = {0u, 0u, 0u, 0u};
         for (int v = tid; v < nv; v += kFThreads) __builtin_nontemporal_store(z, op + v);
@@ -68,50 +95,102 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     }
     const T* base = static_cast<const T*>(a.logits) + b * a.seq_stride + t * a.row_stride;
     const u32x4* vp = reinterpret_cast<const u32x4*>(base);
-    u32x4 q[kMaxVec];
+    u32x4 q[NVEC];
 #pragma unroll
-    for (int j = 0; j < kMaxVec; ++j) {
-        const int v = j * kFThreads + tid;
-        if (v < nv) q[j] = vp[v];  // (plain loads measure 4 % faster here than non-temporal ones, as in the two-pass backward)
+    for (int j = 0; j < NVEC; ++j) {
+        // the address is (uniform base of vector j, in scalar registers) + the lane's index: one vector register
+        // serves all NVEC loads and stores instead of one offset register each.  (Pointers that pass through the
+        // empty asm must say that they point to global memory, or the accesses become flat ones, whose waits are
+        // all-or-nothing.)
+        GlobalVecIn* vj = (GlobalVecIn*)vp + j * kFThreads;
+        asm volatile("" : "+s"(vj));
+        int tj = tid;
+        if (j >= kTail) tj = min(tid, nv - 1 - j * kFThreads);  // (a lane beyond the row's end re-reads the last vector and ignores it)
+        q[j] = vj[tj];  // (plain loads: non-temporal ones measure the same to 1 % either way)
     }
-    // the per-row scalars travel while the row does
-    const int64_t idx = a.index[row];
     const bool idx_ok = idx >= 0 && idx < a.vocab;
-    const float x_t = idx_ok ? E::load1(base + idx) : NAN;
-    const float A = a.adv[b * a.adv_stride_b + t * a.adv_stride_t];
-    const float old_lp = a.old_logp ? a.old_logp[row] : 0.f;
-    const float ref_lp = a.beta != 0.f ? a.ref_logp[row] : 0.f;
-    const float w = a.token_weight ? a.token_weight[row] : 1.f;
-    const float coef = a.seq_coef ? a.seq_coef[b] : 0.f;
-    const float scale = a.row_scale[b];
-    const float h = a.ent_weight ? a.ent_weight[row] : 0.f;
+    T x_t_raw = base[idx_ok ? idx : 0];  // requested right behind the row; converted only when the sums are done
     const float inv_t = 1.f / a.temperature, c = kLog2e * inv_t;
 
-    // lane maximum, then the lane's sums relative to it
-    float lm = -INFINITY;
+    // sums of 2^(x c - r0) and of the same times x, vector by vector as the loads retire
+    float r0 = 0.f, s = 0.f, u = 0.f;
 #pragma unroll
-    for (int j = 0; j < kMaxVec; ++j)
-        if (j * kFThreads + tid < nv) {
+    for (int j = 0; j < NVEC; ++j) {
+        asm volatile("" : "+v"(q[j]));  // (pins the order: vector j is waited for and consumed before vector j + 1)
+        if (j < kTail || j * kFThreads + tid < nv) {
             float x[EPV];
             E::unpack(q[j], x);
+            if (j == 0) {
+                float mx = x[0];
+#pragma unroll
+                for (int i = 1; i < EPV; ++i) mx = fmaxf(mx, x[i]);
+                r0 = ceilf(mx * c);
+            }
+#pragma unroll
+            for (int i = 0; i < EPV; ++i) {
+                const float e = fast_exp2(fmaf(x[i], c, -r0));
+                s += e;
+                u = fmaf(e, x[i], u);
+            }
+        }
+    }
+    // bring the lanes' sums to a common exponent K >= r0 + log2(s) of every lane
+    int es = 0;
+    (void)frexpf(s, &es);
+    const bool has_data = tid < nv;
+    const float key = has_data ? r0 + float(es) : -INFINITY;
+    const bool bad = !(s < INFINITY) || !(fabsf(u) < INFINITY);  // overflow of a term, or inf / NaN in the row
+    const float wk = wave_max(key);
+    const bool wbad = __any(bad);
+    if (lane == 0) {
+        red[0][wave] = wk;
+        red[3][wave] = wbad ? 1.f : 0.f;
+    }
+    __syncthreads();
+    float K = -INFINITY, any_bad = 0.f;
+#pragma unroll
+    for (int k = 0; k < kFWaves; ++k) {
+        K = fmaxf(K, red[0][k]);
+        any_bad += red[3][k];
+    }
+    float lse2;  // log2 of sum exp(z), z = x / T
+    float S = 0.f, U = 0.f;
+    if (any_bad == 0.f) {
+        const int sh = int(fminf(fmaxf(r0 - K, -300.f), 300.f));
+        s = wave_sum(ldexpf(s, sh));
+        u = wave_sum(ldexpf(u, sh));
+        if (lane == 0) {
+            red[1][wave] = s;
+            red[2][wave] = u;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < kFWaves; ++k) {
+            S += red[1][k];
+            U += red[2][k];
+        }
+        lse2 = K + __builtin_amdgcn_logf(S);
+    } else {
+        // the exact reduction: the row's maximum first, then the sums relative to it.  Rare, so it re-reads the row
+        // from memory instead of competing with the fast path for the registers that hold it.
+        float lm = -INFINITY;
+        for (int v = tid; v < nv; v += kFThreads) {
+            float x[EPV];
+            E::unpack(vp[v], x);
 #pragma unroll
             for (int i = 0; i < EPV; ++i) lm = fmaxf(lm, x[i]);
         }
-    // (the compiler must not keep the unpacked values of one pass alive for the next: 152 floats per lane)
+        float M = wave_max(lm);
+        if (lane == 0) red[4][wave] = M;
+        __syncthreads();
 #pragma unroll
-    for (int j = 0; j < kMaxVec; ++j) asm volatile("" : "+v"(q[j]));
-    float M = wave_max(lm);
-    if (lane == 0) red[0][wave] = M;
-    __syncthreads();
-#pragma unroll
-    for (int k = 0; k < kFWaves; ++k) M = fmaxf(M, red[0][k]);
-    const float mc = M * c;
-    float s = 0.f, u = 0.f;
-#pragma unroll
-    for (int j = 0; j < kMaxVec; ++j)
-        if (j * kFThreads + tid < nv) {
+        for (int k = 0; k < kFWaves; ++k) M = fmaxf(M, red[4][k]);
+        const float mc = M * c;
+        s = 0.f;
+        u = 0.f;
+        for (int v = tid; v < nv; v += kFThreads) {
             float x[EPV];
-            E::unpack(q[j], x);
+            E::unpack(vp[v], x);
 #pragma unroll
             for (int i = 0; i < EPV; ++i) {
                 const float e = fast_exp2(fmaf(x[i], c, -mc));
@@ -119,22 +198,25 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
                 u = fmaf(e, x[i], u);
             }
         }
+        s = wave_sum(s);
+        u = wave_sum(u);
+        if (lane == 0) {
+            red[5][wave] = s;
+            red[6][wave] = u;
+        }
+        __syncthreads();
 #pragma unroll
-    for (int j = 0; j < kMaxVec; ++j) asm volatile("" : "+v"(q[j]));
-    s = wave_sum(s);
-    u = wave_sum(u);
-    if (lane == 0) {
-        red[1][wave] = s;
-        red[2][wave] = u;
+        for (int k = 0; k < kFWaves; ++k) {
+            S += red[5][k];
+            U += red[6][k];
+        }
+        lse2 = mc + __builtin_amdgcn_logf(S);
     }
-    __syncthreads();
-    float S = 0.f, U = 0.f;
+    // (the compiler must not keep the unpacked values of one sweep alive for the next: 8 floats per vector and lane)
 #pragma unroll
-    for (int k = 0; k < kFWaves; ++k) {
-        S += red[1][k];
-        U += red[2][k];
-    }
-    const float lse2 = mc + __builtin_amdgcn_logf(S);  // log2 of sum exp(z), z = x / T
+    for (int j = 0; j < NVEC; ++j) asm volatile("" : "+v"(q[j]));
+    asm volatile("" : "+v"(x_t_raw));
+    const float x_t = idx_ok ? E::to_float(x_t_raw) : NAN;
     const float lse = lse2 * kLn2;
     const float ent = lse - (U / S) * inv_t;
     const float lp = x_t * inv_t - lse;
@@ -157,9 +239,9 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     const float a0 = (-g - h * ent) * inv_t;
     const float b0 = -h * kLn2 * inv_t;
 #pragma unroll
-    for (int j = 0; j < kMaxVec; ++j) {
+    for (int j = 0; j < NVEC; ++j) {
         const int v = j * kFThreads + tid;
-        if (v < nv) {
+        if (j < kTail || v < nv) {
             float x[EPV], d[EPV];
             E::unpack(q[j], x);
 #pragma unroll
@@ -167,7 +249,9 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
                 const float tt = fmaf(x[i], c, -lse2);
                 d[i] = fast_exp2(tt) * fmaf(b0, tt, a0);
             }
-            op[v] = E::pack(d);  // (plain: measured 3 % faster than non-temporal here; the zero-fill above is faster non-temporal)
+            GlobalVecOut* oj = (GlobalVecOut*)op + j * kFThreads;
+            asm volatile("" : "+s"(oj));
+            __builtin_nontemporal_store(E::pack(d), oj + tid);  // (streaming stores: 2-3 % faster than plain ones here)
         }
     }
     // one-hot term: the lane that stored the target's vector rewrites that element (same lane, same
@@ -176,6 +260,17 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
         T* out = reinterpret_cast<T*>(op);
         const float tt = fmaf(x_t, c, -lse2);
         E::store1(out + idx, fast_exp2(tt) * fmaf(b0, tt, a0) + g * inv_t);
+    }
+}
+
+template <int DT>
+void launch_fused(const FusedArgs& a, int nvec, unsigned rows, hipStream_t s) {
+    switch ((nvec + kVecStep - 1) / kVecStep) {
+        case 1: hipLaunchKernelGGL((grpo_fused_kernel<DT, 4>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        case 2: hipLaunchKernelGGL((grpo_fused_kernel<DT, 8>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        case 3: hipLaunchKernelGGL((grpo_fused_kernel<DT, 12>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        case 4: hipLaunchKernelGGL((grpo_fused_kernel<DT, 16>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        default: hipLaunchKernelGGL((grpo_fused_kernel<DT, 20>), dim3(rows), dim3(kFThreads), 0, s, a); break;
     }
 }
 
@@ -299,9 +394,10 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
     a.error_flag = d_error_flag;
     a.all_rows = compute_masked_rows != 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const int nvec = int((vocab / 8 + kFThreads - 1) / kFThreads);  // 16-byte vectors of the row per lane
     if (dtype == TRLK_BF16)
-        hipLaunchKernelGGL(grpo_fused_kernel<TRLK_BF16>, dim3((unsigned)orows), dim3(kFThreads), 0, s, a);
+        launch_fused<TRLK_BF16>(a, nvec, unsigned(orows), s);
     else
-        hipLaunchKernelGGL(grpo_fused_kernel<TRLK_F16>, dim3((unsigned)orows), dim3(kFThreads), 0, s, a);
+        launch_fused<TRLK_F16>(a, nvec, unsigned(orows), s);
     return launch_status("grpo_fused");
 }
