@@ -374,6 +374,7 @@ def test_golden_vectors_go_through_the_single_pass_kernel(amd, monkeypatch):
         logits32 = torch.from_numpy(g[c + "logits"])
         assert torch.equal(logits32.to(dtype).float(), logits32)  # the 16-bit tensor holds the reference's inputs exactly
         tr = fake_grpo_trainer(amd, case, T, skip_masked=True, single_pass=True)
+        tr.trl_amd_single_pass_fp16 = True  # (fp16 logits take the one pass only with a gradient scaler or on request)
         leaf = logits32.to(dtype).to(DEV).requires_grad_(True)
         dev = lambda key: torch.from_numpy(np.asarray(g[c + key])).to(DEV)  # noqa: E731
         inputs = dict(prompt_ids=dev("prompt_ids"), prompt_mask=torch.ones(B, P, dtype=torch.long, device=DEV),
@@ -565,3 +566,94 @@ def test_full_size_config4_single_pass(amd, monkeypatch):
     adv = amd.group_advantages(rewards, 16)
     _full_size_check(amd, monkeypatch, logits, g, K, 1.0, 512, adv, [0, 13, 31], [0, 300, 511, 2047, 4095],
                      loss_type="dapo", epsilon_low=0.2, epsilon_high=0.28, beta=0.0)
+
+
+# ------------------------------------------------------------------ upstream gradients other than 1
+def test_known_upstream_scale_is_folded_into_the_forward(amd, monkeypatch):
+    """fp16 logits, a 32768-entry vocabulary and a loss scale of 65536 (what a `GradScaler` starts with): with
+    `upstream_scale` the forward writes the scaled gradient -- scaled in fp32 before the one rounding to fp16 -- and
+    `backward` leaves the buffer untouched; the result matches the two-pass path, which scales in fp32 as the
+    reference's autograd does (trl/trainer/grpo_trainer.py:3124-3142 for who divides what).  Without it the
+    gradient is rounded to fp16 first and most of a softmax row (p_v * 1e-4 * 1e-5) is flushed to zero."""
+    from trl_amd import ops
+
+    B, K, V, T = 2, 8, 32768, 1.0
+    logits, ids, mask, adv, g = _inputs(B, K, V, dtype=torch.float16, seed=41)
+    mask[:] = 1
+    scale = torch.tensor(65536.0, device=DEV)
+    kw = dict(loss_type="dapo", beta=0.0, num_items_in_batch=torch.tensor(4096.0, device=DEV))
+    leaf2, loss2, _, _, _ = _two_pass(amd, logits, ids, mask, adv, T, **kw)
+    (loss2 * scale).backward()
+    written = []
+    real = ops.grpo_fused_fwd_bwd
+    monkeypatch.setattr(ops, "grpo_fused_fwd_bwd", lambda *a, **k: written.append(real(*a, **k)) or written[-1])
+    leaf1 = logits.detach().clone().requires_grad_(True)
+    loss1 = amd.grpo_loss_from_logits(leaf1, ids, adv, mask, temperature=T, upstream_scale=scale, **kw)[0]
+    torch.testing.assert_close(loss1, loss2, rtol=1e-5, atol=1e-7)  # the returned loss is not scaled
+    before = written[-1][3].clone()
+    (loss1 * scale).backward()
+    assert torch.equal(leaf1.grad, before)  # bit for bit what the forward wrote: nothing was rescaled
+    assert _rel_l2(leaf1.grad, leaf2.grad) < 2e-3
+    nz2 = float((leaf2.grad != 0).float().mean())
+    assert abs(float((leaf1.grad != 0).float().mean()) - nz2) < 1e-3
+    # a float works as well as a device scalar; an unexpected upstream gradient is still honoured
+    leaf3 = logits.detach().clone().requires_grad_(True)
+    (amd.grpo_loss_from_logits(leaf3, ids, adv, mask, temperature=T, upstream_scale=65536.0, **kw)[0] * (2 * scale)).backward()
+    assert _rel_l2(leaf3.grad.float(), 2 * leaf2.grad.float()) < 2e-3
+    # scaling after the rounding loses the small entries: this is what the scale argument is for
+    leaf0 = logits.detach().clone().requires_grad_(True)
+    (amd.grpo_loss_from_logits(leaf0, ids, adv, mask, temperature=T, **kw)[0] * scale).backward()
+    assert float((leaf0.grad != 0).float().mean()) < 0.9 * nz2 or _rel_l2(leaf0.grad, leaf2.grad) > 2e-3
+
+
+def test_backward_runs_once(amd):
+    logits, ids, mask, adv, _ = _inputs(2, 4, 512, seed=43)
+    leaf = logits.detach().clone().requires_grad_(True)
+    loss = amd.grpo_loss_from_logits(leaf, ids, adv, mask, loss_type="bnpo")[0]
+    loss.backward(retain_graph=True)
+    first = leaf.grad.clone()
+    with pytest.raises(RuntimeError, match="only once"):
+        loss.backward()
+    assert torch.equal(leaf.grad, first)
+
+
+@pytest.mark.parametrize("with_scaler", [True, False])
+def test_trainer_method_takes_fp16_only_with_a_known_scale(amd, monkeypatch, with_scaler):
+    """`GRPOLossMixin._compute_loss` on fp16 logits: with a gradient scaler on the accelerator the one-pass kernel runs
+    with the scaler's factor folded in; without one the two-pass path runs (its gradient is scaled in fp32)."""
+    from conftest import fake_grpo_trainer
+    from types import SimpleNamespace
+
+    from trl_amd import ops
+
+    B, P, K, V = 4, 2, 8, 4096
+    g = torch.Generator(device=DEV).manual_seed(47)
+    logits = (2.0 * torch.randn((B, P + K, V), generator=g, device=DEV)).half()
+    case = dict(loss_type="grpo", beta=0.0, eps_low=0.2, eps_high=0.2)
+    inputs = dict(prompt_ids=torch.randint(0, V, (B, P), generator=g, device=DEV),
+                  prompt_mask=torch.ones(B, P, dtype=torch.long, device=DEV),
+                  completion_ids=torch.randint(0, V, (B, K), generator=g, device=DEV),
+                  completion_mask=torch.ones(B, K, dtype=torch.long, device=DEV),
+                  advantages=torch.randn(B, generator=g, device=DEV))
+    calls = []
+    real = ops.grpo_fused_fwd_bwd
+    monkeypatch.setattr(ops, "grpo_fused_fwd_bwd", lambda *a, **k: calls.append(1) or real(*a, **k))
+
+    class Scaler:
+        def is_enabled(self):
+            return True
+
+        def scale(self, x):
+            return x * 1024.0
+
+    grads = {}
+    for single in (True, False):
+        tr = fake_grpo_trainer(amd, case, K, skip_masked=True, single_pass=single)
+        tr.accelerator.scaler = Scaler() if with_scaler else None
+        leaf = logits.detach().clone().requires_grad_(True)
+        n = len(calls)
+        loss = tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None), inputs)
+        assert len(calls) == n + (1 if single and with_scaler else 0)
+        (tr.accelerator.scaler.scale(loss) if with_scaler else loss).backward()
+        grads[single] = leaf.grad
+    assert _rel_l2(grads[True], grads[False]) < 2e-3

@@ -282,6 +282,16 @@ class _GRPOFromLogits(torch.autograd.Function):
                 ent_weight = mask_f * (-float(kw["entropy_coef"]) * row_scale[0])
             else:
                 ent_weight = mask_f * (-float(kw["entropy_coef"]) / mask_f.sum().clamp(min=1.0) / ga)
+        up = kw.get("upstream_scale")
+        if up is not None:
+            # the caller will multiply the loss by this factor before backward (a gradient scaler's scale, a loss
+            # divisor): the gradient is written already scaled -- before its single rounding to the logits dtype --
+            # and `backward` has nothing left to do
+            up = (up.to(device=logits.device, dtype=torch.float32).reshape(()) if torch.is_tensor(up)
+                  else torch.tensor(float(up), dtype=torch.float32, device=logits.device))
+            row_scale = row_scale * up
+            if ent_weight is not None:
+                ent_weight = ent_weight * up
         delta = kw["delta"]
         logp, ent, _, dlogits = ops.grpo_fused_fwd_bwd(
             logits, ids, float(temperature), keep_start, keep_len, mask_f, advantages, row_scale,
@@ -307,16 +317,26 @@ class _GRPOFromLogits(torch.autograd.Function):
             use_bias_correction_kl=kw["use_bias_correction_kl"], token_weight=kw["token_weight"],
             entropy_coef=kw["entropy_coef"],
             sapo_temperature_pos=kw["sapo_temperature_pos"], sapo_temperature_neg=kw["sapo_temperature_neg"])
-        ctx.save_for_backward(dlogits)
+        ctx.save_for_backward(dlogits, *(() if up is None else (up,)))
         ctx.mark_non_differentiable(metrics, logp, ent)
+        ctx.consumed = False
         return loss, metrics, logp, ent
 
     @staticmethod
+    @torch.autograd.function.once_differentiable
     def backward(ctx, g_loss, g_metrics, g_logp, g_ent):
-        (dlogits,) = ctx.saved_tensors
+        dlogits, *rest = ctx.saved_tensors
         if g_loss is None:
             return None, None, None, None, None, None
-        # in place: the buffer belongs to this node and is handed on once
+        if ctx.consumed:
+            # the gradient buffer is scaled in place and handed on: a second pass would scale it again
+            raise RuntimeError("grpo_loss_from_logits: its backward can run only once (the gradient written by the "
+                               "forward pass is handed to the graph in place); call the function again instead of "
+                               "retain_graph=True")
+        ctx.consumed = True
+        if rest:  # the forward already applied this factor: what remains is g_loss / factor, exactly 1 as a rule
+            g_loss = g_loss.to(torch.float32) / rest[0]
+        # in place: the buffer belongs to this node and is handed on once (the kernel returns at once for a scale of 1)
         return ops.scale_unless_one_(dlogits, g_loss), None, None, None, None, None
 
 
@@ -345,6 +365,7 @@ def grpo_loss_from_logits(
     sapo_temperature_neg: float = 1.05,
     skip_masked_rows: bool = True,
     keep_start: int | None = None,
+    upstream_scale: Tensor | float | None = None,
 ) -> tuple[Tensor, Tensor, Tensor, Tensor]:
     """`[B, L, V]` model logits -> `(loss, metrics, per_token_logps [B, K], entropies [B, K])` with ONE pass over
     the logits: what `per_token_logps_and_entropies` + `grpo_loss` + `loss.backward()` do with two reads and a
@@ -355,7 +376,14 @@ def grpo_loss_from_logits(
     as `grpo_loss`; `keep_start` names another first row of the window.  Only for
     `grpo_single_pass_supported(...)` configurations.  The rows outside `mask` are never read and their log-prob /
     entropy come back as 0, unless `skip_masked_rows=False` asks for them (their gradient is zero either way).  `loss.backward()` hands the `[B, L, V]` gradient
-    to the graph behind `logits`; the returned log-probs and entropies are detached."""
+    to the graph behind `logits`; the returned log-probs and entropies are detached.
+
+    The gradient is written by the forward pass for an upstream gradient of 1; any other upstream gradient costs
+    `backward` one more read and write of the buffer.  A caller that knows the factor it will put on the loss
+    before `backward()` -- the scale of a `GradScaler`, a loss divisor -- passes it as `upstream_scale` (a float or a
+    0-d device tensor): the forward pass then writes the scaled gradient (scaled in fp32 before its one rounding,
+    which is what keeps small fp16 gradients from flushing to zero) and `backward` leaves the buffer alone.  The
+    returned loss is NOT multiplied by it.  `backward` can run once per call."""
     if loss_type not in ops.LOSS_TYPES:
         raise ValueError(f"Unknown loss type: {loss_type}")
     if not grpo_single_pass_supported(logits, loss_type):
@@ -393,7 +421,7 @@ def grpo_loss_from_logits(
               num_processes=num_processes, grad_accum_steps=grad_accum_steps,
               use_bias_correction_kl=use_bias_correction_kl, token_weight=token_weight, entropy_coef=entropy_coef,
               sapo_temperature_pos=sapo_temperature_pos, sapo_temperature_neg=sapo_temperature_neg,
-              skip_masked_rows=skip_masked_rows, keep_start=keep_start)
+              skip_masked_rows=skip_masked_rows, keep_start=keep_start, upstream_scale=upstream_scale)
     return _GRPOFromLogits.apply(logits, completion_ids, advantages, mask, temperature, kw)
 
 
@@ -484,7 +512,15 @@ class GRPOLossMixin:
             logits = outputs.logits
             if logits.shape[-1] > 1 and logits.stride(-1) != 1:
                 logits = logits.contiguous()
-            if grpo_single_pass_supported(logits, self.loss_type):
+            # the factor a gradient scaler (fp16 mixed precision) will put on the loss: a 0-d device tensor, no sync
+            scaler = getattr(self.accelerator, "scaler", None)
+            upstream = None
+            if scaler is not None and getattr(scaler, "is_enabled", lambda: True)():
+                upstream = scaler.scale(torch.ones((), dtype=torch.float32, device=logits.device))
+            # fp16 gradients of a 1e5-entry softmax row sit near the bottom of the fp16 range: the one pass rounds
+            # them once, so it is only taken when the scale is known at that point (or on request)
+            fp16_ok = upstream is not None or getattr(self, "trl_amd_single_pass_fp16", False)
+            if grpo_single_pass_supported(logits, self.loss_type) and (logits.dtype != torch.float16 or fp16_ok):
                 token_weight = None
                 if self.use_vllm and self.vllm_importance_sampling_correction:
                     token_weight = inputs["importance_sampling_ratio"].float().expand(mask.shape)
@@ -498,7 +534,7 @@ class GRPOLossMixin:
                     grad_accum_steps=grad_accum, use_bias_correction_kl=self.args.use_bias_correction_kl,
                     token_weight=token_weight, entropy_coef=apply_coef,
                     sapo_temperature_pos=getattr(self.args, "sapo_temperature_pos", 1.0),
-                    sapo_temperature_neg=getattr(self.args, "sapo_temperature_neg", 1.05))
+                    sapo_temperature_neg=getattr(self.args, "sapo_temperature_neg", 1.05), upstream_scale=upstream)
                 return self._finish_loss(loss, metrics, entropies, mask, None, aux_loss, aux_enabled, grad_accum, mode, bonus)
             # these logits need the two-pass kernels (fp32, a vocabulary too large for one workgroup, ...)
             per_token_logps, entropies = per_token_logps_and_entropies(
