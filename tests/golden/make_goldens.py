@@ -107,6 +107,16 @@ GRPO_CASES = [
          grad_accum=2, adaptive=dict(target=5.0, delta=0.005, max=0.1, min=0.0, last=9.0, sync=True, window=[30.0, 12.0])),
     dict(name="vllm_is_ratio", loss_type="dapo", beta=0.04, eps_low=0.2, eps_high=0.2, is_ratio=True),
     dict(name="vespo_is_ratio", loss_type="vespo", beta=0.0, eps_low=0.2, eps_high=0.2, is_ratio=True),
+    # forms whose per-token term is [B, T] where the common configuration has [B, 1]
+    dict(name="luspo_token", loss_type="luspo", beta=0.04, eps_low=0.2, eps_high=0.2, grad_accum=2),
+    dict(name="luspo_seq_beta", loss_type="luspo", beta=0.04, eps_low=0.05, eps_high=0.05, is_level="sequence", old_noise=0.05),
+    dict(name="luspo_seq_is_ratio", loss_type="luspo", beta=0.0, eps_low=0.05, eps_high=0.05, is_level="sequence",
+         is_ratio=True, old_noise=0.05),
+    dict(name="grpo_seq_is_adv2d", loss_type="grpo", beta=0.04, eps_low=0.05, eps_high=0.05, is_level="sequence",
+         adv_2d=True, old_noise=0.05),
+    dict(name="vespo_adv2d", loss_type="vespo", beta=0.04, eps_low=0.2, eps_high=0.2, adv_2d=True),
+    dict(name="cispo_seq_adv2d", loss_type="cispo", beta=0.0, eps_low=0.2, eps_high=1.02, is_level="sequence", adv_2d=True,
+         old_noise=0.05),
 ]
 
 

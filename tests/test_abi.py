@@ -82,8 +82,6 @@ def test_host_side_argument_validation():
     assert grpo(beta=0.0, term=7) == -5
     assert grpo(beta=0.0, term=_lib.TERM_WEIGHTED_LOGP) == -1  # needs the per-sequence coefficients
     assert grpo(beta=0.0, term=_lib.TERM_SAPO, tau=0.0) == -5
-    assert grpo(beta=0.0, seq=1, adv_stride_t=1) == -7  # sequence-level weights with per-token advantages
-    assert grpo(beta=0.0, loss_type=_lib.LUSPO) == -7  # LUSPO only with sequence-level weights
     assert lib.trlk_grpo_workspace_bytes(64) >= 64 * 10 * 4
     # dpo: odd batch
     assert lib.trlk_dpo_loss(fake, fake, fake, fake, 3, 8, 0.1, fake, fake, fake, fake, None) == -2

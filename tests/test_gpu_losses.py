@@ -81,7 +81,9 @@ def test_golden_grpo_compute_loss_through_trainer_methods(amd, skip_masked, sing
             want_ent = oracle.entropy_from_logits_f32(cpu_logits[:, :-1][:, -T:], tr.temperature)
         else:
             want_lp, want_ent = _t(g[c + "out_logps"]), _t(g[c + "out_entropies"])
-        keep = _t(g[c + "completion_mask"]).float() if skip_masked else torch.ones_like(want_lp)
+        # (luspo's [B, T] forms average over the padding too, so its rows are never skipped)
+        keep = (_t(g[c + "completion_mask"]).float() if skip_masked and case["loss_type"] != "luspo"
+                else torch.ones_like(want_lp))
         if captured:  # (the one-pass branch does not go through the log-prob method)
             torch.testing.assert_close(captured["lp"].detach().cpu(), want_lp * keep, atol=tol, rtol=0)
             torch.testing.assert_close(captured["ent"].detach().cpu(), want_ent * keep, atol=tol, rtol=0)
@@ -104,7 +106,7 @@ def test_golden_grpo_compute_loss_through_trainer_methods(amd, skip_masked, sing
                 torch.testing.assert_close(tr._entropy_window_stats.cpu(), torch.tensor(want["window"]), rtol=1e-5, atol=1e-4)
             assert ("entropy_coef" in got_metrics) == ("entropy_coef" in case["metrics"]), case["name"]
         ran += 1
-    assert ran >= 33
+    assert ran >= 39
 
 
 def test_grpo_loss_against_oracle_random(amd):
@@ -171,8 +173,29 @@ def test_grpo_loss_against_oracle_random(amd):
                 if name == "entropy_coef":
                     continue
                 assert abs(md[name] - want) <= 1e-5 * max(1.0, abs(want)), (tag, name, md[name], want)
-    with pytest.raises(NotImplementedError):
-        amd.grpo_loss(lp.to(DEV), adv.to(DEV), mask.to(DEV), loss_type="luspo", old_per_token_logps=old.to(DEV))
+    # the [B, T] forms: LUSPO with token-level weights / a KL term (its mean then runs over the padding too), and
+    # per-token advantages under sequence-level weights and under vespo
+    adv_bt = adv[:, None] * (0.5 + torch.rand(B, T, generator=g)) - 0.2
+    for lt, level, beta, a_in, o in (("luspo", "token", 0.0, adv, old), ("luspo", "token", 0.04, adv, old),
+                                     ("luspo", "sequence", 0.04, adv, old_seq), ("luspo", "sequence", 0.0, adv_bt, old_seq),
+                                     ("grpo", "sequence", 0.04, adv_bt, old_seq), ("cispo", "sequence", 0.0, adv_bt, old_seq),
+                                     ("dapo", "token", 0.04, adv_bt, old), ("vespo", "token", 0.04, adv_bt, old_seq)):
+        kw = dict(entropies=ent, old_per_token_logps=o, ref_per_token_logps=ref, loss_type=lt, epsilon_low=0.002,
+                  epsilon_high=1.05 if lt == "cispo" else 0.003, beta=beta, max_completion_length=T,
+                  num_items_in_batch=n_items, grad_accum_steps=2.0, importance_sampling_level=level)
+        olp = lp.clone().requires_grad_(True)
+        oloss, ometrics = oracle.grpo_loss(olp, a_in, mask, **kw)
+        oloss.backward()
+        dlp = lp.to(DEV).requires_grad_(True)
+        dkw = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in kw.items()}
+        loss, metrics = amd.grpo_loss(dlp, a_in.to(DEV), mask.to(DEV), **dkw)
+        loss.backward()
+        tag = (lt, level, beta, tuple(a_in.shape))
+        assert abs(float(loss) - float(oloss)) <= 1e-5 * max(1.0, abs(float(oloss))), (tag, float(loss), float(oloss))
+        assert _rel_l2(dlp.grad, olp.grad) < 1e-5, tag
+        md = amd.trainer.metrics_to_dict(metrics, beta, loss_type=lt)
+        for name, want in ometrics.items():
+            assert abs(md[name] - want) <= 1e-5 * max(1.0, abs(want)), (tag, name, md[name], want)
     # determinism: identical bits on a second call
     a = amd.grpo_loss(lp.to(DEV), adv.to(DEV), mask.to(DEV), loss_type="grpo", old_per_token_logps=old.to(DEV))
     b = amd.grpo_loss(lp.to(DEV), adv.to(DEV), mask.to(DEV), loss_type="grpo", old_per_token_logps=old.to(DEV))
@@ -498,3 +521,44 @@ def test_rloo_mixin_compute_loss(amd, skip_masked):
         got = {k: v[-1] for k, v in tr._metrics["train"].items()}
         for name, want_m in case["metrics"].items():
             assert abs(got[name] - want_m) <= 1e-5 * max(1.0, abs(want_m)), (name, got[name], want_m)
+
+
+def test_multimodal_sub_batches_through_the_logprob_method(amd):
+    """`_get_per_token_logps_and_entropies` with `batch_size < B` on a multimodal batch
+    (trl/trainer/grpo_trainer.py:1460-1510): a model whose forward accepts exactly the reference's keyword set sees,
+    per sub-batch, the patch rows and grid rows of that sub-batch's images; the log-probs equal those of one call on
+    the whole batch.  Same keyword set on the one-pass branch of `_compute_loss`."""
+    B, P, T, V, D = 4, 2, 6, 64, 3
+    g = torch.Generator().manual_seed(91)
+    logits = (2.0 * torch.randn(B, P + T, V, generator=g)).bfloat16().to(DEV)
+    ids = torch.randint(0, V, (B, P + T), generator=g).to(DEV)
+    attn = torch.ones(B, P + T, dtype=torch.long, device=DEV)
+    grid = torch.tensor([[1, 2, 2], [1, 2, 3], [1, 1, 4], [1, 3, 2]], device=DEV)
+    num_images = [1, 2, 0, 1]
+    pixels = torch.randn(20, D, generator=g).to(DEV)
+    seen = []
+
+    def model(*, input_ids, attention_mask, pixel_values, image_grid_thw, use_cache, mm_token_type_ids=None):
+        seen.append((input_ids.shape[0], pixel_values.shape[0], image_grid_thw.shape[0]))
+        assert int(image_grid_thw.prod(-1).sum()) == pixel_values.shape[0]
+        rows = [int((ids == r).all(1).nonzero()[0]) for r in input_ids]  # which samples these are
+        return SimpleNamespace(logits=logits[rows], aux_loss=None)
+
+    case = dict(loss_type="dapo", beta=0.0, eps_low=0.2, eps_high=0.2)
+    tr = _fake_trainer(amd, case, T)
+    kw = dict(pixel_values=pixels, image_grid_thw=grid, num_images=num_images)
+    whole, ent_whole, _ = tr._get_per_token_logps_and_entropies(model, ids, attn, T, compute_entropy=True, **kw)
+    parts, ent_parts, _ = tr._get_per_token_logps_and_entropies(model, ids, attn, T, batch_size=2, compute_entropy=True, **kw)
+    assert seen == [(4, 20, 4), (2, 14, 3), (2, 6, 1)]
+    assert torch.equal(whole, parts) and torch.equal(ent_whole, ent_parts)
+    one, _, _ = tr._get_per_token_logps_and_entropies(model, ids, attn, T, batch_size=1, **kw)
+    assert torch.equal(whole, one) and seen[-4:] == [(1, 4, 1), (1, 10, 2), (1, 0, 0), (1, 6, 1)]
+    # `_compute_loss`, both branches: the same keyword set reaches the model (num_images is never passed on)
+    for single_pass in (False, True):
+        tr = _fake_trainer(amd, case, T, skip_masked=True, single_pass=single_pass)
+        inputs = dict(prompt_ids=ids[:, :P], prompt_mask=attn[:, :P], completion_ids=ids[:, P:], completion_mask=attn[:, P:],
+                      advantages=torch.randn(B, generator=g).to(DEV), num_items_in_batch=torch.tensor(24.0, device=DEV),
+                      pixel_values=pixels, image_grid_thw=grid, num_images=num_images)
+        seen.clear()
+        loss = tr._compute_loss(model, inputs)
+        assert seen == [(4, 20, 4)] and math.isfinite(float(loss))

@@ -77,6 +77,7 @@ struct GrpoArgs {
     int64_t adv_stride_b, adv_stride_t;
     int64_t B, T;
     int loss_type, policy_term, seq_level;
+    int luspo_dense;  // LUSPO whose per-token term is [B, T]: every position counts, the padding too (:3143-3148)
     float eps_low, eps_high, delta, beta;
     int bias_kl;
     float grad_accum, dr_denominator;
@@ -100,24 +101,29 @@ __global__ __launch_bounds__(kThreads) void grpo_rows_kernel(GrpoArgs a) {
 
     // sequence-level importance weight: exp(masked mean of the token log-ratios)   (:3057-3059)
     float n_b = 0.f, c_seq = 1.f;
-    if (a.seq_level) {
+    if (a.seq_level || a.luspo_dense) {
         float s1 = 0.f, s0 = 0.f;
         for (int64_t t = tid; t < a.T; t += kThreads) {
             const float m = a.mask[off + t];
             if (m == 0.f) continue;
             s0 += m;
-            if (a.old_logp) s1 += (a.logp[off + t] - a.old_logp[off + t]) * m;
+            if (a.seq_level && a.old_logp) s1 += (a.logp[off + t] - a.old_logp[off + t]) * m;
         }
         s1 = block_sum<kThreads>(s1, scratch);
         n_b = block_sum<kThreads>(s0, scratch);
         c_seq = expf(s1 / fmaxf(n_b, 1.f));
     }
+    // with per-token advantages the clip flags of a sequence-level ratio are per token again (:3237-3250)
+    const bool seq_flags = a.seq_level && a.adv_stride_t == 0;
 
     float s_mask = 0, s_loss = 0, s_kl = 0, s_ent = 0, s_low = 0, s_high = 0, s_reg = 0, s_ent_eff = 0, s_eff = 0;
     float s_aux = 0, s_glnc = 0;
     for (int64_t t = tid; t < a.T; t += kThreads) {
         const float m = a.mask[off + t];
-        if (m == 0.f) {  // a masked token contributes exactly nothing, whatever its (possibly skipped) inputs hold
+        // weight of the token in the loss: the mask, except for the [B, T] form of LUSPO, which averages over
+        // every position of the padded batch
+        const float ml = a.luspo_dense ? 1.f : m;
+        if (ml == 0.f) {  // a masked token contributes exactly nothing, whatever its (possibly skipped) inputs hold
             a.out_dlogp[off + t] = 0.f;
             continue;
         }
@@ -131,7 +137,7 @@ __global__ __launch_bounds__(kThreads) void grpo_rows_kernel(GrpoArgs a) {
         const float H = a.entropy ? a.entropy[off + t] : 0.f;
         const float eff = a.entropy_mask ? m * a.entropy_mask[off + t] : m;
         s_mask += m;
-        s_loss += pl * m;
+        s_loss += pl * ml;
         s_kl += kl * m;
         s_ent += H * m;
         s_low += p.low * m;
@@ -141,15 +147,16 @@ __global__ __launch_bounds__(kThreads) void grpo_rows_kernel(GrpoArgs a) {
         s_ent_eff += H * eff;
         s_eff += eff;
         if (a.seq_level) {
-            s_glnc += g_lnc * m;
-            a.out_dlogp[off + t] = g_lp * m;
+            s_glnc += g_lnc * ml;
+            a.out_dlogp[off + t] = g_lp * ml;
         } else {
-            a.out_dlogp[off + t] = (g_lp + g_lnc) * m;
+            a.out_dlogp[off + t] = (g_lp + g_lnc) * ml;
         }
     }
     float* ws = a.ws + b * kRowStats;
     const float r_mask = block_sum<kThreads>(s_mask, scratch);
-    const float r_loss = block_sum<kThreads>(s_loss, scratch);
+    float r_loss = block_sum<kThreads>(s_loss, scratch);
+    if (a.luspo_dense) r_loss *= r_mask;  // every position's term times the sequence's active-token count
     const float r_kl = block_sum<kThreads>(s_kl, scratch);
     const float r_ent = block_sum<kThreads>(s_ent, scratch);
     float r_low = block_sum<kThreads>(s_low, scratch);
@@ -166,6 +173,8 @@ __global__ __launch_bounds__(kThreads) void grpo_rows_kernel(GrpoArgs a) {
             const float m = a.mask[off + t];
             if (m != 0.f) a.out_dlogp[off + t] += g_seq * m;
         }
+    }
+    if (seq_flags) {
         // clip flags are per sequence: one value each, also for a sequence without active tokens
         const PolicyTerm p = policy_term(a, c_seq, a.adv[b * a.adv_stride_b], 0.f, coef);
         r_low = p.low;
@@ -242,6 +251,10 @@ __global__ __launch_bounds__(kThreads) void grpo_finish_kernel(GrpoArgs a) {
         case TRLK_LUSPO:  // mean over sequences of (per-sequence loss * active tokens)   (:3143-3148)
             loss = tot[RS_LOSS] / Bf;
             norm_rows = 1.f / Bf;
+            if (a.luspo_dense) {  // the same mean taken over all B * T entries of a [B, T] term
+                loss /= float(a.T);
+                norm_rows /= float(a.T);
+            }
             break;
         case TRLK_BNPO:
             loss = tot[RS_LOSS] / fmaxf(tot[RS_MASK], 1.f);
@@ -294,8 +307,9 @@ __global__ __launch_bounds__(kThreads) void grpo_finish_kernel(GrpoArgs a) {
         mt[TRLK_M_AUX_SUM] = tot[RS_AUX];
         mt[TRLK_M_AUX_COUNT] = tot[RS_AUX_CNT];
     }
-    const float row_scale =
-        (a.loss_type == TRLK_GRPO) ? norm_rows / fmaxf(a.ws[b * kRowStats + RS_MASK], 1.f) : norm_rows;
+    const float row_scale = (a.loss_type == TRLK_GRPO) ? norm_rows / fmaxf(a.ws[b * kRowStats + RS_MASK], 1.f)
+                            : a.luspo_dense           ? norm_rows * a.ws[b * kRowStats + RS_MASK]
+                                                      : norm_rows;
     const int64_t off = b * a.T;
     for (int64_t t = tid; t < a.T; t += kThreads) {
         a.out_dlogp[off + t] *= row_scale;
@@ -485,11 +499,6 @@ int grpo_loss_validate(const GrpoLossCall& c) {
                  "grpo_loss: the weighted-logp policy term needs the per-sequence coefficients");
     TRLK_REQUIRE(c.policy_term != TRLK_TERM_SAPO || (c.sapo_temperature_pos > 0.f && c.sapo_temperature_neg > 0.f),
                  TRLK_ERR_BAD_VALUE, "grpo_loss: SAPO temperatures must be positive");
-    TRLK_REQUIRE(c.loss_type != TRLK_LUSPO || (c.sequence_level && c.beta == 0.f && c.d_token_weight == nullptr),
-                 TRLK_ERR_UNSUPPORTED,
-                 "grpo_loss: LUSPO is built for sequence-level importance weights without KL term or token weights");
-    TRLK_REQUIRE(!c.sequence_level || c.adv_stride_t == 0, TRLK_ERR_UNSUPPORTED,
-                 "grpo_loss: sequence-level importance weights need one advantage per sequence");
     TRLK_REQUIRE(c.d_logp && c.d_advantages && c.d_mask && c.d_out_loss && c.d_out_metrics && c.d_out_dlogp, TRLK_ERR_NULL_POINTER,
                  "grpo_loss: a required pointer is null");
     TRLK_REQUIRE(c.beta == 0.f || c.d_ref_logp != nullptr, TRLK_ERR_NULL_POINTER,
@@ -509,9 +518,14 @@ int grpo_loss_validate(const GrpoLossCall& c) {
 // The two launches of the GRPO loss; `ws` holds kRowStats floats per sequence, all of which the first
 // kernel writes before the second reads them (nothing has to be cleared).
 int grpo_loss_launch(const GrpoLossCall& c, float* ws, trlk_stream_t stream) {
+    // LUSPO's per-token term is one value per sequence only with sequence-level weights, one advantage per
+    // sequence, no KL term and no per-token weights; in every other case it is [B, T] and the reference's
+    // mean runs over all B * T entries, masked or not
+    const int luspo_dense = c.loss_type == TRLK_LUSPO &&
+                            !(c.sequence_level && c.beta == 0.f && c.d_token_weight == nullptr && c.adv_stride_t == 0);
     GrpoArgs a{c.d_logp, c.d_old_logp, c.d_ref_logp, c.d_entropy, c.d_advantages, c.d_mask, c.d_token_weight,
                c.d_entropy_mask, c.d_seq_coef, c.adv_stride_b, c.adv_stride_t, c.n_seq, c.seq_len, c.loss_type,
-               c.policy_term, c.sequence_level != 0, c.epsilon_low, c.epsilon_high, c.delta, c.beta,
+               c.policy_term, c.sequence_level != 0, luspo_dense, c.epsilon_low, c.epsilon_high, c.delta, c.beta,
                c.use_bias_correction_kl, c.grad_accum_steps, c.dr_grpo_denominator, c.d_dapo_normalizer,
                c.num_processes, c.entropy_coef, c.sapo_temperature_pos, c.sapo_temperature_neg, c.d_out_loss,
                c.d_out_metrics, c.d_out_dlogp, c.d_out_dentropy, ws};

@@ -67,9 +67,10 @@ def patch_trl(grpo: bool = True, liger: bool = False, dpo: bool = False, rloo: b
             _saved.append((GRPOTrainer, name, GRPOTrainer.__dict__[name]))
             setattr(GRPOTrainer, name, getattr(_grpo.GRPOLossMixin, name))
             count += 1
-        # helper of the mix-in's `_compute_loss` (no method of that name in the reference class)
-        _saved.append((GRPOTrainer, "_finish_loss", GRPOTrainer.__dict__.get("_finish_loss", _MISSING)))
-        GRPOTrainer._finish_loss = _grpo.GRPOLossMixin._finish_loss
+        # helpers of the mix-in's methods (no methods of these names in the reference class)
+        for name in ("_finish_loss", "_model_inputs"):
+            _saved.append((GRPOTrainer, name, GRPOTrainer.__dict__.get(name, _MISSING)))
+            setattr(GRPOTrainer, name, getattr(_grpo.GRPOLossMixin, name))
     if rloo:
         from trl.trainer.rloo_trainer import RLOOTrainer
 
@@ -79,6 +80,8 @@ def patch_trl(grpo: bool = True, liger: bool = False, dpo: bool = False, rloo: b
             _saved.append((RLOOTrainer, name, RLOOTrainer.__dict__[name]))
             setattr(RLOOTrainer, name, getattr(RLOOLossMixin, name))
             count += 1
+        _saved.append((RLOOTrainer, "_model_inputs", RLOOTrainer.__dict__.get("_model_inputs", _MISSING)))
+        RLOOTrainer._model_inputs = RLOOLossMixin._model_inputs
     if kto:
         from trl.trainer.kto_trainer import KTOTrainer
 

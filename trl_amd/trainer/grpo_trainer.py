@@ -184,22 +184,23 @@ def grpo_loss(
     if beta != 0.0 and ref_per_token_logps is None:
         raise KeyError("ref_per_token_logps")
     seq_level = importance_sampling_level == "sequence"
-    if seq_level and advantages.dim() == 2 and advantages.shape[1] != 1:
-        raise NotImplementedError("sequence-level importance weights with per-token advantages are not implemented")
-    if loss_type == "luspo" and (not seq_level or beta != 0.0 or token_weight is not None):
-        # the reference then averages a [B, T] tensor over padding as well; only the (B, 1) form is built here
-        raise NotImplementedError(
-            "luspo is implemented for importance_sampling_level='sequence' without KL term or per-token weights")
     reduce_code, term_code = ops.LOSS_TYPES[loss_type]
     dev = per_token_logps.device
     seq_coef = None
+    phi_tokens = None
     if loss_type == "vespo":
         old = per_token_logps.detach() if old_per_token_logps is None else old_per_token_logps
         adv2 = advantages.unsqueeze(1) if advantages.dim() == 1 else advantages
-        if adv2.shape[1] != 1:
-            raise NotImplementedError("vespo with per-token advantages is not implemented")
-        seq_coef = get_gamma_weights(adv2.float(), per_token_logps.detach().float() - old.float(), mask.float(),
-                                     importance_sampling_ratio, *vespo_params)
+        phi = get_gamma_weights(adv2.float(), per_token_logps.detach().float() - old.float(), mask.float(),
+                                importance_sampling_ratio, *vespo_params)
+        if phi.shape[1] == 1:
+            seq_coef = phi
+        else:
+            # per-token advantages make the coefficients per token (the sign of each advantage picks k and lambda):
+            # they act exactly like a per-token weight on -A * logp, so that is how the kernel gets them
+            phi_tokens = phi
+            seq_coef = torch.ones((phi.shape[0], 1), dtype=torch.float32, device=dev)
+            token_weight = phi if token_weight is None else token_weight.float() * phi
     dapo_norm = None
     dr_denominator = 1.0
     if reduce_code == _lib.DAPO:
@@ -221,6 +222,12 @@ def grpo_loss(
         float(grad_accum_steps), dr_denominator, float(num_processes), float(entropy_coef), term_code, seq_level,
         seq_coef, float(sapo_temperature_pos), float(sapo_temperature_neg),
     )
+    if phi_tokens is not None:  # the logged coefficient is then the masked token mean of phi (grpo_trainer.py:3257-3258)
+        m = mask.float()
+        metrics = metrics.clone()
+        metrics[_METRIC_INDEX["AUX_SUM"]] = (phi_tokens * m).sum()
+        metrics[_METRIC_INDEX["AUX_COUNT"]] = m.sum()
+        metrics[_METRIC_INDEX["AUX_MEAN"]] = metrics[_METRIC_INDEX["AUX_SUM"]] / m.sum().clamp(min=1.0)
     return loss, metrics
 
 
@@ -428,32 +435,76 @@ def grpo_loss_from_logits(
 class GRPOLossMixin:
     """Methods with the reference's names and signatures; bind them onto a `GRPOTrainer`."""
 
+    def _model_inputs(self, input_ids, attention_mask, start, stop, logits_to_keep, compute_aux_loss, *, pixel_values=None,
+                      image_grid_thw=None, num_images=None, pixel_attention_mask=None, spatial_shapes=None,
+                      num_tiles=None, image_sizes=None, token_type_ids=None, mm_token_type_ids=None,
+                      image_position_ids=None):
+        """Keyword arguments of the model call for the samples `start:stop` (trl/trainer/grpo_trainer.py:1463-1510).
+        The vision tensors are indexed by patch row, image or tile rather than by sample, so the sample range is
+        translated through `image_grid_thw` / `num_images` / `num_tiles`; those two lists only steer the slicing
+        and are never model arguments."""
+        out = {"input_ids": input_ids[start:stop], "attention_mask": attention_mask[start:stop]}
+        if pixel_values is not None:
+            if image_grid_thw is not None:  # patch rows of all images concatenated; one grid row per image
+                first_image = [0]
+                for n in num_images:
+                    first_image.append(first_image[-1] + int(n))
+                rows_per_image = image_grid_thw.prod(dim=-1)
+                img0, img1 = first_image[start], first_image[stop]
+                row0 = int(rows_per_image[:img0].sum())
+                row1 = row0 + int(rows_per_image[img0:img1].sum())
+                out["pixel_values"] = pixel_values[row0:row1]
+                out["image_grid_thw"] = image_grid_thw[img0:img1]
+            elif image_position_ids is not None:  # image-indexed tensors
+                img0, img1 = sum(int(n) for n in num_images[:start]), sum(int(n) for n in num_images[:stop])
+                out["pixel_values"] = pixel_values[img0:img1]
+                out["image_position_ids"] = image_position_ids[img0:img1]
+            elif spatial_shapes is not None:  # tile-indexed tensors
+                t0, t1 = sum(int(n) for n in num_tiles[:start]), sum(int(n) for n in num_tiles[:stop])
+                out["pixel_values"] = pixel_values[t0:t1]
+                out["pixel_attention_mask"] = pixel_attention_mask[t0:t1]
+                out["spatial_shapes"] = spatial_shapes[t0:t1]
+            else:
+                out["pixel_values"] = pixel_values[start:stop]
+        if pixel_attention_mask is not None and spatial_shapes is None:
+            out["pixel_attention_mask"] = pixel_attention_mask[start:stop]
+        for name, value in (("image_sizes", image_sizes), ("token_type_ids", token_type_ids),
+                            ("mm_token_type_ids", mm_token_type_ids)):
+            if value is not None:
+                out[name] = value[start:stop]
+        if "logits_to_keep" in getattr(self, "model_kwarg_keys", ()):
+            out["logits_to_keep"] = logits_to_keep + 1  # (the last position is dropped afterwards)
+        out["use_cache"] = False
+        if compute_aux_loss:
+            out["output_router_logits"] = True
+        return out
+
     def _get_per_token_logps_and_entropies(
         self, model, input_ids, attention_mask, logits_to_keep, batch_size=None, compute_entropy=False,
-        compute_aux_loss=False, skip_rows_mask=None, **model_extra_inputs,
+        compute_aux_loss=False, pixel_values=None, image_grid_thw=None, num_images=None, pixel_attention_mask=None,
+        spatial_shapes=None, num_tiles=None, image_sizes=None, token_type_ids=None, mm_token_type_ids=None,
+        image_position_ids=None, skip_rows_mask=None,
     ):
-        """Reference: trl/trainer/grpo_trainer.py:1435-1541.  Multimodal extras are forwarded to the
-        model only when the whole batch goes through in one piece (no per-sample splitting here).
+        """Reference: trl/trainer/grpo_trainer.py:1435-1541, sub-batches and multimodal inputs included.
         `skip_rows_mask` (`[B, logits_to_keep]`, not in the reference) names rows whose log-prob and
         entropy the caller will discard: they are not read and come back as 0."""
-        batch_size = batch_size or input_ids.size(0)
-        extras = {k: v for k, v in model_extra_inputs.items() if v is not None}
-        if extras and batch_size < input_ids.size(0):
-            raise NotImplementedError("sub-batching of multimodal inputs is not supported by trl_amd")
+        total = input_ids.size(0)
+        batch_size = batch_size or total
+        vision = dict(pixel_values=pixel_values, image_grid_thw=image_grid_thw, num_images=num_images,
+                      pixel_attention_mask=pixel_attention_mask, spatial_shapes=spatial_shapes, num_tiles=num_tiles,
+                      image_sizes=image_sizes, token_type_ids=token_type_ids, mm_token_type_ids=mm_token_type_ids,
+                      image_position_ids=image_position_ids)
         all_logps, all_entropies, all_aux = [], [], []
         entropy_grad = bool(getattr(self, "_entropy_bonus_enabled", False))
-        for start in range(0, input_ids.size(0), batch_size):
-            ids = input_ids[start : start + batch_size]
-            model_inputs = {"input_ids": ids, "attention_mask": attention_mask[start : start + batch_size], **extras}
-            if "logits_to_keep" in getattr(self, "model_kwarg_keys", ()):
-                model_inputs["logits_to_keep"] = logits_to_keep + 1
-            model_inputs["use_cache"] = False
-            if compute_aux_loss:
-                model_inputs["output_router_logits"] = True
+        for start in range(0, total, batch_size):
+            stop = min(start + batch_size, total)
+            model_inputs = self._model_inputs(input_ids, attention_mask, start, stop, logits_to_keep, compute_aux_loss,
+                                              **vision)
             outputs = model(**model_inputs)
-            rows = None if skip_rows_mask is None else skip_rows_mask[start : start + batch_size]
+            rows = None if skip_rows_mask is None else skip_rows_mask[start:stop]
             logps, ent = per_token_logps_and_entropies(
-                outputs.logits, ids, logits_to_keep, self.temperature, compute_entropy, entropy_grad, rows
+                outputs.logits, model_inputs["input_ids"], logits_to_keep, self.temperature, compute_entropy,
+                entropy_grad, rows
             )
             all_logps.append(logps)
             if compute_entropy:
@@ -482,6 +533,8 @@ class GRPOLossMixin:
         # Every use of the log-probs and entropies below is multiplied by `mask`, so rows with mask == 0
         # need not be computed at all (set `trl_amd_skip_masked_rows = False` on the trainer to compute them).
         skip = mask if getattr(self, "trl_amd_skip_masked_rows", True) else None
+        if self.loss_type == "luspo":
+            skip = None  # (its [B, T] forms average over the padding as well: every row's log-prob is needed)
         advantages = inputs["advantages"]
         mode = "train" if self.model.training else "eval"
         grad_accum = self.current_gradient_accumulation_steps if mode == "train" else 1.0
@@ -501,12 +554,8 @@ class GRPOLossMixin:
             and self.top_entropy_quantile >= 1.0 and self.off_policy_mask_threshold is None
         )
         if single_pass:
-            model_inputs = {"input_ids": input_ids, "attention_mask": attention_mask, "use_cache": False,
-                            **{k: inputs[k] for k in extra_keys if inputs.get(k) is not None}}
-            if "logits_to_keep" in getattr(self, "model_kwarg_keys", ()):
-                model_inputs["logits_to_keep"] = logits_to_keep + 1
-            if aux_enabled:
-                model_inputs["output_router_logits"] = True
+            model_inputs = self._model_inputs(input_ids, attention_mask, 0, input_ids.size(0), logits_to_keep, aux_enabled,
+                                              **{k: inputs.get(k) for k in extra_keys})
             outputs = model(**model_inputs)
             aux_loss = outputs.aux_loss if aux_enabled else None
             logits = outputs.logits

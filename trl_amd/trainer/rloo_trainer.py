@@ -44,6 +44,7 @@ class RLOOLossMixin:
     from .grpo_trainer import GRPOLossMixin as _G
 
     _get_per_token_logps_and_entropies = _G._get_per_token_logps_and_entropies
+    _model_inputs = _G._model_inputs
     del _G
 
     def _compute_loss(self, model, inputs):
