@@ -52,6 +52,9 @@ class IdentityAccelerator:
     def pad_across_processes(self, x, dim=0, pad_index=0):
         return x
 
+    def unwrap_model(self, model):
+        return model
+
 
 def fake_grpo_trainer(amd, case, T, skip_masked=False, single_pass=False):
     """A bare object with `GRPOLossMixin`'s methods and the trainer attributes they read, set from one golden case

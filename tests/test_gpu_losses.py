@@ -308,6 +308,62 @@ def test_dpo_mixin_compute_loss(amd):
     seq = amd.dpo_sequence_logps(leaf.detach(), inputs["input_ids"], inputs["completion_mask"])
     oseq, _ = oracle.dpo_sequence_logps(_t(g[c + "logits"]), _t(g[c + "input_ids"]), _t(g[c + "completion_mask"]))
     torch.testing.assert_close(seq.cpu(), oseq, rtol=1e-5, atol=1e-5)
+    # reference log-probs computed inside the loss: from `ref_model`, and from the policy itself with its PEFT
+    # adapters switched off or switched to the adapter named "ref" (dpo_trainer.py:1187-1195, 1373-1394).  The
+    # stand-in model answers with other logits while it is in its reference state; the loss must equal the one
+    # computed from those logits' sequence log-probs handed in precomputed.
+    g2 = torch.Generator().manual_seed(5)
+    ref_logits = (_t(g[c + "logits"]) + 0.3 * torch.randn(_t(g[c + "logits"]).shape, generator=g2)).to(DEV)
+    ref_seq = amd.dpo_sequence_logps(ref_logits, inputs["input_ids"], inputs["completion_mask"], case["ld_alpha"])
+    tr.precompute_ref_logps = True
+    want = tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None),
+                            dict(inputs, ref_chosen_logps=ref_seq[:3], ref_rejected_logps=ref_seq[3:]), False)
+
+    class FakePeft:
+        def __init__(self, adapters):
+            self.peft_config = {name: object() for name in adapters}
+            self.active_adapter = "default"
+            self.disabled = False
+            self.log = []
+
+        def set_adapter(self, name):
+            self.log.append(name)
+            self.active_adapter = name
+
+        def disable_adapter(self):
+            from contextlib import contextmanager
+
+            @contextmanager
+            def ctx():
+                self.disabled = True
+                self.log.append("off")
+                try:
+                    yield
+                finally:
+                    self.disabled = False
+                    self.log.append("on")
+
+            return ctx()
+
+        def __call__(self, **kw):
+            assert "output_router_logits" not in kw
+            in_ref_state = self.disabled or self.active_adapter == "ref"
+            return SimpleNamespace(logits=ref_logits if in_ref_state else leaf, aux_loss=None)
+
+    live = {k: v for k, v in inputs.items() if not k.startswith("ref_")}
+    tr.precompute_ref_logps = False
+    for adapters, trace in ((["default"], ["off", "on"]), (["default", "ref"], ["ref", "default"])):
+        peft = FakePeft(adapters)
+        tr.ref_model, tr.model = None, peft
+        peft.training = True
+        got = tr._compute_loss(peft, live, False)
+        assert torch.equal(got, want) and peft.log == trace and peft.active_adapter == "default" and not peft.disabled
+    tr.ref_model = lambda **kw: SimpleNamespace(logits=ref_logits)
+    tr.model = SimpleNamespace(training=True)
+    assert torch.equal(tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None), live, False), want)
+    tr.ref_model = None
+    with pytest.raises(ValueError, match="reference log-probs"):
+        tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None), live, False)
 
 
 @pytest.mark.parametrize("skip_masked", [True, False])

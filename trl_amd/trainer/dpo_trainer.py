@@ -3,6 +3,8 @@ the fused sigmoid path (`dpo_sigmoid_loss`, one loss kernel) and the general one
 loss types, `ld_alpha`, WPO weighting, f-divergences, every logged metric from one pass over the logits)."""
 from __future__ import annotations
 
+from contextlib import contextmanager
+
 import torch
 import torch.nn.functional as F
 from torch import Tensor
@@ -199,13 +201,30 @@ def dpo_metrics_to_dict(metrics: dict) -> dict[str, float]:
     }
 
 
+@contextmanager
+def _reference_adapter(peft_model):
+    """Puts a PEFT model into its reference state for the block (trl/trainer/utils.py:1199-1236 as used at
+    dpo_trainer.py:1187-1195, 1373-1380): the adapter named "ref" if there is one, otherwise no adapter at all;
+    the previous state comes back afterwards."""
+    if "ref" in peft_model.peft_config:
+        previous = peft_model.active_adapter
+        peft_model.set_adapter("ref")
+        try:
+            yield
+        finally:
+            peft_model.set_adapter(previous)
+    else:
+        with peft_model.disable_adapter():
+            yield
+
+
 class DPOLossMixin:
     """`_compute_loss` with the reference's name and signature; bind it onto a `DPOTrainer`."""
 
     def _compute_loss(self, model, inputs, return_outputs):
         """Reference: trl/trainer/dpo_trainer.py:1329-1655.  The policy forward is the model's own; the log-prob,
         loss and metric arithmetic runs on the kernels.  Without precomputed reference log-probs the reference
-        model is run under `no_grad` (the PEFT adapter-switching variant is left to the reference)."""
+        model is run under `no_grad`, or the policy itself with its PEFT adapters switched to the reference."""
         mode = "train" if self.model.training else "eval"
         skip = {"completion_mask", "ref_chosen_logps", "ref_rejected_logps"}
         model_kwargs = {k: v for k, v in inputs.items() if k not in skip}
@@ -221,11 +240,19 @@ class DPOLossMixin:
         if self.precompute_ref_logps:
             ref_c, ref_r = inputs["ref_chosen_logps"], inputs["ref_rejected_logps"]
         else:
-            if getattr(self, "ref_model", None) is None:
-                raise NotImplementedError("reference log-probs from a PEFT adapter switch are not implemented by trl_amd")
             with torch.no_grad():
                 ref_kwargs = {k: v for k, v in model_kwargs.items() if k != "output_router_logits"}
-                ref_logits = self.ref_model(**ref_kwargs).logits
+                if getattr(self, "ref_model", None) is not None:
+                    ref_logits = self.ref_model(**ref_kwargs).logits
+                else:
+                    # adapter training without a separate reference model: the reference is the same network with
+                    # its adapters switched off, or with the frozen copy named "ref" active (dpo_trainer.py:1373-1380)
+                    peft_model = self.accelerator.unwrap_model(model)
+                    if not hasattr(peft_model, "peft_config"):
+                        raise ValueError("DPO needs reference log-probs: precomputed, from `ref_model`, or from a PEFT "
+                                         "model whose adapters can be switched off")
+                    with _reference_adapter(peft_model):
+                        ref_logits = self.model(**ref_kwargs).logits
                 ref_seq = dpo_sequence_logps(ref_logits, input_ids, completion_mask, self.ld_alpha)
             ref_c, ref_r = ref_seq.chunk(2)
         loss, parts = dpo_compute_loss(
