@@ -1,20 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the GRPO log-prob + loss forward/backward path on one MI355X.
 
-One "step" = one pass of the hot path over one synthetic batch that is already resident in HBM:
-  K1  log-prob + entropy forward over bf16 logits [64, 1024, 151936] (temperature 0.9)
-  K2  GRPO loss + metrics + d loss/d logp on [64, 1024]
-  K3  recompute backward writing dlogits [64, 1024, 151936] bf16
-(benchmark configuration "GRPO loss fwd+bwd").  Prints ONE JSON line.
+One "step" = one pass of the hot path over one synthetic batch that is already resident in HBM.  For the headline
+workload (benchmark configuration "GRPO loss fwd+bwd": bf16 logits [64, 1024, 151936], temperature 0.9) the step
+is timed four ways -- two passes over the logits (K1 log-prob kernel, [B, T] loss kernel, K3 gradient kernel) and one
+pass (K7, which writes a row's gradient from the registers that hold the row), each with and without the rows outside
+the completion mask -- and the headline is the fastest that produces every stated output.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--loss-type dapo] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--loss-type dapo] [--no-cpu-baseline]
 
-`value` is token positions per second over the K timed steps (events on torch's current stream,
-which is the stream the kernels are enqueued on, bracketed by device synchronisation).
-`roofline` is for the dominant kernel (K3): algorithmic bytes per launch / average launch time,
-measured live with events around K launches of that kernel alone.
-`cpu_baseline` times the CPU oracle (a port of the reference path, oracle/) on a bounded row
-sample of the same workload on this host's cores.
+`value` is token positions per second over the K timed steps (events on torch's current stream, which is the stream
+the kernels are enqueued on, bracketed by device synchronisation).  `roofline` is for the dominant kernel of the
+headline step: algorithmic bytes per launch / average launch time, measured live with events around back-to-back
+launches of that kernel alone; `step_hbm_GBps` prices the whole step by the bytes its kernels move.
+`cpu_baseline` times the CPU oracle (a port of the reference path, oracle/) on a bounded row sample of the same
+workload on this host's cores.  Without `--workload` the line also carries `secondary`: the other loss types of the
+headline workload and the other benchmark configurations (long context, DPO, fused head), each with its step time,
+its dominant kernel's roofline figures and -- where the one-pass kernel runs -- the relative L2 distance between its
+gradient and the two-pass gradient.
 """
 from __future__ import annotations
 
@@ -30,17 +33,15 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
-# HBM bytes per K3 launch from rocprofv3 FETCH_SIZE / WRITE_SIZE (two --pmc runs of this file, scaled by a plain
-# device copy of known size: FETCH x 2.000, WRITE x 1.000 KiB); the inputs are seeded, so the figure is stable.
-MEASURED_K3_TRAFFIC_BYTES = {("grpo_c3", "dapo"): (10116130 + 19461194) * 1024}
-# The same two counters for one forward launch of the fused head with its stash stores (FETCH_SIZE varies between
-# 36.6e6 and 44.0e6 over the launches of a run; the mean is used): what leaves the L2s towards memory.  The writes
-# are the stash plus the partial results; the reads are the operand tiles that miss the L2 of their XCD, about 60
-# times the 1.3 GB of the two operands.
-# The same for one launch of the single-pass kernel (rows without gradient zero-filled, not read: FETCH 5058750 x 2 KiB,
-# WRITE 19481000 KiB; with every row read: FETCH 9731350 x 2 KiB, WRITE 19470000 KiB).
-MEASURED_K7_TRAFFIC_BYTES = {("grpo_c3", "dapo"): (2 * 5058750 + 19481000) * 1024}
-MEASURED_HEAD_FWD_TRAFFIC_BYTES = {"head_c5": (2 * 40600000 + 19497000) * 1024}
+# HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE (two --pmc runs of this file,
+# each scaled by the same counter's reading for a plain device copy of known size: FETCH x 2.000, WRITE x 1.000 KiB;
+# summaries under profiles/).  The inputs are seeded, so the figures are stable; they are records of those runs, not
+# measured by the run that prints them, and None where no counter run was made for that workload / loss type.
+MEASURED_TRAFFIC_BYTES = {
+    ("K3", "grpo_c3", "dapo"): (10116130 + 19461194) * 1024,
+    ("K7", "grpo_c3", "dapo"): (2 * 5058750 + 19481000) * 1024,
+    ("head_fwd", "head_c5", "dapo"): (2 * 40600000 + 19497000) * 1024,
+}
 
 WORKLOADS = {
     # name: (n_seq, completion_len, vocab, temperature, group_size, min_len)
@@ -305,7 +306,7 @@ def bench_head(args, w):
         # two sub-0.1 ms helper kernels)
         "roofline": {"bound": "mfma", "kernel": "fused_head_fwd_kernel", "achieved": fwd_tf,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": fwd_tf / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": MEASURED_HEAD_FWD_TRAFFIC_BYTES.get(args.workload) if stash else None,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(("head_fwd", args.workload, "dapo")) if stash else None,
                      "algorithmic_flop": flop, "avg_launch_ms": fwd_ms,
                      "forward_plus_backward": {"achieved": total_tf, "frac": total_tf / MFMA_BF16_PEAK_TFLOPS,
                                                "executed_flop": flop + bwd_flop, "ms": fwd_ms + bwd_ms}},
@@ -328,7 +329,7 @@ def bench_head(args, w):
         torch.cuda.synchronize()
         result["calibration_copy_bytes_each_way"] = V * H * 2
         del dst
-    print(json.dumps(result))
+    return result
 
 
 def bench_dpo(args, w):
@@ -417,55 +418,54 @@ def bench_dpo(args, w):
                        "note": "only rows inside the completion mask are read; loss, metrics and dlogits identical"},
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_dpo(w),
     }
-    print(json.dumps(result))
+    return result
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="grpo_c3", choices=sorted(WORKLOADS))
-    ap.add_argument("--loss-type", default="dapo", choices=["grpo", "dapo", "dr_grpo", "bnpo"])
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run a plain device copy of the logits (known bytes) to scale profiler counters by")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        sys.exit("bench.py: this build runs on ONE GPU; rows are independent, so N GPUs would each run this same "
-                 "kernel on B/N sequences and exchange a handful of scalars per step. Run with --gpus 1.")
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible; the hot path has no CPU fallback.")
+def _grad_distance(run_a, run_b, leaf):
+    """Relative L2 distance between the gradients two step functions leave in `leaf.grad`, accumulated sequence
+    by sequence (no logits-sized fp32 temporaries)."""
+    run_a()
+    ga = leaf.grad
+    leaf.grad = None
+    run_b()
+    gb = leaf.grad
+    num = den = 0.0
+    for b in range(ga.shape[0]):
+        x, y = ga[b].float(), gb[b].float()
+        num += float((x - y).square().sum())
+        den += float(y.square().sum())
+    leaf.grad = None
+    del ga, gb
+    return (num / max(den, 1e-300)) ** 0.5
 
+
+def bench_grpo(args, w, loss_type, shared=None, full=True):
+    """One GRPO workload and loss type.  `shared` carries the inputs of an earlier call on the same workload;
+    `full` adds the two-pass kernel timings, the mask-aware two-pass leg and the scaled-upstream-gradient leg."""
     import trl_amd
     from trl_amd import ops
 
-    w = WORKLOADS[args.workload]
-    if w.get("head"):
-        torch.cuda.set_device(0)
-        return bench_head(args, w)
-    if w.get("dpo"):
-        torch.cuda.set_device(0)
-        return bench_dpo(args, w)
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
     B, T, V = w["B"], w["T"], w["V"]
     R = B * T
-    logits, ids, mask, rewards, g = make_inputs(w, dev)
-    adv = trl_amd.group_advantages(rewards, w["G"])
-    with torch.no_grad():
-        base, _ = trl_amd.logps_and_entropies(logits, ids, w["temperature"])
-    old = base + 0.05 * torch.randn(base.shape, generator=g, device=dev)
-    ref = base + 0.1 * torch.randn(base.shape, generator=g, device=dev) if w["beta"] else None
-    n_items = mask.sum().float()
-    leaf = logits.requires_grad_(True)
+    if shared is None:
+        logits, ids, mask, rewards, g = make_inputs(w, dev)
+        adv = trl_amd.group_advantages(rewards, w["G"])
+        with torch.no_grad():
+            base, _ = trl_amd.logps_and_entropies(logits, ids, w["temperature"])
+        old = base + 0.05 * torch.randn(base.shape, generator=g, device=dev)
+        ref = base + 0.1 * torch.randn(base.shape, generator=g, device=dev) if w["beta"] else None
+        shared = dict(logits=logits, ids=ids, mask=mask, adv=adv, old=old, ref=ref, n_items=mask.sum().float(),
+                      leaf=logits.requires_grad_(True))
+    logits, ids, mask, adv, old, ref, n_items, leaf = (shared[k] for k in ("logits", "ids", "mask", "adv", "old", "ref",
+                                                                        "n_items", "leaf"))
 
     def step(row_mask=None):
         leaf.grad = None
         lp, ent = trl_amd.logps_and_entropies(leaf, ids, w["temperature"], row_mask=row_mask)
         loss, metrics = trl_amd.grpo_loss(
             lp, adv, mask, entropies=ent.detach(), old_per_token_logps=old, ref_per_token_logps=ref,
-            loss_type=args.loss_type, epsilon_low=w["eps_low"], epsilon_high=w["eps_high"], beta=w["beta"],
+            loss_type=loss_type, epsilon_low=w["eps_low"], epsilon_high=w["eps_high"], beta=w["beta"],
             max_completion_length=T, num_items_in_batch=n_items)
         loss.backward()
         return loss, metrics
@@ -488,27 +488,36 @@ def main():
     # entropy is produced (the configuration's stated outputs)
     ms_two_pass, loss_value = timed(lambda: step(None))
     assert loss_value == loss_value, "loss is NaN"
-    # the forward also skips the rows the completion mask zeroes (what `_compute_loss` does by default)
-    ms_mask_aware, loss_mask_aware = timed(lambda: step(mask))
-    assert abs(loss_mask_aware - loss_value) <= 1e-6 * max(1.0, abs(loss_value)), "mask-aware loss differs"
+    ms_mask_aware = None
+    if full:  # the forward also skips the rows the completion mask zeroes (what `_compute_loss` does by default)
+        ms_mask_aware, loss_mask_aware = timed(lambda: step(mask))
+        assert abs(loss_mask_aware - loss_value) <= 1e-6 * max(1.0, abs(loss_value)), "mask-aware loss differs"
 
     # one pass over the logits: the kernel that computes a row's log-prob also writes that row's gradient
     single = None
-    if trl_amd.grpo_single_pass_supported(leaf, args.loss_type):
-        def sp_step(skip):
+    if trl_amd.grpo_single_pass_supported(leaf, loss_type):
+        def sp_step(skip, factor=None, tell=False):
             leaf.grad = None
             loss, metrics, _, _ = trl_amd.grpo_loss_from_logits(
                 leaf, ids, adv, mask, temperature=w["temperature"], old_per_token_logps=old, ref_per_token_logps=ref,
-                loss_type=args.loss_type, epsilon_low=w["eps_low"], epsilon_high=w["eps_high"], beta=w["beta"],
-                max_completion_length=T, num_items_in_batch=n_items, keep_start=0, skip_masked_rows=skip)
-            loss.backward()
+                loss_type=loss_type, epsilon_low=w["eps_low"], epsilon_high=w["eps_high"], beta=w["beta"],
+                max_completion_length=T, num_items_in_batch=n_items, keep_start=0, skip_masked_rows=skip,
+                upstream_scale=factor if tell else None)
+            (loss if factor is None else loss * factor).backward()
             return loss, metrics
 
         ms_sp_all, loss_sp = timed(lambda: sp_step(False))
         assert abs(loss_sp - loss_value) <= 1e-6 * max(1.0, abs(loss_value)), "single-pass loss differs"
         ms_sp_skip, loss_sp2 = timed(lambda: sp_step(True))
         assert abs(loss_sp2 - loss_value) <= 1e-6 * max(1.0, abs(loss_value)), "single-pass (mask-aware) loss differs"
-        single = {"all_rows_ms": ms_sp_all, "mask_aware_ms": ms_sp_skip}
+        single = {"all_rows_ms": ms_sp_all, "mask_aware_ms": ms_sp_skip,
+                  # the gradient of the one pass against the gradient of the two passes (both rounded to bf16 once)
+                  "dlogits_rel_l2_vs_two_pass": _grad_distance(lambda: sp_step(False), lambda: step(None), leaf)}
+        if full:
+            # an upstream gradient other than 1 (a gradient scaler): announced to the forward it costs nothing,
+            # unannounced it costs a further read + write of the gradient in `backward`
+            single["scaled_upstream_ms"] = {"announced": timed(lambda: sp_step(True, 1024.0, True))[0],
+                                            "unannounced": timed(lambda: sp_step(True, 1024.0, False))[0]}
     # headline: the fastest path that produces every stated output (log-prob and entropy of every row, loss, dlogits)
     ms_per_step = min(ms_two_pass, single["all_rows_ms"]) if single else ms_two_pass
     headline_single = single is not None and single["all_rows_ms"] <= ms_two_pass
@@ -518,11 +527,10 @@ def main():
     idx = ids.reshape(R, 1)
     with torch.no_grad():
         lp_flat, ent_flat, lse = ops.logp_entropy_fwd(logits.detach(), idx, w["temperature"], 0, T, None)
-    g_logp = (leaf.grad is not None) and None
     loss2, _, dlogp, _ = ops.grpo_loss_op(
         lp_flat.view(B, T), old, ref, ent_flat.view(B, T), adv, mask, None, None, n_items,
-        ops.LOSS_TYPES[args.loss_type][0], w["eps_low"], w["eps_high"], float("nan"), w["beta"], False, 1.0,
-        float(B * T), 1.0, 0.0, ops.LOSS_TYPES[args.loss_type][1])
+        ops.LOSS_TYPES[loss_type][0], w["eps_low"], w["eps_high"], float("nan"), w["beta"], False, 1.0,
+        float(B * T), 1.0, 0.0, ops.LOSS_TYPES[loss_type][1])
     g_logp = dlogp.reshape(R, 1).contiguous()
     leaf.grad = None
     reps = max(3, min(args.steps, 10))
@@ -539,31 +547,40 @@ def main():
         torch.cuda.synchronize()
         return a.elapsed_time(b) / reps
 
-    with torch.no_grad():
-        fwd_ms = time_kernel(lambda: ops.logp_entropy_fwd(logits.detach(), idx, w["temperature"], 0, T, None))
-        bwd_ms = time_kernel(lambda: ops.logp_entropy_bwd(logits.detach(), idx, w["temperature"], 0, T, lse, None,
-                                                          g_logp, None))
     row_bytes = V * 2
     active_rows = int((g_logp != 0).sum())
     fwd_bytes = R * row_bytes
     bwd_bytes = active_rows * 2 * row_bytes + (R - active_rows) * row_bytes  # masked rows: zero-fill write only
-    fwd_gbps = fwd_bytes / (fwd_ms * 1e-3) / 1e9
-    bwd_gbps = bwd_bytes / (bwd_ms * 1e-3) / 1e9
-    roofline = {
-        "bound": "hbm", "kernel": "logp_entropy_bwd_kernel (K3)", "achieved": bwd_gbps, "peak": HBM_PEAK_GBPS,
-        "unit": "GB/s", "frac": bwd_gbps / HBM_PEAK_GBPS,
-        "traffic": MEASURED_K3_TRAFFIC_BYTES.get((args.workload, args.loss_type)), "algorithmic_bytes": bwd_bytes,
-        "avg_launch_ms": bwd_ms,
-    }
     kernels = {}
+    roofline = None
+    fwd_ms = bwd_ms = None
+    if full or not headline_single:
+        with torch.no_grad():
+            fwd_ms = time_kernel(lambda: ops.logp_entropy_fwd(logits.detach(), idx, w["temperature"], 0, T, None))
+            bwd_ms = time_kernel(lambda: ops.logp_entropy_bwd(logits.detach(), idx, w["temperature"], 0, T, lse, None,
+                                                              g_logp, None))
+        fwd_gbps = fwd_bytes / (fwd_ms * 1e-3) / 1e9
+        bwd_gbps = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+        roofline = {
+            "bound": "hbm", "kernel": "logp_entropy_bwd_kernel (K3)", "achieved": bwd_gbps, "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s", "frac": bwd_gbps / HBM_PEAK_GBPS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(("K3", args.workload, loss_type)), "algorithmic_bytes": bwd_bytes,
+            "avg_launch_ms": bwd_ms,
+        }
+        kernels.update({
+            "logp_entropy_fwd_kernel (K1)": {"avg_launch_ms": fwd_ms, "algorithmic_bytes": fwd_bytes,
+                                             "achieved_GBps": fwd_gbps, "frac": fwd_gbps / HBM_PEAK_GBPS},
+            "logp_entropy_bwd_kernel (K3)": {"avg_launch_ms": bwd_ms, "algorithmic_bytes": bwd_bytes,
+                                             "achieved_GBps": bwd_gbps, "frac": bwd_gbps / HBM_PEAK_GBPS},
+            "two_pass_step_hbm_GBps": (fwd_bytes + bwd_bytes) / (ms_two_pass * 1e-3) / 1e9,
+        })
+    step_bytes = fwd_bytes + bwd_bytes  # what the two-pass step moves
     if single:
-        reduce_code, term_code = ops.LOSS_TYPES[args.loss_type]
+        reduce_code, term_code = ops.LOSS_TYPES[loss_type]
         if reduce_code == 0:  # per-sequence mean
             row_scale = 1.0 / B / mask.float().sum(1).clamp(min=1.0)
-        elif args.loss_type == "dr_grpo":
+        elif loss_type == "dr_grpo":
             row_scale = torch.full((B,), 1.0 / (B * T), device=dev)
-        elif args.loss_type == "bnpo":
-            row_scale = (1.0 / n_items.clamp(min=1.0)).expand(B)
         else:
             row_scale = (1.0 / n_items.clamp(min=1.0)).expand(B)
 
@@ -573,26 +590,30 @@ def main():
                                           1.0, 1.05, all_rows)
 
         with torch.no_grad():
-            sp_all_ms = time_kernel(lambda: fused(True))
             sp_skip_ms = time_kernel(lambda: fused(False))
+            sp_all_ms = time_kernel(lambda: fused(True)) if full else None
         sp_all_bytes = 2 * R * row_bytes                              # every row read, every gradient row written
         sp_skip_bytes = active_rows * 2 * row_bytes + (R - active_rows) * row_bytes
         for name, ms_k, nbytes in (("grpo_fused_kernel (K7), masked rows not read", sp_skip_ms, sp_skip_bytes),
                                    ("grpo_fused_kernel (K7), every row read (C entry only)", sp_all_ms, sp_all_bytes)):
-            kernels[name] = {"avg_launch_ms": ms_k, "algorithmic_bytes": nbytes,
-                             "achieved_GBps": nbytes / (ms_k * 1e-3) / 1e9,
-                             "frac": nbytes / (ms_k * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+            if ms_k is not None:
+                kernels[name] = {"avg_launch_ms": ms_k, "algorithmic_bytes": nbytes,
+                                 "achieved_GBps": nbytes / (ms_k * 1e-3) / 1e9,
+                                 "frac": nbytes / (ms_k * 1e-3) / 1e9 / HBM_PEAK_GBPS}
         if headline_single:
             # the headline step = this kernel on the rows with gradient (the others zero-filled) + the forward kernel
             # on the rows without gradient, for their log-probs and entropies
             gbps = sp_skip_bytes / (sp_skip_ms * 1e-3) / 1e9
+            step_bytes = sp_skip_bytes + (R - active_rows) * row_bytes
             roofline = {"bound": "hbm", "kernel": "grpo_fused_kernel (K7)", "achieved": gbps, "peak": HBM_PEAK_GBPS,
                         "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
-                        "traffic": MEASURED_K7_TRAFFIC_BYTES.get((args.workload, args.loss_type)),
-                        "algorithmic_bytes": sp_skip_bytes, "avg_launch_ms": sp_skip_ms,
-                        # the work of the headline step priced as the two-pass kernels' bytes (forward read of every
-                        # row, backward read + write): what the step replaces, not what it moves
-                        "two_pass_equivalent_GBps": (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9}
+                        "traffic": MEASURED_TRAFFIC_BYTES.get(("K7", args.workload, loss_type)),
+                        "algorithmic_bytes": sp_skip_bytes, "avg_launch_ms": sp_skip_ms}
+    # the whole step priced by the bytes its own kernels move (K7's bytes + the forward read of the other rows, or
+    # K1's + K3's): bytes / step time
+    roofline["step_hbm_bytes"] = step_bytes
+    roofline["step_hbm_GBps"] = step_bytes / (ms_per_step * 1e-3) / 1e9
+    roofline["step_hbm_frac"] = roofline["step_hbm_GBps"] / HBM_PEAK_GBPS
 
     result = {
         "metric": "tokens/sec + achieved HBM TB/s (% of peak) for GRPO logprob+loss fwd+bwd",
@@ -608,18 +629,12 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": args.workload, "description": w["desc"], "rows": R, "vocab": V,
-                   "loss_type": args.loss_type, "active_rows": active_rows, "loss": loss_value,
+                   "loss_type": loss_type, "active_rows": active_rows, "loss": loss_value,
                    "path": "single pass over the logits (K7) for the rows with gradient + forward kernel (K1) for the "
                            "log-probs and entropies of the others" if headline_single
                            else "two passes over the logits (K1, K3)"},
         "roofline": roofline,
-        "kernels": dict(kernels, **{
-            "logp_entropy_fwd_kernel (K1)": {"avg_launch_ms": fwd_ms, "algorithmic_bytes": fwd_bytes,
-                                             "achieved_GBps": fwd_gbps, "frac": fwd_gbps / HBM_PEAK_GBPS},
-            "logp_entropy_bwd_kernel (K3)": {"avg_launch_ms": bwd_ms, "algorithmic_bytes": bwd_bytes,
-                                             "achieved_GBps": bwd_gbps, "frac": bwd_gbps / HBM_PEAK_GBPS},
-            "two_pass_step_hbm_GBps": (fwd_bytes + bwd_bytes) / (ms_two_pass * 1e-3) / 1e9,
-        }),
+        "kernels": kernels,
         "two_pass": {"ms_per_step": ms_two_pass, "tokens_per_s": R / (ms_two_pass * 1e-3),
                      "note": "log-prob kernel (K1), [B, T] loss kernel, gradient kernel (K3): two reads and one write "
                              "of the logits-sized data; the path of every configuration the single pass does not take"},
@@ -627,24 +642,91 @@ def main():
             "ms_per_step": single["all_rows_ms"], "tokens_per_s": R / (single["all_rows_ms"] * 1e-3),
             "mask_aware_ms_per_step": single["mask_aware_ms"],
             "mask_aware_tokens_per_s": R / (single["mask_aware_ms"] * 1e-3),
+            "dlogits_rel_l2_vs_two_pass": single["dlogits_rel_l2_vs_two_pass"],
+            "scaled_upstream_ms": single.get("scaled_upstream_ms"),
             "note": "grpo_loss_from_logits: the rows with gradient are read once and their gradient written by the same "
                     "kernel; same loss, log-probs, entropies and dlogits; the log-probs and entropies of the other rows "
                     "come from the forward kernel; mask-aware = those rows are not read at all (what `_compute_loss` "
-                    "does by default)"},
-        "mask_aware": {"ms_per_step": ms_mask_aware, "tokens_per_s": R / (ms_mask_aware * 1e-3),
-                       "note": "forward also skips rows with completion_mask == 0 (their outputs are 0); "
-                               "loss, metrics and dlogits identical"},
+                    "does by default); scaled_upstream_ms = mask-aware step with loss * 1024 before backward"},
     }
-    if args.calibrate_copy:
+    if ms_mask_aware is not None:
+        result["mask_aware"] = {"ms_per_step": ms_mask_aware, "tokens_per_s": R / (ms_mask_aware * 1e-3),
+                                "note": "forward also skips rows with completion_mask == 0 (their outputs are 0); "
+                                        "loss, metrics and dlogits identical"}
+    if args.calibrate_copy and full:
         dst = torch.empty_like(logits)
         for _ in range(3):
             dst.copy_(logits.detach())  # reads and writes R*V*2 bytes each
         torch.cuda.synchronize()
         result["calibration_copy_bytes_each_way"] = fwd_bytes
         del dst
+    return result, shared
+
+
+def _brief(r):
+    """What a secondary entry keeps of a full result."""
+    out = {"workload": r["config"]["workload"], "loss_type": r["config"].get("loss_type"), "value": r["value"],
+           "unit": r["unit"], "ms_per_step": r["ms_per_step"], "path": r["config"].get("path"),
+           "roofline": r["roofline"]}
+    if r.get("single_pass"):
+        out["single_pass_ms_per_step"] = r["single_pass"]["ms_per_step"]
+        out["single_pass_mask_aware_ms_per_step"] = r["single_pass"]["mask_aware_ms_per_step"]
+        out["dlogits_rel_l2_vs_two_pass"] = r["single_pass"]["dlogits_rel_l2_vs_two_pass"]
+    if r.get("two_pass"):
+        out["two_pass_ms_per_step"] = r["two_pass"]["ms_per_step"]
+    if r.get("mask_aware"):
+        out["mask_aware_ms_per_step"] = r["mask_aware"]["ms_per_step"]
+    if "kernels" in r:
+        out["kernels"] = {k: v for k, v in r["kernels"].items() if isinstance(v, dict) and ("frac" in v or "avg_ms" in v)}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS),
+                    help="one workload only (default: grpo_c3 as the headline plus the others as `secondary`)")
+    ap.add_argument("--loss-type", default="dapo", choices=["grpo", "dapo", "dr_grpo", "bnpo"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain device copy of the logits (known bytes) to scale profiler counters by")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; rows are independent, so N GPUs would each run this same "
+                 "kernel on B/N sequences and exchange a handful of scalars per step. Run with --gpus 1.")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the hot path has no CPU fallback.")
+    torch.cuda.set_device(0)
+    secondary_wanted = args.workload is None and not args.no_secondary
+    args.workload = args.workload or "grpo_c3"
+    w = WORKLOADS[args.workload]
+    if w.get("head"):
+        return print(json.dumps(bench_head(args, w)))
+    if w.get("dpo"):
+        return print(json.dumps(bench_dpo(args, w)))
+    result, shared = bench_grpo(args, w, args.loss_type)
+    secondary = []
+    if secondary_wanted:
+        few = argparse.Namespace(**{**vars(args), "steps": max(3, args.steps // 2), "warmup": 2, "no_cpu_baseline": True,
+                                    "calibrate_copy": False})
+        for lt in ("grpo", "dr_grpo"):
+            if lt != args.loss_type:
+                secondary.append(_brief(bench_grpo(few, w, lt, shared, full=False)[0]))
+    del shared
+    torch.cuda.empty_cache()
+    if secondary_wanted:
+        for name in ("grpo_c4", "dpo_c2", "head_c5"):
+            few.workload = name
+            w2 = WORKLOADS[name]
+            r = bench_head(few, w2) if w2.get("head") else bench_dpo(few, w2) if w2.get("dpo") else bench_grpo(few, w2, "dapo")[0]
+            secondary.append(_brief(r))
+            del r
+            torch.cuda.empty_cache()
+        result["secondary"] = secondary
     if not args.no_cpu_baseline:
-        del leaf, logits
-        torch.cuda.empty_cache()
         base = cpu_baseline(w, args.loss_type, repeats=1)
         secs = 32 * 512 / base["value"]
         if secs < 5.0:  # a fast host: the sample grows towards ~10 s of work per run

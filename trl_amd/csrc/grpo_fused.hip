@@ -274,19 +274,21 @@ void launch_fused(const FusedArgs& a, int nvec, unsigned rows, hipStream_t s) {
     }
 }
 
-// data *= *scale over 16-byte vectors, unless the scale is exactly 1 (then nothing is read or written).
+// data *= *scale over 16-byte vectors, unless the scale is exactly 1 (then nothing is read or written).  One vector
+// per lane and 4 KiB per workgroup, consecutive workgroups on consecutive addresses: the access pattern this
+// memory system serves fastest for a read-modify-write sweep.
 template <int DT>
 __global__ __launch_bounds__(256) void scale_unless_one_kernel(u32x4* data, int64_t n_vec, const float* scale) {
     typedef Elem<DT> E;
     const float sc = *scale;
     if (sc == 1.f) return;
-    for (int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x; v < n_vec; v += int64_t(gridDim.x) * 256) {
-        float x[E::EPV];
-        E::unpack(data[v], x);
+    const int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (v >= n_vec) return;
+    float x[E::EPV];
+    E::unpack(__builtin_nontemporal_load(data + v), x);
 #pragma unroll
-        for (int i = 0; i < E::EPV; ++i) x[i] *= sc;
-        data[v] = E::pack(x);
-    }
+    for (int i = 0; i < E::EPV; ++i) x[i] *= sc;
+    __builtin_nontemporal_store(E::pack(x), data + v);
 }
 
 }  // namespace
@@ -302,7 +304,8 @@ extern "C" int trlk_scale_unless_one(void* d_data, int dtype, int64_t n_elems, c
     TRLK_REQUIRE(d_data && d_scale && reinterpret_cast<uintptr_t>(d_data) % 16 == 0, TRLK_ERR_NULL_POINTER,
                  "scale_unless_one: null or misaligned pointer");
     const int64_t n_vec = n_elems / 8;
-    const unsigned grid = unsigned(n_vec < 256 * 8192 ? (n_vec + 255) / 256 : 8192);
+    TRLK_REQUIRE(n_vec <= int64_t(256) * 0x7fffffff, TRLK_ERR_BAD_SHAPE, "scale_unless_one: too many elements");
+    const unsigned grid = unsigned((n_vec + 255) / 256);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == TRLK_BF16)
         hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_BF16>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, d_scale);
