@@ -39,7 +39,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # measured by the run that prints them, and None where no counter run was made for that workload / loss type.
 MEASURED_TRAFFIC_BYTES = {
     ("K3", "grpo_c3", "dapo"): (10116130 + 19461194) * 1024,
-    ("K7", "grpo_c3", "dapo"): (2 * 5058750 + 19481000) * 1024,
+    ("K7", "grpo_c3", "dapo"): (2 * 5064150 + 19488700) * 1024,
     ("head_fwd", "head_c5", "dapo"): (2 * 40600000 + 19497000) * 1024,
 }
 
