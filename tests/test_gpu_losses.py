@@ -618,3 +618,25 @@ def test_multimodal_sub_batches_through_the_logprob_method(amd):
         seen.clear()
         loss = tr._compute_loss(model, inputs)
         assert seen == [(4, 20, 4)] and math.isfinite(float(loss))
+
+
+@pytest.mark.parametrize("single_pass", [False, True])
+def test_trainer_method_raises_on_a_token_id_outside_the_vocabulary(amd, single_pass):
+    """The reference's gather raises (CPU) or device-asserts (GPU) on an id outside [0, V)
+    (trl/trainer/utils.py:507,516); the kernels set a device flag instead, and the mix-in reads it with the copy of
+    the metrics it makes anyway: `_compute_loss` raises IndexError, and the next clean call passes."""
+    B, P, T, V = 2, 1, 4, 64
+    g = torch.Generator().manual_seed(7)
+    leaf = (torch.randn(B, P + T, V, generator=g)).bfloat16().to(DEV).requires_grad_(True)
+    case = dict(loss_type="grpo", beta=0.0, eps_low=0.2, eps_high=0.2)
+    inputs = dict(prompt_ids=torch.zeros(B, P, dtype=torch.long, device=DEV), prompt_mask=torch.ones(B, P, dtype=torch.long, device=DEV),
+                  completion_ids=torch.randint(0, V, (B, T), generator=g).to(DEV),
+                  completion_mask=torch.ones(B, T, dtype=torch.long, device=DEV), advantages=torch.randn(B, generator=g).to(DEV))
+    model = lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None)  # noqa: E731
+    bad = dict(inputs, completion_ids=inputs["completion_ids"].clone())
+    bad["completion_ids"][1, 2] = V + 3
+    tr = _fake_trainer(amd, case, T, skip_masked=True, single_pass=single_pass)
+    with pytest.raises(IndexError):
+        tr._compute_loss(model, bad)
+    assert math.isfinite(float(tr._compute_loss(model, inputs)))
+    amd.check_device_errors()

@@ -53,6 +53,22 @@ def check_device_errors() -> None:
             raise RuntimeError(f"trl_amd: device error flag {bits:#x}")
 
 
+def device_error_bits(device: torch.device) -> Tensor:
+    """The error word of `device` as a one-element fp32 tensor, for callers that are about to copy metrics to the
+    host anyway and append it to that copy (then pass the value to `raise_for_error_bits`): no extra sync."""
+    return _error_flag(device).to(torch.float32)
+
+
+def raise_for_error_bits(bits: float, device: torch.device) -> None:
+    """Raises what `check_device_errors` would for an error word already on the host (and clears the word)."""
+    bits = int(bits)
+    if bits:
+        _error_flag(device).zero_()
+        if bits & _lib.FLAG_INDEX_OUT_OF_RANGE:
+            raise IndexError("trl_amd: an index passed to a log-prob kernel was outside [0, vocab)")
+        raise RuntimeError(f"trl_amd: device error flag {bits:#x}")
+
+
 # --------------------------------------------------------------------------------------------
 # log-prob + entropy (K1 / K3)
 # --------------------------------------------------------------------------------------------

@@ -266,7 +266,10 @@ class DPOLossMixin:
         acc = self.accelerator
         counts = torch.stack([parts[k] for k in ("entropy_sum", "n_tokens", "logits_chosen_sum", "n_chosen_tokens",
                                                   "logits_rejected_sum", "n_rejected_tokens", "correct_tokens")])
-        ent_sum, n_tok, lc, nc, lr, nr, correct = acc.gather_for_metrics(counts.unsqueeze(0)).sum(dim=0).tolist()
+        bits = ops.device_error_bits(counts.device)  # (a token id outside the vocabulary raises here)
+        ent_sum, n_tok, lc, nc, lr, nr, correct, bits = torch.cat(
+            [acc.gather_for_metrics(counts.unsqueeze(0)).sum(dim=0), bits.to(counts.dtype)]).tolist()
+        ops.raise_for_error_bits(bits, counts.device)
         log["entropy"].append(ent_sum / n_tok if n_tok > 0 else 0.0)
         if mode == "train":
             self._total_train_tokens += acc.gather_for_metrics(inputs["attention_mask"].sum()).sum().item()

@@ -643,8 +643,11 @@ class GRPOLossMixin:
         totals = self.accelerator.reduce(torch.cat([sums, clip]), reduction="sum")
         low_min = nanmin(self.accelerator.gather(m[5:6]))
         high_max = nanmax(self.accelerator.gather(m[6:7]))
-        host = torch.cat([totals, low_min.reshape(1), high_max.reshape(1), m[7:8]]).tolist()
-        kl_sum, ent_sum, cnt, clip_cnt, aux_sum, aux_cnt, low, high, region, lmin, hmax, policy_loss = host
+        # (the kernels' error word rides along: a token id outside the vocabulary raises here, as the reference's
+        # gather would, instead of surfacing as a NaN loss)
+        host = torch.cat([totals, low_min.reshape(1), high_max.reshape(1), m[7:8], ops.device_error_bits(m.device)]).tolist()
+        kl_sum, ent_sum, cnt, clip_cnt, aux_sum, aux_cnt, low, high, region, lmin, hmax, policy_loss, bits = host
+        ops.raise_for_error_bits(bits, m.device)
         cnt, clip_cnt, aux_cnt = max(cnt, 1.0), max(clip_cnt, 1.0), max(aux_cnt, 1.0)
         log = self._metrics[mode]
         if bonus:

@@ -145,8 +145,9 @@ class KTOLossMixin:
                  "n_rejected_tokens", "num_chosen", "num_rejected", "chosen_rewards_sum", "rejected_rewards_sum",
                  "chosen_logps_sum", "rejected_logps_sum")
         sums = torch.stack([parts[k].to(torch.float32) for k in names])
-        (ent_sum, n_tok, lc, nc, lr, nr, n_c, n_r, rew_c, rew_r, lp_c, lp_r) = (
-            acc.gather_for_metrics(sums.unsqueeze(0)).nansum(dim=0).tolist())
+        (ent_sum, n_tok, lc, nc, lr, nr, n_c, n_r, rew_c, rew_r, lp_c, lp_r, bits) = torch.cat(
+            [acc.gather_for_metrics(sums.unsqueeze(0)).nansum(dim=0), ops.device_error_bits(sums.device)]).tolist()
+        ops.raise_for_error_bits(bits, sums.device)  # (a token id outside the vocabulary raises here)
         log["entropy"].append(ent_sum / n_tok if n_tok > 0 else 0.0)
         if mode == "train":
             self._total_train_tokens += acc.gather_for_metrics(batch["attention_mask"].sum()).sum().item()

@@ -70,7 +70,9 @@ class RLOOLossMixin:
             log["aux_loss"].append(self.accelerator.gather_for_metrics(aux_loss).mean().item())
         m = completion_mask.to(torch.float32)
         ent = self.accelerator.reduce(torch.stack([(entropies.detach() * m).sum(), m.sum()]), reduction="sum")
-        log["entropy"].append((ent[0] / ent[1].clamp(min=1.0)).item())
+        ent_ratio, bits = torch.cat([(ent[0] / ent[1].clamp(min=1.0)).reshape(1), ops.device_error_bits(ent.device)]).tolist()
+        ops.raise_for_error_bits(bits, ent.device)  # (a token id outside the vocabulary raises here)
+        log["entropy"].append(ent_ratio)
         if self.accelerator.num_processes == 1:
             for name, value in zip(RLOO_METRIC_NAMES, metrics.detach()[: len(RLOO_METRIC_NAMES)].tolist()):
                 log[name].append(value)
