@@ -111,6 +111,21 @@ int trlk_logp_entropy_bwd(const void* d_logits, int dtype, int64_t n_seq, int64_
                           const float* d_g_entropy, void* d_dlogits, int64_t out_rows_per_seq, int64_t out_row_offset,
                           int64_t out_seq_stride, int64_t out_row_stride, trlk_stream_t stream);
 
+/* fp64 logits (the float64 case of selective_log_softmax / entropy_from_logits, trl/trainer/utils.py:506-510,526-560,
+ * which the reference's own unit tests run: tests/test_utils.py:866-905): the same two operations with double
+ * operands, double arithmetic and double outputs.  Same argument meaning as the entry points above; no row
+ * statistics.  Written for exactness (two sweeps per row), not for bandwidth. */
+int trlk_logp_entropy_fwd_f64(const double* d_logits, int64_t n_seq, int64_t rows_per_seq, int64_t vocab,
+                              int64_t seq_stride, int64_t row_stride, const int64_t* d_index, int32_t n_index,
+                              double temperature, const uint8_t* d_row_mask, double* d_out_logp, double* d_out_entropy,
+                              double* d_out_lse, int32_t* d_error_flag, trlk_stream_t stream);
+int trlk_logp_entropy_bwd_f64(const double* d_logits, int64_t n_seq, int64_t rows_per_seq, int64_t vocab,
+                              int64_t seq_stride, int64_t row_stride, const int64_t* d_index, int32_t n_index,
+                              double temperature, const double* d_lse, const double* d_entropy, const double* d_g_logp,
+                              const double* d_g_entropy, double* d_dlogits, int64_t out_rows_per_seq,
+                              int64_t out_row_offset, int64_t out_seq_stride, int64_t out_row_stride,
+                              trlk_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------
  * K2a  group-relative advantages (trl/trainer/grpo_trainer.py:2685-2707, 2730 with nanstd,
  * trl/trainer/utils.py:874-880).  d_rewards fp32 [n] (NaN = unscorable), groups are

@@ -137,7 +137,7 @@ def test_check_raises_python_exceptions():
     with pytest.raises(TypeError):
         import torch
 
-        _lib.dtype_code(torch.float64)
+        _lib.dtype_code(torch.complex64)
 
 
 def test_cpu_tensors_fail_loudly():

@@ -99,6 +99,51 @@ def test_entropy_reference_unit_test_shapes(amd, dtype, shape):
                                    rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("k", [None, 1, 8])
+def test_float64_logits(amd, k):
+    """The float64 case of the reference's unit tests (tests/test_utils.py:866-905, 615-628): double in, double
+    out, against torch's own double `log_softmax` / entropy on the host, forward and gradient (duplicate indices,
+    a strided view, a skipped row and a temperature included)."""
+    g = torch.Generator().manual_seed(64)
+    logits = torch.randn(4, 32, 1024, generator=g, dtype=torch.float64)
+    idx = torch.randint(0, 1024, (4, 32) if k is None else (4, 32, k), generator=g)
+    if k == 8:
+        idx[0, 0, 1] = idx[0, 0, 0]
+    got = amd.selective_log_softmax(logits.to(DEV), idx.to(DEV))
+    want = torch.gather(logits.log_softmax(-1), -1, idx.unsqueeze(-1) if k is None else idx)
+    want = want.squeeze(-1) if k is None else want
+    assert got.dtype == torch.float64 and got.shape == want.shape
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-12, atol=1e-12)
+    ent = amd.entropy_from_logits(logits.to(DEV))
+    lsm = logits.log_softmax(-1)
+    assert ent.dtype == torch.float64
+    torch.testing.assert_close(ent.cpu(), -(lsm.exp() * lsm).sum(-1), rtol=1e-12, atol=1e-12)
+    # gradients through a window of the rows, with a temperature and an entropy term
+    dl = logits.to(DEV).requires_grad_(True)
+    ids3 = idx if k is not None else idx.unsqueeze(-1)
+    win = ids3[:, 3:29]
+    rm = torch.ones(4, 26, dtype=torch.long)
+    rm[2, 5] = 0
+    lp, h = amd.logps_and_entropies(dl, win.to(DEV), 0.8, 3, 26, rm.to(DEV))
+    # (a skipped row's outputs are the constant 0: by contract no gradient arrives there)
+    glp = torch.randn(lp.shape, generator=g, dtype=torch.float64) * rm.double().unsqueeze(-1)
+    gh = torch.randn(h.shape, generator=g, dtype=torch.float64) * rm.double()
+    ((lp * glp.to(DEV)).sum() + (h * gh.to(DEV)).sum()).backward()
+    ol = logits.clone().requires_grad_(True)
+    z = (ol / 0.8)[:, 3:29].log_softmax(-1)
+    keep = rm.double()
+    olp = torch.gather(z, -1, win) * keep.unsqueeze(-1)
+    oh = -(z.exp() * z).sum(-1) * keep
+    ((olp * glp).sum() + (oh * gh).sum()).backward()
+    assert lp.dtype == torch.float64 and float(lp[2, 5].abs().sum()) == 0.0 and float(h[2, 5]) == 0.0
+    torch.testing.assert_close(lp.detach().cpu(), olp.detach(), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(h.detach().cpu(), oh.detach(), rtol=1e-12, atol=1e-12)
+    assert dl.grad.dtype == torch.float64
+    torch.testing.assert_close(dl.grad.cpu(), ol.grad, rtol=1e-10, atol=1e-13)
+    assert float(dl.grad[:, :3].abs().max()) == 0.0 and float(dl.grad[:, 29:].abs().max()) == 0.0
+    amd.check_device_errors()
+
+
 # ------------------------------------------------------------------ benchmark configuration 1 at full size
 def test_config1_full_size_fp32(amd):
     g = torch.Generator().manual_seed(0)

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_double, c_float, c_int32, c_int64, c_size_t, c_void_p
 
 import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 
@@ -38,6 +38,16 @@ SIGNATURES = {
         c_int32,
         [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int32, c_float, c_void_p,
          c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p],
+    ),
+    "trlk_logp_entropy_fwd_f64": (
+        c_int32,
+        [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int32, c_double, c_void_p, c_void_p,
+         c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
+    "trlk_logp_entropy_bwd_f64": (
+        c_int32,
+        [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int32, c_double, c_void_p, c_void_p,
+         c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p],
     ),
     "trlk_group_advantages": (c_int32, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p]),
     "trlk_grpo_workspace_bytes": (c_size_t, [c_int64]),

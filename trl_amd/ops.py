@@ -198,6 +198,93 @@ logp_entropy_fwd.register_autograd(_lpe_backward, setup_context=_lpe_setup)
 logp_entropy_stats_fwd.register_autograd(_lpe_backward, setup_context=_lpe_setup)
 
 
+# ---- the same pair for fp64 logits: double operands, arithmetic and outputs --------------------------------
+@torch.library.custom_op("trl_amd::logp_entropy_fwd_f64", mutates_args=(), device_types="cuda")
+def logp_entropy_fwd_f64(
+    logits: Tensor, index: Tensor, temperature: float, keep_start: int, keep_len: int, row_mask: Optional[Tensor]
+) -> tuple[Tensor, Tensor, Tensor]:
+    """`logp_entropy_fwd` for float64 logits (trl/trainer/utils.py:506-510): returns float64
+    (logp [rows, K], entropy [rows], lse [rows])."""
+    _check_logits3d(logits)
+    if logits.dtype != torch.float64:
+        raise TypeError("logp_entropy_fwd_f64 takes float64 logits")
+    n_seq, _, vocab = logits.shape
+    rows, k, dev = n_seq * keep_len, index.shape[-1], logits.device
+    logp = torch.empty((rows, k), dtype=torch.float64, device=dev)
+    ent = torch.empty((rows,), dtype=torch.float64, device=dev)
+    lse = torch.empty((rows,), dtype=torch.float64, device=dev)
+    if rows == 0:
+        return logp, ent, lse
+    index = index.contiguous()
+    view = logits[:, keep_start : keep_start + keep_len]
+    with torch.cuda.device(dev):
+        check(lib.trlk_logp_entropy_fwd_f64(view.data_ptr(), n_seq, keep_len, vocab, view.stride(0), view.stride(1),
+                                            ptr(index), k, temperature, ptr(row_mask), ptr(logp), ptr(ent), ptr(lse),
+                                            ptr(_error_flag(dev)), current_stream(dev)))
+    if _SYNC_CHECKS:
+        check_device_errors()
+    return logp, ent, lse
+
+
+@logp_entropy_fwd_f64.register_fake
+def _(logits, index, temperature, keep_start, keep_len, row_mask):
+    rows = logits.shape[0] * keep_len
+    f = lambda *s: torch.empty(s, dtype=torch.float64, device=logits.device)  # noqa: E731
+    return f(rows, index.shape[-1]), f(rows), f(rows)
+
+
+@torch.library.custom_op("trl_amd::logp_entropy_bwd_f64", mutates_args=(), device_types="cuda")
+def logp_entropy_bwd_f64(
+    logits: Tensor, index: Tensor, temperature: float, keep_start: int, keep_len: int, lse: Tensor,
+    entropy: Optional[Tensor], g_logp: Optional[Tensor], g_entropy: Optional[Tensor],
+) -> Tensor:
+    """`logp_entropy_bwd` for float64 logits: the float64 gradient of the whole [n_seq, L, V] input."""
+    _check_logits3d(logits)
+    n_seq, length, vocab = logits.shape
+    dlogits = torch.empty((n_seq, length, vocab), dtype=torch.float64, device=logits.device)
+    if dlogits.numel() == 0:
+        return dlogits
+    dev = logits.device
+    view = logits[:, keep_start : keep_start + keep_len]
+    k = index.shape[-1] if g_logp is not None else 0
+    index = index.contiguous()
+    g_logp = None if g_logp is None else g_logp.contiguous().double()
+    g_entropy = None if g_entropy is None else g_entropy.contiguous().double()
+    with torch.cuda.device(dev):
+        check(lib.trlk_logp_entropy_bwd_f64(view.data_ptr(), n_seq, keep_len, vocab, view.stride(0), view.stride(1),
+                                            ptr(index), k, temperature, ptr(lse),
+                                            ptr(entropy if g_entropy is not None else None), ptr(g_logp), ptr(g_entropy),
+                                            ptr(dlogits), length, keep_start, dlogits.stride(0), dlogits.stride(1),
+                                            current_stream(dev)))
+    return dlogits
+
+
+@logp_entropy_bwd_f64.register_fake
+def _(logits, index, temperature, keep_start, keep_len, lse, entropy, g_logp, g_entropy):
+    return torch.empty(logits.shape, dtype=torch.float64, device=logits.device)
+
+
+def _lpe64_backward(ctx, g_logp, g_ent, g_lse):
+    logits, index, lse, ent = ctx.saved_tensors
+    temperature, keep_start, keep_len = ctx.cfg
+    if g_logp is None and g_ent is None:
+        return None, None, None, None, None, None
+    if g_logp is None and index.shape[-1] > 0:
+        g_logp = torch.zeros(index.shape, dtype=torch.float64, device=logits.device)
+    d = logp_entropy_bwd_f64(logits, index, temperature, keep_start, keep_len, lse, ent, g_logp, g_ent)
+    return d, None, None, None, None, None
+
+
+logp_entropy_fwd_f64.register_autograd(_lpe64_backward, setup_context=_lpe_setup)
+
+
+def logp_entropy_forward(logits: Tensor, index: Tensor, temperature: float, keep_start: int, keep_len: int,
+                         row_mask: Optional[Tensor]) -> tuple[Tensor, Tensor, Tensor]:
+    """The forward op for these logits: the double-precision pair for float64, the streaming kernels otherwise."""
+    op = logp_entropy_fwd_f64 if logits.dtype == torch.float64 else logp_entropy_fwd
+    return op(logits, index, temperature, keep_start, keep_len, row_mask)
+
+
 # --------------------------------------------------------------------------------------------
 # group advantages (K2a)
 # --------------------------------------------------------------------------------------------

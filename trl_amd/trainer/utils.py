@@ -59,7 +59,7 @@ def logps_and_entropies(
     rm = None
     if row_mask is not None:
         rm = (row_mask.reshape(-1) != 0).to(torch.uint8).contiguous()
-    logp, ent, _ = ops.logp_entropy_fwd(logits, idx, float(temperature), keep_start, keep_len, rm)
+    logp, ent, _ = ops.logp_entropy_forward(logits, idx, float(temperature), keep_start, keep_len, rm)
     logp = logp.view(n_seq, keep_len) if squeeze else logp.view(n_seq, keep_len, -1)
     return logp, ent.view(n_seq, keep_len)
 
@@ -68,7 +68,7 @@ def selective_log_softmax(logits: Tensor, index: Tensor, out_dtype: torch.dtype 
     """`torch.gather(logits.log_softmax(-1), -1, index)` without materialising the log-softmax
     (reference: trl/trainer/utils.py:479-523).  `index` has shape `(...)` or `(..., K)`.
 
-    The kernel always computes in fp32.  `out_dtype=None` returns the logits dtype as the
+    The kernel computes in fp32 (in fp64 for float64 logits).  `out_dtype=None` returns the logits dtype as the
     reference does (for bf16/fp16 logits the fp32 result is rounded once to that dtype);
     `out_dtype=torch.float32` keeps the unrounded values."""
     squeeze = index.dim() == logits.dim() - 1
@@ -83,10 +83,10 @@ def selective_log_softmax(logits: Tensor, index: Tensor, out_dtype: torch.dtype 
     idx = index.reshape(x.shape[0] * x.shape[1], k)
     if idx.dtype != torch.int64:
         raise RuntimeError(f"gather(): Expected dtype int64 for index, got {idx.dtype}")
-    logp, _, _ = ops.logp_entropy_fwd(x, idx, 1.0, 0, x.shape[1], None)
+    logp, _, _ = ops.logp_entropy_forward(x, idx, 1.0, 0, x.shape[1], None)
     logp = logp.view(index.shape)
     out_dtype = logits.dtype if out_dtype is None else out_dtype
-    return logp if out_dtype == torch.float32 else logp.to(out_dtype)
+    return logp if out_dtype == logp.dtype else logp.to(out_dtype)
 
 
 def entropy_from_logits(logits: Tensor, chunk_size: int = 128, out_dtype: torch.dtype | None = None) -> Tensor:
@@ -95,10 +95,10 @@ def entropy_from_logits(logits: Tensor, chunk_size: int = 128, out_dtype: torch.
     compatibility; the kernel streams each row once and needs no chunking."""
     x = _as_3d(logits)
     idx = torch.empty((x.shape[0] * x.shape[1], 0), dtype=torch.int64, device=logits.device)
-    _, ent, _ = ops.logp_entropy_fwd(x, idx, 1.0, 0, x.shape[1], None)
+    _, ent, _ = ops.logp_entropy_forward(x, idx, 1.0, 0, x.shape[1], None)
     ent = ent.view(logits.shape[:-1])
     out_dtype = logits.dtype if out_dtype is None else out_dtype
-    return ent if out_dtype == torch.float32 else ent.to(out_dtype)
+    return ent if out_dtype == ent.dtype else ent.to(out_dtype)
 
 
 # ----------------------------------------------------------------------------------------------
@@ -176,7 +176,7 @@ def _fp32_head_forward(hidden, weight, targets, temperature, cap, logit_scale, b
             lp, e, l, st = ops.logp_entropy_stats_fwd(z.unsqueeze(0), idx, temperature, 0, r1 - r0, None)
             hit[r0:r1] = st[:, 2]
         else:
-            lp, e, l = ops.logp_entropy_fwd(z.unsqueeze(0), idx, temperature, 0, r1 - r0, None)
+            lp, e, l = ops.logp_entropy_forward(z.unsqueeze(0), idx, temperature, 0, r1 - r0, None)
         logp[r0:r1], ent[r0:r1], lse[r0:r1] = lp.view(-1), e, l
     return (logp, ent, lse, hit) if want_hit else (logp, ent, lse)
 
