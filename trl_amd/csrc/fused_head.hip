@@ -15,11 +15,11 @@
 // epilogue needs no cross-lane traffic; a workgroup keeps 256 tokens and walks over its share of
 // the vocabulary tiles, the logits exist only as accumulators.
 //
-// Backward (K6), per vocabulary chunk: (1) dz = dL/dlogits (bf16), written both as [tokens, chunk]
+// Backward (K6), per vocabulary chunk: (1) dz = dL/dlogits (scaled fp16), written both as [tokens, chunk]
 // and as [chunk, tokens] -- from a recompute of the chunk's logits (same tile loop), or, when the
 // forward was asked to stash its raw products, from one elementwise sweep over that stash;
 // (2) dHidden += dz * W_chunk as an NT product against W^T; (3) dW_chunk = dz^T * hidden as an NT
-// product against hidden^T.  The contraction of (2)/(3) is over a different axis than the
+// product against hidden^T, both on fp16 operands (bf16 inputs are converted while they are transposed).  The contraction of (2)/(3) is over a different axis than the
 // recompute, and with H in the thousands the output tile of a fused kernel cannot stay in
 // registers, so dz goes through a chunk-sized workspace (never the whole [N, V] matrix).
 #include "common.hpp"
@@ -525,10 +525,30 @@ struct HeadArgs {
     const float* stash_in;  // backward: the same buffer, or null (recompute)
     const int32_t* stash_cols;  // backward: stash column of token n (tokens were compacted since the forward), or null
     int64_t ld_stash;
-    uint16_t* dz;        // [N, ldz]   (columns = chunk-local vocabulary index)
-    uint16_t* dzT;       // [chunk rows padded, ldzt]
+    uint16_t* dz;        // [N, ldz]   (columns = chunk-local vocabulary index), fp16, row n scaled by dz_row_scale(g[n])
+    uint16_t* dzT;       // [chunk rows padded, ldzt], fp16, scaled by dz_scale(*g_max)
     int64_t ldz, ldzt;
+    const uint32_t* g_max;  // backward: bit pattern of max |g| over the tokens
 };
+
+// ---- scaled fp16 copies of the backward's operands -----------------------------------------------------------------
+// The two backward products run on fp16 operands whatever the dtype of the problem: d logits rounded to bf16 would
+// carry 8 significant bits into both gradients (relative error 3e-3), fp16 carries 11 (4e-4) at the same matrix-core
+// rate.  fp16 has 5 exponent bits, so every operand is multiplied by a power of two that puts its largest magnitude
+// into [2^13, 2^14) (exact, undone in the products' epilogue): the token-major d logits per token (|dz[n, :]| <=
+// |g[n]| * logit_scale / T), the vocabulary-major copy by the largest |g|, W^T and hidden^T of a bf16 problem by
+// their largest magnitude (bf16 -> fp16 is then exact down to 2^-31 of that maximum).
+__device__ __forceinline__ float pow2_scale(float m) {
+    if (!(m > 0.f) || !(m < INFINITY)) return 1.f;
+    int e;
+    (void)frexpf(m, &e);  // m = f * 2^e with f in [0.5, 1)
+    int k = 14 - e;
+    k = k > 100 ? 100 : (k < -100 ? -100 : k);
+    return ldexpf(1.f, k);
+}
+__device__ __forceinline__ float slot_scale(const uint32_t* slot, float mult) {
+    return slot != nullptr ? pow2_scale(__uint_as_float(*slot) * mult) : 1.f;
+}
 
 // z = logit in natural units after logit_scale, optional soft-capping and temperature.
 __device__ __forceinline__ float head_z(float y, const HeadArgs& a) {
@@ -752,7 +772,6 @@ __global__ void head_merge_kernel(const float* partial, const float* tgt, const 
 template <int DT>
 TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    typedef Elem<DT> E;
     const int n_tb = (a.N + BN - 1) / BN;
     const int n_vt = (a.c1 - a.c0 + BM - 1) / BM;
     int tb, vt;
@@ -769,11 +788,15 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
     // with one scale folded into the exponent; the target's one-hot term is patched afterwards.
     const float zs = a.logit_scale * a.inv_t, zs2 = zs * kLog2e;
     const bool plain = a.softcap <= 0.f && m0 + BM <= a.c1 && a.bias == nullptr;
+    typedef Elem<TRLK_F16> EO;  // storage of both dz copies
+    const float s_all = slot_scale(a.g_max, zs);
+    float to_all[NB];  // token-major scale -> scale of the vocabulary-major copy, per token block
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         const int tok = n0 + acc_col(wn, nb, lane);
         const bool tok_ok = tok < a.N;
-        const float g = tok_ok ? a.g[tok] : 0.f;
+        const float g = tok_ok ? a.g[tok] * pow2_scale(fabsf(a.g[tok]) * zs) : 0.f;  // g carries the token's scale
+        to_all[nb] = tok_ok ? s_all / pow2_scale(fabsf(a.g[tok]) * zs) : 0.f;
         const float lzc = tok_ok ? a.log_z[tok] * kLog2e : INFINITY;  // rows beyond N: exp2(-inf) = 0
         const int64_t tg = tok_ok ? a.targets[tok] : -1;
         const int64_t rel = tg - (m0 + wm * WM);  // target row relative to this wave's rows
@@ -815,8 +838,8 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 uint2 w;
-                w.x = E::pack2(d[q * 4 + 0], d[q * 4 + 1]);
-                w.y = E::pack2(d[q * 4 + 2], d[q * 4 + 3]);
+                w.x = EO::pack2(d[q * 4 + 0], d[q * 4 + 1]);
+                w.y = EO::pack2(d[q * 4 + 2], d[q * 4 + 3]);
                 *reinterpret_cast<uint2*>(smem + acc_col(wn, nb, lane) * kDzLdsRow + acc_row(wm, mb, q * 4, lane) * 2) = w;
             }
 #pragma unroll
@@ -846,11 +869,11 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
             for (int r = 0; r < 16; r += 2) {
-                const float mine0 = acc[mb][nb][r], mine1 = acc[mb][nb][r + 1];
+                const float mine0 = acc[mb][nb][r] * to_all[nb], mine1 = acc[mb][nb][r + 1] * to_all[nb];
                 const float give = odd ? mine0 : mine1;
                 const float got = __builtin_bit_cast(
                     float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, give), 0xB1 /* quad_perm 1,0,3,2 */, 0xf, 0xf, true));
-                const uint32_t w = odd ? E::pack2(got, mine1) : E::pack2(mine0, got);
+                const uint32_t w = odd ? EO::pack2(got, mine1) : EO::pack2(mine0, got);
                 const int vrow = acc_row(wm, mb, r, lane) + odd;
                 *reinterpret_cast<uint32_t*>(smem + vrow * kDzLdsRow + tcol) = w;
             }
@@ -876,9 +899,9 @@ constexpr int kSdzRows = 64, kSdzTokens = TRLK_SDZ_TOKENS, kSdzLdsRow = kSdzRows
 constexpr int kSdzLanesPerRow = kSdzTokens / 4, kSdzPairsPerWave = 64 / kSdzLanesPerRow;
 static_assert(kSdzTokens == 256 || kSdzTokens == 128, "a row of the tile is one wave or half a wave wide");
 // COLS: the tokens were compacted since the forward, a.stash_cols maps them to their stash columns.
-template <int DT, bool COLS>
+template <bool COLS>
 __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
-    typedef Elem<DT> E;
+    typedef Elem<TRLK_F16> E;  // both dz copies are scaled fp16
     __shared__ __attribute__((aligned(16))) char lds[kSdzTokens * kSdzLdsRow];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // consecutive workgroups take consecutive row groups of one token block: their 128-byte pieces of
@@ -887,16 +910,18 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
     const int rows = a.c1 - a.c0;
     const float zs = a.logit_scale * a.inv_t, zs2 = zs * kLog2e;
     const bool plain = a.softcap <= 0.f && a.bias == nullptr;
-    float g[4], lzc[4];
+    float g[4], lzc[4], to_tok[4];  // g carries the scale of the vocabulary-major copy; to_tok: that scale -> the token's own
     int64_t tg[4];
     int col[4];
     const int tl0 = (lane % kSdzLanesPerRow) * 4, sub = lane / kSdzLanesPerRow;  // first token of the lane, row pair
+    const float s_all = slot_scale(a.g_max, zs);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int tok = n0 + tl0 + j;
         const bool ok = tok < a.N;
         col[j] = (COLS && ok) ? a.stash_cols[tok] : -1;
-        g[j] = ok ? a.g[tok] : 0.f;
+        g[j] = ok ? a.g[tok] * s_all : 0.f;
+        to_tok[j] = ok ? pow2_scale(fabsf(a.g[tok]) * zs) / s_all : 0.f;
         lzc[j] = ok ? a.log_z[tok] * kLog2e : INFINITY;
         tg[j] = ok ? a.targets[tok] - a.c0 : -1;  // chunk-local target row
     }
@@ -963,7 +988,7 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            *reinterpret_cast<uint32_t*>(lds + (tl0 + j) * kSdzLdsRow + rl * 2) = E::pack2(d[0][j], d[1][j]);
+            *reinterpret_cast<uint32_t*>(lds + (tl0 + j) * kSdzLdsRow + rl * 2) = E::pack2(d[0][j] * to_tok[j], d[1][j] * to_tok[j]);
     }
     __syncthreads();
     constexpr int kPieces = kSdzRows / 8;  // 16-byte pieces per staged token row
@@ -982,6 +1007,9 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
 //   MODE 0: store to `out_lp` in the storage dtype.
 //   MODE 1: fp32 accumulate into `out_f32` (first = overwrite).
 //   MODE 2: like 1 but the sum is rounded into `out_lp` instead of being written back (last chunk).
+//   The accumulators are multiplied by 1 / (scale of A * scale of B) first: the scales are powers of two derived from
+//   the maxima in `max_a` (times `mult_a`) and `max_b` (null = 1), and, when `g_rows` is given, row m of A carries its
+//   own scale pow2_scale(|g_rows[m]| * mult_a) instead of the common one.
 struct GemmArgs {
     Operand A, B;
     int M, N, K;
@@ -990,11 +1018,16 @@ struct GemmArgs {
     uint16_t* out_lp;
     int64_t ld_lp;
     int first;
+    const uint32_t* max_a;
+    const uint32_t* max_b;
+    const float* g_rows;
+    float mult_a;
 };
 
-template <int DT, int MODE>
+// DT: dtype of the operands (the matrix-core instruction), ODT: storage dtype of `out_lp`.
+template <int DT, int MODE, int ODT>
 __device__ __forceinline__ void gemm_nt_body(const GemmArgs& a, int block, char* smem) {
-    typedef Elem<DT> E;
+    typedef Elem<ODT> E;
     const int n_mt = (a.M + BM - 1) / BM, n_nt = (a.N + BN - 1) / BN;
     int tm, tn;
     xcd_patch(block, n_mt, n_nt, tm, tn);
@@ -1004,11 +1037,19 @@ __device__ __forceinline__ void gemm_nt_body(const GemmArgs& a, int block, char*
     const int m0 = tm * BM, n0 = tn * BN;
     f32x16 acc[MB][NB];
     gemm_tile_nt<DT, TRLK_HEAD_BK_GEMM>(a.A, m0, a.B, n0, a.K, acc, smem);
+    const float inv_b = 1.f / slot_scale(a.max_b, 1.f);
+    const float inv_common = inv_b / slot_scale(a.max_a, a.mult_a);
     // The running sum of a block is read as a whole before any of the block is written: with a load
     // and a store of the same array per element the compiler keeps them in program order, one memory
     // latency per element (67 us per tile instead of a few).
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+    for (int mb = 0; mb < MB; ++mb) {
+        float inv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = m0 + acc_row(wm, mb, r, lane);
+            inv[r] = (a.g_rows != nullptr && row < a.M) ? inv_b / pow2_scale(fabsf(a.g_rows[row]) * a.mult_a) : inv_common;
+        }
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             const int col = n0 + acc_col(wn, nb, lane);
@@ -1023,42 +1064,84 @@ __device__ __forceinline__ void gemm_nt_body(const GemmArgs& a, int block, char*
             for (int r = 0; r < 16; ++r) {
                 const int row = m0 + acc_row(wm, mb, r, lane);
                 if (row >= a.M) continue;
-                const float v = acc[mb][nb][r] + prev[r];
+                const float v = fmaf(acc[mb][nb][r], inv[r], prev[r]);
                 if (MODE == 1)
                     a.out_f32[int64_t(row) * a.ld_f32 + col] = v;
                 else
                     E::store1(a.out_lp + int64_t(row) * a.ld_lp + col, v);
             }
         }
-}
-
-template <int DT, int MODE>
-TRLK_HEAD_KERNEL void gemm_nt_kernel(GemmArgs a) {
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    gemm_nt_body<DT, MODE>(a, blockIdx.x, smem);
+    }
 }
 
 // Two independent products in one launch: workgroups [0, grid_a) take `a` (epilogue MODE_A), the rest take `b`
 // (epilogue 0).  When the tile count of one product is not a multiple of the CU count, the other product's
 // tiles fill the CUs its last round leaves idle.  grid_a is a multiple of 8 (the XCD mapping of `b` is kept).
-template <int DT, int MODE_A>
+template <int MODE_A, int ODT>
 TRLK_HEAD_KERNEL void gemm_nt_pair_kernel(GemmArgs a, int grid_a, GemmArgs b) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     if (int(blockIdx.x) < grid_a)
-        gemm_nt_body<DT, MODE_A>(a, blockIdx.x, smem);
+        gemm_nt_body<TRLK_F16, MODE_A, ODT>(a, blockIdx.x, smem);
     else
-        gemm_nt_body<DT, 0>(b, int(blockIdx.x) - grid_a, smem);
+        gemm_nt_body<TRLK_F16, 0, ODT>(b, int(blockIdx.x) - grid_a, smem);
+}
+
+// Largest magnitude of a bf16 [R, C8 * 8] matrix (row stride ld) as the bit pattern of that float, through an atomic
+// maximum on `out` (non-negative floats order like unsigned integers; the caller clears `out`).
+__global__ __launch_bounds__(256) void maxabs_bf16_kernel(const uint16_t* in, int64_t ld, int R, int C8, uint32_t* out) {
+    uint32_t m = 0;
+    auto take = [&](u32x4 q) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t lo = (q[i] << 16) & 0x7fff0000u, hi = q[i] & 0x7fff0000u;
+            m = max(m, max(lo, hi));
+        }
+    };
+    if (ld == int64_t(C8) * 8) {  // dense rows: one flat sweep, four loads in flight per lane
+        const u32x4* p = reinterpret_cast<const u32x4*>(in);
+        const int64_t n = int64_t(R) * C8, step = int64_t(gridDim.x) * 256;
+        int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x;
+        for (; v + 3 * step < n; v += 4 * step) {
+            const u32x4 q0 = __builtin_nontemporal_load(p + v), q1 = __builtin_nontemporal_load(p + v + step),
+                        q2 = __builtin_nontemporal_load(p + v + 2 * step), q3 = __builtin_nontemporal_load(p + v + 3 * step);
+            take(q0), take(q1), take(q2), take(q3);
+        }
+        for (; v < n; v += step) take(__builtin_nontemporal_load(p + v));
+    } else {
+        for (int r = blockIdx.x; r < R; r += gridDim.x) {
+            const u32x4* row = reinterpret_cast<const u32x4*>(in + int64_t(r) * ld);
+            for (int c = threadIdx.x; c < C8; c += 256) take(row[c]);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = max(m, uint32_t(__shfl_xor(int(m), off, 64)));
+    if ((threadIdx.x & 63) == 0 && m != 0) atomicMax(out, m);
+}
+// The same for an fp32 vector.
+__global__ __launch_bounds__(256) void maxabs_f32_kernel(const float* in, int64_t n, uint32_t* out) {
+    uint32_t m = 0;
+    for (int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x; i < n; i += int64_t(gridDim.x) * 256)
+        m = max(m, __float_as_uint(in[i]) & 0x7fffffffu);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = max(m, uint32_t(__shfl_xor(int(m), off, 64)));
+    if ((threadIdx.x & 63) == 0 && m != 0) atomicMax(out, m);
 }
 
 // [R, C] (ld) -> [C, ldo] with columns >= R zero-filled up to `fill`: 64 x 64 tiles through LDS.
+// TO_F16: the input is bf16 and the output fp16, multiplied by the power of two that `in_max` (the input's largest
+// magnitude) asks for.
+template <bool TO_F16>
 __global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* in, int64_t ld, int R, int C, uint16_t* out,
-                                                          int64_t ldo, int64_t fill) {
+                                                          int64_t ldo, int64_t fill, const uint32_t* in_max) {
     __shared__ uint16_t tile[64][66];
     const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const float sc = TO_F16 ? slot_scale(in_max, 1.f) : 1.f;
     for (int i = ty; i < 64; i += 4) {
         const int r = r0 + i, c = c0 + tx;
-        tile[i][tx] = (r < R && c < C) ? in[int64_t(r) * ld + c] : uint16_t(0);
+        uint16_t v = (r < R && c < C) ? in[int64_t(r) * ld + c] : uint16_t(0);
+        if (TO_F16) v = __builtin_bit_cast(uint16_t, _Float16(Elem<TRLK_BF16>::to_float(v) * sc));
+        tile[i][tx] = v;
     }
     __syncthreads();
     for (int i = ty; i < 64; i += 4) {
@@ -1070,9 +1153,9 @@ __global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* in, in
 int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
 // d bias[v] = sum over tokens of dz[token, v]: row sums of the transposed dz copy (padding columns are zero).
-template <int DT>
-__global__ __launch_bounds__(256) void dz_row_sum_kernel(const uint16_t* dzT, int64_t ld, int n_cols8, float* out) {
-    typedef Elem<DT> E;
+__global__ __launch_bounds__(256) void dz_row_sum_kernel(const uint16_t* dzT, int64_t ld, int n_cols8, float* out,
+                                                         const uint32_t* g_max, float zs) {
+    typedef Elem<TRLK_F16> E;
     const uint16_t* row = dzT + int64_t(blockIdx.x) * ld;
     float acc = 0.f;
     for (int c = threadIdx.x; c < n_cols8; c += 256) {
@@ -1087,7 +1170,7 @@ __global__ __launch_bounds__(256) void dz_row_sum_kernel(const uint16_t* dzT, in
     __shared__ float part[4];
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
     __syncthreads();
-    if (threadIdx.x == 0) out[blockIdx.x] = part[0] + part[1] + part[2] + part[3];
+    if (threadIdx.x == 0) out[blockIdx.x] = (part[0] + part[1] + part[2] + part[3]) / slot_scale(g_max, zs);
 }
 
 // Row strides of the workspace matrices carry 128 extra bytes: their padded extents are multiples
@@ -1097,7 +1180,8 @@ constexpr int64_t kLdSkew = 64;
 struct BwdLayout {
     int64_t vpad, npad, cpad;    // padded extents (zero-filled)
     int64_t ld_v, ld_n, ld_c;    // row strides of [*, vpad], [*, npad], [*, cpad] matrices
-    size_t off_wt, off_ht, off_dz, off_dzt, off_dh, total;
+    size_t off_wt, off_ht, off_dz, off_dzt, off_dh, off_max, total;
+    int64_t n_chunks;
 };
 BwdLayout bwd_layout(int64_t N, int64_t V, int64_t H, int64_t chunk) {
     BwdLayout l;
@@ -1118,6 +1202,8 @@ BwdLayout bwd_layout(int64_t N, int64_t V, int64_t H, int64_t chunk) {
     l.off_dz = take(size_t(N) * l.ld_c * 2);
     l.off_dzt = take(size_t(l.cpad) * l.ld_n * 2);
     l.off_dh = take(size_t(N) * H * 4);
+    l.n_chunks = (V + l.cpad - 1) / l.cpad;
+    l.off_max = take(size_t(2 + l.n_chunks) * 4);  // largest magnitudes: g, hidden, each chunk of W
     l.total = o;
     return l;
 }
@@ -1323,9 +1409,24 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     uint16_t* dz = reinterpret_cast<uint16_t*>(ws + l.off_dz);    // [N, cpad], row stride ld_c
     uint16_t* dzt = reinterpret_cast<uint16_t*>(ws + l.off_dzt);  // [cpad, npad], row stride ld_n
     float* dh = reinterpret_cast<float*>(ws + l.off_dh);          // [N, H]
+    uint32_t* maxima = reinterpret_cast<uint32_t*>(ws + l.off_max);  // [0] g, [1] hidden, [2 + i] chunk i of W
     const int H = int(hidden_size), N = int(n_tokens), V = int(vocab);
-    hipLaunchKernelGGL(transpose16_kernel, dim3((H + 63) / 64, unsigned((l.npad + 63) / 64)), dim3(256), 0, s,
-                       static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.ld_n, l.npad);
+    const bool from_bf16 = dtype == TRLK_BF16;  // the products' operands are fp16: bf16 inputs are converted on the way
+    const uint32_t* max_g = maxima;
+    const uint32_t* max_h = from_bf16 ? maxima + 1 : nullptr;
+    hipLaunchKernelGGL(head_fill_kernel, dim3(unsigned((2 + l.n_chunks + 255) / 256)), dim3(256), 0, s,
+                       reinterpret_cast<float*>(maxima), 2 + l.n_chunks, 0.f);
+    hipLaunchKernelGGL(maxabs_f32_kernel, dim3(unsigned(N < 65536 ? (N + 255) / 256 : 256)), dim3(256), 0, s, d_g_logp,
+                       n_tokens, maxima);
+    if (from_bf16) {
+        hipLaunchKernelGGL(maxabs_bf16_kernel, dim3(unsigned(N < 2048 ? N : 2048)), dim3(256), 0, s,
+                           static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H / 8, maxima + 1);
+        hipLaunchKernelGGL(transpose16_kernel<true>, dim3((H + 63) / 64, unsigned((l.npad + 63) / 64)), dim3(256), 0, s,
+                           static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.ld_n, l.npad, max_h);
+    } else {
+        hipLaunchKernelGGL(transpose16_kernel<false>, dim3((H + 63) / 64, unsigned((l.npad + 63) / 64)), dim3(256), 0, s,
+                           static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.ld_n, l.npad, max_h);
+    }
     if (int rc = launch_status("fused_head_bwd (hidden^T)")) return rc;
 
     HeadArgs a{};
@@ -1350,6 +1451,8 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     a.dzT = dzt;
     a.ldz = l.ld_c;
     a.ldzt = l.ld_n;
+    a.g_max = max_g;
+    const float zs = logit_scale / temperature;  // |dz[n, v]| <= |g[n]| * zs
     const int n_tb = int((n_tokens + BN - 1) / BN);
     const int n_ht = (H + BN - 1) / BN;
     for (int64_t c0 = 0; c0 < vocab; c0 += chunk) {
@@ -1362,14 +1465,10 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         int rc;
         if (d_stash != nullptr) {
             const dim3 grid(unsigned(kpad / kSdzRows), unsigned(l.npad / kSdzTokens));
-            if (dtype == TRLK_BF16 && d_stash_cols)
-                hipLaunchKernelGGL((head_dz_from_stash_kernel<TRLK_BF16, true>), grid, dim3(256), 0, s, a);
-            else if (dtype == TRLK_BF16)
-                hipLaunchKernelGGL((head_dz_from_stash_kernel<TRLK_BF16, false>), grid, dim3(256), 0, s, a);
-            else if (d_stash_cols)
-                hipLaunchKernelGGL((head_dz_from_stash_kernel<TRLK_F16, true>), grid, dim3(256), 0, s, a);
+            if (d_stash_cols)
+                hipLaunchKernelGGL(head_dz_from_stash_kernel<true>, grid, dim3(256), 0, s, a);
             else
-                hipLaunchKernelGGL((head_dz_from_stash_kernel<TRLK_F16, false>), grid, dim3(256), 0, s, a);
+                hipLaunchKernelGGL(head_dz_from_stash_kernel<false>, grid, dim3(256), 0, s, a);
             rc = launch_status("fused_head_bwd (dz from the stash)");
         } else {
             rc = dtype == TRLK_BF16
@@ -1378,20 +1477,25 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         }
         if (rc) return rc;
         if (d_out_dbias) {
-            if (dtype == TRLK_BF16)
-                hipLaunchKernelGGL(dz_row_sum_kernel<TRLK_BF16>, dim3(rows), dim3(256), 0, s, dzt, l.ld_n, int(l.npad / 8),
-                                   d_out_dbias + c0);
-            else
-                hipLaunchKernelGGL(dz_row_sum_kernel<TRLK_F16>, dim3(rows), dim3(256), 0, s, dzt, l.ld_n, int(l.npad / 8),
-                                   d_out_dbias + c0);
+            hipLaunchKernelGGL(dz_row_sum_kernel, dim3(rows), dim3(256), 0, s, dzt, l.ld_n, int(l.npad / 8), d_out_dbias + c0,
+                               max_g, zs);
             if (int rc2 = launch_status("fused_head_bwd (dBias)")) return rc2;
         }
         const bool first = c0 == 0, last = c1 == vocab;
         // W_chunk^T [H, kpad] (columns beyond the chunk's rows are zero): the chunk's own transposed copy keeps the
         // row stride of this operand as short as that of the other three
-        hipLaunchKernelGGL(transpose16_kernel, dim3((H + 63) / 64, unsigned((kpad + 63) / 64)), dim3(256), 0, s,
-                           static_cast<const uint16_t*>(d_weight) + c0 * weight_stride, weight_stride, rows, H, wt, l.ld_c,
-                           int64_t(kpad));
+        const uint16_t* w_chunk = static_cast<const uint16_t*>(d_weight) + c0 * weight_stride;
+        const uint32_t* max_w = from_bf16 ? maxima + 2 + c0 / chunk : nullptr;
+        const dim3 tgrid((H + 63) / 64, unsigned((kpad + 63) / 64));
+        if (from_bf16) {
+            hipLaunchKernelGGL(maxabs_bf16_kernel, dim3(unsigned(rows < 2048 ? rows : 2048)), dim3(256), 0, s, w_chunk,
+                               weight_stride, rows, H / 8, maxima + 2 + c0 / chunk);
+            hipLaunchKernelGGL(transpose16_kernel<true>, tgrid, dim3(256), 0, s, w_chunk, weight_stride, rows, H, wt, l.ld_c,
+                               int64_t(kpad), max_w);
+        } else {
+            hipLaunchKernelGGL(transpose16_kernel<false>, tgrid, dim3(256), 0, s, w_chunk, weight_stride, rows, H, wt, l.ld_c,
+                               int64_t(kpad), max_w);
+        }
         if (int rc2 = launch_status("fused_head_bwd (W^T)")) return rc2;
         // dHidden[N, H] += dz[N, chunk] * (W_chunk^T[H, chunk])^T
         GemmArgs gh{};
@@ -1405,6 +1509,10 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         gh.out_lp = static_cast<uint16_t*>(d_out_dhidden);
         gh.ld_lp = H;
         gh.first = first;
+        gh.max_a = nullptr;  // the rows of dz carry their own scales
+        gh.g_rows = d_g_logp;
+        gh.mult_a = zs;
+        gh.max_b = max_w;
         const int ghgrid = xcd_patch_grid(n_tb, n_ht);
         // dW[chunk, H] = dz^T[chunk, N] * (hidden^T[H, N])^T
         GemmArgs gw{};
@@ -1416,15 +1524,19 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         gw.out_lp = static_cast<uint16_t*>(d_out_dweight) + c0 * hidden_size;
         gw.ld_lp = hidden_size;
         gw.first = 1;
+        gw.max_a = max_g;
+        gw.g_rows = nullptr;
+        gw.mult_a = zs;
+        gw.max_b = max_h;
         // both products of the chunk in one launch (dHidden's workgroups first)
         const int gwgrid = xcd_patch_grid(n_vt, n_ht);
         const char* what = "fused_head_bwd (dHidden, dW)";
         if (last)
-            rc = dtype == TRLK_BF16 ? launch_head_pair(gemm_nt_pair_kernel<TRLK_BF16, 2>, ghgrid, gh, gwgrid, gw, s, what)
-                                    : launch_head_pair(gemm_nt_pair_kernel<TRLK_F16, 2>, ghgrid, gh, gwgrid, gw, s, what);
+            rc = from_bf16 ? launch_head_pair(gemm_nt_pair_kernel<2, TRLK_BF16>, ghgrid, gh, gwgrid, gw, s, what)
+                           : launch_head_pair(gemm_nt_pair_kernel<2, TRLK_F16>, ghgrid, gh, gwgrid, gw, s, what);
         else
-            rc = dtype == TRLK_BF16 ? launch_head_pair(gemm_nt_pair_kernel<TRLK_BF16, 1>, ghgrid, gh, gwgrid, gw, s, what)
-                                    : launch_head_pair(gemm_nt_pair_kernel<TRLK_F16, 1>, ghgrid, gh, gwgrid, gw, s, what);
+            rc = from_bf16 ? launch_head_pair(gemm_nt_pair_kernel<1, TRLK_BF16>, ghgrid, gh, gwgrid, gw, s, what)
+                           : launch_head_pair(gemm_nt_pair_kernel<1, TRLK_F16>, ghgrid, gh, gwgrid, gw, s, what);
         if (rc) return rc;
     }
     return TRLK_OK;
