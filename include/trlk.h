@@ -310,6 +310,22 @@ int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, const int64_
                         void* d_out_dweight, float* d_out_dbias, void* d_workspace, size_t workspace_bytes,
                         trlk_stream_t stream);
 
+/* fp32 operands of the fused head (the dtype of the reference's own unit test of _ChunkedLogProbFunction,
+ * tests/test_utils.py:1161-1232; the reference runs `torch.mm(last_hidden, w_chunk.t())` in the operands'
+ * dtype and the two backward products in fp32, trl/trainer/utils.py:1327-1328,1421-1422).  The matrix cores take 16-bit operands, so an
+ * fp32 matrix is split into three bf16 pieces (24 significant bits in all, fp32's exponent range) laid out along
+ * the contraction axis: trlk_split_bf16x3 turns fp32 [rows, cols] into bf16 [rows, 6 * cpad] (cpad = cols rounded
+ * up to 8, padding zero-filled; side 0 for the left operand of an NT product, 1 for the right one), and an NT
+ * product of a side-0 and a side-1 matrix over the 6 * cpad columns is the fp32 product to fp32 rounding.  The
+ * forward runs trlk_fused_head_fwd on such pieces (hidden_size = 6 * cpad); trlk_gemm_nt is the plain product
+ * C[m, n] (+)= A[m, k] * B[n, k]^T (16-bit operands with k contiguous, fp32 output) for the backward's logits
+ * recompute and its two gradient products on pieces of d logits.
+ */
+int trlk_split_bf16x3(const float* d_in, int64_t rows, int64_t cols, int64_t ld_in, int side, void* d_out,
+                      int64_t ld_out, trlk_stream_t stream);
+int trlk_gemm_nt(const void* d_a, int64_t lda, const void* d_b, int64_t ldb, int dtype, int64_t m, int64_t n,
+                 int64_t k, float* d_out, int64_t ldo, int accumulate, trlk_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------
  * K7  GRPO loss gradient straight from the logits: one read and one write of the logits-sized
  * data instead of K1 + K3's two reads and one write.  Stands in for the whole chain

@@ -123,6 +123,18 @@ def test_host_side_argument_validation():
                                    0, None, 0, None, fake16, fake16, None, fake16, 1 << 40, None) == -5  # chunk_size
     assert lib.trlk_fused_head_bwd(fake16, fake16, fake, _lib.BF16, 300, 1000, 64, 64, 64, 1.0, 0.0, 1.0, None, fake, fake,
                                    256, None, 0, fake16, fake16, fake16, None, fake16, 1 << 40, None) == -1  # columns, no stash
+    # fp32 operands as bf16 pieces, and the plain product on them: side, strides, contraction length, dtype, alignment
+    assert lib.trlk_split_bf16x3(fake16, 4, 10, 10, 2, fake16, 96, None) == -5 and "side" in _lib.last_error()
+    assert lib.trlk_split_bf16x3(fake16, 4, 10, 10, 0, fake16, 60, None) == -4  # 6 * 16 columns are needed
+    assert lib.trlk_split_bf16x3(fake16, 4, 10, 8, 0, fake16, 96, None) == -4
+    assert lib.trlk_split_bf16x3(None, 4, 10, 10, 0, fake16, 96, None) == -1
+    assert lib.trlk_split_bf16x3(None, 0, 10, 10, 0, None, 96, None) == 0
+
+    def gemm(a=fake16, lda=64, ldb=64, dtype=_lib.BF16, k=64, ldo=16):
+        return lib.trlk_gemm_nt(a, lda, fake16, ldb, dtype, 8, 16, k, fake16, ldo, 0, None)
+
+    assert gemm(dtype=_lib.F32) == -3 and gemm(k=60) == -4 and gemm(lda=56) == -4 and gemm(ldo=8) == -4
+    assert gemm(a=fake16 + 2) == -4 and gemm(a=None) == -1 and gemm(k=0) == -2
     # an empty problem is a successful no-op
     assert lib.trlk_logp_entropy_fwd(None, _lib.F32, 0, 4, 8, 32, 8, None, 1, 1.0, None, None, None, None, None, None, None) == 0
     assert _lib.last_error() == ""

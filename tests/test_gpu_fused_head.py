@@ -346,12 +346,63 @@ def test_fp32_operands_blocks_bias_and_ragged_shapes(amd, monkeypatch):
     rent = -(lp_all.exp() * lp_all).sum(-1)
     (rlp * gout).sum().backward()
     dh, dw, db = (x.to(DEV).requires_grad_(True) for x in (hidden, weight, bias))
-    lp, ent = amd._ChunkedLogProbFunction.apply(dh, dw, labels.to(DEV), 0.8, 64, 5.0, 0.5, db)
-    (lp * gout.to(DEV)).sum().backward()
+
+    def no_library_product(*args, **kwargs):
+        raise AssertionError("the fp32 head must not call the GEMM library")
+
+    with monkeypatch.context() as mp:  # every product of the operator comes from this library's matrix-core kernels
+        for name in ("matmul", "mm", "addmm", "bmm", "einsum"):
+            mp.setattr(torch, name, no_library_product)
+        for name in ("__matmul__", "matmul", "mm", "addmm_", "addmm"):
+            mp.setattr(torch.Tensor, name, no_library_product)
+        lp, ent = amd._ChunkedLogProbFunction.apply(dh, dw, labels.to(DEV), 0.8, 64, 5.0, 0.5, db)
+        (lp * gout.to(DEV)).sum().backward()
     torch.testing.assert_close(lp.detach().cpu(), rlp.detach(), atol=1e-5, rtol=1e-5)
     torch.testing.assert_close(ent.cpu(), rent.detach(), atol=1e-5, rtol=1e-5)
     for got, want in ((dh, rh), (dw, rw), (db, rb)):
         torch.testing.assert_close(got.grad.cpu(), want.grad, atol=2e-5, rtol=1e-4)
+
+
+def test_bf16_pieces_give_the_fp32_product(amd):
+    """`split_bf16x3`: the three pieces add up to the fp32 value (to 2^-24), padding columns are zero, and
+    `gemm_nt` of a left-side and a right-side split equals the float64 product of the fp32 matrices to fp32 rounding
+    -- on values spread over 12 orders of magnitude, ragged sizes, with and without accumulation."""
+    from trl_amd import ops
+
+    g = torch.Generator().manual_seed(5)
+    m, n, k = 300, 517, 203
+    a = (torch.randn(m, k, generator=g) * torch.exp(4 * torch.randn(m, k, generator=g))).to(DEV)
+    b = (torch.randn(n, k, generator=g) * torch.exp(4 * torch.randn(n, k, generator=g))).to(DEV)
+    kp = (k + 7) // 8 * 8
+    for side, x in ((0, a), (1, b)):
+        p = ops.split_bf16x3(x, side).float().view(x.shape[0], 6, kp)
+        assert float(p[:, :, k:].abs().max()) == 0.0
+        slots = {0: (2, 1, 0, 1, 0, 0), 1: (0, 1, 2, 0, 1, 0)}[side]
+        first = {piece: slots.index(piece) for piece in (0, 1, 2)}
+        total = p[:, first[0], :k].double() + p[:, first[1], :k].double() + p[:, first[2], :k].double()
+        assert float(((total - x.double()).abs() / x.double().abs().clamp(min=1e-300)).max()) <= 2.0**-23
+        for sl, piece in enumerate(slots):
+            assert torch.equal(p[:, sl], p[:, first[piece]])
+        assert torch.equal(p[:, first[0], :k], x.bfloat16().float())
+    want = a.double() @ b.double().t()
+    scale = a.double().abs() @ b.double().abs().t()  # the size of the terms that were added
+    got = ops.gemm_nt(ops.split_bf16x3(a, 0), ops.split_bf16x3(b, 1))
+    err = (got.double() - want).abs() / scale
+    lib_err = ((a @ b.t()).double() - want).abs() / scale  # the GEMM library's fp32 product of the same matrices
+    print(f"error / sum of |terms|: pieces max {float(err.max()):.2e} rms {float(err.pow(2).mean().sqrt()):.2e}; "
+          f"library fp32 max {float(lib_err.max()):.2e} rms {float(lib_err.pow(2).mean().sqrt()):.2e}")
+    assert float(err.max()) < 2e-6 and float(err.pow(2).mean().sqrt()) < 2e-7
+    assert float(err.pow(2).mean().sqrt()) <= float(lib_err.pow(2).mean().sqrt())  # measured: about half
+    twice = ops.gemm_nt(ops.split_bf16x3(a, 0), ops.split_bf16x3(b, 1), out=got.clone(), accumulate=True)
+    torch.testing.assert_close(twice, 2 * got, rtol=1e-6, atol=0)
+    # plain 16-bit operands: exact products, fp32 accumulation
+    for dt in (torch.bfloat16, torch.float16):
+        a16, b16 = torch.randn(70, 72, generator=g).to(dt).to(DEV), torch.randn(33, 72, generator=g).to(dt).to(DEV)
+        torch.testing.assert_close(ops.gemm_nt(a16, b16), a16.float() @ b16.float().t(), rtol=1e-5, atol=1e-5)
+    with pytest.raises(ValueError):
+        ops.gemm_nt(a16, b16[:, :64])
+    with pytest.raises(ValueError):
+        ops.gemm_nt(a16[:, :68], b16[:, :68])  # K must be a multiple of 8
 
 
 def test_fp64_operands_are_rejected_loudly(amd):

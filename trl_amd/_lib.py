@@ -75,6 +75,11 @@ SIGNATURES = {
          c_void_p, c_void_p],
     ),
     "trlk_scale_unless_one": (c_int32, [c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
+    "trlk_split_bf16x3": (c_int32, [c_void_p, c_int64, c_int64, c_int64, c_int32, c_void_p, c_int64, c_void_p]),
+    "trlk_gemm_nt": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_int64, c_int32, c_int64, c_int64, c_int64, c_void_p, c_int64, c_int32, c_void_p],
+    ),
     "trlk_dpo_loss": (
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float, c_void_p, c_void_p, c_void_p, c_void_p,

@@ -1086,6 +1086,44 @@ TRLK_HEAD_KERNEL void gemm_nt_pair_kernel(GemmArgs a, int grid_a, GemmArgs b) {
         gemm_nt_body<TRLK_F16, 0, ODT>(b, int(blockIdx.x) - grid_a, smem);
 }
 
+// A single product (epilogue 1: fp32 output, overwritten or accumulated into).
+template <int DT>
+TRLK_HEAD_KERNEL void gemm_nt_kernel(GemmArgs a) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    gemm_nt_body<DT, 1, DT>(a, blockIdx.x, smem);
+}
+
+// fp32 [R, C] (row stride ld) -> bf16 [R, 6 * cpad] (row stride ldo, cpad = C rounded up to 8, padding zero): the three
+// bf16 pieces x = p0 + p1 + p2 (p0 = bf16(x), p1 = bf16(x - p0), p2 = bf16(x - p0 - p1); 24 significant bits in all,
+// with the exponent range of fp32) laid out along the contraction axis so that an NT product of an "A side" and a
+// "B side" matrix sums the six piece products that matter, smallest first:
+//   slot        0      1      2      3      4      5
+//   A side      p2     p1     p0     p1     p0     p0
+//   B side      p0     p1     p2     p0     p1     p0      (p1*p2, p2*p1, p2*p2 are below fp32 rounding: dropped)
+__global__ __launch_bounds__(256) void split_bf16x3_kernel(const float* in, int64_t ld, int64_t R, int C, int cpad, int side,
+                                                           uint16_t* out, int64_t ldo) {
+    typedef Elem<TRLK_BF16> E;
+    const int64_t r = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (r >= R || c >= cpad) return;
+    float p[3] = {0.f, 0.f, 0.f};
+    if (c < C) {
+        const float x = in[r * ld + c];
+        uint16_t h;
+        E::store1(&h, x);
+        p[0] = E::to_float(h);
+        const float r1 = x - p[0];
+        E::store1(&h, r1);
+        p[1] = E::to_float(h);
+        E::store1(&h, r1 - p[1]);
+        p[2] = E::to_float(h);
+    }
+    const int a_map[6] = {2, 1, 0, 1, 0, 0}, b_map[6] = {0, 1, 2, 0, 1, 0};
+    uint16_t* o = out + r * ldo + c;
+#pragma unroll
+    for (int sl = 0; sl < 6; ++sl) E::store1(o + int64_t(sl) * cpad, p[side == 0 ? a_map[sl] : b_map[sl]]);
+}
+
 // Largest magnitude of a bf16 [R, C8 * 8] matrix (row stride ld) as the bit pattern of that float, through an atomic
 // maximum on `out` (non-negative floats order like unsigned integers; the caller clears `out`).
 __global__ __launch_bounds__(256) void maxabs_bf16_kernel(const uint16_t* in, int64_t ld, int R, int C8, uint32_t* out) {
@@ -1540,4 +1578,61 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         if (rc) return rc;
     }
     return TRLK_OK;
+}
+
+extern "C" int trlk_split_bf16x3(const float* d_in, int64_t rows, int64_t cols, int64_t ld_in, int side, void* d_out,
+                                 int64_t ld_out, trlk_stream_t stream) {
+    clear_error();
+    TRLK_REQUIRE(rows >= 0 && cols >= 1 && cols < (int64_t(1) << 28), TRLK_ERR_BAD_SHAPE, "split_bf16x3: bad shape %lld x %lld",
+                 (long long)rows, (long long)cols);
+    TRLK_REQUIRE(side == 0 || side == 1, TRLK_ERR_BAD_VALUE, "split_bf16x3: side must be 0 (A) or 1 (B), got %d", side);
+    const int64_t cpad = round_up(cols, 8);
+    TRLK_REQUIRE(ld_in >= cols && ld_out >= 6 * cpad && ld_out % 8 == 0, TRLK_ERR_BAD_STRIDE,
+                 "split_bf16x3: row strides too short (in %lld for %lld columns, out %lld for %lld)", (long long)ld_in,
+                 (long long)cols, (long long)ld_out, (long long)(6 * cpad));
+    if (rows == 0) return TRLK_OK;
+    TRLK_REQUIRE(d_in && d_out, TRLK_ERR_NULL_POINTER, "split_bf16x3: null pointer");
+    TRLK_REQUIRE(rows < 65536 * int64_t(32768), TRLK_ERR_BAD_SHAPE, "split_bf16x3: too many rows");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    for (int64_t r0 = 0; r0 < rows; r0 += 65535) {  // grid.y limit
+        const int64_t nr = rows - r0 < 65535 ? rows - r0 : 65535;
+        hipLaunchKernelGGL(split_bf16x3_kernel, dim3(unsigned((cpad + 255) / 256), unsigned(nr)), dim3(256), 0, s,
+                           d_in + r0 * ld_in, ld_in, nr, int(cols), int(cpad), side,
+                           static_cast<uint16_t*>(d_out) + r0 * ld_out, ld_out);
+    }
+    return launch_status("split_bf16x3");
+}
+
+extern "C" int trlk_gemm_nt(const void* d_a, int64_t lda, const void* d_b, int64_t ldb, int dtype, int64_t m, int64_t n,
+                            int64_t k, float* d_out, int64_t ldo, int accumulate, trlk_stream_t stream) {
+    clear_error();
+    TRLK_REQUIRE(dtype == TRLK_BF16 || dtype == TRLK_F16, TRLK_ERR_BAD_DTYPE, "gemm_nt: bf16 or fp16 operands (dtype code %d)",
+                 dtype);
+    TRLK_REQUIRE(m >= 0 && n >= 0 && k >= 8 && m < (int64_t(1) << 31) - BM && n < (int64_t(1) << 31) - BN &&
+                     k < (int64_t(1) << 31) - BK,
+                 TRLK_ERR_BAD_SHAPE, "gemm_nt: bad sizes m=%lld n=%lld k=%lld", (long long)m, (long long)n, (long long)k);
+    TRLK_REQUIRE(k % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && lda >= k && ldb >= k && ldo >= n, TRLK_ERR_BAD_STRIDE,
+                 "gemm_nt: k and the operands' row strides must be multiples of 8 elements (k=%lld lda=%lld ldb=%lld ldo=%lld)",
+                 (long long)k, (long long)lda, (long long)ldb, (long long)ldo);
+    // tile-relative operand offsets are 32-bit
+    TRLK_REQUIRE(lda * 2 * BM < (int64_t(1) << 32) && ldb * 2 * BN < (int64_t(1) << 32), TRLK_ERR_BAD_STRIDE,
+                 "gemm_nt: row strides too long (lda=%lld ldb=%lld)", (long long)lda, (long long)ldb);
+    if (m == 0 || n == 0) return TRLK_OK;
+    TRLK_REQUIRE(d_a && d_b && d_out, TRLK_ERR_NULL_POINTER, "gemm_nt: null pointer");
+    TRLK_REQUIRE(reinterpret_cast<uintptr_t>(d_a) % 16 == 0 && reinterpret_cast<uintptr_t>(d_b) % 16 == 0, TRLK_ERR_BAD_STRIDE,
+                 "gemm_nt: operands must be 16-byte aligned");
+    GemmArgs g{};
+    g.A = Operand{static_cast<const uint16_t*>(d_a), lda, int(m)};
+    g.B = Operand{static_cast<const uint16_t*>(d_b), ldb, int(n)};
+    g.M = int(m);
+    g.N = int(n);
+    g.K = int(k);
+    g.out_f32 = d_out;
+    g.ld_f32 = ldo;
+    g.first = accumulate ? 0 : 1;
+    g.mult_a = 1.f;
+    const int grid = xcd_patch_grid(int((m + BM - 1) / BM), int((n + BN - 1) / BN));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dtype == TRLK_BF16 ? launch_head(gemm_nt_kernel<TRLK_BF16>, grid, g, s, "gemm_nt")
+                              : launch_head(gemm_nt_kernel<TRLK_F16>, grid, g, s, "gemm_nt");
 }

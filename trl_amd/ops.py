@@ -783,6 +783,44 @@ def _(hidden, weight, targets, temperature, softcap, logit_scale, log_z, g_logp,
             torch.empty((weight.shape[0] if bias is not None else 0,), dtype=torch.float32, device=hidden.device))
 
 
+def split_bf16x3(x: Tensor, side: int) -> Tensor:
+    """fp32 `[R, C]` -> bf16 `[R, 6 * cpad]` (`cpad` = C rounded up to 8): the three bf16 pieces of every entry, laid
+    out along the contraction axis for the left (`side` 0) or right (`side` 1) operand of an NT product, so that the
+    matrix cores return the fp32 product to fp32 rounding (`trlk_split_bf16x3`)."""
+    if x.dim() != 2 or x.dtype != torch.float32 or not x.is_cuda:
+        raise TypeError("split_bf16x3: expected a 2-D float32 tensor on the GPU")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    rows, cols = x.shape
+    cpad = (cols + 7) // 8 * 8
+    out = torch.empty((rows, 6 * cpad), dtype=torch.bfloat16, device=x.device)
+    with torch.cuda.device(x.device):
+        check(lib.trlk_split_bf16x3(ptr(x), rows, cols, x.stride(0) if rows > 1 else cols, side, ptr(out), 6 * cpad,
+                                    current_stream(x.device)))
+    return out
+
+
+def gemm_nt(a: Tensor, b: Tensor, out: Optional[Tensor] = None, accumulate: bool = False) -> Tensor:
+    """`a [M, K] @ b [N, K].T` on the matrix cores (bf16 / fp16 operands with K contiguous, fp32 accumulation) into a
+    float32 `[M, N]` tensor; with `accumulate` the product is added to `out` (`trlk_gemm_nt`)."""
+    if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1] or a.dtype != b.dtype or not a.is_cuda:
+        raise ValueError(f"gemm_nt: operands do not match: {tuple(a.shape)} {a.dtype}, {tuple(b.shape)} {b.dtype}")
+    a = a if a.stride(1) == 1 else a.contiguous()
+    b = b if b.stride(1) == 1 else b.contiguous()
+    m, k = a.shape
+    n = b.shape[0]
+    if out is None:
+        if accumulate:
+            raise ValueError("gemm_nt: accumulate needs an output to add to")
+        out = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    elif out.shape != (m, n) or out.dtype != torch.float32 or out.stride(1) != 1:
+        raise ValueError("gemm_nt: out must be a float32 [M, N] tensor with contiguous rows")
+    with torch.cuda.device(a.device):
+        check(lib.trlk_gemm_nt(ptr(a), a.stride(0), ptr(b), b.stride(0), dtype_code(a.dtype), m, n, k, ptr(out),
+                               out.stride(0), int(accumulate), current_stream(a.device)))
+    return out
+
+
 def head_backward(hidden: Tensor, weight: Tensor, targets: Tensor, temperature: float, softcap: float,
                   logit_scale: float, log_z: Tensor, g_logp: Tensor, chunk_size: int, bias: Optional[Tensor] = None,
                   stash: Optional[Tensor] = None) -> tuple[Tensor, Tensor, Tensor]:

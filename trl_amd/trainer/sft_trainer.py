@@ -19,7 +19,7 @@ class _FusedNLLFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, weight, labels, chunk_size, softcap, logit_scale, bias=None):
         ctx.cfg = (int(chunk_size), softcap, logit_scale)
-        if hidden.dtype == torch.float32:  # fp32 operands: library GEMMs around the streaming kernels
+        if hidden.dtype == torch.float32:  # fp32 operands: three bf16 pieces each through the same kernels
             if not hidden.is_cuda:
                 raise NotImplementedError("the fused head runs on the GPU only")
             logp, ent, log_z, hit = _fp32_head_forward(hidden, weight.float(), labels.long(), 1.0, softcap, logit_scale,

@@ -141,66 +141,53 @@ def nanmax(tensor: Tensor) -> Tensor:
 # fused lm_head + log-prob (reference: trl/trainer/utils.py:1291-1517)
 # ----------------------------------------------------------------------------------------------
 def _fp32_head_block_rows(vocab: int) -> int:
-    """Token rows per block of the fp32-operand path: about 1 GiB of fp32 logits at a time."""
+    """Token rows per block of the fp32-operand backward: about 1 GiB of fp32 logits at a time."""
     return max(64, min(8192, (1 << 28) // max(vocab, 1)))
 
 
-def _fp32_head_logits(hidden_blk, weight, bias, cap, logit_scale):
-    """fp32 `[rows, V]` logits of a block of tokens before the temperature, and the soft-cap's tanh (or None)."""
-    y = hidden_blk @ weight.t()
-    if bias is not None:
-        y += bias
-    if logit_scale != 1.0:
-        y *= logit_scale
-    th = None
-    if cap > 0.0:
-        th = torch.tanh(y / cap)
-        y = th * cap
-    return y, th
-
-
 def _fp32_head_forward(hidden, weight, targets, temperature, cap, logit_scale, bias, want_hit=False):
-    """fp32 operands: the products come from the fp32 GEMM library one block of tokens at a time, the log-sum-exp,
-    entropy and gather of each block from the streaming log-prob kernel (whole vocabulary rows, so no online merge)."""
-    n, v = hidden.shape[0], weight.shape[0]
-    logp = torch.empty(n, dtype=torch.float32, device=hidden.device)
-    ent = torch.empty_like(logp)
-    lse = torch.empty_like(logp)
-    hit = torch.empty_like(logp) if want_hit else None
-    step = _fp32_head_block_rows(v)
-    for r0 in range(0, n, step):
-        r1 = min(r0 + step, n)
-        z, _ = _fp32_head_logits(hidden[r0:r1], weight, bias, cap, logit_scale)
-        idx = targets[r0:r1].reshape(-1, 1)
-        if want_hit:  # the row statistics carry the arg-max flag of the target
-            lp, e, l, st = ops.logp_entropy_stats_fwd(z.unsqueeze(0), idx, temperature, 0, r1 - r0, None)
-            hit[r0:r1] = st[:, 2]
-        else:
-            lp, e, l = ops.logp_entropy_forward(z.unsqueeze(0), idx, temperature, 0, r1 - r0, None)
-        logp[r0:r1], ent[r0:r1], lse[r0:r1] = lp.view(-1), e, l
+    """fp32 operands through the same fused kernel: both are split into three bf16 pieces laid out along the
+    contraction axis (`ops.split_bf16x3`), on which the matrix cores return the fp32 products to fp32 rounding; the
+    logits are never written to memory.  Costs six times the matrix work of bf16 operands and a `[V, 6 H]` bf16 copy
+    of the weight: this is the dtype of the reference's unit test (tests/test_utils.py:1161-1232), not of training."""
+    hp, wp = ops.split_bf16x3(hidden, 0), ops.split_bf16x3(weight, 1)
+    logp, ent, lse, hit, _ = ops.fused_head_fwd(hp, wp, targets, temperature, cap, logit_scale, bias, False)
     return (logp, ent, lse, hit) if want_hit else (logp, ent, lse)
 
 
 def _fp32_head_backward(hidden, weight, targets, temperature, cap, logit_scale, bias, lse, grad_logprobs):
-    """Recompute per block of tokens, d logits from the streaming backward kernel, the two products from the GEMM
-    library; everything in fp32."""
+    """fp32 operands: per block of tokens the logits are recomputed (`ops.gemm_nt` on bf16 pieces), d logits come
+    from the streaming backward kernel in fp32, and both gradient products run on the bf16 pieces of d logits,
+    W^T and hidden^T -- everything on this library's matrix-core kernel at fp32 accuracy, as the reference's fp32
+    `grad_logits @ w_chunk.float()` / `grad_logits.t() @ hidden.float()` (trl/trainer/utils.py:1421-1422)."""
     n, v = hidden.shape[0], weight.shape[0]
     d_hidden = torch.empty_like(hidden)
     d_weight = torch.zeros_like(weight)
     d_bias = torch.zeros(v, dtype=torch.float32, device=hidden.device) if bias is not None else None
     g = grad_logprobs.contiguous().float()
+    wp = ops.split_bf16x3(weight, 1)                   # [V, 6 H]: right operand of the logits
+    wtp = ops.split_bf16x3(weight.t().contiguous(), 1)  # [H, 6 V]: right operand of d hidden = dz @ W
     step = _fp32_head_block_rows(v)
     for r0 in range(0, n, step):
         r1 = min(r0 + step, n)
-        z, th = _fp32_head_logits(hidden[r0:r1], weight, bias, cap, logit_scale)
-        dz = ops.logp_entropy_bwd(z.unsqueeze(0), targets[r0:r1].reshape(-1, 1), temperature, 0, r1 - r0, lse[r0:r1], None,
+        y = ops.gemm_nt(ops.split_bf16x3(hidden[r0:r1], 0), wp)
+        if bias is not None:
+            y += bias
+        if logit_scale != 1.0:
+            y *= logit_scale
+        th = None
+        if cap > 0.0:
+            th = torch.tanh(y / cap)
+            y = th * cap
+        dz = ops.logp_entropy_bwd(y.unsqueeze(0), targets[r0:r1].reshape(-1, 1), temperature, 0, r1 - r0, lse[r0:r1], None,
                                   g[r0:r1].reshape(-1, 1), None).squeeze(0)
         if th is not None:
             dz *= 1.0 - th * th
         if logit_scale != 1.0:
             dz *= logit_scale
-        d_hidden[r0:r1] = dz @ weight
-        d_weight.addmm_(dz.t(), hidden[r0:r1])
+        ops.gemm_nt(ops.split_bf16x3(dz, 0), wtp, out=d_hidden[r0:r1])
+        ops.gemm_nt(ops.split_bf16x3(dz.t().contiguous(), 0), ops.split_bf16x3(hidden[r0:r1].t().contiguous(), 1),
+                    out=d_weight, accumulate=r0 > 0)
         if d_bias is not None:
             d_bias += dz.sum(0)
     return d_hidden, d_weight, d_bias
@@ -216,8 +203,9 @@ class _ChunkedLogProbFunction(torch.autograd.Function):
     sizes the backward's dz workspace).  When a gradient is required and the fp32 `[V, N]` products fit
     `ops.head_stash_fits` (24 GiB by default), the forward keeps them and the backward skips the
     reference's recompute of the logits; otherwise it recomputes them chunk by chunk as the reference does.
-    fp32 operands take a separate path: fp32 library GEMMs over blocks of tokens around the streaming log-prob
-    kernels (the matrix-core kernels take 16-bit operands only); fp64 is rejected.
+    fp32 operands run through the same kernels as three bf16 pieces each (`ops.split_bf16x3`: the matrix cores take
+    16-bit operands, six piece products give the fp32 product to fp32 rounding); their backward recomputes the logits
+    per block of tokens and takes d logits in fp32 from the streaming backward kernel.  fp64 is rejected.
     The entropy output is not differentiable, as in the reference.
     One argument beyond the reference's: `bias` [V], the `lm_head` bias the fused-linear losses take."""
 
