@@ -274,21 +274,34 @@ void launch_fused(const FusedArgs& a, int nvec, unsigned rows, hipStream_t s) {
     }
 }
 
-// data *= *scale over 16-byte vectors, unless the scale is exactly 1 (then nothing is read or written).  One vector
-// per lane and 4 KiB per workgroup, consecutive workgroups on consecutive addresses: the access pattern this
-// memory system serves fastest for a read-modify-write sweep.
+// data *= *scale over 16-byte vectors, unless the scale is exactly 1 (then nothing is read or written, and what the
+// launch costs is the dispatch of its workgroups: each takes a 64 KiB span so that a 20 GB buffer needs 300 000 of
+// them, about 0.06 ms, where one workgroup per 4 KiB costs a whole millisecond).  Inside a span the workgroup walks
+// 16 KiB at a time, four vectors per lane in flight.
+constexpr int kScaleSpanVec = 4096;  // vectors per workgroup
 template <int DT>
 __global__ __launch_bounds__(256) void scale_unless_one_kernel(u32x4* data, int64_t n_vec, const float* scale) {
     typedef Elem<DT> E;
     const float sc = *scale;
     if (sc == 1.f) return;
-    const int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x;
-    if (v >= n_vec) return;
-    float x[E::EPV];
-    E::unpack(__builtin_nontemporal_load(data + v), x);
+    const int64_t base = int64_t(blockIdx.x) * kScaleSpanVec + threadIdx.x;
+#pragma unroll 1
+    for (int it = 0; it < kScaleSpanVec / 1024; ++it) {
+        u32x4 q[4];
+        const int64_t v0 = base + it * 1024;
 #pragma unroll
-    for (int i = 0; i < E::EPV; ++i) x[i] *= sc;
-    __builtin_nontemporal_store(E::pack(x), data + v);
+        for (int j = 0; j < 4; ++j)
+            if (v0 + j * 256 < n_vec) q[j] = __builtin_nontemporal_load(data + v0 + j * 256);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (v0 + j * 256 >= n_vec) continue;
+            float x[E::EPV];
+            E::unpack(q[j], x);
+#pragma unroll
+            for (int i = 0; i < E::EPV; ++i) x[i] *= sc;
+            __builtin_nontemporal_store(E::pack(x), data + v0 + j * 256);
+        }
+    }
 }
 
 }  // namespace
@@ -304,8 +317,8 @@ extern "C" int trlk_scale_unless_one(void* d_data, int dtype, int64_t n_elems, c
     TRLK_REQUIRE(d_data && d_scale && reinterpret_cast<uintptr_t>(d_data) % 16 == 0, TRLK_ERR_NULL_POINTER,
                  "scale_unless_one: null or misaligned pointer");
     const int64_t n_vec = n_elems / 8;
-    TRLK_REQUIRE(n_vec <= int64_t(256) * 0x7fffffff, TRLK_ERR_BAD_SHAPE, "scale_unless_one: too many elements");
-    const unsigned grid = unsigned((n_vec + 255) / 256);
+    TRLK_REQUIRE(n_vec <= int64_t(kScaleSpanVec) * 0x7fffffff, TRLK_ERR_BAD_SHAPE, "scale_unless_one: too many elements");
+    const unsigned grid = unsigned((n_vec + kScaleSpanVec - 1) / kScaleSpanVec);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == TRLK_BF16)
         hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_BF16>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, d_scale);
