@@ -40,8 +40,15 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 MEASURED_TRAFFIC_BYTES = {
     ("K3", "grpo_c3", "dapo"): (10116130 + 19461194) * 1024,
     ("K7", "grpo_c3", "dapo"): (2 * 5064150 + 19488700) * 1024,
+    ("K3", "grpo_c4", "dapo"): (2 * 10693437 + 38927000) * 1024,
+    ("K7", "grpo_c4", "dapo"): (2 * 10701061 + 38975505) * 1024,
+    ("K3", "dpo_c2", None): (2 * 6612423 + 32860500) * 1024,
     ("head_fwd", "head_c5", "dapo"): (2 * 40600000 + 19497000) * 1024,
 }
+# the loss type changes per-row scalars only: the same rows are read and written, by the same launches
+for _k in ("K3", "K7"):
+    for _lt in ("grpo", "dr_grpo"):
+        MEASURED_TRAFFIC_BYTES[(_k, "grpo_c3", _lt)] = MEASURED_TRAFFIC_BYTES[(_k, "grpo_c3", "dapo")]
 
 WORKLOADS = {
     # name: (n_seq, completion_len, vocab, temperature, group_size, min_len)
@@ -410,7 +417,8 @@ def bench_dpo(args, w):
                    "loss": loss_dense},
         "roofline": {"bound": "hbm", "kernel": "logp_entropy_bwd_kernel (K3)", "achieved": bwd_bytes / (bwd_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": bwd_bytes / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                     "traffic": None, "algorithmic_bytes": bwd_bytes, "avg_launch_ms": bwd_ms},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(("K3", args.workload, None)), "algorithmic_bytes": bwd_bytes,
+                     "avg_launch_ms": bwd_ms},
         "kernels": {"logp_entropy_fwd_kernel with row statistics (K1)": {
             "avg_launch_ms": fwd_ms, "algorithmic_bytes": fwd_bytes, "achieved_GBps": fwd_bytes / (fwd_ms * 1e-3) / 1e9,
             "frac": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}},
