@@ -1,0 +1,86 @@
+"""The kernels under HIP graph capture: a captured micro-step is replayed on new inputs several times, with eager
+work and synchronisations between the replays, and every replay must equal the eager result bit for bit (the same
+kernels run in both).  Two graphs: log-prob kernel -> GRPO loss through the entry point that allocates nothing ->
+gradient kernel; and the single-pass GRPO kernel.  The library records no memset into a graph and keeps no host
+state between launches, which is what these replays would show if it did."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+B, T, V = 6, 40, 4096
+
+
+def _new_inputs(buf, seed):
+    """Fills the static input buffers in place (eagerly) with the problem of this seed."""
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    buf["logits"].copy_((2.0 * torch.randn((B, T + 1, V), generator=g, device=DEV)).bfloat16())
+    buf["ids"].copy_(torch.randint(0, V, (B, T), generator=g, device=DEV))
+    lengths = torch.randint(0, T + 1, (B,), generator=g, device=DEV)
+    buf["mask"].copy_((torch.arange(T, device=DEV)[None] < lengths[:, None]).float())
+    buf["adv"].copy_(torch.randn((B,), generator=g, device=DEV))
+    buf["old_noise"].copy_(0.05 * torch.randn((B, T), generator=g, device=DEV))
+    buf["n_items"].copy_(buf["mask"].sum().clamp(min=1.0).reshape(1))
+
+
+def _buffers():
+    return dict(
+        logits=torch.zeros((B, T + 1, V), dtype=torch.bfloat16, device=DEV), ids=torch.zeros((B, T), dtype=torch.int64, device=DEV),
+        mask=torch.zeros((B, T), device=DEV), adv=torch.zeros((B,), device=DEV), old_noise=torch.zeros((B, T), device=DEV),
+        n_items=torch.ones((1,), device=DEV), loss=torch.zeros((), device=DEV), metrics=torch.zeros((16,), device=DEV),
+        dlogp=torch.zeros((B, T), device=DEV), row_scale=torch.zeros((B,), device=DEV))
+
+
+def _two_pass_step(buf):
+    from trl_amd import _lib, ops
+
+    idx = buf["ids"].reshape(B * T, 1)
+    lp, ent, lse = ops.logp_entropy_fwd(buf["logits"], idx, 0.9, 0, T, None)
+    lp2 = lp.view(B, T)
+    old = lp2 + buf["old_noise"]
+    ops.grpo_loss_static_(buf["loss"], buf["metrics"], buf["dlogp"], None, lp2, old, None, ent.view(B, T), buf["adv"], buf["mask"],
+                          None, None, buf["n_items"], _lib.DAPO, 0.2, 0.28, math.nan, 0.0, False, 1.0, float(B * T), 1.0, 0.0)
+    dlogits = ops.logp_entropy_bwd(buf["logits"], idx, 0.9, 0, T, lse, None, buf["dlogp"].view(B * T, 1), None)
+    return lp, ent, buf["loss"], buf["metrics"], dlogits
+
+
+def _single_pass_step(buf):
+    from trl_amd import _lib, ops
+
+    buf["row_scale"].copy_((1.0 / buf["n_items"]).expand(B))  # dapo: 1 / num_items for every sequence
+    return ops.grpo_fused_fwd_bwd(buf["logits"], buf["ids"], 0.9, 0, T, buf["mask"], buf["adv"], buf["row_scale"], None, None,
+                                  None, None, _lib.TERM_CLIP, 0.2, 0.28, math.nan, 0.0, False, 1.0, 1.05)
+
+
+@pytest.mark.parametrize("step", [_two_pass_step, _single_pass_step], ids=["two_pass", "single_pass"])
+def test_graph_replays_equal_eager(step):
+    from trl_amd import _lib
+
+    assert _lib.lib.trlk_init() == 0
+    buf = _buffers()
+    _new_inputs(buf, 100)
+    side = torch.cuda.Stream()  # warm-up off the capture stream: lazy buffers of the library and of torch exist afterwards
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(buf)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step(buf)
+    for rep in range(4):
+        _new_inputs(buf, 200 + rep)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        scratch = torch.randn((1 << 20,), device=DEV).sum()  # eager work of the program's own between the replays
+        want = step(buf)
+        torch.cuda.synchronize()
+        assert math.isfinite(float(scratch))
+        for i, (g, w) in enumerate(zip(got, want)):
+            assert torch.equal(g.nan_to_num(nan=-7.0), w.nan_to_num(nan=-7.0)), (rep, i)
+        assert float(got[-1].float().abs().sum()) > 0 or float(buf["mask"].sum()) == 0
