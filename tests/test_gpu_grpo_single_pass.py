@@ -86,6 +86,63 @@ def test_matches_two_pass(amd, loss_type, beta):
     amd.check_device_errors()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rows_that_leave_the_fast_reduction(amd, dtype):
+    """The kernel sums the exponentials against the maximum of a lane's FIRST vector while the row still arrives; a
+    row whose later logits exceed that by more than 128 / (log2(e) / T), or that holds an infinity or a NaN, takes
+    the exact two-sweep reduction instead.  Such rows -- a spike late in the row, a wide ramp, -inf entries (a masked
+    vocabulary), one +inf, one NaN -- against the two-pass path and, where the row is finite, against float64."""
+    B, K, V, T = 4, 12, 8192, 0.7
+    logits, ids, _, adv, g = _inputs(B, K, V, dtype=dtype, seed=21, extra_rows=1)
+    mask = torch.ones((B, K), dtype=torch.long, device=DEV)
+    big = 30000.0 if dtype == torch.float16 else 1e4
+    x = logits.float()
+    x[0, 0, V - 5] = 300.0                                   # one spike at the end of the row
+    x[0, 1] = torch.linspace(-400.0, 400.0, V, device=DEV)   # a ramp: every later vector is larger than the first
+    x[0, 2, 1024:] = float("-inf")                           # most of the vocabulary masked out
+    x[0, 3] = float("-inf")
+    x[0, 3, 77] = 1.5                                        # a single admissible token
+    x[0, 4, 4000] = big                                      # near the largest finite value of the dtype
+    x[0, 5, 123] = float("inf")
+    x[0, 6, 4567] = float("nan")
+    x[1, 0, :8] = -300.0                                     # the FIRST vector far below the rest
+    ids[0, 2], ids[0, 3] = 5, 77
+    logits = x.to(dtype)
+    kw = dict(loss_type="grpo", epsilon_low=0.2, epsilon_high=0.28, beta=0.0, max_completion_length=K,
+              num_items_in_batch=mask.sum().float())
+    leaf2, loss2, _, lp2, ent2 = _two_pass(amd, logits, ids, mask, adv, T, **kw)
+    loss2.backward()
+    leaf1 = logits.detach().clone().requires_grad_(True)
+    loss1, _, lp1, ent1 = amd.grpo_loss_from_logits(leaf1, ids, adv, mask, temperature=T, **kw)
+    loss1.backward()
+    torch.testing.assert_close(lp1, lp2, rtol=1e-5, atol=1e-5, equal_nan=True)
+    # (the entropy is lse - E_p[z] on both paths, as in the reference's fused operator, utils.py:1357: its absolute
+    # error grows with the size of the logits, two fp32 steps of the largest |z| of the row)
+    zmax = (logits[:, :K].float().nan_to_num(nan=0.0, posinf=0.0, neginf=0.0).abs().amax(-1) / T)
+    ent_tol = 2e-5 + 2.5e-7 * zmax
+    ok = ((ent1 - ent2).abs() <= ent_tol) | (torch.isnan(ent1) & torch.isnan(ent2))
+    assert bool(ok.all()), (ent1 - ent2).abs().max()
+    g1, g2 = leaf1.grad[:, :K].float(), leaf2.grad[:, :K].float()
+    bad = torch.zeros((B, K), dtype=torch.bool, device=DEV)
+    bad[0, 5] = bad[0, 6] = True  # +inf / NaN rows: NaN outputs on both paths, as the reference's log_softmax gives
+    assert bool(torch.isnan(lp1[bad]).all()) and bool(torch.isnan(lp2[bad]).all())
+    finite = ~bad
+    assert bool(torch.isfinite(lp1[finite]).all()) and bool(torch.isfinite(g1[finite]).all())
+    for b, t in ((0, 0), (0, 1), (0, 2), (0, 3), (0, 4), (1, 0), (2, 3)):
+        assert float((g1[b, t] - g2[b, t]).norm()) <= 2e-3 * float(g2[b, t].norm()) + 1e-7, (b, t)
+        z = logits[b, t].double() / T
+        want = torch.log_softmax(z, -1)
+        assert abs(float(lp1[b, t]) - float(want[ids[b, t]])) < 1e-5 * max(1.0, abs(float(want[ids[b, t]]))), (b, t)
+        if bool(torch.isinf(z).any()):  # the reference's -sum p log p is NaN for a row with a -inf logit (0 * -inf)
+            assert math.isnan(float(ent1[b, t])) and math.isnan(float(ent2[b, t]))
+            continue
+        h = -(want.exp() * want).sum()
+        assert abs(float(ent1[b, t]) - float(h)) < float(ent_tol[b, t]) + 2e-5 * float(h), (b, t, float(ent1[b, t]), float(h))
+    # the single admissible token: log-prob 0, gradient zero (the entropy of a row with -inf entries is NaN, as the
+    # reference's -sum p log p is)
+    assert abs(float(lp1[0, 3])) < 1e-6 and float(g1[0, 3].abs().max()) < 1e-6
+
+
 def test_window_given_by_keep_start(amd):
     """`keep_start` places the K-row window anywhere in the logits (here: all rows, no position dropped)."""
     B, K, V = 3, 8, 512

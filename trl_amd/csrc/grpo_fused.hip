@@ -236,8 +236,12 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     if (!idx_ok) g = 0.f;  // an invalid index leaves a zero row (its log-prob is NaN and the flag is set)
     // dlogits[v] = p_v (a0 + b0 tt_v) (+ g / T at the target), p_v = 2^tt_v, tt_v = x c - lse2 = (z_v - lse) log2(e):
     // -g p_v / T from the log-prob, -h p_v ((z_v - lse) + H) / T from the entropy
-    const float a0 = (-g - h * ent) * inv_t;
-    const float b0 = -h * kLn2 * inv_t;
+    // Without an entropy term (h == 0, uniform over the workgroup) the factor is the constant a0: a logit of -inf
+    // (a masked vocabulary entry) then gets the gradient 0 it has in the reference, where b0 * tt would be 0 * -inf,
+    // and an entropy that is NaN for such a row (as the reference's is) stays out of the gradient.
+    const bool with_h = h != 0.f;
+    const float a0 = with_h ? (-g - h * ent) * inv_t : -g * inv_t;
+    const float b0 = with_h ? -h * kLn2 * inv_t : 0.f;
 #pragma unroll
     for (int j = 0; j < NVEC; ++j) {
         const int v = j * kFThreads + tid;
@@ -247,7 +251,7 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
 #pragma unroll
             for (int i = 0; i < EPV; ++i) {
                 const float tt = fmaf(x[i], c, -lse2);
-                d[i] = fast_exp2(tt) * fmaf(b0, tt, a0);
+                d[i] = fast_exp2(tt) * (with_h ? fmaf(b0, tt, a0) : a0);
             }
             GlobalVecOut* oj = (GlobalVecOut*)op + j * kFThreads;
             asm volatile("" : "+s"(oj));
@@ -259,7 +263,7 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     if (idx_ok && int((idx / EPV) % kFThreads) == tid) {
         T* out = reinterpret_cast<T*>(op);
         const float tt = fmaf(x_t, c, -lse2);
-        E::store1(out + idx, fast_exp2(tt) * fmaf(b0, tt, a0) + g * inv_t);
+        E::store1(out + idx, fast_exp2(tt) * (with_h ? fmaf(b0, tt, a0) : a0) + g * inv_t);
     }
 }
 
