@@ -262,6 +262,28 @@ def test_minus_inf_logits_and_row_mask(amd):
     assert torch.count_nonzero(ent.cpu()[mask == 0]) == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
+def test_minus_inf_logits_backward(amd, dtype):
+    """The gradient of the log-probs at a -inf logit (a masked-out vocabulary entry) is 0, as autograd's
+    log_softmax backward gives (trl/trainer/utils.py:510 / :519-521), and the other entries are unaffected."""
+    g = torch.Generator().manual_seed(12)
+    logits = (2.0 * torch.randn(2, 5, 512, generator=g)).to(dtype)
+    logits[:, :, 100:300] = -math.inf
+    logits[0, 1, 300:] = -math.inf  # one row with a single block of admissible tokens
+    idx = torch.randint(0, 100, (2, 5), generator=g)
+    gout = torch.randn(2, 5, generator=g)
+    ref = logits.clone().double().requires_grad_(True)
+    (torch.log_softmax(ref / 0.8, -1).gather(-1, idx[..., None]).squeeze(-1) * gout.double()).sum().backward()
+    leaf = logits.clone().to(DEV).requires_grad_(True)
+    lp, _ = amd.logps_and_entropies(leaf, idx.to(DEV), temperature=0.8)
+    (lp.double() * gout.to(DEV).double()).sum().backward()
+    got = leaf.grad.double().cpu()
+    assert bool(torch.isfinite(got).all())
+    assert float(got[:, :, 100:300].abs().max()) == 0.0
+    tol = {torch.float32: 1e-5, torch.bfloat16: 1e-2, torch.float64: 1e-12}[dtype]
+    assert float((got - ref.grad).norm() / ref.grad.norm()) < tol
+
+
 def test_index_out_of_range_sets_flag(amd):
     logits = torch.randn(1, 2, 64, device=DEV)
     idx = torch.tensor([[3, 64]], device=DEV)

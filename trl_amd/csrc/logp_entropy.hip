@@ -411,12 +411,15 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_bwd_kernel(BwdArgs a, i
     const float c = kLog2e * inv_t;
     const float lsec = a.lse[row] * kLog2e;
     // dz_v = p_v * (a0 + b0 * tt),  tt = x*c - lse*log2e = (z - lse) * log2e
-    const float a0 = HAS_H ? (-gsum - h * a.entropy[row]) * inv_t : -gsum * inv_t;
-    const float b0 = HAS_H ? -h * kLn2 * inv_t : 0.f;
+    // (a row without an entropy gradient of its own keeps the constant factor: its entropy may be NaN, as the
+    // reference's is for a row with -inf logits, and b0 * tt would be 0 * -inf at such a logit)
+    const bool with_h = HAS_H && h != 0.f;
+    const float a0 = with_h ? (-gsum - h * a.entropy[row]) * inv_t : -gsum * inv_t;
+    const float b0 = with_h ? -h * kLn2 * inv_t : 0.f;
     auto grad_of = [&](float x) {
         const float tt = fmaf(x, c, -lsec);
         const float p = fast_exp2(tt);
-        return HAS_H ? p * fmaf(b0, tt, a0) : p * a0;
+        return with_h ? p * fmaf(b0, tt, a0) : p * a0;
     };
 
     if constexpr (VEC) {

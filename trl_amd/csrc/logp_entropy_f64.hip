@@ -127,7 +127,8 @@ __global__ __launch_bounds__(kT64) void logp_entropy_bwd_f64_kernel(Bwd64 a) {
     const double H = a.g_entropy ? a.entropy[row] : 0.0;
     for (int64_t v = tid; v < a.vocab; v += kT64) {
         const double tt = x[v] * a.inv_t - lse;
-        out[v] = exp(tt) * (-gsum - h * (tt + H)) * a.inv_t;
+        // (without an entropy gradient the factor is the constant -gsum: h * tt would be 0 * -inf at a -inf logit)
+        out[v] = exp(tt) * (h != 0.0 ? -gsum - h * (tt + H) : -gsum) * a.inv_t;
     }
     __syncthreads();  // the one-hot terms are added by one lane after every softmax term of the row is stored
     if (tid == 0)
