@@ -282,7 +282,7 @@ class _GRPOFromLogits(torch.autograd.Function):
             n_items = kw["num_items_in_batch"]
             n_items = (n_items.to(device=logits.device, dtype=torch.float32) if torch.is_tensor(n_items)
                        else torch.tensor(float(n_items), dtype=torch.float32, device=logits.device))
-            row_scale = (1.0 / (n_items.clamp(min=1.0) / float(kw["num_processes"]))).reshape(1).expand(n_seq)
+            row_scale = (float(kw["num_processes"]) / n_items.clamp(min=1.0)).reshape(1).expand(n_seq)
         ent_weight = None
         if kw["entropy_coef"] != 0.0:  # d loss / d entropy = -coef * mask / normaliser (grpo_trainer.py:3155-3181)
             if reduce_code == _lib.DAPO:
@@ -326,6 +326,7 @@ class _GRPOFromLogits(torch.autograd.Function):
             sapo_temperature_pos=kw["sapo_temperature_pos"], sapo_temperature_neg=kw["sapo_temperature_neg"])
         ctx.save_for_backward(dlogits, *(() if up is None else (up,)))
         ctx.mark_non_differentiable(metrics, logp, ent)
+        ctx.set_materialize_grads(False)  # (no zero tensors for the outputs that carry no gradient)
         ctx.consumed = False
         return loss, metrics, logp, ent
 
