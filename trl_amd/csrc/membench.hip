@@ -11,6 +11,8 @@
 //   row    one 1024-lane workgroup per 304 KB row, the row held in registers between its loads and its stores
 //          (the access pattern of the single-pass GRPO kernel), every row or the benchmark's mask (48 % of the
 //          rows are only zero-filled)
+//   piece  the same with a row cut into 2 or 4 pieces, one workgroup per piece (several workgroups per CU at a
+//          time, as a kernel whose workgroups exchange the row's statistics would run, without that exchange)
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -102,6 +104,38 @@ __global__ __launch_bounds__(1024) void row_kernel(const u32x4* in, u32x4* out, 
         }
 }
 
+template <int THREADS, int PARTS>
+__global__ __launch_bounds__(THREADS) void piece_kernel(const u32x4* in, u32x4* out, const uint8_t* active) {
+    constexpr int kPieceVec = (kRowVec + PARTS - 1) / PARTS;
+    constexpr int PER = (kPieceVec + THREADS - 1) / THREADS;
+    const int tid = threadIdx.x;
+    const int64_t row = blockIdx.x / PARTS;
+    const int v0 = int(blockIdx.x % PARTS) * kPieceVec, nv = min(v0 + kPieceVec, kRowVec) - v0;
+    const u32x4* ip = in + row * kRowVec + v0;
+    u32x4* op = out + row * kRowVec + v0;
+    if (!active[row]) {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        for (int v = tid; v < nv; v += THREADS) __builtin_nontemporal_store(z, op + v);
+        return;
+    }
+    u32x4 q[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        GIn* vj = (GIn*)ip + j * THREADS;
+        asm volatile("" : "+s"(vj));
+        if (j * THREADS < nv) q[j] = vj[max(min(tid, nv - 1 - j * THREADS), 0)];
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j) asm volatile("" : "+v"(q[j]));
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+        if (j * THREADS + tid < nv) {
+            GOut* oj = (GOut*)op + j * THREADS;
+            asm volatile("" : "+s"(oj));
+            __builtin_nontemporal_store(q[j], oj + tid);
+        }
+}
+
 int main() {
     const int B = 64, T = 1024;
     const int64_t rows = int64_t(B) * T, n = rows * kRowVec;
@@ -160,6 +194,14 @@ int main() {
             [&] { hipLaunchKernelGGL((row_kernel<false, true>), dim3(unsigned(rows)), dim3(1024), 0, 0, in, out, act_d); });
         run(masked ? "row in registers, benchmark mask, nt/nt" : "row in registers, every row, nt/nt", moved,
             [&] { hipLaunchKernelGGL((row_kernel<true, true>), dim3(unsigned(rows)), dim3(1024), 0, 0, in, out, act_d); });
+        run(masked ? "2 pieces of 1024 lanes, benchmark mask, plain/nt" : "2 pieces of 1024 lanes, every row, plain/nt", moved,
+            [&] { hipLaunchKernelGGL((piece_kernel<1024, 2>), dim3(unsigned(rows * 2)), dim3(1024), 0, 0, in, out, act_d); });
+        run(masked ? "2 pieces of 512 lanes, benchmark mask, plain/nt" : "2 pieces of 512 lanes, every row, plain/nt", moved,
+            [&] { hipLaunchKernelGGL((piece_kernel<512, 2>), dim3(unsigned(rows * 2)), dim3(512), 0, 0, in, out, act_d); });
+        run(masked ? "4 pieces of 1024 lanes, benchmark mask, plain/nt" : "4 pieces of 1024 lanes, every row, plain/nt", moved,
+            [&] { hipLaunchKernelGGL((piece_kernel<1024, 4>), dim3(unsigned(rows * 4)), dim3(1024), 0, 0, in, out, act_d); });
+        run(masked ? "4 pieces of 256 lanes, benchmark mask, plain/nt" : "4 pieces of 256 lanes, every row, plain/nt", moved,
+            [&] { hipLaunchKernelGGL((piece_kernel<256, 4>), dim3(unsigned(rows * 4)), dim3(256), 0, 0, in, out, act_d); });
     }
     run("hipMemcpyAsync device to device", 2.0 * bytes, [&] { CHECK(hipMemcpyAsync(out, in, bytes, hipMemcpyDeviceToDevice, 0)); });
     return 0;
