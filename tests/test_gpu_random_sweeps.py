@@ -1,0 +1,217 @@
+"""Seeded random sweeps over configurations, shapes and dtypes: the HIP path against the CPU oracle (GRPO and DPO
+losses with their gradients), the single-pass GRPO kernel against the two-pass path, and the fused head against
+fp32 autograd.  The golden vectors pin chosen configurations; these sweeps walk the combinations between them (loss
+type x importance-sampling level x delta x KL x masks x advantage shape x entropy bonus ..., odd sizes, empty
+sequences).  Bars as in the other GPU tests: fp32 2e-5, 16-bit gradients by relative L2."""
+import math
+import os
+import random
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def amd():
+    import trl_amd
+
+    return trl_amd
+
+
+def _rel(a, b):
+    a, b = a.double().cpu(), b.double().cpu()
+    return float((a - b).norm() / b.norm().clamp(min=1e-30))
+
+
+def test_grpo_loss_kernel_against_the_oracle(amd):
+    """300 configurations of the `[B, T]` loss kernel: loss and d loss / d logp (and d loss / d entropy) against the
+    oracle's autograd."""
+    rnd = random.Random(1)
+    torch.manual_seed(1)
+    ran = 0
+    for case in range(300):
+        B, T = rnd.choice([1, 2, 3, 8]), rnd.choice([1, 5, 17, 64])
+        lt = rnd.choice(["grpo", "bnpo", "dr_grpo", "dapo", "cispo", "sapo", "luspo", "vespo"])
+        beta = rnd.choice([0.0, 0.04, 0.5])
+        lp = -3 * torch.rand(B, T)
+        old = rnd.choice([None, lp + rnd.choice([0.0, 0.05, 0.5, 2.0]) * torch.randn(B, T)])
+        ref = lp + 0.2 * torch.randn(B, T) if beta else None
+        mask = (torch.arange(T)[None] < torch.randint(0, T + 1, (B,))[:, None]).long()
+        if rnd.random() < 0.2:
+            mask = (torch.rand(B, T) < 0.6).long()
+        adv = rnd.choice([torch.randn(B), torch.randn(B, T) if lt != "luspo" else torch.randn(B)])
+        if rnd.random() < 0.1:
+            adv = torch.zeros_like(adv)
+        ent = 3 * torch.rand(B, T)
+        kw = dict(old_per_token_logps=old, ref_per_token_logps=ref, loss_type=lt, epsilon_low=rnd.choice([0.2, 0.1]),
+                  epsilon_high=rnd.choice([0.2, 0.28, 3.0 if lt == "cispo" else 0.2]), beta=beta,
+                  delta=rnd.choice([None, None, 1.5, 4.0]) if lt not in ("cispo", "sapo", "vespo") else None,
+                  max_completion_length=T, num_items_in_batch=float(int(mask.sum())) * rnd.choice([1.0, 2.0]),
+                  num_processes=rnd.choice([1, 2]), grad_accum_steps=rnd.choice([1.0, 4.0]),
+                  importance_sampling_level=rnd.choice(["token", "token", "sequence"]),
+                  use_bias_correction_kl=old is not None and rnd.random() < 0.3, entropy_coef=rnd.choice([0.0, 0.0, 0.01]))
+        olp, oent = lp.clone().requires_grad_(True), ent.clone().requires_grad_(True)
+        try:
+            oloss, _ = oracle.grpo_loss(olp, adv, mask, entropies=oent, **kw)
+        except (ValueError, NotImplementedError):
+            continue  # a combination the reference rejects too
+        oloss.backward()
+        glp, gent = lp.to(DEV).requires_grad_(True), ent.to(DEV).requires_grad_(True)
+        gkw = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in kw.items()}
+        gloss, _ = amd.grpo_loss(glp, adv.to(DEV), mask.to(DEV), entropies=gent, **gkw)
+        gloss.backward()
+        what = (case, lt, kw["importance_sampling_level"], beta, kw["delta"], tuple(adv.shape))
+        assert abs(float(gloss.detach()) - float(oloss.detach())) <= 2e-5 * max(1.0, abs(float(oloss.detach()))), what
+        scale = float(olp.grad.abs().max())
+        assert float((glp.grad.cpu() - olp.grad).abs().max()) <= 2e-5 * scale + 1e-7, what
+        if kw["entropy_coef"]:
+            ge = gent.grad.cpu() if gent.grad is not None else torch.zeros_like(ent)
+            assert float((ge - oent.grad).abs().max()) <= 2e-5 * float(oent.grad.abs().max()) + 1e-8, what
+        ran += 1
+    assert ran >= 200
+
+
+def test_single_pass_kernel_against_the_two_pass_path(amd):
+    """250 configurations the single-pass kernel takes (loss types, KL, delta, bias-corrected KL, token weights,
+    per-token advantages, entropy bonus, temperatures, bf16 / fp16, vocabularies 8 ... 20488, empty sequences, ragged
+    masks): loss, metrics, log-probs and dlogits against K1 + loss kernel + K3."""
+    rnd = random.Random(2)
+    torch.manual_seed(2)
+    for case in range(250):
+        B, K, V = rnd.choice([1, 2, 5]), rnd.choice([1, 7, 33]), rnd.choice([8, 64, 264, 1000, 4096, 20488])
+        L = K + rnd.choice([1, 1, 3])
+        dt = rnd.choice([torch.bfloat16, torch.float16])
+        lt = rnd.choice(["grpo", "bnpo", "dr_grpo", "dapo", "cispo", "sapo"])
+        beta, T = rnd.choice([0.0, 0.04]), rnd.choice([1.0, 0.7, 1.3])
+        logits = (rnd.choice([0.5, 2.0, 6.0]) * torch.randn(B, L, V, device=DEV)).to(dt)
+        ids = torch.randint(0, V, (B, K), device=DEV)
+        mask = (torch.arange(K, device=DEV)[None] < torch.randint(0, K + 1, (B,), device=DEV)[:, None]).long()
+        if rnd.random() < 0.2:
+            mask = (torch.rand(B, K, device=DEV) < 0.5).long()
+        adv = rnd.choice([torch.randn(B, device=DEV), torch.randn(B, K, device=DEV)])
+        with torch.no_grad():
+            base, _ = amd.per_token_logps_and_entropies(logits, ids, K, T)
+        old = rnd.choice([None, base + rnd.choice([0.05, 0.5]) * torch.randn(B, K, device=DEV)])
+        kw = dict(old_per_token_logps=old, ref_per_token_logps=base + 0.2 * torch.randn(B, K, device=DEV) if beta else None,
+                  loss_type=lt, epsilon_low=0.2, epsilon_high=0.28, beta=beta,
+                  delta=rnd.choice([None, 2.0]) if lt not in ("cispo", "sapo") else None, max_completion_length=K,
+                  num_items_in_batch=mask.sum().float() * 2, grad_accum_steps=rnd.choice([1.0, 2.0]),
+                  use_bias_correction_kl=old is not None and rnd.random() < 0.3,
+                  token_weight=rnd.choice([None, None, 0.5 + torch.rand(B, K, device=DEV)]),
+                  entropy_coef=rnd.choice([0.0, 0.0, 0.02]))
+        leaf2 = logits.detach().clone().requires_grad_(True)
+        lp2, ent2 = amd.per_token_logps_and_entropies(leaf2, ids, K, T, True, True)
+        loss2, met2 = amd.grpo_loss(lp2, adv, mask, entropies=ent2, **kw)
+        loss2.backward()
+        leaf1 = logits.detach().clone().requires_grad_(True)
+        loss1, met1, lp1, _ = amd.grpo_loss_from_logits(leaf1, ids, adv, mask, temperature=T, **kw)
+        loss1.backward()
+        what = (case, lt, str(dt), V, beta, T, kw["delta"], kw["entropy_coef"])
+        assert abs(float(loss1.detach()) - float(loss2.detach())) <= 2e-5 * max(1.0, abs(float(loss2.detach()))), what
+        torch.testing.assert_close(met1, met2, rtol=1e-4, atol=1e-5, equal_nan=True)
+        m = mask.bool()
+        if bool(m.any()):
+            assert float((lp1[m] - lp2.detach()[m]).abs().max()) <= 2e-5 * max(1.0, float(lp2.detach()[m].abs().max())), what
+        if float(leaf2.grad.float().abs().max()) > 0:
+            assert _rel(leaf1.grad, leaf2.grad) < 4e-3, what
+        else:
+            assert float(leaf1.grad.float().abs().max()) == 0.0, what
+    amd.check_device_errors()
+
+
+def test_dpo_loss_against_the_oracle(amd):
+    """300 configurations of `dpo_compute_loss` (fifteen loss types alone and in weighted pairs, label smoothing,
+    ld_alpha, WPO weighting, f-divergences, fp32 and bf16 logits, ragged completion masks): loss and dlogits."""
+    rnd = random.Random(3)
+    torch.manual_seed(3)
+    types = ["sigmoid", "hinge", "ipo", "exo_pair", "nca_pair", "robust", "bco_pair", "sppo_hard", "aot", "aot_unpaired",
+             "apo_zero", "apo_down", "discopop", "sft", "sigmoid_norm"]
+    ran = 0
+    for case in range(300):
+        P, L, V = rnd.choice([1, 2, 5]), rnd.choice([2, 6, 19]), rnd.choice([5, 64, 257, 1000])
+        dt = rnd.choice([torch.float32, torch.float32, torch.bfloat16])
+        logits = (2.0 * torch.randn(2 * P, L, V)).to(dt)
+        ids = torch.randint(0, V, (2 * P, L))
+        start, end = torch.randint(0, L, (2 * P,)), torch.randint(0, L + 1, (2 * P,))
+        ar = torch.arange(L)[None]
+        cm = ((ar >= start[:, None]) & (ar < torch.maximum(end, start + 1)[:, None])).long()
+        refc, refr = -5 * torch.rand(P), -5 * torch.rand(P)
+        n_types = rnd.choice([1, 1, 2])
+        kw = dict(beta=rnd.choice([0.1, 0.5]), loss_types=tuple(rnd.sample(types, n_types)),
+                  loss_weights=None if n_types == 1 else [0.7, 1.3], label_smoothing=rnd.choice([0.0, 0.1]),
+                  ld_alpha=rnd.choice([None, None, 0.3]), use_weighting=rnd.random() < 0.25,
+                  f_divergence_type=rnd.choice(["reverse_kl", "reverse_kl", "js_divergence", "alpha_divergence"]))
+        ol = logits.float().clone().requires_grad_(True)
+        oloss, _ = oracle.dpo_compute_loss(ol, ids, cm, refc, refr, f_alpha=0.5, **kw)
+        if not math.isfinite(float(oloss.detach())) or abs(float(oloss.detach())) > 1e6:
+            continue  # (exo_pair without label smoothing is log 0, an f-divergence may overflow: in the reference too)
+        oloss.backward()
+        gl = logits.clone().to(DEV).requires_grad_(True)
+        gloss, _ = amd.dpo_compute_loss(gl, ids.to(DEV), cm.to(DEV), refc.to(DEV), refr.to(DEV), f_alpha_divergence_coef=0.5, **kw)
+        gloss.backward()
+        what = (case, kw["loss_types"], str(dt), kw["ld_alpha"], kw["use_weighting"], kw["f_divergence_type"])
+        tol = 2e-5 if dt == torch.float32 else 2e-2
+        assert abs(float(gloss.detach()) - float(oloss.detach())) <= tol * max(1.0, abs(float(oloss.detach()))), what
+        if float(ol.grad.abs().max()) > 1e-10:
+            assert _rel(gl.grad.float(), ol.grad) <= (2e-4 if dt == torch.float32 else 2e-2), what
+        else:
+            assert float(gl.grad.float().abs().max()) <= 1e-7, what
+        ran += 1
+    assert ran >= 200
+
+
+def test_fused_head_against_fp32_autograd(amd, monkeypatch):
+    """120 fused-head problems: token / hidden / vocabulary sizes around the tile edges (1, 255, 256, 257, ...), chunk
+    sizes, temperature, soft-capping, logit scale, bias, bf16 / fp16 / fp32 operands, with and without the stash,
+    with and without tokens whose upstream gradient is zero."""
+    rnd = random.Random(4)
+    torch.manual_seed(4)
+    for case in range(120):
+        n, h = rnd.choice([1, 3, 64, 255, 256, 257, 300, 513, 700]), rnd.choice([8, 24, 64, 136, 256, 520])
+        v = rnd.choice([2, 7, 255, 256, 257, 1000, 2305, 5000])
+        chunk, T = rnd.choice([1, 100, 256, 1024, 8192]), rnd.choice([1.0, 0.7])
+        cap, scale = rnd.choice([None, None, 5.0]), rnd.choice([1.0, 0.5])
+        dt = rnd.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+        use_bias = rnd.random() < 0.3
+        monkeypatch.setenv("TRL_AMD_HEAD_STASH_GIB", rnd.choice(["24", "0"]))
+        hidden, weight = torch.randn(n, h).to(dt), (torch.randn(v, h) * (2.0 / h**0.5)).to(dt)
+        bias = torch.randn(v).to(dt) if use_bias else None
+        labels, gout = torch.randint(0, v, (n,)), torch.randn(n)
+        if rnd.random() < 0.4:
+            gout[torch.rand(n) < 0.6] = 0.0
+        rh, rw = hidden.clone().float().requires_grad_(True), weight.clone().float().requires_grad_(True)
+        rb = bias.clone().float().requires_grad_(True) if use_bias else None
+        y = rh @ rw.t()
+        y = (y + rb if use_bias else y) * scale
+        if cap:
+            y = torch.tanh(y / cap) * cap
+        lsm = F.log_softmax(y / T, -1)
+        rlp, rent = lsm.gather(-1, labels[:, None]).squeeze(-1), -(lsm.exp() * lsm).sum(-1)
+        (rlp * gout).sum().backward()
+        dh, dw = hidden.clone().to(DEV).requires_grad_(True), weight.clone().to(DEV).requires_grad_(True)
+        db = bias.clone().to(DEV).requires_grad_(True) if use_bias else None
+        lp, ent = amd._ChunkedLogProbFunction.apply(dh, dw, labels.to(DEV), T, chunk, cap, scale, db)
+        (lp * gout.to(DEV)).sum().backward()
+        what = (case, n, h, v, chunk, str(dt), cap, use_bias, os.environ["TRL_AMD_HEAD_STASH_GIB"])
+        ftol = 1e-5 if dt == torch.float32 else 3e-3
+        assert float((lp.detach().cpu() - rlp.detach()).abs().max()) <= ftol * max(1.0, float(rlp.detach().abs().max())), what
+        assert float((ent.cpu() - rent.detach()).abs().max()) <= 4 * ftol, what
+        # (a vocabulary of a few entries is ill-conditioned: d logits = g (1 - p) cancels for a target of probability
+        # near 1, and the sums over tokens of a gradient of two or seven signed terms cancel again, so the rounding of
+        # the 16-bit d logits -- and fp32's own -- shows in the relative error of the result)
+        gtol = {torch.float32: 2e-5, torch.bfloat16: 1.2e-2, torch.float16: 2e-3}[dt]
+        if v < 16:
+            gtol = 2e-3 if dt == torch.float32 else 3e-2
+        pairs = [(dh.grad, rh.grad), (dw.grad, rw.grad)] + ([(db.grad, rb.grad)] if use_bias else [])
+        for got, want in pairs:
+            if float(gout.abs().max()) == 0.0:
+                assert float(got.float().abs().max()) == 0.0, what
+            else:
+                assert _rel(got, want) < gtol, (what, _rel(got, want))
+    amd.check_device_errors()
