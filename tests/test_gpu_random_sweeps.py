@@ -215,3 +215,57 @@ def test_fused_head_against_fp32_autograd(amd, monkeypatch):
             else:
                 assert _rel(got, want) < gtol, (what, _rel(got, want))
     amd.check_device_errors()
+
+
+def test_rloo_and_kto_losses_against_the_oracle(amd):
+    """150 RLOO problems (sequence-level clipped loss, its gradient and clip metrics) and 150 KTO problems (both loss
+    types, class weights, with and without the KL baseline, all-desirable and all-undesirable batches, fp32 / bf16)."""
+    rnd = random.Random(5)
+    torch.manual_seed(5)
+    for case in range(150):
+        B, T = rnd.choice([1, 2, 7, 16]), rnd.choice([1, 9, 40])
+        lp = -2 * torch.rand(B, T)
+        mask = (torch.arange(T)[None] < torch.randint(0, T + 1, (B,))[:, None]).float()
+        seq = (lp * mask).sum(1)
+        old = seq + rnd.choice([0.0, 0.1, 0.5]) * torch.randn(B)
+        adv = torch.randn(B)
+        eps = (rnd.choice([0.2, 0.1]), rnd.choice([0.2, 0.3]))
+        olp = lp.clone().requires_grad_(True)
+        oloss, om = oracle.rloo_loss(olp, mask, old, adv, *eps)
+        oloss.backward()
+        glp = lp.to(DEV).requires_grad_(True)
+        gloss, gseq, gm = amd.rloo_loss(glp, mask.to(DEV), old.to(DEV), adv.to(DEV), *eps)
+        gloss.backward()
+        assert abs(float(gloss.detach()) - float(oloss.detach())) <= 2e-5 * max(1.0, abs(float(oloss.detach()))), case
+        torch.testing.assert_close(gseq.detach().cpu(), seq, rtol=1e-5, atol=1e-5)
+        assert float((glp.grad.cpu() - olp.grad).abs().max()) <= 2e-5 * float(olp.grad.abs().max()) + 1e-7, case
+        want = [om["clip_ratio/low_mean"], om["clip_ratio/low_min"], om["clip_ratio/high_mean"], om["clip_ratio/high_max"],
+                om["clip_ratio/region_mean"]]
+        torch.testing.assert_close(gm[:5].cpu(), torch.tensor(want), rtol=1e-5, atol=1e-6, equal_nan=True)
+    for case in range(150):
+        B, L, V = rnd.choice([1, 2, 6]), rnd.choice([2, 7, 20]), rnd.choice([5, 64, 257])
+        dt = rnd.choice([torch.float32, torch.float32, torch.bfloat16])
+        logits = (2.0 * torch.randn(B, L, V)).to(dt)
+        ids = torch.randint(0, V, (B, L))
+        start = torch.randint(0, L, (B,))
+        cm = (torch.arange(L)[None] >= start[:, None]).long()
+        label = torch.rand(B) < rnd.choice([0.0, 0.5, 0.5, 1.0])
+        ref = -5 * torch.rand(B)
+        with_kl = rnd.random() < 0.6
+        kw = dict(kl_logps=-5 * torch.rand(B) if with_kl else None, ref_kl_logps=-5 * torch.rand(B) if with_kl else None,
+                  beta=rnd.choice([0.1, 0.5]), loss_type=rnd.choice(["kto", "apo_zero_unpaired"]),
+                  desirable_weight=rnd.choice([1.0, 1.33]), undesirable_weight=rnd.choice([1.0, 0.7]))
+        ol = logits.float().clone().requires_grad_(True)
+        oloss, _ = oracle.kto_compute_loss(ol, ids, cm, label, ref, **kw)
+        oloss.backward()
+        gl = logits.clone().to(DEV).requires_grad_(True)
+        gkw = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in kw.items()}
+        gloss, _ = amd.kto_compute_loss(gl, ids.to(DEV), cm.to(DEV), label.to(DEV), ref.to(DEV), **gkw)
+        gloss.backward()
+        what = (case, str(dt), kw["loss_type"], with_kl, label.tolist())
+        tol = 2e-5 if dt == torch.float32 else 2e-2
+        assert abs(float(gloss.detach()) - float(oloss.detach())) <= tol * max(1.0, abs(float(oloss.detach()))), what
+        if float(ol.grad.abs().max()) > 1e-10:
+            assert _rel(gl.grad.float(), ol.grad) <= (2e-4 if dt == torch.float32 else 2e-2), what
+        else:
+            assert gl.grad is None or float(gl.grad.float().abs().max()) <= 1e-7, what
