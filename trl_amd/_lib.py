@@ -1,6 +1,6 @@
 """ctypes binding of libtrlk.so (the C ABI declared in include/trlk.h).
 
-The library is built in-tree by `trl_amd.build` / `make -C trl_amd/csrc`; there is no
+The library is built in-tree by `python trl_amd/build.py` / `make -C trl_amd/csrc`; there is no
 fallback implementation: if it is missing, importing this module raises.
 `import torch` happens first on purpose, so that the HIP runtime torch ships is the one
 the kernels are enqueued on (stream handles and device pointers are shared with torch).
@@ -119,7 +119,7 @@ class TrlkArgumentError(ValueError):
 def _load():
     if not os.path.exists(LIB_PATH):
         raise ImportError(
-            f"{LIB_PATH} is missing: build the HIP kernels first (python -m trl_amd.build, or "
+            f"{LIB_PATH} is missing: build the HIP kernels first (python trl_amd/build.py, or "
             "make -C trl_amd/csrc). There is no fallback implementation."
         )
     lib = ctypes.CDLL(LIB_PATH)

@@ -1,4 +1,4 @@
-"""Builds trl_amd/lib/libtrlk.so with hipcc for gfx950 (`python -m trl_amd.build`)."""
+"""Builds trl_amd/lib/libtrlk.so with hipcc for gfx950 (`python trl_amd/build.py`: run as a script, because importing the package needs the library)."""
 from __future__ import annotations
 
 import os
