@@ -1172,20 +1172,41 @@ __global__ __launch_bounds__(256) void maxabs_f32_kernel(const float* in, int64_
 template <bool TO_F16>
 __global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* in, int64_t ld, int R, int C, uint16_t* out,
                                                           int64_t ldo, int64_t fill, const uint32_t* in_max) {
-    __shared__ uint16_t tile[64][66];
+    // C, ld, ldo and fill are multiples of 8 and both matrices 16-byte aligned (the callers' operands are): a lane
+    // moves 8 elements at a time.  Tile rows are skewed by 8 elements per group of 8 rows, which spreads the
+    // 2-byte column reads of the second phase over all banks.
+    constexpr int kStride = 136;
+    __shared__ __attribute__((aligned(16))) uint16_t tile[64 * kStride];
     const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
-    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int tid = threadIdx.x, hi = tid >> 3, lo = tid & 7;
     const float sc = TO_F16 ? slot_scale(in_max, 1.f) : 1.f;
-    for (int i = ty; i < 64; i += 4) {
-        const int r = r0 + i, c = c0 + tx;
-        uint16_t v = (r < R && c < C) ? in[int64_t(r) * ld + c] : uint16_t(0);
-        if (TO_F16) v = __builtin_bit_cast(uint16_t, _Float16(Elem<TRLK_BF16>::to_float(v) * sc));
-        tile[i][tx] = v;
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        const int row = hi + 32 * p, cc = lo * 8;
+        u32x4 q = {0u, 0u, 0u, 0u};
+        if (r0 + row < R && c0 + cc < C) q = *reinterpret_cast<const u32x4*>(in + int64_t(r0 + row) * ld + c0 + cc);
+        if (TO_F16) {
+            float x[8];
+            Elem<TRLK_BF16>::unpack(q, x);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[i] *= sc;
+            q = Elem<TRLK_F16>::pack(x);
+        }
+        *reinterpret_cast<u32x4*>(tile + row * kStride + cc + 8 * (row >> 3)) = q;
     }
     __syncthreads();
-    for (int i = ty; i < 64; i += 4) {
-        const int c = c0 + i, r = r0 + tx;
-        if (c < C && r < fill) out[int64_t(c) * ldo + r] = tile[tx][i];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        const int c = hi + 32 * p, r8 = lo;  // output row c0 + c, its columns r0 + 8 r8 .. + 7
+        if (c0 + c < C && r0 + r8 * 8 < fill) {
+            const uint16_t* src = tile + (r8 * 8) * kStride + c + 8 * r8;
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                w[i] = uint32_t(src[(2 * i) * kStride]) | (uint32_t(src[(2 * i + 1) * kStride]) << 16);
+            const u32x4 q = {w[0], w[1], w[2], w[3]};
+            *reinterpret_cast<u32x4*>(out + int64_t(c0 + c) * ldo + r0 + r8 * 8) = q;
+        }
     }
 }
 
