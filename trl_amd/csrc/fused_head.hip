@@ -1470,7 +1470,7 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     uint16_t* dz = reinterpret_cast<uint16_t*>(ws + l.off_dz);    // [N, cpad], row stride ld_c
     uint16_t* dzt = reinterpret_cast<uint16_t*>(ws + l.off_dzt);  // [cpad, npad], row stride ld_n
     float* dh = reinterpret_cast<float*>(ws + l.off_dh);          // [N, H]
-    uint32_t* maxima = reinterpret_cast<uint32_t*>(ws + l.off_max);  // [0] g, [1] hidden, [2 + i] chunk i of W
+    uint32_t* maxima = reinterpret_cast<uint32_t*>(ws + l.off_max);  // [0] g, [1] hidden, [2] W
     const int H = int(hidden_size), N = int(n_tokens), V = int(vocab);
     const bool from_bf16 = dtype == TRLK_BF16;  // the products' operands are fp16: bf16 inputs are converted on the way
     const uint32_t* max_g = maxima;
@@ -1482,6 +1482,9 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     if (from_bf16) {
         hipLaunchKernelGGL(maxabs_bf16_kernel, dim3(unsigned(N < 2048 ? N : 2048)), dim3(256), 0, s,
                            static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H / 8, maxima + 1);
+        // one scale for the whole weight: a single sweep over it instead of one per chunk
+        hipLaunchKernelGGL(maxabs_bf16_kernel, dim3(unsigned(V < 4096 ? V : 4096)), dim3(256), 0, s,
+                           static_cast<const uint16_t*>(d_weight), weight_stride, V, H / 8, maxima + 2);
         hipLaunchKernelGGL(transpose16_kernel<true>, dim3((H + 63) / 64, unsigned((l.npad + 63) / 64)), dim3(256), 0, s,
                            static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.ld_n, l.npad, max_h);
     } else {
@@ -1546,11 +1549,9 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         // W_chunk^T [H, kpad] (columns beyond the chunk's rows are zero): the chunk's own transposed copy keeps the
         // row stride of this operand as short as that of the other three
         const uint16_t* w_chunk = static_cast<const uint16_t*>(d_weight) + c0 * weight_stride;
-        const uint32_t* max_w = from_bf16 ? maxima + 2 + c0 / chunk : nullptr;
+        const uint32_t* max_w = from_bf16 ? maxima + 2 : nullptr;
         const dim3 tgrid((H + 63) / 64, unsigned((kpad + 63) / 64));
         if (from_bf16) {
-            hipLaunchKernelGGL(maxabs_bf16_kernel, dim3(unsigned(rows < 2048 ? rows : 2048)), dim3(256), 0, s, w_chunk,
-                               weight_stride, rows, H / 8, maxima + 2 + c0 / chunk);
             hipLaunchKernelGGL(transpose16_kernel<true>, tgrid, dim3(256), 0, s, w_chunk, weight_stride, rows, H, wt, l.ld_c,
                                int64_t(kpad), max_w);
         } else {
