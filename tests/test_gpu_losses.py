@@ -427,6 +427,96 @@ def test_golden_kto_compute_loss(amd, skip_masked):
             assert abs(value - want_m) <= tol, (case["name"], name, value, want_m)
 
 
+def test_kto_reference_pass_inside_the_loss(amd):
+    """Reference log-probs computed inside `_compute_loss` (kto_trainer.py:1532-1549): from `ref_model`, and from
+    the policy itself with its PEFT adapters switched off or switched to the adapter named "ref".  The stand-in
+    model answers with other logits while it is in its reference state; the loss must equal the one computed from
+    those logits' sequence log-probs handed in precomputed, and the model must be back in its training state."""
+    from contextlib import contextmanager
+
+    cases, g = load_golden("kto_compute_loss")
+    case = next(c for c in cases if c["kl"] and c["dtype"] == "float32")
+    c = f"c{case['id']}_"
+    leaf = _t(g[c + "logits"]).to(DEV)
+    kl_logits = _t(g[c + "kl_logits"]).to(DEV)
+    gen = torch.Generator().manual_seed(11)
+    ref_logits = (leaf.cpu() + 0.3 * torch.randn(leaf.shape, generator=gen)).to(DEV)
+    ref_kl_logits = (kl_logits.cpu() + 0.3 * torch.randn(kl_logits.shape, generator=gen)).to(DEV)
+    kl_len = case["kl_len"]
+    assert kl_len != leaf.shape[1]
+
+    class Trainer(amd.KTOLossMixin):
+        pass
+
+    tr = Trainer()
+    tr.accelerator = _Identity()
+    tr.accelerator.gather_for_metrics = lambda x: x
+    tr.accelerator.device = torch.device(DEV)
+    tr.aux_loss_enabled = False
+    tr.calculate_KL = True
+    tr.beta, tr.loss_type = case["beta"], case["loss_type"]
+    tr.desirable_weight, tr.undesirable_weight = case.get("desirable_weight", 1.0), case.get("undesirable_weight", 1.0)
+    tr._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
+    tr._total_train_tokens = 0
+    live = dict(input_ids=_t(g[c + "input_ids"]), attention_mask=_t(g[c + "attention_mask"]),
+                completion_mask=_t(g[c + "completion_mask"]), label=torch.tensor(case["labels"], dtype=torch.bool),
+                KL_input_ids=_t(g[c + "kl_input_ids"]), KL_attention_mask=_t(g[c + "kl_attention_mask"]),
+                KL_completion_mask=_t(g[c + "kl_completion_mask"]))
+
+    def answer(in_ref_state, input_ids):
+        is_kl = input_ids.shape[1] == kl_len
+        return SimpleNamespace(logits=(ref_kl_logits if is_kl else ref_logits) if in_ref_state else (kl_logits if is_kl else leaf),
+                               aux_loss=None)
+
+    ref_seq = amd.kto_sequence_logps(ref_logits, live["input_ids"].to(DEV), live["completion_mask"].to(DEV))
+    ref_kl_seq = amd.kto_sequence_logps(ref_kl_logits, live["KL_input_ids"].to(DEV), live["KL_completion_mask"].to(DEV))
+    tr.precompute_ref_logps = True
+    tr.model = SimpleNamespace(training=True)
+    want = tr._compute_loss(lambda input_ids=None, **kw: answer(False, input_ids),
+                            dict(live, ref_logps=ref_seq, ref_KL_logps=ref_kl_seq), False)
+    assert math.isfinite(float(want))
+
+    class FakePeft:
+        training = True
+
+        def __init__(self, adapters):
+            self.peft_config = {name: object() for name in adapters}
+            self.active_adapter = "default"
+            self.disabled = False
+            self.log = []
+
+        def set_adapter(self, name):
+            self.log.append(name)
+            self.active_adapter = name
+
+        @contextmanager
+        def disable_adapter(self):
+            self.disabled = True
+            self.log.append("off")
+            try:
+                yield
+            finally:
+                self.disabled = False
+                self.log.append("on")
+
+        def __call__(self, input_ids=None, **kw):
+            assert "output_router_logits" not in kw
+            return answer(self.disabled or self.active_adapter == "ref", input_ids)
+
+    tr.precompute_ref_logps = False
+    for adapters, trace in ((["default"], ["off", "on"]), (["default", "ref"], ["ref", "default"])):
+        peft = FakePeft(adapters)
+        tr.ref_model, tr.model = None, peft
+        got = tr._compute_loss(peft, live, False)
+        assert torch.equal(got, want) and peft.log == trace and peft.active_adapter == "default" and not peft.disabled
+    tr.ref_model = lambda input_ids=None, **kw: answer(True, input_ids)
+    tr.model = SimpleNamespace(training=True)
+    assert torch.equal(tr._compute_loss(lambda input_ids=None, **kw: answer(False, input_ids), live, False), want)
+    tr.ref_model = None
+    with pytest.raises(ValueError, match="reference log-probs"):
+        tr._compute_loss(lambda input_ids=None, **kw: answer(False, input_ids), live, False)
+
+
 def test_golden_dpo_compute_loss(amd):
     """The fused sigmoid path (one loss kernel) on the plain sigmoid cases."""
     cases, g = load_golden("dpo_compute_loss")

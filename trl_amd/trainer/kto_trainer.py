@@ -7,6 +7,7 @@ import torch
 from torch import Tensor
 
 from .. import ops
+from .dpo_trainer import _reference_adapter
 
 __all__ = ["kto_sequence_logps", "kto_compute_loss", "KTOLossMixin"]
 
@@ -128,12 +129,22 @@ class KTOLossMixin:
             ref_logps = batch["ref_logps"]
             ref_kl = batch["ref_KL_logps"] if self.calculate_KL else None
         else:
-            if getattr(self, "ref_model", None) is None:
-                raise NotImplementedError("reference log-probs from a PEFT adapter switch are not implemented by trl_amd")
             ref_kwargs = {k: v for k, v in model_kwargs.items() if k != "output_router_logits"}
-            ref_kl = self._compute_kl_logps(self.ref_model, batch)
-            with torch.no_grad():
-                ref_logits = self.ref_model(**ref_kwargs).logits
+            if getattr(self, "ref_model", None) is not None:
+                ref_kl = self._compute_kl_logps(self.ref_model, batch)
+                with torch.no_grad():
+                    ref_logits = self.ref_model(**ref_kwargs).logits
+            else:
+                # adapter training without a separate reference model: the same network with its adapters switched
+                # off, or with the frozen copy named "ref" active (kto_trainer.py:1534-1541)
+                peft_model = acc.unwrap_model(self.model)
+                if not hasattr(peft_model, "peft_config"):
+                    raise ValueError("KTO needs reference log-probs: precomputed, from `ref_model`, or from a PEFT "
+                                     "model whose adapters can be switched off")
+                with _reference_adapter(peft_model):
+                    ref_kl = self._compute_kl_logps(self.model, batch)
+                    with torch.no_grad():
+                        ref_logits = self.model(**ref_kwargs).logits
             ref_logps = kto_sequence_logps(ref_logits, batch["input_ids"], batch["completion_mask"])
         loss, parts = kto_compute_loss(
             outputs.logits, batch["input_ids"], batch["completion_mask"], batch["label"], ref_logps, kl_logps, ref_kl,
