@@ -15,7 +15,8 @@ headline step: algorithmic bytes per launch / average launch time, measured live
 launches of that kernel alone; `step_hbm_GBps` prices the whole step by the bytes its kernels move.
 `cpu_baseline` times the CPU oracle (a port of the reference path, oracle/) on a bounded row sample of the same
 workload on this host's cores.  Without `--workload` the line also carries `secondary`: the other loss types of the
-headline workload and the other benchmark configurations (long context, DPO, fused head), each with its step time,
+headline workload and the other benchmark configurations (fused head, long context, DPO, and the fp32 forward-only
+configuration small enough for the host to run whole), each with its step time,
 its dominant kernel's roofline figures and -- where the one-pass kernel runs -- the relative L2 distance between its
 gradient and the two-pass gradient.
 """
@@ -62,6 +63,8 @@ WORKLOADS = {
     "dpo_c2": dict(B=64, T=2048, V=128256, beta=0.1, dpo=True,
                    desc="DPO sequence log-probs + sigmoid loss fwd+bwd, bf16 logits [64,2048,128256], 32 pairs, "
                         "prompt~U[64,512], completion~U[128,1536]"),
+    "logp_c1": dict(B=8, T=256, V=32000, logp=True,
+                    desc="selective_log_softmax + entropy_from_logits forward, fp32 logits [8,256,32000] = 3*randn (seed 0)"),
     "tiny": dict(B=8, T=64, V=151936, temperature=0.9, G=8, min_len=8, beta=0.04, eps_low=0.2, eps_high=0.2,
                  rewards="normal", desc="reduced-size functional check (not a benchmark configuration)"),
 }
@@ -429,6 +432,76 @@ def bench_dpo(args, w):
     return result
 
 
+def bench_logp_c1(args, w):
+    """Config 1, the reference's CPU-runnable case: per-token log-probs and entropies of fp32 logits, forward only.
+    The inputs come from a CPU generator, so the oracle on the host sees the same bits and the whole output is
+    compared with it (1e-5, against its fp64 evaluation) before anything is timed.  The 262 MB of logits would stay in the memory-side cache
+    between launches: the timed launches rotate over eight copies."""
+    import oracle
+    import trl_amd
+    from trl_amd import ops
+
+    dev = torch.device("cuda:0")
+    B, T, V = w["B"], w["T"], w["V"]
+    R = B * T
+    g = torch.Generator().manual_seed(0)
+    host_logits = 3.0 * torch.randn((B, T, V), generator=g)
+    host_ids = torch.randint(0, V, (B, T), generator=g)
+    torch.set_num_threads(os.cpu_count() or 1)
+    best = float("inf")
+    for _ in range(3):
+        t0 = time.perf_counter()
+        want_lp = oracle.selective_log_softmax(host_logits, host_ids)
+        want_h = oracle.entropy_from_logits(host_logits)
+        best = min(best, time.perf_counter() - t0)
+    # parity against the same functions in fp64 (the fp32 host result carries ~2e-5 of summation error itself)
+    want_lp = oracle.selective_log_softmax(host_logits.double(), host_ids)
+    want_h = oracle.entropy_from_logits(host_logits.double())
+    copies = [host_logits.to(dev) for _ in range(8)]
+    ids = host_ids.to(dev)
+    lp, ent = trl_amd.logps_and_entropies(copies[0], ids)
+    err_lp = float((lp.cpu().double() - want_lp).abs().max())
+    err_h = float((ent.cpu().double() - want_h).abs().max())
+    assert err_lp <= 1e-5 and err_h <= 1e-5, (err_lp, err_h)
+    idx = ids.reshape(R, 1)
+
+    def timed(fn, reps):
+        for c in copies:
+            fn(c)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        a.record()
+        for i in range(reps):
+            fn(copies[i % len(copies)])
+        b.record()
+        torch.cuda.synchronize()
+        return max((time.perf_counter() - t0) * 1e3, a.elapsed_time(b)) / reps, a.elapsed_time(b) / reps
+
+    reps = max(args.steps, 10) * 8
+    ms_step, _ = timed(lambda x: trl_amd.logps_and_entropies(x, ids), reps)
+    ms_two, _ = timed(lambda x: (trl_amd.selective_log_softmax(x, ids), trl_amd.entropy_from_logits(x)), reps)
+    _, ms_kernel = timed(lambda x: ops.logp_entropy_fwd(x, idx, 1.0, 0, T, None), reps)
+    nbytes = R * V * 4
+    gbps = nbytes / (ms_kernel * 1e-3) / 1e9
+    return {
+        "metric": "tokens/sec + achieved HBM TB/s (% of peak) for log-prob + entropy forward",
+        "value": R / (ms_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": reps, "warmup": len(copies),
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "description": w["desc"], "rows": R, "vocab": V,
+                   "max_abs_err_logps_vs_oracle": err_lp, "max_abs_err_entropy_vs_oracle": err_h},
+        "roofline": {"bound": "hbm", "kernel": "logp_entropy_fwd_kernel (K1)", "achieved": gbps, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "algorithmic_bytes": nbytes,
+                     "avg_launch_ms": ms_kernel,
+                     "note": "back-to-back launches over eight copies of the logits (each launch reads cold data)"},
+        "two_calls_ms_per_step": ms_two,
+        "cpu_baseline": {"value": R / best, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+                         "sample": f"oracle selective_log_softmax + entropy_from_logits on the full configuration, "
+                                   f"best of 3, {best:.3f} s; torch {torch.__version__} CPU"},
+    }
+
+
 def _grad_distance(run_a, run_b, leaf):
     """Relative L2 distance between the gradients two step functions leave in `leaf.grad`, accumulated sequence
     by sequence (no logits-sized fp32 temporaries)."""
@@ -686,6 +759,11 @@ def _brief(r):
         out["mask_aware_ms_per_step"] = r["mask_aware"]["ms_per_step"]
     if "kernels" in r:
         out["kernels"] = {k: v for k, v in r["kernels"].items() if isinstance(v, dict) and ("frac" in v or "avg_ms" in v)}
+    if r["config"]["workload"] == "logp_c1":  # small enough for the host to run whole: its own baseline and parity
+        out["cpu_baseline"] = r["cpu_baseline"]
+        out["two_calls_ms_per_step"] = r["two_calls_ms_per_step"]
+        out["max_abs_err_vs_oracle"] = max(r["config"]["max_abs_err_logps_vs_oracle"],
+                                           r["config"]["max_abs_err_entropy_vs_oracle"])
     return out
 
 
@@ -715,6 +793,8 @@ def main():
         return print(json.dumps(bench_head(args, w)))
     if w.get("dpo"):
         return print(json.dumps(bench_dpo(args, w)))
+    if w.get("logp"):
+        return print(json.dumps(bench_logp_c1(args, w)))
     result, shared = bench_grpo(args, w, args.loss_type)
     secondary = []
     if secondary_wanted:
@@ -728,10 +808,11 @@ def main():
     if secondary_wanted:
         # (the matrix-core workload first: its clock is set by the power budget and falls as the part warms up,
         # the streaming workloads are bound by memory and hardly notice)
-        for name in ("head_c5", "grpo_c4", "dpo_c2"):
+        for name in ("head_c5", "grpo_c4", "dpo_c2", "logp_c1"):
             few.workload = name
             w2 = WORKLOADS[name]
-            r = bench_head(few, w2) if w2.get("head") else bench_dpo(few, w2) if w2.get("dpo") else bench_grpo(few, w2, "dapo")[0]
+            r = (bench_head(few, w2) if w2.get("head") else bench_dpo(few, w2) if w2.get("dpo")
+                 else bench_logp_c1(few, w2) if w2.get("logp") else bench_grpo(few, w2, "dapo")[0])
             secondary.append(_brief(r))
             del r
             torch.cuda.empty_cache()
