@@ -484,25 +484,35 @@ __device__ __forceinline__ int acc_col(int wn, int nb, int lane) { return wn * W
 // as many a tiles per XCD as n_a needs, so that (almost) no workgroup of the grid is empty: the
 // hardware deals workgroups to the CUs in order, and with empty ones interleaved at a fixed stride
 // the real ones end up on a fraction of the CUs (measured: a third more time for 65 instead of 64
-// a tiles with a grid padded to whole bands).  The caller skips ta >= n_a.
+// a tiles with a grid padded to whole bands).  The n_a % 8 a tiles that are left when every XCD has
+// the same number are not given to that many XCDs whole (one XCD in eight would then carry an a
+// tile more than the others and the launch would wait for it): their n_b tiles each are dealt out
+// in equal runs over all eight XCDs, a innermost.  The caller skips ta >= n_a or tb >= n_b.
 __device__ __forceinline__ void xcd_patch(int w, int n_a, int n_b, int& ta, int& tb) {
     const int xcd = w & 7, q = w >> 3;
-    const int bands = n_a >> 5;                    // full bands of 32 a tiles
+    const int groups = n_a >> 3;                   // a tiles every XCD owns whole
+    const int bands = groups >> 2;                 // full bands of 4 of them
     const int full = bands * 4 * n_b;              // workgroups of this XCD in the full bands
+    const int m = groups & 3;                      // whole a tiles per XCD in the last band
     if (q < full) {
         const int rem = q % (4 * n_b);
         tb = rem >> 2;
         ta = ((q / (4 * n_b)) * 4 + (rem & 3)) * 8 + xcd;
-    } else {
-        const int m = (n_a - bands * 32 + 7) >> 3;  // a tiles per XCD in the last band (1..4; 0 = no last band)
+    } else if (q < full + m * n_b) {
         const int qq = q - full;
-        tb = m > 0 ? qq / m : n_b;
-        ta = (bands * 4 + (m > 0 ? qq % m : 0)) * 8 + xcd;
+        tb = qq / m;
+        ta = (bands * 4 + qq % m) * 8 + xcd;
+    } else {
+        const int r = n_a & 7, left = r * n_b;     // the a tiles that are left, and their tiles
+        const int share = (left + 7) >> 3;
+        const int t = xcd * share + (q - full - m * n_b);
+        const bool real = q - full - m * n_b < share && t < left;
+        ta = real ? groups * 8 + t % r : n_a;      // a innermost, as in the bands: neighbours share the b slab
+        tb = real ? t / r : n_b;
     }
 }
 inline int xcd_patch_grid(int n_a, int n_b) {
-    const int bands = n_a / 32, m = (n_a - bands * 32 + 7) / 8;
-    return 8 * (bands * 4 + m) * n_b;
+    return 8 * ((n_a / 8) * n_b + ((n_a % 8) * n_b + 7) / 8);
 }
 
 struct HeadArgs {
