@@ -24,6 +24,11 @@ def amd():
     return trl_amd
 
 
+def _amax(x):
+    """Largest magnitude, 0 for an empty tensor."""
+    return float(x.abs().max()) if x.numel() else 0.0
+
+
 def _rel(a, b):
     a, b = a.double().cpu(), b.double().cpu()
     return float((a - b).norm() / b.norm().clamp(min=1e-30))
@@ -75,6 +80,69 @@ def test_grpo_loss_kernel_against_the_oracle(amd):
             assert float((ge - oent.grad).abs().max()) <= 2e-5 * float(oent.grad.abs().max()) + 1e-8, what
         ran += 1
     assert ran >= 200
+
+
+def test_logprob_kernels_against_fp64(amd):
+    """400 problems through `logps_and_entropies` and its gradient: fp32 / bf16 / fp16 / fp64 logits, vocabularies
+    that are and are not multiples of the vector width, one to three indices per row, a window of the rows, views
+    with strides in both leading dimensions, row masks, temperatures; the reference is torch's log_softmax in fp64
+    on the stored values, forward and autograd."""
+    rnd = random.Random(7)
+    torch.manual_seed(7)
+    for case in range(400):
+        n_seq, length = rnd.choice([1, 2, 3]), rnd.choice([1, 2, 5, 9])
+        V = rnd.choice([1, 2, 7, 8, 33, 256, 257, 1000, 4096, 4099, 20488])
+        dt = rnd.choice([torch.float32, torch.float32, torch.bfloat16, torch.float16, torch.float64])
+        K = rnd.choice([0, 1, 1, 2, 3])  # 0: index without the trailing axis
+        T = rnd.choice([1.0, 0.7, 1.3])
+        keep_start = rnd.randrange(0, length)
+        keep_len = rnd.randrange(0, length - keep_start + 1)
+        scale = rnd.choice([0.5, 3.0, 8.0])
+        pad0, pad1 = rnd.choice([0, 1]), rnd.choice([0, 2])
+        big = (scale * torch.randn(n_seq + pad0, length + pad1, V, device=DEV)).to(dt)
+        view = big[pad0:, pad1 // 2 : pad1 // 2 + length]  # strides of the larger tensor
+        leaf = view.detach().clone().requires_grad_(True) if rnd.random() < 0.3 else None
+        src = leaf if leaf is not None else view.detach().requires_grad_(True)
+        shape = (n_seq, keep_len) if K == 0 else (n_seq, keep_len, K)
+        index = torch.randint(0, V, shape, device=DEV)
+        row_mask = (torch.rand(n_seq, keep_len, device=DEV) < 0.6) if rnd.random() < 0.3 else None
+        logp, ent = amd.logps_and_entropies(src, index, T, keep_start, keep_len, row_mask)
+        assert logp.shape == shape and ent.shape == (n_seq, keep_len)
+        out_dt = torch.float64 if dt == torch.float64 else torch.float32
+        assert logp.dtype == out_dt and ent.dtype == out_dt
+        ref_src = view.detach().double().requires_grad_(True)
+        z = ref_src[:, keep_start : keep_start + keep_len] / T
+        lsm = F.log_softmax(z, dim=-1)
+        want_lp = lsm.gather(-1, index if K else index.unsqueeze(-1))
+        want_lp = want_lp if K else want_lp.squeeze(-1)
+        want_h = -(lsm.exp() * lsm).sum(-1)
+        live = torch.ones(n_seq, keep_len, dtype=torch.bool, device=DEV) if row_mask is None else row_mask
+        what = (case, str(dt), V, K, T, keep_start, keep_len, pad0, pad1, row_mask is not None)
+        tol = 1e-12 if dt == torch.float64 else 2e-5
+        zmax = float(z.detach().abs().max()) if z.numel() else 0.0
+        if keep_len:
+            lm = live if K == 0 else live.unsqueeze(-1).expand(shape)
+            assert _amax((logp.detach().double() - want_lp.detach())[lm]) <= tol * max(1.0, zmax), what
+            assert _amax((ent.detach().double() - want_h.detach())[live]) <= tol * max(1.0, zmax) + (0 if dt == torch.float64 else 2.5e-7 * zmax), what
+            if row_mask is not None:  # skipped rows come back as exact zeros
+                assert _amax(logp.detach()[~lm]) == 0.0 and _amax(ent.detach()[~live]) == 0.0, what
+        g_lp = torch.randn(shape, device=DEV, dtype=torch.float64)
+        g_h = torch.randn(n_seq, keep_len, device=DEV, dtype=torch.float64) * (0.0 if rnd.random() < 0.5 else 1.0)
+        lmask = live.double() if K == 0 else live.double().unsqueeze(-1)
+        ((logp.double() * g_lp * lmask).sum() + (ent.double() * g_h * live.double()).sum()).backward()
+        ((want_lp * g_lp * lmask).sum() + (want_h * g_h * live.double()).sum()).backward()
+        got = src.grad
+        assert got.shape == view.shape and got.dtype == dt, what
+        want = ref_src.grad
+        bar = {torch.float64: 1e-12, torch.float32: 2e-5, torch.bfloat16: 4e-3, torch.float16: 2e-3}[dt]
+        if float(want.abs().max()) == 0.0:  # (a one-entry vocabulary has no gradient; rounding may leave g * (1 - p))
+            assert _amax(got.double()) <= bar * (_amax(g_lp) + _amax(g_h)), what
+        else:
+            assert _rel(got, want) <= bar, (what, _rel(got, want))
+        outside = torch.ones(length, dtype=torch.bool, device=DEV)
+        outside[keep_start : keep_start + keep_len] = False
+        assert _amax(got[:, outside].double()) == 0.0, what  # rows outside the window: exact zeros
+    amd.check_device_errors()
 
 
 def test_single_pass_kernel_against_the_two_pass_path(amd):

@@ -53,14 +53,14 @@ def logps_and_entropies(
     if keep_start < 0 or keep_len < 0 or keep_start + keep_len > length:
         raise ValueError(f"rows [{keep_start}, {keep_start + keep_len}) are outside the {length} rows of the logits")
     squeeze = index.dim() == 2
-    idx = index.reshape(n_seq * keep_len, -1)
+    idx = index.reshape(n_seq * keep_len, 1 if squeeze else index.shape[-1])
     if idx.dtype != torch.int64:
         idx = idx.long()
     rm = None
     if row_mask is not None:
         rm = (row_mask.reshape(-1) != 0).to(torch.uint8).contiguous()
     logp, ent, _ = ops.logp_entropy_forward(logits, idx, float(temperature), keep_start, keep_len, rm)
-    logp = logp.view(n_seq, keep_len) if squeeze else logp.view(n_seq, keep_len, -1)
+    logp = logp.view(n_seq, keep_len) if squeeze else logp.view(n_seq, keep_len, index.shape[-1])
     return logp, ent.view(n_seq, keep_len)
 
 
