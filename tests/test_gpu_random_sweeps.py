@@ -145,6 +145,88 @@ def test_logprob_kernels_against_fp64(amd):
     amd.check_device_errors()
 
 
+def test_drop_in_functions_at_any_shape(amd):
+    """300 calls of `selective_log_softmax` / `entropy_from_logits` as the reference's callers make them: logits
+    of one to four dimensions, views whose leading dimensions are strided or permuted, index with and without a
+    trailing axis, every float dtype; results in the logits' dtype (one rounding of the fp32 value for 16-bit
+    logits) against torch in fp64, gradients against fp64 autograd."""
+    rnd = random.Random(8)
+    torch.manual_seed(8)
+    ulp = {torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}
+    for case in range(300):
+        lead = rnd.choice([(), (5,), (3, 4), (2, 3, 2), (1, 1), (4, 1)])
+        V = rnd.choice([2, 8, 41, 768, 1000, 4099])
+        dt = rnd.choice([torch.float32, torch.float32, torch.bfloat16, torch.float16, torch.float64])
+        base = (rnd.choice([1.0, 4.0]) * torch.randn(*lead, V, device=DEV)).to(dt)
+        how = rnd.choice(["plain", "permute", "slice"]) if len(lead) >= 2 else "plain"
+        if how == "permute":
+            perm = list(range(len(lead)))
+            rnd.shuffle(perm)
+            inv = [perm.index(i) for i in range(len(lead))]
+            view = base.permute(*perm, len(lead)).contiguous().permute(*inv, len(lead))  # same values, permuted strides
+        elif how == "slice":
+            big = torch.cat([base, base], dim=0)
+            view = big[::2] if lead[0] > 1 else big[:1]
+            base = view.clone()
+        else:
+            view = base
+        K = rnd.choice([None, 1, 3])
+        index = torch.randint(0, V, lead + (() if K is None else (K,)), device=DEV)
+        leaf = view.detach().requires_grad_(True)
+        got_lp = amd.selective_log_softmax(leaf, index)
+        got_h = amd.entropy_from_logits(leaf, chunk_size=rnd.choice([1, 16, 128]))
+        assert got_lp.shape == index.shape and got_h.shape == lead and got_lp.dtype == dt and got_h.dtype == dt
+        ref = base.detach().double().requires_grad_(True)
+        lsm = F.log_softmax(ref, dim=-1)
+        want_lp = lsm.gather(-1, index.unsqueeze(-1)).squeeze(-1) if K is None else lsm.gather(-1, index)
+        want_h = -(lsm.exp() * lsm).sum(-1)
+        what = (case, lead, V, str(dt), how, K)
+        for got, want in ((got_lp, want_lp), (got_h, want_h)):
+            err = (got.detach().double() - want.detach()).abs()
+            if dt == torch.float64:
+                assert _amax(err) <= 1e-12, what
+            elif dt == torch.float32:
+                assert _amax(err) <= 2e-5, what
+            else:  # one rounding of a value that is itself good to 2e-5
+                assert bool((err <= 0.5 * ulp[dt] * want.detach().abs().clamp(min=2.0**-14) * 2 + 2e-5).all()), what
+        g_lp, g_h = torch.randn(index.shape, device=DEV, dtype=torch.float64), torch.randn(lead, device=DEV, dtype=torch.float64)
+        ((got_lp.double() * g_lp).sum() + (got_h.double() * g_h).sum()).backward()
+        ((want_lp * g_lp).sum() + (want_h * g_h).sum()).backward()
+        assert leaf.grad.shape == view.shape and leaf.grad.dtype == dt
+        # 16-bit: the upstream gradients reach the kernel rounded to the outputs' dtype, then one rounding of dlogits
+        bar = {torch.float64: 1e-12, torch.float32: 2e-5, torch.bfloat16: 8e-3, torch.float16: 2e-3}[dt]
+        assert _rel(leaf.grad, ref.grad) <= bar, (what, _rel(leaf.grad, ref.grad))
+    amd.check_device_errors()
+
+
+def test_advantages_against_the_oracle(amd):
+    """300 reward vectors through the group-advantage kernel and the leave-one-out baseline: group sizes 1 ... 16,
+    the three scaling modes, NaN rewards (single ones, whole groups), constant groups; against the oracle."""
+    rnd = random.Random(9)
+    torch.manual_seed(9)
+    for case in range(300):
+        G = rnd.choice([1, 2, 3, 8, 16])
+        n_groups = rnd.choice([1, 2, 5, 32])
+        rewards = rnd.choice([1.0, 100.0]) * torch.randn(G * n_groups)
+        if rnd.random() < 0.3:
+            rewards = torch.bernoulli(torch.full((G * n_groups,), 0.3))
+        if rnd.random() < 0.4:
+            rewards[torch.rand(G * n_groups) < 0.2] = float("nan")
+        if rnd.random() < 0.2:
+            rewards.view(n_groups, G)[rnd.randrange(n_groups)] = float("nan")
+        if rnd.random() < 0.2:
+            rewards.view(n_groups, G)[rnd.randrange(n_groups)] = 0.5
+        mode = rnd.choice(["group", "batch", "none"])
+        got = amd.group_advantages(rewards.to(DEV), G, mode).cpu()
+        want = oracle.group_advantages(rewards, G, mode)
+        torch.testing.assert_close(got, want, rtol=2e-5, atol=2e-5, msg=lambda m: f"{(case, G, n_groups, mode)}: {m}")
+        assert bool((got[want == 0] == 0).all())  # constant and unscorable groups: exactly zero
+        norm = rnd.random() < 0.5
+        got = amd.rloo_advantages(rewards.to(DEV), G, norm).cpu()
+        want = oracle.rloo_advantages(rewards, G, norm)
+        torch.testing.assert_close(got, want, rtol=2e-5, atol=2e-5, msg=lambda m: f"{(case, G, n_groups, norm)}: {m}")
+
+
 def test_single_pass_kernel_against_the_two_pass_path(amd):
     """250 configurations the single-pass kernel takes (loss types, KL, delta, bias-corrected KL, token weights,
     per-token advantages, entropy bonus, temperatures, bf16 / fp16, vocabularies 8 ... 20488, empty sequences, ragged
