@@ -367,6 +367,52 @@ def test_fused_head_against_fp32_autograd(amd, monkeypatch):
     amd.check_device_errors()
 
 
+def test_sft_chunked_loss_against_the_oracle(amd):
+    """120 problems through the SFT `chunked_nll` loss: labels or pre-shifted labels with -100 holes (all of them
+    in some), bias, logit scale, soft-capping, `num_items_in_batch`, bf16 / fp16 / fp32 operands; loss, argmax
+    count, entropy sum and the gradients of hidden states, weight and bias against the oracle's autograd."""
+    from trl_amd.trainer.sft_trainer import _chunked_cross_entropy_loss
+
+    rnd = random.Random(10)
+    torch.manual_seed(10)
+    for case in range(120):
+        B, S, H, V = rnd.choice([1, 2, 3]), rnd.choice([2, 7, 33]), rnd.choice([8, 64, 72]), rnd.choice([8, 250, 256, 1000])
+        dt = rnd.choice([torch.float32, torch.bfloat16, torch.float16])
+        hidden = torch.randn(B, S, H)
+        weight = rnd.choice([0.05, 0.3]) * torch.randn(V, H)
+        bias = 0.5 * torch.randn(V) if rnd.random() < 0.3 else None
+        labels = torch.randint(0, V, (B, S))
+        labels[torch.rand(B, S) < rnd.choice([0.0, 0.3, 1.0])] = -100
+        shifted = rnd.random() < 0.4
+        kw = dict(logit_scale=rnd.choice([1.0, 1.0, 0.5]), final_logit_softcapping=rnd.choice([None, None, 5.0]),
+                  num_items_in_batch=rnd.choice([None, 17, torch.tensor(23.0)]))
+        lab_kw = dict(shift_labels=labels) if shifted else dict(labels=labels)
+        q = lambda t: None if t is None else t.to(dt)  # noqa: E731
+        dev_in = [q(hidden).to(DEV).requires_grad_(True), q(weight).to(DEV).requires_grad_(True),
+                  None if bias is None else q(bias).to(DEV).requires_grad_(True)]
+        host_in = [q(hidden).float().requires_grad_(True), q(weight).float().requires_grad_(True),
+                   None if bias is None else q(bias).float().requires_grad_(True)]
+        got = _chunked_cross_entropy_loss(dev_in[0], dev_in[1], rnd.choice([16, 4096]), lm_head_bias=dev_in[2],
+                                          **{k: v.to(DEV) for k, v in lab_kw.items()}, **kw)
+        want = oracle.chunked_cross_entropy_loss(host_in[0], host_in[1], 64, lm_head_bias=host_in[2], **lab_kw, **kw)
+        what = (case, B, S, H, V, str(dt), shifted, bias is not None, kw["logit_scale"], kw["final_logit_softcapping"])
+        assert int(got[3]) == int(want[3]), what
+        low = dt != torch.float32
+        assert abs(float(got[0].detach()) - float(want[0].detach())) <= (2e-4 if low else 2e-5) * max(1.0, abs(float(want[0].detach()))), what
+        assert abs(float(got[2].detach()) - float(want[2].detach())) <= (2e-4 if low else 2e-5) * max(1.0, abs(float(want[2].detach()))), what
+        assert abs(float(got[1].detach()) - float(want[1].detach())) <= (1 if low else 0), what  # (a near-tie may flip under 16-bit products)
+        got[0].backward()
+        want[0].backward()
+        for g_t, w_t, name in zip(dev_in, host_in, ("hidden", "weight", "bias")):
+            if g_t is None:
+                continue
+            if float(w_t.grad.abs().max()) == 0.0:
+                assert g_t.grad is None or float(g_t.grad.float().abs().max()) == 0.0, (what, name)
+            else:
+                assert _rel(g_t.grad, w_t.grad) <= (6e-3 if dt == torch.bfloat16 else 1e-3 if low else 2e-5), (what, name, _rel(g_t.grad, w_t.grad))
+    amd.check_device_errors()
+
+
 def test_rloo_and_kto_losses_against_the_oracle(amd):
     """150 RLOO problems (sequence-level clipped loss, its gradient and clip metrics) and 150 KTO problems (both loss
     types, class weights, with and without the KL baseline, all-desirable and all-undesirable batches, fp32 / bf16)."""
