@@ -96,12 +96,20 @@ def dpo_compute_loss(
     rm = (smask.reshape(-1) != 0).to(torch.uint8).contiguous() if skip_masked_rows else None
     logp, ent, _, stats = ops.logp_entropy_stats_fwd(logits, idx, 1.0, 0, length - 1, rm)
     m = smask.to(torch.float32)
-    tok = logp.view(n_seq, length - 1) * m
     ent = ent.view(n_seq, length - 1).detach()
     stats = stats.view(n_seq, length - 1, 4).detach()
+    ref_c, ref_r = ref_chosen_logps.to(torch.float32), ref_rejected_logps.to(torch.float32)
+    ls = float(label_smoothing)
+    if (tuple(loss_types) == ("sigmoid",) and ls == 0.0 and ld_alpha is None and not use_weighting
+            and f_divergence_type == "reverse_kl" and (loss_weights is None or [float(x) for x in loss_weights] == [1.0])):
+        # the default configuration: masked sequence sums, loss and d loss / d log-prob from one loss kernel
+        loss, seq, _, _ = ops.dpo_loss_op(logp.view(n_seq, length - 1), m, ref_c, ref_r, float(beta))
+        chosen, rejected = seq.detach().chunk(2)
+        return loss, _dpo_metric_parts(ent, stats, m, chosen, rejected, ref_c, ref_r, beta)
+    tok = logp.view(n_seq, length - 1) * m
 
     if ld_alpha is None:
-        seq = tok.sum(dim=1)
+        seq = _masked_row_sums(logp.view(n_seq, length - 1), m)
     else:  # tokens beyond the shorter completion of a pair count with weight ld_alpha (:1351-1361)
         pos = smask.cumsum(dim=1)
         lens = smask.sum(dim=1)
@@ -110,12 +118,10 @@ def dpo_compute_loss(
         tail = (pos > shared).to(torch.float32)
         seq = (tok * head).sum(dim=1) + ld_alpha * (tok * tail).sum(dim=1)
     chosen, rejected = seq.chunk(2)
-    ref_c, ref_r = ref_chosen_logps.to(torch.float32), ref_rejected_logps.to(torch.float32)
     c_lr, r_lr = chosen - ref_c, rejected - ref_r
     c_sc, r_sc = _f_divergence_scores(c_lr, r_lr, f_divergence_type, f_alpha_divergence_coef)
     d = c_sc - r_sc
     c_n, r_n = (x.to(torch.float32).sum(dim=1).clamp(min=1.0) for x in completion_mask.chunk(2))
-    ls = float(label_smoothing)
 
     def smoothed(delta):
         return -F.logsigmoid(beta * delta) * (1 - ls) - F.logsigmoid(-beta * delta) * ls
@@ -169,18 +175,33 @@ def dpo_compute_loss(
             term = term * pair_weight
         loss = loss + term.mean() * lw
 
-    with torch.no_grad():
-        cm, rmk = m.chunk(2)
-        c_rew, r_rew = beta * c_lr.detach(), beta * r_lr.detach()
-        metrics = {
-            "entropy_sum": (ent * m).sum(), "n_tokens": m.sum(),
-            "logits_chosen_sum": (stats[..., 0].chunk(2)[0] * cm).sum(), "n_chosen_tokens": cm.sum(),
-            "logits_rejected_sum": (stats[..., 0].chunk(2)[1] * rmk).sum(), "n_rejected_tokens": rmk.sum(),
-            "correct_tokens": (stats[..., 2].chunk(2)[0] * cm).sum(),
-            "chosen_rewards": c_rew, "rejected_rewards": r_rew,
-            "chosen_logps": chosen.detach(), "rejected_logps": rejected.detach(),
-        }
-    return loss, metrics
+    return loss, _dpo_metric_parts(ent, stats, m, chosen.detach(), rejected.detach(), ref_c, ref_r, beta)
+
+
+def _masked_row_sums(token_logps: Tensor, mask: Tensor) -> Tensor:
+    """`[2P]` sums of the log-probs inside the mask, from the loss kernel's own row reduction (differentiable).  Every
+    place that sums a sequence uses this one order of summation: reference log-probs taken from the same logits then
+    cancel the policy's exactly, and the first step of a run starts at ln 2 as it does in the reference."""
+    zero = token_logps.new_zeros((token_logps.shape[0] // 2,), dtype=torch.float32)
+    return ops.dpo_loss_op(token_logps, mask, zero, zero, 1.0)[1]
+
+
+@torch.no_grad()
+def _dpo_metric_parts(ent, stats, m, chosen, rejected, ref_c, ref_r, beta):
+    """The parts of the logged metrics (dpo_trainer.py:1587-1653) as device scalars / `[P]` vectors: masked sums of
+    the entropies, the mean logits and the arg-max hits per half of the batch, from one stacked reduction."""
+    n_seq = m.shape[0]
+    vals = torch.stack((ent, stats[..., 0], stats[..., 2], torch.ones_like(ent)), dim=0)  # [4, 2P, L-1]
+    halves = (vals * m).view(4, 2, (n_seq // 2) * m.shape[1]).sum(dim=2)  # [quantity, chosen | rejected]
+    both = halves.sum(dim=1)
+    return {
+        "entropy_sum": both[0], "n_tokens": both[3],
+        "logits_chosen_sum": halves[1, 0], "n_chosen_tokens": halves[3, 0],
+        "logits_rejected_sum": halves[1, 1], "n_rejected_tokens": halves[3, 1],
+        "correct_tokens": halves[2, 0],
+        "chosen_rewards": beta * (chosen - ref_c), "rejected_rewards": beta * (rejected - ref_r),
+        "chosen_logps": chosen, "rejected_logps": rejected,
+    }
 
 
 def dpo_metrics_to_dict(metrics: dict) -> dict[str, float]:
@@ -296,9 +317,9 @@ def dpo_sequence_logps(logits: Tensor, input_ids: Tensor, completion_mask: Tenso
     rm = (smask.reshape(-1) != 0).to(torch.uint8).contiguous()
     with torch.no_grad():
         logp, _ = logps_and_entropies(logits, input_ids[:, 1:], 1.0, 0, length - 1, rm.view(n_seq, length - 1))
-        tok = logp * smask
         if ld_alpha is None:
-            return tok.sum(dim=1)
+            return _masked_row_sums(logp, smask.to(torch.float32))
+        tok = logp * smask
         pos = smask.cumsum(dim=1)
         shared = torch.minimum(*smask.sum(dim=1).chunk(2)).repeat(2).unsqueeze(1)
         return (tok * ((pos > 0) & (pos <= shared))).sum(dim=1) + ld_alpha * (tok * (pos > shared)).sum(dim=1)
