@@ -295,6 +295,11 @@ def bench_head(args, w):
             del saved
             fwd_plain = time_op(lambda: ops.fused_head_fwd(*fwd_args))
             bwd_rec = time_op(lambda: ops.fused_head_bwd(*fwd_args, log_z, gl, HEAD_CHUNK))
+            kernels["fused_head_fwd_no_grad"] = {
+                "avg_ms": fwd_plain, "TFLOPs": flop / (fwd_plain * 1e-3) / 1e12,
+                "frac": flop / (fwd_plain * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                "note": "the forward when nothing asks for a gradient (log-probs of the old and of the reference "
+                        "policy): same kernel, no products kept for a backward"}
             kernels["recompute_scheme"] = {
                 "fwd_ms": fwd_plain, "bwd_ms": bwd_rec, "fwd_TFLOPs": flop / (fwd_plain * 1e-3) / 1e12,
                 "bwd_TFLOPs": 3 * flop / (bwd_rec * 1e-3) / 1e12,
