@@ -807,7 +807,10 @@ def main():
                                     "calibrate_copy": False})
         for lt in ("grpo", "dr_grpo"):
             if lt != args.loss_type:
-                secondary.append(_brief(bench_grpo(few, w, lt, shared, full=False)[0]))
+                try:
+                    secondary.append(_brief(bench_grpo(few, w, lt, shared, full=False)[0]))
+                except Exception as exc:
+                    secondary.append({"workload": args.workload, "loss_type": lt, "error": f"{type(exc).__name__}: {exc}"[:500]})
     del shared
     torch.cuda.empty_cache()
     if secondary_wanted:
@@ -816,10 +819,13 @@ def main():
         for name in ("head_c5", "grpo_c4", "dpo_c2", "logp_c1"):
             few.workload = name
             w2 = WORKLOADS[name]
-            r = (bench_head(few, w2) if w2.get("head") else bench_dpo(few, w2) if w2.get("dpo")
-                 else bench_logp_c1(few, w2) if w2.get("logp") else bench_grpo(few, w2, "dapo")[0])
-            secondary.append(_brief(r))
-            del r
+            try:
+                r = (bench_head(few, w2) if w2.get("head") else bench_dpo(few, w2) if w2.get("dpo")
+                     else bench_logp_c1(few, w2) if w2.get("logp") else bench_grpo(few, w2, "dapo")[0])
+                secondary.append(_brief(r))
+                del r
+            except Exception as exc:  # a secondary workload never takes the headline line with it
+                secondary.append({"workload": name, "error": f"{type(exc).__name__}: {exc}"[:500]})
             torch.cuda.empty_cache()
         result["secondary"] = secondary
     if not args.no_cpu_baseline:
