@@ -606,7 +606,8 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
         if (a.stash != nullptr) {
             // The tile's raw products go to memory for the backward (vocabulary-major, fp32): for one
             // accumulator register the 32 lanes of a half-wave hold 32 consecutive tokens of one
-            // vocabulary row = one 128-byte line per store.  The buffer is padded to whole tiles.
+            // vocabulary row = one 128-byte line per store (plain stores: measured 0.5 % ahead of non-temporal
+            // ones over the whole sweep).  The buffer is padded to whole tiles.
             const int uw = __builtin_amdgcn_readfirstlane(wave);
             const int uwm = uw / WGN, uwn = uw % WGN;
             const uint32_t lane_off = uint32_t((lane >> 5) * 4) * uint32_t(a.ld_stash) + uint32_t(lane & 31);
@@ -617,7 +618,7 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
                     float* blk = a.stash + int64_t(m0 + uwm * WM + mb * 32) * a.ld_stash + (n0 + uwn * WN + nb * 32);
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
-                        __builtin_nontemporal_store(acc[mb][nb][r], blk + int64_t((r >> 2) * 8 + (r & 3)) * a.ld_stash + lane_off);
+                        blk[int64_t((r >> 2) * 8 + (r & 3)) * a.ld_stash + lane_off] = acc[mb][nb][r];
                 }
         }
         const bool partial_tile = m0 + BM > a.V;
