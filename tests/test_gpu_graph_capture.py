@@ -1,7 +1,7 @@
 """The kernels under HIP graph capture: a captured micro-step is replayed on new inputs several times, with eager
 work and synchronisations between the replays, and every replay must equal the eager result bit for bit (the same
-kernels run in both).  Two graphs: log-prob kernel -> GRPO loss through the entry point that allocates nothing ->
-gradient kernel; and the single-pass GRPO kernel.  The library records no memset into a graph and keeps no host
+kernels run in both).  Three graphs: log-prob kernel -> GRPO loss through the entry point that allocates nothing ->
+gradient kernel; the single-pass GRPO kernel; the fused head forward (products kept) and backward, bf16 and fp16.  The library records no memset into a graph and keeps no host
 state between launches, which is what these replays would show if it did."""
 import math
 
@@ -84,3 +84,53 @@ def test_graph_replays_equal_eager(step):
         for i, (g, w) in enumerate(zip(got, want)):
             assert torch.equal(g.nan_to_num(nan=-7.0), w.nan_to_num(nan=-7.0)), (rep, i)
         assert float(got[-1].float().abs().sum()) > 0 or float(buf["mask"].sum()) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_fused_head_graph_replays_equal_eager(dtype):
+    """Forward with its products kept, then both gradient products from them: every buffer between the two (the
+    kept products, the scaled fp16 operand copies, the maxima behind their scales) is rewritten inside the graph."""
+    from trl_amd import ops
+
+    n, h, v = 300, 128, 1000  # two token tiles, four vocabulary tiles, both with remainders
+    hidden = torch.zeros((n, h), dtype=dtype, device=DEV)
+    weight = torch.zeros((v, h), dtype=dtype, device=DEV)
+    targets = torch.zeros((n,), dtype=torch.int64, device=DEV)
+    g_logp = torch.zeros((n,), device=DEV)
+
+    def new_inputs(seed):
+        g = torch.Generator(device=DEV).manual_seed(seed)
+        hidden.copy_(torch.randn((n, h), generator=g, device=DEV).to(dtype))
+        weight.copy_((0.1 * torch.randn((v, h), generator=g, device=DEV)).to(dtype))
+        targets.copy_(torch.randint(0, v, (n,), generator=g, device=DEV))
+        g_logp.copy_(torch.randn((n,), generator=g, device=DEV) * (torch.rand((n,), generator=g, device=DEV) < 0.7))
+
+    def step():
+        lp, ent, log_z, hit, kept = ops.fused_head_fwd(hidden, weight, targets, 0.8, 0.0, 1.0, None, True)
+        d_hidden, d_weight, _ = ops.fused_head_bwd(hidden, weight, targets, 0.8, 0.0, 1.0, log_z, g_logp, 512, None, kept)
+        return lp, ent, hit, d_hidden, d_weight
+
+    new_inputs(1)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    for rep in range(4):
+        new_inputs(10 + rep)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        scratch = torch.randn((1 << 20,), device=DEV).sum()
+        want = step()
+        torch.cuda.synchronize()
+        assert math.isfinite(float(scratch))
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), (rep, i)
+        assert float(got[3].float().abs().sum()) > 0 and float(got[4].float().abs().sum()) > 0
