@@ -134,3 +134,65 @@ def test_fused_head_graph_replays_equal_eager(dtype):
         for i, (a, b) in enumerate(zip(got, want)):
             assert torch.equal(a, b), (rep, i)
         assert float(got[3].float().abs().sum()) > 0 and float(got[4].float().abs().sum()) > 0
+
+
+def test_two_host_threads_on_their_own_streams():
+    """The entry points keep no state between calls (workspaces and outputs belong to the caller), so two host
+    threads, each on a stream of its own, can run the two-pass step, the single-pass kernel and the fused head at the
+    same time: each thread's results equal the ones the same inputs gave when run alone."""
+    import threading
+
+    import trl_amd
+    from trl_amd import ops
+
+    def make(seed):
+        buf = _buffers()
+        _new_inputs(buf, seed)
+        g = torch.Generator(device=DEV).manual_seed(seed)
+        head = (torch.randn((300, 128), generator=g, device=DEV).bfloat16(),
+                (0.1 * torch.randn((1000, 128), generator=g, device=DEV)).bfloat16(),
+                torch.randint(0, 1000, (300,), generator=g, device=DEV), torch.randn((300,), generator=g, device=DEV))
+        return buf, head
+
+    def work(buf, head):
+        h, w, tg, gl = head
+        # (the two-pass step through the ordinary loss entry point: the one that allocates nothing shares one
+        # scratch array per GPU between all its callers and is documented as not to be overlapped)
+        leaf = buf["logits"].detach().clone().requires_grad_(True)
+        lp2, ent2 = trl_amd.per_token_logps_and_entropies(leaf, buf["ids"], T, 0.9, True, False)
+        loss, metrics = trl_amd.grpo_loss(lp2, buf["adv"], buf["mask"], entropies=ent2,
+                                          old_per_token_logps=lp2.detach() + buf["old_noise"], loss_type="dapo",
+                                          epsilon_low=0.2, epsilon_high=0.28, num_items_in_batch=buf["n_items"])
+        loss.backward()
+        out = [lp2.detach(), ent2.detach(), loss.detach(), metrics.detach(), leaf.grad]
+        out += [t.clone() for t in _single_pass_step(buf)]
+        lp, ent, log_z, hit, kept = ops.fused_head_fwd(h, w, tg, 0.8, 0.0, 1.0, None, True)
+        out += [lp, ent, *ops.fused_head_bwd(h, w, tg, 0.8, 0.0, 1.0, log_z, gl, 512, None, kept)[:2]]
+        return out
+
+    problems = [make(31), make(32)]
+    torch.cuda.synchronize()
+    alone = [work(*p) for p in problems]
+    torch.cuda.synchronize()
+    results, errors = [None, None], []
+
+    def run(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(10):
+                    results[i] = work(*problems[i])
+            stream.synchronize()
+        except Exception as exc:  # surfaced below, in the main thread
+            errors.append(exc)
+
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    torch.cuda.synchronize()
+    for i in range(2):
+        for j, (a, b) in enumerate(zip(results[i], alone[i])):
+            assert torch.equal(a.nan_to_num(nan=-7.0), b.nan_to_num(nan=-7.0)), (i, j)
