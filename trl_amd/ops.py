@@ -659,7 +659,11 @@ def _head_operands(hidden: Tensor, weight: Tensor, targets: Tensor):
     if weight.dtype != hidden.dtype:
         weight = weight.to(hidden.dtype)  # the reference casts the weight slab to the hidden dtype (utils.py:1328)
     if hidden.shape[1] % 8 != 0:
-        raise ValueError("fused head: hidden_size must be a multiple of 8")
+        # rows of 16-byte vectors: zero columns up to the next multiple of 8 add nothing to any product (copies of
+        # both operands per call -- hidden sizes of real models are multiples of 8 and never come here)
+        pad = (-hidden.shape[1]) % 8
+        hidden = torch.nn.functional.pad(hidden, (0, pad))
+        weight = torch.nn.functional.pad(weight, (0, pad))
 
     def rows_ok(t):
         return t.stride(1) == 1 and t.stride(0) % 8 == 0 and t.stride(0) >= t.shape[1] and t.data_ptr() % 16 == 0
@@ -743,6 +747,7 @@ def fused_head_bwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
     `stash`: the fifth output of a `fused_head_fwd(..., stash=True)` on the same operands (skips the recompute);
     `stash_cols` (int32 [N]): the forward's row of each token when rows were dropped since (see `head_backward`)."""
     w_dtype = weight.dtype
+    h_true = hidden.shape[1] if hidden.dim() == 2 else 0
     hidden, weight, targets = _head_operands(hidden, weight, targets)
     n, h = hidden.shape
     v = weight.shape[0]
@@ -773,6 +778,8 @@ def fused_head_bwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
                                       stash.stride(0) if stash is not None else 0, ptr(stash_cols), ptr(d_hidden),
                                       ptr(d_weight),
                                       ptr(d_bias) if bias is not None else None, ptr(ws), ws_bytes, current_stream(dev)))
+    if h != h_true:  # the operands were padded to a multiple of 8 columns
+        d_hidden, d_weight = d_hidden[:, :h_true].contiguous(), d_weight[:, :h_true].contiguous()
     return d_hidden, (d_weight if w_dtype == d_weight.dtype else d_weight.to(w_dtype)), d_bias
 
 
