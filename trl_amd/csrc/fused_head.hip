@@ -503,7 +503,7 @@ __device__ __forceinline__ void xcd_patch(int w, int n_a, int n_b, int& ta, int&
         tb = qq / m;
         ta = (bands * 4 + qq % m) * 8 + xcd;
     } else {
-        const int r = n_a & 7, left = r * n_b;     // the a tiles that are left, and their tiles
+        const int r = (n_a & 7) ? (n_a & 7) : 1, left = (n_a & 7) * n_b;  // the a tiles that are left, and their tiles
         const int share = (left + 7) >> 3;
         const int t = xcd * share + (q - full - m * n_b);
         const bool real = q - full - m * n_b < share && t < left;

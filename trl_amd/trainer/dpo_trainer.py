@@ -182,6 +182,8 @@ def _masked_row_sums(token_logps: Tensor, mask: Tensor) -> Tensor:
     """`[2P]` sums of the log-probs inside the mask, from the loss kernel's own row reduction (differentiable).  Every
     place that sums a sequence uses this one order of summation: reference log-probs taken from the same logits then
     cancel the policy's exactly, and the first step of a run starts at ln 2 as it does in the reference."""
+    if token_logps.shape[0] % 2:  # not a batch of pairs (a caller summing sequences on their own): plain torch
+        return (token_logps.float() * (mask != 0)).sum(dim=1)
     zero = token_logps.new_zeros((token_logps.shape[0] // 2,), dtype=torch.float32)
     return ops.dpo_loss_op(token_logps, mask, zero, zero, 1.0)[1]
 
