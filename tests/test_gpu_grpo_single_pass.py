@@ -239,6 +239,54 @@ def test_real_vocabulary_and_limits(amd):
     amd.check_device_errors()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_rows_that_overflow_into_lds(amd, dtype):
+    """Rows longer than the registers hold (more than 163840 logits): the rest of the row waits in the CU's LDS.
+    Vocabularies of current 200k-entry tokenizers, one that ends inside every LDS build (3, 6, 9 vectors per lane),
+    the first size past the registers and the largest one; targets in the register part, in the LDS part and on the
+    row's last entry; entropy bonus on (its gradient term runs over the LDS part too).  Against the two-pass path,
+    and log-probs / entropies / gradient of one case against the oracle."""
+    import oracle
+
+    assert amd.ops.grpo_fused_max_vocab(dtype) == 29 * 1024 * 8
+    for V in (163848, 180000, 200064, 202048, 221184, 237568):
+        B, K = 2, 3
+        logits, ids, mask, adv, g = _inputs(B, K, V, dtype=dtype, seed=V % 89, extra_rows=1)
+        mask[:] = 1
+        mask[1, 2] = 0
+        ids[0, 0], ids[0, 1], ids[0, 2], ids[1, 0] = 5, 163840 + 7, V - 1, 20 * 8192 - 1
+        assert amd.grpo_single_pass_supported(logits)
+        kw = dict(loss_type="bnpo", beta=0.0, entropy_coef=0.02 if V % 3 == 0 else 0.0)
+        leaf, loss2, met2, lp2, ent2 = _two_pass(amd, logits, ids, mask, adv, 0.9, **kw) if not kw["entropy_coef"] else (None,) * 5
+        if leaf is None:
+            leaf = logits.detach().clone().requires_grad_(True)
+            lp_g, ent_g = amd.per_token_logps_and_entropies(leaf, ids, K, 0.9, True, True)
+            loss2, met2 = amd.grpo_loss(lp_g, adv, mask, entropies=ent_g, **kw)
+            lp2, ent2 = lp_g.detach(), ent_g.detach()
+        loss2.backward()
+        leaf1 = logits.detach().clone().requires_grad_(True)
+        loss1, met1, lp1, ent1 = amd.grpo_loss_from_logits(leaf1, ids, adv, mask, temperature=0.9, **kw)
+        loss1.backward()
+        m = mask.bool()
+        torch.testing.assert_close(loss1, loss2, rtol=1e-5, atol=1e-7)
+        torch.testing.assert_close(lp1[m], lp2[m], rtol=0, atol=1e-5)
+        torch.testing.assert_close(ent1[m], ent2[m], rtol=0, atol=1e-5)
+        assert _rel_l2(leaf1.grad, leaf.grad) < 2e-3, V
+        assert float(leaf1.grad[1, 2].float().abs().max()) == 0.0 and float(leaf1.grad[:, K:].float().abs().max()) == 0.0
+        assert float(leaf1.grad[0, 0, 163840:].float().abs().max()) > 0.0  # the part of the row that came through LDS
+        if V == 200064:
+            cpu_leaf = logits.detach().float().cpu().requires_grad_(True)
+            lp, ent = oracle.logps_and_entropies_from_logits(cpu_leaf, ids.cpu(), K, 0.9, True)
+            want, _ = oracle.grpo_loss(lp, adv.cpu(), mask.cpu(), entropies=ent, loss_type="bnpo", beta=0.0,
+                                       entropy_coef=kw["entropy_coef"])
+            want.backward()
+            torch.testing.assert_close(lp1.cpu()[m.cpu()], lp.detach()[m.cpu()], atol=2e-3, rtol=0)
+            torch.testing.assert_close(ent1.cpu()[m.cpu()], ent.detach()[m.cpu()], atol=2e-3, rtol=0)
+            torch.testing.assert_close(loss1.detach().cpu(), want.detach(), atol=1e-6, rtol=1e-3)
+            assert _rel_l2(leaf1.grad.float().cpu(), cpu_leaf.grad) < 5e-3
+    amd.check_device_errors()
+
+
 def test_unsupported_configurations_raise(amd):
     logits, ids, mask, adv, _ = _inputs(2, 4, 1024)
     assert amd.grpo_single_pass_supported(logits)

@@ -17,8 +17,13 @@ namespace {
 
 constexpr int kFThreads = 1024;
 constexpr int kFWaves = kFThreads / kWave;
-constexpr int kMaxVec = 20;  // 16-byte vectors of a row per lane: rows of up to 20 * 1024 * 8 = 163840 logits
+constexpr int kMaxVec = 20;  // 16-byte vectors of a row per lane in registers: rows of up to 20 * 1024 * 8 = 163840 logits
 constexpr int kVecStep = 4;  // the kernel is built for 4, 8, ... kMaxVec vectors per lane; the host picks the smallest that holds the row
+// Longer rows keep what the registers cannot hold in the CU's LDS: up to kMaxLdsVec more vectors per lane (16 KiB of
+// LDS each; 9 of them leave room for the reduction scratch in the 160 KiB), in builds of kLdsStep: rows of up to
+// 29 * 1024 * 8 = 237568 logits.
+constexpr int kMaxLdsVec = 9, kLdsStep = 3;
+constexpr int kWideVec = kMaxVec;  // register vectors of the builds with vectors in LDS
 
 typedef __attribute__((address_space(1))) const u32x4 GlobalVecIn;
 typedef __attribute__((address_space(1))) u32x4 GlobalVecOut;
@@ -42,6 +47,17 @@ struct FusedArgs {
     int all_rows;  // also read the rows with mask == 0 for their log-prob and entropy (their gradient is zero either way)
 };
 
+// One 1 KiB transfer from memory straight into LDS: 16 bytes per lane from `src` to LDS address `lds` + 16 * lane
+// (`lds` uniform over the wave).  (m0 is a reserved register; naming it as clobbered keeps the compiler's values out.)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void lds_transfer(const u32x4* src, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds),
+                 "v"(reinterpret_cast<uint64_t>(src))
+                 : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
 // One workgroup of 1024 lanes per output row; NVEC = 16-byte vectors of the row a lane holds (the last kVecStep of
 // them may lie beyond the row's end for some lanes).  A workgroup fills its CU's register file, so nothing else
 // runs beside it: the arithmetic has to overlap the row's own memory traffic.  Hence
@@ -52,12 +68,18 @@ struct FusedArgs {
 //     vector as its load retires.  Later logits may exceed the first vector's by 128 / (log2(e) / T) before a
 //     term overflows; a row where that happens (or one that holds inf / NaN) is detected by its non-finite sums
 //     and takes the exact two-sweep reduction over the registers instead.
-template <int DT, int NVEC>
+//   * NLDS > 0 (rows too long for the registers): vectors NVEC ... NVEC + NLDS - 1 of a lane travel from memory straight
+//     into LDS, 1 KiB per wave and transfer, issued before the register loads; a lane only ever reads back the 16
+//     bytes its own transfer wrote, so the wave's own wait for its transfers is all the synchronisation they need.
+template <int DT, int NVEC, int NLDS>
 __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     typedef Elem<DT> E;
     typedef typename E::type T;
     constexpr int EPV = E::EPV;
+    // (the last register vectors keep their end-of-row test in the builds with vectors in LDS too, where it is always
+    // true: without it the compiler unpacks every register vector ahead of its use and spills a hundred registers)
     constexpr int kTail = NVEC - kVecStep;
+    extern __shared__ __attribute__((aligned(16))) char overflow[];  // [NLDS][1024 lanes] 16-byte vectors
     __shared__ float red[7][kFWaves];
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int64_t orow = blockIdx.x;
@@ -95,6 +117,18 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     }
     const T* base = static_cast<const T*>(a.logits) + b * a.seq_stride + t * a.row_stride;
     const u32x4* vp = reinterpret_cast<const u32x4*>(base);
+    if constexpr (NLDS > 0) {
+        const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(overflow)) +
+                              uint32_t(__builtin_amdgcn_readfirstlane(wave)) * (kWave * 16);
+#pragma unroll
+        for (int jl = 0; jl < NLDS; ++jl) {
+            const int v0 = (NVEC + jl) * kFThreads;
+            if (v0 < nv) {  // (uniform over the workgroup; lanes beyond the row's end re-read its last vector)
+                const int tj = min(tid, nv - 1 - v0);
+                lds_transfer(vp + v0 + tj, lds0 + uint32_t(jl) * (kFThreads * 16));
+            }
+        }
+    }
     u32x4 q[NVEC];
 #pragma unroll
     for (int j = 0; j < NVEC; ++j) {
@@ -131,6 +165,24 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
                 const float e = fast_exp2(fmaf(x[i], c, -r0));
                 s += e;
                 u = fmaf(e, x[i], u);
+            }
+        }
+    }
+    const u32x4* lds_q = reinterpret_cast<const u32x4*>(overflow) + tid;  // + jl * kFThreads
+    if constexpr (NLDS > 0) {
+        // the transfers were issued before every register load and loads return in order: they have landed
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll 1  // (one vector at a time: the registers are full of the row)
+        for (int jl = 0; jl < NLDS; ++jl) {
+            if ((NVEC + jl) * kFThreads + tid < nv) {
+                float x[EPV];
+                E::unpack(lds_q[jl * kFThreads], x);
+#pragma unroll
+                for (int i = 0; i < EPV; ++i) {
+                    const float e = fast_exp2(fmaf(x[i], c, -r0));
+                    s += e;
+                    u = fmaf(e, x[i], u);
+                }
             }
         }
     }
@@ -258,6 +310,22 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
             __builtin_nontemporal_store(E::pack(d), oj + tid);  // (streaming stores: 2-3 % faster than plain ones here)
         }
     }
+    if constexpr (NLDS > 0) {
+#pragma unroll 1
+        for (int jl = 0; jl < NLDS; ++jl) {
+            const int v = (NVEC + jl) * kFThreads + tid;
+            if (v < nv) {
+                float x[EPV], d[EPV];
+                E::unpack(lds_q[jl * kFThreads], x);
+#pragma unroll
+                for (int i = 0; i < EPV; ++i) {
+                    const float tt = fmaf(x[i], c, -lse2);
+                    d[i] = fast_exp2(tt) * (with_h ? fmaf(b0, tt, a0) : a0);
+                }
+                __builtin_nontemporal_store(E::pack(d), op + v);
+            }
+        }
+    }
     // one-hot term: the lane that stored the target's vector rewrites that element (same lane, same
     // address: ordered after its first store)
     if (idx_ok && int((idx / EPV) % kFThreads) == tid) {
@@ -267,15 +335,55 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     }
 }
 
+// dynamic LDS above 64 KiB has to be allowed per kernel and device once
+template <typename Kern>
+int reserve_overflow_lds(Kern kern, int bytes) {
+    struct Done {
+        const void* kern;
+        int device;
+    };
+    static thread_local Done configured[16] = {};
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) device = 0;
+    const void* key = reinterpret_cast<const void*>(kern);
+    for (const Done& c : configured)
+        if (c.kern == key && c.device == device) return TRLK_OK;
+    const hipError_t e = hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return fail(int(e), "grpo_fused: cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(e));
+    for (Done& c : configured)
+        if (c.kern == nullptr) {
+            c.kern = key;
+            c.device = device;
+            break;
+        }
+    return TRLK_OK;
+}
+
+template <int DT, int NLDS>
+int launch_fused_wide(const FusedArgs& a, unsigned rows, hipStream_t s) {
+    constexpr int kBytes = NLDS * kFThreads * 16;
+    if (int rc = reserve_overflow_lds(grpo_fused_kernel<DT, kWideVec, NLDS>, kBytes)) return rc;
+    hipLaunchKernelGGL((grpo_fused_kernel<DT, kWideVec, NLDS>), dim3(rows), dim3(kFThreads), kBytes, s, a);
+    return TRLK_OK;
+}
+
 template <int DT>
-void launch_fused(const FusedArgs& a, int nvec, unsigned rows, hipStream_t s) {
-    switch ((nvec + kVecStep - 1) / kVecStep) {
-        case 1: hipLaunchKernelGGL((grpo_fused_kernel<DT, 4>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-        case 2: hipLaunchKernelGGL((grpo_fused_kernel<DT, 8>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-        case 3: hipLaunchKernelGGL((grpo_fused_kernel<DT, 12>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-        case 4: hipLaunchKernelGGL((grpo_fused_kernel<DT, 16>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-        default: hipLaunchKernelGGL((grpo_fused_kernel<DT, 20>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+int launch_fused(const FusedArgs& a, int nvec, unsigned rows, hipStream_t s) {
+    if (nvec > kMaxVec) {
+        switch ((nvec - kWideVec + kLdsStep - 1) / kLdsStep) {
+            case 1: return launch_fused_wide<DT, 3>(a, rows, s);
+            case 2: return launch_fused_wide<DT, 6>(a, rows, s);
+            default: return launch_fused_wide<DT, 9>(a, rows, s);
+        }
     }
+    switch ((nvec + kVecStep - 1) / kVecStep) {
+        case 1: hipLaunchKernelGGL((grpo_fused_kernel<DT, 4, 0>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        case 2: hipLaunchKernelGGL((grpo_fused_kernel<DT, 8, 0>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        case 3: hipLaunchKernelGGL((grpo_fused_kernel<DT, 12, 0>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        case 4: hipLaunchKernelGGL((grpo_fused_kernel<DT, 16, 0>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        default: hipLaunchKernelGGL((grpo_fused_kernel<DT, 20, 0>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+    }
+    return TRLK_OK;
 }
 
 // data *= *scale over 16-byte vectors, unless the scale is exactly 1 (then nothing is read or written, and what the
@@ -332,7 +440,7 @@ extern "C" int trlk_scale_unless_one(void* d_data, int dtype, int64_t n_elems, c
 }
 
 extern "C" int64_t trlk_grpo_fused_max_vocab(int dtype) {
-    return dtype == TRLK_BF16 || dtype == TRLK_F16 ? int64_t(kMaxVec) * kFThreads * 8 : 0;
+    return dtype == TRLK_BF16 || dtype == TRLK_F16 ? int64_t(kWideVec + kMaxLdsVec) * kFThreads * 8 : 0;
 }
 
 extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t n_seq, int64_t rows_per_seq, int64_t vocab,
@@ -415,9 +523,8 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
     a.all_rows = compute_masked_rows != 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int nvec = int((vocab / 8 + kFThreads - 1) / kFThreads);  // 16-byte vectors of the row per lane
-    if (dtype == TRLK_BF16)
-        launch_fused<TRLK_BF16>(a, nvec, unsigned(orows), s);
-    else
-        launch_fused<TRLK_F16>(a, nvec, unsigned(orows), s);
+    if (int rc = dtype == TRLK_BF16 ? launch_fused<TRLK_BF16>(a, nvec, unsigned(orows), s)
+                                    : launch_fused<TRLK_F16>(a, nvec, unsigned(orows), s))
+        return rc;
     return launch_status("grpo_fused");
 }
