@@ -97,9 +97,9 @@ def test_host_side_argument_validation():
                                            None, None, fake, None, term, 0.2, 0.2, float("nan"), beta, 0, 1.0, 1.05, fake, fake,
                                            fake, fake16, out_rows, offset, out_rows * vocab, vocab, 0, None, None)
 
-    assert lib.trlk_grpo_fused_max_vocab(_lib.BF16) == 29 * 1024 * 8 and lib.trlk_grpo_fused_max_vocab(_lib.F32) == 0
+    assert lib.trlk_grpo_fused_max_vocab(_lib.BF16) == 37 * 1024 * 8 and lib.trlk_grpo_fused_max_vocab(_lib.F32) == 0
     assert fused(dtype=_lib.F32) == -3 and "two-pass" in _lib.last_error()
-    assert fused(vocab=4100) == -7 and fused(vocab=29 * 1024 * 8 + 8) == -7
+    assert fused(vocab=4100) == -7 and fused(vocab=37 * 1024 * 8 + 8) == -7
     assert fused(logits=fake16 + 2) == -4 and fused(row_stride=4100) == -4
     assert fused(beta=0.1) == -1 and fused(term=9) == -5
     assert fused(out_rows=3) == -2 and fused(out_rows=8, offset=5) == -2

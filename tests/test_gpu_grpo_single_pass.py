@@ -241,15 +241,17 @@ def test_real_vocabulary_and_limits(amd):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 def test_rows_that_overflow_into_lds(amd, dtype):
-    """Rows longer than the registers hold (more than 163840 logits): the rest of the row waits in the CU's LDS.
-    Vocabularies of current 200k-entry tokenizers, one that ends inside every LDS build (3, 6, 9 vectors per lane),
-    the first size past the registers and the largest one; targets in the register part, in the LDS part and on the
+    """Rows longer than the registers hold (more than 163840 logits): the rest of the row waits in the CU's LDS, and
+    what does not fit there either (more than 237568 logits) is read twice.  Vocabularies of current 200k- and
+    256k-entry tokenizers, one that ends inside every LDS build (3, 6, 9 vectors per lane), the first sizes past the
+    registers and past the LDS, and the largest one; targets in the register part, in the LDS part and on the
     row's last entry; entropy bonus on (its gradient term runs over the LDS part too).  Against the two-pass path,
     and log-probs / entropies / gradient of one case against the oracle."""
     import oracle
 
-    assert amd.ops.grpo_fused_max_vocab(dtype) == 29 * 1024 * 8
-    for V in (163848, 180000, 200064, 202048, 221184, 237568):
+    assert amd.ops.grpo_fused_max_vocab(dtype) == 37 * 1024 * 8
+    # (beyond 29 * 8192 = 237568 logits the last vectors of a row are read twice instead of kept: 256000, 262144, ...)
+    for V in (163848, 180000, 200064, 202048, 221184, 237568, 237576, 256000, 262144, 303104):
         B, K = 2, 3
         logits, ids, mask, adv, g = _inputs(B, K, V, dtype=dtype, seed=V % 89, extra_rows=1)
         mask[:] = 1

@@ -23,6 +23,10 @@ constexpr int kVecStep = 4;  // the kernel is built for 4, 8, ... kMaxVec vector
 // LDS each; 9 of them leave room for the reduction scratch in the 160 KiB), in builds of kLdsStep: rows of up to
 // 29 * 1024 * 8 = 237568 logits.
 constexpr int kMaxLdsVec = 9, kLdsStep = 3;
+// Rows longer still (the 256000- and 262144-entry vocabularies) read their last vectors twice: once ahead of the row
+// for the sums, once after it for the gradient, by which time the workgroup has read them so recently that they
+// come from the L2.  Up to kMaxExtraVec such vectors per lane: rows of up to 37 * 1024 * 8 = 303104 logits.
+constexpr int kMaxExtraVec = 8;
 constexpr int kWideVec = kMaxVec;  // register vectors of the builds with vectors in LDS
 
 typedef __attribute__((address_space(1))) const u32x4 GlobalVecIn;
@@ -71,7 +75,10 @@ __device__ __forceinline__ void lds_transfer(const u32x4* src, uint32_t lds) {
 //   * NLDS > 0 (rows too long for the registers): vectors NVEC ... NVEC + NLDS - 1 of a lane travel from memory straight
 //     into LDS, 1 KiB per wave and transfer, issued before the register loads; a lane only ever reads back the 16
 //     bytes its own transfer wrote, so the wave's own wait for its transfers is all the synchronisation they need.
-template <int DT, int NVEC, int NLDS>
+//   * EXTRA (rows too long for registers and LDS together): the vectors beyond are summed before the row proper is
+//     requested (four loads in flight; their registers are free again when the row's loads go out) and read again at
+//     the end for their gradient.
+template <int DT, int NVEC, int NLDS, bool EXTRA = false>
 __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     typedef Elem<DT> E;
     typedef typename E::type T;
@@ -117,6 +124,38 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     }
     const T* base = static_cast<const T*>(a.logits) + b * a.seq_stride + t * a.row_stride;
     const u32x4* vp = reinterpret_cast<const u32x4*>(base);
+    const float inv_t = 1.f / a.temperature, c = kLog2e * inv_t;
+    // sums of 2^(x c - r0) and of the same times x
+    float r0 = 0.f, s = 0.f, u = 0.f;
+    [[maybe_unused]] bool have_r0 = false;
+    constexpr int kOnChip = (NVEC + NLDS) * kFThreads;  // vectors of the row the workgroup holds
+    if constexpr (EXTRA) {
+        for (int v0 = kOnChip; v0 < nv; v0 += 4 * kFThreads) {
+            u32x4 e4[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) e4[k] = vp[min(v0 + k * kFThreads + tid, nv - 1)];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                if (v0 + k * kFThreads + tid < nv) {
+                    float x[EPV];
+                    E::unpack(e4[k], x);
+                    if (!have_r0) {
+                        float mx = x[0];
+#pragma unroll
+                        for (int i = 1; i < EPV; ++i) mx = fmaxf(mx, x[i]);
+                        r0 = ceilf(mx * c);
+                        have_r0 = true;
+                    }
+#pragma unroll
+                    for (int i = 0; i < EPV; ++i) {
+                        const float e = fast_exp2(fmaf(x[i], c, -r0));
+                        s += e;
+                        u = fmaf(e, x[i], u);
+                    }
+                }
+            }
+        }
+    }
     if constexpr (NLDS > 0) {
         const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>(overflow)) +
                               uint32_t(__builtin_amdgcn_readfirstlane(wave)) * (kWave * 16);
@@ -144,17 +183,15 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     }
     const bool idx_ok = idx >= 0 && idx < a.vocab;
     T x_t_raw = base[idx_ok ? idx : 0];  // requested right behind the row; converted only when the sums are done
-    const float inv_t = 1.f / a.temperature, c = kLog2e * inv_t;
 
-    // sums of 2^(x c - r0) and of the same times x, vector by vector as the loads retire
-    float r0 = 0.f, s = 0.f, u = 0.f;
+    // the sums, vector by vector as the loads retire
 #pragma unroll
     for (int j = 0; j < NVEC; ++j) {
         asm volatile("" : "+v"(q[j]));  // (pins the order: vector j is waited for and consumed before vector j + 1)
         if (j < kTail || j * kFThreads + tid < nv) {
             float x[EPV];
             E::unpack(q[j], x);
-            if (j == 0) {
+            if (j == 0 && !(EXTRA && have_r0)) {
                 float mx = x[0];
 #pragma unroll
                 for (int i = 1; i < EPV; ++i) mx = fmaxf(mx, x[i]);
@@ -326,6 +363,27 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
             }
         }
     }
+    if constexpr (EXTRA) {
+        for (int v0 = kOnChip; v0 < nv; v0 += 4 * kFThreads) {
+            u32x4 e4[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) e4[k] = vp[min(v0 + k * kFThreads + tid, nv - 1)];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int v = v0 + k * kFThreads + tid;
+                if (v < nv) {
+                    float x[EPV], d[EPV];
+                    E::unpack(e4[k], x);
+#pragma unroll
+                    for (int i = 0; i < EPV; ++i) {
+                        const float tt = fmaf(x[i], c, -lse2);
+                        d[i] = fast_exp2(tt) * (with_h ? fmaf(b0, tt, a0) : a0);
+                    }
+                    __builtin_nontemporal_store(E::pack(d), op + v);
+                }
+            }
+        }
+    }
     // one-hot term: the lane that stored the target's vector rewrites that element (same lane, same
     // address: ordered after its first store)
     if (idx_ok && int((idx / EPV) % kFThreads) == tid) {
@@ -369,6 +427,12 @@ int launch_fused_wide(const FusedArgs& a, unsigned rows, hipStream_t s) {
 
 template <int DT>
 int launch_fused(const FusedArgs& a, int nvec, unsigned rows, hipStream_t s) {
+    if (nvec > kWideVec + kMaxLdsVec) {
+        constexpr int kBytes = kMaxLdsVec * kFThreads * 16;
+        if (int rc = reserve_overflow_lds(grpo_fused_kernel<DT, kWideVec, kMaxLdsVec, true>, kBytes)) return rc;
+        hipLaunchKernelGGL((grpo_fused_kernel<DT, kWideVec, kMaxLdsVec, true>), dim3(rows), dim3(kFThreads), kBytes, s, a);
+        return TRLK_OK;
+    }
     if (nvec > kMaxVec) {
         switch ((nvec - kWideVec + kLdsStep - 1) / kLdsStep) {
             case 1: return launch_fused_wide<DT, 3>(a, rows, s);
@@ -440,7 +504,7 @@ extern "C" int trlk_scale_unless_one(void* d_data, int dtype, int64_t n_elems, c
 }
 
 extern "C" int64_t trlk_grpo_fused_max_vocab(int dtype) {
-    return dtype == TRLK_BF16 || dtype == TRLK_F16 ? int64_t(kWideVec + kMaxLdsVec) * kFThreads * 8 : 0;
+    return dtype == TRLK_BF16 || dtype == TRLK_F16 ? int64_t(kWideVec + kMaxLdsVec + kMaxExtraVec) * kFThreads * 8 : 0;
 }
 
 extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t n_seq, int64_t rows_per_seq, int64_t vocab,

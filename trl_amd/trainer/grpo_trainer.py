@@ -238,7 +238,7 @@ def grpo_single_pass_supported(logits: Tensor, loss_type: str = "dapo", importan
                                entropy_coef: float = 0.0, entropy_mask: Tensor | None = None) -> bool:
     """Whether `grpo_loss_from_logits` can go from these logits to their gradient in one pass: a token-level
     loss type, with or without entropy bonus but without an entropy-quantile mask (the gradient coefficients of
-    a token then depend on nothing but that token), 16-bit logits whose rows fit one workgroup's registers and LDS and
+    a token then depend on nothing but that token), 16-bit logits whose rows the kernel takes (`ops.grpo_fused_max_vocab`) and
     are 16-byte aligned."""
     if loss_type not in _SINGLE_PASS_LOSS_TYPES or importance_sampling_level != "token":
         return False
