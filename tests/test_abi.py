@@ -97,13 +97,14 @@ def test_host_side_argument_validation():
                                            None, None, fake, None, term, 0.2, 0.2, float("nan"), beta, 0, 1.0, 1.05, fake, fake,
                                            fake, fake16, out_rows, offset, out_rows * vocab, vocab, 0, None, None)
 
-    assert lib.trlk_grpo_fused_max_vocab(_lib.BF16) == 37 * 1024 * 8 and lib.trlk_grpo_fused_max_vocab(_lib.F32) == 0
-    assert fused(dtype=_lib.F32) == -3 and "two-pass" in _lib.last_error()
-    assert fused(vocab=4100) == -7 and fused(vocab=37 * 1024 * 8 + 8) == -7
+    assert lib.trlk_grpo_fused_max_vocab(_lib.BF16) == 41 * 1024 * 8 and lib.trlk_grpo_fused_max_vocab(_lib.F32) == 41 * 1024 * 4
+    assert lib.trlk_grpo_fused_max_vocab(99) == 0
+    assert fused(dtype=99) == -3 and "two-pass" in _lib.last_error()
+    assert fused(vocab=4100) == -7 and fused(vocab=41 * 1024 * 8 + 8) == -7
     assert fused(logits=fake16 + 2) == -4 and fused(row_stride=4100) == -4
     assert fused(beta=0.1) == -1 and fused(term=9) == -5
     assert fused(out_rows=3) == -2 and fused(out_rows=8, offset=5) == -2
-    assert lib.trlk_scale_unless_one(fake16, _lib.F32, 64, fake, None) == -3
+    assert lib.trlk_scale_unless_one(fake16, 99, 64, fake, None) == -3
     assert lib.trlk_scale_unless_one(fake16, _lib.BF16, 60, fake, None) == -2
     # fused head: fp32 operands, ragged hidden size, a stash whose rows are too short, missing workspace
 

@@ -249,9 +249,9 @@ def test_rows_that_overflow_into_lds(amd, dtype):
     and log-probs / entropies / gradient of one case against the oracle."""
     import oracle
 
-    assert amd.ops.grpo_fused_max_vocab(dtype) == 37 * 1024 * 8
+    assert amd.ops.grpo_fused_max_vocab(dtype) == 41 * 1024 * 8
     # (beyond 29 * 8192 = 237568 logits the last vectors of a row are read twice instead of kept: 256000, 262144, ...)
-    for V in (163848, 180000, 200064, 202048, 221184, 237568, 237576, 256000, 262144, 303104):
+    for V in (163848, 180000, 200064, 202048, 221184, 237568, 237576, 256000, 262144, 335872):
         B, K = 2, 3
         logits, ids, mask, adv, g = _inputs(B, K, V, dtype=dtype, seed=V % 89, extra_rows=1)
         mask[:] = 1
@@ -289,10 +289,59 @@ def test_rows_that_overflow_into_lds(amd, dtype):
     amd.check_device_errors()
 
 
+def test_fp32_logits(amd):
+    """fp32 logits (four per 16-byte vector): rows that fit the registers (32000), that overflow into LDS (100000)
+    and whose end is read twice (151936, 167936); the gradient is fp32 and not rounded, so it agrees with the
+    two-pass path to fp32 rounding, and with the oracle's autograd on one case."""
+    import oracle
+
+    assert amd.ops.grpo_fused_max_vocab(torch.float32) == 41 * 1024 * 4
+    for V in (32000, 81920, 100000, 151936, 167936):
+        B, K = 2, 3
+        logits, ids, mask, adv, g = _inputs(B, K, V, dtype=torch.float32, seed=V % 83, extra_rows=1)
+        mask[:] = 1
+        mask[1, 2] = 0
+        ids[0, 0], ids[0, 1], ids[0, 2] = 3, V // 2 + 1, V - 1
+        assert amd.grpo_single_pass_supported(logits)
+        with torch.no_grad():
+            base, _ = amd.per_token_logps_and_entropies(logits, ids, K, 0.9)
+        kw = dict(loss_type="dapo", beta=0.04, old_per_token_logps=base + 0.3 * torch.randn(base.shape, generator=g, device=DEV),
+                  ref_per_token_logps=base - 0.1, num_items_in_batch=mask.sum().float(), epsilon_low=0.2, epsilon_high=0.28)
+        leaf, loss2, met2, lp2, ent2 = _two_pass(amd, logits, ids, mask, adv, 0.9, **kw)
+        loss2.backward()
+        leaf1 = logits.detach().clone().requires_grad_(True)
+        loss1, met1, lp1, ent1 = amd.grpo_loss_from_logits(leaf1, ids, adv, mask, temperature=0.9, **kw)
+        loss1.backward()
+        assert leaf1.grad.dtype == torch.float32
+        m = mask.bool()
+        torch.testing.assert_close(loss1, loss2, rtol=1e-5, atol=1e-7)
+        torch.testing.assert_close(met1, met2, rtol=1e-5, atol=1e-6, equal_nan=True)
+        torch.testing.assert_close(lp1[m], lp2[m], rtol=0, atol=1e-5)
+        torch.testing.assert_close(ent1[m], ent2[m], rtol=0, atol=1e-5)
+        assert _rel_l2(leaf1.grad, leaf.grad) < 2e-5, V
+        assert float(leaf1.grad[1, 2].abs().max()) == 0.0 and float(leaf1.grad[:, K:].abs().max()) == 0.0
+        if V == 100000:
+            cpu_leaf = logits.detach().cpu().requires_grad_(True)
+            lp, ent = oracle.logps_and_entropies_from_logits(cpu_leaf, ids.cpu(), K, 0.9, True)
+            okw = {k: (v.cpu() if torch.is_tensor(v) else v) for k, v in kw.items()}
+            want, _ = oracle.grpo_loss(lp, adv.cpu(), mask.cpu(), entropies=ent, **okw)
+            want.backward()
+            torch.testing.assert_close(lp1.cpu()[m.cpu()], lp.detach()[m.cpu()], atol=2e-5, rtol=0)
+            torch.testing.assert_close(loss1.detach().cpu(), want.detach(), atol=1e-6, rtol=1e-5)
+            assert _rel_l2(leaf1.grad.cpu(), cpu_leaf.grad) < 2e-5
+    # an upstream gradient other than 1 scales the fp32 buffer in place
+    leaf1 = logits.detach().clone().requires_grad_(True)
+    loss1, _, _, _ = amd.grpo_loss_from_logits(leaf1, ids, adv, mask, temperature=0.9, **kw)
+    (loss1 * 3.0).backward()
+    assert _rel_l2(leaf1.grad, 3.0 * leaf.grad) < 2e-5
+    amd.check_device_errors()
+
+
 def test_unsupported_configurations_raise(amd):
     logits, ids, mask, adv, _ = _inputs(2, 4, 1024)
     assert amd.grpo_single_pass_supported(logits)
-    assert not amd.grpo_single_pass_supported(logits.float())
+    assert amd.grpo_single_pass_supported(logits.float()) and not amd.grpo_single_pass_supported(logits.double())
+    assert not amd.grpo_single_pass_supported(logits.float()[..., :1022])
     assert not amd.grpo_single_pass_supported(logits, "vespo")
     assert not amd.grpo_single_pass_supported(logits, "dapo", "sequence")
     assert amd.grpo_single_pass_supported(logits, entropy_coef=0.01)
@@ -301,7 +350,7 @@ def test_unsupported_configurations_raise(amd):
     big = torch.empty((1, 2, amd.ops.grpo_fused_max_vocab(torch.bfloat16) + 8), dtype=torch.bfloat16, device=DEV)
     assert not amd.grpo_single_pass_supported(big)
     with pytest.raises(NotImplementedError):
-        amd.grpo_loss_from_logits(logits.float(), ids, adv, mask, loss_type="bnpo")
+        amd.grpo_loss_from_logits(logits.double(), ids, adv, mask, loss_type="bnpo")
     with pytest.raises(KeyError):
         amd.grpo_loss_from_logits(logits, ids, adv, mask, loss_type="dapo")
     with pytest.raises(KeyError):
@@ -445,7 +494,8 @@ def _round_to(t, dtype):
     return t.to(dtype).float()
 
 
-def test_golden_vectors_go_through_the_single_pass_kernel(amd, monkeypatch):
+@pytest.mark.parametrize("keep_fp32", [False, True], ids=["as16bit", "as_fp32"])
+def test_golden_vectors_go_through_the_single_pass_kernel(amd, monkeypatch, keep_fp32):
     """`tests/golden/grpo_single_pass.*`: the reference's `GRPOTrainer._compute_loss` + backward on a mocked trainer
     (trl/trainer/grpo_trainer.py:2991-3260), for every configuration the one-pass kernel takes, on vocabularies
     that are multiples of 8.  The fixture's fp32 logits hold bf16-exact (or fp16-exact) values, so the reference did
@@ -453,7 +503,8 @@ def test_golden_vectors_go_through_the_single_pass_kernel(amd, monkeypatch):
     entropies are held to fp32 bars, and the gradient to the reference's gradient ROUNDED to the 16-bit dtype (what
     an exact kernel would store).  Two cases ran the reference in true bf16 / fp16 arithmetic (its log-probs are
     rounded to 16 bits) and are comparable at 2e-2 only.  The call into the one-pass kernel is counted: a case
-    that falls back to the two-pass path fails."""
+    that falls back to the two-pass path fails.  `as_fp32`: the fixture's fp32 logits go in as they are, which is
+    the very computation the reference ran: loss, metrics and the fp32 gradient are held to fp32 bars."""
     from conftest import fake_grpo_trainer, load_golden
     from types import SimpleNamespace
 
@@ -477,9 +528,13 @@ def test_golden_vectors_go_through_the_single_pass_kernel(amd, monkeypatch):
         c = f"c{case['id']}_"
         B, P, T, V = case["shape"]
         true_low = "dtype" in case
+        if true_low and keep_fp32:
+            continue  # (the reference ran these two in 16-bit arithmetic)
         dtype = getattr(torch, case["dtype"] if true_low else case["values"])
         logits32 = torch.from_numpy(g[c + "logits"])
         assert torch.equal(logits32.to(dtype).float(), logits32)  # the 16-bit tensor holds the reference's inputs exactly
+        if keep_fp32:
+            dtype = torch.float32
         tr = fake_grpo_trainer(amd, case, T, skip_masked=True, single_pass=True)
         tr.trl_amd_single_pass_fp16 = True  # (fp16 logits take the one pass only with a gradient scaler or on request)
         leaf = logits32.to(dtype).to(DEV).requires_grad_(True)
@@ -513,6 +568,8 @@ def test_golden_vectors_go_through_the_single_pass_kernel(amd, monkeypatch):
         assert float(got_g[~full].abs().max()) == 0.0 and float(want_g[~full].abs().max()) == 0.0, name
         if true_low:
             assert _rel_l2(got_g, want_g) < 2e-2, (name, _rel_l2(got_g, want_g))
+        elif keep_fp32:
+            assert _rel_l2(got_g, want_g) < 2e-5, (name, _rel_l2(got_g, want_g))
         else:
             # against what an exact kernel would store: the fp32 gradient rounded once to the logits dtype
             exact = _round_to(want_g, dtype)
@@ -530,7 +587,10 @@ def test_golden_vectors_go_through_the_single_pass_kernel(amd, monkeypatch):
                 torch.testing.assert_close(tr._entropy_window_stats.cpu(), torch.tensor(want["window"]), rtol=1e-5, atol=1e-4)
         seen.add((case["loss_type"], str(dtype)))
     for lt in ("dapo", "grpo", "dr_grpo", "bnpo", "cispo", "sapo"):
-        assert (lt, "torch.bfloat16") in seen and (lt, "torch.float16") in seen
+        if keep_fp32:
+            assert (lt, "torch.float32") in seen
+        else:
+            assert (lt, "torch.bfloat16") in seen and (lt, "torch.float16") in seen
     amd.check_device_errors()
 
 

@@ -229,7 +229,7 @@ def test_advantages_against_the_oracle(amd):
 
 def test_single_pass_kernel_against_the_two_pass_path(amd):
     """250 configurations the single-pass kernel takes (loss types, KL, delta, bias-corrected KL, token weights,
-    per-token advantages, entropy bonus, temperatures, bf16 / fp16, vocabularies 8 ... 20488 and one whose rows overflow
+    per-token advantages, entropy bonus, temperatures, bf16 / fp16 / fp32, vocabularies 8 ... 20488 and one whose rows overflow
     into LDS, empty sequences, ragged
     masks): loss, metrics, log-probs and dlogits against K1 + loss kernel + K3."""
     rnd = random.Random(2)
@@ -237,7 +237,9 @@ def test_single_pass_kernel_against_the_two_pass_path(amd):
     for case in range(250):
         B, K, V = rnd.choice([1, 2, 5]), rnd.choice([1, 7, 33]), rnd.choice([8, 64, 264, 1000, 4096, 20488, 172040])
         L = K + rnd.choice([1, 1, 3])
-        dt = rnd.choice([torch.bfloat16, torch.float16])
+        dt = rnd.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+        if dt == torch.float32 and V > 167936:  # (fp32 rows hold half as many logits)
+            V = 83976
         lt = rnd.choice(["grpo", "bnpo", "dr_grpo", "dapo", "cispo", "sapo"])
         beta, T = rnd.choice([0.0, 0.04]), rnd.choice([1.0, 0.7, 1.3])
         logits = (rnd.choice([0.5, 2.0, 6.0]) * torch.randn(B, L, V, device=DEV)).to(dt)
@@ -270,7 +272,7 @@ def test_single_pass_kernel_against_the_two_pass_path(amd):
         if bool(m.any()):
             assert float((lp1[m] - lp2.detach()[m]).abs().max()) <= 2e-5 * max(1.0, float(lp2.detach()[m].abs().max())), what
         if float(leaf2.grad.float().abs().max()) > 0:
-            assert _rel(leaf1.grad, leaf2.grad) < 4e-3, what
+            assert _rel(leaf1.grad, leaf2.grad) < (2e-5 if dt == torch.float32 else 4e-3), what
         else:
             assert float(leaf1.grad.float().abs().max()) == 0.0, what
     amd.check_device_errors()

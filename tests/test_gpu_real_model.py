@@ -123,7 +123,7 @@ def test_grpo_compute_loss_through_a_real_model(amd, base_model, dtype, loss_typ
     loss = tr._compute_loss(model, inputs)
     loss.backward()
     got_loss, got = float(loss.detach()), _grads(model)
-    assert len(calls) == (1 if dtype == torch.bfloat16 else 0)  # 16-bit logits take the single pass, fp32 two passes
+    assert len(calls) == 1  # the single pass, for fp32 logits as for bf16 ones
 
     host = {k: v.cpu() for k, v in inputs.items()}
 

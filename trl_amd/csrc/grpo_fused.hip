@@ -4,7 +4,7 @@
 // between them.  For the token-level GRPO losses the gradient coefficient of a token depends only on that
 // token's own log-prob, on per-token inputs (old / reference log-probs, advantage, mask, weight) and on
 // normalisers that are known from the mask before any logit is read.  A 1024-lane workgroup can hold a whole
-// vocabulary row of 16-bit logits in registers (up to kMaxVec 16-byte vectors per lane), so one workgroup
+// vocabulary row of logits in registers (up to kMaxVec 16-byte vectors per lane: 8 16-bit or 4 fp32 logits each), so one workgroup
 // per row loads the row once, reduces it to (lse, entropy, target logit), evaluates the token's loss terms
 // with the same device functions as the [B, T]-sized loss kernel, and writes the row's dlogits from the
 // registers.  Rows outside the completion mask are never read: their gradient row is zero-filled and their
@@ -25,8 +25,9 @@ constexpr int kVecStep = 4;  // the kernel is built for 4, 8, ... kMaxVec vector
 constexpr int kMaxLdsVec = 9, kLdsStep = 3;
 // Rows longer still (the 256000- and 262144-entry vocabularies) read their last vectors twice: once ahead of the row
 // for the sums, once after it for the gradient, by which time the workgroup has read them so recently that they
-// come from the L2.  Up to kMaxExtraVec such vectors per lane: rows of up to 37 * 1024 * 8 = 303104 logits.
-constexpr int kMaxExtraVec = 8;
+// come from the L2.  Up to kMaxExtraVec such vectors per lane: rows of up to 41 * 1024 * 8 = 335872 16-bit logits
+// (half as many fp32 ones).
+constexpr int kMaxExtraVec = 12;  // (37 on-chip + extra vectors x 1024 x 4 fp32 logits covers the 151936-entry rows in fp32 too)
 constexpr int kWideVec = kMaxVec;  // register vectors of the builds with vectors in LDS
 
 typedef __attribute__((address_space(1))) const u32x4 GlobalVecIn;
@@ -487,24 +488,30 @@ using namespace trlk;
 
 extern "C" int trlk_scale_unless_one(void* d_data, int dtype, int64_t n_elems, const float* d_scale, trlk_stream_t stream) {
     clear_error();
-    TRLK_REQUIRE(dtype == TRLK_BF16 || dtype == TRLK_F16, TRLK_ERR_BAD_DTYPE, "scale_unless_one: 16-bit data only");
-    TRLK_REQUIRE(n_elems >= 0 && n_elems % 8 == 0, TRLK_ERR_BAD_SHAPE, "scale_unless_one: element count must be a multiple of 8");
+    TRLK_REQUIRE(dtype == TRLK_BF16 || dtype == TRLK_F16 || dtype == TRLK_F32, TRLK_ERR_BAD_DTYPE,
+                 "scale_unless_one: bf16, fp16 or fp32 data (dtype code %d)", dtype);
+    const int64_t epv = dtype == TRLK_F32 ? 4 : 8;
+    TRLK_REQUIRE(n_elems >= 0 && n_elems % epv == 0, TRLK_ERR_BAD_SHAPE,
+                 "scale_unless_one: element count must be a multiple of %lld", (long long)epv);
     if (n_elems == 0) return TRLK_OK;
     TRLK_REQUIRE(d_data && d_scale && reinterpret_cast<uintptr_t>(d_data) % 16 == 0, TRLK_ERR_NULL_POINTER,
                  "scale_unless_one: null or misaligned pointer");
-    const int64_t n_vec = n_elems / 8;
+    const int64_t n_vec = n_elems / epv;
     TRLK_REQUIRE(n_vec <= int64_t(kScaleSpanVec) * 0x7fffffff, TRLK_ERR_BAD_SHAPE, "scale_unless_one: too many elements");
     const unsigned grid = unsigned((n_vec + kScaleSpanVec - 1) / kScaleSpanVec);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == TRLK_BF16)
         hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_BF16>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, d_scale);
-    else
+    else if (dtype == TRLK_F16)
         hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_F16>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, d_scale);
+    else
+        hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_F32>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, d_scale);
     return launch_status("scale_unless_one");
 }
 
 extern "C" int64_t trlk_grpo_fused_max_vocab(int dtype) {
-    return dtype == TRLK_BF16 || dtype == TRLK_F16 ? int64_t(kWideVec + kMaxLdsVec + kMaxExtraVec) * kFThreads * 8 : 0;
+    const int64_t vectors = int64_t(kWideVec + kMaxLdsVec + kMaxExtraVec) * kFThreads;
+    return dtype == TRLK_BF16 || dtype == TRLK_F16 ? vectors * 8 : dtype == TRLK_F32 ? vectors * 4 : 0;
 }
 
 extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t n_seq, int64_t rows_per_seq, int64_t vocab,
@@ -519,12 +526,13 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
                                        int64_t out_row_stride, int compute_masked_rows, int32_t* d_error_flag,
                                        trlk_stream_t stream) {
     clear_error();
-    TRLK_REQUIRE(dtype == TRLK_BF16 || dtype == TRLK_F16, TRLK_ERR_BAD_DTYPE,
-                 "grpo_fused: 16-bit logits only (dtype code %d); use the two-pass path", dtype);
+    TRLK_REQUIRE(dtype == TRLK_BF16 || dtype == TRLK_F16 || dtype == TRLK_F32, TRLK_ERR_BAD_DTYPE,
+                 "grpo_fused: bf16, fp16 or fp32 logits (dtype code %d); use the two-pass path", dtype);
+    const int64_t es = int64_t(elem_size(dtype)), epv = 16 / es;
     TRLK_REQUIRE(n_seq >= 0 && rows_per_seq >= 0 && vocab >= 1, TRLK_ERR_BAD_SHAPE, "grpo_fused: bad sizes");
-    TRLK_REQUIRE(vocab % 8 == 0 && vocab <= trlk_grpo_fused_max_vocab(dtype), TRLK_ERR_UNSUPPORTED,
-                 "grpo_fused: vocab must be a multiple of 8 and at most %lld (got %lld); use the two-pass path",
-                 (long long)trlk_grpo_fused_max_vocab(dtype), (long long)vocab);
+    TRLK_REQUIRE(vocab % epv == 0 && vocab <= trlk_grpo_fused_max_vocab(dtype), TRLK_ERR_UNSUPPORTED,
+                 "grpo_fused: vocab must be a multiple of %lld and at most %lld (got %lld); use the two-pass path",
+                 (long long)epv, (long long)trlk_grpo_fused_max_vocab(dtype), (long long)vocab);
     TRLK_REQUIRE(out_row_offset >= 0 && out_row_offset + rows_per_seq <= out_rows_per_seq, TRLK_ERR_BAD_SHAPE,
                  "grpo_fused: input rows [%lld, %lld) do not fit the %lld output rows per sequence",
                  (long long)out_row_offset, (long long)(out_row_offset + rows_per_seq), (long long)out_rows_per_seq);
@@ -544,8 +552,8 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
                      "grpo_fused: the weighted log-prob term needs seq_coef");
         TRLK_REQUIRE(row_stride >= vocab || rows_per_seq <= 1, TRLK_ERR_BAD_STRIDE, "grpo_fused: rows overlap");
     }
-    const auto al16 = [](const void* p, int64_t s0, int64_t s1) {
-        return reinterpret_cast<uintptr_t>(p) % 16 == 0 && (s0 * 2) % 16 == 0 && (s1 * 2) % 16 == 0;
+    const auto al16 = [es](const void* p, int64_t s0, int64_t s1) {
+        return reinterpret_cast<uintptr_t>(p) % 16 == 0 && (s0 * es) % 16 == 0 && (s1 * es) % 16 == 0;
     };
     TRLK_REQUIRE(al16(d_logits, seq_stride, row_stride) && al16(d_dlogits, out_seq_stride, out_row_stride),
                  TRLK_ERR_BAD_STRIDE, "grpo_fused: logits and dlogits rows must be 16-byte aligned; use the two-pass path");
@@ -586,9 +594,10 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
     a.error_flag = d_error_flag;
     a.all_rows = compute_masked_rows != 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const int nvec = int((vocab / 8 + kFThreads - 1) / kFThreads);  // 16-byte vectors of the row per lane
-    if (int rc = dtype == TRLK_BF16 ? launch_fused<TRLK_BF16>(a, nvec, unsigned(orows), s)
-                                    : launch_fused<TRLK_F16>(a, nvec, unsigned(orows), s))
+    const int nvec = int((vocab / epv + kFThreads - 1) / kFThreads);  // 16-byte vectors of the row per lane
+    if (int rc = dtype == TRLK_BF16  ? launch_fused<TRLK_BF16>(a, nvec, unsigned(orows), s)
+                 : dtype == TRLK_F16 ? launch_fused<TRLK_F16>(a, nvec, unsigned(orows), s)
+                                     : launch_fused<TRLK_F32>(a, nvec, unsigned(orows), s))
         return rc;
     return launch_status("grpo_fused");
 }

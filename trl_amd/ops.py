@@ -477,7 +477,7 @@ def grpo_loss_static_(
 # --------------------------------------------------------------------------------------------
 def grpo_fused_max_vocab(dtype: torch.dtype) -> int:
     """Largest vocabulary the single-pass kernel takes for this dtype (0: not supported)."""
-    return int(lib.trlk_grpo_fused_max_vocab(dtype_code(dtype))) if dtype in (torch.bfloat16, torch.float16) else 0
+    return int(lib.trlk_grpo_fused_max_vocab(dtype_code(dtype))) if dtype in (torch.bfloat16, torch.float16, torch.float32) else 0
 
 
 def grpo_fused_fwd_bwd(
@@ -487,7 +487,7 @@ def grpo_fused_fwd_bwd(
     use_bias_correction_kl: bool, sapo_temperature_pos: float, sapo_temperature_neg: float,
     compute_masked_rows: bool = False, entropy_weight: Optional[Tensor] = None,
 ) -> tuple[Tensor, Tensor, Tensor, Tensor]:
-    """One pass over `logits[:, keep_start : keep_start + keep_len]` (`[B, L, V]`, 16-bit): returns
+    """One pass over `logits[:, keep_start : keep_start + keep_len]` (`[B, L, V]`, bf16 / fp16 / fp32): returns
     `(logp [B, K], entropy [B, K], lse [B, K], dlogits [B, L, V])`, the gradient for an upstream gradient of 1 on
     the loss whose per-sequence normalisation is `row_scale [B]`.  Rows with `mask == 0` are not read (outputs 0)
     unless `compute_masked_rows`.  `entropy_weight [B, K]` is d loss / d entropy per token (entropy bonus)."""
@@ -540,10 +540,10 @@ def grpo_fused_fwd_bwd(
 
 
 def scale_unless_one_(data: Tensor, scale: Tensor) -> Tensor:
-    """In place `data *= scale` for a contiguous 16-bit tensor and a one-element device scalar; when the scalar is
-    exactly 1 the launched kernel touches nothing (no host synchronisation either way)."""
-    if not data.is_contiguous() or data.dtype not in (torch.bfloat16, torch.float16):
-        raise ValueError("scale_unless_one_: contiguous bf16/fp16 data expected")
+    """In place `data *= scale` for a contiguous bf16 / fp16 / fp32 tensor and a one-element device scalar; when the
+    scalar is exactly 1 the launched kernel touches nothing (no host synchronisation either way)."""
+    if not data.is_contiguous() or data.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise ValueError("scale_unless_one_: contiguous bf16 / fp16 / fp32 data expected")
     scale = scale.reshape(1).to(device=data.device, dtype=torch.float32)
     with torch.cuda.device(data.device):
         check(lib.trlk_scale_unless_one(data.data_ptr(), dtype_code(data.dtype), data.numel(), ptr(scale),

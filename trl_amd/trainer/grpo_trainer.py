@@ -238,18 +238,19 @@ def grpo_single_pass_supported(logits: Tensor, loss_type: str = "dapo", importan
                                entropy_coef: float = 0.0, entropy_mask: Tensor | None = None) -> bool:
     """Whether `grpo_loss_from_logits` can go from these logits to their gradient in one pass: a token-level
     loss type, with or without entropy bonus but without an entropy-quantile mask (the gradient coefficients of
-    a token then depend on nothing but that token), 16-bit logits whose rows the kernel takes (`ops.grpo_fused_max_vocab`) and
-    are 16-byte aligned."""
+    a token then depend on nothing but that token), bf16 / fp16 / fp32 logits whose rows the kernel takes
+    (`ops.grpo_fused_max_vocab`) and are 16-byte aligned."""
     if loss_type not in _SINGLE_PASS_LOSS_TYPES or importance_sampling_level != "token":
         return False
     if entropy_mask is not None:  # (a mask derived from every token's entropy needs the forward pass first)
         return False
-    if logits.dim() != 3 or not logits.is_cuda or logits.dtype not in (torch.bfloat16, torch.float16):
+    if logits.dim() != 3 or not logits.is_cuda or logits.dtype not in (torch.bfloat16, torch.float16, torch.float32):
         return False
     vocab = logits.shape[-1]
-    if vocab % 8 != 0 or vocab > ops.grpo_fused_max_vocab(logits.dtype) or (vocab > 1 and logits.stride(-1) != 1):
+    per_vector = 16 // logits.element_size()
+    if vocab % per_vector != 0 or vocab > ops.grpo_fused_max_vocab(logits.dtype) or (vocab > 1 and logits.stride(-1) != 1):
         return False
-    return logits.data_ptr() % 16 == 0 and logits.stride(0) % 8 == 0 and logits.stride(1) % 8 == 0
+    return logits.data_ptr() % 16 == 0 and logits.stride(0) % per_vector == 0 and logits.stride(1) % per_vector == 0
 
 
 class _GRPOFromLogits(torch.autograd.Function):
@@ -397,8 +398,9 @@ def grpo_loss_from_logits(
     if not grpo_single_pass_supported(logits, loss_type):
         raise NotImplementedError(
             "grpo_loss_from_logits: this configuration needs the two-pass path (per_token_logps_and_entropies + "
-            "grpo_loss): token-level loss types, 16-bit logits, vocab % 8 == 0 and at most "
-            f"{ops.grpo_fused_max_vocab(logits.dtype) if logits.dtype in (torch.bfloat16, torch.float16) else 0}")
+            "grpo_loss): token-level loss types, bf16 / fp16 / fp32 logits in rows of whole 16-byte vectors, at most "
+            f"{ops.grpo_fused_max_vocab(logits.dtype) if logits.dtype in (torch.bfloat16, torch.float16, torch.float32) else 0} "
+            "entries long")
     if beta != 0.0 and ref_per_token_logps is None:
         raise KeyError("ref_per_token_logps")
     if ops.LOSS_TYPES[loss_type][0] == _lib.DAPO and num_items_in_batch is None:
