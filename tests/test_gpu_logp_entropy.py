@@ -422,3 +422,54 @@ def test_row_statistics_of_the_same_pass():
         lp2, ent2, lse2 = ops.logp_entropy_fwd(logits.to(DEV), ids.reshape(-1, 1).to(DEV), 1.0, 0, L,
                                                mask.reshape(-1).to(DEV))
         assert torch.equal(logp, lp2) and torch.equal(ent, ent2) and torch.equal(lse, lse2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "fp16"])
+def test_rows_that_are_not_whole_vectors(amd, dtype):
+    """Vocabularies that are no multiple of the 16-byte vector (a tokenizer with a few added tokens: 32001, 50257,
+    128257 ...): every row then starts at another alignment; the kernels peel it to its first 16-byte boundary, take
+    aligned vectors from there and finish element by element.  Targets, duplicate targets and the row maximum are put
+    into the peeled head, into the body and into the last elements of rows at every alignment; vocabularies around one
+    and several gradient chunks; forward, row statistics and gradient against torch in fp64."""
+    import torch.nn.functional as F
+
+    from trl_amd import ops
+
+    per_vec = 16 // torch.empty((), dtype=dtype).element_size()
+    chunk = 8192 // torch.empty((), dtype=dtype).element_size()  # elements per gradient workgroup
+    for V in (1, 3, per_vec - 1, per_vec + 1, 41, 2 * per_vec + 3, chunk + 3, chunk + per_vec + 1, 2 * chunk - 1, 32001, 50257):
+        n_seq, L = 2, 9  # 18 rows: every row alignment of an odd vocabulary occurs
+        g = torch.Generator(device=DEV).manual_seed(V)
+        logits = (3.0 * torch.randn((n_seq, L, V), generator=g, device=DEV)).to(dtype)
+        K = 3
+        index = torch.randint(0, V, (n_seq, L, K), generator=g, device=DEV)
+        index[:, :, 0] = torch.arange(L, device=DEV)[None].clamp(max=V - 1)  # positions 0 .. 8: inside every possible head
+        index[:, 1::2, 1] = V - 1 - torch.arange(L, device=DEV)[None, 1::2].clamp(max=V - 1) % min(V, per_vec)  # the last elements
+        index[:, ::3, 2] = index[:, ::3, 0]  # a duplicate target
+        peak = index[:, :, 0].clone()
+        peak[:, 2::3] = index[:, 2::3, 1]
+        logits.scatter_(-1, peak.unsqueeze(-1), 40.0)  # the row maximum sits on the first target of most rows
+        leaf = logits.detach().clone().requires_grad_(True)
+        lp, ent = amd.logps_and_entropies(leaf, index, 0.8)
+        ref = logits.detach().double().requires_grad_(True)
+        lsm = F.log_softmax(ref / 0.8, -1)
+        want_lp, want_h = lsm.gather(-1, index), -(lsm.exp() * lsm).sum(-1)
+        assert float((lp.detach().double() - want_lp.detach()).abs().max()) <= 2e-5 * 50, V
+        assert float((ent.detach().double() - want_h.detach()).abs().max()) <= 2e-5 * 50, V
+        gl, gh = torch.randn(lp.shape, generator=g, device=DEV, dtype=torch.float64), torch.randn(ent.shape, generator=g, device=DEV, dtype=torch.float64)
+        ((lp.double() * gl).sum() + (ent.double() * gh).sum()).backward()
+        ((want_lp * gl).sum() + (want_h * gh).sum()).backward()
+        bar = {torch.float32: 2e-5, torch.bfloat16: 4e-3, torch.float16: 1e-3}[dtype]
+        if V == 1:  # (no gradient in exact arithmetic: g * (1 - p) with p one rounding away from 1)
+            assert float(leaf.grad.double().abs().max()) <= bar * float(gl.abs().max() + gh.abs().max()), V
+        else:
+            err = float((leaf.grad.double() - ref.grad).norm() / ref.grad.norm())
+            assert err <= bar, (V, err)
+        # row statistics: mean logit, and whether the first target is the row's arg-max (first maximal position)
+        idx = index.reshape(n_seq * L, K)
+        _, _, _, stats = ops.logp_entropy_stats_fwd(logits, idx, 1.0, 0, L, None)
+        x = logits.double()
+        assert float((stats[:, 0].double() - x.mean(-1).reshape(-1)).abs().max()) <= 1e-4 * 50, V
+        want_hit = (x.argmax(-1) == index[:, :, 0]).reshape(-1)
+        assert torch.equal(stats[:, 2] != 0, want_hit), V
+    amd.check_device_errors()

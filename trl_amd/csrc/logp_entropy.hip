@@ -37,14 +37,28 @@ constexpr int kUnroll = TRLK_FWD_UNROLL;
 static_assert(kUnroll >= 2, "the row tail of the forward holds up to kUnroll - 1 vectors per lane");
 constexpr int kBwdUnroll = TRLK_BWD_UNROLL;
 
-template <bool NT>
-__device__ __forceinline__ u32x4 stream_load(const u32x4* p) {
+// A 16-byte vector at any element alignment: rows whose length is no multiple of the vector width start at 2- or
+// 4-byte aligned addresses.  The hardware takes such accesses as they are (one instruction; a wave's kilobyte then
+// touches nine cache lines instead of eight).
+typedef u32x4 u32x4_u __attribute__((aligned(2)));
+template <bool ALIGNED>
+struct VecOf {
+    typedef u32x4 type;
+};
+template <>
+struct VecOf<false> {
+    typedef u32x4_u type;
+};
+
+template <bool NT, typename V>
+__device__ __forceinline__ u32x4 stream_load(const V* p) {
     if constexpr (NT)
         return __builtin_nontemporal_load(p);
     else
         return *p;
 }
-__device__ __forceinline__ void stream_store(u32x4 v, u32x4* p) {
+template <typename V>
+__device__ __forceinline__ void stream_store(u32x4 v, V* p) {
 #if TRLK_NT_STORE
     __builtin_nontemporal_store(v, p);
 #else
@@ -126,7 +140,8 @@ __device__ __forceinline__ float max_of(const float* x) {
     return a;
 }
 
-// VEC: rows are 16-byte aligned and vocab is a multiple of the vector width.
+// VEC: rows are 16-byte aligned and vocab is a multiple of the vector width.  Otherwise a row is read in aligned
+// vectors from its first 16-byte boundary on, and the few elements before that and after the last whole vector one by one.
 // STATS: also produce the row statistics of `out_stats`.
 template <int DT, bool VEC, bool STATS>
 __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
@@ -203,10 +218,22 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
             acc.add(x, c);
         }
     };
-    if constexpr (VEC) {
+    {
         constexpr int EPV = E::EPV;
-        const u32x4* vp = reinterpret_cast<const u32x4*>(base);
-        const int nvec = int(V / EPV);
+        // Rows that are not whole aligned vectors (not VEC): the `head` elements before the row's first 16-byte
+        // boundary go one by one (first: a lane's positions must come in increasing order), then aligned vectors,
+        // then what is left after the last whole one.
+        const int head = VEC ? 0 : int(min(V, int64_t(((16 - (reinterpret_cast<uintptr_t>(base) & 15)) & 15) / sizeof(T))));
+        if constexpr (!VEC) {
+            if (tid < head) {
+                const float x = E::load1(base + tid);
+                raise(x);
+                add(x);
+                if constexpr (STATS) stat_elem(x, tid);
+            }
+        }
+        const u32x4* vp = reinterpret_cast<const u32x4*>(base + head);
+        const int nvec = int((V - head) / EPV);
         int v = tid;
         for (; v + (kUnroll - 1) * kThreads < nvec; v += kUnroll * kThreads) {
             u32x4 q[kUnroll];
@@ -228,7 +255,7 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
             if constexpr (STATS) {
 #pragma unroll
                 for (int j = 0; j < kUnroll; ++j)  // increasing positions: j-th vector before the (j+1)-th
-                    stat_vec(x + j * EPV, int64_t(v + j * kThreads) * EPV, EPV, bmj[j]);
+                    stat_vec(x + j * EPV, head + int64_t(v + j * kThreads) * EPV, EPV, bmj[j]);
             }
         }
         // the row's tail: fewer than kUnroll vectors are left for this lane; their loads go out together
@@ -248,16 +275,17 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
                     raise(bm);
 #pragma unroll
                     for (int i = 0; i < EPV; ++i) add(x[i]);
-                    if constexpr (STATS) stat_vec(x, int64_t(v + j * kThreads) * EPV, EPV, bm);
+                    if constexpr (STATS) stat_vec(x, head + int64_t(v + j * kThreads) * EPV, EPV, bm);
                 }
             }
         }
-    } else {
-        for (int64_t v = tid; v < V; v += kThreads) {
-            const float x = E::load1(base + v);
-            raise(x);
-            add(x);
-            if constexpr (STATS) stat_elem(x, v);
+        if constexpr (!VEC) {  // what is left of the row after its whole vectors (these positions come last for a lane)
+            for (int64_t e = head + int64_t(nvec) * EPV + tid; e < V; e += kThreads) {
+                const float x = E::load1(base + e);
+                raise(x);
+                add(x);
+                if constexpr (STATS) stat_elem(x, e);
+            }
         }
     }
 
@@ -377,9 +405,16 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_bwd_kernel(BwdArgs a, i
     const int64_t b = orow / a.out_rows_per_seq;
     const int64_t to = orow - b * a.out_rows_per_seq;
     const int64_t t = to - a.out_row_offset;
-    const int e0 = chunk * CE;                                   // first element of this chunk
-    const int e1 = int(a.vocab < int64_t(e0) + CE ? a.vocab : int64_t(e0) + CE);
     T* out = static_cast<T*>(a.dlogits) + b * a.out_seq_stride + to * a.out_row_stride;
+    // Rows that are not whole aligned vectors (not VEC) are walked from the first 16-byte boundary of the OUTPUT row:
+    // the `head` elements before it and what is left after the last whole vector go one by one, the vectors between
+    // through accesses that need no alignment (when the logits row sits like the gradient row -- two contiguous
+    // tensors of one shape -- both sides are in fact aligned).  The chunks count from that boundary.
+    const int head = VEC ? 0 : int(min(a.vocab, int64_t(((16 - (reinterpret_cast<uintptr_t>(out) & 15)) & 15) / sizeof(T))));
+    const int body = int(a.vocab) - head;
+    const int e0 = chunk * CE;                                   // first element of this chunk, counted from `head`
+    const int e1 = max(e0, body < e0 + CE ? body : e0 + CE);     // (an empty range in a last chunk that the head made superfluous)
+    out += head;
 
     // Everything below up to the streaming loop is uniform over the workgroup (scalar loads).
     bool live = t >= 0 && t < a.rows_per_seq;
@@ -397,17 +432,19 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_bwd_kernel(BwdArgs a, i
     }
     const float h = (HAS_H && live) ? a.g_entropy[row] : 0.f;
     live = live && (any || h != 0.f);
+    typedef typename VecOf<VEC>::type Vec;  // (not VEC: whole vectors through unaligned accesses, the row's last elements one by one)
+    const int v_end = e1 / E::EPV;          // whole vectors of the row end here (e1 is the row's end in its last chunk)
     if (!live) {  // outside the kept window, or all upstream gradients are zero: zero-fill
-        if constexpr (VEC) {
-            u32x4* op = reinterpret_cast<u32x4*>(out);
-            const u32x4 z = {0u, 0u, 0u, 0u};
-            for (int v = e0 / E::EPV + tid; v < e1 / E::EPV; v += kThreads) stream_store(z, op + v);
-        } else {
-            for (int e = e0 + tid; e < e1; e += kThreads) E::store1(out + e, 0.f);
+        Vec* op = reinterpret_cast<Vec*>(out);
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        for (int v = e0 / E::EPV + tid; v < v_end; v += kThreads) stream_store(z, op + v);
+        if constexpr (!VEC) {
+            for (int e = v_end * E::EPV + tid; e < e1; e += kThreads) E::store1(out + e, 0.f);
+            if (chunk == 0 && tid < head) E::store1(out - head + tid, 0.f);
         }
         return;
     }
-    const T* base = static_cast<const T*>(a.logits) + b * a.seq_stride + t * a.row_stride;
+    const T* base = static_cast<const T*>(a.logits) + b * a.seq_stride + t * a.row_stride + head;
     const float c = kLog2e * inv_t;
     const float lsec = a.lse[row] * kLog2e;
     // dz_v = p_v * (a0 + b0 * tt),  tt = x*c - lse*log2e = (z - lse) * log2e
@@ -422,11 +459,11 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_bwd_kernel(BwdArgs a, i
         return with_h ? p * fmaf(b0, tt, a0) : p * a0;
     };
 
-    if constexpr (VEC) {
+    {
         constexpr int EPV = E::EPV;
-        const u32x4* vp = reinterpret_cast<const u32x4*>(base);
-        u32x4* op = reinterpret_cast<u32x4*>(out);
-        const int v0 = e0 / EPV + tid, v_end = e1 / EPV;
+        const Vec* vp = reinterpret_cast<const Vec*>(base);
+        Vec* op = reinterpret_cast<Vec*>(out);
+        const int v0 = e0 / EPV + tid;
         auto one_vector = [&](u32x4 q, int v) {
             float x[EPV], d[EPV];
             E::unpack(q, x);
@@ -443,22 +480,29 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_bwd_kernel(BwdArgs a, i
         } else {
             for (int v = v0; v < v_end; v += kThreads) one_vector(stream_load<kBwdNt>(vp + v), v);
         }
-    } else {
-        for (int e = e0 + tid; e < e1; e += kThreads) E::store1(out + e, grad_of(E::load1(base + e)));
+        if constexpr (!VEC) {
+            for (int e = v_end * EPV + tid; e < e1; e += kThreads) E::store1(out + e, grad_of(E::load1(base + e)));
+            if (chunk == 0 && tid < head) E::store1(out - head + tid, grad_of(E::load1(base - head + tid)));
+        }
     }
     // One-hot terms.  The streaming part above wrote only the softmax term; the lane that stored
     // the element at index[k] now rewrites it with the gathered gradients added (a later store of
     // the same lane to the same address is ordered after the first).  Entries of one row that
     // share an index are summed in k order by the first of them.
-    constexpr int kElemsPerLaneStep = VEC ? E::EPV : 1;
     for (int k = 0; k < K; ++k) {
-        const int64_t idx = a.index[row * K + k];
-        if (idx < e0 || idx >= e1) continue;  // also drops indices outside [0, vocab)
-        if (int((idx - e0) / kElemsPerLaneStep) % kThreads != tid) continue;
+        const int64_t idx = a.index[row * K + k] - head;  // counted from `head` like the chunks
+        // this chunk's elements, or (chunk 0) the head; also drops indices outside [0, vocab)
+        const bool in_head = !VEC && chunk == 0 && idx < 0 && idx >= -int64_t(head);
+        if (!in_head && (idx < e0 || idx >= e1)) continue;
+        // (whole vectors: lane (vector number in the chunk) mod kThreads; the elements before and after them: one lane each)
+        const int owner = in_head ? int(idx + head)
+                                  : idx < int64_t(v_end) * E::EPV ? int((idx - e0) / E::EPV) % kThreads
+                                                                  : int(idx - int64_t(v_end) * E::EPV);
+        if (owner != tid) continue;
         float add = 0.f;
         bool first = true;
         for (int j = 0; j < K; ++j) {
-            if (a.index[row * K + j] != idx) continue;
+            if (a.index[row * K + j] - head != idx) continue;
             if (j < k) first = false;
             add += a.g_logp[row * K + j] * inv_t;
         }
