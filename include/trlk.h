@@ -337,9 +337,10 @@ int trlk_gemm_nt(const void* d_a, int64_t lda, const void* d_b, int64_t ldb, int
  *   d_entropy_weight fp32 [n_seq, rows_per_seq] or NULL = d loss / d entropy of each token (the entropy bonus of
  *   grpo_trainer.py:3155-3181 with its normaliser folded in);
  *   the other per-token inputs, the policy terms and their parameters are those of trlk_grpo_loss.
- * bf16, fp16 or fp32 logits, rows of whole 16-byte vectors, vocab <= trlk_grpo_fused_max_vocab(dtype) (a row is held
+ * bf16, fp16 or fp32 logits, vocab <= trlk_grpo_fused_max_vocab(dtype) (a row is held
  * in the registers of one workgroup, the end of a row of more than 163840 logits in its LDS, and what
- * lies beyond 237568 logits is read twice), rows 16-byte aligned.  Outputs: log-prob, entropy and lse of
+ * lies beyond 237568 logits is read twice); rows that are not whole aligned 16-byte vectors are peeled to
+ * their alignment (at least two vectors' worth of entries then).  Outputs: log-prob, entropy and lse of
  * every row of the completion mask (the others are not read and yield 0, unless compute_masked_rows
  * asks for their outputs too), and the full
  * [n_seq, out_rows_per_seq, vocab] gradient laid out as trlk_logp_entropy_bwd writes it, for an

@@ -100,12 +100,12 @@ def test_host_side_argument_validation():
     assert lib.trlk_grpo_fused_max_vocab(_lib.BF16) == 41 * 1024 * 8 and lib.trlk_grpo_fused_max_vocab(_lib.F32) == 41 * 1024 * 4
     assert lib.trlk_grpo_fused_max_vocab(99) == 0
     assert fused(dtype=99) == -3 and "two-pass" in _lib.last_error()
-    assert fused(vocab=4100) == -7 and fused(vocab=41 * 1024 * 8 + 8) == -7
-    assert fused(logits=fake16 + 2) == -4 and fused(row_stride=4100) == -4
+    assert fused(vocab=12) == -7 and fused(vocab=41 * 1024 * 8 + 8) == -7  # (4100 would go ahead: rows need not be whole vectors)
+    assert fused(logits=fake16 + 1) == -4  # (not even aligned to an element; 2-byte aligned rows are taken)
     assert fused(beta=0.1) == -1 and fused(term=9) == -5
     assert fused(out_rows=3) == -2 and fused(out_rows=8, offset=5) == -2
     assert lib.trlk_scale_unless_one(fake16, 99, 64, fake, None) == -3
-    assert lib.trlk_scale_unless_one(fake16, _lib.BF16, 60, fake, None) == -2
+    assert lib.trlk_scale_unless_one(fake16, _lib.BF16, -8, fake, None) == -2
     # fused head: fp32 operands, ragged hidden size, a stash whose rows are too short, missing workspace
 
     def head_fwd(dtype=_lib.BF16, h=64, stash=None, stash_ld=0, ws=fake16, ws_bytes=1 << 30):

@@ -337,16 +337,73 @@ def test_fp32_logits(amd):
     amd.check_device_errors()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "fp16", "fp32"])
+def test_rows_that_are_not_whole_vectors(amd, dtype):
+    """Vocabularies that are no multiple of the 16-byte vector (50257, 32001 and 151665 after a tokenizer gained
+    tokens; sizes that also overflow into LDS or are read twice at the end): every row sits at another alignment,
+    the kernel peels it to its first 16-byte boundary.  Targets in the peeled head, in the last elements and in
+    the body; entropy bonus on; a view whose rows are aligned while the gradient's are not.  Against the two-pass
+    path (itself checked against fp64 on such rows)."""
+    per_vec = 16 // torch.empty((), dtype=dtype).element_size()
+    sizes = [2 * per_vec + 1, 41, 1019, 32001, 50257, 151665]
+    sizes += [83971] if dtype == torch.float32 else [200067, 262147]
+    for V in sizes:
+        B, K = 3, 3
+        logits, ids, mask, adv, g = _inputs(B, K, V, dtype=dtype, seed=V % 79, extra_rows=1)
+        mask[:] = 1
+        mask[2, 1:] = 0
+        ids[0, 0], ids[0, 1], ids[0, 2] = 0, V - 1, V // 2
+        ids[1, 0], ids[1, 1], ids[1, 2] = min(3, V - 1), V - 2, 1
+        assert amd.grpo_single_pass_supported(logits)
+        kw = dict(loss_type="bnpo", beta=0.0, entropy_coef=0.02 if V % 2 else 0.0)
+        leaf = logits.detach().clone().requires_grad_(True)
+        lp_g, ent_g = amd.per_token_logps_and_entropies(leaf, ids, K, 0.9, True, True)
+        loss2, met2 = amd.grpo_loss(lp_g, adv, mask, entropies=ent_g, **kw)
+        loss2.backward()
+        leaf1 = logits.detach().clone().requires_grad_(True)
+        loss1, met1, lp1, ent1 = amd.grpo_loss_from_logits(leaf1, ids, adv, mask, temperature=0.9, **kw)
+        loss1.backward()
+        m = mask.bool()
+        torch.testing.assert_close(loss1, loss2, rtol=1e-5, atol=1e-7)
+        torch.testing.assert_close(met1, met2, rtol=1e-5, atol=1e-6, equal_nan=True)
+        torch.testing.assert_close(lp1[m], lp_g.detach()[m], rtol=0, atol=1e-5)
+        torch.testing.assert_close(ent1[m], ent_g.detach()[m], rtol=0, atol=1e-5)
+        assert _rel_l2(leaf1.grad, leaf.grad) < (2e-5 if dtype == torch.float32 else 2e-3), V
+        assert float(leaf1.grad[2, 1:].float().abs().max()) == 0.0  # masked rows and the row past the window: exact zeros
+        # an upstream gradient other than 1: the buffer (not a whole number of vectors) is scaled in place
+        leaf3 = logits.detach().clone().requires_grad_(True)
+        loss3, _, _, _ = amd.grpo_loss_from_logits(leaf3, ids, adv, mask, temperature=0.9, **kw)
+        (loss3 * 0.5).backward()
+        assert _rel_l2(leaf3.grad.float(), 0.5 * leaf1.grad.float()) < (1e-6 if dtype == torch.float32 else 3e-3), V
+    # rows of the logits aligned (a slice of a wider tensor), rows of the gradient not
+    wide, ids, mask, adv, g = _inputs(2, 3, 1024, dtype=dtype, seed=5, extra_rows=1)
+    mask[:] = 1
+    view = wide[..., :1019]
+    ids = ids.clamp(max=1018)
+    assert amd.grpo_single_pass_supported(view)
+    leaf = view.detach().clone().requires_grad_(True)
+    lp_g, ent_g = amd.per_token_logps_and_entropies(leaf, ids, 3, 1.0, True, False)
+    loss2, _ = amd.grpo_loss(lp_g, adv, mask, entropies=ent_g, loss_type="bnpo")
+    loss2.backward()
+    src = wide.detach().clone().requires_grad_(True)
+    loss1, _, _, _ = amd.grpo_loss_from_logits(src[..., :1019], ids, adv, mask, loss_type="bnpo")
+    loss1.backward()
+    torch.testing.assert_close(loss1, loss2, rtol=1e-5, atol=1e-7)
+    assert _rel_l2(src.grad[..., :1019], leaf.grad) < (2e-5 if dtype == torch.float32 else 2e-3)
+    assert float(src.grad[..., 1019:].float().abs().max()) == 0.0
+    amd.check_device_errors()
+
+
 def test_unsupported_configurations_raise(amd):
     logits, ids, mask, adv, _ = _inputs(2, 4, 1024)
     assert amd.grpo_single_pass_supported(logits)
     assert amd.grpo_single_pass_supported(logits.float()) and not amd.grpo_single_pass_supported(logits.double())
-    assert not amd.grpo_single_pass_supported(logits.float()[..., :1022])
+    assert amd.grpo_single_pass_supported(logits.float()[..., :1022]) and amd.grpo_single_pass_supported(logits[..., :1019])
+    assert not amd.grpo_single_pass_supported(logits[..., :15]) and not amd.grpo_single_pass_supported(logits[..., ::2])
     assert not amd.grpo_single_pass_supported(logits, "vespo")
     assert not amd.grpo_single_pass_supported(logits, "dapo", "sequence")
     assert amd.grpo_single_pass_supported(logits, entropy_coef=0.01)
     assert not amd.grpo_single_pass_supported(logits, entropy_mask=mask)
-    assert not amd.grpo_single_pass_supported(logits[..., :1020])
     big = torch.empty((1, 2, amd.ops.grpo_fused_max_vocab(torch.bfloat16) + 8), dtype=torch.bfloat16, device=DEV)
     assert not amd.grpo_single_pass_supported(big)
     with pytest.raises(NotImplementedError):

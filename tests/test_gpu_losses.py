@@ -38,9 +38,10 @@ def test_golden_grpo_compute_loss_through_trainer_methods(amd, skip_masked, sing
     """The reference's `GRPOTrainer._compute_loss` ran these inputs on a mocked trainer; the same
     mock drives our mix-in methods on the device.  With `skip_masked` the forward kernel skips the
     rows the completion mask zeroes; loss, metrics and gradients must not change.  With `single_pass` the
-    trainer asks for the one-pass kernel, which none of these cases can take (V = 41 is no multiple of 8, most
-    logits are fp32): this leg checks the fall-back to the two kernels on the logits of the same model call.
-    The reference-written vectors that DO go through the one-pass kernel are `grpo_single_pass.*`
+    trainer asks for the one-pass kernel: the cases whose configuration it takes go through it (fp32 logits of 41
+    entries: rows that are not whole vectors, peeled to their alignment), the others (sequence-level weights,
+    masks derived from the log-probs, vespo, luspo) fall back to the two kernels on the logits of the same model
+    call.  More reference-written vectors for the one-pass kernel: `grpo_single_pass.*`
     (tests/test_gpu_grpo_single_pass.py)."""
     cases, g = load_golden("grpo_compute_loss")
     ran = 0

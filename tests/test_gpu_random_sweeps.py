@@ -229,13 +229,13 @@ def test_advantages_against_the_oracle(amd):
 
 def test_single_pass_kernel_against_the_two_pass_path(amd):
     """250 configurations the single-pass kernel takes (loss types, KL, delta, bias-corrected KL, token weights,
-    per-token advantages, entropy bonus, temperatures, bf16 / fp16 / fp32, vocabularies 8 ... 20488 and one whose rows overflow
+    per-token advantages, entropy bonus, temperatures, bf16 / fp16 / fp32, vocabularies 8 ... 20488 (two that are no multiple of the vector) and one whose rows overflow
     into LDS, empty sequences, ragged
     masks): loss, metrics, log-probs and dlogits against K1 + loss kernel + K3."""
     rnd = random.Random(2)
     torch.manual_seed(2)
     for case in range(250):
-        B, K, V = rnd.choice([1, 2, 5]), rnd.choice([1, 7, 33]), rnd.choice([8, 64, 264, 1000, 4096, 20488, 172040])
+        B, K, V = rnd.choice([1, 2, 5]), rnd.choice([1, 7, 33]), rnd.choice([8, 64, 264, 1000, 1003, 4096, 4099, 20488, 172040])
         L = K + rnd.choice([1, 1, 3])
         dt = rnd.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
         if dt == torch.float32 and V > 167936:  # (fp32 rows hold half as many logits)

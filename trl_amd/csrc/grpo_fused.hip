@@ -32,6 +32,8 @@ constexpr int kWideVec = kMaxVec;  // register vectors of the builds with vector
 
 typedef __attribute__((address_space(1))) const u32x4 GlobalVecIn;
 typedef __attribute__((address_space(1))) u32x4 GlobalVecOut;
+typedef u32x4 u32x4_u __attribute__((aligned(2)));  // a 16-byte vector at any element alignment
+typedef __attribute__((address_space(1))) u32x4_u GlobalVecOutU;
 
 struct FusedArgs {
     const void* logits;
@@ -79,7 +81,12 @@ __device__ __forceinline__ void lds_transfer(const u32x4* src, uint32_t lds) {
 //   * EXTRA (rows too long for registers and LDS together): the vectors beyond are summed before the row proper is
 //     requested (four loads in flight; their registers are free again when the row's loads go out) and read again at
 //     the end for their gradient.
-template <int DT, int NVEC, int NLDS, bool EXTRA = false>
+//   * RAGGED (rows that are not whole aligned vectors: a vocabulary that is no multiple of the vector width): the
+//     row is taken in aligned vectors from its first 16-byte boundary on; the up to EPV - 1 elements before that and
+//     after the last whole vector belong to one lane each, which reads its element ahead of the row for the sums
+//     and again after the row's stores for its gradient.  The gradient row may sit at another alignment than the
+//     logits row: its vectors are stored through accesses that need none.
+template <int DT, int NVEC, int NLDS, bool EXTRA = false, bool RAGGED = false>
 __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     typedef Elem<DT> E;
     typedef typename E::type T;
@@ -96,7 +103,7 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     const int64_t t = to - a.out_row_offset;
     const bool inside = t >= 0 && t < a.rows_per_seq;
     const int64_t row = b * a.rows_per_seq + (inside ? t : 0);
-    const int nv = int(a.vocab / EPV);
+    int nv = int(a.vocab / EPV);  // whole vectors of the row (RAGGED: counted from its first 16-byte boundary, set below)
     float m = 0.f, A = 0.f, old_lp = 0.f, ref_lp = 0.f, w = 1.f, coef = 0.f, scale = 0.f, h = 0.f;
     int64_t idx = -1;
     if (inside) {
@@ -110,10 +117,26 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
         scale = a.row_scale[b];
         if (a.ent_weight) h = a.ent_weight[row];
     }
-    u32x4* op = reinterpret_cast<u32x4*>(static_cast<T*>(a.dlogits) + b * a.out_seq_stride + to * a.out_row_stride);
+    T* out = static_cast<T*>(a.dlogits) + b * a.out_seq_stride + to * a.out_row_stride;
+    typedef typename std::conditional<RAGGED, u32x4_u, u32x4>::type OutVec;
+    // RAGGED: `head` elements before the logits row's first 16-byte boundary, `nv` whole vectors from there, then the
+    // last elements; lane tid < head + tail owns edge element number `edge` of the row
+    int head = 0, edge = -1;
+    if constexpr (RAGGED) {
+        const T* row0 = static_cast<const T*>(a.logits) + b * a.seq_stride + (inside ? t : 0) * a.row_stride;
+        head = int(min(a.vocab, int64_t(((16 - (reinterpret_cast<uintptr_t>(row0) & 15)) & 15) / sizeof(T))));
+        nv = int((a.vocab - head) / EPV);
+        const int tail0 = head + nv * EPV;
+        if (tid < head)
+            edge = tid;
+        else if (tid - head < int(a.vocab) - tail0)
+            edge = tail0 + (tid - head);
+    }
+    OutVec* op = reinterpret_cast<OutVec*>(out + head);
     if (m == 0.f) {  // no gradient reaches this row: zero-fill
         const u32x4 z = {0u, 0u, 0u, 0u};
         for (int v = tid; v < nv; v += kFThreads) __builtin_nontemporal_store(z, op + v);
+        if (RAGGED && edge >= 0) E::store1(out + edge, 0.f);
     }
     if (m == 0.f && !(inside && a.all_rows)) {  // and nothing is read
         if (inside && tid == 0) {
@@ -124,11 +147,20 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
         return;
     }
     const T* base = static_cast<const T*>(a.logits) + b * a.seq_stride + t * a.row_stride;
-    const u32x4* vp = reinterpret_cast<const u32x4*>(base);
+    const u32x4* vp = reinterpret_cast<const u32x4*>(base + head);
     const float inv_t = 1.f / a.temperature, c = kLog2e * inv_t;
     // sums of 2^(x c - r0) and of the same times x
     float r0 = 0.f, s = 0.f, u = 0.f;
     [[maybe_unused]] bool have_r0 = false;
+    if constexpr (RAGGED) {
+        if (edge >= 0) {
+            const float x = E::load1(base + edge);
+            r0 = ceilf(x * c);
+            have_r0 = true;
+            s = fast_exp2(fmaf(x, c, -r0));
+            u = s * x;
+        }
+    }
     constexpr int kOnChip = (NVEC + NLDS) * kFThreads;  // vectors of the row the workgroup holds
     if constexpr (EXTRA) {
         for (int v0 = kOnChip; v0 < nv; v0 += 4 * kFThreads) {
@@ -192,7 +224,7 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
         if (j < kTail || j * kFThreads + tid < nv) {
             float x[EPV];
             E::unpack(q[j], x);
-            if (j == 0 && !(EXTRA && have_r0)) {
+            if (j == 0 && !((EXTRA || RAGGED) && have_r0)) {
                 float mx = x[0];
 #pragma unroll
                 for (int i = 1; i < EPV; ++i) mx = fmaxf(mx, x[i]);
@@ -227,7 +259,7 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     // bring the lanes' sums to a common exponent K >= r0 + log2(s) of every lane
     int es = 0;
     (void)frexpf(s, &es);
-    const bool has_data = tid < nv;
+    const bool has_data = tid < nv || (RAGGED && edge >= 0);
     const float key = has_data ? r0 + float(es) : -INFINITY;
     const bool bad = !(s < INFINITY) || !(fabsf(u) < INFINITY);  // overflow of a term, or inf / NaN in the row
     const float wk = wave_max(key);
@@ -270,6 +302,7 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
 #pragma unroll
             for (int i = 0; i < EPV; ++i) lm = fmaxf(lm, x[i]);
         }
+        if (RAGGED && edge >= 0) lm = fmaxf(lm, E::load1(base + edge));
         float M = wave_max(lm);
         if (lane == 0) red[4][wave] = M;
         __syncthreads();
@@ -287,6 +320,12 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
                 s += e;
                 u = fmaf(e, x[i], u);
             }
+        }
+        if (RAGGED && edge >= 0) {
+            const float x = E::load1(base + edge);
+            const float e = fast_exp2(fmaf(x, c, -mc));
+            s += e;
+            u = fmaf(e, x, u);
         }
         s = wave_sum(s);
         u = wave_sum(u);
@@ -343,7 +382,8 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
                 const float tt = fmaf(x[i], c, -lse2);
                 d[i] = fast_exp2(tt) * (with_h ? fmaf(b0, tt, a0) : a0);
             }
-            GlobalVecOut* oj = (GlobalVecOut*)op + j * kFThreads;
+            typedef typename std::conditional<RAGGED, GlobalVecOutU, GlobalVecOut>::type GOut;
+            GOut* oj = (GOut*)op + j * kFThreads;
             asm volatile("" : "+s"(oj));
             __builtin_nontemporal_store(E::pack(d), oj + tid);  // (streaming stores: 2-3 % faster than plain ones here)
         }
@@ -385,10 +425,20 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
             }
         }
     }
-    // one-hot term: the lane that stored the target's vector rewrites that element (same lane, same
-    // address: ordered after its first store)
-    if (idx_ok && int((idx / EPV) % kFThreads) == tid) {
-        T* out = reinterpret_cast<T*>(op);
+    if constexpr (RAGGED) {
+        if (edge >= 0) {
+            const float tt = fmaf(E::load1(base + edge), c, -lse2);
+            E::store1(out + edge, fast_exp2(tt) * (with_h ? fmaf(b0, tt, a0) : a0));
+        }
+    }
+    // one-hot term: the lane that stored the target's vector (or edge element) rewrites that element (same lane,
+    // same address: ordered after its first store)
+    int owner = int((idx / EPV) % kFThreads);
+    if constexpr (RAGGED) {
+        const int64_t tail0 = head + int64_t(nv) * EPV;
+        owner = idx < head ? int(idx) : idx >= tail0 ? head + int(idx - tail0) : int(((idx - head) / EPV) % kFThreads);
+    }
+    if (idx_ok && owner == tid) {
         const float tt = fmaf(x_t, c, -lse2);
         E::store1(out + idx, fast_exp2(tt) * (with_h ? fmaf(b0, tt, a0) : a0) + g * inv_t);
     }
@@ -418,37 +468,38 @@ int reserve_overflow_lds(Kern kern, int bytes) {
     return TRLK_OK;
 }
 
-template <int DT, int NLDS>
+template <int DT, int NLDS, bool EXTRA, bool R>
 int launch_fused_wide(const FusedArgs& a, unsigned rows, hipStream_t s) {
     constexpr int kBytes = NLDS * kFThreads * 16;
-    if (int rc = reserve_overflow_lds(grpo_fused_kernel<DT, kWideVec, NLDS>, kBytes)) return rc;
-    hipLaunchKernelGGL((grpo_fused_kernel<DT, kWideVec, NLDS>), dim3(rows), dim3(kFThreads), kBytes, s, a);
+    if (int rc = reserve_overflow_lds(grpo_fused_kernel<DT, kWideVec, NLDS, EXTRA, R>, kBytes)) return rc;
+    hipLaunchKernelGGL((grpo_fused_kernel<DT, kWideVec, NLDS, EXTRA, R>), dim3(rows), dim3(kFThreads), kBytes, s, a);
+    return TRLK_OK;
+}
+
+// R: rows that are not whole aligned vectors
+template <int DT, bool R>
+int launch_fused(const FusedArgs& a, int nvec, unsigned rows, hipStream_t s) {
+    if (nvec > kWideVec + kMaxLdsVec) return launch_fused_wide<DT, kMaxLdsVec, true, R>(a, rows, s);
+    if (nvec > kMaxVec) {
+        switch ((nvec - kWideVec + kLdsStep - 1) / kLdsStep) {
+            case 1: return launch_fused_wide<DT, 3, false, R>(a, rows, s);
+            case 2: return launch_fused_wide<DT, 6, false, R>(a, rows, s);
+            default: return launch_fused_wide<DT, 9, false, R>(a, rows, s);
+        }
+    }
+    switch ((nvec + kVecStep - 1) / kVecStep) {
+        case 1: hipLaunchKernelGGL((grpo_fused_kernel<DT, 4, 0, false, R>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        case 2: hipLaunchKernelGGL((grpo_fused_kernel<DT, 8, 0, false, R>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        case 3: hipLaunchKernelGGL((grpo_fused_kernel<DT, 12, 0, false, R>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        case 4: hipLaunchKernelGGL((grpo_fused_kernel<DT, 16, 0, false, R>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        default: hipLaunchKernelGGL((grpo_fused_kernel<DT, 20, 0, false, R>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+    }
     return TRLK_OK;
 }
 
 template <int DT>
-int launch_fused(const FusedArgs& a, int nvec, unsigned rows, hipStream_t s) {
-    if (nvec > kWideVec + kMaxLdsVec) {
-        constexpr int kBytes = kMaxLdsVec * kFThreads * 16;
-        if (int rc = reserve_overflow_lds(grpo_fused_kernel<DT, kWideVec, kMaxLdsVec, true>, kBytes)) return rc;
-        hipLaunchKernelGGL((grpo_fused_kernel<DT, kWideVec, kMaxLdsVec, true>), dim3(rows), dim3(kFThreads), kBytes, s, a);
-        return TRLK_OK;
-    }
-    if (nvec > kMaxVec) {
-        switch ((nvec - kWideVec + kLdsStep - 1) / kLdsStep) {
-            case 1: return launch_fused_wide<DT, 3>(a, rows, s);
-            case 2: return launch_fused_wide<DT, 6>(a, rows, s);
-            default: return launch_fused_wide<DT, 9>(a, rows, s);
-        }
-    }
-    switch ((nvec + kVecStep - 1) / kVecStep) {
-        case 1: hipLaunchKernelGGL((grpo_fused_kernel<DT, 4, 0>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-        case 2: hipLaunchKernelGGL((grpo_fused_kernel<DT, 8, 0>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-        case 3: hipLaunchKernelGGL((grpo_fused_kernel<DT, 12, 0>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-        case 4: hipLaunchKernelGGL((grpo_fused_kernel<DT, 16, 0>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-        default: hipLaunchKernelGGL((grpo_fused_kernel<DT, 20, 0>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-    }
-    return TRLK_OK;
+int launch_fused_any(const FusedArgs& a, int nvec, bool ragged, unsigned rows, hipStream_t s) {
+    return ragged ? launch_fused<DT, true>(a, nvec, rows, s) : launch_fused<DT, false>(a, nvec, rows, s);
 }
 
 // data *= *scale over 16-byte vectors, unless the scale is exactly 1 (then nothing is read or written, and what the
@@ -457,10 +508,14 @@ int launch_fused(const FusedArgs& a, int nvec, unsigned rows, hipStream_t s) {
 // 16 KiB at a time, four vectors per lane in flight.
 constexpr int kScaleSpanVec = 16384;  // vectors per workgroup
 template <int DT>
-__global__ __launch_bounds__(256) void scale_unless_one_kernel(u32x4* data, int64_t n_vec, const float* scale) {
+__global__ __launch_bounds__(256) void scale_unless_one_kernel(u32x4* data, int64_t n_vec, int n_tail, const float* scale) {
     typedef Elem<DT> E;
     const float sc = *scale;
     if (sc == 1.f) return;
+    if (blockIdx.x == 0 && int(threadIdx.x) < n_tail) {  // the elements after the last whole vector
+        typename E::type* p = reinterpret_cast<typename E::type*>(data + n_vec) + threadIdx.x;
+        E::store1(p, E::load1(p) * sc);
+    }
     const int64_t base = int64_t(blockIdx.x) * kScaleSpanVec + threadIdx.x;
 #pragma unroll 1
     for (int it = 0; it < kScaleSpanVec / 1024; ++it) {
@@ -491,21 +546,21 @@ extern "C" int trlk_scale_unless_one(void* d_data, int dtype, int64_t n_elems, c
     TRLK_REQUIRE(dtype == TRLK_BF16 || dtype == TRLK_F16 || dtype == TRLK_F32, TRLK_ERR_BAD_DTYPE,
                  "scale_unless_one: bf16, fp16 or fp32 data (dtype code %d)", dtype);
     const int64_t epv = dtype == TRLK_F32 ? 4 : 8;
-    TRLK_REQUIRE(n_elems >= 0 && n_elems % epv == 0, TRLK_ERR_BAD_SHAPE,
-                 "scale_unless_one: element count must be a multiple of %lld", (long long)epv);
+    TRLK_REQUIRE(n_elems >= 0, TRLK_ERR_BAD_SHAPE, "scale_unless_one: negative element count");
     if (n_elems == 0) return TRLK_OK;
     TRLK_REQUIRE(d_data && d_scale && reinterpret_cast<uintptr_t>(d_data) % 16 == 0, TRLK_ERR_NULL_POINTER,
                  "scale_unless_one: null or misaligned pointer");
     const int64_t n_vec = n_elems / epv;
+    const int n_tail = int(n_elems - n_vec * epv);
     TRLK_REQUIRE(n_vec <= int64_t(kScaleSpanVec) * 0x7fffffff, TRLK_ERR_BAD_SHAPE, "scale_unless_one: too many elements");
-    const unsigned grid = unsigned((n_vec + kScaleSpanVec - 1) / kScaleSpanVec);
+    const unsigned grid = unsigned((n_vec + kScaleSpanVec - 1) / kScaleSpanVec) + (n_vec == 0 ? 1u : 0u);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == TRLK_BF16)
-        hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_BF16>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, d_scale);
+        hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_BF16>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, n_tail, d_scale);
     else if (dtype == TRLK_F16)
-        hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_F16>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, d_scale);
+        hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_F16>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, n_tail, d_scale);
     else
-        hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_F32>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, d_scale);
+        hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_F32>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, n_tail, d_scale);
     return launch_status("scale_unless_one");
 }
 
@@ -530,8 +585,8 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
                  "grpo_fused: bf16, fp16 or fp32 logits (dtype code %d); use the two-pass path", dtype);
     const int64_t es = int64_t(elem_size(dtype)), epv = 16 / es;
     TRLK_REQUIRE(n_seq >= 0 && rows_per_seq >= 0 && vocab >= 1, TRLK_ERR_BAD_SHAPE, "grpo_fused: bad sizes");
-    TRLK_REQUIRE(vocab % epv == 0 && vocab <= trlk_grpo_fused_max_vocab(dtype), TRLK_ERR_UNSUPPORTED,
-                 "grpo_fused: vocab must be a multiple of %lld and at most %lld (got %lld); use the two-pass path",
+    TRLK_REQUIRE(vocab >= epv && vocab <= trlk_grpo_fused_max_vocab(dtype), TRLK_ERR_UNSUPPORTED,
+                 "grpo_fused: vocab must be at least %lld and at most %lld (got %lld); use the two-pass path",
                  (long long)epv, (long long)trlk_grpo_fused_max_vocab(dtype), (long long)vocab);
     TRLK_REQUIRE(out_row_offset >= 0 && out_row_offset + rows_per_seq <= out_rows_per_seq, TRLK_ERR_BAD_SHAPE,
                  "grpo_fused: input rows [%lld, %lld) do not fit the %lld output rows per sequence",
@@ -555,8 +610,15 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
     const auto al16 = [es](const void* p, int64_t s0, int64_t s1) {
         return reinterpret_cast<uintptr_t>(p) % 16 == 0 && (s0 * es) % 16 == 0 && (s1 * es) % 16 == 0;
     };
-    TRLK_REQUIRE(al16(d_logits, seq_stride, row_stride) && al16(d_dlogits, out_seq_stride, out_row_stride),
-                 TRLK_ERR_BAD_STRIDE, "grpo_fused: logits and dlogits rows must be 16-byte aligned; use the two-pass path");
+    TRLK_REQUIRE(reinterpret_cast<uintptr_t>(d_logits) % es == 0 && reinterpret_cast<uintptr_t>(d_dlogits) % es == 0,
+                 TRLK_ERR_BAD_STRIDE, "grpo_fused: logits and dlogits must be aligned to their element size");
+    // rows that are not whole aligned vectors take the builds that peel a row to its first 16-byte boundary
+    const bool ragged = vocab % epv != 0 || !al16(d_logits, seq_stride, row_stride) ||
+                        !al16(d_dlogits, out_seq_stride, out_row_stride);
+    // (a peeled row must still hold one whole vector)
+    TRLK_REQUIRE(!ragged || vocab >= 2 * epv, TRLK_ERR_UNSUPPORTED,
+                 "grpo_fused: rows that are not whole aligned vectors need at least %lld entries (got %lld); use the two-pass path",
+                 (long long)(2 * epv), (long long)vocab);
     FusedArgs a{};
     a.logits = d_logits;
     a.rows_per_seq = rows_per_seq;
@@ -595,9 +657,9 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
     a.all_rows = compute_masked_rows != 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int nvec = int((vocab / epv + kFThreads - 1) / kFThreads);  // 16-byte vectors of the row per lane
-    if (int rc = dtype == TRLK_BF16  ? launch_fused<TRLK_BF16>(a, nvec, unsigned(orows), s)
-                 : dtype == TRLK_F16 ? launch_fused<TRLK_F16>(a, nvec, unsigned(orows), s)
-                                     : launch_fused<TRLK_F32>(a, nvec, unsigned(orows), s))
+    if (int rc = dtype == TRLK_BF16  ? launch_fused_any<TRLK_BF16>(a, nvec, ragged, unsigned(orows), s)
+                 : dtype == TRLK_F16 ? launch_fused_any<TRLK_F16>(a, nvec, ragged, unsigned(orows), s)
+                                     : launch_fused_any<TRLK_F32>(a, nvec, ragged, unsigned(orows), s))
         return rc;
     return launch_status("grpo_fused");
 }

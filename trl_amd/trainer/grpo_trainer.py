@@ -239,7 +239,7 @@ def grpo_single_pass_supported(logits: Tensor, loss_type: str = "dapo", importan
     """Whether `grpo_loss_from_logits` can go from these logits to their gradient in one pass: a token-level
     loss type, with or without entropy bonus but without an entropy-quantile mask (the gradient coefficients of
     a token then depend on nothing but that token), bf16 / fp16 / fp32 logits whose rows the kernel takes
-    (`ops.grpo_fused_max_vocab`) and are 16-byte aligned."""
+    (`ops.grpo_fused_max_vocab`)."""
     if loss_type not in _SINGLE_PASS_LOSS_TYPES or importance_sampling_level != "token":
         return False
     if entropy_mask is not None:  # (a mask derived from every token's entropy needs the forward pass first)
@@ -248,9 +248,13 @@ def grpo_single_pass_supported(logits: Tensor, loss_type: str = "dapo", importan
         return False
     vocab = logits.shape[-1]
     per_vector = 16 // logits.element_size()
-    if vocab % per_vector != 0 or vocab > ops.grpo_fused_max_vocab(logits.dtype) or (vocab > 1 and logits.stride(-1) != 1):
+    if vocab > ops.grpo_fused_max_vocab(logits.dtype) or (vocab > 1 and logits.stride(-1) != 1):
         return False
-    return logits.data_ptr() % 16 == 0 and logits.stride(0) % per_vector == 0 and logits.stride(1) % per_vector == 0
+    whole = (vocab % per_vector == 0 and logits.data_ptr() % 16 == 0 and logits.stride(0) % per_vector == 0
+             and logits.stride(1) % per_vector == 0)
+    # (rows that are not whole aligned 16-byte vectors are peeled to their alignment by the kernel, and must still
+    # hold a whole vector then)
+    return vocab >= (per_vector if whole else 2 * per_vector)
 
 
 class _GRPOFromLogits(torch.autograd.Function):
@@ -398,7 +402,7 @@ def grpo_loss_from_logits(
     if not grpo_single_pass_supported(logits, loss_type):
         raise NotImplementedError(
             "grpo_loss_from_logits: this configuration needs the two-pass path (per_token_logps_and_entropies + "
-            "grpo_loss): token-level loss types, bf16 / fp16 / fp32 logits in rows of whole 16-byte vectors, at most "
+            "grpo_loss): token-level loss types, bf16 / fp16 / fp32 logits with a contiguous vocabulary axis of at most "
             f"{ops.grpo_fused_max_vocab(logits.dtype) if logits.dtype in (torch.bfloat16, torch.float16, torch.float32) else 0} "
             "entries long")
     if beta != 0.0 and ref_per_token_logps is None:
