@@ -370,11 +370,14 @@ def test_rows_that_are_not_whole_vectors(amd, dtype):
         torch.testing.assert_close(ent1[m], ent_g.detach()[m], rtol=0, atol=1e-5)
         assert _rel_l2(leaf1.grad, leaf.grad) < (2e-5 if dtype == torch.float32 else 2e-3), V
         assert float(leaf1.grad[2, 1:].float().abs().max()) == 0.0  # masked rows and the row past the window: exact zeros
-        # an upstream gradient other than 1: the buffer (not a whole number of vectors) is scaled in place
+        # an upstream gradient other than 1: the buffer (not a whole number of vectors) is scaled in place; and the
+        # rows outside the mask read for their log-probs and entropies as well
         leaf3 = logits.detach().clone().requires_grad_(True)
-        loss3, _, _, _ = amd.grpo_loss_from_logits(leaf3, ids, adv, mask, temperature=0.9, **kw)
+        loss3, _, lp3, ent3 = amd.grpo_loss_from_logits(leaf3, ids, adv, mask, temperature=0.9, skip_masked_rows=False, **kw)
         (loss3 * 0.5).backward()
         assert _rel_l2(leaf3.grad.float(), 0.5 * leaf1.grad.float()) < (1e-6 if dtype == torch.float32 else 3e-3), V
+        torch.testing.assert_close(lp3, lp_g.detach(), rtol=0, atol=1e-5)
+        torch.testing.assert_close(ent3, ent_g.detach(), rtol=0, atol=1e-5)
     # rows of the logits aligned (a slice of a wider tensor), rows of the gradient not
     wide, ids, mask, adv, g = _inputs(2, 3, 1024, dtype=dtype, seed=5, extra_rows=1)
     mask[:] = 1
