@@ -51,6 +51,7 @@ struct FusedArgs {
     void* dlogits;
     int64_t out_rows_per_seq, out_row_offset, out_seq_stride, out_row_stride;
     int32_t* error_flag;
+    int64_t total_rows;  // output rows: the grid is rounded up to a multiple of 8
     int all_rows;  // also read the rows with mask == 0 for their log-prob and entropy (their gradient is zero either way)
 };
 
@@ -97,7 +98,13 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     extern __shared__ __attribute__((aligned(16))) char overflow[];  // [NLDS][1024 lanes] 16-byte vectors
     __shared__ float red[7][kFWaves];
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    const int64_t orow = blockIdx.x;
+    // The hardware deals consecutive workgroups to the eight XCDs in turn.  Each XCD takes one contiguous eighth of
+    // the rows and walks it in order, instead of every eighth row of the whole tensor: eight separate streams of reads
+    // and writes, one per XCD.  Measured on bf16 [64, 1024, 151936] with the benchmark's mask: 5.65 -> 5.24 ms
+    // (every row read: 7.25 -> 6.86 ms; every row active: 7.55 -> 7.28 ms).
+    const int64_t per_xcd = int64_t(gridDim.x) >> 3;  // (the grid is a multiple of 8)
+    const int64_t orow = int64_t(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (orow >= a.total_rows) return;
     const int64_t b = orow / a.out_rows_per_seq;
     const int64_t to = orow - b * a.out_rows_per_seq;
     const int64_t t = to - a.out_row_offset;
@@ -472,7 +479,7 @@ template <int DT, int NLDS, bool EXTRA, bool R>
 int launch_fused_wide(const FusedArgs& a, unsigned rows, hipStream_t s) {
     constexpr int kBytes = NLDS * kFThreads * 16;
     if (int rc = reserve_overflow_lds(grpo_fused_kernel<DT, kWideVec, NLDS, EXTRA, R>, kBytes)) return rc;
-    hipLaunchKernelGGL((grpo_fused_kernel<DT, kWideVec, NLDS, EXTRA, R>), dim3(rows), dim3(kFThreads), kBytes, s, a);
+    hipLaunchKernelGGL((grpo_fused_kernel<DT, kWideVec, NLDS, EXTRA, R>), dim3((rows + 7) / 8 * 8), dim3(kFThreads), kBytes, s, a);
     return TRLK_OK;
 }
 
@@ -488,11 +495,11 @@ int launch_fused(const FusedArgs& a, int nvec, unsigned rows, hipStream_t s) {
         }
     }
     switch ((nvec + kVecStep - 1) / kVecStep) {
-        case 1: hipLaunchKernelGGL((grpo_fused_kernel<DT, 4, 0, false, R>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-        case 2: hipLaunchKernelGGL((grpo_fused_kernel<DT, 8, 0, false, R>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-        case 3: hipLaunchKernelGGL((grpo_fused_kernel<DT, 12, 0, false, R>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-        case 4: hipLaunchKernelGGL((grpo_fused_kernel<DT, 16, 0, false, R>), dim3(rows), dim3(kFThreads), 0, s, a); break;
-        default: hipLaunchKernelGGL((grpo_fused_kernel<DT, 20, 0, false, R>), dim3(rows), dim3(kFThreads), 0, s, a); break;
+        case 1: hipLaunchKernelGGL((grpo_fused_kernel<DT, 4, 0, false, R>), dim3((rows + 7) / 8 * 8), dim3(kFThreads), 0, s, a); break;
+        case 2: hipLaunchKernelGGL((grpo_fused_kernel<DT, 8, 0, false, R>), dim3((rows + 7) / 8 * 8), dim3(kFThreads), 0, s, a); break;
+        case 3: hipLaunchKernelGGL((grpo_fused_kernel<DT, 12, 0, false, R>), dim3((rows + 7) / 8 * 8), dim3(kFThreads), 0, s, a); break;
+        case 4: hipLaunchKernelGGL((grpo_fused_kernel<DT, 16, 0, false, R>), dim3((rows + 7) / 8 * 8), dim3(kFThreads), 0, s, a); break;
+        default: hipLaunchKernelGGL((grpo_fused_kernel<DT, 20, 0, false, R>), dim3((rows + 7) / 8 * 8), dim3(kFThreads), 0, s, a); break;
     }
     return TRLK_OK;
 }
@@ -597,7 +604,7 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
                  "grpo_fused: unknown policy term %d", policy_term);
     const int64_t orows = n_seq * out_rows_per_seq;
     if (orows == 0) return TRLK_OK;
-    TRLK_REQUIRE(orows < (int64_t(1) << 31), TRLK_ERR_BAD_SHAPE, "grpo_fused: too many rows (%lld)", (long long)orows);
+    TRLK_REQUIRE(orows < (int64_t(1) << 31) - 8, TRLK_ERR_BAD_SHAPE, "grpo_fused: too many rows (%lld)", (long long)orows);
     TRLK_REQUIRE(d_dlogits != nullptr, TRLK_ERR_NULL_POINTER, "grpo_fused: dlogits pointer is null");
     if (n_seq * rows_per_seq > 0) {
         TRLK_REQUIRE(d_logits && d_index && d_advantages && d_mask && d_row_scale && d_out_logp && d_out_entropy && d_out_lse,
@@ -655,6 +662,7 @@ extern "C" int trlk_grpo_fused_fwd_bwd(const void* d_logits, int dtype, int64_t 
     a.out_row_stride = out_row_stride;
     a.error_flag = d_error_flag;
     a.all_rows = compute_masked_rows != 0;
+    a.total_rows = orows;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int nvec = int((vocab / epv + kFThreads - 1) / kFThreads);  // 16-byte vectors of the row per lane
     if (int rc = dtype == TRLK_BF16  ? launch_fused_any<TRLK_BF16>(a, nvec, ragged, unsigned(orows), s)

@@ -379,6 +379,7 @@ struct BwdArgs {
     const float* g_entropy;
     void* dlogits;
     int64_t out_rows_per_seq, out_row_offset, out_seq_stride, out_row_stride;
+    int64_t total_chunks;  // rows x chunks per row
 };
 
 // The backward has no reduction, so a row is cut into chunks of kChunkElems elements and one
@@ -400,8 +401,15 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_bwd_kernel(BwdArgs a, i
     constexpr int CE = chunk_elems<DT>();
 
     const int tid = threadIdx.x;
-    const int64_t orow = blockIdx.x / chunks_per_row;
-    const int chunk = int(blockIdx.x - orow * chunks_per_row);
+    // The hardware deals consecutive workgroups to the eight XCDs in turn.  Each XCD walks one contiguous eighth of the
+    // chunks (address-linear inside it) instead of every eighth chunk of the whole buffer: eight narrow write windows,
+    // one per XCD.  Measured on bf16 [64, 1024, 151936]: zero-filled rows 3.39 -> 2.97 ms, the benchmark's prefix mask
+    // 5.20 -> 4.95 ms, every row active 6.3 -> 6.5 ms; 16, 32 or 64 such regions are slower than either.
+    const int64_t per_xcd = int64_t(gridDim.x) >> 3;  // (the grid is a multiple of 8)
+    const int64_t linear = int64_t(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (linear >= a.total_chunks) return;
+    const int64_t orow = linear / chunks_per_row;
+    const int chunk = int(linear - orow * chunks_per_row);
     const int64_t b = orow / a.out_rows_per_seq;
     const int64_t to = orow - b * a.out_rows_per_seq;
     const int64_t t = to - a.out_row_offset;
@@ -632,10 +640,11 @@ extern "C" int trlk_logp_entropy_bwd(const void* d_logits, int dtype, int64_t n_
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t chunk = kChunkBytes / int64_t(es);
     const int64_t chunks_per_row = (vocab + chunk - 1) / chunk;
-    TRLK_REQUIRE(orows * chunks_per_row < (int64_t(1) << 31), TRLK_ERR_BAD_SHAPE,
+    TRLK_REQUIRE(orows * chunks_per_row < (int64_t(1) << 31) - 8, TRLK_ERR_BAD_SHAPE,
                  "logp_entropy_bwd: %lld rows x %lld chunks exceed the grid limit", (long long)orows,
                  (long long)chunks_per_row);
-    const dim3 grid((unsigned)(orows * chunks_per_row)), block(kThreads);
+    a.total_chunks = orows * chunks_per_row;
+    const dim3 grid((unsigned)(((a.total_chunks + 7) / 8) * 8)), block(kThreads);
     const int cpr = int(chunks_per_row);
 #define TRLK_LAUNCH_BWD(DT)                                                                              \
     if (vec && has_h)                                                                                    \
