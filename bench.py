@@ -39,11 +39,11 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # summaries under profiles/).  The inputs are seeded, so the figures are stable; they are records of those runs, not
 # measured by the run that prints them, and None where no counter run was made for that workload / loss type.
 MEASURED_TRAFFIC_BYTES = {
-    ("K3", "grpo_c3", "dapo"): (10116130 + 19461194) * 1024,
-    ("K7", "grpo_c3", "dapo"): (2 * 5064150 + 19488700) * 1024,
-    ("K3", "grpo_c4", "dapo"): (2 * 10693437 + 38927000) * 1024,
-    ("K7", "grpo_c4", "dapo"): (2 * 10701061 + 38975505) * 1024,
-    ("K3", "dpo_c2", None): (2 * 6612423 + 32860500) * 1024,
+    ("K3", "grpo_c3", "dapo"): (2 * 5054241 + 19454900) * 1024,
+    ("K7", "grpo_c3", "dapo"): (2 * 5055205 + 19474750) * 1024,
+    ("K3", "grpo_c4", "dapo"): (2 * 10685504 + 38911700) * 1024,
+    ("K7", "grpo_c4", "dapo"): (2 * 10686905 + 38959000) * 1024,
+    ("K3", "dpo_c2", None): (2 * 6605806 + 32849200) * 1024,
     ("head_fwd", "head_c5", "dapo"): (2 * 40600000 + 19497000) * 1024,
 }
 # the loss type changes per-row scalars only: the same rows are read and written, by the same launches

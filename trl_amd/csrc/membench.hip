@@ -70,11 +70,13 @@ __global__ __launch_bounds__(THREADS) void flat_kernel(const u32x4* __restrict__
     }
 }
 
-template <bool NT_LOAD, bool NT_STORE>
+// REGIONAL: consecutive workgroups go to the eight XCDs in turn; each XCD walks one contiguous eighth of the rows
+// instead of every eighth row (the grid is a multiple of 8).
+template <bool NT_LOAD, bool NT_STORE, bool REGIONAL = false>
 __global__ __launch_bounds__(1024) void row_kernel(const u32x4* in, u32x4* out, const uint8_t* active) {
     constexpr int PER = (kRowVec + 1023) / 1024;
     const int tid = threadIdx.x;
-    const int64_t row = blockIdx.x;
+    const int64_t row = REGIONAL ? int64_t(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3) : int64_t(blockIdx.x);
     const u32x4* ip = in + row * kRowVec;
     u32x4* op = out + row * kRowVec;
     if (!active[row]) {
@@ -194,6 +196,9 @@ int main() {
             [&] { hipLaunchKernelGGL((row_kernel<false, true>), dim3(unsigned(rows)), dim3(1024), 0, 0, in, out, act_d); });
         run(masked ? "row in registers, benchmark mask, nt/nt" : "row in registers, every row, nt/nt", moved,
             [&] { hipLaunchKernelGGL((row_kernel<true, true>), dim3(unsigned(rows)), dim3(1024), 0, 0, in, out, act_d); });
+        run(masked ? "row in registers, one region of rows per XCD, benchmark mask, plain/nt"
+                   : "row in registers, one region of rows per XCD, every row, plain/nt", moved,
+            [&] { hipLaunchKernelGGL((row_kernel<false, true, true>), dim3(unsigned(rows)), dim3(1024), 0, 0, in, out, act_d); });
         run(masked ? "2 pieces of 1024 lanes, benchmark mask, plain/nt" : "2 pieces of 1024 lanes, every row, plain/nt", moved,
             [&] { hipLaunchKernelGGL((piece_kernel<1024, 2>), dim3(unsigned(rows * 2)), dim3(1024), 0, 0, in, out, act_d); });
         run(masked ? "2 pieces of 512 lanes, benchmark mask, plain/nt" : "2 pieces of 512 lanes, every row, plain/nt", moved,
