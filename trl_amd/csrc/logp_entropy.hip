@@ -27,7 +27,7 @@ namespace {
 #define TRLK_FWD_NT_LOAD 1
 #endif
 #ifndef TRLK_BWD_NT_LOAD
-#define TRLK_BWD_NT_LOAD 0
+#define TRLK_BWD_NT_LOAD 1  // (with every XCD on its own region of the chunks: 2-3 % ahead of plain loads; no difference before)
 #endif
 #ifndef TRLK_NT_STORE
 #define TRLK_NT_STORE 1
