@@ -411,7 +411,9 @@ def bench_dpo(args, w):
             torch.cuda.synchronize()
             return a.elapsed_time(b) / reps
 
-        fwd_ms = time_kernel(lambda: ops.logp_entropy_stats_fwd(logits.detach(), idx, 1.0, 0, L - 1, None))
+        # (as the step above runs it: without the sum of squared probabilities, which only the WPO weights read)
+        fwd_ms = time_kernel(lambda: ops.logp_entropy_stats_fwd(logits.detach(), idx, 1.0, 0, L - 1, None, False))
+        fwd_p2_ms = time_kernel(lambda: ops.logp_entropy_stats_fwd(logits.detach(), idx, 1.0, 0, L - 1, None, True))
         bwd_ms = time_kernel(lambda: ops.logp_entropy_bwd(logits.detach(), idx, 1.0, 0, L - 1, lse, None, g_logp, None))
     row_bytes = V * 2
     fwd_bytes = R * row_bytes
@@ -429,7 +431,8 @@ def bench_dpo(args, w):
                      "avg_launch_ms": bwd_ms},
         "kernels": {"logp_entropy_fwd_kernel with row statistics (K1)": {
             "avg_launch_ms": fwd_ms, "algorithmic_bytes": fwd_bytes, "achieved_GBps": fwd_bytes / (fwd_ms * 1e-3) / 1e9,
-            "frac": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}},
+            "frac": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "with_sum_of_squared_probabilities_ms": fwd_p2_ms}},
         "mask_aware": {"ms_per_step": ms_aware, "tokens_per_s": R / (ms_aware * 1e-3),
                        "note": "only rows inside the completion mask are read; loss, metrics and dlogits identical"},
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_dpo(w),

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define TRLK_VERSION 1
+#define TRLK_VERSION 2
 
 typedef void* trlk_stream_t; /* hipStream_t */
 
@@ -82,7 +82,8 @@ const char* trlk_last_error(void);
  * three more passes over the logits (trl/trainer/dpo_trainer.py:1563-1574 WPO weights, :1605-1618
  * logits means, :1620-1631 token accuracy):
  *   [0] mean_v logits[r, v]                       (raw logits, not divided by the temperature)
- *   [1] log sum_v softmax(z[r])_v^2 = logsumexp(2 z) - 2 logsumexp(z)
+ *   [1] log sum_v softmax(z[r])_v^2 = logsumexp(2 z) - 2 logsumexp(z) if row_stats_sum_p2 is non-zero, else 0
+ *       (only the WPO weights use it, and it costs the kernel one more multiply-add per logit)
  *   [2] 1 if index[r, 0] is the row's arg-max (the FIRST maximal position, as torch.argmax), else 0
  *   [3] 0 (reserved)  An index outside [0, vocab) yields NaN for that entry and sets
  * TRLK_FLAG_INDEX_OUT_OF_RANGE in *d_error_flag.
@@ -90,7 +91,8 @@ const char* trlk_last_error(void);
 int trlk_logp_entropy_fwd(const void* d_logits, int dtype, int64_t n_seq, int64_t rows_per_seq, int64_t vocab,
                           int64_t seq_stride, int64_t row_stride, const int64_t* d_index, int32_t n_index,
                           float temperature, const uint8_t* d_row_mask, float* d_out_logp, float* d_out_entropy,
-                          float* d_out_lse, float* d_out_row_stats, int32_t* d_error_flag, trlk_stream_t stream);
+                          float* d_out_lse, float* d_out_row_stats, int32_t row_stats_sum_p2, int32_t* d_error_flag,
+                          trlk_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------
  * K3  backward of K1 by recomputation from the saved lse: one read and one write of the

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(raw, name), f"{name} is declared in include/trlk.h but not exported"
         assert name in _lib.SIGNATURES, f"{name} has no ctypes signature in trl_amd/_lib.py"
-    assert _lib.lib.trlk_version() == 1
+    assert _lib.lib.trlk_version() == _lib.ABI_VERSION == 2
 
 
 def test_host_side_argument_validation():
@@ -35,23 +35,23 @@ def test_host_side_argument_validation():
     lib = _lib.lib
     fake = 0x1000  # never dereferenced: every call below must fail validation first
     # vocab = 0
-    rc = lib.trlk_logp_entropy_fwd(fake, _lib.BF16, 1, 1, 0, 0, 0, fake, 1, 1.0, None, fake, None, None, None, None, None)
+    rc = lib.trlk_logp_entropy_fwd(fake, _lib.BF16, 1, 1, 0, 0, 0, fake, 1, 1.0, None, fake, None, None, None, 0, None, None)
     assert rc == -2 and "vocab" in _lib.last_error()
     # unsupported dtype code
-    rc = lib.trlk_logp_entropy_fwd(fake, 7, 1, 1, 8, 8, 8, fake, 1, 1.0, None, fake, None, None, None, None, None)
+    rc = lib.trlk_logp_entropy_fwd(fake, 7, 1, 1, 8, 8, 8, fake, 1, 1.0, None, fake, None, None, None, 0, None, None)
     assert rc == -3 and "dtype" in _lib.last_error()
     # null logits
-    rc = lib.trlk_logp_entropy_fwd(None, _lib.F32, 1, 1, 8, 8, 8, fake, 1, 1.0, None, fake, None, None, None, None, None)
+    rc = lib.trlk_logp_entropy_fwd(None, _lib.F32, 1, 1, 8, 8, 8, fake, 1, 1.0, None, fake, None, None, None, 0, None, None)
     assert rc == -1
     # overlapping rows
-    rc = lib.trlk_logp_entropy_fwd(fake, _lib.F32, 1, 4, 8, 32, 4, fake, 1, 1.0, None, fake, None, None, None, None, None)
+    rc = lib.trlk_logp_entropy_fwd(fake, _lib.F32, 1, 4, 8, 32, 4, fake, 1, 1.0, None, fake, None, None, None, 0, None, None)
     assert rc == -4 and "row_stride" in _lib.last_error()
     # temperature <= 0
-    rc = lib.trlk_logp_entropy_fwd(fake, _lib.F32, 1, 4, 8, 32, 8, fake, 1, 0.0, None, fake, None, None, None, None, None)
+    rc = lib.trlk_logp_entropy_fwd(fake, _lib.F32, 1, 4, 8, 32, 8, fake, 1, 0.0, None, fake, None, None, None, 0, None, None)
     assert rc == -5 and "temperature" in _lib.last_error()
     # row statistics: vocabulary too large for the exact count
     rc = lib.trlk_logp_entropy_fwd(fake, _lib.BF16, 1, 1, 1 << 24, 1 << 24, 1 << 24, fake, 1, 1.0, None, fake, None, None,
-                                   fake, None, None)
+                                   fake, 1, None, None)
     assert rc == -7 and "row statistics" in _lib.last_error()
     # backward: window does not fit the output rows
     rc = lib.trlk_logp_entropy_bwd(fake, _lib.F32, 1, 4, 8, 32, 8, fake, 1, 1.0, fake, None, fake, None, fake, 4, 1, 32,
@@ -137,7 +137,7 @@ def test_host_side_argument_validation():
     assert gemm(dtype=_lib.F32) == -3 and gemm(k=60) == -4 and gemm(lda=56) == -4 and gemm(ldo=8) == -4
     assert gemm(a=fake16 + 2) == -4 and gemm(a=None) == -1 and gemm(k=0) == -2
     # an empty problem is a successful no-op
-    assert lib.trlk_logp_entropy_fwd(None, _lib.F32, 0, 4, 8, 32, 8, None, 1, 1.0, None, None, None, None, None, None, None) == 0
+    assert lib.trlk_logp_entropy_fwd(None, _lib.F32, 0, 4, 8, 32, 8, None, 1, 1.0, None, None, None, None, None, 0, None, None) == 0
     assert _lib.last_error() == ""
 
 
@@ -146,7 +146,7 @@ def test_check_raises_python_exceptions():
 
     with pytest.raises(_lib.TrlkArgumentError, match="vocab"):
         _lib.check(_lib.lib.trlk_logp_entropy_fwd(0x1000, _lib.BF16, 1, 1, 0, 0, 0, 0x1000, 1, 1.0, None, 0x1000, None,
-                                                  None, None, None, None))
+                                                  None, None, 0, None, None))
     with pytest.raises(TypeError):
         import torch
 

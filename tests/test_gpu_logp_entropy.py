@@ -418,6 +418,13 @@ def test_row_statistics_of_the_same_pass():
         assert torch.equal(stats[..., 2][keep], want_hit[keep])
         assert want_hit[0, 2] == 0 and want_hit[1, 4] == 1 and want_hit[:, 1].sum() == B
         assert torch.equal(stats[1, 6], torch.zeros(4)) and float(logp.view(B, L)[1, 6]) == 0.0
+        # without the sum of squared probabilities: the same pass minus that sum, 0 in its slot, all else bit for bit
+        logp1, ent1, lse1, stats1 = ops.logp_entropy_stats_fwd(logits.to(DEV), ids.reshape(-1, 1).to(DEV), 1.0, 0, L,
+                                                               mask.reshape(-1).to(DEV), False)
+        stats1 = stats1.cpu().view(B, L, 4)
+        assert torch.equal(logp1, logp) and torch.equal(ent1, ent) and torch.equal(lse1, lse)
+        assert torch.equal(stats1[..., 1], torch.zeros(B, L))
+        assert torch.equal(stats1[..., [0, 2, 3]], stats[..., [0, 2, 3]])
         # the other outputs are those of the plain forward
         lp2, ent2, lse2 = ops.logp_entropy_fwd(logits.to(DEV), ids.reshape(-1, 1).to(DEV), 1.0, 0, L,
                                                mask.reshape(-1).to(DEV))

@@ -32,7 +32,7 @@ SIGNATURES = {
     "trlk_logp_entropy_fwd": (
         c_int32,
         [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int32, c_float, c_void_p,
-         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+         c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p],
     ),
     "trlk_logp_entropy_bwd": (
         c_int32,
@@ -108,6 +108,9 @@ SIGNATURES = {
 }
 
 
+ABI_VERSION = 2  # TRLK_VERSION of include/trlk.h that SIGNATURES was written against
+
+
 class TrlkError(RuntimeError):
     """A launch failed (positive status = hipError_t)."""
 
@@ -127,6 +130,10 @@ def _load():
         fn = getattr(lib, name)  # AttributeError here = the built library is stale
         fn.restype = restype
         fn.argtypes = argtypes
+    built = lib.trlk_version()
+    if built != ABI_VERSION:  # the signatures above would not match the library's
+        raise ImportError(f"{LIB_PATH} was built for interface version {built}, this package binds version "
+                          f"{ABI_VERSION}: rebuild it (python trl_amd/build.py)")
     return lib
 
 

@@ -510,10 +510,10 @@ int launch_fused_any(const FusedArgs& a, int nvec, bool ragged, unsigned rows, h
 }
 
 // data *= *scale over 16-byte vectors, unless the scale is exactly 1 (then nothing is read or written, and what the
-// launch costs is the dispatch of its workgroups: each takes a 256 KiB span so that a 20 GB buffer needs 76 000 of
-// them, about 0.02 ms, where one workgroup per 4 KiB costs a whole millisecond).  Inside a span the workgroup walks
+// launch costs is the dispatch of its workgroups: each takes a 1 MiB span so that a 20 GB buffer needs 19 000 of
+// them, a few microseconds, where one workgroup per 4 KiB costs a whole millisecond).  Inside a span the workgroup walks
 // 16 KiB at a time, four vectors per lane in flight.
-constexpr int kScaleSpanVec = 16384;  // vectors per workgroup
+constexpr int kScaleSpanVec = 65536;  // vectors per workgroup (1 MiB)
 template <int DT>
 __global__ __launch_bounds__(256) void scale_unless_one_kernel(u32x4* data, int64_t n_vec, int n_tail, const float* scale) {
     typedef Elem<DT> E;

@@ -142,8 +142,10 @@ __device__ __forceinline__ float max_of(const float* x) {
 
 // VEC: rows are 16-byte aligned and vocab is a multiple of the vector width.  Otherwise a row is read in aligned
 // vectors from its first 16-byte boundary on, and the few elements before that and after the last whole vector one by one.
-// STATS: also produce the row statistics of `out_stats`.
-template <int DT, bool VEC, bool STATS>
+// STATS: 1 or 2 also produce the row statistics of `out_stats`; only 2 accumulates the sum of squared probabilities
+// (one more multiply-add per logit in a loop that is bound by its arithmetic: 5.4 against 5.0 ms on 33.6 GB of bf16
+// logits), 1 reports 0 in its place.
+template <int DT, bool VEC, int STATS>
 __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
     typedef Elem<DT> E;
     typedef typename E::type T;
@@ -199,7 +201,7 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
         }
     };
     auto raise = [&](float bm) {
-        if constexpr (STATS) {
+        if constexpr (STATS == 2) {
             const float need = ceilf(bm * c);
             if (need > acc.r) {
                 const float sc = fast_exp2(acc.r - need);
@@ -209,7 +211,7 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
         acc.raise(bm, c);
     };
     auto add = [&](float x) {
-        if constexpr (STATS) {
+        if constexpr (STATS == 2) {
             const float e = fast_exp2(fmaf(x, c, -acc.rr));
             acc.s += e;
             acc.u = fmaf(e, x, acc.u);
@@ -306,7 +308,7 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
         red[2][wave] = u;
     }
     if constexpr (STATS) {
-        const float s2 = wave_sum(st.s2 * sc * sc);
+        const float s2 = STATS == 2 ? wave_sum(st.s2 * sc * sc) : 0.f;
         const float sx = wave_sum(st.sx);
         // the row maximum and the smallest position among the lanes that hold it
         const float wmax = wave_max(st.vmax);
@@ -340,7 +342,7 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
             const int64_t tpos = a.n_index > 0 ? a.index[row * a.n_index] : -1;
             float* o = a.out_stats + row * 4;
             o[0] = SX / float(V);
-            o[1] = logf(S2) - 2.f * logf(S);  // log sum_v softmax(z)_v^2: the common reference cancels
+            o[1] = STATS == 2 ? logf(S2) - 2.f * logf(S) : 0.f;  // log sum_v softmax(z)_v^2: the common reference cancels
             o[2] = (tpos >= 0 && tpos < V && float(tpos) == vpos) ? 1.f : 0.f;
             o[3] = 0.f;
         }
@@ -554,7 +556,8 @@ extern "C" int trlk_logp_entropy_fwd(const void* d_logits, int dtype, int64_t n_
                                      int64_t vocab, int64_t seq_stride, int64_t row_stride, const int64_t* d_index,
                                      int32_t n_index, float temperature, const uint8_t* d_row_mask,
                                      float* d_out_logp, float* d_out_entropy, float* d_out_lse,
-                                     float* d_out_row_stats, int32_t* d_error_flag, trlk_stream_t stream) {
+                                     float* d_out_row_stats, int32_t row_stats_sum_p2, int32_t* d_error_flag,
+                                     trlk_stream_t stream) {
     clear_error();
     if (int rc = check_view("logp_entropy_fwd: logits", d_logits, dtype, n_seq, rows_per_seq, vocab, seq_stride,
                             row_stride))
@@ -578,16 +581,20 @@ extern "C" int trlk_logp_entropy_fwd(const void* d_logits, int dtype, int64_t n_
     const bool vec = aligned16(d_logits, es, {seq_stride, row_stride}) && vocab % int64_t(16 / es) == 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)rows), block(kThreads);
-    const bool stats = d_out_row_stats != nullptr;
-#define TRLK_LAUNCH_FWD(DT)                                                                    \
-    if (vec && stats)                                                                          \
-        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, true, true>), grid, block, 0, s, a);   \
-    else if (vec)                                                                              \
-        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, true, false>), grid, block, 0, s, a);  \
-    else if (stats)                                                                            \
-        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, false, true>), grid, block, 0, s, a);  \
+    const int stats = d_out_row_stats == nullptr ? 0 : (row_stats_sum_p2 ? 2 : 1);
+#define TRLK_LAUNCH_FWD_VEC(DT, VEC)                                                           \
+    if (stats == 2)                                                                            \
+        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, VEC, 2>), grid, block, 0, s, a);       \
+    else if (stats == 1)                                                                       \
+        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, VEC, 1>), grid, block, 0, s, a);       \
     else                                                                                       \
-        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, false, false>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, VEC, 0>), grid, block, 0, s, a);
+#define TRLK_LAUNCH_FWD(DT)                                                                    \
+    if (vec) {                                                                                 \
+        TRLK_LAUNCH_FWD_VEC(DT, true)                                                          \
+    } else {                                                                                   \
+        TRLK_LAUNCH_FWD_VEC(DT, false)                                                         \
+    }
     if (dtype == TRLK_F32) {
         TRLK_LAUNCH_FWD(TRLK_F32)
     } else if (dtype == TRLK_BF16) {
@@ -596,6 +603,7 @@ extern "C" int trlk_logp_entropy_fwd(const void* d_logits, int dtype, int64_t n_
         TRLK_LAUNCH_FWD(TRLK_F16)
     }
 #undef TRLK_LAUNCH_FWD
+#undef TRLK_LAUNCH_FWD_VEC
     return launch_status("logp_entropy_fwd");
 }
 

@@ -94,7 +94,8 @@ def dpo_compute_loss(
     if idx.dtype != torch.int64:
         idx = idx.long()
     rm = (smask.reshape(-1) != 0).to(torch.uint8).contiguous() if skip_masked_rows else None
-    logp, ent, _, stats = ops.logp_entropy_stats_fwd(logits, idx, 1.0, 0, length - 1, rm)
+    # (the sum of squared probabilities is wanted by the WPO weights only)
+    logp, ent, _, stats = ops.logp_entropy_stats_fwd(logits, idx, 1.0, 0, length - 1, rm, bool(use_weighting))
     m = smask.to(torch.float32)
     ent = ent.view(n_seq, length - 1).detach()
     stats = stats.view(n_seq, length - 1, 4).detach()

@@ -314,11 +314,11 @@ class _GRPOFromLogits(torch.autograd.Function):
         if not kw["skip_masked_rows"] and keep_len > 0:
             # the outputs of the rows without gradient come from the streaming forward kernel, which reads them
             # faster than the one-workgroup-per-CU kernel would (its `compute_masked_rows` mode)
-            rest = (mask_f == 0).to(torch.uint8)
+            rest = mask_f == 0
             lp0, ent0, _ = ops.logp_entropy_fwd(logits.detach(), ids.reshape(-1, 1), float(temperature), keep_start,
-                                                keep_len, rest.reshape(-1).contiguous())
-            logp = torch.where(rest.bool(), lp0.view_as(logp), logp)
-            ent = torch.where(rest.bool(), ent0.view_as(ent), ent)
+                                                keep_len, rest.view(torch.uint8).reshape(-1))
+            logp = torch.where(rest, lp0.view_as(logp), logp)
+            ent = torch.where(rest, ent0.view_as(ent), ent)
         # loss value and every metric from the [B, K]-sized kernel, on the log-probs of the same pass
         loss, metrics = grpo_loss(
             logp, advantages, mask_f, entropies=ent, old_per_token_logps=kw["old_per_token_logps"],

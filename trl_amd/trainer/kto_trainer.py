@@ -22,7 +22,7 @@ def _shifted_logps(logits: Tensor, input_ids: Tensor, completion_mask: Tensor, s
         idx = idx.long()
     rm = (smask.reshape(-1) != 0).to(torch.uint8).contiguous() if skip_masked_rows else None
     if stats:
-        logp, ent, _, st = ops.logp_entropy_stats_fwd(logits, idx, 1.0, 0, length - 1, rm)
+        logp, ent, _, st = ops.logp_entropy_stats_fwd(logits, idx, 1.0, 0, length - 1, rm, False)
         st = st.view(n_seq, length - 1, 4).detach()
         ent = ent.view(n_seq, length - 1).detach()
     else:
