@@ -198,6 +198,25 @@ def test_upstream_gradient_scales(amd):
     assert _rel_l2(b.grad.float(), a.grad.float() * 0.25) == 0.0
 
 
+def test_scale_kernel_reaches_every_element(amd):
+    """`ops.scale_unless_one_` on buffers from one element to many pieces per workgroup and region (its workgroups
+    step through eight regions of the buffer piece by piece): every element scaled exactly once, bit for bit what
+    torch gives; a scale of 1 leaves the buffer as it is."""
+    from trl_amd import ops
+
+    g = torch.Generator(device=DEV).manual_seed(91)
+    piece = 8 * 1024  # 16-bit elements of one 16 KiB piece
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        per = piece if dtype != torch.float32 else piece // 2
+        for n in (1, 5, 8, per - 1, per, 3 * per + 1, 8 * per, 9 * per + 7, 520 * per + 13, (64 * 8 * 2 + 77) * per + 5):
+            x = torch.randn((n,), generator=g, device=DEV).to(dtype)
+            want = (x.float() * 0.37).to(dtype)
+            got = ops.scale_unless_one_(x.clone(), torch.tensor(0.37, device=DEV))
+            assert torch.equal(got, want), (dtype, n)
+            same = ops.scale_unless_one_(x.clone(), torch.tensor(1.0, device=DEV))
+            assert torch.equal(same, x), (dtype, n)
+
+
 def test_fp16_and_token_weight_and_per_token_advantages(amd):
     B, K, V = 4, 24, 1024
     logits, ids, mask, _, g = _inputs(B, K, V, dtype=torch.float16, seed=7)

@@ -510,10 +510,13 @@ int launch_fused_any(const FusedArgs& a, int nvec, bool ragged, unsigned rows, h
 }
 
 // data *= *scale over 16-byte vectors, unless the scale is exactly 1 (then nothing is read or written, and what the
-// launch costs is the dispatch of its workgroups: each takes a 1 MiB span so that a 20 GB buffer needs 19 000 of
-// them, a few microseconds, where one workgroup per 4 KiB costs a whole millisecond).  Inside a span the workgroup walks
-// 16 KiB at a time, four vectors per lane in flight.
-constexpr int kScaleSpanVec = 65536;  // vectors per workgroup (1 MiB)
+// launch costs is the dispatch of its workgroups: each takes 64 pieces of 16 KiB so that a 20 GB buffer needs 19 000
+// of them, a few microseconds, where one workgroup per 4 KiB costs a whole millisecond).  The buffer is cut into eight
+// contiguous regions, one per XCD (the hardware deals consecutive workgroups to the XCDs in turn), and the workgroups
+// of a region step through it together, piece by piece, so that what is read and written at one time is one narrow
+// window per XCD.
+constexpr int kScalePieceVec = 1024;  // vectors per piece (16 KiB): four per lane in flight
+constexpr int kScalePieces = 64;      // pieces per workgroup
 template <int DT>
 __global__ __launch_bounds__(256) void scale_unless_one_kernel(u32x4* data, int64_t n_vec, int n_tail, const float* scale) {
     typedef Elem<DT> E;
@@ -523,11 +526,14 @@ __global__ __launch_bounds__(256) void scale_unless_one_kernel(u32x4* data, int6
         typename E::type* p = reinterpret_cast<typename E::type*>(data + n_vec) + threadIdx.x;
         E::store1(p, E::load1(p) * sc);
     }
-    const int64_t base = int64_t(blockIdx.x) * kScaleSpanVec + threadIdx.x;
+    const int64_t n_pieces = (n_vec + kScalePieceVec - 1) / kScalePieceVec;
+    const int64_t per_xcd = (n_pieces + 7) >> 3;
+    const int64_t slots = int64_t(gridDim.x) >> 3;  // the host launches a multiple of eight workgroups
+    const int64_t first = int64_t(blockIdx.x & 7) * per_xcd;
 #pragma unroll 1
-    for (int it = 0; it < kScaleSpanVec / 1024; ++it) {
+    for (int64_t c = blockIdx.x >> 3; c < per_xcd && first + c < n_pieces; c += slots) {
         u32x4 q[4];
-        const int64_t v0 = base + it * 1024;
+        const int64_t v0 = (first + c) * kScalePieceVec + threadIdx.x;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             if (v0 + j * 256 < n_vec) q[j] = __builtin_nontemporal_load(data + v0 + j * 256);
@@ -559,8 +565,10 @@ extern "C" int trlk_scale_unless_one(void* d_data, int dtype, int64_t n_elems, c
                  "scale_unless_one: null or misaligned pointer");
     const int64_t n_vec = n_elems / epv;
     const int n_tail = int(n_elems - n_vec * epv);
-    TRLK_REQUIRE(n_vec <= int64_t(kScaleSpanVec) * 0x7fffffff, TRLK_ERR_BAD_SHAPE, "scale_unless_one: too many elements");
-    const unsigned grid = unsigned((n_vec + kScaleSpanVec - 1) / kScaleSpanVec) + (n_vec == 0 ? 1u : 0u);
+    const int64_t n_pieces = (n_vec + kScalePieceVec - 1) / kScalePieceVec;
+    const int64_t slots = ((n_pieces + 7) / 8 + kScalePieces - 1) / kScalePieces;  // workgroups per region
+    TRLK_REQUIRE(slots <= 0x0fffffff, TRLK_ERR_BAD_SHAPE, "scale_unless_one: too many elements");
+    const unsigned grid = 8u * unsigned(slots > 0 ? slots : 1);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == TRLK_BF16)
         hipLaunchKernelGGL(scale_unless_one_kernel<TRLK_BF16>, dim3(grid), dim3(256), 0, s, static_cast<u32x4*>(d_data), n_vec, n_tail, d_scale);
