@@ -493,6 +493,40 @@ def test_trainer_method_takes_the_single_pass(amd, loss_type, beta, is_ratio, en
         assert (math.isnan(m1[k]) and math.isnan(m2[k])) or abs(m1[k] - m2[k]) <= 1e-5 * max(1.0, abs(m2[k])), k
 
 
+def test_trainer_method_picks_the_path_by_row_length(amd, monkeypatch):
+    """Without `trl_amd_single_pass` on the trainer the one pass is taken for rows of at least 40 KiB only (shorter
+    rows are faster through the two kernels); `True` takes it for every row the kernel accepts, `False` never."""
+    from types import SimpleNamespace
+
+    from test_gpu_losses import _fake_trainer
+    from trl_amd import ops
+
+    B, P, K = 2, 1, 5
+    g = torch.Generator(device=DEV).manual_seed(17)
+    case = dict(temperature=1.0, beta=0.0, loss_type="dapo", eps_low=0.2, eps_high=0.2)
+    calls = []
+    inner = ops.grpo_fused_fwd_bwd
+    monkeypatch.setattr(ops, "grpo_fused_fwd_bwd", lambda *a, **k: (calls.append(1), inner(*a, **k))[1])
+    for V, dtype, want, expect in ((1024, torch.bfloat16, None, 0), (20480, torch.bfloat16, None, 1), (20472, torch.bfloat16, None, 0),
+                                   (10240, torch.float32, None, 1), (1024, torch.bfloat16, True, 1),
+                                   (20480, torch.bfloat16, False, 0)):
+        logits = torch.randn((B, P + K, V), generator=g, device=DEV).to(dtype)
+        completion_ids = torch.randint(0, V, (B, K), generator=g, device=DEV)
+        cmask = torch.ones((B, K), dtype=torch.long, device=DEV)
+        inputs = dict(prompt_ids=torch.zeros((B, P), dtype=torch.long, device=DEV),
+                      prompt_mask=torch.ones((B, P), dtype=torch.long, device=DEV), completion_ids=completion_ids,
+                      completion_mask=cmask, advantages=torch.randn((B,), generator=g, device=DEV),
+                      num_items_in_batch=cmask.sum().float())
+        tr = _fake_trainer(amd, case, K, skip_masked=True, single_pass=want)
+        if want is None:
+            del tr.trl_amd_single_pass
+        leaf = logits.detach().clone().requires_grad_(True)
+        del calls[:]
+        tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None), inputs).backward()
+        assert len(calls) == expect, (V, dtype, want)
+        assert leaf.grad is not None and torch.isfinite(leaf.grad.float()).all()
+
+
 @pytest.mark.parametrize("loss_type", ["dapo", "grpo", "dr_grpo", "bnpo"])
 def test_against_the_oracle_autograd(amd, loss_type):
     """Independent of the two-pass kernels: the CPU oracle's log-probs, loss and autograd gradient on the same

@@ -234,6 +234,12 @@ def grpo_loss(
 _SINGLE_PASS_LOSS_TYPES = ("grpo", "bnpo", "dr_grpo", "dapo", "cispo", "sapo")
 
 
+# Rows shorter than this go through the two-pass kernels by default: on bf16 [64, 1024, V] logits with half of the
+# rows masked the one pass takes 0.70 / 0.78 / 0.82 / 1.15 ms at V = 8192 / 16384 / 20480 / 32000, the two passes
+# 0.51 / 0.79 / 0.94 / 1.41 ms.
+_SINGLE_PASS_MIN_ROW_BYTES = 40960
+
+
 def grpo_single_pass_supported(logits: Tensor, loss_type: str = "dapo", importance_sampling_level: str = "token",
                                entropy_coef: float = 0.0, entropy_mask: Tensor | None = None) -> bool:
     """Whether `grpo_loss_from_logits` can go from these logits to their gradient in one pass: a token-level
@@ -548,15 +554,18 @@ class GRPOLossMixin:
         bonus = bool(getattr(self, "_entropy_bonus_enabled", False))
         # One pass over the logits (log-probs and gradient from the same read) when nothing between the two
         # needs the log-probs of other tokens: token-level weights, no mask derived from the log-probs or
-        # entropies.  `trl_amd_single_pass = False` on the trainer keeps the two-pass path.
+        # entropies.  `trl_amd_single_pass` on the trainer: False keeps the two-pass path, True takes the one pass
+        # whenever the kernel accepts the logits, unset (the default) takes it when it also pays: rows of at least
+        # `_SINGLE_PASS_MIN_ROW_BYTES` (a workgroup per row spends more time between rows than on them below that).
         adaptive = bonus and bool(getattr(self, "use_adaptive_entropy", False))
         # the coefficient of the end of the previous optimizer step applies to the whole accumulation window;
         # under adaptive control only while the last window's entropy was at or below the target (:3173-3179)
         apply_coef = self.entropy_coef if bonus else 0.0
         if adaptive and not (self._last_world_entropy <= self.args.entropy_target):
             apply_coef = 0.0
+        want_single = getattr(self, "trl_amd_single_pass", None)
         single_pass = (
-            getattr(self, "trl_amd_single_pass", True) and skip is not None
+            want_single is not False and skip is not None
             and self.loss_type in _SINGLE_PASS_LOSS_TYPES and self.importance_sampling_level == "token"
             and self.top_entropy_quantile >= 1.0 and self.off_policy_mask_threshold is None
         )
@@ -576,7 +585,9 @@ class GRPOLossMixin:
             # fp16 gradients of a 1e5-entry softmax row sit near the bottom of the fp16 range: the one pass rounds
             # them once, so it is only taken when the scale is known at that point (or on request)
             fp16_ok = upstream is not None or getattr(self, "trl_amd_single_pass_fp16", False)
-            if grpo_single_pass_supported(logits, self.loss_type) and (logits.dtype != torch.float16 or fp16_ok):
+            pays = want_single is True or logits.shape[-1] * logits.element_size() >= _SINGLE_PASS_MIN_ROW_BYTES
+            if (pays and grpo_single_pass_supported(logits, self.loss_type)
+                    and (logits.dtype != torch.float16 or fp16_ok)):
                 token_weight = None
                 if self.use_vllm and self.vllm_importance_sampling_correction:
                     token_weight = inputs["importance_sampling_ratio"].float().expand(mask.shape)
