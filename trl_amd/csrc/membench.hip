@@ -106,6 +106,35 @@ __global__ __launch_bounds__(1024) void row_kernel(const u32x4* in, u32x4* out, 
         }
 }
 
+// GROUP workgroups of one XCD share GROUP neighbouring rows: each takes the same slice (a GROUP-th of the row, at most
+// 1024 vectors) of every one of them, so that a row is read and written by GROUP compute units at the same time and
+// a workgroup still holds a row's worth of vectors.  (What a kernel that keeps its rows on chip would look like to
+// the memory if the rows were spread over the compute units of an XCD; the statistics such a kernel needs per row
+// would have to be exchanged between the workgroups, which this copy does not do.)
+template <int GROUP>
+__global__ __launch_bounds__(1024) void slice_kernel(const u32x4* in, u32x4* out, const uint8_t* active, int64_t rows_per_xcd) {
+    constexpr int kSliceVec = (kRowVec + GROUP - 1) / GROUP;
+    static_assert(kSliceVec <= 1024, "a slice is at most one vector per lane");
+    const int tid = threadIdx.x;
+    const int64_t slot = blockIdx.x >> 3;
+    const int64_t group = slot / GROUP;
+    const int slice = int(slot % GROUP);
+    const int64_t row0 = int64_t(blockIdx.x & 7) * rows_per_xcd + group * GROUP;
+    if (group * GROUP + GROUP > rows_per_xcd) return;  // (the last few rows of a region are left out of this test)
+    const int v = slice * kSliceVec + tid;
+    const bool mine = tid < kSliceVec && v < kRowVec;
+    u32x4 q[GROUP];
+#pragma unroll
+    for (int j = 0; j < GROUP; ++j)
+        if (mine && active[row0 + j]) q[j] = in[(row0 + j) * kRowVec + v];
+#pragma unroll
+    for (int j = 0; j < GROUP; ++j) asm volatile("" : "+v"(q[j]));
+    const u32x4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < GROUP; ++j)
+        if (mine) __builtin_nontemporal_store(active[row0 + j] ? q[j] : z, out + (row0 + j) * kRowVec + v);
+}
+
 template <int THREADS, int PARTS>
 __global__ __launch_bounds__(THREADS) void piece_kernel(const u32x4* in, u32x4* out, const uint8_t* active) {
     constexpr int kPieceVec = (kRowVec + PARTS - 1) / PARTS;
@@ -199,6 +228,19 @@ int main() {
         run(masked ? "row in registers, one region of rows per XCD, benchmark mask, plain/nt"
                    : "row in registers, one region of rows per XCD, every row, plain/nt", moved,
             [&] { hipLaunchKernelGGL((row_kernel<false, true, true>), dim3(unsigned(rows)), dim3(1024), 0, 0, in, out, act_d); });
+        {
+            constexpr int G = 19;
+            const int64_t per_xcd = rows / 8, groups = per_xcd / G;
+            int64_t act_in = 0, all_in = 0;  // the rows the grouped kernel covers
+            for (int x = 0; x < 8; ++x)
+                for (int64_t r = 0; r < groups * G; ++r) {
+                    act_in += masked ? act[x * per_xcd + r] : 1;
+                    ++all_in;
+                }
+            const double moved_g = (act_in * 2 + (all_in - act_in)) * row_bytes;
+            run(masked ? "19 rows sliced over 19 workgroups of an XCD, benchmark mask" : "19 rows sliced over 19 workgroups of an XCD, every row",
+                moved_g, [&] { hipLaunchKernelGGL((slice_kernel<G>), dim3(unsigned(8 * groups * G)), dim3(1024), 0, 0, in, out, act_d, per_xcd); });
+        }
         run(masked ? "2 pieces of 1024 lanes, benchmark mask, plain/nt" : "2 pieces of 1024 lanes, every row, plain/nt", moved,
             [&] { hipLaunchKernelGGL((piece_kernel<1024, 2>), dim3(unsigned(rows * 2)), dim3(1024), 0, 0, in, out, act_d); });
         run(masked ? "2 pieces of 512 lanes, benchmark mask, plain/nt" : "2 pieces of 512 lanes, every row, plain/nt", moved,
