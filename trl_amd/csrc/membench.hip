@@ -135,6 +135,43 @@ __global__ __launch_bounds__(1024) void slice_kernel(const u32x4* in, u32x4* out
         if (mine) __builtin_nontemporal_store(active[row0 + j] ? q[j] : z, out + (row0 + j) * kRowVec + v);
 }
 
+// A workgroup takes RUN consecutive rows and refills every register with the next row's vector as soon as it has stored
+// the current row's: a compute unit then reads and writes all the time instead of a row's worth of loads followed by a
+// row's worth of stores, and the next row's load latency hides behind the current row's stores.
+template <int RUN>
+__global__ __launch_bounds__(1024) void row_run_kernel(const u32x4* in, u32x4* out, const uint8_t* active, int64_t rows_per_xcd) {
+    constexpr int PER = (kRowVec + 1023) / 1024;
+    const int tid = threadIdx.x;
+    const int64_t row0 = int64_t(blockIdx.x & 7) * rows_per_xcd + int64_t(blockIdx.x >> 3) * RUN;
+    u32x4 q[PER];
+    // the flags of the whole run first: a flag loaded inside the loop would wait for everything in flight
+    uint64_t flags = 0;
+    for (int i = 0; i < RUN; ++i) flags |= uint64_t(active[row0 + i] != 0) << i;
+    flags = __builtin_amdgcn_readfirstlane(uint32_t(flags)) | uint64_t(__builtin_amdgcn_readfirstlane(uint32_t(flags >> 32))) << 32;
+    bool have = flags & 1;
+    if (have) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j)
+            if (j * 1024 + tid < kRowVec) q[j] = in[row0 * kRowVec + j * 1024 + tid];
+    }
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    // (short runs are unrolled: across a loop's back edge the compiler waits for everything in flight, the stores'
+    // acknowledgements included, and the straight-line form waits for exactly the load it stores next)
+#pragma unroll(RUN <= 8 ? RUN : 1)
+    for (int i = 0; i < RUN; ++i) {
+        const int64_t row = row0 + i;
+        const bool next = i + 1 < RUN && ((flags >> (i + 1)) & 1);
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            if (j * 1024 + tid < kRowVec) {
+                __builtin_nontemporal_store(have ? q[j] : z, out + row * kRowVec + j * 1024 + tid);
+                if (next) q[j] = in[(row + 1) * kRowVec + j * 1024 + tid];
+            }
+        }
+        have = next;
+    }
+}
+
 template <int THREADS, int PARTS>
 __global__ __launch_bounds__(THREADS) void piece_kernel(const u32x4* in, u32x4* out, const uint8_t* active) {
     constexpr int kPieceVec = (kRowVec + PARTS - 1) / PARTS;
@@ -241,6 +278,12 @@ int main() {
             run(masked ? "19 rows sliced over 19 workgroups of an XCD, benchmark mask" : "19 rows sliced over 19 workgroups of an XCD, every row",
                 moved_g, [&] { hipLaunchKernelGGL((slice_kernel<G>), dim3(unsigned(8 * groups * G)), dim3(1024), 0, 0, in, out, act_d, per_xcd); });
         }
+        run(masked ? "runs of 4 rows per workgroup, refilled while storing, benchmark mask" : "runs of 4 rows per workgroup, refilled while storing, every row",
+            moved, [&] { hipLaunchKernelGGL((row_run_kernel<4>), dim3(unsigned(rows / 4)), dim3(1024), 0, 0, in, out, act_d, rows / 8); });
+        run(masked ? "runs of 8 rows per workgroup, refilled while storing, benchmark mask" : "runs of 8 rows per workgroup, refilled while storing, every row",
+            moved, [&] { hipLaunchKernelGGL((row_run_kernel<8>), dim3(unsigned(rows / 8)), dim3(1024), 0, 0, in, out, act_d, rows / 8); });
+        run(masked ? "runs of 64 rows per workgroup, refilled while storing, benchmark mask" : "runs of 64 rows per workgroup, refilled while storing, every row",
+            moved, [&] { hipLaunchKernelGGL((row_run_kernel<64>), dim3(unsigned(rows / 64)), dim3(1024), 0, 0, in, out, act_d, rows / 8); });
         run(masked ? "2 pieces of 1024 lanes, benchmark mask, plain/nt" : "2 pieces of 1024 lanes, every row, plain/nt", moved,
             [&] { hipLaunchKernelGGL((piece_kernel<1024, 2>), dim3(unsigned(rows * 2)), dim3(1024), 0, 0, in, out, act_d); });
         run(masked ? "2 pieces of 512 lanes, benchmark mask, plain/nt" : "2 pieces of 512 lanes, every row, plain/nt", moved,
