@@ -304,6 +304,26 @@ def bench_head(args, w):
                 "fwd_ms": fwd_plain, "bwd_ms": bwd_rec, "fwd_TFLOPs": flop / (fwd_plain * 1e-3) / 1e12,
                 "bwd_TFLOPs": 3 * flop / (bwd_rec * 1e-3) / 1e12,
                 "TFLOPs": 4 * flop / ((fwd_plain + bwd_rec) * 1e-3) / 1e12}
+    # the SFT loss on the same operands: next-token cross-entropy of the completion tokens (prompt and padding
+    # positions labelled -100 and dropped before the head), forward + backward, through the same kernels
+    from trl_amd.trainer.sft_trainer import _chunked_cross_entropy_loss
+    sft_labels = torch.where(mask.bool(), targets.view(B, T), torch.full_like(targets.view(B, T), -100))
+
+    def sft_step():
+        hidden.grad = weight.grad = None
+        out = _chunked_cross_entropy_loss(hidden.view(B, T, H), weight, HEAD_CHUNK, shift_labels=sft_labels)
+        out[0].backward()
+        return out
+
+    sft_ms = time_op(sft_step)
+    sft_out = sft_step()
+    n_sft = int(sft_out[3])
+    hidden.grad = weight.grad = None
+    kernels["sft_chunked_nll_step"] = {
+        "ms_per_step": sft_ms, "tokens_with_label": n_sft, "tokens_per_s": N / (sft_ms * 1e-3),
+        "loss": float(sft_out[0].detach()), "TFLOPs": 3 * 2.0 * n_sft * H * V / (sft_ms * 1e-3) / 1e12,
+        "note": "SFTTrainer's chunked_nll loss (loss, correct-token count, entropy sum) forward + backward on the "
+                "tokens that carry a label; three products of 2*n*H*V flop"}
     bwd_flop = (2 if stash else 3) * flop  # products actually executed by the backward
     fwd_tf, bwd_tf = flop / (fwd_ms * 1e-3) / 1e12, bwd_flop / (bwd_ms * 1e-3) / 1e12
     total_tf = (flop + bwd_flop) / ((fwd_ms + bwd_ms) * 1e-3) / 1e12
@@ -415,6 +435,18 @@ def bench_dpo(args, w):
         fwd_ms = time_kernel(lambda: ops.logp_entropy_stats_fwd(logits.detach(), idx, 1.0, 0, L - 1, None, False))
         fwd_p2_ms = time_kernel(lambda: ops.logp_entropy_stats_fwd(logits.detach(), idx, 1.0, 0, L - 1, None, True))
         bwd_ms = time_kernel(lambda: ops.logp_entropy_bwd(logits.detach(), idx, 1.0, 0, L - 1, lse, None, g_logp, None))
+    # the KTO loss on the same logits (first half of the batch desirable, second half undesirable; no KL batch):
+    # one pass with row statistics, [B]-sized arithmetic, the gradient kernel
+    kto_label = torch.arange(B, device=dev) < B // 2
+
+    def kto_step():
+        leaf.grad = None
+        loss, _ = trl_amd.kto_compute_loss(leaf, ids, cmask, kto_label, ref, beta=w["beta"], skip_masked_rows=False)
+        loss.backward()
+        return loss
+
+    kto_ms = time_kernel(kto_step, reps=3)
+    leaf.grad = None
     row_bytes = V * 2
     fwd_bytes = R * row_bytes
     bwd_bytes = active * 2 * row_bytes + (B * L - active) * row_bytes  # masked rows and the last position: zero fill
@@ -433,6 +465,8 @@ def bench_dpo(args, w):
             "avg_launch_ms": fwd_ms, "algorithmic_bytes": fwd_bytes, "achieved_GBps": fwd_bytes / (fwd_ms * 1e-3) / 1e9,
             "frac": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "with_sum_of_squared_probabilities_ms": fwd_p2_ms}},
+        "kto": {"ms_per_step": kto_ms, "tokens_per_s": R / (kto_ms * 1e-3),
+                "note": "KTOTrainer's loss (kto, no KL batch) forward + backward on the same logits: the same two kernels"},
         "mask_aware": {"ms_per_step": ms_aware, "tokens_per_s": R / (ms_aware * 1e-3),
                        "note": "only rows inside the completion mask are read; loss, metrics and dlogits identical"},
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_dpo(w),

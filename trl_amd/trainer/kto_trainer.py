@@ -63,35 +63,36 @@ def kto_compute_loss(
     seq = tok.sum(dim=1)
     dev = logits.device
     is_chosen = torch.as_tensor(label, dtype=torch.bool, device=dev)
-    chosen_idx = torch.nonzero(is_chosen).view(-1)
-    rejected_idx = torch.nonzero(~is_chosen).view(-1)
-    ref = ref_logps.to(torch.float32)
-    c_lr = seq.index_select(0, chosen_idx) - ref.index_select(0, chosen_idx)
-    r_lr = seq.index_select(0, rejected_idx) - ref.index_select(0, rejected_idx)
+    # (desirable and undesirable examples are told apart by masks, not gathered by index: `nonzero` would make the
+    # host wait for the pass over the logits that was just launched)
+    lr = seq - ref_logps.to(torch.float32)
     if kl_logps is not None:
         kl = (kl_logps.float() - ref_kl_logps.float()).mean().detach()
         kl = (kl if kl_reduce is None else kl_reduce(kl)).clamp(min=0)
     else:
         kl = torch.zeros(1, device=dev)
     if loss_type == "kto":
-        c_loss = 1 - torch.sigmoid(beta * (c_lr - kl))
-        r_loss = 1 - torch.sigmoid(beta * (kl - r_lr))
+        c_loss = 1 - torch.sigmoid(beta * (lr - kl))
+        r_loss = 1 - torch.sigmoid(beta * (kl - lr))
     else:
-        c_loss = 1 - torch.sigmoid(beta * c_lr)
-        r_loss = torch.sigmoid(beta * r_lr)
-    loss = torch.cat((desirable_weight * c_loss, undesirable_weight * r_loss), 0).nanmean()
+        c_loss = 1 - torch.sigmoid(beta * lr)
+        r_loss = torch.sigmoid(beta * lr)
+    loss = torch.where(is_chosen, desirable_weight * c_loss, undesirable_weight * r_loss).nanmean()
     with torch.no_grad():
-        cm = m.index_select(0, chosen_idx)
-        rm_ = m.index_select(0, rejected_idx)
+        chosen_f = is_chosen.to(torch.float32)
+        cm, rm_ = m * chosen_f[:, None], m * (1 - chosen_f)[:, None]
         mean_logit = stats[..., 0]
+        zero = torch.zeros((), device=dev)
+        lr_d, seq_d = lr.detach(), seq.detach()
         metrics = {
             "kl": kl, "entropy_sum": (ent * m).sum(), "n_tokens": m.sum(),
-            "logits_chosen_sum": (mean_logit.index_select(0, chosen_idx) * cm).sum(), "n_chosen_tokens": cm.sum(),
-            "logits_rejected_sum": (mean_logit.index_select(0, rejected_idx) * rm_).sum(), "n_rejected_tokens": rm_.sum(),
+            "logits_chosen_sum": torch.where(cm > 0, mean_logit, zero).sum(), "n_chosen_tokens": cm.sum(),
+            "logits_rejected_sum": torch.where(rm_ > 0, mean_logit, zero).sum(), "n_rejected_tokens": rm_.sum(),
             "num_chosen": is_chosen.sum(), "num_rejected": (~is_chosen).sum(),
-            "chosen_rewards_sum": (beta * c_lr.detach()).nansum(), "rejected_rewards_sum": (beta * r_lr.detach()).nansum(),
-            "chosen_logps_sum": seq.detach().index_select(0, chosen_idx).nansum(),
-            "rejected_logps_sum": seq.detach().index_select(0, rejected_idx).nansum(),
+            "chosen_rewards_sum": torch.where(is_chosen, beta * lr_d, zero).nansum(),
+            "rejected_rewards_sum": torch.where(is_chosen, zero, beta * lr_d).nansum(),
+            "chosen_logps_sum": torch.where(is_chosen, seq_d, zero).nansum(),
+            "rejected_logps_sum": torch.where(is_chosen, zero, seq_d).nansum(),
         }
     return loss, metrics
 
