@@ -291,23 +291,29 @@ class DPOLossMixin:
         counts = torch.stack([parts[k] for k in ("entropy_sum", "n_tokens", "logits_chosen_sum", "n_chosen_tokens",
                                                   "logits_rejected_sum", "n_rejected_tokens", "correct_tokens")])
         bits = ops.device_error_bits(counts.device)  # (a token id outside the vocabulary raises here)
-        ent_sum, n_tok, lc, nc, lr, nr, correct, bits = torch.cat(
-            [acc.gather_for_metrics(counts.unsqueeze(0)).sum(dim=0), bits.to(counts.dtype)]).tolist()
+        c_rew, r_rew = acc.gather(parts["chosen_rewards"]), acc.gather(parts["rejected_rewards"])
+        means = torch.stack([c_rew.mean(), r_rew.mean(), (c_rew > r_rew).float().mean(), (c_rew - r_rew).mean(),
+                             acc.gather(parts["chosen_logps"]).mean(), acc.gather(parts["rejected_logps"]).mean()])
+        n_train = (acc.gather_for_metrics(inputs["attention_mask"].sum()).sum().reshape(1) if mode == "train"
+                   else counts.new_zeros(1))
+        # every logged number in ONE copy to the host (each `.item()` would make the host wait for the device again)
+        (ent_sum, n_tok, lc, nc, lr, nr, correct, bits, rew_c, rew_r, rew_acc, rew_margin, logp_c, logp_r,
+         n_train) = torch.cat([acc.gather_for_metrics(counts.unsqueeze(0)).sum(dim=0).double(), bits.double(),
+                               means.double(), n_train.double()]).tolist()
         ops.raise_for_error_bits(bits, counts.device)
         log["entropy"].append(ent_sum / n_tok if n_tok > 0 else 0.0)
         if mode == "train":
-            self._total_train_tokens += acc.gather_for_metrics(inputs["attention_mask"].sum()).sum().item()
+            self._total_train_tokens += int(n_train)
         log["num_tokens"] = [self._total_train_tokens]
         log["logits/chosen"].append(lc / nc if nc > 0 else 0.0)
         log["logits/rejected"].append(lr / nr if nr > 0 else 0.0)
         log["mean_token_accuracy"].append(correct / nc if nc > 0 else 0.0)
-        c_rew, r_rew = acc.gather(parts["chosen_rewards"]), acc.gather(parts["rejected_rewards"])
-        log["rewards/chosen"].append(c_rew.mean().item())
-        log["rewards/rejected"].append(r_rew.mean().item())
-        log["rewards/accuracies"].append((c_rew > r_rew).float().mean().item())
-        log["rewards/margins"].append((c_rew - r_rew).mean().item())
-        log["logps/chosen"].append(acc.gather(parts["chosen_logps"]).mean().item())
-        log["logps/rejected"].append(acc.gather(parts["rejected_logps"]).mean().item())
+        log["rewards/chosen"].append(rew_c)
+        log["rewards/rejected"].append(rew_r)
+        log["rewards/accuracies"].append(rew_acc)
+        log["rewards/margins"].append(rew_margin)
+        log["logps/chosen"].append(logp_c)
+        log["logps/rejected"].append(logp_r)
         return (loss, outputs) if return_outputs else loss
 
 

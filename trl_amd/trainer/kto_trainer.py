@@ -152,17 +152,21 @@ class KTOLossMixin:
             beta=self.beta, loss_type=self.loss_type, desirable_weight=self.desirable_weight,
             undesirable_weight=self.undesirable_weight, kl_reduce=lambda kl: acc.gather_for_metrics(kl).mean())
         log = self._metrics[mode]
-        log["kl"].append(parts["kl"].item())
         names = ("entropy_sum", "n_tokens", "logits_chosen_sum", "n_chosen_tokens", "logits_rejected_sum",
                  "n_rejected_tokens", "num_chosen", "num_rejected", "chosen_rewards_sum", "rejected_rewards_sum",
                  "chosen_logps_sum", "rejected_logps_sum")
         sums = torch.stack([parts[k].to(torch.float32) for k in names])
-        (ent_sum, n_tok, lc, nc, lr, nr, n_c, n_r, rew_c, rew_r, lp_c, lp_r, bits) = torch.cat(
-            [acc.gather_for_metrics(sums.unsqueeze(0)).nansum(dim=0), ops.device_error_bits(sums.device)]).tolist()
+        n_train = (acc.gather_for_metrics(batch["attention_mask"].sum()).sum().reshape(1) if mode == "train"
+                   else sums.new_zeros(1))
+        # every logged number in ONE copy to the host
+        (ent_sum, n_tok, lc, nc, lr, nr, n_c, n_r, rew_c, rew_r, lp_c, lp_r, bits, kl, n_train) = torch.cat(
+            [acc.gather_for_metrics(sums.unsqueeze(0)).nansum(dim=0).double(), ops.device_error_bits(sums.device).double(),
+             parts["kl"].reshape(1).double(), n_train.double()]).tolist()
         ops.raise_for_error_bits(bits, sums.device)  # (a token id outside the vocabulary raises here)
+        log["kl"].append(kl)
         log["entropy"].append(ent_sum / n_tok if n_tok > 0 else 0.0)
         if mode == "train":
-            self._total_train_tokens += acc.gather_for_metrics(batch["attention_mask"].sum()).sum().item()
+            self._total_train_tokens += int(n_train)
         log["num_tokens"] = [self._total_train_tokens]
         if nc > 0:
             log["logits/chosen"].append(lc / nc)
