@@ -70,11 +70,15 @@ class RLOOLossMixin:
             log["aux_loss"].append(self.accelerator.gather_for_metrics(aux_loss).mean().item())
         m = completion_mask.to(torch.float32)
         ent = self.accelerator.reduce(torch.stack([(entropies.detach() * m).sum(), m.sum()]), reduction="sum")
-        ent_ratio, bits = torch.cat([(ent[0] / ent[1].clamp(min=1.0)).reshape(1), ops.device_error_bits(ent.device)]).tolist()
+        single = self.accelerator.num_processes == 1
+        # (one copy to the host: the entropy, the error word and, on one process, the loss kernel's metrics)
+        ent_ratio, bits, *values = torch.cat(
+            [(ent[0] / ent[1].clamp(min=1.0)).reshape(1), ops.device_error_bits(ent.device).to(torch.float32)]
+            + ([metrics.detach()[: len(RLOO_METRIC_NAMES)].to(torch.float32)] if single else [])).tolist()
         ops.raise_for_error_bits(bits, ent.device)  # (a token id outside the vocabulary raises here)
         log["entropy"].append(ent_ratio)
-        if self.accelerator.num_processes == 1:
-            for name, value in zip(RLOO_METRIC_NAMES, metrics.detach()[: len(RLOO_METRIC_NAMES)].tolist()):
+        if single:
+            for name, value in zip(RLOO_METRIC_NAMES, values):
                 log[name].append(value)
         else:  # per-sequence flags are gathered as in the reference (:1711-1721)
             from .utils import nanmax, nanmin
