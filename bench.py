@@ -801,6 +801,10 @@ def _brief(r):
         out["mask_aware_ms_per_step"] = r["mask_aware"]["ms_per_step"]
     if "kernels" in r:
         out["kernels"] = {k: v for k, v in r["kernels"].items() if isinstance(v, dict) and ("frac" in v or "avg_ms" in v)}
+        if "sft_chunked_nll_step" in r["kernels"]:  # the SFT loss on the head workload's operands
+            out["sft_chunked_nll_step"] = r["kernels"]["sft_chunked_nll_step"]
+    if r.get("kto"):  # the KTO loss on the DPO workload's logits
+        out["kto"] = r["kto"]
     if r["config"]["workload"] == "logp_c1":  # small enough for the host to run whole: its own baseline and parity
         out["cpu_baseline"] = r["cpu_baseline"]
         out["two_calls_ms_per_step"] = r["two_calls_ms_per_step"]
