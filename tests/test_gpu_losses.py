@@ -89,7 +89,7 @@ def test_golden_grpo_compute_loss_through_trainer_methods(amd, skip_masked, sing
             torch.testing.assert_close(captured["lp"].detach().cpu(), want_lp * keep, atol=tol, rtol=0)
             torch.testing.assert_close(captured["ent"].detach().cpu(), want_ent * keep, atol=tol, rtol=0)
         want_loss = float(g[c + "out_loss"])
-        assert abs(float(loss) - want_loss) <= (2e-2 if low else 1e-5) * max(1.0, abs(want_loss)), case["name"]
+        assert abs(float(loss.detach()) - want_loss) <= (2e-2 if low else 1e-5) * max(1.0, abs(want_loss)), case["name"]
         rel = _rel_l2(leaf.grad.float(), _t(g[c + "out_dlogits"]))
         assert rel < (2e-2 if low else 1e-4), (case["name"], rel)
         got_metrics = {k: v[-1] for k, v in tr._metrics["train"].items()}

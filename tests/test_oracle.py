@@ -340,11 +340,11 @@ def test_golden_dpo_compute_loss():
             assert abs(metrics[name] - want) <= tol, (case["name"], name, metrics[name], want)
         if case.get("ref_equal") and dtype == torch.float32:
             # closed form: policy == reference -> ln 2 (tests/invariant/references/dpo.json step 1)
-            assert abs(float(loss) - 0.6931471824645996) < 1e-6
+            assert abs(float(loss.detach()) - 0.6931471824645996) < 1e-6
         if case["name"] == "sigmoid_f32":  # the sequence-level pieces agree with the full restatement
             seq, _ = oracle.dpo_sequence_logps(logits.detach(), _t(g[c + "input_ids"]), _t(g[c + "completion_mask"]))
             l2, _ = oracle.dpo_sigmoid_loss(seq, refc, refr, case["beta"])
-            assert abs(float(l2) - float(loss)) < 1e-7
+            assert abs(float(l2.detach()) - float(loss.detach())) < 1e-7
 
 
 def test_golden_kto_compute_loss():
