@@ -378,7 +378,7 @@ def test_golden_kto_compute_loss():
     logits = _t(g["c0_logits"])
     seq = oracle.kto_sequence_logps(logits, _t(g["c0_input_ids"]), _t(g["c0_completion_mask"]))
     loss, _ = oracle.kto_compute_loss(logits, _t(g["c0_input_ids"]), _t(g["c0_completion_mask"]), [1, 0, 1, 1, 0, 0], seq)
-    assert abs(float(loss) - 0.5) < 1e-7
+    assert abs(float(loss.detach()) - 0.5) < 1e-7
 
 
 def test_golden_rloo_compute_loss():
@@ -490,7 +490,7 @@ def test_golden_sft_chunked_nll():
     hs.requires_grad_(True)
     loss, correct, ent, nv = oracle.chunked_cross_entropy_loss(hs, w, 4, labels=torch.full((2, 7), -100))
     loss.backward()
-    assert float(loss) == 0.0 and int(nv) == 0 and torch.count_nonzero(hs.grad) == 0
+    assert float(loss.detach()) == 0.0 and int(nv) == 0 and torch.count_nonzero(hs.grad) == 0
 
 
 def test_fused_linear_contracts_reduce_to_closed_forms():
@@ -504,7 +504,7 @@ def test_fused_linear_contracts_reduce_to_closed_forms():
     target = torch.randint(0, V, (2 * P, T), generator=g)
     target[:, :2] = -100
     loss, m = oracle.fused_linear_dpo_loss(weight, hidden, target, hidden, weight, beta=0.1)
-    assert abs(float(loss) - math.log(2.0)) < 1e-6 and len(m) == 7
+    assert abs(float(loss.detach()) - math.log(2.0)) < 1e-6 and len(m) == 7
     assert torch.equal(m[5], torch.zeros(P)) and torch.equal(m[6], torch.zeros(P)) and float(m[4]) == 0.0
     logits = hidden.reshape(-1, H) @ weight.t()
     assert abs(float(m[2]) - float(logits.view(2 * P, T, V)[:P].mean())) < 1e-6
@@ -516,6 +516,6 @@ def test_fused_linear_contracts_reduce_to_closed_forms():
     loss, m = oracle.fused_linear_grpo_loss(hidden, weight, ids, mask, adv, 1.0, None, logps, None, beta=0.04,
                                             loss_type="bnpo")
     assert len(m) == 2 and abs(m[0]) < 1e-7 and m[1] == 0.0
-    assert abs(float(loss) + float(adv.mean())) < 1e-6  # -(sum A * 1) / tokens
+    assert abs(float(loss.detach()) + float(adv.mean())) < 1e-6  # -(sum A * 1) / tokens
     loss, m = oracle.fused_linear_grpo_loss(hidden, weight, ids, mask, adv, 1.0, beta=0.0, loss_type="bnpo")
     assert len(m) == 1
