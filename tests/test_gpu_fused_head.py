@@ -488,12 +488,12 @@ def test_golden_sft_chunked_nll(amd):
         if has_bias:
             assert _rel_l2(db.grad.float(), ob.grad) < 1e-2
         assert int(nv) == int(onv) == int(g[c + "out_n_valid"])
-        assert abs(float(loss) - float(oloss)) <= 1e-3 * abs(float(oloss))
-        assert abs(float(correct) - float(ocorrect)) <= 1.0  # a near-tie between the two largest logits may flip
-        assert abs(float(ent) - float(oent)) <= 2e-3 * int(nv)
+        assert abs(float(loss.detach()) - float(oloss.detach())) <= 1e-3 * abs(float(oloss.detach()))
+        assert abs(float(correct.detach()) - float(ocorrect.detach())) <= 1.0  # a near-tie between the two largest logits may flip
+        assert abs(float(ent.detach()) - float(oent.detach())) <= 2e-3 * int(nv)
         assert _rel_l2(dhs.grad.float(), ohs.grad) < 1e-2 and _rel_l2(dw.grad.float(), ow.grad) < 1e-2
         if case["dtype"] == "float32":  # and loosely against the reference's own fp32 numbers (bf16 operand rounding)
-            assert abs(float(loss) - float(g[c + "out_loss"])) <= 2e-2 * abs(float(g[c + "out_loss"]))
+            assert abs(float(loss.detach()) - float(g[c + "out_loss"])) <= 2e-2 * abs(float(g[c + "out_loss"]))
             # fp32 operands: the reference's numbers at fp32 accuracy
             fhs, fw = _t(g[c + "hidden"]).to(DEV).requires_grad_(True), _t(g[c + "weight"]).to(DEV).requires_grad_(True)
             fb = _t(g[c + "bias"]).to(DEV).requires_grad_(True) if has_bias else None
@@ -501,9 +501,9 @@ def test_golden_sft_chunked_nll(amd):
             loss.backward()
             if has_bias:
                 torch.testing.assert_close(fb.grad.cpu(), _t(g[c + "out_dbias"]), atol=1e-6, rtol=1e-4)
-            assert abs(float(loss) - float(g[c + "out_loss"])) <= 1e-5 * max(1.0, abs(float(g[c + "out_loss"])))
-            assert float(correct) == float(g[c + "out_correct"])
-            assert abs(float(ent) - float(g[c + "out_entropy_sum"])) <= 1e-4 * abs(float(g[c + "out_entropy_sum"]))
+            assert abs(float(loss.detach()) - float(g[c + "out_loss"])) <= 1e-5 * max(1.0, abs(float(g[c + "out_loss"])))
+            assert float(correct.detach()) == float(g[c + "out_correct"])
+            assert abs(float(ent.detach()) - float(g[c + "out_entropy_sum"])) <= 1e-4 * abs(float(g[c + "out_entropy_sum"]))
             torch.testing.assert_close(fhs.grad.cpu(), _t(g[c + "out_dhidden"]), atol=1e-6, rtol=1e-4)
             torch.testing.assert_close(fw.grad.cpu(), _t(g[c + "out_dweight"]), atol=1e-6, rtol=1e-4)
     # all positions masked: zero loss that still backpropagates
@@ -511,7 +511,7 @@ def test_golden_sft_chunked_nll(amd):
     dw = torch.randn(64, 32, device=DEV).bfloat16().requires_grad_(True)
     loss, correct, ent, nv = _chunked_cross_entropy_loss(dhs, dw, 256, labels=torch.full((2, 5), -100, device=DEV))
     loss.backward()
-    assert float(loss) == 0.0 and int(nv) == 0 and torch.count_nonzero(dw.grad) == 0
+    assert float(loss.detach()) == 0.0 and int(nv) == 0 and torch.count_nonzero(dw.grad) == 0
 
 
 def test_target_logit_every_tile_position(amd):

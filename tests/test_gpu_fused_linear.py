@@ -62,7 +62,7 @@ def test_fused_linear_grpo_loss(amd, loss_type, level, beta):
                        advantages=adv.to(DEV), bias=None, old_per_token_logps=old.to(DEV),
                        ref_per_token_logps=ref.to(DEV) if beta else None, vllm_is_ratio=ratio.to(DEV))
     loss.backward()
-    assert abs(float(loss) - float(oloss)) <= 1e-3 * max(1.0, abs(float(oloss)))
+    assert abs(float(loss.detach()) - float(oloss.detach())) <= 1e-3 * max(1.0, abs(float(oloss.detach())))
     assert len(metrics) == len(ometrics) == (2 if beta else 1)
     for got, want in zip(metrics, ometrics):
         if want == want:  # sapo / cispo log no clip ratio in the reference
@@ -96,7 +96,7 @@ def test_fused_linear_dpo_loss(amd, loss_type):
     dw = weight.to(DEV).requires_grad_(True)
     loss, m = op(dw, dh, target.to(DEV), None, ref_hidden.to(DEV), ref_weight.to(DEV), None)
     loss.backward()
-    assert abs(float(loss) - float(oloss)) <= 1e-3 * max(1.0, abs(float(oloss)))
+    assert abs(float(loss.detach()) - float(oloss.detach())) <= 1e-3 * max(1.0, abs(float(oloss.detach())))
     assert len(m) == 7
     for i in (0, 1, 5, 6):
         torch.testing.assert_close(m[i].cpu(), om[i], rtol=1e-3, atol=2e-3)
@@ -125,7 +125,7 @@ def test_fused_linear_losses_with_lm_head_bias(amd):
     dh, dw, db = (x.to(DEV).requires_grad_(True) for x in (hidden, weight, bias))
     loss, m = op(dh, dw, ids.to(DEV), mask.to(DEV), adv.to(DEV), db)
     loss.backward()
-    assert abs(float(loss) - float(oloss)) <= 1e-3 * max(1.0, abs(float(oloss)))
+    assert abs(float(loss.detach()) - float(oloss.detach())) <= 1e-3 * max(1.0, abs(float(oloss.detach())))
     assert db.grad.dtype == torch.bfloat16 and db.grad.shape == (V,)
     for got, want in ((dh, oh), (dw, ow), (db, ob)):
         assert _rel_l2(got.grad.float(), want.grad) < 1e-2
@@ -141,7 +141,7 @@ def test_fused_linear_losses_with_lm_head_bias(amd):
     loss, m = amd.FusedLinearDPOLoss(beta=0.1)(dw, dh, target.to(DEV), db, ref_hidden.to(DEV), ref_weight.to(DEV),
                                                 ref_bias.to(DEV))
     loss.backward()
-    assert abs(float(loss) - float(oloss)) <= 1e-3 * max(1.0, abs(float(oloss)))
+    assert abs(float(loss.detach()) - float(oloss.detach())) <= 1e-3 * max(1.0, abs(float(oloss.detach())))
     for i in (0, 1, 5, 6):
         torch.testing.assert_close(m[i].cpu(), om[i], rtol=1e-3, atol=2e-3)
     for i in (2, 3):
@@ -169,7 +169,7 @@ def test_fused_linear_kto_loss(amd, kl):
                     ref_input=ref_hidden.to(DEV), ref_weight=ref_weight.to(DEV), ref_bias=bias.to(DEV),
                     kl=None if kl is None else torch.tensor([kl], device=DEV))
     loss.backward()
-    assert abs(float(loss) - float(oloss)) <= 1e-3 * max(1.0, abs(float(oloss)))
+    assert abs(float(loss.detach()) - float(oloss.detach())) <= 1e-3 * max(1.0, abs(float(oloss.detach())))
     assert len(sums) == 6
     for got, want in zip(sums, osums):
         assert abs(float(got) - float(want)) <= 2e-3 * max(1.0, abs(float(want))), (float(got), float(want))

@@ -666,7 +666,7 @@ def test_golden_vectors_go_through_the_single_pass_kernel(amd, monkeypatch, keep
         name = (case["name"], str(dtype))
         rtol = 2e-2 if true_low else 2e-5
         want_loss = float(g[c + "out_loss"])
-        assert abs(float(loss) - want_loss) <= rtol * max(1.0, abs(want_loss)), (name, float(loss), want_loss)
+        assert abs(float(loss.detach()) - want_loss) <= rtol * max(1.0, abs(want_loss)), (name, float(loss.detach()), want_loss)
         got_metrics = {k: v[-1] for k, v in tr._metrics["train"].items()}
         assert set(case["metrics"]) <= set(got_metrics), (name, set(case["metrics"]) - set(got_metrics))
         for key, want in case["metrics"].items():
@@ -731,7 +731,7 @@ def test_golden_vectors_functional_form_logps_and_entropies(amd):
         torch.testing.assert_close(lp.cpu(), torch.from_numpy(g[c + "out_logps"]), atol=1e-5, rtol=0)
         torch.testing.assert_close(ent.cpu(), torch.from_numpy(g[c + "out_entropies"]), atol=1e-5, rtol=0)
         want_loss = float(g[c + "out_loss"])
-        assert abs(float(loss) - want_loss) <= 2e-5 * max(1.0, abs(want_loss)), case["name"]
+        assert abs(float(loss.detach()) - want_loss) <= 2e-5 * max(1.0, abs(want_loss)), case["name"]
 
 
 # ------------------------------------------------------------------ the benchmark shapes through the single pass
@@ -798,7 +798,7 @@ def _full_size_check(amd, monkeypatch, logits, g, K, temperature, lengths_lo, ad
     okw = {k: (v.cpu() if torch.is_tensor(v) else v) for k, v in kw.items()}
     o_lp = base.cpu().clone().requires_grad_(True)
     o_loss, o_metrics = oracle.grpo_loss(o_lp, adv.cpu(), mask.cpu(), entropies=base_ent.cpu(), **okw)
-    assert abs(float(loss) - float(o_loss)) <= 2e-6 + 1e-4 * abs(float(o_loss)), (float(loss), float(o_loss))
+    assert abs(float(loss.detach()) - float(o_loss.detach())) <= 2e-6 + 1e-4 * abs(float(o_loss.detach())), (float(loss.detach()), float(o_loss.detach()))
     md = amd.trainer.metrics_to_dict(metrics, beta, loss_type=kw["loss_type"])
     for name, want in o_metrics.items():
         if name in md:

@@ -138,7 +138,7 @@ def test_grpo_loss_against_oracle_random(amd):
             dkw["entropies"] = dent
             loss, metrics = amd.grpo_loss(dlp, adv.to(DEV), mask.to(DEV), **dkw)
             loss.backward()
-            assert abs(float(loss) - float(oloss)) <= 1e-5 * max(1.0, abs(float(oloss))), (lt, delta)
+            assert abs(float(loss.detach()) - float(oloss.detach())) <= 1e-5 * max(1.0, abs(float(oloss.detach()))), (lt, delta)
             assert _rel_l2(dlp.grad, olp.grad) < 1e-5, (lt, delta)
             assert _rel_l2(dent.grad, oent.grad) < 1e-5, (lt, delta)
             md = amd.trainer.metrics_to_dict(metrics, 0.04)
