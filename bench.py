@@ -18,7 +18,8 @@ workload on this host's cores.  Without `--workload` the line also carries `seco
 headline workload and the other benchmark configurations (fused head, long context, DPO, and the fp32 forward-only
 configuration small enough for the host to run whole), each with its step time,
 its dominant kernel's roofline figures and -- where the one-pass kernel runs -- the relative L2 distance between its
-gradient and the two-pass gradient.
+gradient and the two-pass gradient.  The fused-head record also times the SFT chunked cross-entropy on its operands,
+the DPO record the KTO loss on its logits.
 """
 from __future__ import annotations
 
