@@ -200,7 +200,9 @@ int trlk_grpo_loss(const float* d_logp, const float* d_old_logp, const float* d_
  * share that GPU's array: calls that overlap on one GPU (different streams or threads) race and must be serialised by
  * the caller.  Same arguments, outputs and bit-exact results as trlk_grpo_loss.
  * trlk_init looks up the array's address on the current device (once per device); a caller that captures graphs
- * calls it beforehand, with each device current -- otherwise the first trlk_grpo_loss_static call on a device does it. */
+ * calls it beforehand, with each device current -- otherwise the first trlk_grpo_loss_static call on a device does it.
+ * trlk_init also allows the builds of trlk_grpo_fused_fwd_bwd that keep part of a row in LDS (rows above 163840
+ * 16-bit or 81920 fp32 logits) their LDS on the current device, which otherwise happens at the first such launch. */
 int trlk_init(void);
 int64_t trlk_grpo_loss_static_max_seq(void);
 int trlk_grpo_loss_static(const float* d_logp, const float* d_old_logp, const float* d_ref_logp, const float* d_entropy,

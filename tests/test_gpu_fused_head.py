@@ -461,6 +461,114 @@ def test_real_head_shape_paths_agree(amd, monkeypatch):
     assert float(a[0].max()) <= 0.0
 
 
+def test_full_size_config5(amd, monkeypatch):
+    """Benchmark configuration 5 at its size: hidden bf16 [16 x 2048, 3584], W bf16 [151936, 3584], a prefix mask per
+    sequence, `_ChunkedLogProbFunction` -> GRPO loss (G = 8, beta = 0.04) -> backward.  Run three ways -- forward
+    products kept and zero-gradient tokens dropped (what the operator does by default), logits recomputed with every
+    token in the products (the reference's scheme, trl/trainer/utils.py:1291-1424), and `FusedLinearGRPOLoss` on the
+    same inputs.  Size-independent properties on the whole result, and a 64-token subsample of log-prob / entropy /
+    dHidden plus a 64-row slab of dW against the naive fp32 head evaluated on the host (the comparison the reference's
+    own test makes at N, H, V = 64, 32, 128, tests/test_utils.py:1161-1232)."""
+    B, T, H, V, G, temperature = 16, 2048, 3584, 151936, 8, 1.0
+    N = B * T
+    g = torch.Generator(device=DEV).manual_seed(5)
+    hidden = torch.randn((N, H), generator=g, device=DEV).bfloat16()
+    weight = (0.02 * torch.randn((V, H), generator=g, device=DEV)).bfloat16()
+    targets = torch.randint(0, V, (N,), generator=g, device=DEV)
+    lengths = torch.randint(64, T + 1, (B,), generator=g, device=DEV)
+    mask = (torch.arange(T, device=DEV)[None] < lengths[:, None]).long()
+    active = mask.bool().reshape(-1)
+    adv = amd.group_advantages(torch.randn((B,), generator=g, device=DEV), G)
+    with torch.no_grad():
+        base = amd._ChunkedLogProbFunction.apply(hidden, weight, targets, temperature, 32768)[0].view(B, T)
+    old = base + 0.05 * torch.randn(base.shape, generator=g, device=DEV)
+    ref = base + 0.1 * torch.randn(base.shape, generator=g, device=DEV)
+    loss_kw = dict(old_per_token_logps=old, ref_per_token_logps=ref, loss_type="dapo", epsilon_low=0.2,
+                   epsilon_high=0.2, beta=0.04, max_completion_length=T, num_items_in_batch=mask.sum().float())
+    out = {}
+    for mode, gib, drop in (("stash", "24", "1"), ("recompute", "0", "0")):
+        monkeypatch.setenv("TRL_AMD_HEAD_STASH_GIB", gib)
+        monkeypatch.setenv("TRL_AMD_HEAD_DROP_ZERO_GRAD", drop)
+        hh, ww = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+        lp, ent = amd._ChunkedLogProbFunction.apply(hh, ww, targets, temperature, 32768)
+        loss, _ = amd.grpo_loss(lp.view(B, T), adv, mask, entropies=ent.view(B, T), **loss_kw)
+        loss.backward()
+        out[mode] = (lp.detach(), ent.detach(), hh.grad, ww.grad, loss.detach())
+        del hh, ww, lp, ent, loss
+    monkeypatch.setenv("TRL_AMD_HEAD_STASH_GIB", "24")
+    monkeypatch.setenv("TRL_AMD_HEAD_DROP_ZERO_GRAD", "1")
+    fl = amd.FusedLinearGRPOLoss(beta=0.04, epsilon_low=0.2, epsilon_high=0.2, temperature=temperature,
+                                 use_ref_model=True, loss_type="dapo", max_completion_length=T, chunk_size=32768)
+    hh, ww = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+    fl_loss, _ = fl(hh.view(B, T, H), ww, targets.view(B, T), mask, adv, None, old, ref)
+    fl_loss.backward()
+    a, b = out["stash"], out["recompute"]
+    # the forward does not depend on what it keeps for the backward
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    assert bool(torch.equal(a[0].view(B, T), base))
+    # the three losses
+    assert float(a[4]) == float(b[4])
+    assert abs(float(fl_loss.detach()) - float(a[4])) <= 1e-6 * max(1.0, abs(float(a[4])))
+    # gradients: the two schemes agree; tokens outside the mask get exactly nothing
+    assert _rel_l2(a[2].float(), b[2].float()) < 2e-3 and _rel_l2(a[3].float(), b[3].float()) < 2e-3
+    assert _rel_l2(hh.grad.float(), a[2].float()) < 2e-3 and _rel_l2(ww.grad.float(), a[3].float()) < 2e-3
+    for dh in (a[2], b[2], hh.grad):
+        assert torch.count_nonzero(dh[~active]) == 0 and torch.count_nonzero(dh[active]) > 0
+    # softmax gradients are orthogonal to a constant shift of the logits: sum_v dW[v, :] = 0
+    for dw in (a[3], b[3]):
+        assert float(dw.float().sum(0).abs().max()) < 2e-2 * float(dw.float().abs().sum(0).max())
+    assert float(a[1].min()) >= 0.0 and float(a[1].max()) <= float(np.log(V)) + 1e-3 and float(a[0].max()) <= 0.0
+
+    # ---- against the host: the upstream gradient of every token from the oracle's loss on the device's log-probs
+    lp_host = a[0].view(B, T).cpu().clone().requires_grad_(True)
+    host_kw = {k: (v.cpu() if torch.is_tensor(v) else v) for k, v in loss_kw.items()}
+    oloss, _ = oracle.grpo_loss(lp_host, adv.cpu(), mask.cpu(), entropies=a[1].view(B, T).cpu(), **host_kw)
+    oloss.backward()
+    assert abs(float(oloss) - float(a[4])) <= 1e-5 * max(1.0, abs(float(oloss)))
+    g_tok = lp_host.grad.reshape(-1)
+    # 64 tokens: first and last of a sequence, around the end of a mask, and a random draw over the active ones
+    first_len = int(lengths[0])
+    picks = [0, 1, first_len - 1, first_len, N - T, N - 1]
+    act_idx = torch.nonzero(active.cpu()).reshape(-1)
+    sel = torch.randperm(act_idx.numel(), generator=torch.Generator().manual_seed(6))[: 64 - len(picks)]
+    sub = torch.tensor(picks + act_idx[sel].tolist())
+    host_w = weight.cpu()
+    sub_h = hidden[sub.to(DEV)].cpu().float().requires_grad_(True)
+    ow = host_w.float()
+    olp, oent = oracle.chunked_logprob_naive(sub_h, ow, targets.cpu()[sub], temperature)
+    (olp * g_tok[sub]).sum().backward()
+    torch.testing.assert_close(a[0].cpu()[sub], olp.detach(), atol=2e-3, rtol=0)
+    torch.testing.assert_close(a[1].cpu()[sub], oent.detach(), atol=2e-3, rtol=0)
+    for dh in (a[2], b[2], hh.grad):
+        got = dh[sub.to(DEV)].cpu().float()
+        assert _rel_l2(got, sub_h.grad) < 1e-2
+        assert _rel_l2(got, sub_h.grad.bfloat16().float()) < 3e-3
+    # a 64-row slab of dW needs every active token: dW[v, :] = sum_n dz[n, v] hidden[n, :] with
+    # dz[n, v] = g[n] (1[v == target_n] - exp(z[n, v] - lse_n)) / T.  The log-sum-exp of every token comes from plain
+    # torch on the device (fp32 matrix product + logsumexp in blocks of tokens, none of this library's kernels) and is
+    # itself checked against the host's naive head on the 64 tokens above; the slab arithmetic runs on the host.
+    lse = torch.empty(N, device=DEV)
+    w32 = weight.float()
+    for lo in range(0, N, 1024):
+        lse[lo:lo + 1024] = torch.logsumexp((hidden[lo:lo + 1024].float() @ w32.t()) / temperature, dim=-1)
+    del w32
+    with torch.no_grad():
+        olse = torch.logsumexp((sub_h.detach() @ ow.t()) / temperature, dim=-1)
+    torch.testing.assert_close(lse.cpu()[sub], olse, atol=1e-4, rtol=0)
+    for v0 in (0, 75008, V - 64):
+        rows = act_idx
+        hid_a = hidden.cpu()[rows].double()
+        z = (hid_a @ host_w[v0:v0 + 64].double().t()) / temperature
+        p = torch.exp(z - lse.cpu()[rows].double()[:, None])
+        onehot = (targets.cpu()[rows][:, None] == torch.arange(v0, v0 + 64)[None]).double()
+        dz = g_tok[rows].double()[:, None] * (onehot - p) / temperature
+        want = dz.t() @ hid_a
+        for dw in (a[3], b[3], ww.grad):
+            got = dw[v0:v0 + 64].cpu().float()
+            assert _rel_l2(got, want) < 1e-2
+            assert _rel_l2(got, want.float().bfloat16().float()) < 3e-3
+
+
 def test_golden_sft_chunked_nll(amd):
     """The reference's `_chunked_cross_entropy_loss` wrote these; fp32 cases are run in bf16 on the device
     (the matrix-core kernels take bf16/fp16) and compared with the oracle on the bf16-rounded operands."""

@@ -86,6 +86,54 @@ def test_graph_replays_equal_eager(step):
         assert float(got[-1].float().abs().sum()) > 0 or float(buf["mask"].sum()) == 0
 
 
+def test_single_pass_wide_row_first_launch_is_inside_the_capture():
+    """Rows of 172032 bf16 logits take a build of the single-pass kernel that keeps part of the row in LDS and needs
+    more dynamic LDS than a kernel gets by default.  `trlk_init` allows it beforehand, so the first launch of that
+    build may sit inside a capture: no warm-up launch here."""
+    from trl_amd import _lib, ops
+
+    b, t, v = 2, 5, 172032
+    assert v * 2 > 163840 * 2 and v <= ops.grpo_fused_max_vocab(torch.bfloat16)
+    assert _lib.lib.trlk_init() == 0
+    logits = torch.zeros((b, t, v), dtype=torch.bfloat16, device=DEV)
+    ids = torch.zeros((b, t), dtype=torch.int64, device=DEV)
+    mask = torch.ones((b, t), device=DEV)
+    adv = torch.zeros((b,), device=DEV)
+    row_scale = torch.full((b,), 1.0 / (b * t), device=DEV)
+
+    def new_inputs(seed):
+        g = torch.Generator(device=DEV).manual_seed(seed)
+        logits.copy_((2.0 * torch.randn((b, t, v), generator=g, device=DEV)).bfloat16())
+        ids.copy_(torch.randint(0, v, (b, t), generator=g, device=DEV))
+        adv.copy_(torch.randn((b,), generator=g, device=DEV))
+        mask.copy_((torch.rand((b, t), generator=g, device=DEV) < 0.8).float())
+
+    def step():
+        return ops.grpo_fused_fwd_bwd(logits, ids, 1.0, 0, t, mask, adv, row_scale, None, None, None, None,
+                                      _lib.TERM_CLIP, 0.2, 0.28, math.nan, 0.0, False, 1.0, 1.05)
+
+    new_inputs(300)
+    ops.check_device_errors()
+    ops._error_flag(torch.device(DEV))  # (the word the kernels report bad indices in exists before the capture)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    for rep in range(3):
+        new_inputs(301 + rep)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [x.clone() for x in captured]
+        scratch = torch.randn((1 << 20,), device=DEV).sum()
+        want = step()
+        torch.cuda.synchronize()
+        assert math.isfinite(float(scratch))
+        for i, (g_, w_) in enumerate(zip(got, want)):
+            assert torch.equal(g_.nan_to_num(nan=-7.0), w_.nan_to_num(nan=-7.0)), (rep, i)
+        assert float(got[-1].float().abs().sum()) > 0
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 def test_fused_head_graph_replays_equal_eager(dtype):
     """Forward with its products kept, then both gradient products from them: every buffer between the two (the

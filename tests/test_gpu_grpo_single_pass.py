@@ -937,3 +937,76 @@ def test_trainer_method_takes_fp16_only_with_a_known_scale(amd, monkeypatch, wit
         (tr.accelerator.scaler.scale(loss) if with_scaler else loss).backward()
         grads[single] = leaf.grad
     assert _rel_l2(grads[True], grads[False]) < 2e-3
+
+
+@pytest.mark.parametrize("with_scaler", [False, True])
+@pytest.mark.parametrize("loss_type", ["grpo", "dapo", "dr_grpo"])
+@pytest.mark.parametrize("grad_accum", [2, 3, 8])
+def test_trainer_divisor_is_folded_into_the_forward(amd, monkeypatch, grad_accum, loss_type, with_scaler):
+    """`transformers.Trainer.training_step` divides the loss by `current_gradient_accumulation_steps` before
+    `accelerator.backward` when the trainer has `model_accepts_loss_kwargs = False` and no `compute_loss_func`
+    (the reference sets the former, trl/trainer/grpo_trainer.py:1128-1131, and passes a placeholder for the latter,
+    :944-950; a trainer that only does the former gets the division).  `_compute_loss` must announce that divisor
+    (times the gradient scaler's factor) to the single pass, so that `backward` finds an upstream gradient of exactly
+    1 and leaves the gradient buffer as the forward wrote it; a trainer that switches the division off must find
+    the same."""
+    from conftest import fake_grpo_trainer
+    from types import SimpleNamespace
+
+    from trl_amd import ops
+
+    B, P, K, V = 4, 2, 8, 4096
+    g = torch.Generator(device=DEV).manual_seed(53 + grad_accum)
+    logits = (2.0 * torch.randn((B, P + K, V), generator=g, device=DEV)).bfloat16()
+    case = dict(loss_type=loss_type, beta=0.04, eps_low=0.2, eps_high=0.2, grad_accum=grad_accum)
+    lengths = torch.tensor([8, 3, 0, 5], device=DEV)
+    inputs = dict(prompt_ids=torch.randint(0, V, (B, P), generator=g, device=DEV),
+                  prompt_mask=torch.ones(B, P, dtype=torch.long, device=DEV),
+                  completion_ids=torch.randint(0, V, (B, K), generator=g, device=DEV),
+                  completion_mask=(torch.arange(K, device=DEV)[None] < lengths[:, None]).long(),
+                  advantages=torch.randn(B, generator=g, device=DEV),
+                  num_items_in_batch=torch.tensor(37.0, device=DEV))
+    with torch.no_grad():
+        base, _ = amd.per_token_logps_and_entropies(logits, torch.cat([inputs["prompt_ids"], inputs["completion_ids"]], 1), K, 1.0)
+    inputs["old_per_token_logps"] = base + 0.2 * torch.randn(base.shape, generator=g, device=DEV)
+    inputs["ref_per_token_logps"] = base + 0.1 * torch.randn(base.shape, generator=g, device=DEV)
+    written = []
+    real = ops.grpo_fused_fwd_bwd
+    monkeypatch.setattr(ops, "grpo_fused_fwd_bwd", lambda *a, **k: written.append(real(*a, **k)) or written[-1])
+
+    class Scaler:
+        def is_enabled(self):
+            return True
+
+        def scale(self, x):
+            return x * 4096.0
+
+    def training_step(tr, leaf):
+        """What the parent class does around `compute_loss` (transformers Trainer.training_step, accelerate
+        Accelerator.backward), for a single process."""
+        loss = tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None), inputs)
+        if not tr.model_accepts_loss_kwargs and tr.compute_loss_func is None:
+            loss = loss / tr.current_gradient_accumulation_steps
+        loss = loss / tr.accelerator.gradient_accumulation_steps
+        if tr.accelerator.scaler is not None:
+            loss = tr.accelerator.scaler.scale(loss)
+        return loss
+
+    for divides in (True, False):
+        grads = {}
+        for single in (True, False):
+            tr = fake_grpo_trainer(amd, case, K, skip_masked=True, single_pass=single)
+            tr.accelerator.scaler = Scaler() if with_scaler else None
+            tr.accelerator.gradient_accumulation_steps = 1
+            tr.model_accepts_loss_kwargs = False
+            tr.compute_loss_func = None if divides else "non-None value to disable scaling"
+            leaf = logits.detach().clone().requires_grad_(True)
+            n = len(written)
+            loss = training_step(tr, leaf)
+            assert len(written) == n + (1 if single else 0)
+            before = written[-1][3].clone() if single else None
+            loss.backward()
+            if single:  # bit for bit what the forward wrote: the scale kernel had nothing left to do
+                assert torch.equal(leaf.grad, before), (divides, grad_accum, loss_type)
+            grads[single] = leaf.grad
+        assert _rel_l2(grads[True], grads[False]) < 1e-3

@@ -47,14 +47,51 @@ def test_static_scratch_entry_matches_workspace_entry(loss_type, term, seq_level
         metrics = torch.full((_lib.GRPO_NUM_METRICS,), math.nan, device=DEV)
         dlogp = torch.full((B, T), math.nan, device=DEV)
         dent = torch.full((B, T), math.nan, device=DEV) if coef else None
+        torch.cuda.synchronize()
+        held = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.memory_stats()["allocation.all.allocated"])
         ops.grpo_loss_static_(loss, metrics, dlogp, dent, p["logp"], p["old"], p["ref"] if beta else None, p["ent"],
                               p["adv"], p["mask"], weight, None, p["n_items"], *cfg)
+        torch.cuda.synchronize()
+        # nothing was allocated through torch, not even a block that was freed again before the call returned
+        assert held == (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(),
+                        torch.cuda.memory_stats()["allocation.all.allocated"])
         assert torch.equal(loss, want[0]), (B, float(loss), float(want[0]))
         assert torch.equal(metrics.nan_to_num(nan=-7.0), want[1].nan_to_num(nan=-7.0))
         assert torch.equal(dlogp, want[2])
         if coef:
             assert torch.equal(dent, want[3])
         assert math.isfinite(float(loss))
+
+
+def test_static_scratch_entry_checks_its_operands():
+    """The Python wrapper hands raw pointers to the library: layout, dtype and device of every operand are checked
+    before that."""
+    from trl_amd import _lib, ops
+
+    B, T = 4, 8
+    p = _problem(B, T, 9)
+    out = dict(loss=torch.zeros((), device=DEV), metrics=torch.zeros(_lib.GRPO_NUM_METRICS, device=DEV),
+               dlogp=torch.zeros(B, T, device=DEV))
+    cfg = [_lib.DAPO, 0.2, 0.2, math.nan, 0.0, False, 1.0, float(B * T), 1.0, 0.0, _lib.TERM_CLIP, False, None, 1.0, 1.05]
+
+    def call(loss=None, metrics=None, n_items=None, seq_coef=None, adv=None, term=_lib.TERM_CLIP):
+        c = list(cfg)
+        c[10], c[12] = term, seq_coef
+        ops.grpo_loss_static_(out["loss"] if loss is None else loss, out["metrics"] if metrics is None else metrics,
+                              out["dlogp"], None, p["logp"], p["old"], None, None, p["adv"] if adv is None else adv,
+                              p["mask"], None, None, p["n_items"] if n_items is None else n_items, *c)
+
+    call()  # the well-formed call goes through
+    with pytest.raises(ValueError, match="out_metrics"):
+        call(metrics=torch.zeros(2 * _lib.GRPO_NUM_METRICS, device=DEV)[::2])
+    with pytest.raises(ValueError, match="dapo_normalizer"):
+        call(n_items=p["n_items"].bfloat16())
+    with pytest.raises(ValueError, match="seq_coef"):
+        call(seq_coef=torch.ones(B, 2, device=DEV)[:, 0], term=_lib.TERM_WEIGHTED_LOGP)
+    with pytest.raises(ValueError, match="is on cpu"):
+        call(adv=p["adv"].cpu())
+    with pytest.raises(ValueError, match="advantages"):
+        call(adv=torch.zeros(2, B // 2, device=DEV).t())
 
 
 def test_static_scratch_entry_rejects_what_does_not_fit():

@@ -12,6 +12,7 @@ namespace trlk {
 int fail(int code, const char* fmt, ...);  // records the text, returns `code`
 void clear_error();
 int launch_status(const char* what);  // hipGetLastError() -> 0 or positive hipError_t (text recorded)
+int grpo_fused_reserve_lds();          // grpo_fused.hip: LDS of the single-pass kernel's wide builds, current device
 
 #define TRLK_REQUIRE(cond, code, ...)                    \
     do {                                                 \

@@ -9,6 +9,9 @@
 // with the same device functions as the [B, T]-sized loss kernel, and writes the row's dlogits from the
 // registers.  Rows outside the completion mask are never read: their gradient row is zero-filled and their
 // outputs are 0.
+#include <mutex>
+#include <vector>
+
 #include "common.hpp"
 #include "grpo_token.hpp"
 
@@ -451,28 +454,38 @@ __global__ __launch_bounds__(kFThreads) void grpo_fused_kernel(FusedArgs a) {
     }
 }
 
-// dynamic LDS above 64 KiB has to be allowed per kernel and device once
+// dynamic LDS above 64 KiB has to be allowed per kernel and device once (a process-wide record: the thread that
+// launches need not be the one that called trlk_init)
 template <typename Kern>
 int reserve_overflow_lds(Kern kern, int bytes) {
     struct Done {
         const void* kern;
         int device;
     };
-    static thread_local Done configured[16] = {};
+    static std::mutex guard;
+    static std::vector<Done> configured;
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess) device = 0;
     const void* key = reinterpret_cast<const void*>(kern);
+    std::lock_guard<std::mutex> lock(guard);
     for (const Done& c : configured)
         if (c.kern == key && c.device == device) return TRLK_OK;
     const hipError_t e = hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
     if (e != hipSuccess) return fail(int(e), "grpo_fused: cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(e));
-    for (Done& c : configured)
-        if (c.kern == nullptr) {
-            c.kern = key;
-            c.device = device;
-            break;
-        }
+    configured.push_back(Done{key, device});
     return TRLK_OK;
+}
+
+template <int DT, int NLDS, bool EXTRA, bool R>
+int reserve_one() {
+    return reserve_overflow_lds(grpo_fused_kernel<DT, kWideVec, NLDS, EXTRA, R>, NLDS * kFThreads * 16);
+}
+template <int DT, bool R>
+int reserve_dtype() {
+    if (int rc = reserve_one<DT, 3, false, R>()) return rc;
+    if (int rc = reserve_one<DT, 6, false, R>()) return rc;
+    if (int rc = reserve_one<DT, 9, false, R>()) return rc;
+    return reserve_one<DT, kMaxLdsVec, true, R>();
 }
 
 template <int DT, int NLDS, bool EXTRA, bool R>
@@ -550,6 +563,17 @@ __global__ __launch_bounds__(256) void scale_unless_one_kernel(u32x4* data, int6
 }
 
 }  // namespace
+
+// Every build of the single-pass kernel that keeps part of a row in LDS, allowed its LDS on the current device: what a
+// caller does through trlk_init before it captures a graph, so that no launch inside the capture has to.
+int grpo_fused_reserve_lds() {
+    if (int rc = reserve_dtype<TRLK_BF16, false>()) return rc;
+    if (int rc = reserve_dtype<TRLK_BF16, true>()) return rc;
+    if (int rc = reserve_dtype<TRLK_F16, false>()) return rc;
+    if (int rc = reserve_dtype<TRLK_F16, true>()) return rc;
+    if (int rc = reserve_dtype<TRLK_F32, false>()) return rc;
+    return reserve_dtype<TRLK_F32, true>();
+}
 }  // namespace trlk
 
 using namespace trlk;

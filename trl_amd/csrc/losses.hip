@@ -598,7 +598,8 @@ int static_scratch_for_current_device(float** out) {
 extern "C" int trlk_init(void) {
     clear_error();
     float* p = nullptr;
-    return static_scratch_for_current_device(&p);
+    if (int rc = static_scratch_for_current_device(&p)) return rc;
+    return grpo_fused_reserve_lds();
 }
 
 extern "C" int64_t trlk_grpo_loss_static_max_seq(void) { return kStaticMaxSeq; }

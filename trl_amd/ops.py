@@ -454,15 +454,29 @@ def grpo_loss_static_(
             raise ValueError(f"grpo_loss_static_: {name} must be a contiguous fp32 [{B}, {T}] tensor")
     if advantages.dtype != torch.float32 or not advantages.is_contiguous():
         raise ValueError("grpo_loss_static_: advantages must be contiguous fp32")
-    if advantages.numel() == B:
+    if tuple(advantages.shape) in ((B,), (B, 1)):
         sb, st = 1, 0
     elif tuple(advantages.shape) == (B, T):
         sb, st = T, 1
     else:
         raise ValueError(f"grpo_loss_static_: advantages of shape {tuple(advantages.shape)} do not match [B] or [B, T]")
-    if out_loss.dtype != torch.float32 or out_metrics.dtype != torch.float32 or out_metrics.numel() < _lib.GRPO_NUM_METRICS:
-        raise ValueError("grpo_loss_static_: out_loss / out_metrics must be fp32 ([] and [16])")
+    if (out_loss.dtype != torch.float32 or out_loss.numel() != 1 or out_metrics.dtype != torch.float32
+            or out_metrics.dim() != 1 or out_metrics.numel() < _lib.GRPO_NUM_METRICS or not out_metrics.is_contiguous()):
+        raise ValueError("grpo_loss_static_: out_loss / out_metrics must be contiguous fp32 ([] and [16])")
+    if seq_coef is not None and (seq_coef.dtype != torch.float32 or not seq_coef.is_contiguous()
+                                 or tuple(seq_coef.shape) != (B,)):
+        raise ValueError(f"grpo_loss_static_: seq_coef must be a contiguous fp32 [{B}] tensor")
+    if dapo_normalizer is not None and (dapo_normalizer.dtype != torch.float32 or dapo_normalizer.numel() != 1):
+        raise ValueError("grpo_loss_static_: dapo_normalizer must be a one-element fp32 tensor")
     dev = logp.device
+    if dev.type != "cuda":
+        raise ValueError("grpo_loss_static_: the operands must live on the GPU")
+    for name, t in (("old_logp", old_logp), ("ref_logp", ref_logp), ("entropy", entropy), ("advantages", advantages),
+                    ("mask", mask), ("token_weight", token_weight), ("entropy_mask", entropy_mask),
+                    ("dapo_normalizer", dapo_normalizer), ("seq_coef", seq_coef), ("out_loss", out_loss),
+                    ("out_metrics", out_metrics), ("out_dlogp", out_dlogp), ("out_dentropy", out_dentropy)):
+        if t is not None and t.device != dev:
+            raise ValueError(f"grpo_loss_static_: {name} is on {t.device}, logp on {dev}")
     with torch.cuda.device(dev):
         check(
             lib.trlk_grpo_loss_static(

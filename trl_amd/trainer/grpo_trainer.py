@@ -577,14 +577,13 @@ class GRPOLossMixin:
             logits = outputs.logits
             if logits.shape[-1] > 1 and logits.stride(-1) != 1:
                 logits = logits.contiguous()
-            # the factor a gradient scaler (fp16 mixed precision) will put on the loss: a 0-d device tensor, no sync
-            scaler = getattr(self.accelerator, "scaler", None)
-            upstream = None
-            if scaler is not None and getattr(scaler, "is_enabled", lambda: True)():
-                upstream = scaler.scale(torch.ones((), dtype=torch.float32, device=logits.device))
+            # the factor the training step will put on the loss before `backward`: a 0-d device tensor, no sync
+            upstream = self._announced_upstream_scale(logits.device, mode)
             # fp16 gradients of a 1e5-entry softmax row sit near the bottom of the fp16 range: the one pass rounds
             # them once, so it is only taken when the scale is known at that point (or on request)
-            fp16_ok = upstream is not None or getattr(self, "trl_amd_single_pass_fp16", False)
+            scaler = getattr(self.accelerator, "scaler", None)
+            scaled = scaler is not None and getattr(scaler, "is_enabled", lambda: True)()
+            fp16_ok = scaled or getattr(self, "trl_amd_single_pass_fp16", False)
             pays = want_single is True or logits.shape[-1] * logits.element_size() >= _SINGLE_PASS_MIN_ROW_BYTES
             if (pays and grpo_single_pass_supported(logits, self.loss_type)
                     and (logits.dtype != torch.float16 or fp16_ok)):
@@ -645,6 +644,45 @@ class GRPOLossMixin:
             importance_sampling_ratio=inputs.get("importance_sampling_ratio"),
         )
         return self._finish_loss(loss, metrics, entropies, mask, entropy_mask, aux_loss, aux_enabled, grad_accum, mode, bonus)
+
+    def _announced_upstream_scale(self, device, mode):
+        """The upstream gradient `loss.backward()` will deliver to `_compute_loss`'s result, as far as the trainer's
+        own attributes tell it, or None when that is 1.  Three factors sit between the returned loss and `backward`
+        (transformers `Trainer.training_step`, accelerate `Accelerator.backward`):
+        - `Trainer.training_step` divides by `current_gradient_accumulation_steps` unless `compute_loss_func` is set
+          or the model takes loss kwargs.  The reference's `GRPOTrainer` sets `model_accepts_loss_kwargs = False`
+          (trl/trainer/grpo_trainer.py:1128-1131) and hands the parent a non-None `compute_loss_func`
+          (:944-950) to switch that division off; a trainer that only does the former gets the division;
+        - `Accelerator.backward` divides by the accelerator's own `gradient_accumulation_steps` (1 under `Trainer`)
+          except with DeepSpeed;
+        - a gradient scaler (fp16 mixed precision) multiplies by its scale.
+        The factors are applied to a 0-d tensor in the order autograd's backward meets them, with the operations it
+        uses, so that `g_loss / factor` comes out as exactly 1 and `backward` has nothing to rescale.  A trainer whose
+        step does something else still gets the right gradient: `backward` applies whatever part of the upstream
+        gradient was not announced."""
+        factor = None
+        scaler = getattr(self.accelerator, "scaler", None)
+        if scaler is not None and getattr(scaler, "is_enabled", lambda: True)():
+            factor = scaler.scale(torch.ones((), dtype=torch.float32, device=device))
+        if mode != "train":
+            return factor
+        divisors = []
+        acc_steps = getattr(self.accelerator, "gradient_accumulation_steps", 1)
+        if isinstance(acc_steps, (int, float)) and acc_steps != 1 and "DEEPSPEED" not in str(
+                getattr(self.accelerator, "distributed_type", "")):
+            divisors.append(acc_steps)
+        # (attributes of transformers.Trainer; an object without them is no Trainer and divides nothing)
+        if (hasattr(self, "model_accepts_loss_kwargs") and not self.model_accepts_loss_kwargs
+                and getattr(self, "compute_loss_func", None) is None
+                and getattr(self, "trl_amd_trainer_divides_loss", True)):
+            ga = self.current_gradient_accumulation_steps
+            if isinstance(ga, (int, float)) and ga != 1:
+                divisors.append(ga)
+        for d in divisors:
+            if factor is None:
+                factor = torch.ones((), dtype=torch.float32, device=device)
+            factor = factor / d
+        return factor
 
     def _finish_loss(self, loss, metrics, entropies, mask, entropy_mask, aux_loss, aux_enabled, grad_accum, mode, bonus):
         """Auxiliary loss, the adaptive entropy controller and the logged metrics (grpo_trainer.py:3152-3258)."""

@@ -161,8 +161,9 @@ def _fp32_head_backward(hidden, weight, targets, temperature, cap, logit_scale, 
     W^T and hidden^T -- everything on this library's matrix-core kernel at fp32 accuracy, as the reference's fp32
     `grad_logits @ w_chunk.float()` / `grad_logits.t() @ hidden.float()` (trl/trainer/utils.py:1421-1422)."""
     n, v = hidden.shape[0], weight.shape[0]
-    d_hidden = torch.empty_like(hidden)
-    d_weight = torch.zeros_like(weight)
+    # (dense rows whatever the operands' strides: the products write through `out=` with a unit inner stride)
+    d_hidden = torch.empty(hidden.shape, dtype=hidden.dtype, device=hidden.device)
+    d_weight = torch.zeros(weight.shape, dtype=weight.dtype, device=weight.device)
     d_bias = torch.zeros(v, dtype=torch.float32, device=hidden.device) if bias is not None else None
     g = grad_logprobs.contiguous().float()
     wp = ops.split_bf16x3(weight, 1)                   # [V, 6 H]: right operand of the logits
