@@ -545,6 +545,62 @@ def bench_logp_c1(args, w):
     }
 
 
+def _trainer_step_legs(args, w, loss_type, shared, timed):
+    """`GRPOLossMixin._compute_loss` as a `transformers.Trainer` runs it with 4 gradient-accumulation steps: the parent
+    class divides the returned loss by 4 before `backward` (a trainer with `model_accepts_loss_kwargs = False` and no
+    `compute_loss_func`).  Three ways: the mix-in as it is (it announces the divisor to the single pass), the same
+    with the announcement switched off (`backward` then rescales the whole gradient), and the two-pass path.  The
+    model is a stand-in that returns the resident logits; one prompt token, T - 1 completion tokens."""
+    from collections import defaultdict
+    from types import SimpleNamespace
+
+    import trl_amd
+
+    logits, ids, mask, adv, old, ref, leaf = (shared[k] for k in ("logits", "ids", "mask", "adv", "old", "ref", "leaf"))
+    B, T = ids.shape
+    K = T - 1
+
+    class Accelerator:
+        num_processes, sync_gradients, scaler, gradient_accumulation_steps = 1, True, None, 1
+        gather = gather_for_metrics = staticmethod(lambda x: x)
+        reduce = staticmethod(lambda x, reduction="sum": x)
+
+    class Trainer(trl_amd.GRPOLossMixin):
+        pass
+
+    inputs = dict(prompt_ids=ids[:, :1], prompt_mask=torch.ones_like(ids[:, :1]), completion_ids=ids[:, 1:],
+                  completion_mask=mask[:, 1:], advantages=adv, old_per_token_logps=old[:, 1:],
+                  num_items_in_batch=mask[:, 1:].sum().float())
+    if ref is not None:
+        inputs["ref_per_token_logps"] = ref[:, 1:]
+    out = {}
+    for name, single, announce in (("single_pass", True, True), ("single_pass_divisor_not_announced", True, False),
+                                   ("two_pass", False, True)):
+        tr = Trainer()
+        tr.accelerator, tr.temperature, tr.model_kwarg_keys = Accelerator(), w["temperature"], set()
+        tr._entropy_bonus_enabled, tr.entropy_coef, tr.use_adaptive_entropy, tr.aux_loss_enabled = False, 0.0, False, False
+        tr.top_entropy_quantile, tr.off_policy_mask_threshold, tr.importance_sampling_level = 1.0, None, "token"
+        tr.beta, tr.loss_type, tr.epsilon_low, tr.epsilon_high = w["beta"], loss_type, w["eps_low"], w["eps_high"]
+        tr.use_vllm = tr.vllm_importance_sampling_correction = False
+        tr.max_completion_length, tr.current_gradient_accumulation_steps = K, 4
+        tr.args = SimpleNamespace(delta=None, use_bias_correction_kl=False)
+        tr._metrics = {"train": defaultdict(list), "eval": defaultdict(list)}
+        tr.model = SimpleNamespace(training=True)
+        tr.model_accepts_loss_kwargs, tr.compute_loss_func = False, None
+        tr.trl_amd_single_pass, tr.trl_amd_trainer_divides_loss = single, announce
+
+        def training_step(tr=tr):
+            leaf.grad = None
+            loss = tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None), inputs)
+            loss = loss / tr.current_gradient_accumulation_steps  # transformers Trainer.training_step
+            loss.backward()
+            return loss, None
+
+        out[name] = timed(training_step)[0]
+    leaf.grad = None
+    return out
+
+
 def _grad_distance(run_a, run_b, leaf):
     """Relative L2 distance between the gradients two step functions leave in `leaf.grad`, accumulated sequence
     by sequence (no logits-sized fp32 temporaries)."""
@@ -642,6 +698,7 @@ def bench_grpo(args, w, loss_type, shared=None, full=True):
             # unannounced it costs a further read + write of the gradient in `backward`
             single["scaled_upstream_ms"] = {"announced": timed(lambda: sp_step(True, 1024.0, True))[0],
                                             "unannounced": timed(lambda: sp_step(True, 1024.0, False))[0]}
+            single["trainer_step_grad_accum_4_ms"] = _trainer_step_legs(args, w, loss_type, shared, timed)
     # headline: the fastest path that produces every stated output (log-prob and entropy of every row, loss, dlogits)
     ms_per_step = min(ms_two_pass, single["all_rows_ms"]) if single else ms_two_pass
     headline_single = single is not None and single["all_rows_ms"] <= ms_two_pass
@@ -713,13 +770,20 @@ def bench_grpo(args, w, loss_type, shared=None, full=True):
                                           None, term_code, w["eps_low"], w["eps_high"], float("nan"), w["beta"], False,
                                           1.0, 1.05, all_rows)
 
+        def fused_dense():  # every row inside the mask: each is read and its gradient written
+            return ops.grpo_fused_fwd_bwd(logits.detach(), ids, w["temperature"], 0, T, torch.ones_like(mask), adv,
+                                          row_scale, old, ref, None, None, term_code, w["eps_low"], w["eps_high"],
+                                          float("nan"), w["beta"], False, 1.0, 1.05, False)
+
         with torch.no_grad():
             sp_skip_ms = time_kernel(lambda: fused(False))
             sp_all_ms = time_kernel(lambda: fused(True)) if full else None
+            sp_dense_ms = time_kernel(fused_dense) if full else None
         sp_all_bytes = 2 * R * row_bytes                              # every row read, every gradient row written
         sp_skip_bytes = active_rows * 2 * row_bytes + (R - active_rows) * row_bytes
         for name, ms_k, nbytes in (("grpo_fused_kernel (K7), masked rows not read", sp_skip_ms, sp_skip_bytes),
-                                   ("grpo_fused_kernel (K7), every row read (C entry only)", sp_all_ms, sp_all_bytes)):
+                                   ("grpo_fused_kernel (K7), every row read (C entry only)", sp_all_ms, sp_all_bytes),
+                                   ("grpo_fused_kernel (K7), every row active (a mask of ones)", sp_dense_ms, sp_all_bytes)):
             if ms_k is not None:
                 kernels[name] = {"avg_launch_ms": ms_k, "algorithmic_bytes": nbytes,
                                  "achieved_GBps": nbytes / (ms_k * 1e-3) / 1e9,
@@ -768,10 +832,13 @@ def bench_grpo(args, w, loss_type, shared=None, full=True):
             "mask_aware_tokens_per_s": R / (single["mask_aware_ms"] * 1e-3),
             "dlogits_rel_l2_vs_two_pass": single["dlogits_rel_l2_vs_two_pass"],
             "scaled_upstream_ms": single.get("scaled_upstream_ms"),
+            "trainer_step_grad_accum_4_ms": single.get("trainer_step_grad_accum_4_ms"),
             "note": "grpo_loss_from_logits: the rows with gradient are read once and their gradient written by the same "
                     "kernel; same loss, log-probs, entropies and dlogits; the log-probs and entropies of the other rows "
                     "come from the forward kernel; mask-aware = those rows are not read at all (what `_compute_loss` "
-                    "does by default); scaled_upstream_ms = mask-aware step with loss * 1024 before backward"},
+                    "does by default); scaled_upstream_ms = mask-aware step with loss * 1024 before backward; "
+                    "trainer_step_grad_accum_4_ms = `GRPOLossMixin._compute_loss` on a trainer whose parent class divides "
+                    "the loss by 4 accumulation steps before backward, host-side metrics copy included"},
     }
     if ms_mask_aware is not None:
         result["mask_aware"] = {"ms_per_step": ms_mask_aware, "tokens_per_s": R / (ms_mask_aware * 1e-3),
@@ -814,6 +881,175 @@ def _brief(r):
     return out
 
 
+LEGS = ("k1", "k1_stats", "k3", "k7_masked", "k7_all_rows", "k7_dense_mask", "head_fwd_stash", "head_fwd_plain",
+        "head_bwd_every_token", "head_bwd_step")
+
+
+def bench_one_leg(args, w):
+    """One kernel of one workload in one mode, `--steps` launches back to back between two events.  Under a profiler
+    every launch of the kernel in the trace then moves the same bytes (or does the same flop), so the trace's average
+    duration belongs to one figure:
+      k1 / k1_stats          log-prob forward kernel (with row statistics: the DPO workload's form), every row
+      k3                     gradient kernel with the workload's mask (rows outside it are zero-filled, not read)
+      k7_masked              single-pass kernel, rows outside the mask zero-filled without being read
+      k7_all_rows            single-pass kernel, rows outside the mask read for their log-prob and entropy
+      k7_dense_mask          single-pass kernel with a mask of ones: every row read and written
+      head_fwd_stash/_plain  fused head forward with / without keeping its products
+      head_bwd_every_token   fused head backward (from the kept products) with a gradient on every token
+      head_bwd_step          the same with the benchmark's mask (tokens without gradient dropped first)"""
+    import trl_amd
+    from trl_amd import ops
+
+    dev = torch.device("cuda:0")
+    leg = args.only_leg
+    B, T, V = w["B"], w["T"], w["V"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    unit, peak = "GB/s", HBM_PEAK_GBPS
+    if w.get("head"):
+        if not leg.startswith("head_"):
+            sys.exit(f"bench.py: leg {leg} does not belong to workload {args.workload}")
+        N, H = B * T, w["H"]
+        hidden = torch.randn((N, H), generator=g, device=dev).bfloat16()
+        weight = (0.02 * torch.randn((V, H), generator=g, device=dev)).bfloat16()
+        targets = torch.randint(0, V, (N,), generator=g, device=dev)
+        lengths = torch.randint(w["min_len"], T + 1, (B,), generator=g, device=dev)
+        mask = (torch.arange(T, device=dev)[None] < lengths[:, None]).reshape(-1)
+        fwd_args = (hidden, weight, targets, w["temperature"], 0.0, 1.0)
+        gl = torch.randn((N,), generator=g, device=dev)
+        work = 2.0 * N * H * V
+        unit, peak = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS
+        with torch.no_grad():
+            if leg == "head_fwd_plain":
+                fn = lambda: ops.fused_head_fwd(*fwd_args)  # noqa: E731
+            elif leg == "head_fwd_stash":
+                fn = lambda: ops.fused_head_fwd(*fwd_args, None, True)  # noqa: E731
+            else:
+                out = ops.fused_head_fwd(*fwd_args, None, True)
+                log_z, saved = out[2], out[4]
+                del out
+                if leg == "head_bwd_every_token":
+                    work *= 2
+                    fn = lambda: ops.fused_head_bwd(*fwd_args, log_z, gl, HEAD_CHUNK, None, saved)  # noqa: E731
+                else:
+                    g_step = gl * mask.float()
+                    work *= 2.0 * float(mask.sum()) / N
+                    fn = lambda: ops.head_backward(*fwd_args, log_z, g_step, HEAD_CHUNK, None, saved)  # noqa: E731
+    elif w.get("logp") or w.get("dpo"):
+        if leg not in ("k1", "k1_stats", "k3") or (w.get("logp") and leg != "k1"):
+            sys.exit(f"bench.py: leg {leg} does not belong to workload {args.workload}")
+        dtype = torch.float32 if w.get("logp") else torch.bfloat16
+        L = T
+        K = T if w.get("logp") else T - 1
+        logits = torch.empty((B, L, V), dtype=dtype, device=dev)
+        for b in range(B):
+            logits[b] = ((3.0 if w.get("logp") else 2.0) * torch.randn((L, V), generator=g, device=dev)).to(dtype)
+        ids = torch.randint(0, V, (B, L), generator=g, device=dev)
+        R = B * K
+        idx = (ids if w.get("logp") else ids[:, 1:]).reshape(R, 1).contiguous()
+        row_bytes = V * logits.element_size()
+        if leg == "k1":
+            work = R * row_bytes
+            fn = lambda: ops.logp_entropy_fwd(logits, idx, 1.0, 0, K, None)  # noqa: E731
+        elif leg == "k1_stats":
+            work = R * row_bytes
+            fn = lambda: ops.logp_entropy_stats_fwd(logits, idx, 1.0, 0, K, None, False)  # noqa: E731
+        else:
+            prompt = torch.randint(64, 513, (B // 2,), generator=g, device=dev).repeat(2)
+            comp = torch.randint(128, 1537, (B,), generator=g, device=dev)
+            pos = torch.arange(L, device=dev)[None]
+            cmask = ((pos >= prompt[:, None]) & (pos < (prompt + comp)[:, None])).long()
+            lse = ops.logp_entropy_fwd(logits, idx, 1.0, 0, K, None)[2]
+            g_logp = (cmask[:, 1:].reshape(R, 1) * 0.01).float().contiguous()
+            active = int(cmask[:, 1:].sum())
+            work = active * 2 * row_bytes + (B * L - active) * row_bytes
+            fn = lambda: ops.logp_entropy_bwd(logits, idx, 1.0, 0, K, lse, None, g_logp, None)  # noqa: E731
+    else:
+        if leg not in ("k1", "k3", "k7_masked", "k7_all_rows", "k7_dense_mask"):
+            sys.exit(f"bench.py: leg {leg} does not belong to workload {args.workload}")
+        logits, ids, mask, rewards, g = make_inputs(w, dev)
+        R = B * T
+        idx = ids.reshape(R, 1)
+        adv = trl_amd.group_advantages(rewards, w["G"])
+        row_bytes = V * 2
+        active = int(mask.sum())
+        with torch.no_grad():
+            base, _, lse = ops.logp_entropy_fwd(logits, idx, w["temperature"], 0, T, None)
+        base = base.view(B, T)
+        old = base + 0.05 * torch.randn(base.shape, generator=g, device=dev)
+        ref = base + 0.1 * torch.randn(base.shape, generator=g, device=dev) if w["beta"] else None
+        n_items = mask.sum().float()
+        row_scale = (1.0 / n_items.clamp(min=1.0)).expand(B)
+        if leg == "k1":
+            work = R * row_bytes
+            fn = lambda: ops.logp_entropy_fwd(logits, idx, w["temperature"], 0, T, None)  # noqa: E731
+        elif leg == "k3":
+            g_logp = (mask.reshape(R, 1) * 0.01).float().contiguous()
+            work = active * 2 * row_bytes + (R - active) * row_bytes
+            fn = lambda: ops.logp_entropy_bwd(logits, idx, w["temperature"], 0, T, lse, None, g_logp, None)  # noqa: E731
+        else:
+            m = torch.ones_like(mask) if leg == "k7_dense_mask" else mask
+            every = leg == "k7_all_rows"
+            work = 2 * R * row_bytes if leg != "k7_masked" else active * 2 * row_bytes + (R - active) * row_bytes
+            fn = lambda: ops.grpo_fused_fwd_bwd(logits, ids, w["temperature"], 0, T, m, adv, row_scale, old, ref, None,  # noqa: E731
+                                                None, 0, w["eps_low"], w["eps_high"], float("nan"), w["beta"], False,
+                                                1.0, 1.05, every)
+    with torch.no_grad():
+        for _ in range(max(1, args.warmup)):
+            out = fn()
+            del out
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(args.steps):
+            out = fn()
+            del out
+        b.record()
+        torch.cuda.synchronize()
+    ms = a.elapsed_time(b) / args.steps
+    achieved = work / (ms * 1e-3) / (1e9 if unit == "GB/s" else 1e12)
+    return {"workload": args.workload, "leg": leg, "launches": args.steps, "warmup_launches": max(1, args.warmup),
+            "avg_launch_ms": ms, "algorithmic_bytes" if unit == "GB/s" else "algorithmic_flop": work,
+            "achieved": achieved, "unit": unit, "peak": peak, "frac": achieved / peak}
+
+
+def _summary_rows(r):
+    """Compact rows for the end of the line: per workload / loss type the step time, the dominant kernel's fraction of
+    its roofline and the step's own (HBM workloads) or the TFLOP/s (matrix workload); numbers rounded."""
+    cfg = r.get("config", {})
+    name, lt = r.get("workload") or cfg.get("workload"), r.get("loss_type") or cfg.get("loss_type")
+    if "error" in r:
+        return [{"w": name, "lt": lt, "error": r["error"][:80]}]
+    roof = r["roofline"]
+    kern = {"grpo_fused_kernel (K7)": "K7", "logp_entropy_bwd_kernel (K3)": "K3", "logp_entropy_fwd_kernel (K1)": "K1",
+            "fused_head_fwd_kernel": "head_fwd"}.get(roof["kernel"], roof["kernel"])
+    row = {"w": name, "lt": lt, "ms": round(r["ms_per_step"], 3), "k": kern, "frac": round(roof["frac"], 3)}
+    if roof.get("step_hbm_frac") is not None:
+        row["step_frac"] = round(roof["step_hbm_frac"], 3)
+    rows = [row]
+    kernels = r.get("kernels") or {}
+    if roof["bound"] == "mfma":
+        row["TFLOPs"] = round(roof["achieved"])
+        bwd = kernels.get("fused_head_bwd")
+        if bwd:
+            rows.append({"w": name, "k": "head_bwd_every_token", "ms": round(bwd["avg_ms"], 2), "frac": round(bwd["frac"], 3),
+                         "TFLOPs": round(bwd["TFLOPs"])})
+        plain = kernels.get("fused_head_fwd_no_grad")
+        if plain:
+            rows.append({"w": name, "k": "head_fwd_no_stash", "ms": round(plain["avg_ms"], 2), "frac": round(plain["frac"], 3)})
+    for key, short in (("grpo_fused_kernel (K7), every row active (a mask of ones)", "K7_dense_mask"),
+                       ("logp_entropy_fwd_kernel (K1)", "K1"), ("logp_entropy_bwd_kernel (K3)", "K3"),
+                       ("logp_entropy_fwd_kernel with row statistics (K1)", "K1_stats")):
+        k = kernels.get(key)
+        if k and short != kern:
+            rows.append({"w": name, "k": short, "ms": round(k["avg_launch_ms"], 3), "frac": round(k["frac"], 3)})
+    return rows
+
+
+def _is_hip_runtime_error(exc):
+    text = f"{type(exc).__name__}: {exc}"
+    return "HIP error" in text or "hipError" in text or "AcceleratorError" in text
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -826,6 +1062,9 @@ def main():
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain device copy of the logits (known bytes) to scale profiler counters by")
+    ap.add_argument("--only-leg", default=None, choices=sorted(LEGS),
+                    help="launch ONE kernel of --workload in ONE mode --steps times and print its event-timed average "
+                         "(for profiler runs: every launch of that kernel in the trace then moves the same bytes)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs on ONE GPU; rows are independent, so N GPUs would each run this same "
@@ -836,6 +1075,8 @@ def main():
     secondary_wanted = args.workload is None and not args.no_secondary
     args.workload = args.workload or "grpo_c3"
     w = WORKLOADS[args.workload]
+    if args.only_leg:
+        return print(json.dumps(bench_one_leg(args, w)))
     if w.get("head"):
         return print(json.dumps(bench_head(args, w)))
     if w.get("dpo"):
@@ -844,21 +1085,26 @@ def main():
         return print(json.dumps(bench_logp_c1(args, w)))
     result, shared = bench_grpo(args, w, args.loss_type)
     secondary = []
+    device_lost = False  # after a HIP runtime error every later launch fails the same way: no further legs
     if secondary_wanted:
         few = argparse.Namespace(**{**vars(args), "steps": max(3, args.steps // 2), "warmup": 2, "no_cpu_baseline": True,
                                     "calibrate_copy": False})
         for lt in ("grpo", "dr_grpo"):
-            if lt != args.loss_type:
+            if lt != args.loss_type and not device_lost:
                 try:
                     secondary.append(_brief(bench_grpo(few, w, lt, shared, full=False)[0]))
                 except Exception as exc:
                     secondary.append({"workload": args.workload, "loss_type": lt, "error": f"{type(exc).__name__}: {exc}"[:500]})
+                    device_lost = _is_hip_runtime_error(exc)
     del shared
-    torch.cuda.empty_cache()
     if secondary_wanted:
         # (the matrix-core workload first: its clock is set by the power budget and falls as the part warms up,
         # the streaming workloads are bound by memory and hardly notice)
         for name in ("head_c5", "grpo_c4", "dpo_c2", "logp_c1"):
+            if device_lost:
+                secondary.append({"workload": name, "error": "not run: an earlier workload ended in a HIP runtime error"})
+                continue
+            torch.cuda.empty_cache()
             few.workload = name
             w2 = WORKLOADS[name]
             try:
@@ -868,7 +1114,7 @@ def main():
                 del r
             except Exception as exc:  # a secondary workload never takes the headline line with it
                 secondary.append({"workload": name, "error": f"{type(exc).__name__}: {exc}"[:500]})
-            torch.cuda.empty_cache()
+                device_lost = _is_hip_runtime_error(exc)
         result["secondary"] = secondary
     if not args.no_cpu_baseline:
         base = cpu_baseline(w, args.loss_type, repeats=1)
@@ -878,7 +1124,17 @@ def main():
         result["cpu_baseline"] = base
     else:
         result["cpu_baseline"] = None
+    # the end of the line: what a reader of its last 2000 characters needs -- every workload's step time and roofline
+    # fractions, and whether a secondary workload failed
+    errors = [f"{r.get('workload')}/{r.get('loss_type')}: {r['error']}"[:200] for r in secondary if "error" in r]
+    result["secondary_errors"] = errors
+    summary = _summary_rows(result)
+    for r in secondary:
+        summary += _summary_rows(r)
+    result["summary"] = summary
     print(json.dumps(result))
+    if errors:
+        sys.exit(f"bench.py: {len(errors)} secondary workload(s) failed: {errors}")
 
 
 if __name__ == "__main__":

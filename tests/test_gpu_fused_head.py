@@ -405,6 +405,30 @@ def test_bf16_pieces_give_the_fp32_product(amd):
         ops.gemm_nt(a16[:, :68], b16[:, :68])  # K must be a multiple of 8
 
 
+def test_fp32_operands_with_strides(amd):
+    """fp32 hidden states and weight that are views with other strides (a transposed buffer, every other row): the
+    gradients come back dense, equal to those of contiguous copies."""
+    g = torch.Generator(device=DEV).manual_seed(91)
+    n, h, v = 70, 48, 200
+    hidden_t = torch.randn((h, n), generator=g, device=DEV)
+    weight_2 = 0.2 * torch.randn((2 * v, h), generator=g, device=DEV)
+    labels = torch.randint(0, v, (n,), generator=g, device=DEV)
+    gout = torch.randn((n,), generator=g, device=DEV)
+    res = []
+    for hid, wt in ((hidden_t.t(), weight_2[::2]), (hidden_t.t().contiguous(), weight_2[::2].contiguous())):
+        hh, ww = hid.detach().requires_grad_(True), wt.detach().requires_grad_(True)
+        assert hh.is_contiguous() == ww.is_contiguous()
+        lp, _ = amd._ChunkedLogProbFunction.apply(hh, ww, labels, 0.9, 64)
+        (lp * gout).sum().backward()
+        res.append((lp.detach(), hh.grad, ww.grad))
+    assert not hidden_t.t().is_contiguous() and not weight_2[::2].is_contiguous()
+    for a, b in zip(res[0], res[1]):
+        torch.testing.assert_close(a, b, rtol=1e-6, atol=1e-7)
+    rlp, _, rdh, rdw = _fp32_reference(hidden_t.t().cpu(), weight_2[::2].cpu(), labels.cpu(), 0.9, None, 1.0, gout.cpu())
+    torch.testing.assert_close(res[0][0].cpu(), rlp, rtol=1e-5, atol=1e-5)
+    assert _rel_l2(res[0][1], rdh) < 1e-5 and _rel_l2(res[0][2], rdw) < 1e-5
+
+
 def test_fp64_operands_are_rejected_loudly(amd):
     with pytest.raises(TypeError):
         amd._ChunkedLogProbFunction.apply(torch.randn(4, 8, device=DEV, dtype=torch.float64),
