@@ -35,17 +35,21 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
-# HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE (two --pmc runs of this file,
-# each scaled by the same counter's reading for a plain device copy of known size: FETCH x 2.000, WRITE x 1.000 KiB;
-# summaries under profiles/).  The inputs are seeded, so the figures are stable; they are records of those runs, not
-# measured by the run that prints them, and None where no counter run was made for that workload / loss type.
+# HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE: two --pmc runs of
+# `bench.py --workload W --only-leg LEG --calibrate-copy` per entry (every dispatch of the kernel in such a run is the
+# same launch), each counter scaled by its reading for the 1 GiB device copy of the same run (FETCH x 2.000,
+# WRITE x 1.000 KiB; summaries under profiles/).  The inputs are seeded, so the figures are stable; they are records of
+# those runs, not measured by the run that prints them, and None where no counter run was made.
 MEASURED_TRAFFIC_BYTES = {
-    ("K3", "grpo_c3", "dapo"): (2 * 5054241 + 19454900) * 1024,
-    ("K7", "grpo_c3", "dapo"): (2 * 5055205 + 19474750) * 1024,
-    ("K3", "grpo_c4", "dapo"): (2 * 10685504 + 38911700) * 1024,
-    ("K7", "grpo_c4", "dapo"): (2 * 10686905 + 38959000) * 1024,
-    ("K3", "dpo_c2", None): (2 * 6605806 + 32849200) * 1024,
-    ("head_fwd", "head_c5", "dapo"): (2 * 40600000 + 19497000) * 1024,
+    ("K3", "grpo_c3", "dapo"): (2 * 5056283 + 19450543) * 1024,       # --only-leg k3
+    ("K7", "grpo_c3", "dapo"): (2 * 5055232 + 19469108) * 1024,       # --only-leg k7_masked
+    ("K3", "grpo_c4", "dapo"): (2 * 10689829 + 38900940) * 1024,
+    ("K7", "grpo_c4", "dapo"): (2 * 10686914 + 38943851) * 1024,
+    ("K3", "dpo_c2", None): (2 * 6608991 + 32838146) * 1024,
+    ("K1", "logp_c1", None): (2 * 128206 + 192) * 1024,
+    # (the forward's operand re-reads vary from launch to launch with how closely the workgroups of an XCD stay in
+    # step: 55.4-68.0 M KiB of fetches over three launches; the stash itself is 19.49 M KiB of writes)
+    ("head_fwd", "head_c5", "dapo"): (2 * 29849519 + 19491843) * 1024,  # --only-leg head_fwd_stash
 }
 # the loss type changes per-row scalars only: the same rows are read and written, by the same launches
 for _k in ("K3", "K7"):
@@ -535,7 +539,8 @@ def bench_logp_c1(args, w):
         "config": {"workload": args.workload, "description": w["desc"], "rows": R, "vocab": V,
                    "max_abs_err_logps_vs_oracle": err_lp, "max_abs_err_entropy_vs_oracle": err_h},
         "roofline": {"bound": "hbm", "kernel": "logp_entropy_fwd_kernel (K1)", "achieved": gbps, "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "algorithmic_bytes": nbytes,
+                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(("K1", args.workload, None)), "algorithmic_bytes": nbytes,
                      "avg_launch_ms": ms_kernel,
                      "note": "back-to-back launches over eight copies of the logits (each launch reads cold data)"},
         "two_calls_ms_per_step": ms_two,
@@ -947,7 +952,17 @@ def bench_one_leg(args, w):
         R = B * K
         idx = (ids if w.get("logp") else ids[:, 1:]).reshape(R, 1).contiguous()
         row_bytes = V * logits.element_size()
-        if leg == "k1":
+        if leg == "k1" and w.get("logp"):
+            # 262 MB would stay in the memory-side cache between launches: rotate over eight copies, as the workload's
+            # own bench leg does, so that every launch reads cold data
+            work = R * row_bytes
+            copies = [logits] + [logits.clone() for _ in range(7)]
+            turn = [0]
+
+            def fn():
+                turn[0] += 1
+                return ops.logp_entropy_fwd(copies[turn[0] % 8], idx, 1.0, 0, K, None)
+        elif leg == "k1":
             work = R * row_bytes
             fn = lambda: ops.logp_entropy_fwd(logits, idx, 1.0, 0, K, None)  # noqa: E731
         elif leg == "k1_stats":
@@ -1007,6 +1022,12 @@ def bench_one_leg(args, w):
         torch.cuda.synchronize()
     ms = a.elapsed_time(b) / args.steps
     achieved = work / (ms * 1e-3) / (1e9 if unit == "GB/s" else 1e12)
+    if args.calibrate_copy:  # a plain device copy of known size, to scale the profiler's byte counters by
+        src = torch.empty((1 << 28,), dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)  # reads and writes 1 GiB each
+        torch.cuda.synchronize()
     return {"workload": args.workload, "leg": leg, "launches": args.steps, "warmup_launches": max(1, args.warmup),
             "avg_launch_ms": ms, "algorithmic_bytes" if unit == "GB/s" else "algorithmic_flop": work,
             "achieved": achieved, "unit": unit, "peak": peak, "frac": achieved / peak}

@@ -145,18 +145,22 @@ __device__ __forceinline__ float max_of(const float* x) {
 // STATS: 1 or 2 also produce the row statistics of `out_stats`; only 2 accumulates the sum of squared probabilities
 // (one more multiply-add per logit in a loop that is bound by its arithmetic: 5.14 against 4.95 ms on 33.6 GB of bf16
 // logits), 1 reports 0 in its place.
-template <int DT, bool VEC, int STATS>
-__global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
+// TH lanes per row, UN 16-byte loads in flight per lane: 256 x 4 on long batches; launches of few rows take 512 x 2
+// (the same bytes in flight per workgroup, half as many dependent rounds per row: 44.3 -> 42.2 us on 2048 fp32 rows
+// of 32000, where the ramp and the tail of a launch that is one round of workgroups are a tenth of its time).
+template <int DT, bool VEC, int STATS, int TH = kThreads, int UN = kUnroll>
+__global__ __launch_bounds__(TH) void logp_entropy_fwd_kernel(FwdArgs a) {
+    static_assert(UN >= 2, "the row tail holds up to UN - 1 vectors per lane");
     typedef Elem<DT> E;
     typedef typename E::type T;
-    constexpr int NW = kThreads / kWave;
+    constexpr int NW = TH / kWave;
     __shared__ float red[STATS ? 7 : 3][NW];
     __shared__ float bcast[2];
 
     const int64_t row = blockIdx.x;
     const int tid = threadIdx.x;
     if (a.row_mask != nullptr && a.row_mask[row] == 0) {
-        for (int k = tid; k < a.n_index; k += kThreads) a.out_logp[row * a.n_index + k] = 0.f;
+        for (int k = tid; k < a.n_index; k += TH) a.out_logp[row * a.n_index + k] = 0.f;
         if (tid == 0) {
             if (a.out_entropy) a.out_entropy[row] = 0.f;
             if (a.out_lse) a.out_lse[row] = 0.f;
@@ -237,42 +241,42 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
         const u32x4* vp = reinterpret_cast<const u32x4*>(base + head);
         const int nvec = int((V - head) / EPV);
         int v = tid;
-        for (; v + (kUnroll - 1) * kThreads < nvec; v += kUnroll * kThreads) {
-            u32x4 q[kUnroll];
+        for (; v + (UN - 1) * TH < nvec; v += UN * TH) {
+            u32x4 q[UN];
 #pragma unroll
-            for (int j = 0; j < kUnroll; ++j) q[j] = stream_load<kFwdNt>(vp + v + j * kThreads);
+            for (int j = 0; j < UN; ++j) q[j] = stream_load<kFwdNt>(vp + v + j * TH);
             if constexpr (STATS) {
 #pragma unroll
-                for (int j = 0; j < kUnroll; ++j) stat_sum(q[j]);
+                for (int j = 0; j < UN; ++j) stat_sum(q[j]);
             }
-            float x[kUnroll * EPV];
+            float x[UN * EPV];
 #pragma unroll
-            for (int j = 0; j < kUnroll; ++j) E::unpack(q[j], x + j * EPV);
-            const float bm = max_of<kUnroll * EPV>(x);  // one maximum over the whole group
+            for (int j = 0; j < UN; ++j) E::unpack(q[j], x + j * EPV);
+            const float bm = max_of<UN * EPV>(x);  // one maximum over the whole group
             raise(bm);
 #pragma unroll
-            for (int i = 0; i < kUnroll * EPV; ++i) add(x[i]);
+            for (int i = 0; i < UN * EPV; ++i) add(x[i]);
             if constexpr (STATS) {
                 // the lane's running maximum moves a few times per row: only then is the position looked for, over
                 // the group's vectors in the order of their positions (the j-th lies before the (j+1)-th)
                 if (bm > st.vmax) {
                     st.vmax = bm;
-                    int first = kUnroll * EPV - 1;
-                    for (int i = kUnroll * EPV - 2; i >= 0; --i) first = x[i] == bm ? i : first;
-                    st.vpos = float(head + int64_t(v + (first / EPV) * kThreads) * EPV + first % EPV);
+                    int first = UN * EPV - 1;
+                    for (int i = UN * EPV - 2; i >= 0; --i) first = x[i] == bm ? i : first;
+                    st.vpos = float(head + int64_t(v + (first / EPV) * TH) * EPV + first % EPV);
                 }
             }
         }
-        // the row's tail: fewer than kUnroll vectors are left for this lane; their loads go out together
+        // the row's tail: fewer than UN vectors are left for this lane; their loads go out together
         // (one after the other they would cost a memory round trip each, at the end of every row)
         {
-            u32x4 q[kUnroll - 1];
+            u32x4 q[UN - 1];
 #pragma unroll
-            for (int j = 0; j < kUnroll - 1; ++j)
-                if (v + j * kThreads < nvec) q[j] = stream_load<kFwdNt>(vp + v + j * kThreads);
+            for (int j = 0; j < UN - 1; ++j)
+                if (v + j * TH < nvec) q[j] = stream_load<kFwdNt>(vp + v + j * TH);
 #pragma unroll
-            for (int j = 0; j < kUnroll - 1; ++j) {
-                if (v + j * kThreads < nvec) {
+            for (int j = 0; j < UN - 1; ++j) {
+                if (v + j * TH < nvec) {
                     if constexpr (STATS) stat_sum(q[j]);
                     float x[EPV];
                     E::unpack(q[j], x);
@@ -280,12 +284,12 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
                     raise(bm);
 #pragma unroll
                     for (int i = 0; i < EPV; ++i) add(x[i]);
-                    if constexpr (STATS) stat_vec(x, head + int64_t(v + j * kThreads) * EPV, EPV, bm);
+                    if constexpr (STATS) stat_vec(x, head + int64_t(v + j * TH) * EPV, EPV, bm);
                 }
             }
         }
         if constexpr (!VEC) {  // what is left of the row after its whole vectors (these positions come last for a lane)
-            for (int64_t e = head + int64_t(nvec) * EPV + tid; e < V; e += kThreads) {
+            for (int64_t e = head + int64_t(nvec) * EPV + tid; e < V; e += TH) {
                 const float x = E::load1(base + e);
                 raise(x);
                 add(x);
@@ -359,7 +363,7 @@ __global__ __launch_bounds__(kThreads) void logp_entropy_fwd_kernel(FwdArgs a) {
     }
     __syncthreads();
     const float lse = bcast[0];
-    for (int k = tid; k < a.n_index; k += kThreads) {
+    for (int k = tid; k < a.n_index; k += TH) {
         const int64_t idx = a.index[row * a.n_index + k];
         float r;
         if (idx < 0 || idx >= V) {
@@ -585,8 +589,12 @@ extern "C" int trlk_logp_entropy_fwd(const void* d_logits, int dtype, int64_t n_
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)rows), block(kThreads);
     const int stats = d_out_row_stats == nullptr ? 0 : (row_stats_sum_p2 ? 2 : 1);
+    // a launch that is at most two rounds of workgroups over rows of several iterations each: more lanes per row
+    const bool few_rows = stats == 0 && rows <= 4096 && vocab * int64_t(es) >= 32768;
 #define TRLK_LAUNCH_FWD_VEC(DT, VEC)                                                           \
-    if (stats == 2)                                                                            \
+    if (few_rows)                                                                              \
+        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, VEC, 0, 512, 2>), grid, dim3(512), 0, s, a); \
+    else if (stats == 2)                                                                       \
         hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, VEC, 2>), grid, block, 0, s, a);       \
     else if (stats == 1)                                                                       \
         hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, VEC, 1>), grid, block, 0, s, a);       \
