@@ -192,7 +192,7 @@ def test_grpo_loss_against_oracle_random(amd):
         loss, metrics = amd.grpo_loss(dlp, a_in.to(DEV), mask.to(DEV), **dkw)
         loss.backward()
         tag = (lt, level, beta, tuple(a_in.shape))
-        assert abs(float(loss) - float(oloss)) <= 1e-5 * max(1.0, abs(float(oloss))), (tag, float(loss), float(oloss))
+        assert abs(float(loss.detach()) - float(oloss.detach())) <= 1e-5 * max(1.0, abs(float(oloss.detach()))), (tag, float(loss.detach()), float(oloss.detach()))
         assert _rel_l2(dlp.grad, olp.grad) < 1e-5, tag
         md = amd.trainer.metrics_to_dict(metrics, beta, loss_type=lt)
         for name, want in ometrics.items():

@@ -145,9 +145,7 @@ __device__ __forceinline__ float max_of(const float* x) {
 // STATS: 1 or 2 also produce the row statistics of `out_stats`; only 2 accumulates the sum of squared probabilities
 // (one more multiply-add per logit in a loop that is bound by its arithmetic: 5.14 against 4.95 ms on 33.6 GB of bf16
 // logits), 1 reports 0 in its place.
-// TH lanes per row, UN 16-byte loads in flight per lane: 256 x 4 on long batches; launches of few rows take 512 x 2
-// (the same bytes in flight per workgroup, half as many dependent rounds per row: 44.3 -> 42.2 us on 2048 fp32 rows
-// of 32000, where the ramp and the tail of a launch that is one round of workgroups are a tenth of its time).
+// TH lanes per row, UN 16-byte loads in flight per lane.
 template <int DT, bool VEC, int STATS, int TH = kThreads, int UN = kUnroll>
 __global__ __launch_bounds__(TH) void logp_entropy_fwd_kernel(FwdArgs a) {
     static_assert(UN >= 2, "the row tail holds up to UN - 1 vectors per lane");
@@ -589,12 +587,11 @@ extern "C" int trlk_logp_entropy_fwd(const void* d_logits, int dtype, int64_t n_
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)rows), block(kThreads);
     const int stats = d_out_row_stats == nullptr ? 0 : (row_stats_sum_p2 ? 2 : 1);
-    // a launch that is at most two rounds of workgroups over rows of several iterations each: more lanes per row
-    const bool few_rows = stats == 0 && rows <= 4096 && vocab * int64_t(es) >= 32768;
+    // (One launch shape whatever the number of rows: 512 lanes x 2 loads per row is 5 % faster on launches that are a
+    // single round of workgroups, but it sums a row in another order, and a row's log-prob must not depend on how many
+    // other rows the launch holds -- a reference pass over part of a batch has to reproduce the policy pass bit for bit.)
 #define TRLK_LAUNCH_FWD_VEC(DT, VEC)                                                           \
-    if (few_rows)                                                                              \
-        hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, VEC, 0, 512, 2>), grid, dim3(512), 0, s, a); \
-    else if (stats == 2)                                                                       \
+    if (stats == 2)                                                                            \
         hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, VEC, 2>), grid, block, 0, s, a);       \
     else if (stats == 1)                                                                       \
         hipLaunchKernelGGL((logp_entropy_fwd_kernel<DT, VEC, 1>), grid, block, 0, s, a);       \
