@@ -606,6 +606,51 @@ def _trainer_step_legs(args, w, loss_type, shared, timed):
     return out
 
 
+def _parity_sample(w, loss_type, shared, run_step, n_rows=24):
+    """The headline step's outputs against the CPU oracle on a sample of rows, inside the run that times it: the
+    log-prob and entropy of `n_rows` token rows from the stored bf16 logits (fp32 arithmetic on the host), the loss from
+    the oracle's loss on the step's log-probs, and those rows of the gradient from the oracle's d loss / d log-prob
+    through the host's log-softmax.  Bars as in the tests: 2e-3 absolute (bf16 logits), loss 1e-3 relative, gradient rows
+    5e-3 relative L2 (the device rounds them to bf16)."""
+    import oracle
+
+    logits, ids, mask, adv, old, ref, n_items, leaf = (shared[k] for k in ("logits", "ids", "mask", "adv", "old", "ref",
+                                                                        "n_items", "leaf"))
+    B, T = ids.shape
+    loss, lp, ent = run_step()
+    grad = leaf.grad
+    pick = torch.Generator().manual_seed(1)
+    active = torch.nonzero(mask.cpu().reshape(-1)).reshape(-1)
+    rows = active[torch.randperm(active.numel(), generator=pick)[:n_rows]]
+    rows = torch.cat([rows, torch.tensor([0, int(active[-1])])]).unique()
+    b_idx, t_idx = (rows // T).to(logits.device), (rows % T).to(logits.device)
+    x = logits.detach()[b_idx, t_idx].cpu().float().requires_grad_(True)
+    tok = ids.cpu().reshape(-1)[rows]
+    temp = w["temperature"]
+    want_lp = oracle.selective_log_softmax_f32(x.detach(), tok, temp)
+    want_ent = oracle.entropy_from_logits_f32(x.detach(), temp)
+    err_lp = float((lp.detach().cpu().reshape(-1)[rows] - want_lp).abs().max())
+    err_ent = float((ent.detach().cpu().reshape(-1)[rows] - want_ent).abs().max())
+    lp_host = lp.detach().cpu().clone().requires_grad_(True)
+    oloss, _ = oracle.grpo_loss(
+        lp_host, adv.cpu(), mask.cpu(), entropies=ent.detach().cpu(), old_per_token_logps=old.cpu(),
+        ref_per_token_logps=None if ref is None else ref.cpu(), loss_type=loss_type, epsilon_low=w["eps_low"],
+        epsilon_high=w["eps_high"], beta=w["beta"], max_completion_length=T, num_items_in_batch=n_items.cpu())
+    oloss.backward()
+    g_tok = lp_host.grad.reshape(-1)[rows]
+    z = x / temp
+    (torch.log_softmax(z, -1).gather(-1, tok[:, None]).squeeze(-1) * g_tok).sum().backward()
+    got = grad[b_idx, t_idx].cpu().float()
+    rel = float((got - x.grad).norm() / x.grad.norm().clamp(min=1e-30))
+    loss_rel = abs(float(loss.detach()) - float(oloss.detach())) / max(1e-12, abs(float(oloss.detach())))
+    leaf.grad = None
+    assert err_lp <= 2e-3 and err_ent <= 2e-3 and loss_rel <= 1e-3 and rel <= 5e-3, (err_lp, err_ent, loss_rel, rel)
+    return {"rows": int(rows.numel()), "max_abs_err_logp": err_lp, "max_abs_err_entropy": err_ent,
+            "loss_rel_err": loss_rel, "dlogits_rel_l2": rel,
+            "note": "the step's outputs on a sample of token rows against the CPU oracle (fp32 arithmetic on the stored "
+                    "bf16 logits; gradient rows through the oracle's loss gradient and the host's log-softmax)"}
+
+
 def _grad_distance(run_a, run_b, leaf):
     """Relative L2 distance between the gradients two step functions leave in `leaf.grad`, accumulated sequence
     by sequence (no logits-sized fp32 temporaries)."""
@@ -698,6 +743,17 @@ def bench_grpo(args, w, loss_type, shared=None, full=True):
         single = {"all_rows_ms": ms_sp_all, "mask_aware_ms": ms_sp_skip,
                   # the gradient of the one pass against the gradient of the two passes (both rounded to bf16 once)
                   "dlogits_rel_l2_vs_two_pass": _grad_distance(lambda: sp_step(False), lambda: step(None), leaf)}
+        if full and not args.no_cpu_baseline:
+            def sp_outputs():
+                leaf.grad = None
+                out = trl_amd.grpo_loss_from_logits(
+                    leaf, ids, adv, mask, temperature=w["temperature"], old_per_token_logps=old, ref_per_token_logps=ref,
+                    loss_type=loss_type, epsilon_low=w["eps_low"], epsilon_high=w["eps_high"], beta=w["beta"],
+                    max_completion_length=T, num_items_in_batch=n_items, keep_start=0, skip_masked_rows=False)
+                out[0].backward()
+                return out[0], out[2], out[3]
+
+            single["parity_vs_oracle"] = _parity_sample(w, loss_type, shared, sp_outputs)
         if full:
             # an upstream gradient other than 1 (a gradient scaler): announced to the forward it costs nothing,
             # unannounced it costs a further read + write of the gradient in `backward`
@@ -836,6 +892,7 @@ def bench_grpo(args, w, loss_type, shared=None, full=True):
             "mask_aware_ms_per_step": single["mask_aware_ms"],
             "mask_aware_tokens_per_s": R / (single["mask_aware_ms"] * 1e-3),
             "dlogits_rel_l2_vs_two_pass": single["dlogits_rel_l2_vs_two_pass"],
+            "parity_vs_oracle": single.get("parity_vs_oracle"),
             "scaled_upstream_ms": single.get("scaled_upstream_ms"),
             "trainer_step_grad_accum_4_ms": single.get("trainer_step_grad_accum_4_ms"),
             "note": "grpo_loss_from_logits: the rows with gradient are read once and their gradient written by the same "
