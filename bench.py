@@ -207,7 +207,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
 # Vocabulary rows per backward chunk of the fused head.  The operator's `chunk_size` only sizes the
 # dz workspace (2 x N x chunk bf16); 32768 rows = 4.3 GB at this shape, a small share of the card's
 # HBM, and leaves 5 chunks instead of 19 (fewer partial waves and dHidden accumulation passes).
-HEAD_CHUNK = 32768
+HEAD_CHUNK = int(os.environ.get("TRL_AMD_BENCH_HEAD_CHUNK", "32768"))
 
 
 def bench_head(args, w):

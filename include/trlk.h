@@ -296,9 +296,9 @@ int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, const int64_
  * for one chunk at a time inside the workspace, as fp16 whatever `dtype` is: both products run on
  * fp16 operands (11 significant bits in dz instead of bf16's 8; the reference keeps fp32 grad_logits,
  * utils.py:1405-1424), each operand multiplied by a power of two taken from its largest magnitude
- * (dz per token and by the largest |g|, and for bf16 inputs W_chunk^T and hidden^T, which convert
- * exactly) and the factors divided out of the fp32 accumulators, so that neither small upstream
- * gradients nor wide-ranged bf16 values leave the fp16 range.
+ * (dz per token, hidden^T's columns by the inverse of that relative to the largest |g|, and for bf16 inputs
+ * W_chunk^T and hidden^T by their own maxima, which convert exactly) and the factors divided out of the fp32
+ * accumulators, so that neither small upstream gradients nor wide-ranged bf16 values leave the fp16 range.
  * d_out_dbias (optional, fp32 [vocab]): sum over tokens of dz, the gradient of d_bias.
  * d_stash_cols (optional, int32 [n_tokens]): the stash column of each token, for a caller that dropped tokens
  * since the forward (those without an upstream gradient contribute nothing to either product); values in

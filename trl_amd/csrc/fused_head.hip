@@ -15,13 +15,15 @@
 // epilogue needs no cross-lane traffic; a workgroup keeps 256 tokens and walks over its share of
 // the vocabulary tiles, the logits exist only as accumulators.
 //
-// Backward (K6), per vocabulary chunk: (1) dz = dL/dlogits (scaled fp16), written both as [tokens, chunk]
-// and as [chunk, tokens] -- from a recompute of the chunk's logits (same tile loop), or, when the
-// forward was asked to stash its raw products, from one elementwise sweep over that stash;
-// (2) dHidden += dz * W_chunk as an NT product against W^T; (3) dW_chunk = dz^T * hidden as an NT
-// product against hidden^T, both on fp16 operands (bf16 inputs are converted while they are transposed).  The contraction of (2)/(3) is over a different axis than the
-// recompute, and with H in the thousands the output tile of a fused kernel cannot stay in
-// registers, so dz goes through a chunk-sized workspace (never the whole [N, V] matrix).
+// Backward (K6), per vocabulary chunk: (1) dz = dL/dlogits as scaled fp16 [chunk, tokens] (vocabulary-major, each
+// token's column in that token's own power-of-two scale) -- from a recompute of the chunk's logits (same tile loop),
+// or, when the forward was asked to stash its raw products, from one elementwise sweep over that stash;
+// (2) dHidden += dz * W_chunk: the tile loop with dz as a K-MAJOR left operand (its k rows go to LDS as they lie in
+// memory and the MFMA fragments come out through the LDS transpose loads, ds_read_b64_tr_b16) against W_chunk^T;
+// (3) dW_chunk = dz^T * hidden as an NT product against hidden^T, whose columns carry the inverse of the tokens'
+// scales; all on fp16 operands (bf16 inputs are converted while they are transposed).  The contraction of (2)/(3)
+// is over a different axis than the recompute, and with H in the thousands the output tile of a fused kernel cannot
+// stay in registers, so dz goes through a chunk-sized workspace (never the whole [N, V] matrix).
 #include "common.hpp"
 
 #include <type_traits>
@@ -61,10 +63,10 @@ constexpr int kLoadsA = BM / kRowStep, kLoadsB = BN / kRowStep;
 constexpr int kTileABytes = BM * kLdsRow * 2, kTileBBytes = BN * kLdsRow * 2;
 constexpr int kStageBytes = kTileABytes + kTileBBytes;
 constexpr int kDirectLdsBytesDecl = 2 * (BM + BN) * 64 * 2;  // direct-to-LDS tile ring: 4 x 32-wide or 2 x 64-wide stages
-constexpr int kDzLdsRow = BM * 2 + 16;     // bytes per token row of the dz tile staged in LDS by the backward
+constexpr int kDzLdsRow = BN * 2 + 16;     // bytes per vocabulary row of the dz tile staged in LDS by the backward
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
-constexpr int kHeadLdsBytes = cmax(cmax(2 * kStageBytes, kDirectLdsBytesDecl), BN * kDzLdsRow);
-static_assert(BN * kDzLdsRow <= kHeadLdsBytes, "dz staging tile");
+constexpr int kHeadLdsBytes = cmax(cmax(2 * kStageBytes, kDirectLdsBytesDecl), BM * kDzLdsRow);
+static_assert(BM * kDzLdsRow <= kHeadLdsBytes, "dz staging tile");
 static_assert(2 * WGM * BN * 4 * 4 <= kHeadLdsBytes && BN <= kHeadThreads, "merge scratch");
 static_assert(BM % kRowStep == 0 && BN % kRowStep == 0 && WM % 32 == 0 && WN % 32 == 0 && BK % 16 == 0, "tile shape");
 
@@ -83,12 +85,17 @@ __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
                                                       0, 0);
 }
 
-// One operand of the NT product: `rows` x K, row-major with leading dimension ld (elements).
+// One operand of the NT product: `rows` x K, row-major with leading dimension ld (elements).  The left operand may
+// instead be given "k-major" (AKM below): K x `rows`, row-major with leading dimension ld -- the transpose of what the
+// product wants, read through the LDS transpose loads; its columns must be readable (and zero) up to the next
+// multiple of the tile size.
 struct Operand {
     const uint16_t* p;
     int64_t ld;
     int rows;
 };
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
 #ifndef TRLK_HEAD_DIRECT_LDS
 #define TRLK_HEAD_DIRECT_LDS 1
@@ -138,9 +145,13 @@ static_assert(DirectCfg<32>::kLdsBytes <= kHeadLdsBytes && DirectCfg<64>::kLdsBy
 
 // Loader side of the direct-to-LDS loop: per-lane source offsets of the wave's tile blocks and the
 // transfer of one stage.
-template <int BKT>
+// AKM: the left operand is k-major.  Its stage is then 64 k rows of 512 bytes (256 columns); one transfer fills two
+// k rows; the 16-byte unit at physical position pu of k row r holds logical unit pu ^ ((r & 3) << 1), which spreads
+// the four k rows that one group of 16 lanes reads with a transpose load over all banks.
+template <int BKT, bool AKM = false>
 struct DirectLoader {
     typedef DirectCfg<BKT> C;
+    static_assert(!AKM || (BKT == 64 && BM == 256), "k-major left operands: 64-wide steps of 256 columns");
     static constexpr int kWaves = kHeadThreads / 64;
     static constexpr int kBlkA = BM / C::kRowsPerBlk / kWaves, kBlkB = BN / C::kRowsPerBlk / kWaves;  // per wave and stage
     static constexpr int kStageLoads = kBlkA + kBlkB;
@@ -148,16 +159,24 @@ struct DirectLoader {
     const char *abase, *bbase;
     char* smem;
     int wave;
+    int64_t akstep;  // bytes between two k of the left operand
     uint32_t ao[kBlkA], bo[kBlkB];
 
     __device__ __forceinline__ DirectLoader(const Operand A, int m0, const Operand B, int n0, char* lds) : smem(lds) {
         const int lane = threadIdx.x & 63;
         wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: LDS targets stay scalar
         const int rr = lane / C::kChunks, pc = lane % C::kChunks;  // row inside a block, chunk position
-        abase = reinterpret_cast<const char*>(A.p + int64_t(m0) * A.ld);
+        abase = reinterpret_cast<const char*>(AKM ? A.p + m0 : A.p + int64_t(m0) * A.ld);
         bbase = reinterpret_cast<const char*>(B.p + int64_t(n0) * B.ld);
+        akstep = AKM ? A.ld * 2 : 2;
 #pragma unroll
         for (int j = 0; j < kBlkA; ++j) {
+            if constexpr (AKM) {
+                const int krow = (wave + kWaves * j) * 2 + (lane >> 5);
+                const int lu = (lane & 31) ^ ((krow & 3) << 1);  // the logical 16-byte unit this lane fetches
+                ao[j] = uint32_t((int64_t(krow) * A.ld + lu * 8) * 2);
+                continue;
+            }
             const int row = (wave + kWaves * j) * C::kRowsPerBlk + rr;
             const int kc = pc ^ C::swizzle(row);  // the logical chunk this lane fetches
             const int r = m0 + row < A.rows ? row : A.rows - 1 - m0;
@@ -190,7 +209,7 @@ struct DirectLoader {
     // transfer j of a stage (A blocks first, then B blocks)
     __device__ __forceinline__ void issue_one(int buf, int k0, int j) const {
         if (j < kBlkA)
-            transfer(abase + int64_t(k0) * 2 + ao[j], lds_base(buf) + (wave + kWaves * j) * 1024);
+            transfer(abase + int64_t(k0) * akstep + ao[j], lds_base(buf) + (wave + kWaves * j) * 1024);
         else
             transfer(bbase + int64_t(k0) * 2 + bo[j - kBlkA], lds_base(buf) + C::kDenseA + (wave + kWaves * (j - kBlkA)) * 1024);
     }
@@ -209,13 +228,13 @@ struct DirectLoader {
 
 // `prefetched`: the caller has already run DirectLoader::prologue for this tile (and nothing has
 // touched the LDS since).
-template <int DT, int BKT>
+template <int DT, int BKT, bool AKM = false>
 __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, const Operand B, int n0, int K,
                                                     f32x16 (&acc)[MB][NB], char* smem, bool prefetched) {
     typedef DirectCfg<BKT> C;
     constexpr int kStages = C::kStages, kRowBytes = C::kRowBytes;
     constexpr int kDenseA = C::kDenseA, kDenseStage = C::kDenseStage;
-    const DirectLoader<BKT> loader(A, m0, B, n0, smem);
+    const DirectLoader<BKT, AKM> loader(A, m0, B, n0, smem);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = loader.wave;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -228,6 +247,31 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
     int koff[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) koff[ks] = ((ks * 2 + hl) ^ swz) * 16;
+    // k-major left operand: a fragment (32 rows x 16 k, 8 k per lane) is two transpose loads of 8 bytes.  The lanes
+    // work in groups of 16: lane t of a group points at the 8 bytes that hold columns 4 (t % 4) .. + 3 of k row t / 4
+    // (of the group's 4 k rows), and receives column t of those 4 k rows.  Groups 0, 1 take columns 0-15, 16-31 of the
+    // block at k 0-3 (second load: 4-7), groups 2, 3 the same columns at k 8-11 (12-15).
+    int fa_km[MB];
+    if constexpr (AKM) {
+        const int t = lane & 15, g = lane >> 4;
+        const int f = (t >> 2) << 1;  // the unit swizzle of this lane's k row ((k row & 3) << 1)
+        const int lu0 = (wm * WM + 16 * (g & 1)) / 8 + ((t & 3) >> 1);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+            fa_km[mb] = (8 * (g >> 1) + (t >> 2)) * 512 + ((lu0 + 4 * mb) ^ f) * 16 + (t & 1) * 8;
+    }
+    auto read_a = [&](const char* sa, int mb, int ks) -> u32x4 {
+        if constexpr (AKM) {
+            const uint32_t at = uint32_t(reinterpret_cast<uintptr_t>(sa)) + uint32_t(fa_km[mb] + ks * 16 * 512);
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_s16x4*>(at));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<lds_s16x4*>(at + 4 * 512));
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            return __builtin_bit_cast(u32x4, both);
+        } else {
+            return *reinterpret_cast<const u32x4*>(sa + fa_row + mb * 32 * kRowBytes + koff[ks]);
+        }
+    };
 
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -241,13 +285,12 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
     // synchronises, so its MFMAs cover the refill of the freed stage and the first fragment reads of
     // the next one.  The compiler's own scheduler sinks every ds_read next to its first use (one
     // exposed LDS latency per MFMA pair), so the issue order is pinned explicitly below.
-    constexpr int kStageLoads = DirectLoader<BKT>::kStageLoads;
+    constexpr int kStageLoads = DirectLoader<BKT, AKM>::kStageLoads;
     auto load_frags = [&](int buf, int ks, u32x4(&fa)[MB], u32x4(&fb)[NB]) {
         const char* sa = smem + buf * kDenseStage;
         const char* sb = sa + kDenseA;
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-            fa[mb] = *reinterpret_cast<const u32x4*>(sa + fa_row + mb * 32 * kRowBytes + koff[ks]);
+        for (int mb = 0; mb < MB; ++mb) fa[mb] = read_a(sa, mb, ks);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
             fb[nb] = *reinterpret_cast<const u32x4*>(sb + fb_row + nb * 32 * kRowBytes + koff[ks]);
@@ -286,11 +329,11 @@ __device__ __forceinline__ void gemm_tile_nt_direct(const Operand A, int m0, con
             if (READ && i < R) {
                 // read order: fa[0], fb[0..NB-1], fa[1..MB-1]
                 if (i == 0)
-                    na[0] = *reinterpret_cast<const u32x4*>(sa + fa_row + koff[rks]);
+                    na[0] = read_a(sa, 0, rks);
                 else if (i <= NB)
                     nb_[i - 1] = *reinterpret_cast<const u32x4*>(sb + fb_row + (i - 1) * 32 * kRowBytes + koff[rks]);
                 else
-                    na[i - NB] = *reinterpret_cast<const u32x4*>(sa + fa_row + (i - NB) * 32 * kRowBytes + koff[rks]);
+                    na[i - NB] = read_a(sa, i - NB, rks);
             }
             if (NL > 0 && (i + 1) * NL / M > i * NL / M) {
                 loader.issue_one(lbuf, lk0, lfirst + issued);
@@ -450,15 +493,20 @@ __device__ __forceinline__ void gemm_tile_nt_staged(const Operand A, int m0, con
     }
 }
 
-template <int DT, int BKT>
+template <int DT, int BKT, bool AKM = false>
 __device__ __forceinline__ void gemm_tile_nt(const Operand A, int m0, const Operand B, int n0, int K,
                                              f32x16 (&acc)[MB][NB], char* smem, bool prefetched = false) {
+    if constexpr (AKM) {  // (callers of this form pad K to whole steps)
+        static_assert(TRLK_HEAD_DIRECT_LDS && BKT == 64, "k-major left operands need the direct-to-LDS loop");
+        gemm_tile_nt_direct<DT, BKT, true>(A, m0, B, n0, K, acc, smem, prefetched);
+    } else {
 #if TRLK_HEAD_DIRECT_LDS
-    if ((K & (BKT - 1)) == 0)
-        gemm_tile_nt_direct<DT, BKT>(A, m0, B, n0, K, acc, smem, prefetched);
-    else
+        if ((K & (BKT - 1)) == 0)
+            gemm_tile_nt_direct<DT, BKT>(A, m0, B, n0, K, acc, smem, prefetched);
+        else
 #endif
-        gemm_tile_nt_staged<DT>(A, m0, B, n0, K, acc, smem);
+            gemm_tile_nt_staged<DT>(A, m0, B, n0, K, acc, smem);
+    }
 }
 
 // Starts the transfers of a tile's first stages so that they overlap whatever the caller does
@@ -535,9 +583,8 @@ struct HeadArgs {
     const float* stash_in;  // backward: the same buffer, or null (recompute)
     const int32_t* stash_cols;  // backward: stash column of token n (tokens were compacted since the forward), or null
     int64_t ld_stash;
-    uint16_t* dz;        // [N, ldz]   (columns = chunk-local vocabulary index), fp16, row n scaled by dz_row_scale(g[n])
-    uint16_t* dzT;       // [chunk rows padded, ldzt], fp16, scaled by dz_scale(*g_max)
-    int64_t ldz, ldzt;
+    uint16_t* dzT;       // [chunk rows padded, ldzt] (columns = tokens), fp16, column n scaled by pow2_scale(|g[n]| * zs)
+    int64_t ldzt;
     const uint32_t* g_max;
     int sdz_token_blocks, sdz_tiles;  // stash sweep: token blocks per row group, tiles of the launch  // backward: bit pattern of max |g| over the tokens
 };
@@ -546,9 +593,15 @@ struct HeadArgs {
 // The two backward products run on fp16 operands whatever the dtype of the problem: d logits rounded to bf16 would
 // carry 8 significant bits into both gradients (relative error 3e-3), fp16 carries 11 (4e-4) at the same matrix-core
 // rate.  fp16 has 5 exponent bits, so every operand is multiplied by a power of two that puts its largest magnitude
-// into [2^13, 2^14) (exact, undone in the products' epilogue): the token-major d logits per token (|dz[n, :]| <=
-// |g[n]| * logit_scale / T), the vocabulary-major copy by the largest |g|, W^T and hidden^T of a bf16 problem by
-// their largest magnitude (bf16 -> fp16 is then exact down to 2^-31 of that maximum).
+// into [2^13, 2^14) (exact, undone in the products' epilogue): d logits per token (|dz[:, n]| <= |g[n]| * logit_scale
+// / T, so token n's column carries s_n = pow2_scale(|g[n]| * logit_scale / T) and a token whose upstream gradient is
+// a million times smaller than the largest keeps its own relative accuracy in dHidden, whose row n the epilogue
+// divides by s_n), W^T and hidden^T of a bf16 problem by their largest magnitude (bf16 -> fp16 is then exact down to
+// 2^-31 of that maximum).  The dW product sums over the tokens, so it needs the columns of d logits in ONE scale: row
+// n of hidden^T's source is multiplied by s_all / s_n on its way (s_all = the scale of the largest |g|, so the factor
+// is a power of two <= 1), which leaves dz^T[v, n] * hidden^T[h, n] in the scale s_all * s_hidden for every n.  A token
+// whose gradient is 2^-25 of the largest starts to lose bits of its hidden row there -- where its whole contribution
+// to dW is below the rounding of the fp32 sum.
 __device__ __forceinline__ float pow2_scale(float m) {
     if (!(m > 0.f) || !(m < INFINITY)) return 1.f;
     int e;
@@ -800,15 +853,12 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
     // with one scale folded into the exponent; the target's one-hot term is patched afterwards.
     const float zs = a.logit_scale * a.inv_t, zs2 = zs * kLog2e;
     const bool plain = a.softcap <= 0.f && m0 + BM <= a.c1 && a.bias == nullptr;
-    typedef Elem<TRLK_F16> EO;  // storage of both dz copies
-    const float s_all = slot_scale(a.g_max, zs);
-    float to_all[NB];  // token-major scale -> scale of the vocabulary-major copy, per token block
+    typedef Elem<TRLK_F16> EO;  // storage of dz
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         const int tok = n0 + acc_col(wn, nb, lane);
         const bool tok_ok = tok < a.N;
         const float g = tok_ok ? a.g[tok] * pow2_scale(fabsf(a.g[tok]) * zs) : 0.f;  // g carries the token's scale
-        to_all[nb] = tok_ok ? s_all / pow2_scale(fabsf(a.g[tok]) * zs) : 0.f;
         const float lzc = tok_ok ? a.log_z[tok] * kLog2e : INFINITY;  // rows beyond N: exp2(-inf) = 0
         const int64_t tg = tok_ok ? a.targets[tok] : -1;
         const int64_t rel = tg - (m0 + wm * WM);  // target row relative to this wave's rows
@@ -844,35 +894,15 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
                     d[r] = (v < a.c1 && tok_ok) ? dzv * chain : 0.f;
                 }
             }
-            // dz [token][chunk column] goes through LDS: a lane owns scattered 8-byte pieces of 32
-            // different token rows, which would reach memory as partial sectors; staged as a
-            // [token][vocabulary] tile they leave as 512-byte runs (below)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint2 w;
-                w.x = EO::pack2(d[q * 4 + 0], d[q * 4 + 1]);
-                w.y = EO::pack2(d[q * 4 + 2], d[q * 4 + 3]);
-                *reinterpret_cast<uint2*>(smem + acc_col(wn, nb, lane) * kDzLdsRow + acc_row(wm, mb, q * 4, lane) * 2) = w;
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[mb][nb][r] = d[r];  // kept for the transposed copy
+            for (int r = 0; r < 16; ++r) acc[mb][nb][r] = d[r];
         }
     }
-    __syncthreads();
-    constexpr int kChunksPerRow = BM / 8;  // 16-byte pieces per row of the staged tile (BM == BN)
-    static_assert(BM == BN, "the two staged copies of the dz tile share one LDS layout");
-#pragma unroll 4
-    for (int c = tid; c < BN * kChunksPerRow; c += kHeadThreads) {
-        const int tok_local = c / kChunksPerRow, vc = c % kChunksPerRow;
-        if (n0 + tok_local < a.N)
-            *reinterpret_cast<u32x4*>(a.dz + int64_t(n0 + tok_local) * a.ldz + vt * BM + vc * 8) =
-                *reinterpret_cast<const u32x4*>(smem + tok_local * kDzLdsRow + vc * 16);
-    }
-    __syncthreads();
     // dz^T [chunk row][token]: the lanes of a block hold consecutive tokens of one vocabulary row.
     // Neighbouring lanes swap one value each, so that the even lane owns two tokens of row r and
     // the odd lane two tokens of row r + 1; the 4-byte pieces are staged as a [vocabulary][token]
-    // tile and leave as 512-byte runs as well.
+    // tile in LDS and leave as 512-byte runs.
+    constexpr int kChunksPerRow = BN / 8;  // 16-byte pieces per row of the staged tile
     const int odd = lane & 1;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
@@ -881,7 +911,7 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
             for (int r = 0; r < 16; r += 2) {
-                const float mine0 = acc[mb][nb][r] * to_all[nb], mine1 = acc[mb][nb][r + 1] * to_all[nb];
+                const float mine0 = acc[mb][nb][r], mine1 = acc[mb][nb][r + 1];
                 const float give = odd ? mine0 : mine1;
                 const float got = __builtin_bit_cast(
                     float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, give), 0xB1 /* quad_perm 1,0,3,2 */, 0xf, 0xf, true));
@@ -900,27 +930,26 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
 }
 
 // dz pass of the backward from the forward's stashed products instead of a recompute: an
-// elementwise sweep over y[v][n] (memory bound: 4 bytes read, 2 x 2 bytes written per logit).
+// elementwise sweep over y[v][n] (memory bound: 4 bytes read, 2 bytes written per logit).
 // One workgroup = 64 vocabulary rows x 256 tokens.  A lane owns 4 consecutive tokens; a wave walks
-// over row pairs.  dz^T (vocabulary-major, like the stash) is written directly, dz (token-major)
-// through an LDS transpose.  Rows beyond the chunk and tokens beyond N are written as zeros.
+// over row pairs.  dz^T (vocabulary-major, like the stash) is written in place, each token's column in
+// that token's own scale.  Rows beyond the chunk and tokens beyond N are written as zeros.
+// (One workgroup per 64 rows x 1024 tokens, 4 KiB of a stash row per memory instruction of the workgroup and eight
+// rows in flight, measured no faster: 63.7 against 63.6 ms for a whole backward.)
 #ifndef TRLK_SDZ_TOKENS
 #define TRLK_SDZ_TOKENS 256
 #endif
-constexpr int kSdzRows = 64, kSdzTokens = TRLK_SDZ_TOKENS, kSdzLdsRow = kSdzRows * 2 + 4;  // bytes per staged token row
+constexpr int kSdzRows = 64, kSdzTokens = TRLK_SDZ_TOKENS;
 constexpr int kSdzLanesPerRow = kSdzTokens / 4, kSdzPairsPerWave = 64 / kSdzLanesPerRow;
 static_assert(kSdzTokens == 256 || kSdzTokens == 128, "a row of the tile is one wave or half a wave wide");
 // COLS: the tokens were compacted since the forward, a.stash_cols maps them to their stash columns.
 template <bool COLS>
 __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
-    typedef Elem<TRLK_F16> E;  // both dz copies are scaled fp16
-    __shared__ __attribute__((aligned(16))) char lds[kSdzTokens * kSdzLdsRow];
+    typedef Elem<TRLK_F16> E;  // dz is scaled fp16
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // consecutive tiles take consecutive token blocks of one row group: the stash rows they read and the
-    // dz^T rows they write are then neighbours in memory (6 of the sweep's 8 bytes per logit; measured 10 % faster
-    // than the other order, which puts the 128-byte pieces of the token-major dz rows next to each other instead).
-    // Consecutive workgroups go to the eight XCDs in turn: each XCD walks one contiguous eighth of the tiles
-    // (compacted tokens: 873 -> 816 us per chunk, every token: 1136 -> 1126 us).
+    // dz^T rows they write are then neighbours in memory.  Consecutive workgroups go to the eight XCDs in turn:
+    // each XCD walks one contiguous eighth of the tiles.
     const int per_xcd = int(gridDim.x) >> 3;  // (the grid is a multiple of 8)
     const int tile = int(blockIdx.x & 7) * per_xcd + int(blockIdx.x >> 3);
     if (tile >= a.sdz_tiles) return;
@@ -928,18 +957,16 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
     const int rows = a.c1 - a.c0;
     const float zs = a.logit_scale * a.inv_t, zs2 = zs * kLog2e;
     const bool plain = a.softcap <= 0.f && a.bias == nullptr;
-    float g[4], lzc[4], to_tok[4];  // g carries the scale of the vocabulary-major copy; to_tok: that scale -> the token's own
+    float g[4], lzc[4];  // g carries the token's own scale
     int64_t tg[4];
     int col[4];
     const int tl0 = (lane % kSdzLanesPerRow) * 4, sub = lane / kSdzLanesPerRow;  // first token of the lane, row pair
-    const float s_all = slot_scale(a.g_max, zs);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int tok = n0 + tl0 + j;
         const bool ok = tok < a.N;
         col[j] = (COLS && ok) ? a.stash_cols[tok] : -1;
-        g[j] = ok ? a.g[tok] * s_all : 0.f;
-        to_tok[j] = ok ? pow2_scale(fabsf(a.g[tok]) * zs) / s_all : 0.f;
+        g[j] = ok ? a.g[tok] * pow2_scale(fabsf(a.g[tok]) * zs) : 0.f;
         lzc[j] = ok ? a.log_z[tok] * kLog2e : INFINITY;
         tg[j] = ok ? a.targets[tok] - a.c0 : -1;  // chunk-local target row
     }
@@ -972,12 +999,12 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
                 }
         }
         const int rl = 2 * (wave * kSdzPairsPerWave + sub + 4 * kSdzPairsPerWave * i);  // row pair rl, rl + 1 of the 64
-        float d[2][4];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int row = r0 + rl + h;
             const f32x4 y4 = yb[i % kSdzBatch][h];
             const float bias = (!plain && a.bias != nullptr && row < rows) ? a.bias[a.c0 + row] : 0.f;
+            float d[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 float dv;
@@ -997,26 +1024,12 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
                     if (tg[j] == row) dv += g[j];
                     dv *= chain;
                 }
-                d[h][j] = (row < rows && g[j] != 0.f) ? dv : 0.f;
+                d[j] = (row < rows && g[j] != 0.f) ? dv : 0.f;
             }
             uint2 w;
-            w.x = E::pack2(d[h][0], d[h][1]);
-            w.y = E::pack2(d[h][2], d[h][3]);
+            w.x = E::pack2(d[0], d[1]);
+            w.y = E::pack2(d[2], d[3]);
             *reinterpret_cast<uint2*>(a.dzT + int64_t(row) * a.ldzt + n0 + tl0) = w;
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            *reinterpret_cast<uint32_t*>(lds + (tl0 + j) * kSdzLdsRow + rl * 2) = E::pack2(d[0][j] * to_tok[j], d[1][j] * to_tok[j]);
-    }
-    __syncthreads();
-    constexpr int kPieces = kSdzRows / 8;  // 16-byte pieces per staged token row
-#pragma unroll 2
-    for (int c = tid; c < kSdzTokens * kPieces; c += 256) {
-        const int tl = c / kPieces, pc = c % kPieces;
-        if (n0 + tl < a.N) {
-            const uint32_t* src = reinterpret_cast<const uint32_t*>(lds + tl * kSdzLdsRow + pc * 16);
-            u32x4 w = {src[0], src[1], src[2], src[3]};
-            *reinterpret_cast<u32x4*>(a.dz + int64_t(n0 + tl) * a.ldz + r0 + pc * 8) = w;
         }
     }
 }
@@ -1043,7 +1056,8 @@ struct GemmArgs {
 };
 
 // DT: dtype of the operands (the matrix-core instruction), ODT: storage dtype of `out_lp`.
-template <int DT, int MODE, int ODT>
+// AKM: A is given k-major ([K, M], leading dimension A.ld).
+template <int DT, int MODE, int ODT, bool AKM = false>
 __device__ __forceinline__ void gemm_nt_body(const GemmArgs& a, int block, char* smem) {
     typedef Elem<ODT> E;
     const int n_mt = (a.M + BM - 1) / BM, n_nt = (a.N + BN - 1) / BN;
@@ -1054,7 +1068,7 @@ __device__ __forceinline__ void gemm_nt_body(const GemmArgs& a, int block, char*
     const int wm = wave / WGN, wn = wave % WGN;
     const int m0 = tm * BM, n0 = tn * BN;
     f32x16 acc[MB][NB];
-    gemm_tile_nt<DT, TRLK_HEAD_BK_GEMM>(a.A, m0, a.B, n0, a.K, acc, smem);
+    gemm_tile_nt<DT, TRLK_HEAD_BK_GEMM, AKM>(a.A, m0, a.B, n0, a.K, acc, smem);
     const float inv_b = 1.f / slot_scale(a.max_b, 1.f);
     const float inv_common = inv_b / slot_scale(a.max_a, a.mult_a);
     // The running sum of a block is read as a whole before any of the block is written: with a load
@@ -1092,14 +1106,14 @@ __device__ __forceinline__ void gemm_nt_body(const GemmArgs& a, int block, char*
     }
 }
 
-// Two independent products in one launch: workgroups [0, grid_a) take `a` (epilogue MODE_A), the rest take `b`
-// (epilogue 0).  When the tile count of one product is not a multiple of the CU count, the other product's
+// Two independent products in one launch: workgroups [0, grid_a) take `a` (epilogue MODE_A; its left operand is
+// k-major), the rest take `b` (epilogue 0).  When the tile count of one product is not a multiple of the CU count, the other product's
 // tiles fill the CUs its last round leaves idle.  grid_a is a multiple of 8 (the XCD mapping of `b` is kept).
 template <int MODE_A, int ODT>
 TRLK_HEAD_KERNEL void gemm_nt_pair_kernel(GemmArgs a, int grid_a, GemmArgs b) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     if (int(blockIdx.x) < grid_a)
-        gemm_nt_body<TRLK_F16, MODE_A, ODT>(a, blockIdx.x, smem);
+        gemm_nt_body<TRLK_F16, MODE_A, ODT, true>(a, blockIdx.x, smem);
     else
         gemm_nt_body<TRLK_F16, 0, ODT>(b, int(blockIdx.x) - grid_a, smem);
 }
@@ -1186,9 +1200,13 @@ __global__ __launch_bounds__(256) void maxabs_f32_kernel(const float* in, int64_
 // [R, C] (ld) -> [C, ldo] with columns >= R zero-filled up to `fill`: 64 x 64 tiles through LDS.
 // TO_F16: the input is bf16 and the output fp16, multiplied by the power of two that `in_max` (the input's largest
 // magnitude) asks for.
-template <bool TO_F16>
+// ROW_G: input row r is also multiplied by s_all / pow2_scale(|row_g[r]| * zs) (0 where row_g[r] is 0), s_all from
+// `g_max`: what brings the columns of hidden^T into the scales of the d logits' columns (see above).
+template <bool TO_F16, bool ROW_G = false>
 __global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* in, int64_t ld, int R, int C, uint16_t* out,
-                                                          int64_t ldo, int64_t fill, const uint32_t* in_max) {
+                                                          int64_t ldo, int64_t fill, const uint32_t* in_max,
+                                                          const float* row_g = nullptr, const uint32_t* g_max = nullptr,
+                                                          float zs = 1.f) {
     // C, ld, ldo and fill are multiples of 8 and both matrices 16-byte aligned (the callers' operands are): a lane
     // moves 8 elements at a time.  Tile rows are skewed by 8 elements per group of 8 rows, which spreads the
     // 2-byte column reads of the second phase over all banks.
@@ -1202,11 +1220,19 @@ __global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* in, in
         const int row = hi + 32 * p, cc = lo * 8;
         u32x4 q = {0u, 0u, 0u, 0u};
         if (r0 + row < R && c0 + cc < C) q = *reinterpret_cast<const u32x4*>(in + int64_t(r0 + row) * ld + c0 + cc);
-        if (TO_F16) {
+        if (TO_F16 || ROW_G) {
+            float f = sc;
+            if (ROW_G) {
+                const float gr = r0 + row < R ? fabsf(row_g[r0 + row]) : 0.f;
+                f = gr > 0.f ? sc * (slot_scale(g_max, zs) / pow2_scale(gr * zs)) : 0.f;
+            }
             float x[8];
-            Elem<TRLK_BF16>::unpack(q, x);
+            if (TO_F16)
+                Elem<TRLK_BF16>::unpack(q, x);
+            else
+                Elem<TRLK_F16>::unpack(q, x);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) x[i] *= sc;
+            for (int i = 0; i < 8; ++i) x[i] *= f;
             q = Elem<TRLK_F16>::pack(x);
         }
         *reinterpret_cast<u32x4*>(tile + row * kStride + cc + 8 * (row >> 3)) = q;
@@ -1231,7 +1257,7 @@ int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
 // d bias[v] = sum over tokens of dz[token, v]: row sums of the transposed dz copy (padding columns are zero).
 __global__ __launch_bounds__(256) void dz_row_sum_kernel(const uint16_t* dzT, int64_t ld, int n_cols8, float* out,
-                                                         const uint32_t* g_max, float zs) {
+                                                         const float* g, int n_tokens, float zs) {
     typedef Elem<TRLK_F16> E;
     const uint16_t* row = dzT + int64_t(blockIdx.x) * ld;
     float acc = 0.f;
@@ -1240,14 +1266,17 @@ __global__ __launch_bounds__(256) void dz_row_sum_kernel(const uint16_t* dzT, in
         float x[8];
         E::unpack(w, x);
 #pragma unroll
-        for (int q = 0; q < 8; ++q) acc += x[q];
+        for (int q = 0; q < 8; ++q) {  // column n is in token n's scale
+            const int n = c * 8 + q;
+            if (n < n_tokens) acc += x[q] / pow2_scale(fabsf(g[n]) * zs);
+        }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
     __shared__ float part[4];
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
     __syncthreads();
-    if (threadIdx.x == 0) out[blockIdx.x] = (part[0] + part[1] + part[2] + part[3]) / slot_scale(g_max, zs);
+    if (threadIdx.x == 0) out[blockIdx.x] = part[0] + part[1] + part[2] + part[3];
 }
 
 // Row strides of the workspace matrices carry 128 extra bytes: their padded extents are multiples
@@ -1257,7 +1286,7 @@ constexpr int64_t kLdSkew = 64;
 struct BwdLayout {
     int64_t vpad, npad, cpad;    // padded extents (zero-filled)
     int64_t ld_v, ld_n, ld_c;    // row strides of [*, vpad], [*, npad], [*, cpad] matrices
-    size_t off_wt, off_ht, off_dz, off_dzt, off_dh, off_max, total;
+    size_t off_wt, off_ht, off_dzt, off_dh, off_max, total;
     int64_t n_chunks;
 };
 BwdLayout bwd_layout(int64_t N, int64_t V, int64_t H, int64_t chunk) {
@@ -1276,7 +1305,6 @@ BwdLayout bwd_layout(int64_t N, int64_t V, int64_t H, int64_t chunk) {
     };
     l.off_wt = take(size_t(H) * l.ld_c * 2);
     l.off_ht = take(size_t(H) * l.ld_n * 2);
-    l.off_dz = take(size_t(N) * l.ld_c * 2);
     l.off_dzt = take(size_t(l.cpad) * l.ld_n * 2);
     l.off_dh = take(size_t(N) * H * 4);
     l.n_chunks = (V + l.cpad - 1) / l.cpad;
@@ -1484,7 +1512,6 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     char* ws = static_cast<char*>(d_workspace);
     uint16_t* wt = reinterpret_cast<uint16_t*>(ws + l.off_wt);    // [H, cpad], row stride ld_c (one chunk at a time)
     uint16_t* ht = reinterpret_cast<uint16_t*>(ws + l.off_ht);    // [H, npad], row stride ld_n
-    uint16_t* dz = reinterpret_cast<uint16_t*>(ws + l.off_dz);    // [N, cpad], row stride ld_c
     uint16_t* dzt = reinterpret_cast<uint16_t*>(ws + l.off_dzt);  // [cpad, npad], row stride ld_n
     float* dh = reinterpret_cast<float*>(ws + l.off_dh);          // [N, H]
     uint32_t* maxima = reinterpret_cast<uint32_t*>(ws + l.off_max);  // [0] g, [1] hidden, [2] W
@@ -1502,11 +1529,13 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         // one scale for the whole weight: a single sweep over it instead of one per chunk
         hipLaunchKernelGGL(maxabs_bf16_kernel, dim3(unsigned(V < 4096 ? V : 4096)), dim3(256), 0, s,
                            static_cast<const uint16_t*>(d_weight), weight_stride, V, H / 8, maxima + 2);
-        hipLaunchKernelGGL(transpose16_kernel<true>, dim3((H + 63) / 64, unsigned((l.npad + 63) / 64)), dim3(256), 0, s,
-                           static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.ld_n, l.npad, max_h);
+        hipLaunchKernelGGL((transpose16_kernel<true, true>), dim3((H + 63) / 64, unsigned((l.npad + 63) / 64)), dim3(256), 0, s,
+                           static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.ld_n, l.npad, max_h, d_g_logp,
+                           max_g, logit_scale / temperature);
     } else {
-        hipLaunchKernelGGL(transpose16_kernel<false>, dim3((H + 63) / 64, unsigned((l.npad + 63) / 64)), dim3(256), 0, s,
-                           static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.ld_n, l.npad, max_h);
+        hipLaunchKernelGGL((transpose16_kernel<false, true>), dim3((H + 63) / 64, unsigned((l.npad + 63) / 64)), dim3(256), 0, s,
+                           static_cast<const uint16_t*>(d_hidden), hidden_stride, N, H, ht, l.ld_n, l.npad, max_h, d_g_logp,
+                           max_g, logit_scale / temperature);
     }
     if (int rc = launch_status("fused_head_bwd (hidden^T)")) return rc;
 
@@ -1528,9 +1557,7 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     a.stash_in = d_stash;
     a.stash_cols = d_stash_cols;
     a.ld_stash = stash_ld;
-    a.dz = dz;
     a.dzT = dzt;
-    a.ldz = l.ld_c;
     a.ldzt = l.ld_n;
     a.g_max = max_g;
     const float zs = logit_scale / temperature;  // |dz[n, v]| <= |g[n]| * zs
@@ -1561,7 +1588,7 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         if (rc) return rc;
         if (d_out_dbias) {
             hipLaunchKernelGGL(dz_row_sum_kernel, dim3(rows), dim3(256), 0, s, dzt, l.ld_n, int(l.npad / 8), d_out_dbias + c0,
-                               max_g, zs);
+                               d_g_logp, N, zs);
             if (int rc2 = launch_status("fused_head_bwd (dBias)")) return rc2;
         }
         const bool first = c0 == 0, last = c1 == vocab;
@@ -1580,7 +1607,7 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
         if (int rc2 = launch_status("fused_head_bwd (W^T)")) return rc2;
         // dHidden[N, H] += dz[N, chunk] * (W_chunk^T[H, chunk])^T
         GemmArgs gh{};
-        gh.A = Operand{dz, l.ld_c, N};
+        gh.A = Operand{dzt, l.ld_n, N};  // k-major: [chunk rows, tokens]
         gh.B = Operand{wt, l.ld_c, H};
         gh.M = N;
         gh.N = H;
