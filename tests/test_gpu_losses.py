@@ -215,7 +215,7 @@ def test_grpo_on_policy_closed_form(amd):
     want = -(adv[:, None] * mask) / mask.sum()
     torch.testing.assert_close(lp.grad, want, rtol=1e-6, atol=1e-9)
     torch.testing.assert_close(loss.detach(), -(adv[:, None] * mask).sum() / mask.sum(), rtol=1e-5, atol=1e-7)
-    assert float(metrics[4]) == 0.0
+    assert float(metrics.detach()[4]) == 0.0
 
 
 def test_group_advantages(amd):
@@ -260,7 +260,7 @@ def test_golden_dpo_compute_loss_all_loss_types(amd, skip_masked):
         loss.backward()
         want = float(g[c + "out_loss"])
         rel = 5e-2 if low else 1e-5
-        assert abs(float(loss) - want) <= rel * max(1.0, abs(want)), (case["name"], float(loss), want)
+        assert abs(float(loss.detach()) - want) <= rel * max(1.0, abs(want)), (case["name"], float(loss.detach()), want)
         assert _rel_l2(leaf.grad.float(), _t(g[c + "out_dlogits"])) < (5e-2 if low else 1e-4), case["name"]
         got = amd.dpo_metrics_to_dict(parts)
         for name, want_m in case["metrics"].items():
@@ -300,7 +300,7 @@ def test_dpo_mixin_compute_loss(amd):
                   ref_rejected_logps=_t(g[c + "ref_rejected_logps"]).to(DEV))
     loss = tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None), inputs, False)
     loss.backward()
-    assert abs(float(loss) - float(g[c + "out_loss"])) <= 1e-5 * max(1.0, abs(float(g[c + "out_loss"])))
+    assert abs(float(loss.detach()) - float(g[c + "out_loss"])) <= 1e-5 * max(1.0, abs(float(g[c + "out_loss"])))
     assert _rel_l2(leaf.grad, _t(g[c + "out_dlogits"])) < 1e-4
     got = {k: v[-1] for k, v in tr._metrics["train"].items()}
     for name, want in case["metrics"].items():
@@ -418,7 +418,7 @@ def test_golden_kto_compute_loss(amd, skip_masked):
             got = {"kl": float(parts["kl"])}
         loss.backward()
         want = float(g[c + "out_loss"])
-        assert abs(float(loss) - want) <= (5e-2 if low else 1e-5) * max(1.0, abs(want)), (case["name"], float(loss), want)
+        assert abs(float(loss.detach()) - want) <= (5e-2 if low else 1e-5) * max(1.0, abs(want)), (case["name"], float(loss.detach()), want)
         assert _rel_l2(leaf.grad.float(), _t(g[c + "out_dlogits"])) < (5e-2 if low else 1e-4), case["name"]
         if skip_masked:
             assert set(got) == set(case["metrics"]), (case["name"], sorted(got))
@@ -533,7 +533,7 @@ def test_golden_dpo_compute_loss(amd):
             _t(g[c + "ref_chosen_logps"]).to(DEV), _t(g[c + "ref_rejected_logps"]).to(DEV), case["beta"], True)
         loss.backward()
         want = float(g[c + "out_loss"])
-        assert abs(float(loss) - want) <= (2e-2 if low else 1e-5) * max(1.0, abs(want)), case["name"]
+        assert abs(float(loss.detach()) - want) <= (2e-2 if low else 1e-5) * max(1.0, abs(want)), case["name"]
         assert _rel_l2(leaf.grad.float(), _t(g[c + "out_dlogits"])) < (2e-2 if low else 1e-4), case["name"]
         for name in ("rewards/chosen", "rewards/rejected", "rewards/accuracies", "rewards/margins", "logps/chosen",
                      "logps/rejected", "entropy"):
@@ -543,7 +543,7 @@ def test_golden_dpo_compute_loss(amd):
                 continue  # ties / near-ties between chosen and rejected rewards: decided by rounding noise
             assert abs(float(named[name]) - want_m) <= tol, (case["name"], name, float(named[name]), want_m)
         if case.get("ref_equal") and not low:
-            assert abs(float(loss) - math.log(2.0)) < 1e-6
+            assert abs(float(loss.detach()) - math.log(2.0)) < 1e-6
 
 
 def test_dpo_against_oracle_config2_shape_subsample(amd):
@@ -567,7 +567,7 @@ def test_dpo_against_oracle_config2_shape_subsample(amd):
     leaf = logits.to(DEV).requires_grad_(True)
     loss, named = amd.dpo_loss_from_logits(leaf, ids.to(DEV), cm.to(DEV), ref[:P].to(DEV), ref[P:].to(DEV), 0.1)
     loss.backward()
-    assert abs(float(loss) - float(oloss)) <= 1e-3 * abs(float(oloss))
+    assert abs(float(loss.detach()) - float(oloss.detach())) <= 1e-3 * abs(float(oloss.detach()))
     torch.testing.assert_close(named["sequence_logps"].cpu(), seq.detach(), rtol=1e-3, atol=2e-3 * 30)
     assert _rel_l2(leaf.grad.float(), of.grad) < 3e-3
     assert torch.count_nonzero(leaf.grad[:, -1]) == 0
@@ -596,7 +596,7 @@ def test_dpo_full_size_config2_closed_form_and_properties(amd):
     seq = amd.dpo_sequence_logps(logits, ids, cm)
     logits.requires_grad_(True)
     loss, parts = amd.dpo_compute_loss(logits, ids, cm, seq[:P], seq[P:], beta=beta)
-    assert abs(float(loss) - math.log(2.0)) < 1e-6
+    assert abs(float(loss.detach()) - math.log(2.0)) < 1e-6
     loss.backward()
     grad = logits.grad
     shift = cm[:, 1:].bool()
@@ -625,12 +625,12 @@ def test_golden_rloo_compute_loss(amd):
                                            _t(g[c + "advantages"]).to(DEV), case["eps_low"], case["eps_high"])
         loss.backward()
         want = float(g[c + "out_loss"])
-        assert abs(float(loss) - want) <= 1e-5 * max(1.0, abs(want))
+        assert abs(float(loss.detach()) - want) <= 1e-5 * max(1.0, abs(want))
         assert _rel_l2(leaf.grad, _t(g[c + "out_dlogits"])) < 1e-4
         from trl_amd.trainer.rloo_trainer import RLOO_METRIC_NAMES
 
         for i, name in enumerate(RLOO_METRIC_NAMES):
-            assert abs(float(metrics[i]) - case["metrics"][name]) <= 1e-6, name
+            assert abs(float(metrics.detach()[i]) - case["metrics"][name]) <= 1e-6, name
     r = torch.tensor([1.0, 2.0, 4.0, 0.5, float("nan"), 2.5])
     torch.testing.assert_close(amd.rloo_advantages(r.to(DEV), 3).cpu(), oracle.rloo_advantages(r, 3))
 
@@ -663,7 +663,7 @@ def test_rloo_mixin_compute_loss(amd, skip_masked):
         loss = tr._compute_loss(lambda **kw: SimpleNamespace(logits=leaf, aux_loss=None), inputs)
         loss.backward()
         want = float(g[c + "out_loss"])
-        assert abs(float(loss) - want) <= 1e-5 * max(1.0, abs(want))
+        assert abs(float(loss.detach()) - want) <= 1e-5 * max(1.0, abs(want))
         assert _rel_l2(leaf.grad, _t(g[c + "out_dlogits"])) < 1e-4
         got = {k: v[-1] for k, v in tr._metrics["train"].items()}
         for name, want_m in case["metrics"].items():
@@ -708,7 +708,7 @@ def test_multimodal_sub_batches_through_the_logprob_method(amd):
                       pixel_values=pixels, image_grid_thw=grid, num_images=num_images)
         seen.clear()
         loss = tr._compute_loss(model, inputs)
-        assert seen == [(4, 20, 4)] and math.isfinite(float(loss))
+        assert seen == [(4, 20, 4)] and math.isfinite(float(loss.detach()))
 
 
 @pytest.mark.parametrize("single_pass", [False, True])
