@@ -48,8 +48,8 @@ MEASURED_TRAFFIC_BYTES = {
     ("K3", "dpo_c2", None): (2 * 6608991 + 32838146) * 1024,
     ("K1", "logp_c1", None): (2 * 128206 + 192) * 1024,
     # (the forward's operand re-reads vary from launch to launch with how closely the workgroups of an XCD stay in
-    # step: 55.4-68.0 M KiB of fetches over three launches; the stash itself is 19.49 M KiB of writes)
-    ("head_fwd", "head_c5", "dapo"): (2 * 29849519 + 19491843) * 1024,  # --only-leg head_fwd_stash
+    # step: 59.7-70.4 M KiB of fetches over four launches; the stash itself is 10.04 M KiB of writes)
+    ("head_fwd", "head_c5", "dapo"): (2 * 31333262 + 10492504) * 1024,  # --only-leg head_fwd_stash
 }
 # the loss type changes per-row scalars only: the same rows are read and written, by the same launches
 for _k in ("K3", "K7"):
@@ -339,7 +339,7 @@ def bench_head(args, w):
         "data": "synthetic",
         "config": {"workload": args.workload, "description": w["desc"], "tokens": N, "hidden": H, "vocab": V,
                    "backward_chunk_rows": HEAD_CHUNK,
-                   "backward_logits": "stashed by the forward (fp32 [V, N])" if stash else "recomputed per chunk",
+                   "backward_logits": "softmax numerators stashed by the forward (fp16, 2.07 bytes per logit)" if stash else "recomputed per chunk",
                    "tokens_with_gradient": int(mask.sum()),
                    "loss_type": args.loss_type, "loss": float(loss.detach())},
         # the dominant kernel: the forward sweep (2*N*H*V flop per launch; the event-timed interval also holds its

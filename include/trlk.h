@@ -270,13 +270,18 @@ int trlk_rloo_loss(const float* d_token_logp, const float* d_mask, const float* 
  */
 size_t trlk_fused_head_fwd_workspace_bytes(int64_t n_tokens);
 
-/* Optional stash of the forward's raw products y = hidden @ weight^T (fp32, vocabulary-major:
- * [vocab rounded up to 256, *out_ld], *out_ld = n_tokens rounded up to 256).  A forward that is given
- * the buffer (d_out_stash, stash_ld) fills it; a backward that is given the same buffer (d_stash)
- * derives dz from it in one memory-bound sweep instead of recomputing the chunk's logits on the
- * matrix cores (a third of the backward's work).  No counterpart in the reference, which always
- * recomputes (trl/trainer/utils.py:1385-1399): it trades vocab * n_tokens * 4 bytes held between
- * forward and backward for that recompute.  Returns the buffer size in bytes.
+/* Optional stash of the forward's softmax numerators: for every logit exp(z - reference) as fp16, where the
+ * reference is the running maximum the forward held when it summed that part of the row (kept beside the
+ * numerators, one fp32 per 64 logits), plus the target's logit of every token.  The layout is the library's own
+ * (vocabulary-major, rows of *out_ld tokens, *out_ld = n_tokens rounded up to 256; `stash_ld` below is that number).
+ * A forward that is given the buffer (d_out_stash, stash_ld) fills it; a backward that is given the same buffer
+ * (d_stash), `vocab` and the other arguments of that forward derives dz from it in one memory-bound sweep (one
+ * multiplication per logit) instead of recomputing the chunk's logits on the matrix cores (a third of the backward's
+ * work).  fp16 keeps 11 significant bits of every probability down to 2^-29 of the row's running maximum and nothing
+ * below 2^-39 of it: what dz keeps anyway once it is rounded to fp16 for the two products.  No counterpart in the
+ * reference, which always recomputes (trl/trainer/utils.py:1385-1399): it trades about vocab * n_tokens * 2.07 bytes
+ * held between forward and backward for that recompute.  Returns the buffer size in bytes; the buffer must be
+ * 16-byte aligned.
  */
 size_t trlk_fused_head_stash_bytes(int64_t n_tokens, int64_t vocab, int64_t* out_ld);
 
@@ -284,7 +289,7 @@ int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, const int64_
                         int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                         int64_t weight_stride, float temperature, float final_logit_softcapping, float logit_scale,
                         const float* d_bias, float* d_out_logp, float* d_out_entropy, float* d_out_log_z,
-                        float* d_out_target_is_max, float* d_out_stash, int64_t stash_ld, int32_t* d_error_flag,
+                        float* d_out_target_is_max, void* d_out_stash, int64_t stash_ld, int32_t* d_error_flag,
                         void* d_workspace, size_t workspace_bytes, trlk_stream_t stream);
 
 /* Backward of the above w.r.t. hidden and weight for an upstream gradient on the log-probs
@@ -310,7 +315,7 @@ int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, const int64_
                         int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                         int64_t weight_stride, float temperature, float final_logit_softcapping, float logit_scale,
                         const float* d_bias, const float* d_log_z, const float* d_g_logp, int64_t chunk_size,
-                        const float* d_stash, int64_t stash_ld, const int32_t* d_stash_cols, void* d_out_dhidden,
+                        const void* d_stash, int64_t stash_ld, const int32_t* d_stash_cols, void* d_out_dhidden,
                         void* d_out_dweight, float* d_out_dbias, void* d_workspace, size_t workspace_bytes,
                         trlk_stream_t stream);
 

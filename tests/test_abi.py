@@ -117,7 +117,7 @@ def test_host_side_argument_validation():
     assert head_fwd(stash=fake16, stash_ld=300) == -4 and "stash" in _lib.last_error()
     assert head_fwd(ws_bytes=16) == -6
     ld = ctypes.c_int64(0)
-    assert lib.trlk_fused_head_stash_bytes(300, 1000, ctypes.addressof(ld)) == 1024 * 512 * 4 and ld.value == 512
+    assert lib.trlk_fused_head_stash_bytes(300, 1000, ctypes.addressof(ld)) == (1024 // 4 + 1024 // 128 + 1) * 512 * 8 and ld.value == 512
     assert lib.trlk_fused_head_bwd(fake16, fake16, fake, _lib.BF16, 300, 1000, 64, 64, 64, 1.0, 0.0, 1.0, None, fake, fake,
                                    256, fake16, 256, None, fake16, fake16, None, fake16, 1 << 40, None) == -4
     assert lib.trlk_fused_head_bwd(fake16, fake16, fake, _lib.BF16, 300, 1000, 64, 64, 64, 1.0, 0.0, 1.0, None, fake, fake,

@@ -198,9 +198,9 @@ def test_fused_head_with_bias(amd, n, h, v, chunk, softcap, scale):
     (1, 8, 3, 8192, None, 1.0, False),
 ])
 def test_backward_from_stashed_products_equals_recompute(amd, monkeypatch, n, h, v, chunk, softcap, scale, bias):
-    """The backward fed by the forward's stashed products gives the recompute path's gradients (same
-    accumulators, same dz arithmetic: equal up to the order of fp32 operations), and the forward's outputs do
-    not depend on stashing."""
+    """The backward fed by the forward's stashed softmax numerators gives the recompute path's gradients (same
+    accumulators; the numerators carry fp16's 11 bits, like dz itself), and the forward's outputs do not depend on
+    stashing."""
     g = torch.Generator().manual_seed(n * 3 + v)
     hidden = torch.randn(n, h, generator=g).bfloat16().to(DEV)
     weight = (torch.randn(v, h, generator=g) * (2.0 / h**0.5)).bfloat16().to(DEV)
@@ -225,7 +225,10 @@ def test_backward_from_stashed_products_equals_recompute(amd, monkeypatch, n, h,
         assert torch.count_nonzero(got_all[2][gout == 0]) == 0, key  # no gradient for tokens without an upstream one
         for got, want in zip(got_all[2:], want_all[2:]):
             if want is not None:
-                assert _rel_l2(got.float(), want.float()) < 2e-3, (key, _rel_l2(got.float(), want.float()))
+                # (a handful of bf16 outputs: one flipped last bit is already 3e-3 of the norm)
+                one_ulp = bool(((got.float() - want.float()).abs() <= want.float().abs() * 2.0**-7).all())
+                assert _rel_l2(got.float(), want.float()) < 2e-3 or (got.numel() <= 64 and one_ulp), (
+                    key, _rel_l2(got.float(), want.float()))
     monkeypatch.setenv("TRL_AMD_HEAD_DROP_ZERO_GRAD", "1")
     hh, ww = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
     lp, _ = amd._ChunkedLogProbFunction.apply(hh, ww, labels, 0.9, chunk, softcap, scale)
@@ -233,9 +236,12 @@ def test_backward_from_stashed_products_equals_recompute(amd, monkeypatch, n, h,
     assert torch.count_nonzero(hh.grad) == 0 and torch.count_nonzero(ww.grad) == 0
     # the op rejects a stash of the wrong shape
     lp, ent, log_z, _, saved = amd.ops.fused_head_fwd(hidden, weight, labels, 0.9, 0.0, 1.0, None, True)
-    assert saved.shape == ((v + 255) // 256 * 256, (n + 255) // 256 * 256)
+    vpad = (v + 255) // 256 * 256
+    assert saved.shape == (vpad // 4 + vpad // 128 + 1, (n + 255) // 256 * 256, 4) and saved.dtype == torch.float16
     with pytest.raises(ValueError):
         amd.ops.fused_head_bwd(hidden, weight, labels, 0.9, 0.0, 1.0, log_z, gout, chunk, None, saved[:, :128])
+    with pytest.raises(ValueError):
+        amd.ops.fused_head_bwd(hidden, weight, labels, 0.9, 0.0, 1.0, log_z, gout, chunk, None, saved[:-1])
 
 
 def test_masked_rows_and_scatter(amd):

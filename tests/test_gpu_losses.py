@@ -541,7 +541,8 @@ def test_golden_dpo_compute_loss(amd):
             tol = (0.15 if low else 1e-5) * max(1.0, abs(want_m))  # bf16 reference sums bf16-rounded log-probs
             if name == "rewards/accuracies" and (low or case.get("ref_equal")):
                 continue  # ties / near-ties between chosen and rejected rewards: decided by rounding noise
-            assert abs(float(named[name]) - want_m) <= tol, (case["name"], name, float(named[name]), want_m)
+            got_m = float(named[name].detach())
+            assert abs(got_m - want_m) <= tol, (case["name"], name, got_m, want_m)
         if case.get("ref_equal") and not low:
             assert abs(float(loss.detach()) - math.log(2.0)) < 1e-6
 

@@ -563,6 +563,28 @@ inline int xcd_patch_grid(int n_a, int n_b) {
     return 8 * ((n_a / 8) * n_b + ((n_a % 8) * n_b + 7) / 8);
 }
 
+// What a forward keeps for the backward when it is given a stash: for every logit its softmax numerator
+//   e[v][n] = exp2(z[v][n] * log2(e) - ref) * 2^15   as fp16,   0 < e <= 2^15,
+// where `ref` is the integer reference exponent that the lane which owned the logit held when it summed the tile
+// (the running maximum of its part of the row, rounded up).  One reference covers the 64 rows of a 128-row block
+// whose row quad (v / 4) has the same parity, for one token.  The backward's sweep turns a numerator into the
+// probability with one multiplication: p = e * exp2(ref - 15 - log_z * log2(e)).  fp16 keeps 11 significant bits of
+// every numerator down to 2^-29 of the running maximum and flushes below 2^-39 of it: the same accuracy d logits
+// has after it is rounded to fp16 for the products, at half the bytes of the raw fp32 products.
+//   quads  [vpad / 4][ld] x 8 bytes: the 4 rows of a quad for one token (rows are the vocabulary, vpad = V rounded up
+//          to the tile; the accumulator layout gives a lane 4 consecutive rows of one token)
+//   refs   [vpad / 128][2][ld] fp32: reference exponent of (128-row block, parity of the row quad, token)
+//   zt     [ld] fp32: the target's logit z (a soft-capped head needs it for the chain factor of the one-hot term)
+struct StashView {
+    char* base;
+    int64_t ld;    // tokens per row (>= N rounded up to the tile, or any with stash_cols)
+    int64_t vpad;  // vocabulary rows the forward covered
+    __host__ __device__ static int64_t rows8(int64_t vpad) { return vpad / 4 + vpad / 128 + 1; }  // rows of ld x 8 bytes
+    __host__ __device__ uint2* quads() const { return reinterpret_cast<uint2*>(base); }
+    __host__ __device__ float* refs() const { return reinterpret_cast<float*>(base + (vpad / 4) * ld * 8); }
+    __host__ __device__ float* zt() const { return reinterpret_cast<float*>(base + (vpad / 4 + vpad / 128) * ld * 8); }
+};
+
 struct HeadArgs {
     const uint16_t* hidden;  // [N, H]
     const uint16_t* weight;  // [V, H]
@@ -579,10 +601,8 @@ struct HeadArgs {
     const float* log_z;  // [N]
     const float* g;      // [N] upstream d loss / d logp
     int c0, c1;          // vocabulary rows of this chunk
-    float* stash;        // forward: raw products y[v][n], [V padded to BM, ld_stash] (vocabulary-major), or null
-    const float* stash_in;  // backward: the same buffer, or null (recompute)
+    StashView stash;     // forward (written) and backward (read): the softmax numerators, or base == null
     const int32_t* stash_cols;  // backward: stash column of token n (tokens were compacted since the forward), or null
-    int64_t ld_stash;
     uint16_t* dzT;       // [chunk rows padded, ldzt] (columns = tokens), fp16, column n scaled by pow2_scale(|g[n]| * zs)
     int64_t ldzt;
     const uint32_t* g_max;
@@ -621,7 +641,9 @@ __device__ __forceinline__ float head_z(float y, const HeadArgs& a) {
     return y * a.inv_t;
 }
 
-template <int DT>
+constexpr float kStashExp = 15.f;  // the numerators are summed and stashed times 2^15 (fp16's range above 1)
+
+template <int DT, bool STASH>
 TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int n_tb = (a.N + BN - 1) / BN;
@@ -657,23 +679,15 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
         gemm_tile_nt<DT, TRLK_HEAD_BK_FWD>(W, m0, Hd, n0, a.H, acc, smem, true);
         // the next tile's first stages travel while this tile's logits are reduced (registers only)
         if (vt + 1 < vt1) gemm_tile_prefetch<TRLK_HEAD_BK_FWD>(W, m0 + BM, Hd, n0, a.H, smem);
-        if (a.stash != nullptr) {
-            // The tile's raw products go to memory for the backward (vocabulary-major, fp32): for one
-            // accumulator register the 32 lanes of a half-wave hold 32 consecutive tokens of one
-            // vocabulary row = one 128-byte line per store (plain stores: measured 0.5 % ahead of non-temporal
-            // ones over the whole sweep).  The buffer is padded to whole tiles.
+        // Stash: for one accumulator quad (4 consecutive vocabulary rows of one token per lane) the 32 lanes of a
+        // half-wave hold 32 consecutive tokens = 256 contiguous bytes per store.  The buffer is padded to whole tiles.
+        char* stash_blk = nullptr;   // uniform
+        uint32_t stash_lane = 0;     // byte offset of the lane (the entry point bounds ld so that it fits)
+        if constexpr (STASH) {
             const int uw = __builtin_amdgcn_readfirstlane(wave);
-            const int uwm = uw / WGN, uwn = uw % WGN;
-            const uint32_t lane_off = uint32_t((lane >> 5) * 4) * uint32_t(a.ld_stash) + uint32_t(lane & 31);
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-                    float* blk = a.stash + int64_t(m0 + uwm * WM + mb * 32) * a.ld_stash + (n0 + uwn * WN + nb * 32);
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        blk[int64_t((r >> 2) * 8 + (r & 3)) * a.ld_stash + lane_off] = acc[mb][nb][r];
-                }
+            stash_blk = reinterpret_cast<char*>(a.stash.quads() + int64_t(m0 / 4 + (uw / WGN) * (WM / 4)) * a.stash.ld +
+                                                (n0 + (uw % WGN) * WN));
+            stash_lane = (uint32_t(lane >> 5) * uint32_t(a.stash.ld) + uint32_t(lane & 31)) * 8u;
         }
         const bool partial_tile = m0 + BM > a.V;
         // Common case (no soft-capping, tile inside the vocabulary): z = y * zs with one positive
@@ -713,28 +727,42 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
                 ref[nb] = need;
                 rr[nb] = need;
             }
+            if constexpr (STASH) {
+                const int tcol = n0 + acc_col(wn, nb, lane);
+                a.stash.refs()[(int64_t(m0 / 128 + wm) * 2 + (lane >> 5)) * a.stash.ld + tcol] = rr[nb];
+            }
+            // numerators times 2^15 (exact; S and U carry the factor until they are written out), with or without a
+            // stash: the outputs must not depend on stashing
+            const float rsub = rr[nb] - kStashExp;
             float s = 0.f, u = 0.f;
-            if (plain) {
+            auto sum_tile = [&](auto is_plain) {
+                constexpr bool kPlain = decltype(is_plain)::value;
+                const float mul = kPlain ? zs2 : kLog2e;  // general path: the accumulators hold z itself by now
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const float y = acc[mb][nb][r];
-                        const float e = fast_exp2(fmaf(y, zs2, -rr[nb]));
-                        s += e;
-                        u = fmaf(e, y, u);
+                    for (int q = 0; q < 4; ++q) {
+                        float e[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float y = acc[mb][nb][q * 4 + i];
+                            e[i] = fast_exp2(fmaf(y, mul, -rsub));
+                            s += e[i];
+                            u = (!kPlain && y == -INFINITY) ? u : fmaf(e[i], y, u);
+                        }
+                        if constexpr (STASH) {
+                            uint2 w;
+                            w.x = Elem<TRLK_F16>::pack2(e[0], e[1]);
+                            w.y = Elem<TRLK_F16>::pack2(e[2], e[3]);
+                            *reinterpret_cast<uint2*>(stash_blk + ((mb * 8 + q * 2) * a.stash.ld + nb * 32) * 8 + stash_lane) = w;
+                        }
                     }
+            };
+            if (plain) {
+                sum_tile(std::true_type{});
                 u *= zs;
             } else {
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const float z = acc[mb][nb][r];
-                        const float e = fast_exp2(fmaf(z, kLog2e, -rr[nb]));
-                        s += e;
-                        u = (z == -INFINITY) ? u : fmaf(e, z, u);
-                    }
+                sum_tile(std::false_type{});
             }
             S[nb] += s;
             U[nb] += u;
@@ -768,8 +796,8 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
         const int part = wm * 2 + (lane >> 5);
         float* dst = sm + (part * BN + col) * 4;
         dst[0] = ref[nb];
-        dst[1] = S[nb];
-        dst[2] = U[nb];
+        dst[1] = S[nb] * 0x1p-15f;
+        dst[2] = U[nb] * 0x1p-15f;
         dst[3] = zmax[nb];
     }
     __syncthreads();
@@ -803,7 +831,7 @@ __global__ void head_fill_kernel(float* p, int64_t n, float v) {
 // merges the vocabulary splits of every token: logp, entropy, log_z
 __global__ void head_merge_kernel(const float* partial, const float* tgt, const int64_t* targets, int N, int V,
                                   int v_splits, float* logp, float* entropy, float* log_z, float* target_is_max,
-                                  int32_t* error_flag) {
+                                  int32_t* error_flag, float* stash_zt) {
     const int n = blockIdx.x * blockDim.x + threadIdx.x;
     if (n >= N) return;
     const float* p = partial + int64_t(n) * v_splits * 4;
@@ -827,6 +855,7 @@ __global__ void head_merge_kernel(const float* partial, const float* tgt, const 
         lp = tgt[n] - lz;
     }
     logp[n] = lp;
+    if (stash_zt) stash_zt[n] = tgt[n];
     entropy[n] = lz - U / S;
     log_z[n] = lz;
     // 1 if the target holds the row maximum, i.e. argmax(logits) == target up to ties
@@ -929,23 +958,17 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
     }
 }
 
-// dz pass of the backward from the forward's stashed products instead of a recompute: an
-// elementwise sweep over y[v][n] (memory bound: 4 bytes read, 2 bytes written per logit).
-// One workgroup = 64 vocabulary rows x 256 tokens.  A lane owns 4 consecutive tokens; a wave walks
-// over row pairs.  dz^T (vocabulary-major, like the stash) is written in place, each token's column in
-// that token's own scale.  Rows beyond the chunk and tokens beyond N are written as zeros.
-// (One workgroup per 64 rows x 1024 tokens, 4 KiB of a stash row per memory instruction of the workgroup and eight
-// rows in flight, measured no faster: 63.7 against 63.6 ms for a whole backward.)
-#ifndef TRLK_SDZ_TOKENS
-#define TRLK_SDZ_TOKENS 256
-#endif
-constexpr int kSdzRows = 64, kSdzTokens = TRLK_SDZ_TOKENS;
-constexpr int kSdzLanesPerRow = kSdzTokens / 4, kSdzPairsPerWave = 64 / kSdzLanesPerRow;
-static_assert(kSdzTokens == 256 || kSdzTokens == 128, "a row of the tile is one wave or half a wave wide");
+// dz pass of the backward from the forward's stashed softmax numerators instead of a recompute: an
+// elementwise sweep (memory bound: 2 bytes read, 2 bytes written per logit, one multiplication each).
+// One workgroup = 128 vocabulary rows x 256 tokens.  A lane owns 4 consecutive tokens, a wave 32 rows = 8 row quads
+// whose 16 loads (32 bytes per quad and lane: 4 tokens x 4 rows) are all issued before the first result is used.
+// dz^T (vocabulary-major, like the stash) is written in place, each token's column in that token's own scale.
+// Rows beyond the chunk and tokens beyond N are written as zeros.
+constexpr int kSdzRows = 128, kSdzTokens = 256, kSdzQuads = kSdzRows / 4 / 4;  // quads per wave
 // COLS: the tokens were compacted since the forward, a.stash_cols maps them to their stash columns.
 template <bool COLS>
 __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
-    typedef Elem<TRLK_F16> E;  // dz is scaled fp16
+    typedef Elem<TRLK_F16> E;  // the numerators and dz are fp16
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // consecutive tiles take consecutive token blocks of one row group: the stash rows they read and the
     // dz^T rows they write are then neighbours in memory.  Consecutive workgroups go to the eight XCDs in turn:
@@ -955,76 +978,93 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
     if (tile >= a.sdz_tiles) return;
     const int n0 = (tile % a.sdz_token_blocks) * kSdzTokens, r0 = (tile / a.sdz_token_blocks) * kSdzRows;  // r0: chunk-local row
     const int rows = a.c1 - a.c0;
-    const float zs = a.logit_scale * a.inv_t, zs2 = zs * kLog2e;
-    const bool plain = a.softcap <= 0.f && a.bias == nullptr;
-    float g[4], lzc[4];  // g carries the token's own scale
-    int64_t tg[4];
-    int col[4];
-    const int tl0 = (lane % kSdzLanesPerRow) * 4, sub = lane / kSdzLanesPerRow;  // first token of the lane, row pair
+    const float zs = a.logit_scale * a.inv_t;
+    const int64_t ld = a.stash.ld;
+    const int tl0 = lane * 4;  // first token of the lane
+    float ngc[4], lzc[4];  // -g * zs in the token's own scale; log_z in base 2
+    int tg[4], col[4];     // chunk-local target row (or -1); stash column
+    bool live[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int tok = n0 + tl0 + j;
         const bool ok = tok < a.N;
-        col[j] = (COLS && ok) ? a.stash_cols[tok] : -1;
-        g[j] = ok ? a.g[tok] * pow2_scale(fabsf(a.g[tok]) * zs) : 0.f;
+        col[j] = ok ? (COLS ? a.stash_cols[tok] : tok) : -1;
+        const float g = ok ? a.g[tok] : 0.f;
+        live[j] = g != 0.f;
+        ngc[j] = -g * pow2_scale(fabsf(g) * zs) * zs;
         lzc[j] = ok ? a.log_z[tok] * kLog2e : INFINITY;
-        tg[j] = ok ? a.targets[tok] - a.c0 : -1;  // chunk-local target row
+        const int64_t t = ok ? a.targets[tok] - a.c0 : -1;
+        tg[j] = (t >= 0 && t < rows) ? int(t) : -1;
     }
-    const bool contiguous = COLS && col[0] >= 0 && col[1] == col[0] + 1 && col[2] == col[0] + 2 && col[3] == col[0] + 3;
-    // The loads of kSdzBatch row pairs are issued before any of their results is used or stored: with
-    // one pair (32 bytes per lane) in flight the sweep is bound by memory latency, not bandwidth.
-    constexpr int kIters = kSdzRows / (8 * kSdzPairsPerWave), kSdzBatch = 4;
-    static_assert(kIters % kSdzBatch == 0, "row pairs per lane");
-    f32x4 yb[kSdzBatch][2];
+    const bool contiguous = !COLS || (col[0] >= 0 && col[1] == col[0] + 1 && col[2] == col[0] + 2 && col[3] == col[0] + 3);
+    const int first_col = COLS ? col[0] : n0 + tl0;  // (tokens beyond N of the last block are inside the padded row)
+    // the numerators of the wave's 8 quads
+    const int row_w = r0 + wave * (kSdzRows / 4);                         // chunk-local first row of the wave
+    const uint2* qrow = a.stash.quads() + int64_t((a.c0 + row_w) / 4) * ld;  // (chunks and tiles start on whole 128-row blocks)
+    uint2 eb[kSdzQuads][4];
 #pragma unroll
-    for (int i = 0; i < kIters; ++i) {
-        if (i % kSdzBatch == 0) {
+    for (int qi = 0; qi < kSdzQuads; ++qi) {
+        const uint2* src = qrow + int64_t(qi) * ld;
+        if (contiguous) {
+            typedef uint32_t u32x4_8 __attribute__((ext_vector_type(4), aligned(8)));
+            const u32x4_8 lo = __builtin_nontemporal_load(reinterpret_cast<const u32x4_8*>(src + first_col));
+            const u32x4_8 hi = __builtin_nontemporal_load(reinterpret_cast<const u32x4_8*>(src + first_col + 2));
+            eb[qi][0] = make_uint2(lo.x, lo.y);
+            eb[qi][1] = make_uint2(lo.z, lo.w);
+            eb[qi][2] = make_uint2(hi.x, hi.y);
+            eb[qi][3] = make_uint2(hi.z, hi.w);
+        } else {
 #pragma unroll
-            for (int ii = 0; ii < kSdzBatch; ++ii)
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const int row = r0 + 2 * (wave * kSdzPairsPerWave + sub + 4 * kSdzPairsPerWave * (i + ii)) + h;
-                    const float* srow = a.stash_in + int64_t(a.c0 + row) * a.ld_stash;
-                    f32x4 y4;
-                    if constexpr (!COLS) {
-                        y4 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(srow + n0 + tl0));
-                    } else if (contiguous) {  // the usual case: the lane's 4 tokens were neighbours in the forward too
-                        typedef float f32x4_dword_aligned __attribute__((ext_vector_type(4), aligned(4)));
-                        y4 = *reinterpret_cast<const f32x4_dword_aligned*>(srow + col[0]);
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) y4[j] = col[j] >= 0 ? __builtin_nontemporal_load(srow + col[j]) : 0.f;
-                    }
-                    yb[ii][h] = y4;
-                }
+            for (int j = 0; j < 4; ++j) eb[qi][j] = col[j] >= 0 ? src[col[j]] : make_uint2(0u, 0u);
         }
-        const int rl = 2 * (wave * kSdzPairsPerWave + sub + 4 * kSdzPairsPerWave * i);  // row pair rl, rl + 1 of the 64
+    }
+    // reference exponents of the two quad parities -> the factor that turns a numerator into -g * zs * p
+    const float* refs = a.stash.refs() + int64_t((a.c0 + row_w) / 128) * 2 * ld;
+    float rf[2][4], pf[2][4];  // p = e * pf
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int row = r0 + rl + h;
-            const f32x4 y4 = yb[i % kSdzBatch][h];
-            const float bias = (!plain && a.bias != nullptr && row < rows) ? a.bias[a.c0 + row] : 0.f;
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int cj = COLS ? col[j] : first_col + j;
+            rf[h][j] = (COLS && cj < 0) ? 0.f : refs[int64_t(h) * ld + cj];
+            pf[h][j] = fast_exp2(rf[h][j] - kStashExp - lzc[j]);
+        }
+    const bool capped = a.softcap > 0.f;
+    float zt[4] = {0.f, 0.f, 0.f, 0.f};
+    if (capped) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) zt[j] = col[j] >= 0 ? a.stash.zt()[col[j]] : 0.f;
+    }
+    const float th_mul = capped ? 1.f / (a.inv_t * a.softcap) : 0.f;  // tanh(.) of a soft-capped logit = z * T / cap
+#pragma unroll
+    for (int qi = 0; qi < kSdzQuads; ++qi) {
+        const int h = qi & 1;  // (the wave's first quad is even)
+        float e[4][4];         // [token][row of the quad]
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            E::unpack2(eb[qi][j].x, &e[j][0]);
+            E::unpack2(eb[qi][j].y, &e[j][2]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = row_w + qi * 4 + i;
             float d[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
+                const float p = e[j][i] * pf[h][j];
                 float dv;
-                if (plain) {
-                    const float ngc = -g[j] * zs;
-                    dv = ngc * fast_exp2(fmaf(y4[j], zs2, -lzc[j]));
-                    if (tg[j] == row) dv -= ngc;
+                if (!capped) {
+                    dv = ngc[j] * p;
+                    if (tg[j] == row) dv -= ngc[j];
                 } else {
-                    float y = (y4[j] + bias) * a.logit_scale;
-                    float chain = zs;
-                    if (a.softcap > 0.f) {
-                        const float th = tanhf(y / a.softcap);
-                        y = th * a.softcap;
-                        chain *= 1.f - th * th;
-                    }
-                    dv = -g[j] * fast_exp2(fmaf(y * a.inv_t, kLog2e, -lzc[j]));
-                    if (tg[j] == row) dv += g[j];
-                    dv *= chain;
+                    // z from the numerator (a flushed one has p = 0 and, unless it is the target, no gradient)
+                    const bool is_t = tg[j] == row;
+                    const float z = is_t ? zt[j] : (__log2f(e[j][i]) - kStashExp + rf[h][j]) * kLn2;
+                    const float th = z * th_mul;
+                    dv = ngc[j] * (is_t ? p - 1.f : p) * (1.f - th * th);
+                    if (!is_t && e[j][i] == 0.f) dv = 0.f;
                 }
-                d[j] = (row < rows && g[j] != 0.f) ? dv : 0.f;
+                d[j] = (row < rows && live[j]) ? dv : 0.f;
             }
             uint2 w;
             w.x = E::pack2(d[0], d[1]);
@@ -1408,7 +1448,7 @@ extern "C" size_t trlk_fused_head_stash_bytes(int64_t n_tokens, int64_t vocab, i
     if (n_tokens <= 0 || vocab <= 0) return 0;
     const int64_t ld = round_up(n_tokens, BN);
     if (out_ld) *out_ld = ld;
-    return size_t(round_up(vocab, BM)) * size_t(ld) * sizeof(float);
+    return size_t(StashView::rows8(round_up(vocab, BM))) * size_t(ld) * 8;
 }
 
 extern "C" size_t trlk_fused_head_bwd_workspace_bytes(int64_t n_tokens, int64_t vocab, int64_t hidden_size,
@@ -1421,7 +1461,7 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
                                    int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                                    int64_t weight_stride, float temperature, float final_logit_softcapping,
                                    float logit_scale, const float* d_bias, float* d_out_logp, float* d_out_entropy,
-                                   float* d_out_log_z, float* d_out_target_is_max, float* d_out_stash,
+                                   float* d_out_log_z, float* d_out_target_is_max, void* d_out_stash,
                                    int64_t stash_ld, int32_t* d_error_flag, void* d_workspace, size_t workspace_bytes,
                                    trlk_stream_t stream) {
     clear_error();
@@ -1444,8 +1484,7 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
     a.weight = static_cast<const uint16_t*>(d_weight);
     a.targets = d_targets;
     a.bias = d_bias;
-    a.stash = d_out_stash;
-    a.ld_stash = stash_ld;
+    a.stash = StashView{static_cast<char*>(d_out_stash), stash_ld, round_up(vocab, BM)};
     a.N = int(n_tokens);
     a.V = int(vocab);
     a.H = int(hidden_size);
@@ -1465,12 +1504,18 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
     if (int rc = launch_status("fused_head_fwd (fill)")) return rc;
     const int n_tb = int((n_tokens + BN - 1) / BN);
     const int grid = xcd_patch_grid(n_tb, splits);
-    int rc = dtype == TRLK_BF16 ? launch_head(fused_head_fwd_kernel<TRLK_BF16>, grid, a, s, "fused_head_fwd")
-                                : launch_head(fused_head_fwd_kernel<TRLK_F16>, grid, a, s, "fused_head_fwd");
+    const char* what = "fused_head_fwd";
+    int rc;
+    if (d_out_stash != nullptr)
+        rc = dtype == TRLK_BF16 ? launch_head(fused_head_fwd_kernel<TRLK_BF16, true>, grid, a, s, what)
+                                : launch_head(fused_head_fwd_kernel<TRLK_F16, true>, grid, a, s, what);
+    else
+        rc = dtype == TRLK_BF16 ? launch_head(fused_head_fwd_kernel<TRLK_BF16, false>, grid, a, s, what)
+                                : launch_head(fused_head_fwd_kernel<TRLK_F16, false>, grid, a, s, what);
     if (rc) return rc;
     hipLaunchKernelGGL(head_merge_kernel, dim3(unsigned((n_tokens + 255) / 256)), dim3(256), 0, s, a.partial, a.tgt,
                        d_targets, int(n_tokens), int(vocab), splits, d_out_logp, d_out_entropy, d_out_log_z,
-                       d_out_target_is_max, d_error_flag);
+                       d_out_target_is_max, d_error_flag, d_out_stash != nullptr ? a.stash.zt() : nullptr);
     return launch_status("fused_head_fwd (merge)");
 }
 
@@ -1478,7 +1523,7 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
                                    int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t hidden_stride,
                                    int64_t weight_stride, float temperature, float final_logit_softcapping,
                                    float logit_scale, const float* d_bias, const float* d_log_z, const float* d_g_logp,
-                                   int64_t chunk_size, const float* d_stash, int64_t stash_ld, const int32_t* d_stash_cols,
+                                   int64_t chunk_size, const void* d_stash, int64_t stash_ld, const int32_t* d_stash_cols,
                                    void* d_out_dhidden, void* d_out_dweight, float* d_out_dbias, void* d_workspace,
                                    size_t workspace_bytes, trlk_stream_t stream) {
     clear_error();
@@ -1554,9 +1599,8 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
     a.softcap = final_logit_softcapping > 0.f ? final_logit_softcapping : 0.f;
     a.log_z = d_log_z;
     a.g = d_g_logp;
-    a.stash_in = d_stash;
+    a.stash = StashView{static_cast<char*>(const_cast<void*>(d_stash)), stash_ld, round_up(vocab, BM)};
     a.stash_cols = d_stash_cols;
-    a.ld_stash = stash_ld;
     a.dzT = dzt;
     a.ldzt = l.ld_n;
     a.g_max = max_g;

@@ -695,12 +695,22 @@ def _head_operands(hidden: Tensor, weight: Tensor, targets: Tensor):
     return hidden, weight, targets.contiguous()
 
 
+def _head_stash_shape(n_tokens: int, vocab: int) -> tuple[int, int, int]:
+    """Shape of the stash as an fp16 tensor `[rows, tokens padded, 4]`: the library's own layout (softmax numerators
+    of 4 vocabulary rows per token, then their reference exponents and the targets' logits)."""
+    ld = ctypes.c_int64(0)
+    nbytes = lib.trlk_fused_head_stash_bytes(n_tokens, vocab, ctypes.addressof(ld))
+    return nbytes // (8 * ld.value), ld.value, 4
+
+
 def head_stash_fits(n_tokens: int, vocab: int) -> bool:
-    """Whether the forward should keep its raw products for the backward: the fp32 `[vocab, n_tokens]` buffer
-    (both padded to 256) must fit the budget `TRL_AMD_HEAD_STASH_GIB` (GiB, default 24; 0 = always recompute)."""
+    """Whether the forward should keep its softmax numerators for the backward: the buffer (2.07 bytes per logit,
+    both dimensions padded to 256) must fit the budget `TRL_AMD_HEAD_STASH_GIB` (GiB, default 24; 0 = always
+    recompute)."""
     budget = float(os.environ.get("TRL_AMD_HEAD_STASH_GIB", "24"))
-    need = ((vocab + 255) // 256 * 256) * ((n_tokens + 255) // 256 * 256) * 4
-    return n_tokens > 0 and need <= budget * 2**30
+    if n_tokens <= 0 or budget <= 0:
+        return False
+    return lib.trlk_fused_head_stash_bytes(n_tokens, vocab, None) <= budget * 2**30
 
 
 def _head_bias(bias, vocab):
@@ -718,7 +728,8 @@ def fused_head_fwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
     """hidden [N, H], weight [V, H] (bf16/fp16), targets int64 [N] -> fp32 (logp, entropy, log_z, target_is_max),
     each [N]; target_is_max is 1 where argmax(logits) == target.  `softcap <= 0` means no soft-capping.
     `bias` [V] (any float dtype) is added to `hidden @ weight.T` before scaling.  With `stash` the fifth
-    output holds the raw products (fp32 `[V padded, N padded]`) for `fused_head_bwd`; it is empty otherwise."""
+    output holds the softmax numerators (fp16, in the library's own layout) for `fused_head_bwd`; it is empty
+    otherwise."""
     hidden, weight, targets = _head_operands(hidden, weight, targets)
     n, h = hidden.shape
     v = weight.shape[0]
@@ -729,20 +740,18 @@ def fused_head_fwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
     log_z = torch.empty((n,), dtype=torch.float32, device=dev)
     hit = torch.empty((n,), dtype=torch.float32, device=dev)
     if n == 0:
-        return logp, ent, log_z, hit, torch.empty((0, 0), dtype=torch.float32, device=dev)
+        return logp, ent, log_z, hit, torch.empty((0, 0, 4), dtype=torch.float16, device=dev)
     if stash:
-        ld = ctypes.c_int64(0)
-        nbytes = lib.trlk_fused_head_stash_bytes(n, v, ctypes.addressof(ld))
-        saved = torch.empty((nbytes // (4 * ld.value), ld.value), dtype=torch.float32, device=dev)
+        saved = torch.empty(_head_stash_shape(n, v), dtype=torch.float16, device=dev)
     else:
-        saved = torch.empty((0, 0), dtype=torch.float32, device=dev)
+        saved = torch.empty((0, 0, 4), dtype=torch.float16, device=dev)
     ws_bytes = lib.trlk_fused_head_fwd_workspace_bytes(n)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         check(lib.trlk_fused_head_fwd(ptr(hidden), ptr(weight), ptr(targets), dtype_code(hidden.dtype), n, v, h,
                                       hidden.stride(0), weight.stride(0), temperature, softcap, logit_scale,
                                       ptr(bias32), ptr(logp), ptr(ent), ptr(log_z), ptr(hit),
-                                      ptr(saved) if stash else None, saved.stride(0) if stash else 0,
+                                      ptr(saved) if stash else None, saved.shape[1] if stash else 0,
                                       ptr(_error_flag(dev)), ptr(ws), ws_bytes, current_stream(dev)))
     if _SYNC_CHECKS:
         check_device_errors()
@@ -752,8 +761,9 @@ def fused_head_fwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
 @fused_head_fwd.register_fake
 def _(hidden, weight, targets, temperature, softcap, logit_scale, bias=None, stash=False):
     f = lambda: torch.empty((hidden.shape[0],), dtype=torch.float32, device=hidden.device)  # noqa: E731
-    rows, cols = ((weight.shape[0] + 255) // 256 * 256, (hidden.shape[0] + 255) // 256 * 256) if stash else (0, 0)
-    return f(), f(), f(), f(), torch.empty((rows, cols), dtype=torch.float32, device=hidden.device)
+    vpad, cols = ((weight.shape[0] + 255) // 256 * 256, (hidden.shape[0] + 255) // 256 * 256) if stash else (0, 0)
+    rows = vpad // 4 + vpad // 128 + 1 if stash else 0
+    return f(), f(), f(), f(), torch.empty((rows, cols, 4), dtype=torch.float16, device=hidden.device)
 
 
 @torch.library.custom_op("trl_amd::fused_head_bwd", mutates_args=(), device_types="cuda")
@@ -783,8 +793,8 @@ def fused_head_bwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
         if stash_cols.dtype != torch.int32 or stash_cols.shape != (n,):
             raise ValueError("fused head: stash_cols must be int32 [N]")
         stash_cols = stash_cols.contiguous()
-    if stash is not None and (stash.dtype != torch.float32 or stash.stride(1) != 1 or
-                              stash.shape[0] < (v + 255) // 256 * 256 or
+    if stash is not None and (stash.dtype != torch.float16 or stash.dim() != 3 or stash.shape[2] != 4 or
+                              not stash.is_contiguous() or stash.shape[0] != _head_stash_shape(1, v)[0] or
                               (stash_cols is None and stash.shape[1] < (n + 255) // 256 * 256)):
         raise ValueError("fused head: the stash does not belong to these operands")
     ws_bytes = lib.trlk_fused_head_bwd_workspace_bytes(max(n, 1), v, h, chunk_size)
@@ -793,7 +803,7 @@ def fused_head_bwd(hidden: Tensor, weight: Tensor, targets: Tensor, temperature:
         check(lib.trlk_fused_head_bwd(ptr(hidden), ptr(weight), ptr(targets), dtype_code(hidden.dtype), n, v, h,
                                       hidden.stride(0), weight.stride(0), temperature, softcap, logit_scale,
                                       ptr(bias32), ptr(log_z), ptr(g), chunk_size, ptr(stash),
-                                      stash.stride(0) if stash is not None else 0, ptr(stash_cols), ptr(d_hidden),
+                                      stash.shape[1] if stash is not None else 0, ptr(stash_cols), ptr(d_hidden),
                                       ptr(d_weight),
                                       ptr(d_bias) if bias is not None else None, ptr(ws), ws_bytes, current_stream(dev)))
     if h != h_true:  # the operands were padded to a multiple of 8 columns
