@@ -197,9 +197,11 @@ struct DirectLoader {
     // (m0 is a reserved register; naming it as clobbered is what tells the compiler not to keep a value there)
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
-    static __device__ __forceinline__ void transfer(const char* src, uint32_t lds) {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds),
-                     "v"(reinterpret_cast<uint64_t>(src))
+    // The source is a uniform 64-bit base (scalar registers) plus the lane's 32-bit byte offset: one vector register
+    // per transfer instead of an address pair, and the k step is added on the scalar side.
+    static __device__ __forceinline__ void transfer(const char* base, uint32_t lane_off, uint32_t lds) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(lane_off),
+                     "s"(reinterpret_cast<uint64_t>(base))
                      : "memory", "m0");
     }
 #pragma clang diagnostic pop
@@ -209,9 +211,9 @@ struct DirectLoader {
     // transfer j of a stage (A blocks first, then B blocks)
     __device__ __forceinline__ void issue_one(int buf, int k0, int j) const {
         if (j < kBlkA)
-            transfer(abase + int64_t(k0) * akstep + ao[j], lds_base(buf) + (wave + kWaves * j) * 1024);
+            transfer(abase + int64_t(k0) * akstep, ao[j], lds_base(buf) + (wave + kWaves * j) * 1024);
         else
-            transfer(bbase + int64_t(k0) * 2 + bo[j - kBlkA], lds_base(buf) + C::kDenseA + (wave + kWaves * (j - kBlkA)) * 1024);
+            transfer(bbase + int64_t(k0) * 2, bo[j - kBlkA], lds_base(buf) + C::kDenseA + (wave + kWaves * (j - kBlkA)) * 1024);
     }
     __device__ __forceinline__ void issue(int buf, int k0) const {
 #pragma unroll
@@ -643,7 +645,10 @@ __device__ __forceinline__ float head_z(float y, const HeadArgs& a) {
 
 constexpr float kStashExp = 15.f;  // the numerators are summed and stashed times 2^15 (fp16's range above 1)
 
-template <int DT, bool STASH>
+// GENERAL: soft-capping, a bias or a non-positive scale (z is computed per logit).  Otherwise z = y * zs with one
+// positive scale: the maximum is taken on the raw accumulators, the scale is folded into the exponent's multiplier and
+// sum(e * z) is accumulated as zs * sum(e * y) -- the kernel of the usual head then carries no code of the other.
+template <int DT, bool STASH, bool GENERAL>
 TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int n_tb = (a.N + BN - 1) / BN;
@@ -681,24 +686,37 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
         if (vt + 1 < vt1) gemm_tile_prefetch<TRLK_HEAD_BK_FWD>(W, m0 + BM, Hd, n0, a.H, smem);
         // Stash: for one accumulator quad (4 consecutive vocabulary rows of one token per lane) the 32 lanes of a
         // half-wave hold 32 consecutive tokens = 256 contiguous bytes per store.  The buffer is padded to whole tiles.
-        char* stash_blk = nullptr;   // uniform
-        uint32_t stash_lane = 0;     // byte offset of the lane (the entry point bounds ld so that it fits)
+        // Addresses are a uniform pointer that walks down the quads (scalar registers, one addition per store) plus
+        // the lane's byte offset (one vector register; the entry point bounds ld so that it fits 32 bits).
+        char* stash_blk = nullptr;
+        float* ref_blk = nullptr;
+        uint32_t stash_lane = 0, ref_lane = 0;
         if constexpr (STASH) {
             const int uw = __builtin_amdgcn_readfirstlane(wave);
-            stash_blk = reinterpret_cast<char*>(a.stash.quads() + int64_t(m0 / 4 + (uw / WGN) * (WM / 4)) * a.stash.ld +
-                                                (n0 + (uw % WGN) * WN));
-            stash_lane = (uint32_t(lane >> 5) * uint32_t(a.stash.ld) + uint32_t(lane & 31)) * 8u;
+            const int uwm = uw / WGN, ucol = n0 + (uw % WGN) * WN;
+            stash_blk = reinterpret_cast<char*>(a.stash.quads() + int64_t(m0 / 4 + uwm * (WM / 4)) * a.stash.ld + ucol);
+            ref_blk = a.stash.refs() + int64_t(m0 / 128 + uwm) * 2 * a.stash.ld + ucol;
+            ref_lane = uint32_t(lane >> 5) * uint32_t(a.stash.ld) + uint32_t(lane & 31);
+            stash_lane = ref_lane * 8u;
         }
         const bool partial_tile = m0 + BM > a.V;
-        // Common case (no soft-capping, tile inside the vocabulary): z = y * zs with one positive
-        // scale, so the maximum is taken on the raw accumulators and the scale is folded into the
-        // exponent's multiplier; sum(e * z) is accumulated as zs * sum(e * y).
         const float zs = a.logit_scale * a.inv_t, zs2 = zs * kLog2e;
-        const bool plain = a.softcap <= 0.f && !partial_tile && zs > 0.f && a.bias == nullptr;
+        constexpr bool plain = !GENERAL;
+        if constexpr (plain) {
+            if (partial_tile) {  // the vocabulary's last tile: rows beyond it count as -inf
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            if (m0 + acc_row(wm, mb, r, lane) >= a.V) acc[mb][nb][r] = -INFINITY;
+            }
+        }
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             float bm = -INFINITY;
-            if (plain) {
+            if constexpr (plain) {
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -727,17 +745,15 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
                 ref[nb] = need;
                 rr[nb] = need;
             }
-            if constexpr (STASH) {
-                const int tcol = n0 + acc_col(wn, nb, lane);
-                a.stash.refs()[(int64_t(m0 / 128 + wm) * 2 + (lane >> 5)) * a.stash.ld + tcol] = rr[nb];
-            }
+            char* stash_p = stash_blk + nb * 32 * 8;  // this token block's column of quads
+            if constexpr (STASH) ref_blk[nb * 32 + ref_lane] = rr[nb];
             // numerators times 2^15 (exact; S and U carry the factor until they are written out), with or without a
             // stash: the outputs must not depend on stashing
             const float rsub = rr[nb] - kStashExp;
             float s = 0.f, u = 0.f;
-            auto sum_tile = [&](auto is_plain) {
-                constexpr bool kPlain = decltype(is_plain)::value;
-                const float mul = kPlain ? zs2 : kLog2e;  // general path: the accumulators hold z itself by now
+            auto sum_tile = [&](auto guard_tag) {
+                constexpr bool kGuard = decltype(guard_tag)::value;  // -inf among the logits (0 * -inf in sum(e * y))
+                const float mul = plain ? zs2 : kLog2e;  // general path: the accumulators hold z itself by now
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -748,22 +764,23 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
                             const float y = acc[mb][nb][q * 4 + i];
                             e[i] = fast_exp2(fmaf(y, mul, -rsub));
                             s += e[i];
-                            u = (!kPlain && y == -INFINITY) ? u : fmaf(e[i], y, u);
+                            u = (kGuard && y == -INFINITY) ? u : fmaf(e[i], y, u);
                         }
                         if constexpr (STASH) {
                             uint2 w;
                             w.x = Elem<TRLK_F16>::pack2(e[0], e[1]);
                             w.y = Elem<TRLK_F16>::pack2(e[2], e[3]);
-                            *reinterpret_cast<uint2*>(stash_blk + ((mb * 8 + q * 2) * a.stash.ld + nb * 32) * 8 + stash_lane) = w;
+                            *reinterpret_cast<uint2*>(stash_p + stash_lane) = w;
+                            stash_p += a.stash.ld * 16;  // two quads down: the other parity is the other half-wave's
+                            asm volatile("" : "+s"(stash_p));  // (keeps it one running pointer, not 16 precomputed ones)
                         }
                     }
             };
-            if (plain) {
+            if (GENERAL || partial_tile)
                 sum_tile(std::true_type{});
-                u *= zs;
-            } else {
+            else
                 sum_tile(std::false_type{});
-            }
+            if constexpr (plain) u *= zs;
             S[nb] += s;
             U[nb] += u;
             // target logit: rarely inside this wave's 128 vocabulary rows.  It is selected into one register
@@ -1506,12 +1523,16 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
     const int grid = xcd_patch_grid(n_tb, splits);
     const char* what = "fused_head_fwd";
     int rc;
+    const bool general = a.softcap > 0.f || d_bias != nullptr || !(a.logit_scale * a.inv_t > 0.f);
+    auto launch_fwd = [&](auto stash_tag, auto general_tag) {
+        constexpr bool kS = decltype(stash_tag)::value, kG = decltype(general_tag)::value;
+        return dtype == TRLK_BF16 ? launch_head(fused_head_fwd_kernel<TRLK_BF16, kS, kG>, grid, a, s, what)
+                                  : launch_head(fused_head_fwd_kernel<TRLK_F16, kS, kG>, grid, a, s, what);
+    };
     if (d_out_stash != nullptr)
-        rc = dtype == TRLK_BF16 ? launch_head(fused_head_fwd_kernel<TRLK_BF16, true>, grid, a, s, what)
-                                : launch_head(fused_head_fwd_kernel<TRLK_F16, true>, grid, a, s, what);
+        rc = general ? launch_fwd(std::true_type{}, std::true_type{}) : launch_fwd(std::true_type{}, std::false_type{});
     else
-        rc = dtype == TRLK_BF16 ? launch_head(fused_head_fwd_kernel<TRLK_BF16, false>, grid, a, s, what)
-                                : launch_head(fused_head_fwd_kernel<TRLK_F16, false>, grid, a, s, what);
+        rc = general ? launch_fwd(std::false_type{}, std::true_type{}) : launch_fwd(std::false_type{}, std::false_type{});
     if (rc) return rc;
     hipLaunchKernelGGL(head_merge_kernel, dim3(unsigned((n_tokens + 255) / 256)), dim3(256), 0, s, a.partial, a.tgt,
                        d_targets, int(n_tokens), int(vocab), splits, d_out_logp, d_out_entropy, d_out_log_z,
