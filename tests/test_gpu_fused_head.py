@@ -244,6 +244,38 @@ def test_backward_from_stashed_products_equals_recompute(amd, monkeypatch, n, h,
         amd.ops.fused_head_bwd(hidden, weight, labels, 0.9, 0.0, 1.0, log_z, gout, chunk, None, saved[:-1])
 
 
+@pytest.mark.parametrize("kind", ["flat", "peaked", "capped_deep_target"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_stashed_numerators_on_flat_peaked_and_capped_rows(amd, monkeypatch, kind, dtype):
+    """The stash holds fp16 softmax numerators relative to a running maximum.  Rows on which that could show: nearly
+    uniform ones (every numerator close to 1), sharply peaked ones (most numerators below fp16's range: flushed,
+    their probabilities are below 2e-12), and soft-capped rows whose target sits 50 nats under the maximum (its
+    numerator is flushed, the chain factor of its one-hot term comes from the target logit the forward keeps)."""
+    n, h, v, chunk = 300, 128, 1500, 512
+    g = torch.Generator().manual_seed({"flat": 1, "peaked": 2, "capped_deep_target": 3}[kind])
+    hidden = torch.randn(n, h, generator=g).to(dtype)
+    gain = {"flat": 0.01, "peaked": 12.0, "capped_deep_target": 12.0}[kind]
+    weight = (torch.randn(v, h, generator=g) * (gain / h**0.5)).to(dtype)
+    softcap = 30.0 if kind == "capped_deep_target" else None
+    logits = hidden.float() @ weight.float().t()
+    if kind == "capped_deep_target":
+        labels = logits.argmin(-1)  # capped to about -30 where the row's maximum is about +30
+        z = torch.tanh(logits / softcap) * softcap
+        assert float((z.max(-1).values - z.gather(-1, labels[:, None]).squeeze(-1)).median()) > 40.0
+    else:
+        labels = torch.randint(0, v, (n,), generator=g)
+    gout = torch.randn(n, generator=g)
+    rlp, rent, rdh, rdw = _fp32_reference(hidden, weight, labels, 1.0, softcap, 1.0, gout)
+    for gib in ("1", "0"):  # from the stash, and recomputed
+        monkeypatch.setenv("TRL_AMD_HEAD_STASH_GIB", gib)
+        assert amd.ops.head_stash_fits(n, v) == (gib == "1")
+        lp, ent, dh, dw = _run_device(amd, hidden, weight, labels, 1.0, chunk, softcap, 1.0, gout)
+        torch.testing.assert_close(lp, rlp, atol=2e-3, rtol=2e-5)
+        torch.testing.assert_close(ent, rent, atol=2e-3, rtol=0)
+        assert torch.isfinite(dh.float()).all() and torch.isfinite(dw.float()).all()
+        _check_beyond_output_rounding(dh, dw, rdh, rdw, dtype)
+
+
 def test_masked_rows_and_scatter(amd):
     # reference tests/test_utils.py:1338-1398: masked == unmasked on completion rows, exact zeros elsewhere,
     # and the lm_head gradient only sees completion rows
