@@ -956,7 +956,7 @@ def bench_one_leg(args, w):
       k7_masked              single-pass kernel, rows outside the mask zero-filled without being read
       k7_all_rows            single-pass kernel, rows outside the mask read for their log-prob and entropy
       k7_dense_mask          single-pass kernel with a mask of ones: every row read and written
-      head_fwd_stash/_plain  fused head forward with / without keeping its products
+      head_fwd_stash/_plain  fused head forward with / without keeping its softmax numerators
       head_bwd_every_token   fused head backward (from the kept products) with a gradient on every token
       head_bwd_step          the same with the benchmark's mask (tokens without gradient dropped first)"""
     import trl_amd

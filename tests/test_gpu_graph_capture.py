@@ -136,8 +136,9 @@ def test_single_pass_wide_row_first_launch_is_inside_the_capture():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 def test_fused_head_graph_replays_equal_eager(dtype):
-    """Forward with its products kept, then both gradient products from them: every buffer between the two (the
-    kept products, the scaled fp16 operand copies, the maxima behind their scales) is rewritten inside the graph."""
+    """Forward with its softmax numerators kept, then both gradient products from them: every buffer between the two
+    (the kept numerators, the scaled fp16 operand copies, the maxima behind their scales) is rewritten inside the
+    graph."""
     from trl_amd import ops
 
     n, h, v = 300, 128, 1000  # two token tiles, four vocabulary tiles, both with remainders

@@ -17,7 +17,7 @@
 //
 // Backward (K6), per vocabulary chunk: (1) dz = dL/dlogits as scaled fp16 [chunk, tokens] (vocabulary-major, each
 // token's column in that token's own power-of-two scale) -- from a recompute of the chunk's logits (same tile loop),
-// or, when the forward was asked to stash its raw products, from one elementwise sweep over that stash;
+// or, when the forward was asked to stash its softmax numerators, from one elementwise sweep over that stash;
 // (2) dHidden += dz * W_chunk: the tile loop with dz as a K-MAJOR left operand (its k rows go to LDS as they lie in
 // memory and the MFMA fragments come out through the LDS transpose loads, ds_read_b64_tr_b16) against W_chunk^T;
 // (3) dW_chunk = dz^T * hidden as an NT product against hidden^T, whose columns carry the inverse of the tokens'
