@@ -511,15 +511,6 @@ __device__ __forceinline__ void gemm_tile_nt(const Operand A, int m0, const Oper
     }
 }
 
-// Starts the transfers of a tile's first stages so that they overlap whatever the caller does
-// before gemm_tile_nt(..., prefetched = true); the LDS must be free and stay untouched until then.
-template <int BKT>
-__device__ __forceinline__ void gemm_tile_prefetch(const Operand A, int m0, const Operand B, int n0, int K, char* smem) {
-#if TRLK_HEAD_DIRECT_LDS
-    if ((K & (BKT - 1)) == 0) DirectLoader<BKT>(A, m0, B, n0, smem).prologue(K);
-#endif
-}
-
 // Row (M index) inside the workgroup tile of accumulator element r of block mb, for this lane.
 __device__ __forceinline__ int acc_row(int wm, int mb, int r, int lane) {
     return wm * WM + mb * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
@@ -636,19 +627,25 @@ __device__ __forceinline__ float slot_scale(const uint32_t* slot, float mult) {
     return slot != nullptr ? pow2_scale(__uint_as_float(*slot) * mult) : 1.f;
 }
 
-// z = logit in natural units after logit_scale, optional soft-capping and temperature.
-__device__ __forceinline__ float head_z(float y, const HeadArgs& a) {
-    y *= a.logit_scale;
-    if (a.softcap > 0.f) y = tanhf(y / a.softcap) * a.softcap;
-    return y * a.inv_t;
+// tanh for soft-capping: sign(x) (1 - t) / (1 + t) with t = exp(-2 |x|) from the hardware's exp2 and reciprocal (a
+// relative error of a few 1e-7), and the odd series x - x^3/3 + 2 x^5/15 below 0.05, where 1 - t cancels.  A third of
+// the instructions of the library routine, in an epilogue that runs it once per logit.
+__device__ __forceinline__ float head_tanh(float x) {
+    const float ax = fabsf(x), x2 = x * x;
+    const float t = fast_exp2(ax * (-2.f * kLog2e));
+    const float big = (1.f - t) * __builtin_amdgcn_rcpf(1.f + t);
+    const float small = ax * fmaf(x2, fmaf(x2, 2.f / 15.f, -1.f / 3.f), 1.f);
+    return copysignf(ax < 0.05f ? small : big, x);
 }
 
 constexpr float kStashExp = 15.f;  // the numerators are summed and stashed times 2^15 (fp16's range above 1)
 
-// GENERAL: soft-capping, a bias or a non-positive scale (z is computed per logit).  Otherwise z = y * zs with one
+// GENERAL: soft-capping or a non-positive scale (z is computed per logit).  Otherwise z = (y + bias) * zs with one
 // positive scale: the maximum is taken on the raw accumulators, the scale is folded into the exponent's multiplier and
 // sum(e * z) is accumulated as zs * sum(e * y) -- the kernel of the usual head then carries no code of the other.
-template <int DT, bool STASH, bool GENERAL>
+// STAGED: the hidden size is not a multiple of the direct-to-LDS loop's k step (a kernel of its own, so that the
+// usual one does not carry the register-staged loop's code and loop-invariant registers through its tile loop).
+template <int DT, bool STASH, bool GENERAL, bool STAGED>
 TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int n_tb = (a.N + BN - 1) / BN;
@@ -677,13 +674,18 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
     }
     const Operand W{a.weight, a.ldw, a.V}, Hd{a.hidden, a.ldh, a.N};
 
-    if (vt0 < vt1) gemm_tile_prefetch<TRLK_HEAD_BK_FWD>(W, vt0 * BM, Hd, n0, a.H, smem);
+    if constexpr (!STAGED)
+        if (vt0 < vt1) DirectLoader<TRLK_HEAD_BK_FWD>(W, vt0 * BM, Hd, n0, smem).prologue(a.H);
     for (int vt = vt0; vt < vt1; ++vt) {
         const int m0 = vt * BM;
         f32x16 acc[MB][NB];
-        gemm_tile_nt<DT, TRLK_HEAD_BK_FWD>(W, m0, Hd, n0, a.H, acc, smem, true);
-        // the next tile's first stages travel while this tile's logits are reduced (registers only)
-        if (vt + 1 < vt1) gemm_tile_prefetch<TRLK_HEAD_BK_FWD>(W, m0 + BM, Hd, n0, a.H, smem);
+        if constexpr (STAGED) {
+            gemm_tile_nt_staged<DT>(W, m0, Hd, n0, a.H, acc, smem);
+        } else {
+            gemm_tile_nt_direct<DT, TRLK_HEAD_BK_FWD>(W, m0, Hd, n0, a.H, acc, smem, true);
+            // the next tile's first stages travel while this tile's logits are reduced (registers only)
+            if (vt + 1 < vt1) DirectLoader<TRLK_HEAD_BK_FWD>(W, m0 + BM, Hd, n0, smem).prologue(a.H);
+        }
         // Stash: for one accumulator quad (4 consecutive vocabulary rows of one token per lane) the 32 lanes of a
         // half-wave hold 32 consecutive tokens = 256 contiguous bytes per store.  The buffer is padded to whole tiles.
         // Addresses are a uniform pointer that walks down the quads (scalar registers, one addition per store) plus
@@ -702,39 +704,77 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
         const bool partial_tile = m0 + BM > a.V;
         const float zs = a.logit_scale * a.inv_t, zs2 = zs * kLog2e;
         constexpr bool plain = !GENERAL;
-        if constexpr (plain) {
-            if (partial_tile) {  // the vocabulary's last tile: rows beyond it count as -inf
+        // Before the reduction, only where needed (a bias, the general form of z, or the vocabulary's last tile, whose
+        // rows beyond the vocabulary count as -inf): the accumulators become y + bias (usual head) or z itself
+        // (general form).  A lane's 16 accumulators of a block are 4 quads of consecutive vocabulary rows, so the bias
+        // comes as one 16-byte load per quad, all of a block row's loads issued before the first is used.
+        if (GENERAL || a.bias != nullptr || partial_tile) {
+            const float inv_cap = a.softcap > 0.f ? 1.f / a.softcap : 0.f;
+            typedef float f32x4_dword_aligned __attribute__((ext_vector_type(4), aligned(4)));
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
+            for (int mb = 0; mb < MB; ++mb) {
+                f32x4 bq[4];
 #pragma unroll
-                    for (int mb = 0; mb < MB; ++mb)
+                for (int q = 0; q < 4; ++q) {
+                    const int v0 = m0 + acc_row(wm, mb, q * 4, lane);
+                    bq[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    if (a.bias != nullptr) {
+                        if (v0 + 3 < a.V) {
+                            bq[q] = *reinterpret_cast<const f32x4_dword_aligned*>(a.bias + v0);
+                        } else {
 #pragma unroll
-                        for (int r = 0; r < 16; ++r)
-                            if (m0 + acc_row(wm, mb, r, lane) >= a.V) acc[mb][nb][r] = -INFINITY;
+                            for (int i = 0; i < 4; ++i)
+                                if (v0 + i < a.V) bq[q][i] = a.bias[v0 + i];
+                        }
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int v0 = m0 + acc_row(wm, mb, q * 4, lane);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const bool beyond = partial_tile && v0 + i >= a.V;
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb) {
+                            float y = acc[mb][nb][q * 4 + i] + bq[q][i];
+                            if constexpr (GENERAL) {
+                                y *= a.logit_scale;
+                                if (a.softcap > 0.f) y = head_tanh(y * inv_cap) * a.softcap;
+                                y *= a.inv_t;
+                            }
+                            acc[mb][nb][q * 4 + i] = beyond ? -INFINITY : y;
+                        }
+                    }
+                }
             }
         }
+        // (With a stash the numerators are stored as they are produced.  Packed into registers and stored in one run
+        // at the end of the epilogue they cost more: 28.6 against 27.8 ms for the benchmark's forward.)
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             float bm = -INFINITY;
-            if constexpr (plain) {
 #pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
+            for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) bm = fmaxf(bm, acc[mb][nb][r]);
-                bm *= zs;
-            } else {
+                for (int r = 0; r < 16; ++r) bm = fmaxf(bm, acc[mb][nb][r]);
+            if constexpr (plain) bm *= zs;
+            // target logit: rarely inside this wave's 128 vocabulary rows.  It is selected into one register
+            // and stored once: a conditional store per accumulator held the wave for about 20 us, and a
+            // workgroup that falls behind the others no longer finds the tiles they share in the L2.
+            const int64_t rel = tg[nb] - (m0 + wm * WM);
+            if (rel >= 0 && rel < WM) {
+                const int want = int(rel) - (lane >> 5) * 4;  // acc_row() without this lane's half-wave offset
+                float tv = 0.f;
+                bool mine = false;
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const int v = m0 + acc_row(wm, mb, r, lane);
-                        float y = acc[mb][nb][r];
-                        if (a.bias != nullptr && v < a.V) y += a.bias[v];
-                        float z = head_z(y, a);
-                        if (partial_tile && v >= a.V) z = -INFINITY;
-                        acc[mb][nb][r] = z;
-                        bm = fmaxf(bm, z);
+                        const bool m = (mb * 32 + (r >> 2) * 8 + (r & 3)) == want;
+                        tv = m ? acc[mb][nb][r] : tv;
+                        mine |= m;
                     }
+                if (mine) a.tgt[n0 + acc_col(wn, nb, lane)] = plain ? tv * zs : tv;
             }
             zmax[nb] = fmaxf(zmax[nb], bm);
             const float need = ceilf(bm * kLog2e);
@@ -745,10 +785,10 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
                 ref[nb] = need;
                 rr[nb] = need;
             }
-            char* stash_p = stash_blk + nb * 32 * 8;  // this token block's column of quads
-            if constexpr (STASH) ref_blk[nb * 32 + ref_lane] = rr[nb];
             // numerators times 2^15 (exact; S and U carry the factor until they are written out), with or without a
             // stash: the outputs must not depend on stashing
+            int64_t stash_off = nb * 32 * 8;  // byte offset of this token block's column of quads (uniform)
+            if constexpr (STASH) ref_blk[nb * 32 + ref_lane] = rr[nb];
             const float rsub = rr[nb] - kStashExp;
             float s = 0.f, u = 0.f;
             auto sum_tile = [&](auto guard_tag) {
@@ -770,9 +810,11 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
                             uint2 w;
                             w.x = Elem<TRLK_F16>::pack2(e[0], e[1]);
                             w.y = Elem<TRLK_F16>::pack2(e[2], e[3]);
-                            *reinterpret_cast<uint2*>(stash_p + stash_lane) = w;
-                            stash_p += a.stash.ld * 16;  // two quads down: the other parity is the other half-wave's
-                            asm volatile("" : "+s"(stash_p));  // (keeps it one running pointer, not 16 precomputed ones)
+                            *reinterpret_cast<uint2*>(stash_blk + stash_off + stash_lane) = w;
+                            stash_off += a.stash.ld * 16;  // two quads down: the other parity is the other half-wave's
+                            // (one running offset, not 16 precomputed ones; an offset, because a pointer that
+                            // passed through here would no longer be known to point to global memory)
+                            asm volatile("" : "+s"(stash_off));
                         }
                     }
             };
@@ -783,24 +825,6 @@ TRLK_HEAD_KERNEL void fused_head_fwd_kernel(HeadArgs a) {
             if constexpr (plain) u *= zs;
             S[nb] += s;
             U[nb] += u;
-            // target logit: rarely inside this wave's 128 vocabulary rows.  It is selected into one register
-            // and stored once: a conditional store per accumulator held the wave for about 20 us, and a
-            // workgroup that falls behind the others no longer finds the tiles they share in the L2.
-            const int64_t rel = tg[nb] - (m0 + wm * WM);
-            if (rel >= 0 && rel < WM) {
-                const int want = int(rel) - (lane >> 5) * 4;  // acc_row() without this lane's half-wave offset
-                float tv = 0.f;
-                bool mine = false;
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const bool m = (mb * 32 + (r >> 2) * 8 + (r & 3)) == want;
-                        tv = m ? acc[mb][nb][r] : tv;
-                        mine |= m;
-                    }
-                if (mine) a.tgt[n0 + acc_col(wn, nb, lane)] = plain ? tv * zs : tv;
-            }
         }
     }
 
@@ -929,7 +953,7 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
                     y *= a.logit_scale;
                     float chain = a.inv_t * a.logit_scale;
                     if (a.softcap > 0.f) {
-                        const float th = tanhf(y / a.softcap);
+                        const float th = head_tanh(y / a.softcap);
                         y = th * a.softcap;
                         chain *= 1.f - th * th;
                     }
@@ -1523,11 +1547,15 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
     const int grid = xcd_patch_grid(n_tb, splits);
     const char* what = "fused_head_fwd";
     int rc;
-    const bool general = a.softcap > 0.f || d_bias != nullptr || !(a.logit_scale * a.inv_t > 0.f);
+    const bool general = a.softcap > 0.f || !(a.logit_scale * a.inv_t > 0.f);
+    const bool staged = !TRLK_HEAD_DIRECT_LDS || hidden_size % TRLK_HEAD_BK_FWD != 0;
     auto launch_fwd = [&](auto stash_tag, auto general_tag) {
         constexpr bool kS = decltype(stash_tag)::value, kG = decltype(general_tag)::value;
-        return dtype == TRLK_BF16 ? launch_head(fused_head_fwd_kernel<TRLK_BF16, kS, kG>, grid, a, s, what)
-                                  : launch_head(fused_head_fwd_kernel<TRLK_F16, kS, kG>, grid, a, s, what);
+        if (staged)
+            return dtype == TRLK_BF16 ? launch_head(fused_head_fwd_kernel<TRLK_BF16, kS, kG, true>, grid, a, s, what)
+                                      : launch_head(fused_head_fwd_kernel<TRLK_F16, kS, kG, true>, grid, a, s, what);
+        return dtype == TRLK_BF16 ? launch_head(fused_head_fwd_kernel<TRLK_BF16, kS, kG, false>, grid, a, s, what)
+                                  : launch_head(fused_head_fwd_kernel<TRLK_F16, kS, kG, false>, grid, a, s, what);
     };
     if (d_out_stash != nullptr)
         rc = general ? launch_fwd(std::true_type{}, std::true_type{}) : launch_fwd(std::true_type{}, std::false_type{});
