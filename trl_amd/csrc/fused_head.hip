@@ -1152,6 +1152,68 @@ __device__ __forceinline__ void gemm_nt_body(const GemmArgs& a, int block, char*
     gemm_tile_nt<DT, TRLK_HEAD_BK_GEMM, AKM>(a.A, m0, a.B, n0, a.K, acc, smem);
     const float inv_b = 1.f / slot_scale(a.max_b, 1.f);
     const float inv_common = inv_b / slot_scale(a.max_a, a.mult_a);
+    // A tile inside the output (nearly every tile): no per-element predicates, addresses as a uniform base plus one
+    // 32-bit lane offset, the 16 running sums of a block loaded before the first is used and its 16 results stored in
+    // one run.  (Written per element with a bounds test each, the compiler lost count of the loads in flight and
+    // waited for EVERYTHING outstanding before each accumulate, i.e. for the previous store's acknowledgement: 128
+    // store round trips per tile.)
+    const bool lp_pairs = (reinterpret_cast<uintptr_t>(a.out_lp) & 3) == 0 && (a.ld_lp & 1) == 0;
+    if (m0 + BM <= a.M && n0 + BN <= a.N && (MODE == 1 || lp_pairs) && a.ld_f32 < (int64_t(1) << 24) &&
+        a.ld_lp < (int64_t(1) << 24)) {
+        const int uw = __builtin_amdgcn_readfirstlane(wave);
+        const int row0 = m0 + (uw / WGN) * WM, col0 = n0 + (uw % WGN) * WN;  // uniform
+        const int half = lane >> 5, l31 = lane & 31, odd = lane & 1;
+        typedef float f32x4_dword_aligned __attribute__((ext_vector_type(4), aligned(4)));
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            float inv[16];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                f32x4 g4 = {0.f, 0.f, 0.f, 0.f};
+                if (a.g_rows != nullptr)
+                    g4 = *reinterpret_cast<const f32x4_dword_aligned*>(a.g_rows + row0 + mb * 32 + q * 8 + half * 4);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    inv[q * 4 + i] = a.g_rows != nullptr ? inv_b / pow2_scale(fabsf(g4[i]) * a.mult_a) : inv_common;
+            }
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                float v[16];
+                if constexpr (MODE != 0) {
+                    float* blk = a.out_f32 + int64_t(row0 + mb * 32) * a.ld_f32 + (col0 + nb * 32);  // uniform
+                    const uint32_t lane_off = uint32_t(half * 4) * uint32_t(a.ld_f32) + uint32_t(l31);
+                    float prev[16];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        prev[r] = a.first ? 0.f : blk[int64_t(((r >> 2) * 8 + (r & 3)) * a.ld_f32) + lane_off];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) v[r] = fmaf(acc[mb][nb][r], inv[r], prev[r]);
+                    if constexpr (MODE == 1) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) blk[int64_t(((r >> 2) * 8 + (r & 3)) * a.ld_f32) + lane_off] = v[r];
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) v[r] = acc[mb][nb][r] * inv[r];
+                }
+                if constexpr (MODE != 1) {
+                    // 16-bit outputs: neighbouring lanes swap one value, the even lane then owns two columns of row
+                    // r and the odd lane two columns of row r + 1 -- 4-byte stores, 64 contiguous bytes per row
+                    typename E::type* blk = a.out_lp + int64_t(row0 + mb * 32) * a.ld_lp + (col0 + nb * 32);  // uniform
+                    const uint32_t lane_off = uint32_t(half * 4 + odd) * uint32_t(a.ld_lp) + uint32_t(l31 & ~1);
+#pragma unroll
+                    for (int r = 0; r < 16; r += 2) {
+                        const float give = odd ? v[r] : v[r + 1];
+                        const float got = __builtin_bit_cast(
+                            float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, give), 0xB1 /* quad_perm 1,0,3,2 */, 0xf, 0xf, true));
+                        const uint32_t w = odd ? E::pack2(got, v[r + 1]) : E::pack2(v[r], got);
+                        *reinterpret_cast<uint32_t*>(blk + int64_t(((r >> 2) * 8 + (r & 3)) * a.ld_lp) + lane_off) = w;
+                    }
+                }
+            }
+        }
+        return;
+    }
     // The running sum of a block is read as a whole before any of the block is written: with a load
     // and a store of the same array per element the compiler keeps them in program order, one memory
     // latency per element (67 us per tile instead of a few).
