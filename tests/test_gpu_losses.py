@@ -730,5 +730,5 @@ def test_trainer_method_raises_on_a_token_id_outside_the_vocabulary(amd, single_
     tr = _fake_trainer(amd, case, T, skip_masked=True, single_pass=single_pass)
     with pytest.raises(IndexError):
         tr._compute_loss(model, bad)
-    assert math.isfinite(float(tr._compute_loss(model, inputs)))
+    assert math.isfinite(float(tr._compute_loss(model, inputs).detach()))
     amd.check_device_errors()
