@@ -1007,7 +1007,9 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
 // Rows beyond the chunk and tokens beyond N are written as zeros.
 constexpr int kSdzRows = 128, kSdzTokens = 256, kSdzQuads = kSdzRows / 4 / 4;  // quads per wave
 // COLS: the tokens were compacted since the forward, a.stash_cols maps them to their stash columns.
-template <bool COLS>
+// CAPPED: soft-capped head (the chain factor needs the logit: a logarithm per numerator); a kernel of its own, so that
+// the usual sweep is straight-line code.
+template <bool COLS, bool CAPPED>
 __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
     typedef Elem<TRLK_F16> E;  // the numerators and dz are fp16
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1070,9 +1072,9 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
             rf[h][j] = (COLS && cj < 0) ? 0.f : refs[int64_t(h) * ld + cj];
             pf[h][j] = fast_exp2(rf[h][j] - kStashExp - lzc[j]);
         }
-    const bool capped = a.softcap > 0.f;
+    constexpr bool capped = CAPPED;
     float zt[4] = {0.f, 0.f, 0.f, 0.f};
-    if (capped) {
+    if constexpr (capped) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) zt[j] = col[j] >= 0 ? a.stash.zt()[col[j]] : 0.f;
     }
@@ -1094,7 +1096,7 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
             for (int j = 0; j < 4; ++j) {
                 const float p = e[j][i] * pf[h][j];
                 float dv;
-                if (!capped) {
+                if constexpr (!capped) {
                     dv = ngc[j] * p;
                     if (tg[j] == row) dv -= ngc[j];
                 } else {
@@ -1730,10 +1732,15 @@ extern "C" int trlk_fused_head_bwd(const void* d_hidden, const void* d_weight, c
             a.sdz_token_blocks = int(l.npad / kSdzTokens);
             a.sdz_tiles = a.sdz_token_blocks * int(kpad / kSdzRows);
             const dim3 grid(unsigned((a.sdz_tiles + 7) / 8 * 8));
-            if (d_stash_cols)
-                hipLaunchKernelGGL(head_dz_from_stash_kernel<true>, grid, dim3(256), 0, s, a);
+            const bool capped = a.softcap > 0.f;
+            if (d_stash_cols && capped)
+                hipLaunchKernelGGL((head_dz_from_stash_kernel<true, true>), grid, dim3(256), 0, s, a);
+            else if (d_stash_cols)
+                hipLaunchKernelGGL((head_dz_from_stash_kernel<true, false>), grid, dim3(256), 0, s, a);
+            else if (capped)
+                hipLaunchKernelGGL((head_dz_from_stash_kernel<false, true>), grid, dim3(256), 0, s, a);
             else
-                hipLaunchKernelGGL(head_dz_from_stash_kernel<false>, grid, dim3(256), 0, s, a);
+                hipLaunchKernelGGL((head_dz_from_stash_kernel<false, false>), grid, dim3(256), 0, s, a);
             rc = launch_status("fused_head_bwd (dz from the stash)");
         } else {
             rc = dtype == TRLK_BF16
