@@ -1112,7 +1112,10 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
             uint2 w;
             w.x = E::pack2(d[0], d[1]);
             w.y = E::pack2(d[2], d[3]);
-            *reinterpret_cast<uint2*>(a.dzT + int64_t(row) * a.ldzt + n0 + tl0) = w;
+            // (non-temporal: 2 GB per chunk that no cache holds until the products read it)
+            typedef uint32_t u32x2_nt __attribute__((ext_vector_type(2)));
+            const u32x2_nt wv = {w.x, w.y};
+            __builtin_nontemporal_store(wv, reinterpret_cast<u32x2_nt*>(a.dzT + int64_t(row) * a.ldzt + n0 + tl0));
         }
     }
 }
