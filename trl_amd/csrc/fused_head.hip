@@ -1001,8 +1001,8 @@ TRLK_HEAD_KERNEL void fused_head_dz_kernel(HeadArgs a) {
 
 // dz pass of the backward from the forward's stashed softmax numerators instead of a recompute: an
 // elementwise sweep (memory bound: 2 bytes read, 2 bytes written per logit, one multiplication each).
-// One workgroup = 128 vocabulary rows x 256 tokens.  A lane owns 4 consecutive tokens, a wave 32 rows = 8 row quads
-// whose 16 loads (32 bytes per quad and lane: 4 tokens x 4 rows) are all issued before the first result is used.
+// One workgroup = 128 vocabulary rows x 256 tokens.  A lane owns two pairs of tokens, a wave 32 rows = 8 row quads
+// whose 16 loads (16 bytes each: 2 tokens x 4 rows) are all issued before the first result is used.
 // dz^T (vocabulary-major, like the stash) is written in place, each token's column in that token's own scale.
 // Rows beyond the chunk and tokens beyond N are written as zeros.
 constexpr int kSdzRows = 128, kSdzTokens = 256, kSdzQuads = kSdzRows / 4 / 4;  // quads per wave
@@ -1023,13 +1023,15 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
     const int rows = a.c1 - a.c0;
     const float zs = a.logit_scale * a.inv_t;
     const int64_t ld = a.stash.ld;
-    const int tl0 = lane * 4;  // first token of the lane
+    // A lane owns two pairs of neighbouring tokens, 128 apart: every load instruction of the wave then reads 1 KiB of
+    // one stash row without gaps (16 bytes = 2 tokens x 4 rows per lane), every store 256 contiguous bytes of a dz row.
+    const int tl[4] = {lane * 2, lane * 2 + 1, 128 + lane * 2, 128 + lane * 2 + 1};
     float ngc[4], lzc[4];  // -g * zs in the token's own scale; log_z in base 2
     int tg[4], col[4];     // chunk-local target row (or -1); stash column
     bool live[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int tok = n0 + tl0 + j;
+        const int tok = n0 + tl[j];
         const bool ok = tok < a.N;
         col[j] = ok ? (COLS ? a.stash_cols[tok] : tok) : -1;
         const float g = ok ? a.g[tok] : 0.f;
@@ -1039,8 +1041,9 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
         const int64_t t = ok ? a.targets[tok] - a.c0 : -1;
         tg[j] = (t >= 0 && t < rows) ? int(t) : -1;
     }
-    const bool contiguous = !COLS || (col[0] >= 0 && col[1] == col[0] + 1 && col[2] == col[0] + 2 && col[3] == col[0] + 3);
-    const int first_col = COLS ? col[0] : n0 + tl0;  // (tokens beyond N of the last block are inside the padded row)
+    // (tokens beyond N of the last block are inside the padded row)
+    const bool pair0 = !COLS || (col[0] >= 0 && col[1] == col[0] + 1), pair1 = !COLS || (col[2] >= 0 && col[3] == col[2] + 1);
+    const int c0 = COLS ? col[0] : n0 + tl[0], c2 = COLS ? col[2] : n0 + tl[2];
     // the numerators of the wave's 8 quads
     const int row_w = r0 + wave * (kSdzRows / 4);                         // chunk-local first row of the wave
     const uint2* qrow = a.stash.quads() + int64_t((a.c0 + row_w) / 4) * ld;  // (chunks and tiles start on whole 128-row blocks)
@@ -1048,17 +1051,22 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
 #pragma unroll
     for (int qi = 0; qi < kSdzQuads; ++qi) {
         const uint2* src = qrow + int64_t(qi) * ld;
-        if (contiguous) {
-            typedef uint32_t u32x4_8 __attribute__((ext_vector_type(4), aligned(8)));
-            const u32x4_8 lo = __builtin_nontemporal_load(reinterpret_cast<const u32x4_8*>(src + first_col));
-            const u32x4_8 hi = __builtin_nontemporal_load(reinterpret_cast<const u32x4_8*>(src + first_col + 2));
+        typedef uint32_t u32x4_8 __attribute__((ext_vector_type(4), aligned(8)));
+        if (pair0) {
+            const u32x4_8 lo = __builtin_nontemporal_load(reinterpret_cast<const u32x4_8*>(src + c0));
             eb[qi][0] = make_uint2(lo.x, lo.y);
             eb[qi][1] = make_uint2(lo.z, lo.w);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) eb[qi][j] = col[j] >= 0 ? src[col[j]] : make_uint2(0u, 0u);
+        }
+        if (pair1) {
+            const u32x4_8 hi = __builtin_nontemporal_load(reinterpret_cast<const u32x4_8*>(src + c2));
             eb[qi][2] = make_uint2(hi.x, hi.y);
             eb[qi][3] = make_uint2(hi.z, hi.w);
         } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) eb[qi][j] = col[j] >= 0 ? src[col[j]] : make_uint2(0u, 0u);
+            for (int j = 2; j < 4; ++j) eb[qi][j] = col[j] >= 0 ? src[col[j]] : make_uint2(0u, 0u);
         }
     }
     // reference exponents of the two quad parities -> the factor that turns a numerator into -g * zs * p
@@ -1068,7 +1076,7 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
     for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int cj = COLS ? col[j] : first_col + j;
+            const int cj = COLS ? col[j] : n0 + tl[j];
             rf[h][j] = (COLS && cj < 0) ? 0.f : refs[int64_t(h) * ld + cj];
             pf[h][j] = fast_exp2(rf[h][j] - kStashExp - lzc[j]);
         }
@@ -1109,13 +1117,10 @@ __global__ __launch_bounds__(256) void head_dz_from_stash_kernel(HeadArgs a) {
                 }
                 d[j] = (row < rows && live[j]) ? dv : 0.f;
             }
-            uint2 w;
-            w.x = E::pack2(d[0], d[1]);
-            w.y = E::pack2(d[2], d[3]);
             // (non-temporal: 2 GB per chunk that no cache holds until the products read it)
-            typedef uint32_t u32x2_nt __attribute__((ext_vector_type(2)));
-            const u32x2_nt wv = {w.x, w.y};
-            __builtin_nontemporal_store(wv, reinterpret_cast<u32x2_nt*>(a.dzT + int64_t(row) * a.ldzt + n0 + tl0));
+            uint32_t* out = reinterpret_cast<uint32_t*>(a.dzT + int64_t(row) * a.ldzt + n0);
+            __builtin_nontemporal_store(E::pack2(d[0], d[1]), out + lane);
+            __builtin_nontemporal_store(E::pack2(d[2], d[3]), out + 64 + lane);
         }
     }
 }
