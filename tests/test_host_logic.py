@@ -1,5 +1,5 @@
-"""Host-side logic of the trainer mix-ins that needs no GPU: how the model call's keyword arguments are built for a
-sub-batch of a multimodal batch (trl/trainer/grpo_trainer.py:1463-1510)."""
+"""Host-side logic that needs no GPU: how the model call's keyword arguments are built for a sub-batch of a multimodal
+batch (trl/trainer/grpo_trainer.py:1463-1510), and when the fused head keeps its stash."""
 import torch
 
 
@@ -66,3 +66,24 @@ def test_image_and_tile_indexed_inputs():
     # text only: nothing but the text arguments
     out = tr._model_inputs(ids, attn, 0, 3, 2, False)
     assert set(out) == {"input_ids", "attention_mask", "logits_to_keep", "use_cache"}
+
+
+def test_head_stash_budget_and_shape(monkeypatch):
+    """The stash of the fused head: its size comes from the library (2 bytes per logit + one reference exponent per 64
+    logits + the targets' logits, both dimensions padded to 256) and the host keeps it only within its budget."""
+    from trl_amd import ops
+
+    n, v = 300, 1000
+    rows, ld, four = ops._head_stash_shape(n, v)
+    vpad = 1024
+    assert (rows, ld, four) == (vpad // 4 + vpad // 128 + 1, 512, 4)
+    nbytes = rows * ld * four * 2
+    monkeypatch.setenv("TRL_AMD_HEAD_STASH_GIB", str((nbytes + 1) / 2**30))
+    assert ops.head_stash_fits(n, v)
+    monkeypatch.setenv("TRL_AMD_HEAD_STASH_GIB", str((nbytes - 1) / 2**30))
+    assert not ops.head_stash_fits(n, v)
+    monkeypatch.setenv("TRL_AMD_HEAD_STASH_GIB", "0")
+    assert not ops.head_stash_fits(n, v) and not ops.head_stash_fits(1, 1)
+    monkeypatch.delenv("TRL_AMD_HEAD_STASH_GIB")
+    assert ops.head_stash_fits(32768, 151936) and not ops.head_stash_fits(0, v)  # 10.3 GB of the default 24 GiB
+    assert not ops.head_stash_fits(131072, 151936)  # 41 GB
