@@ -97,9 +97,6 @@ struct Operand {
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
-#ifndef TRLK_HEAD_DIRECT_LDS
-#define TRLK_HEAD_DIRECT_LDS 1
-#endif
 // k-step width of the direct-to-LDS loop per kernel.  All three use 64-wide steps (two 64 KiB stages, half as
 // many barriers, whole 128-byte lines per row and step); the 32-wide, four-stage ring was only ahead for the
 // short contraction over the hidden size while the forward's workgroups still ran out of step with each other.
@@ -499,14 +496,12 @@ template <int DT, int BKT, bool AKM = false>
 __device__ __forceinline__ void gemm_tile_nt(const Operand A, int m0, const Operand B, int n0, int K,
                                              f32x16 (&acc)[MB][NB], char* smem, bool prefetched = false) {
     if constexpr (AKM) {  // (callers of this form pad K to whole steps)
-        static_assert(TRLK_HEAD_DIRECT_LDS && BKT == 64, "k-major left operands need the direct-to-LDS loop");
+        static_assert(BKT == 64, "k-major left operands need the direct-to-LDS loop with 64-wide steps");
         gemm_tile_nt_direct<DT, BKT, true>(A, m0, B, n0, K, acc, smem, prefetched);
     } else {
-#if TRLK_HEAD_DIRECT_LDS
         if ((K & (BKT - 1)) == 0)
             gemm_tile_nt_direct<DT, BKT>(A, m0, B, n0, K, acc, smem, prefetched);
         else
-#endif
             gemm_tile_nt_staged<DT>(A, m0, B, n0, K, acc, smem);
     }
 }
@@ -1620,7 +1615,7 @@ extern "C" int trlk_fused_head_fwd(const void* d_hidden, const void* d_weight, c
     const char* what = "fused_head_fwd";
     int rc;
     const bool general = a.softcap > 0.f || !(a.logit_scale * a.inv_t > 0.f);
-    const bool staged = !TRLK_HEAD_DIRECT_LDS || hidden_size % TRLK_HEAD_BK_FWD != 0;
+    const bool staged = hidden_size % TRLK_HEAD_BK_FWD != 0;
     auto launch_fwd = [&](auto stash_tag, auto general_tag) {
         constexpr bool kS = decltype(stash_tag)::value, kG = decltype(general_tag)::value;
         if (staged)
